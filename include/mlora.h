@@ -1,0 +1,159 @@
+/*
+ * mlora.h - C ABI of the MI355X (gfx950) multi-LoRA decode/prefill hot path.
+ *
+ * The reference (llm-db/tensor-program-optimization-with-auto-batching) is pure Python and exposes no
+ * FFI; its per-layer operators are TVM Relax ops lowered to generated GPU kernels, or torch modules.
+ * Each entry point below replaces one of those operators and cites it.  A Python host (torch tensors
+ * for device memory and streams) binds this library with ctypes.
+ *
+ * Conventions
+ *   - every pointer is a caller-owned DEVICE pointer unless named host_*; nothing here allocates
+ *     device memory; work is enqueued on `stream` (a hipStream_t passed as void*; NULL = default
+ *     stream) and the call returns without synchronising;
+ *   - fp16 tensors are IEEE binary16, row-major, innermost dimension contiguous;
+ *   - return value 0 = success, negative = MLORA_ERR_*; mlora_last_error() gives the message of the
+ *     last failure on the calling thread;
+ *   - shapes are validated on the host before any launch; a rejected call launches nothing.
+ */
+#ifndef MLORA_H
+#define MLORA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MLORA_OK                 0
+#define MLORA_ERR_INVALID       -1   /* bad shape / argument */
+#define MLORA_ERR_UNSUPPORTED   -2   /* shape outside what the kernels cover */
+#define MLORA_ERR_WORKSPACE     -3   /* workspace missing or too small */
+#define MLORA_ERR_LAUNCH        -4   /* HIP reported a launch error */
+
+#define MLORA_F16 0
+#define MLORA_F32 1
+
+/* y = acc, or y += acc, in the epilogue of the linear kernels */
+#define MLORA_STORE       0
+#define MLORA_ACCUMULATE  1
+
+#define MLORA_PAGE_SIZE 16   /* tokens per KV page; the only page size the kernels accept */
+
+int mlora_version(void);
+const char* mlora_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Adapter-indexed LoRA delta ("gather-matmul"):
+ *     y[t, :] += scaling * B[id_t] . (A[id_t] . x[t, :])      for every t with 0 <= id_t < n_ad
+ * fp16 operands, fp32 accumulation; rows with id_t outside [0, n_ad) are left untouched.
+ *
+ * Replaces: GatherBMMLinear.forward hot branch (huggingface/custom_peft/lora_gatherbmm_linear_layer.py:14-20:
+ *   stack of per-request A / scaled B, two bmm, add to the base result); the TVM adapter forward
+ *   take -> matmul -> matmul -> *scaling (tvm/llama_auto_batcher/compile_tvm.py:106-112) with its fused
+ *   take_matmul kernel (tvm/custom/fuse_take_matmul.py:85-105); and, because rows are addressed by
+ *   token, the row gather/scatter around it in the mixed path (compile_tvm.py:147-153,
+ *   tvm/custom/write_tensor_part.py:3-20).
+ *
+ * Layouts (PEFT orientation): x [T, K] f16; A [n_ad, r, K] f16; B [n_ad, N, r] f16;
+ *   y [T, N] f16 or f32 (y_dtype); tok_adapter [T] int32.
+ * Constraints: r in {8, 16, 32, 64}; K % 8 == 0; N % 8 == 0.
+ * workspace: mlora_gather_mm_workspace_bytes(T, K, r) bytes of device scratch (shrink partials);
+ *   contents need not be initialised.
+ * ------------------------------------------------------------------------------------------- */
+size_t mlora_gather_mm_workspace_bytes(int T, int K, int r);
+int mlora_gather_mm(void* y, int y_dtype, const void* x, const void* A, const void* B,
+                    const int32_t* tok_adapter, float scaling,
+                    int T, int K, int N, int r, int n_ad,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* The two halves of the above, for callers that fuse differently:
+ *   shrink: v_part[c, t, :] = A[id_t][:, chunk c] . x[t, chunk c]   (fp32 partials per K-chunk)
+ *   expand: y[t, :] += scaling * B[id_t] . sum_c v_part[c, t, :]
+ * Same layouts and constraints; v_part is the workspace described above. */
+int mlora_lora_shrink(void* v_part, const void* x, const void* A, const int32_t* tok_adapter,
+                      int T, int K, int r, int n_ad, void* stream);
+int mlora_lora_expand(void* y, int y_dtype, const void* v_part, const void* B, const int32_t* tok_adapter,
+                      float scaling, int T, int K, int N, int r, int n_ad, void* stream);
+
+/* Z = X; Z[ids[a], :] = Y[a, :]  - row scatter of the mixed-adapter-type path.
+ * Replaces: write_tensor_part (tvm/custom/write_tensor_part.py:3-20).  X, Z [B, PH] f16, Y [A, PH] f16,
+ * ids [A] int32 (rows with ids outside [0, B) are skipped).  Z may alias X. */
+int mlora_write_tensor_part(void* Z, const void* X, const void* Y, const int32_t* ids,
+                            int B, int A, int PH, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Base linear  y[T, N] (=|+=) x[T, K] . W[N, K]^T   (bias-free), fp16 operands, fp32 accumulation.
+ * Replaces: nn.Linear(bias=False) of the q/k/v/o, gate/up/down projections and lm_head
+ *   (tvm/llama_auto_batcher/llama_for_causal_lm.py:31-33,44-47,105), including the fp32 cast of the
+ *   logits (:124-128) when y_dtype = MLORA_F32, and the residual add (:80-83) when mode =
+ *   MLORA_ACCUMULATE with an fp32 y.
+ *
+ * mlora_gemv: weight-streaming kernel for T <= 64 (decode).   mlora_gemm: MFMA-tiled kernel for any T.
+ * mlora_linear picks between them.  x row stride ldx (elements) lets x be a column slice.
+ * Constraints: K % 32 == 0, N % 4 == 0, ldx % 8 == 0; MLORA_ACCUMULATE needs y_dtype = MLORA_F32.
+ * ------------------------------------------------------------------------------------------- */
+int mlora_gemv(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W,
+               int T, int K, int N, void* stream);
+int mlora_gemm(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W,
+               int T, int K, int N, void* stream);
+int mlora_linear(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W,
+                 int T, int K, int N, void* stream);
+
+/* y[t, :] = f16( x[t, :] * rsqrt(mean(x[t, :]^2) + eps) * w )   row-wise, statistics in fp32.
+ * Replaces: nn.RMSNorm(hidden, -1, eps, bias=False) (llama_for_causal_lm.py:76-77,93).
+ * x [T, H] f16 or f32 (x_dtype), w [H] f16, y [T, H] f16.  H % 8 == 0, H <= 16384. */
+int mlora_rmsnorm(void* y, const void* x, int x_dtype, const void* w, float eps, int T, int H, void* stream);
+
+/* out[t, i] = f16( silu(gate[t, i]) * up[t, i] );  gate and up are column slices with row stride ld
+ * (elements) so a fused [T, 2I] projection output can be passed as (p, p + I, 2I).
+ * Replaces: op.silu(gate_proj(x)) * up_proj(x) (llama_for_causal_lm.py:35-36).  I % 8 == 0. */
+int mlora_silu_mul(void* out, const void* gate, const void* up, int ld, int T, int I, void* stream);
+
+/* out[t, :] = table[ids[t], :] widened to out_dtype.  Replaces: nn.Embedding lookup
+ * (llama_for_causal_lm.py:121-122).  table [V, H] f16; ids outside [0, V) produce a zero row. */
+int mlora_embed(void* out, int out_dtype, const void* table, const int32_t* ids, int T, int H, int V, void* stream);
+
+/* ids[b] = argmax_v logits[b, v], lowest index on ties (numpy.argmax).
+ * Replaces: the host-side np.argmax over D2H-copied logits (tvm/llama_auto_batcher/llama_exec_graph.py:92,134-137). */
+int mlora_argmax(int32_t* ids, const float* logits, int B, int V, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Paged KV cache (16-token pages) - replaces TVM's TIRPagedKVCache as configured at
+ * llama_for_causal_lm.py:148-174 (RoPE applied inside the cache op, rotary_dim = head_dim, scale 1,
+ * no sliding window) and driven by kv_state_begin_forward / attention_with_fused_qkv / end_forward
+ * (tvm/llama_auto_batcher/llama_exec_graph.py:75-85,121-127; llama_for_causal_lm.py:55-64).
+ *
+ * Layouts, per layer:
+ *   k_cache [n_pages, Hkv, 16, D] f16   - rotated keys, one 16-token page of one head contiguous
+ *   v_cache [n_pages, Hkv, D, 16] f16   - values, token-minor inside a page
+ *   block_table [n_seq, max_blocks] int32 - physical page of logical block j of sequence s
+ *   qkv [T, Hq + 2 Hkv, D] f16 - fused projection output, token-major
+ *   rope_cos / rope_sin [max_pos, D/2] f32 - tables; element i pairs with element i + D/2
+ *
+ * mlora_rope_kv_append: for token t (sequence tok_seq[t], position tok_pos[t]) rotate the q heads in
+ *   place inside qkv, rotate k and write k, v into the page slot of that position.
+ * mlora_paged_attn_decode: one query per sequence; out[b, h, :] = softmax(q . K^T / sqrt(D)) V over the
+ *   first ctx_len[b] cached positions of sequence seq_ids[b] (the new token already appended).
+ * mlora_paged_attn_prefill: query token t (sequence tok_seq[t], position tok_pos[t]) attends to cached
+ *   positions 0..tok_pos[t]; tokens of a sequence must be consecutive in t with increasing positions.
+ * q is read from qkv (already rotated).  out [T, Hq, D] f16.  D in {64, 128}; Hq % Hkv == 0.
+ * ------------------------------------------------------------------------------------------- */
+int mlora_rope_kv_append(void* qkv, void* k_cache, void* v_cache,
+                         const int32_t* block_table, int max_blocks,
+                         const int32_t* tok_seq, const int32_t* tok_pos,
+                         const float* rope_cos, const float* rope_sin, int max_pos,
+                         int T, int Hq, int Hkv, int D, int n_pages, int n_seq, void* stream);
+int mlora_paged_attn_decode(void* out, const void* qkv, const void* k_cache, const void* v_cache,
+                            const int32_t* block_table, int max_blocks,
+                            const int32_t* seq_ids, const int32_t* ctx_len,
+                            int B, int Hq, int Hkv, int D, int n_pages, int n_seq, void* stream);
+int mlora_paged_attn_prefill(void* out, const void* qkv, const void* k_cache, const void* v_cache,
+                             const int32_t* block_table, int max_blocks,
+                             const int32_t* tok_seq, const int32_t* tok_pos,
+                             int T, int Hq, int Hkv, int D, int n_pages, int n_seq, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLORA_H */

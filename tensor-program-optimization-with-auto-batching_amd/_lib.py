@@ -1,0 +1,67 @@
+"""ctypes binding of libmlora_hip.so (the C ABI declared in include/mlora.h).
+
+There is no fallback: if the library has not been built, loading raises and every operator fails.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmlora_hip.so")
+
+F16, F32 = 0, 1
+STORE, ACCUMULATE = 0, 1
+PAGE_SIZE = 16
+
+_p, _i, _f, _z = C.c_void_p, C.c_int, C.c_float, C.c_size_t
+
+# name -> (restype, argtypes); mirrors include/mlora.h one to one
+SIGNATURES = {
+    "mlora_version": (_i, []),
+    "mlora_last_error": (C.c_char_p, []),
+    "mlora_gather_mm_workspace_bytes": (_z, [_i, _i, _i]),
+    "mlora_gather_mm": (_i, [_p, _i, _p, _p, _p, _p, _f, _i, _i, _i, _i, _i, _p, _z, _p]),
+    "mlora_lora_shrink": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),
+    "mlora_lora_expand": (_i, [_p, _i, _p, _p, _p, _f, _i, _i, _i, _i, _i, _p]),
+    "mlora_write_tensor_part": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
+    "mlora_gemv": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
+    "mlora_gemm": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
+    "mlora_linear": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
+    "mlora_rmsnorm": (_i, [_p, _p, _i, _p, _f, _i, _i, _p]),
+    "mlora_silu_mul": (_i, [_p, _p, _p, _i, _i, _i, _p]),
+    "mlora_embed": (_i, [_p, _i, _p, _p, _i, _i, _i, _p]),
+    "mlora_argmax": (_i, [_p, _p, _i, _i, _p]),
+    "mlora_rope_kv_append": (_i, [_p, _p, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "mlora_paged_attn_decode": (_i, [_p, _p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
+    "mlora_paged_attn_prefill": (_i, [_p, _p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
+}
+
+_lib = None
+
+
+class MloraError(RuntimeError):
+    def __init__(self, code: int, msg: str):
+        super().__init__(f"mlora error {code}: {msg}")
+        self.code = code
+
+
+def lib() -> C.CDLL:
+    """The loaded library; raises if libmlora_hip.so is missing (build it with build.py)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} not found: the HIP library is not built (run build.py). There is no CPU fallback.")
+        l = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def check(code: int) -> None:
+    if code != 0:
+        raise MloraError(code, lib().mlora_last_error().decode())

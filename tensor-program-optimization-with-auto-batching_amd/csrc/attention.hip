@@ -1,0 +1,356 @@
+// Paged-KV attention for gfx950: RoPE + cache append, decode attention, prefill attention.
+//
+// Cache layout per layer (16-token pages):
+//   k_cache [n_pages, Hkv, 16, D]  rotated keys   - a page of one head is 16*D contiguous fp16
+//   v_cache [n_pages, Hkv, D, 16]  values         - token-minor, so a lane's 16-byte load holds 8
+//                                                   consecutive tokens of one dim
+// The K layout gives the decode kernel and the MFMA prefill kernel 16-byte loads along D; the V
+// layout gives both of them the P.V contraction (over tokens) without an LDS transpose.
+// The page-table walk is integer-only: page = block_table[seq, pos / 16], slot = pos % 16.
+#include "common.h"
+
+namespace {
+
+constexpr int PAGE = MLORA_PAGE_SIZE;
+
+// grid (T, Hq + 2 Hkv), 64 threads: thread i rotates the pair (i, i + D/2) of one head of one token
+__global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qkv, f16* __restrict__ k_cache,
+                                                            f16* __restrict__ v_cache,
+                                                            const int32_t* __restrict__ block_table, int max_blocks,
+                                                            const int32_t* __restrict__ tok_seq,
+                                                            const int32_t* __restrict__ tok_pos,
+                                                            const float* __restrict__ rope_cos,
+                                                            const float* __restrict__ rope_sin, int max_pos, int Hq,
+                                                            int Hkv, int D, int n_pages, int n_seq) {
+#pragma clang fp contract(off)
+  const int t = blockIdx.x, hh = blockIdx.y, i = threadIdx.x;
+  const int half = D >> 1;
+  if (i >= half) return;
+  const int seq = tok_seq[t], pos = tok_pos[t];
+  if (seq < 0 || seq >= n_seq || pos < 0 || pos >= max_pos || pos / PAGE >= max_blocks) return;
+  f16* src = qkv + ((size_t)t * (Hq + 2 * Hkv) + hh) * D;
+  if (hh >= Hq + Hkv) {
+    const int page = block_table[(size_t)seq * max_blocks + pos / PAGE];
+    if (page < 0 || page >= n_pages) return;
+    f16* dst = v_cache + ((size_t)page * Hkv + (hh - Hq - Hkv)) * D * PAGE + pos % PAGE;
+    dst[(size_t)i * PAGE] = src[i];
+    dst[(size_t)(i + half) * PAGE] = src[i + half];
+    return;
+  }
+  const float c = rope_cos[(size_t)pos * half + i], s = rope_sin[(size_t)pos * half + i];
+  const float x1 = (float)src[i], x2 = (float)src[i + half];
+  // Separately rounded products (fp contraction is off in this kernel) and an fp32 result that is
+  // materialised before the fp16 conversion (the empty asm keeps the compiler from fusing the add
+  // and the convert into one single-rounding instruction): the rotation is then the same IEEE fp32
+  // arithmetic as a plain CPU evaluation, and the stored fp16 keys are reproducible bit for bit.
+  float r1 = x1 * c - x2 * s;
+  float r2 = x2 * c + x1 * s;
+  asm volatile("" : "+v"(r1), "+v"(r2));
+  const f16 o1 = (f16)r1, o2 = (f16)r2;
+  if (hh < Hq) {
+    src[i] = o1;
+    src[i + half] = o2;
+  } else {
+    const int page = block_table[(size_t)seq * max_blocks + pos / PAGE];
+    if (page < 0 || page >= n_pages) return;
+    f16* dst = k_cache + (((size_t)page * Hkv + (hh - Hq)) * PAGE + pos % PAGE) * D;
+    dst[i] = o1;
+    dst[i + half] = o2;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Decode: one workgroup (4 waves) per (sequence, q head).  A wave takes pages w, w+4, ...; a page of
+// K is four (D=128) coalesced 1 KiB loads, as is a page of V.  Scores are reduced inside the group of
+// lanes that shares a token, broadcast with readlane, and folded into an fp32 online softmax; the
+// four waves' (max, sum, acc) states are merged through LDS.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void paged_attn_decode_kernel(f16* __restrict__ out, const f16* __restrict__ qkv,
+                                                                const f16* __restrict__ k_cache,
+                                                                const f16* __restrict__ v_cache,
+                                                                const int32_t* __restrict__ block_table, int max_blocks,
+                                                                const int32_t* __restrict__ seq_ids,
+                                                                const int32_t* __restrict__ ctx_len, int Hq, int Hkv,
+                                                                int n_pages, int n_seq, float scale) {
+  constexpr int LPT = D / 8;          // lanes sharing one token of a K load
+  constexpr int TPL = WAVE / LPT;     // tokens per K load
+  constexpr int NK = PAGE / TPL;      // K loads per page
+  constexpr int NV = D * PAGE / 512;  // V loads per page (512 fp16 each)
+  constexpr int NW = 4;
+  __shared__ float sm[NW], sl[NW];
+  __shared__ float sacc[NW][D];
+
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int kh = h / (Hq / Hkv);
+  const int seq = seq_ids[b];
+  int ctx = ctx_len[b];
+  if (seq < 0 || seq >= n_seq) ctx = 0;
+  if (ctx > max_blocks * PAGE) ctx = max_blocks * PAGE;
+  const int npages = (ctx + PAGE - 1) / PAGE;
+
+  const f16x8 q8 = ld8(qkv + ((size_t)b * (Hq + 2 * Hkv) + h) * D + (lane % LPT) * 8);
+
+  float m = -INFINITY, l = 0.f;
+  float acc[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) acc[i] = 0.f;
+
+  for (int pg = wave; pg < npages; pg += NW) {
+    const int page = block_table[(size_t)seq * max_blocks + pg];
+    if (page < 0 || page >= n_pages) continue;   // wave-uniform
+    const f16* kp = k_cache + ((size_t)page * Hkv + kh) * PAGE * D + lane * 8;
+    const f16* vp = v_cache + ((size_t)page * Hkv + kh) * D * PAGE + lane * 8;
+    f16x8 kf[NK], vf[NV];
+#pragma unroll
+    for (int i = 0; i < NK; ++i) kf[i] = ld8(kp + i * 512);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) vf[i] = ld8(vp + i * 512);
+
+    float sc[PAGE];
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+      float s = dot8(q8, kf[i], 0.f);
+#pragma unroll
+      for (int o = LPT >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, WAVE);
+      s *= scale;
+#pragma unroll
+      for (int g = 0; g < TPL; ++g)
+        sc[i * TPL + g] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s), g * LPT));
+    }
+    float pm = -INFINITY;
+#pragma unroll
+    for (int tk = 0; tk < PAGE; ++tk) {
+      if (pg * PAGE + tk >= ctx) sc[tk] = -INFINITY;
+      pm = fmaxf(pm, sc[tk]);
+    }
+    const float m_new = fmaxf(m, pm);     // finite: the first token of a visited page is < ctx
+    const float alpha = __expf(m - m_new);
+    float ps = 0.f;
+#pragma unroll
+    for (int tk = 0; tk < PAGE; ++tk) {
+      sc[tk] = __expf(sc[tk] - m_new);
+      ps += sc[tk];
+    }
+    l = l * alpha + ps;
+    m = m_new;
+    const bool hi = lane & 1;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      float a = acc[i] * alpha;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) a = fmaf(hi ? sc[8 + e] : sc[e], (float)vf[i][e], a);
+      acc[i] = a;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    acc[i] += __shfl_xor(acc[i], 1, WAVE);
+    if ((lane & 1) == 0) sacc[wave][i * 32 + (lane >> 1)] = acc[i];
+  }
+  if (lane == 0) {
+    sm[wave] = m;
+    sl[wave] = l;
+  }
+  __syncthreads();
+  if (threadIdx.x < D) {
+    float M = sm[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) M = fmaxf(M, sm[w]);
+    float L = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const float f = sm[w] == -INFINITY ? 0.f : __expf(sm[w] - M);
+      L += sl[w] * f;
+      o += sacc[w][threadIdx.x] * f;
+    }
+    out[((size_t)b * Hq + h) * D + threadIdx.x] = (f16)(L > 0.f ? o / L : 0.f);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Prefill: a wave owns 16 consecutive query tokens of one head and walks the pages of their
+// sequence.  S^T = K . Q^T on v_mfma_f32_16x16x32_f16 puts key index on the accumulator rows, which
+// is exactly the A-operand layout the matrix core wants for P in O = P . V (a lane's four
+// accumulator rows are the four keys it must supply) - no LDS, no shuffles between the two products.  A tile that straddles a sequence boundary is processed in one
+// pass per sequence with the other queries masked.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void paged_attn_prefill_kernel(f16* __restrict__ out, const f16* __restrict__ qkv,
+                                                                 const f16* __restrict__ k_cache,
+                                                                 const f16* __restrict__ v_cache,
+                                                                 const int32_t* __restrict__ block_table, int max_blocks,
+                                                                 const int32_t* __restrict__ tok_seq,
+                                                                 const int32_t* __restrict__ tok_pos, int T, int Hq,
+                                                                 int Hkv, int n_pages, int n_seq, float scale) {
+  constexpr int NKB = D / 32;   // k-blocks of the QK^T product
+  constexpr int NDB = D / 16;   // dim blocks of the output
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t0 = (blockIdx.x * 4 + wave) * 16;
+  if (t0 >= T) return;
+  const int h = blockIdx.y;
+  const int kh = h / (Hq / Hkv);
+  const int qi = lane & 15, g = lane >> 4;
+
+  const int tq = t0 + qi;
+  const bool valid_t = tq < T;
+  int my_seq = valid_t ? tok_seq[tq] : -1;
+  int my_pos = valid_t ? tok_pos[tq] : -1;
+  if (my_seq < 0 || my_seq >= n_seq || my_pos < 0 || my_pos >= max_blocks * PAGE) my_seq = -1;
+
+  // Q as the B operand: lane holds q[query qi][kb*32 + g*8 .. +8]
+  f16x8 qf[NKB];
+  {
+    const f16* qp = qkv + ((size_t)(valid_t ? tq : t0) * (Hq + 2 * Hkv) + h) * D + g * 8;
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) qf[kb] = ld8(qp + kb * 32);
+  }
+
+  float m = -INFINITY, l = 0.f;
+  f32x4 O[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) O[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  bool done = my_seq < 0;
+  while (true) {
+    const unsigned long long pending = __ballot(!done);
+    if (!pending) break;
+    const int cur_seq = __shfl(my_seq, __builtin_ctzll(pending), WAVE);
+    const bool in_run = !done && my_seq == cur_seq;
+    int maxpos = in_run ? my_pos : -1;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) maxpos = max(maxpos, __shfl_xor(maxpos, o, WAVE));
+    const int npages = maxpos / PAGE + 1;
+    for (int pg = 0; pg < npages; ++pg) {
+      const int page = block_table[(size_t)cur_seq * max_blocks + pg];
+      if (page < 0 || page >= n_pages) continue;   // wave-uniform
+      const f16* kp = k_cache + (((size_t)page * Hkv + kh) * PAGE + qi) * D + g * 8;   // key qi of the page
+      const f16* vp = v_cache + (((size_t)page * Hkv + kh) * D + qi) * PAGE + g * 4;   // dim qi (+16 db), keys 4g..
+      f16x8 kf[NKB];
+      f16x4 vf[NDB];
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) kf[kb] = ld8(kp + kb * 32);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) vf[db] = *reinterpret_cast<const f16x4*>(vp + db * 16 * PAGE);
+
+      f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f};   // st[r] = S[key 4g + r][query qi]
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) st = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kb], qf[kb], st, 0, 0, 0);
+
+      float pm = -INFINITY;
+      bool msk[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        msk[r] = !in_run || (pg * PAGE + 4 * g + r > my_pos);
+        st[r] = msk[r] ? -INFINITY : st[r] * scale;
+        pm = fmaxf(pm, st[r]);
+      }
+      pm = fmaxf(pm, __shfl_xor(pm, 16, WAVE));
+      pm = fmaxf(pm, __shfl_xor(pm, 32, WAVE));
+      const float m_new = fmaxf(m, pm);
+      const float alpha = m_new == -INFINITY ? 1.f : __expf(m - m_new);
+      // P goes to the matrix core as fp16 hi + lo halves (k-slots 0-3 and 4-7 of one k=32 MFMA, with V
+      // repeated in both), so the product carries ~22 mantissa bits of P instead of 11.
+      f16x8 pa;
+      float ps = 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = msk[r] ? 0.f : __expf(st[r] - m_new);
+        ps += p;
+        const f16 hi = (f16)p;
+        pa[r] = hi;
+        pa[4 + r] = (f16)(p - (float)hi);
+      }
+      l = l * alpha + ps;
+      m = m_new;
+      // O rows are queries 4g + r; their alpha lives in lanes with qi == 4g + r
+      float ar[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) ar[r] = __shfl(alpha, 4 * g + r, WAVE);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) O[db][r] *= ar[r];
+        const f16x8 vv = f16x8{vf[db][0], vf[db][1], vf[db][2], vf[db][3], vf[db][0], vf[db][1], vf[db][2], vf[db][3]};
+        O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vv, O[db], 0, 0, 0);
+      }
+    }
+    done = done || in_run;
+  }
+  l += __shfl_xor(l, 16, WAVE);
+  l += __shfl_xor(l, 32, WAVE);
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float ir = __shfl(inv, 4 * g + r, WAVE);
+    const int t = t0 + 4 * g + r;
+    if (t < T) {
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) out[((size_t)t * Hq + h) * D + db * 16 + qi] = (f16)(O[db][r] * ir);
+    }
+  }
+}
+
+int check_attn(const char* who, int Hq, int Hkv, int D, int n_pages, int n_seq, int max_blocks) {
+  MLORA_CHECK(D == 64 || D == 128, MLORA_ERR_UNSUPPORTED, "%s: head_dim %d not in {64, 128}", who, D);
+  MLORA_CHECK(Hq > 0 && Hkv > 0 && Hq % Hkv == 0, MLORA_ERR_INVALID, "%s: bad heads Hq=%d Hkv=%d", who, Hq, Hkv);
+  MLORA_CHECK(n_pages > 0 && n_seq > 0 && max_blocks > 0, MLORA_ERR_INVALID, "%s: bad cache shape n_pages=%d n_seq=%d max_blocks=%d", who, n_pages, n_seq, max_blocks);
+  MLORA_CHECK(Hq + 2 * Hkv <= 65535, MLORA_ERR_UNSUPPORTED, "%s: too many heads", who);
+  return MLORA_OK;
+}
+
+}  // namespace
+
+extern "C" int mlora_rope_kv_append(void* qkv, void* k_cache, void* v_cache, const int32_t* block_table, int max_blocks,
+                                    const int32_t* tok_seq, const int32_t* tok_pos, const float* rope_cos,
+                                    const float* rope_sin, int max_pos, int T, int Hq, int Hkv, int D, int n_pages,
+                                    int n_seq, void* stream) {
+  if (int e = check_attn("rope_kv_append", Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
+  MLORA_CHECK(qkv && k_cache && v_cache && block_table && tok_seq && tok_pos && rope_cos && rope_sin, MLORA_ERR_INVALID, "rope_kv_append: null pointer");
+  MLORA_CHECK(T >= 0 && max_pos > 0, MLORA_ERR_INVALID, "rope_kv_append: bad T=%d max_pos=%d", T, max_pos);
+  if (T == 0) return MLORA_OK;
+  hipLaunchKernelGGL(rope_kv_append_kernel, dim3(T, Hq + 2 * Hkv), dim3(64), 0, (hipStream_t)stream, (f16*)qkv,
+                     (f16*)k_cache, (f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, rope_cos, rope_sin,
+                     max_pos, Hq, Hkv, D, n_pages, n_seq);
+  return mlora_launch_status("rope_kv_append");
+}
+
+extern "C" int mlora_paged_attn_decode(void* out, const void* qkv, const void* k_cache, const void* v_cache,
+                                       const int32_t* block_table, int max_blocks, const int32_t* seq_ids,
+                                       const int32_t* ctx_len, int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                                       void* stream) {
+  if (int e = check_attn("paged_attn_decode", Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
+  MLORA_CHECK(out && qkv && k_cache && v_cache && block_table && seq_ids && ctx_len, MLORA_ERR_INVALID, "paged_attn_decode: null pointer");
+  MLORA_CHECK(B >= 0, MLORA_ERR_INVALID, "paged_attn_decode: bad B=%d", B);
+  if (B == 0) return MLORA_OK;
+  const float scale = 1.f / sqrtf((float)D);
+  hipStream_t s = (hipStream_t)stream;
+  if (D == 128)
+    hipLaunchKernelGGL(paged_attn_decode_kernel<128>, dim3(B, Hq), dim3(256), 0, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
+                       (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale);
+  else
+    hipLaunchKernelGGL(paged_attn_decode_kernel<64>, dim3(B, Hq), dim3(256), 0, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
+                       (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale);
+  return mlora_launch_status("paged_attn_decode");
+}
+
+extern "C" int mlora_paged_attn_prefill(void* out, const void* qkv, const void* k_cache, const void* v_cache,
+                                        const int32_t* block_table, int max_blocks, const int32_t* tok_seq,
+                                        const int32_t* tok_pos, int T, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                                        void* stream) {
+  if (int e = check_attn("paged_attn_prefill", Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
+  MLORA_CHECK(out && qkv && k_cache && v_cache && block_table && tok_seq && tok_pos, MLORA_ERR_INVALID, "paged_attn_prefill: null pointer");
+  MLORA_CHECK(T >= 0, MLORA_ERR_INVALID, "paged_attn_prefill: bad T=%d", T);
+  if (T == 0) return MLORA_OK;
+  const float scale = 1.f / sqrtf((float)D);
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(ceil_div(T, 64), Hq);
+  if (D == 128)
+    hipLaunchKernelGGL(paged_attn_prefill_kernel<128>, grid, dim3(256), 0, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
+                       (const f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, T, Hq, Hkv, n_pages, n_seq, scale);
+  else
+    hipLaunchKernelGGL(paged_attn_prefill_kernel<64>, grid, dim3(256), 0, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
+                       (const f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, T, Hq, Hkv, n_pages, n_seq, scale);
+  return mlora_launch_status("paged_attn_prefill");
+}

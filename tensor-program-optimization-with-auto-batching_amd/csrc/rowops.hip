@@ -1,0 +1,186 @@
+// Row-wise operators for gfx950: RMSNorm, SiLU*mul, embedding gather, argmax.
+// All are a few hundred KiB per call at decode batch sizes - one pass over the row in registers,
+// 64-lane wave reductions, one LDS exchange between the waves of a block.
+#include "common.h"
+
+namespace {
+
+constexpr int ROW_THREADS = 256;
+
+__device__ __forceinline__ float block_sum(float v, float* lds) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) lds[wave] = v;
+  __syncthreads();
+  float s = 0.f;
+#pragma unroll
+  for (int w = 0; w < ROW_THREADS / WAVE; ++w) s += lds[w];
+  return s;
+}
+
+// One block per row; each thread keeps up to VPT 8-element vectors of the row in registers.
+template <typename XT, int VPT>
+__global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(f16* __restrict__ y, const XT* __restrict__ x,
+                                                              const f16* __restrict__ w, float eps, int H) {
+  __shared__ float lds[ROW_THREADS / WAVE];
+  const int row = blockIdx.x;
+  const XT* xr = x + (size_t)row * H;
+  float v[VPT][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = (i * ROW_THREADS + threadIdx.x) * 8;
+    if (c < H) {
+      if constexpr (sizeof(XT) == 2) {
+        const f16x8 t = ld8((const f16*)xr + c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[i][e] = (float)t[e];
+      } else {
+        const f32x4 lo = *reinterpret_cast<const f32x4*>((const float*)xr + c);
+        const f32x4 hi = *reinterpret_cast<const f32x4*>((const float*)xr + c + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[i][e] = lo[e];
+          v[i][4 + e] = hi[e];
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss = fmaf(v[i][e], v[i][e], ss);
+    }
+  }
+  ss = block_sum(ss, lds);
+  const float inv = rsqrtf(ss / (float)H + eps);
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = (i * ROW_THREADS + threadIdx.x) * 8;
+    if (c < H) {
+      const f16x8 wv = ld8(w + c);
+      f16x8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = (f16)(v[i][e] * inv * (float)wv[e]);
+      st8(y + (size_t)row * H + c, o);
+    }
+  }
+}
+
+__global__ __launch_bounds__(ROW_THREADS) void silu_mul_kernel(f16* __restrict__ out, const f16* __restrict__ gate,
+                                                               const f16* __restrict__ up, int ld, int I) {
+  const int row = blockIdx.y;
+  const int c = (blockIdx.x * ROW_THREADS + threadIdx.x) * 8;
+  if (c >= I) return;
+  const f16x8 g = ld8(gate + (size_t)row * ld + c);
+  const f16x8 u = ld8(up + (size_t)row * ld + c);
+  f16x8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float gf = (float)g[e];
+    o[e] = (f16)(gf / (1.f + expf(-gf)) * (float)u[e]);
+  }
+  st8(out + (size_t)row * I + c, o);
+}
+
+template <typename OT>
+__global__ __launch_bounds__(ROW_THREADS) void embed_kernel(OT* __restrict__ out, const f16* __restrict__ table,
+                                                            const int32_t* __restrict__ ids, int H, int V) {
+  const int row = blockIdx.x;
+  const int id = ids[row];
+  const bool ok = id >= 0 && id < V;
+  for (int c = threadIdx.x * 8; c < H; c += ROW_THREADS * 8) {
+    f16x8 t = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    if (ok) t = ld8(table + (size_t)id * H + c);
+    if constexpr (sizeof(OT) == 2) {
+      st8((f16*)out + (size_t)row * H + c, t);
+    } else {
+      float* o = (float*)out + (size_t)row * H + c;
+      *reinterpret_cast<f32x4*>(o) = f32x4{(float)t[0], (float)t[1], (float)t[2], (float)t[3]};
+      *reinterpret_cast<f32x4*>(o + 4) = f32x4{(float)t[4], (float)t[5], (float)t[6], (float)t[7]};
+    }
+  }
+}
+
+// (value, index) maximum with the lowest index winning ties; NaN never wins.
+__device__ __forceinline__ void amax_merge(float& v, int& i, float ov, int oi) {
+  if (ov > v || (ov == v && oi < i)) {
+    v = ov;
+    i = oi;
+  }
+}
+
+__global__ __launch_bounds__(ROW_THREADS) void argmax_kernel(int32_t* __restrict__ ids, const float* __restrict__ logits, int V) {
+  __shared__ float lv[ROW_THREADS / WAVE];
+  __shared__ int li[ROW_THREADS / WAVE];
+  const int row = blockIdx.x;
+  const float* p = logits + (size_t)row * V;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int c = threadIdx.x; c < V; c += ROW_THREADS) amax_merge(bv, bi, p[c], c);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, WAVE);
+    const int oi = __shfl_xor(bi, o, WAVE);
+    amax_merge(bv, bi, ov, oi);
+  }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) {
+    lv[wave] = bv;
+    li[wave] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < ROW_THREADS / WAVE; ++w) amax_merge(bv, bi, lv[w], li[w]);
+    ids[row] = bi == 0x7fffffff ? 0 : bi;
+  }
+}
+
+}  // namespace
+
+extern "C" int mlora_rmsnorm(void* y, const void* x, int x_dtype, const void* w, float eps, int T, int H, void* stream) {
+  MLORA_CHECK(y && x && w, MLORA_ERR_INVALID, "rmsnorm: null pointer");
+  MLORA_CHECK(T >= 0 && H > 0 && H % 8 == 0 && H <= 16384, MLORA_ERR_UNSUPPORTED, "rmsnorm: need H %% 8 == 0, H <= 16384 (T=%d H=%d)", T, H);
+  MLORA_CHECK(x_dtype == MLORA_F16 || x_dtype == MLORA_F32, MLORA_ERR_INVALID, "rmsnorm: bad x_dtype %d", x_dtype);
+  if (T == 0) return MLORA_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const int vpt = ceil_div(H, ROW_THREADS * 8);
+#define MLORA_RMS(XT, VPT) \
+  hipLaunchKernelGGL((rmsnorm_kernel<XT, VPT>), dim3(T), dim3(ROW_THREADS), 0, s, (f16*)y, (const XT*)x, (const f16*)w, eps, H)
+  if (x_dtype == MLORA_F16) {
+    if (vpt <= 2) MLORA_RMS(f16, 2);
+    else if (vpt <= 4) MLORA_RMS(f16, 4);
+    else MLORA_RMS(f16, 8);
+  } else {
+    if (vpt <= 2) MLORA_RMS(float, 2);
+    else if (vpt <= 4) MLORA_RMS(float, 4);
+    else MLORA_RMS(float, 8);
+  }
+#undef MLORA_RMS
+  return mlora_launch_status("rmsnorm");
+}
+
+extern "C" int mlora_silu_mul(void* out, const void* gate, const void* up, int ld, int T, int I, void* stream) {
+  MLORA_CHECK(out && gate && up, MLORA_ERR_INVALID, "silu_mul: null pointer");
+  MLORA_CHECK(T >= 0 && I > 0 && I % 8 == 0 && ld >= I && ld % 8 == 0, MLORA_ERR_UNSUPPORTED, "silu_mul: need I %% 8 == 0, ld >= I, ld %% 8 == 0 (T=%d I=%d ld=%d)", T, I, ld);
+  MLORA_CHECK(T <= 65535, MLORA_ERR_UNSUPPORTED, "silu_mul: T=%d exceeds 65535", T);
+  if (T == 0) return MLORA_OK;
+  hipLaunchKernelGGL(silu_mul_kernel, dim3(ceil_div(I, ROW_THREADS * 8), T), dim3(ROW_THREADS), 0, (hipStream_t)stream,
+                     (f16*)out, (const f16*)gate, (const f16*)up, ld, I);
+  return mlora_launch_status("silu_mul");
+}
+
+extern "C" int mlora_embed(void* out, int out_dtype, const void* table, const int32_t* ids, int T, int H, int V, void* stream) {
+  MLORA_CHECK(out && table && ids, MLORA_ERR_INVALID, "embed: null pointer");
+  MLORA_CHECK(T >= 0 && H > 0 && H % 8 == 0 && V > 0, MLORA_ERR_UNSUPPORTED, "embed: need H %% 8 == 0 (T=%d H=%d V=%d)", T, H, V);
+  MLORA_CHECK(out_dtype == MLORA_F16 || out_dtype == MLORA_F32, MLORA_ERR_INVALID, "embed: bad out_dtype %d", out_dtype);
+  if (T == 0) return MLORA_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (out_dtype == MLORA_F16) hipLaunchKernelGGL(embed_kernel<f16>, dim3(T), dim3(ROW_THREADS), 0, s, (f16*)out, (const f16*)table, ids, H, V);
+  else hipLaunchKernelGGL(embed_kernel<float>, dim3(T), dim3(ROW_THREADS), 0, s, (float*)out, (const f16*)table, ids, H, V);
+  return mlora_launch_status("embed");
+}
+
+extern "C" int mlora_argmax(int32_t* ids, const float* logits, int B, int V, void* stream) {
+  MLORA_CHECK(ids && logits, MLORA_ERR_INVALID, "argmax: null pointer");
+  MLORA_CHECK(B >= 0 && V > 0, MLORA_ERR_INVALID, "argmax: bad shape B=%d V=%d", B, V);
+  if (B == 0) return MLORA_OK;
+  hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(ROW_THREADS), 0, (hipStream_t)stream, ids, logits, V);
+  return mlora_launch_status("argmax");
+}

@@ -1,0 +1,184 @@
+"""Operator surface over the C ABI: torch tensors supply device memory and the stream, nothing else.
+
+Each function validates dtypes/contiguity on the host, hands raw pointers to libmlora_hip.so and
+enqueues on torch's current stream.  None of them has a CPU path.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import F16, F32, STORE, ACCUMULATE, PAGE_SIZE, check, lib
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, dtype=None, name="tensor") -> int:
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (no CPU path)")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    return t.data_ptr()
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.float16:
+        return F16
+    if t.dtype == torch.float32:
+        return F32
+    raise TypeError(f"expected float16 or float32, got {t.dtype}")
+
+
+def gather_mm_workspace(T: int, K: int, r: int, device) -> torch.Tensor:
+    n = lib().mlora_gather_mm_workspace_bytes(T, K, r)
+    return torch.empty(max(n, 16) // 4, dtype=torch.float32, device=device)
+
+
+def gather_mm(y, x, A, B, tok_adapter, scaling: float, workspace=None):
+    """y[t] += scaling * B[id_t] @ (A[id_t] @ x[t]) in place.  y [T,N] f16|f32, x [T,K] f16,
+    A [n_ad,r,K] f16, B [n_ad,N,r] f16, tok_adapter [T] int32 (-1 = no adapter)."""
+    T, K = x.shape
+    n_ad, r, K2 = A.shape
+    N = B.shape[1]
+    if K2 != K or B.shape != (n_ad, N, r) or y.shape != (T, N) or tok_adapter.shape != (T,):
+        raise ValueError(f"gather_mm: inconsistent shapes y{tuple(y.shape)} x{tuple(x.shape)} A{tuple(A.shape)} "
+                         f"B{tuple(B.shape)} ids{tuple(tok_adapter.shape)}")
+    if workspace is None:
+        workspace = gather_mm_workspace(T, K, r, x.device)
+    check(lib().mlora_gather_mm(_dev(y, None, "y"), _dt(y), _dev(x, torch.float16, "x"), _dev(A, torch.float16, "A"),
+                                _dev(B, torch.float16, "B"), _dev(tok_adapter, torch.int32, "tok_adapter"),
+                                float(scaling), T, K, N, r, n_ad, _dev(workspace, torch.float32, "workspace"),
+                                workspace.numel() * 4, _stream()))
+    return y
+
+
+def lora_shrink(v_part, x, A, tok_adapter):
+    T, K = x.shape
+    n_ad, r, _ = A.shape
+    check(lib().mlora_lora_shrink(_dev(v_part, torch.float32), _dev(x, torch.float16), _dev(A, torch.float16),
+                                  _dev(tok_adapter, torch.int32), T, K, r, n_ad, _stream()))
+    return v_part
+
+
+def lora_expand(y, v_part, B, tok_adapter, scaling: float, K: int):
+    T, N = y.shape
+    n_ad, _, r = B.shape
+    check(lib().mlora_lora_expand(_dev(y), _dt(y), _dev(v_part, torch.float32), _dev(B, torch.float16),
+                                  _dev(tok_adapter, torch.int32), float(scaling), T, K, N, r, n_ad, _stream()))
+    return y
+
+
+def write_tensor_part(X, Y, ids, out=None):
+    """Z = X; Z[ids[a]] = Y[a] over the leading dimension."""
+    Z = torch.empty_like(X) if out is None else out
+    B, A = X.shape[0], Y.shape[0]
+    PH = X[0].numel() if B else (Y[0].numel() if A else 8)
+    check(lib().mlora_write_tensor_part(_dev(Z, torch.float16), _dev(X, torch.float16), _dev(Y, torch.float16),
+                                        _dev(ids, torch.int32), B, A, PH, _stream()))
+    return Z
+
+
+def linear(x, W, out=None, out_dtype=torch.float16, accumulate=False, kernel="auto"):
+    """y (=|+=) x @ W.T.  x [T,K] f16 (row stride may exceed K), W [N,K] f16.
+    accumulate=True adds into the fp32 tensor `out`."""
+    T, K = x.shape
+    N, K2 = W.shape
+    if K2 != K:
+        raise ValueError(f"linear: x{tuple(x.shape)} vs W{tuple(W.shape)}")
+    if not x.is_cuda or x.dtype != torch.float16 or x.stride(1) != 1:
+        raise ValueError("linear: x must be a GPU fp16 tensor with unit inner stride")
+    ldx = x.stride(0) if T > 1 else max(K, x.stride(0))
+    if out is None:
+        if accumulate:
+            raise ValueError("linear: accumulate needs out")
+        out = torch.empty((T, N), dtype=out_dtype, device=x.device)
+    if out.shape != (T, N):
+        raise ValueError(f"linear: out{tuple(out.shape)} expected {(T, N)}")
+    fn = {"auto": lib().mlora_linear, "gemv": lib().mlora_gemv, "gemm": lib().mlora_gemm}[kernel]
+    check(fn(_dev(out), _dt(out), ACCUMULATE if accumulate else STORE, x.data_ptr(), ldx,
+             _dev(W, torch.float16, "W"), T, K, N, _stream()))
+    return out
+
+
+def rmsnorm(x, w, eps: float, out=None):
+    T, H = x.shape
+    if out is None:
+        out = torch.empty((T, H), dtype=torch.float16, device=x.device)
+    check(lib().mlora_rmsnorm(_dev(out, torch.float16), _dev(x), _dt(x), _dev(w, torch.float16), float(eps), T, H, _stream()))
+    return out
+
+
+def silu_mul(gate_up, out=None):
+    """gate_up [T, 2I] (gate columns first) -> silu(gate) * up [T, I]."""
+    T, I2 = gate_up.shape
+    I = I2 // 2
+    if out is None:
+        out = torch.empty((T, I), dtype=torch.float16, device=gate_up.device)
+    p = _dev(gate_up, torch.float16)
+    check(lib().mlora_silu_mul(_dev(out, torch.float16), p, p + I * 2, I2, T, I, _stream()))
+    return out
+
+
+def silu_mul_split(gate, up, out=None):
+    T, I = gate.shape
+    if out is None:
+        out = torch.empty((T, I), dtype=torch.float16, device=gate.device)
+    check(lib().mlora_silu_mul(_dev(out, torch.float16), _dev(gate, torch.float16), _dev(up, torch.float16), I, T, I, _stream()))
+    return out
+
+
+def embed(table, ids, out_dtype=torch.float32, out=None):
+    T = ids.numel()
+    V, H = table.shape
+    if out is None:
+        out = torch.empty((T, H), dtype=out_dtype, device=table.device)
+    check(lib().mlora_embed(_dev(out), _dt(out), _dev(table, torch.float16), _dev(ids, torch.int32), T, H, V, _stream()))
+    return out
+
+
+def argmax(logits, out=None):
+    B, V = logits.shape
+    if out is None:
+        out = torch.empty((B,), dtype=torch.int32, device=logits.device)
+    check(lib().mlora_argmax(_dev(out, torch.int32), _dev(logits, torch.float32), B, V, _stream()))
+    return out
+
+
+def rope_kv_append(qkv, k_cache, v_cache, block_table, tok_seq, tok_pos, rope_cos, rope_sin, Hq, Hkv, D):
+    """qkv [T, Hq+2Hkv, D] f16 (q rotated in place); k_cache [n_pages,Hkv,16,D], v_cache [n_pages,Hkv,D,16]."""
+    T = qkv.shape[0]
+    n_pages = k_cache.shape[0]
+    n_seq, max_blocks = block_table.shape
+    max_pos = rope_cos.shape[0]
+    check(lib().mlora_rope_kv_append(_dev(qkv, torch.float16), _dev(k_cache, torch.float16), _dev(v_cache, torch.float16),
+                                     _dev(block_table, torch.int32), max_blocks, _dev(tok_seq, torch.int32),
+                                     _dev(tok_pos, torch.int32), _dev(rope_cos, torch.float32), _dev(rope_sin, torch.float32),
+                                     max_pos, T, Hq, Hkv, D, n_pages, n_seq, _stream()))
+
+
+def paged_attn_decode(qkv, k_cache, v_cache, block_table, seq_ids, ctx_len, Hq, Hkv, D, out=None):
+    B = qkv.shape[0]
+    n_seq, max_blocks = block_table.shape
+    if out is None:
+        out = torch.empty((B, Hq * D), dtype=torch.float16, device=qkv.device)
+    check(lib().mlora_paged_attn_decode(_dev(out, torch.float16), _dev(qkv, torch.float16), _dev(k_cache, torch.float16),
+                                        _dev(v_cache, torch.float16), _dev(block_table, torch.int32), max_blocks,
+                                        _dev(seq_ids, torch.int32), _dev(ctx_len, torch.int32), B, Hq, Hkv, D,
+                                        k_cache.shape[0], n_seq, _stream()))
+    return out
+
+
+def paged_attn_prefill(qkv, k_cache, v_cache, block_table, tok_seq, tok_pos, Hq, Hkv, D, out=None):
+    T = qkv.shape[0]
+    n_seq, max_blocks = block_table.shape
+    if out is None:
+        out = torch.empty((T, Hq * D), dtype=torch.float16, device=qkv.device)
+    check(lib().mlora_paged_attn_prefill(_dev(out, torch.float16), _dev(qkv, torch.float16), _dev(k_cache, torch.float16),
+                                         _dev(v_cache, torch.float16), _dev(block_table, torch.int32), max_blocks,
+                                         _dev(tok_seq, torch.int32), _dev(tok_pos, torch.int32), T, Hq, Hkv, D,
+                                         k_cache.shape[0], n_seq, _stream()))
+    return out
