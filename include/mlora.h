@@ -100,6 +100,23 @@ int mlora_gemm(void* y, int y_dtype, int mode, const void* x, int ldx, const voi
 int mlora_linear(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W,
                  int T, int K, int N, void* stream);
 
+/* Fragment-ordered weight layout for the same linears.  The reference re-lays out weights once at load
+ * time as well (stack + transpose, tvm/llama_auto_batcher/compile_tvm.py:296-314); here the one-time step
+ * stores W in the order the matrix cores consume it,
+ *     Wp[n/16][k/32][(k%32)/8][n%16][k%8]      (rows padded with zeros to a multiple of 16)
+ * so every (16 rows x 32 k) operand fragment is one contiguous 1 KiB block and a wave streams
+ * consecutive blocks.  mlora_pack_weight writes mlora_packed_weight_elems(N, K) fp16 elements to dst
+ * (dst must not alias src).  The *_packed entry points take Wp in place of W; everything else is as
+ * for mlora_gemv / mlora_gemm / mlora_linear. */
+size_t mlora_packed_weight_elems(int N, int K);
+int mlora_pack_weight(void* dst, const void* src, int N, int K, void* stream);
+int mlora_gemv_packed(void* y, int y_dtype, int mode, const void* x, int ldx, const void* Wp,
+                      int T, int K, int N, void* stream);
+int mlora_gemm_packed(void* y, int y_dtype, int mode, const void* x, int ldx, const void* Wp,
+                      int T, int K, int N, void* stream);
+int mlora_linear_packed(void* y, int y_dtype, int mode, const void* x, int ldx, const void* Wp,
+                        int T, int K, int N, void* stream);
+
 /* y[t, :] = f16( x[t, :] * rsqrt(mean(x[t, :]^2) + eps) * w )   row-wise, statistics in fp32.
  * Replaces: nn.RMSNorm(hidden, -1, eps, bias=False) (llama_for_causal_lm.py:76-77,93).
  * x [T, H] f16 or f32 (x_dtype), w [H] f16, y [T, H] f16.  H % 8 == 0, H <= 16384. */

@@ -28,6 +28,11 @@ SIGNATURES = {
     "mlora_gemv": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
     "mlora_gemm": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
     "mlora_linear": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
+    "mlora_packed_weight_elems": (_z, [_i, _i]),
+    "mlora_pack_weight": (_i, [_p, _p, _i, _i, _p]),
+    "mlora_gemv_packed": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
+    "mlora_gemm_packed": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
+    "mlora_linear_packed": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
     "mlora_rmsnorm": (_i, [_p, _p, _i, _p, _f, _i, _i, _p]),
     "mlora_silu_mul": (_i, [_p, _p, _p, _i, _i, _i, _p]),
     "mlora_embed": (_i, [_p, _i, _p, _p, _i, _i, _i, _p]),

@@ -16,7 +16,7 @@ enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2 };
 
 constexpr int WT = 4;   // 16-wide MFMA tiles per wave along N and along T
 
-template <int OUT>
+template <int OUT, bool PACKED>
 __global__ __launch_bounds__(256) void gemm_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx,
                                                    const f16* __restrict__ W, int T, int K, int N) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -25,13 +25,21 @@ __global__ __launch_bounds__(256) void gemm_kernel(void* __restrict__ yv, const 
   const int t0 = blockIdx.y * 128 + (wave >> 1) * 64;
   if (n0 >= N || t0 >= T) return;
 
+  constexpr int WSTEP = PACKED ? 512 : 32;   // elements between consecutive k-steps of one fragment stream
+  const int tiles = (N + 15) / 16;
   const f16* wp[WT];
   const f16* xp[WT];
 #pragma unroll
   for (int i = 0; i < WT; ++i) {
-    int n = n0 + i * 16 + r16;
-    n = n < N ? n : N - 1;
-    wp[i] = W + (size_t)n * K + kg * 8;
+    if constexpr (PACKED) {
+      int nt = n0 / 16 + i;
+      nt = nt < tiles ? nt : tiles - 1;
+      wp[i] = W + ((size_t)nt * (K / 32)) * 512 + lane * 8;
+    } else {
+      int n = n0 + i * 16 + r16;
+      n = n < N ? n : N - 1;
+      wp[i] = W + (size_t)n * K + kg * 8;
+    }
     int t = t0 + i * 16 + r16;
     t = t < T ? t : T - 1;
     xp[i] = x + (size_t)t * ldx + kg * 8;
@@ -48,13 +56,14 @@ __global__ __launch_bounds__(256) void gemm_kernel(void* __restrict__ yv, const 
     a[i] = ld8(wp[i]);
     b[i] = ld8(xp[i]);
   }
-  for (int k = 32; k <= K; k += 32) {
+  const int KB = K / 32;
+  for (int ks = 1; ks <= KB; ++ks) {
     f16x8 an[WT], bn[WT];
-    const int kc = k < K ? k : 0;   // the last prefetch wraps to a valid address and is discarded
+    const int kc = ks < KB ? ks : 0;   // the last prefetch wraps to a valid address and is discarded
 #pragma unroll
     for (int i = 0; i < WT; ++i) {
-      an[i] = ld8(wp[i] + kc);
-      bn[i] = ld8(xp[i] + kc);
+      an[i] = ld8(wp[i] + (size_t)kc * WSTEP);
+      bn[i] = ld8(xp[i] + kc * 32);
     }
 #pragma unroll
     for (int i = 0; i < WT; ++i)
@@ -90,25 +99,42 @@ __global__ __launch_bounds__(256) void gemm_kernel(void* __restrict__ yv, const 
   }
 }
 
-}  // namespace
-
-extern "C" int mlora_gemm(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K, int N,
-                          void* stream) {
-  if (int e = mlora_check_linear("gemm", y, y_dtype, mode, x, ldx, W, T, K, N)) return e;
+template <bool PACKED>
+int gemm_dispatch(const char* who, void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K,
+                  int N, void* stream) {
+  if (int e = mlora_check_linear(who, y, y_dtype, mode, x, ldx, W, T, K, N)) return e;
   if (T == 0) return MLORA_OK;
-  MLORA_CHECK(ceil_div(T, 128) <= 65535, MLORA_ERR_UNSUPPORTED, "gemm: T=%d too large", T);
+  MLORA_CHECK(ceil_div(T, 128) <= 65535, MLORA_ERR_UNSUPPORTED, "%s: T=%d too large", who, T);
   const dim3 grid(ceil_div(N, 128), ceil_div(T, 128)), block(256);
   hipStream_t s = (hipStream_t)stream;
   const f16* xp = (const f16*)x;
   const f16* Wp = (const f16*)W;
-  if (mode == MLORA_ACCUMULATE) hipLaunchKernelGGL(gemm_kernel<OUT_ACC_F32>, grid, block, 0, s, y, xp, ldx, Wp, T, K, N);
-  else if (y_dtype == MLORA_F32) hipLaunchKernelGGL(gemm_kernel<OUT_F32>, grid, block, 0, s, y, xp, ldx, Wp, T, K, N);
-  else hipLaunchKernelGGL(gemm_kernel<OUT_F16>, grid, block, 0, s, y, xp, ldx, Wp, T, K, N);
-  return mlora_launch_status("gemm");
+  if (mode == MLORA_ACCUMULATE) hipLaunchKernelGGL((gemm_kernel<OUT_ACC_F32, PACKED>), grid, block, 0, s, y, xp, ldx, Wp, T, K, N);
+  else if (y_dtype == MLORA_F32) hipLaunchKernelGGL((gemm_kernel<OUT_F32, PACKED>), grid, block, 0, s, y, xp, ldx, Wp, T, K, N);
+  else hipLaunchKernelGGL((gemm_kernel<OUT_F16, PACKED>), grid, block, 0, s, y, xp, ldx, Wp, T, K, N);
+  return mlora_launch_status(who);
+}
+
+}  // namespace
+
+extern "C" int mlora_gemm(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K, int N,
+                          void* stream) {
+  return gemm_dispatch<false>("gemm", y, y_dtype, mode, x, ldx, W, T, K, N, stream);
+}
+
+extern "C" int mlora_gemm_packed(void* y, int y_dtype, int mode, const void* x, int ldx, const void* Wp, int T, int K,
+                                 int N, void* stream) {
+  return gemm_dispatch<true>("gemm_packed", y, y_dtype, mode, x, ldx, Wp, T, K, N, stream);
 }
 
 extern "C" int mlora_linear(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K, int N,
                             void* stream) {
   if (T <= 64) return mlora_gemv(y, y_dtype, mode, x, ldx, W, T, K, N, stream);
   return mlora_gemm(y, y_dtype, mode, x, ldx, W, T, K, N, stream);
+}
+
+extern "C" int mlora_linear_packed(void* y, int y_dtype, int mode, const void* x, int ldx, const void* Wp, int T, int K,
+                                   int N, void* stream) {
+  if (T <= 64) return mlora_gemv_packed(y, y_dtype, mode, x, ldx, Wp, T, K, N, stream);
+  return mlora_gemm_packed(y, y_dtype, mode, x, ldx, Wp, T, K, N, stream);
 }

@@ -1,23 +1,29 @@
 // Decode-time base linear for gfx950:  y[T, N] (=|+=) x[T, K] . W[N, K]^T  with T <= 64.
 //
 // The weight matrix is read exactly once, straight from HBM into MFMA operand registers: for
-// v_mfma_f32_16x16x32_f16 a lane holds 8 consecutive k of one row, so a wave-wide 16-byte load covers
-// 16 weight rows x 64 contiguous bytes.  The token block x (T x K fp16, L2-resident) is the other
-// operand, so one weight fragment is applied to 16 tokens per MFMA and the kernel stays HBM-bound
-// (32 tokens need 64 flop per weight element - beyond the vector ALUs, well inside the matrix cores).
-// A workgroup of 8 waves owns 16*NT rows of W and splits K eight ways; partial tiles are summed in a
-// fixed order through LDS, so results do not depend on scheduling.
+// v_mfma_f32_16x16x32_f16 a lane holds 8 consecutive k of one row.  The token block x (T x K fp16,
+// L2-resident) is the other operand, so one weight fragment is applied to 16 tokens per MFMA and the
+// kernel stays HBM-bound (32 tokens need 64 flop per weight element - beyond the vector ALUs, well
+// inside the matrix cores).  A workgroup of 8 waves owns 16*NT rows of W and splits K eight ways;
+// partial tiles are summed in a fixed order through LDS, so results do not depend on scheduling.
+//
+// Two weight layouts:
+//   row-major W[N, K]  - a wave-wide 16-byte load covers 16 rows x 64 bytes (one DRAM page each);
+//   packed (mlora_pack_weight) - fragments are stored in operand order,
+//       Wp[n/16][k/32][(k%32)/8][n%16][k%8],
+//     so the fragment of (16 rows, 32 k) is one contiguous 1 KiB block and a wave streams consecutive
+//     blocks: every load is a full DRAM page and consecutive k-steps are consecutive addresses.
 #include "common.h"
 
 namespace {
 
 constexpr int GEMV_WAVES = 8;
 constexpr int KSTEP = 32;   // k per MFMA
-constexpr int UNROLL = 4;   // k-steps in flight per wave
+constexpr int PIPE = 4;     // k-steps in flight per wave
 
 enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2 };
 
-template <int NT, int TT, int OUT>
+template <int NT, int TT, int OUT, bool PACKED>
 __global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx,
                                                                 const f16* __restrict__ W, int T, int K, int N) {
   __shared__ f32x4 red[GEMV_WAVES][NT * TT][WAVE];
@@ -26,14 +32,20 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(void* __restrict
   const int r16 = lane & 15;
   const int kg = lane >> 4;
   const int n0 = blockIdx.x * (16 * NT);
+  const int KB = K / KSTEP;
+  constexpr int WSTEP = PACKED ? 512 : KSTEP;   // elements between consecutive k-steps of one fragment stream
 
   const f16* wp[NT];
   const f16* xp[TT];
 #pragma unroll
   for (int i = 0; i < NT; ++i) {
-    int n = n0 + i * 16 + r16;
-    n = n < N ? n : N - 1;
-    wp[i] = W + (size_t)n * K + kg * 8;
+    if constexpr (PACKED) {
+      wp[i] = W + ((size_t)(blockIdx.x * NT + i) * KB) * 512 + lane * 8;
+    } else {
+      int n = n0 + i * 16 + r16;
+      n = n < N ? n : N - 1;
+      wp[i] = W + (size_t)n * K + kg * 8;
+    }
   }
 #pragma unroll
   for (int j = 0; j < TT; ++j) {
@@ -48,29 +60,32 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(void* __restrict
 #pragma unroll
     for (int j = 0; j < TT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // wave w takes k-steps w, w + 8, w + 16, ...; UNROLL of them are in flight at once
-  const int stride = GEMV_WAVES * KSTEP;
-  for (int k = wave * KSTEP; k < K; k += stride * UNROLL) {
-    f16x8 a[UNROLL][NT], b[UNROLL][TT];
+  // wave w takes k-steps w, w + 8, w + 16, ...; stage s of this wave is k-step w + 8 s.
+  // PIPE stages are always in flight: each buffer is refilled right after it is consumed.
+  const int S = (KB - wave + GEMV_WAVES - 1) / GEMV_WAVES;
+  f16x8 a[PIPE][NT], b[PIPE][TT];
+  auto load_stage = [&](int u, int s) {
+    const bool in = s < S;
+    const int ks = in ? wave + GEMV_WAVES * s : 0;
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int ku = k + u * stride;
-      const bool in = ku < K;
-      const int kc = in ? ku : 0;
-#pragma unroll
-      for (int i = 0; i < NT; ++i) {
-        a[u][i] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(wp[i] + kc));
-        if (!in) a[u][i] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      }
-#pragma unroll
-      for (int j = 0; j < TT; ++j) b[u][j] = ld8(xp[j] + kc);
+    for (int i = 0; i < NT; ++i) {
+      a[u][i] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(wp[i] + (size_t)ks * WSTEP));
+      if (!in) a[u][i] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
+    for (int j = 0; j < TT; ++j) b[u][j] = ld8(xp[j] + ks * KSTEP);
+  };
+#pragma unroll
+  for (int u = 0; u < PIPE; ++u) load_stage(u, u);
+  for (int s0 = 0; s0 < S; s0 += PIPE) {
+#pragma unroll
+    for (int u = 0; u < PIPE; ++u) {
 #pragma unroll
       for (int i = 0; i < NT; ++i)
 #pragma unroll
         for (int j = 0; j < TT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][i], b[u][j], acc[i][j], 0, 0, 0);
+      load_stage(u, s0 + u + PIPE);
+    }
   }
 
 #pragma unroll
@@ -102,12 +117,51 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(void* __restrict
   }
 }
 
-template <int NT, int TT>
+// one thread per 16-byte chunk of the packed array
+__global__ __launch_bounds__(256) void pack_weight_kernel(f16* __restrict__ dst, const f16* __restrict__ src, int N, int K,
+                                                          size_t chunks) {
+  const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= chunks) return;
+  const int KB = K / KSTEP;
+  const int row = c & 15;
+  const int g = (c >> 4) & 3;
+  const size_t blk = c >> 6;
+  const int ks = blk % KB;
+  const size_t nt = blk / KB;
+  const size_t n = nt * 16 + row;
+  f16x8 v = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  if (n < (size_t)N) v = ld8(src + n * K + ks * KSTEP + g * 8);
+  st8(dst + c * 8, v);
+}
+
+template <int NT, int TT, bool PACKED>
 void launch_gemv(void* y, int out, const f16* x, int ldx, const f16* W, int T, int K, int N, hipStream_t s) {
   const dim3 grid(ceil_div(N, 16 * NT)), block(GEMV_WAVES * WAVE);
-  if (out == OUT_F16) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F16>), grid, block, 0, s, y, x, ldx, W, T, K, N);
-  else if (out == OUT_F32) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F32>), grid, block, 0, s, y, x, ldx, W, T, K, N);
-  else hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_ACC_F32>), grid, block, 0, s, y, x, ldx, W, T, K, N);
+  if (out == OUT_F16) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F16, PACKED>), grid, block, 0, s, y, x, ldx, W, T, K, N);
+  else if (out == OUT_F32) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F32, PACKED>), grid, block, 0, s, y, x, ldx, W, T, K, N);
+  else hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_ACC_F32, PACKED>), grid, block, 0, s, y, x, ldx, W, T, K, N);
+}
+
+template <bool PACKED>
+int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K, int N, void* stream) {
+  const int out = mode == MLORA_ACCUMULATE ? OUT_ACC_F32 : (y_dtype == MLORA_F32 ? OUT_F32 : OUT_F16);
+  hipStream_t s = (hipStream_t)stream;
+  const f16* xp = (const f16*)x;
+  const f16* Wp = (const f16*)W;
+  // two 16-row tiles per wave once there are enough rows to give every CU a workgroup; the packed
+  // layout pads N to a multiple of 16, so an odd tile count keeps one tile per wave
+  const int tiles = ceil_div(N, 16);
+  const bool wide = tiles >= 512 && (!PACKED || tiles % 2 == 0);
+  if (T <= 16) {
+    if (wide) launch_gemv<2, 1, PACKED>(y, out, xp, ldx, Wp, T, K, N, s);
+    else launch_gemv<1, 1, PACKED>(y, out, xp, ldx, Wp, T, K, N, s);
+  } else if (T <= 32) {
+    if (wide) launch_gemv<2, 2, PACKED>(y, out, xp, ldx, Wp, T, K, N, s);
+    else launch_gemv<1, 2, PACKED>(y, out, xp, ldx, Wp, T, K, N, s);
+  } else {
+    launch_gemv<1, 4, PACKED>(y, out, xp, ldx, Wp, T, K, N, s);
+  }
+  return mlora_launch_status("gemv");
 }
 
 }  // namespace
@@ -129,20 +183,28 @@ extern "C" int mlora_gemv(void* y, int y_dtype, int mode, const void* x, int ldx
   if (int e = mlora_check_linear("gemv", y, y_dtype, mode, x, ldx, W, T, K, N)) return e;
   MLORA_CHECK(T <= 64, MLORA_ERR_UNSUPPORTED, "gemv: T=%d exceeds 64 (use mlora_gemm)", T);
   if (T == 0) return MLORA_OK;
-  const int out = mode == MLORA_ACCUMULATE ? OUT_ACC_F32 : (y_dtype == MLORA_F32 ? OUT_F32 : OUT_F16);
-  hipStream_t s = (hipStream_t)stream;
-  const f16* xp = (const f16*)x;
-  const f16* Wp = (const f16*)W;
-  // two 16-row tiles per wave once there are enough rows to give every CU two workgroups
-  const bool wide = N >= 32 * 512;
-  if (T <= 16) {
-    if (wide) launch_gemv<2, 1>(y, out, xp, ldx, Wp, T, K, N, s);
-    else launch_gemv<1, 1>(y, out, xp, ldx, Wp, T, K, N, s);
-  } else if (T <= 32) {
-    if (wide) launch_gemv<2, 2>(y, out, xp, ldx, Wp, T, K, N, s);
-    else launch_gemv<1, 2>(y, out, xp, ldx, Wp, T, K, N, s);
-  } else {
-    launch_gemv<1, 4>(y, out, xp, ldx, Wp, T, K, N, s);
-  }
-  return mlora_launch_status("gemv");
+  return gemv_dispatch<false>(y, y_dtype, mode, x, ldx, W, T, K, N, stream);
+}
+
+extern "C" int mlora_gemv_packed(void* y, int y_dtype, int mode, const void* x, int ldx, const void* Wp, int T, int K,
+                                 int N, void* stream) {
+  if (int e = mlora_check_linear("gemv_packed", y, y_dtype, mode, x, ldx, Wp, T, K, N)) return e;
+  MLORA_CHECK(T <= 64, MLORA_ERR_UNSUPPORTED, "gemv_packed: T=%d exceeds 64 (use mlora_gemm_packed)", T);
+  if (T == 0) return MLORA_OK;
+  return gemv_dispatch<true>(y, y_dtype, mode, x, ldx, Wp, T, K, N, stream);
+}
+
+extern "C" size_t mlora_packed_weight_elems(int N, int K) {
+  if (N <= 0 || K <= 0) return 0;
+  return (size_t)ceil_div(N, 16) * 16 * (size_t)K;
+}
+
+extern "C" int mlora_pack_weight(void* dst, const void* src, int N, int K, void* stream) {
+  MLORA_CHECK(dst && src && dst != src, MLORA_ERR_INVALID, "pack_weight: null or aliasing pointers");
+  MLORA_CHECK(N > 0 && K > 0 && K % 32 == 0, MLORA_ERR_UNSUPPORTED, "pack_weight: need K %% 32 == 0 (N=%d K=%d)", N, K);
+  const size_t chunks = mlora_packed_weight_elems(N, K) / 8;
+  MLORA_CHECK(chunks / 256 + 1 < 0x7fffffffULL, MLORA_ERR_UNSUPPORTED, "pack_weight: matrix too large");
+  hipLaunchKernelGGL(pack_weight_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, (hipStream_t)stream, (f16*)dst,
+                     (const f16*)src, N, K, chunks);
+  return mlora_launch_status("pack_weight");
 }

@@ -82,10 +82,26 @@ def write_tensor_part(X, Y, ids, out=None):
     return Z
 
 
+class PackedWeight:
+    """A [N, K] fp16 weight stored in matrix-core fragment order (see mlora_pack_weight)."""
+
+    def __init__(self, W: torch.Tensor):
+        N, K = W.shape
+        self.N, self.K = N, K
+        n = lib().mlora_packed_weight_elems(N, K)
+        self.data = torch.empty(n, dtype=torch.float16, device=W.device)
+        check(lib().mlora_pack_weight(_dev(self.data), _dev(W, torch.float16, "W"), N, K, _stream()))
+
+    @property
+    def shape(self):
+        return (self.N, self.K)
+
+
 def linear(x, W, out=None, out_dtype=torch.float16, accumulate=False, kernel="auto"):
-    """y (=|+=) x @ W.T.  x [T,K] f16 (row stride may exceed K), W [N,K] f16.
+    """y (=|+=) x @ W.T.  x [T,K] f16 (row stride may exceed K), W [N,K] f16 or a PackedWeight.
     accumulate=True adds into the fp32 tensor `out`."""
     T, K = x.shape
+    packed = isinstance(W, PackedWeight)
     N, K2 = W.shape
     if K2 != K:
         raise ValueError(f"linear: x{tuple(x.shape)} vs W{tuple(W.shape)}")
@@ -98,9 +114,13 @@ def linear(x, W, out=None, out_dtype=torch.float16, accumulate=False, kernel="au
         out = torch.empty((T, N), dtype=out_dtype, device=x.device)
     if out.shape != (T, N):
         raise ValueError(f"linear: out{tuple(out.shape)} expected {(T, N)}")
-    fn = {"auto": lib().mlora_linear, "gemv": lib().mlora_gemv, "gemm": lib().mlora_gemm}[kernel]
-    check(fn(_dev(out), _dt(out), ACCUMULATE if accumulate else STORE, x.data_ptr(), ldx,
-             _dev(W, torch.float16, "W"), T, K, N, _stream()))
+    if packed:
+        fn = {"auto": lib().mlora_linear_packed, "gemv": lib().mlora_gemv_packed, "gemm": lib().mlora_gemm_packed}[kernel]
+        wptr = W.data.data_ptr()
+    else:
+        fn = {"auto": lib().mlora_linear, "gemv": lib().mlora_gemv, "gemm": lib().mlora_gemm}[kernel]
+        wptr = _dev(W, torch.float16, "W")
+    check(fn(_dev(out), _dt(out), ACCUMULATE if accumulate else STORE, x.data_ptr(), ldx, wptr, T, K, N, _stream()))
     return out
 
 

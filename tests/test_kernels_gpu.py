@@ -87,11 +87,14 @@ def test_write_tensor_part(ops):
 @pytest.mark.parametrize("T,K,N", [(32, 4096, 4096), (32, 4096, 12288), (32, 11008, 4096), (32, 4096, 22016),
                                    (64, 4096, 4096), (4, 1024, 3072), (1, 1024, 1024), (17, 2752, 1024), (5, 64, 36)])
 @pytest.mark.parametrize("kernel", ["gemv", "gemm"])
-def test_linear_matches_oracle(ops, synth, T, K, N, kernel):
-    print(f"case linear {kernel} T={T} K={K} N={N}", flush=True)
+@pytest.mark.parametrize("packed", [False, True])
+def test_linear_matches_oracle(ops, synth, T, K, N, kernel, packed):
+    print(f"case linear {kernel} packed={packed} T={T} K={K} N={N}", flush=True)
     x = synth.normal(7, f"lin.x.{T}.{K}", (T, K), 1.0, torch.float16, DEV)
     W = synth.normal(7, f"lin.W.{N}.{K}", (N, K), 0.02, torch.float16, DEV)
     ref = _np(x).astype(np.float64) @ _np(W).astype(np.float64).T
+    if packed:
+        W = ops.PackedWeight(W)
     y16 = ops.linear(x, W, kernel=kernel)
     y32 = ops.linear(x, W, out_dtype=torch.float32, kernel=kernel)
     r0 = synth.normal(7, f"lin.r.{T}.{N}", (T, N), 1.0, torch.float32, DEV)
@@ -103,13 +106,27 @@ def test_linear_matches_oracle(ops, synth, T, K, N, kernel):
     assert max_rel_err(_np(racc), _np(r0) + ref, floor=1e-2) <= 5e-4
 
 
-def test_gemm_large_T(ops, synth):
+@pytest.mark.parametrize("packed", [False, True])
+def test_gemm_large_T(ops, synth, packed):
     T, K, N = 300, 1024, 520
     x = synth.normal(8, "gemm.x", (T, K), 1.0, torch.float16, DEV)
     W = synth.normal(8, "gemm.W", (N, K), 0.02, torch.float16, DEV)
-    y = ops.linear(x, W, out_dtype=torch.float32)
+    y = ops.linear(x, ops.PackedWeight(W) if packed else W, out_dtype=torch.float32)
     torch.cuda.synchronize()
-    assert max_rel_err(_np(y), _np(x).astype(np.float64) @ _np(W).astype(np.float64).T) <= 5e-4
+    assert max_rel_err(_np(y), _np(x).astype(np.float64) @ _np(W).astype(np.float64).T, floor=1e-2) <= 5e-4
+
+
+def test_pack_weight_is_a_permutation(ops, synth):
+    """Bit-exact: every element of W appears at its fragment-order position, padding rows are zero."""
+    N, K = 40, 64
+    W = synth.normal(8, "pack.W", (N, K), 1.0, torch.float16, DEV)
+    P = ops.PackedWeight(W)
+    torch.cuda.synchronize()
+    Wn = _np(W)
+    pad = np.zeros((48, K), np.float32)
+    pad[:N] = Wn
+    exp = pad.reshape(3, 16, K // 32, 4, 8).transpose(0, 2, 3, 1, 4).reshape(-1)
+    assert np.array_equal(_np(P.data), exp)
 
 
 def test_linear_strided_x(ops, synth):
