@@ -56,13 +56,14 @@ const char* mlora_last_error(void);
  *   tvm/custom/write_tensor_part.py:3-20).
  *
  * Layouts (PEFT orientation): x [T, K] f16; A [n_ad, r, K] f16; B [n_ad, N, r] f16;
- *   y [T, N] f16 or f32 (y_dtype); tok_adapter [T] int32.
- * Constraints: r in {8, 16, 32, 64}; K % 8 == 0; N % 8 == 0.
+ *   y [T, N] f16 or f32 (y_dtype) with row stride ldy elements (y may be a column slice of a fused
+ *   projection output); tok_adapter [T] int32.
+ * Constraints: r in {8, 16, 32, 64}; K % 8 == 0; N % 8 == 0; ldy >= N, ldy % 8 == 0.
  * workspace: mlora_gather_mm_workspace_bytes(T, K, r) bytes of device scratch (shrink partials);
  *   contents need not be initialised.
  * ------------------------------------------------------------------------------------------- */
 size_t mlora_gather_mm_workspace_bytes(int T, int K, int r);
-int mlora_gather_mm(void* y, int y_dtype, const void* x, const void* A, const void* B,
+int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, const void* A, const void* B,
                     const int32_t* tok_adapter, float scaling,
                     int T, int K, int N, int r, int n_ad,
                     void* workspace, size_t workspace_bytes, void* stream);
@@ -73,7 +74,7 @@ int mlora_gather_mm(void* y, int y_dtype, const void* x, const void* A, const vo
  * Same layouts and constraints; v_part is the workspace described above. */
 int mlora_lora_shrink(void* v_part, const void* x, const void* A, const int32_t* tok_adapter,
                       int T, int K, int r, int n_ad, void* stream);
-int mlora_lora_expand(void* y, int y_dtype, const void* v_part, const void* B, const int32_t* tok_adapter,
+int mlora_lora_expand(void* y, int y_dtype, int ldy, const void* v_part, const void* B, const int32_t* tok_adapter,
                       float scaling, int T, int K, int N, int r, int n_ad, void* stream);
 
 /* Z = X; Z[ids[a], :] = Y[a, :]  - row scatter of the mixed-adapter-type path.

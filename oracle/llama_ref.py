@@ -232,12 +232,15 @@ def greedy_generate_ref(model, prompts, tok_adapter, max_gen_len, n_pages, page_
     is not EOS and fewer than `max_gen_len` tokens have been produced (`:94-100`); the batch shrinks
     as sequences finish.  `tok_adapter`: dict tag -> per-request adapter ids [B] (-1 = none).
     np.argmax breaks ties towards the lowest index (`:92,137`).
-    Returns a list of B lists of token ids (each of length <= max_gen_len)."""
+    Returns a list of B lists of token ids (each of length <= max_gen_len); with return_logits=True also
+    the top-1 minus top-2 logit margin of every generated token, in the same nesting, and the logit
+    standard deviation of each token's row (the scale against which a margin is small or large)."""
     B = len(prompts)
     max_pos = max(len(p) for p in prompts) + max_gen_len + 1
     kv = model.new_cache(n_pages, page_size, max_pos, free_pages)
     outputs = {}
-    margins = []
+    margins = {sid: [] for sid in range(B)}
+    scales = {sid: [] for sid in range(B)}
     for sid in range(B):
         kv.add_sequence(sid)
         n = len(prompts[sid])
@@ -246,7 +249,8 @@ def greedy_generate_ref(model, prompts, tok_adapter, max_gen_len, n_pages, page_
         logits = model.forward(np.asarray(prompts[sid]), kv, ta, logits_rows=[n - 1])
         kv.end_forward()
         outputs[sid] = [int(np.argmax(logits[0]))]
-        margins.append(_margin(logits[0]))
+        margins[sid].append(_margin(logits[0]))
+        scales[sid].append(float(logits[0].std()))
     live = [sid for sid in range(B) if _alive(outputs[sid], max_gen_len, eos_token_id)]
     while live:
         toks = np.asarray([outputs[sid][-1] for sid in live])
@@ -256,10 +260,13 @@ def greedy_generate_ref(model, prompts, tok_adapter, max_gen_len, n_pages, page_
         kv.end_forward()
         for i, sid in enumerate(live):
             outputs[sid].append(int(np.argmax(logits[i])))
-            margins.append(_margin(logits[i]))
+            margins[sid].append(_margin(logits[i]))
+            scales[sid].append(float(logits[i].std()))
         live = [sid for sid in live if _alive(outputs[sid], max_gen_len, eos_token_id)]
     out = [outputs[sid] for sid in range(B)]
-    return (out, np.asarray(margins)) if return_logits else out
+    if return_logits:
+        return out, [margins[sid] for sid in range(B)], [scales[sid] for sid in range(B)]
+    return out
 
 
 def _alive(out, max_gen_len, eos):

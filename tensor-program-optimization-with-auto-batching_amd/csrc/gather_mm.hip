@@ -141,7 +141,7 @@ template <int R, typename YT>
 __global__ __launch_bounds__(64) void lora_expand_kernel(YT* __restrict__ y, const float* __restrict__ vpart,
                                                          const f16* __restrict__ B,
                                                          const int32_t* __restrict__ ids, float scaling,
-                                                         int T, int N, int KC) {
+                                                         int T, int N, int ldy, int KC) {
   constexpr int LPR = R / 8;           // lanes sharing one row of B
   constexpr int RPI = WAVE / LPR;      // rows per load instruction
   constexpr int NI = 8;                // load instructions (1 KiB each) per wave
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(64) void lora_expand_kernel(YT* __restrict__ y, con
         float d[RPL];
 #pragma unroll
         for (int q = 0; q < RPL; ++q) d[q] = stage[parity][lane * RPL + q];
-        rmw_add<YT, RPL>(y + (size_t)t * N + n, d);
+        rmw_add<YT, RPL>(y + (size_t)t * ldy + n, d);
       }
       parity ^= 1;
     }
@@ -242,11 +242,11 @@ void launch_shrink(float* vpart, const f16* x, const f16* A, const int32_t* ids,
 }
 
 template <int R, typename YT>
-void launch_expand(YT* y, const float* vpart, const f16* B, const int32_t* ids, float scaling, int T, int K, int N,
+void launch_expand(YT* y, int ldy, const float* vpart, const f16* B, const int32_t* ids, float scaling, int T, int K, int N,
                    int n_ad, hipStream_t s) {
   constexpr int CH = 8 * (WAVE / (R / 8));
   hipLaunchKernelGGL((lora_expand_kernel<R, YT>), dim3(n_ad, ceil_div(N, CH)), dim3(64), 0, s, y, vpart, B, ids, scaling,
-                     T, N, k_split(K).kc);
+                     T, N, ldy, k_split(K).kc);
 }
 
 }  // namespace
@@ -274,9 +274,11 @@ extern "C" int mlora_lora_shrink(void* v_part, const void* x, const void* A, con
   return mlora_launch_status("lora_shrink");
 }
 
-extern "C" int mlora_lora_expand(void* y, int y_dtype, const void* v_part, const void* B, const int32_t* tok_adapter,
-                                 float scaling, int T, int K, int N, int r, int n_ad, void* stream) {
+extern "C" int mlora_lora_expand(void* y, int y_dtype, int ldy, const void* v_part, const void* B,
+                                 const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
+                                 void* stream) {
   if (int e = check_lora_shape(T, K, N, r, n_ad)) return e;
+  MLORA_CHECK(ldy >= N && ldy % 8 == 0, MLORA_ERR_INVALID, "lora_expand: need ldy >= N and ldy %% 8 == 0 (ldy=%d N=%d)", ldy, N);
   MLORA_CHECK(y && v_part && B && tok_adapter, MLORA_ERR_INVALID, "lora_expand: null pointer");
   MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "lora_expand: bad y_dtype %d", y_dtype);
   if (T == 0) return MLORA_OK;
@@ -284,8 +286,8 @@ extern "C" int mlora_lora_expand(void* y, int y_dtype, const void* v_part, const
   const float* vp = (const float*)v_part;
   const f16* Bp = (const f16*)B;
 #define MLORA_EXPAND(R)                                                                                   \
-  if (y_dtype == MLORA_F16) launch_expand<R, f16>((f16*)y, vp, Bp, tok_adapter, scaling, T, K, N, n_ad, s); \
-  else launch_expand<R, float>((float*)y, vp, Bp, tok_adapter, scaling, T, K, N, n_ad, s)
+  if (y_dtype == MLORA_F16) launch_expand<R, f16>((f16*)y, ldy, vp, Bp, tok_adapter, scaling, T, K, N, n_ad, s); \
+  else launch_expand<R, float>((float*)y, ldy, vp, Bp, tok_adapter, scaling, T, K, N, n_ad, s)
   switch (r) {
     case 8: MLORA_EXPAND(8); break;
     case 16: MLORA_EXPAND(16); break;
@@ -296,7 +298,7 @@ extern "C" int mlora_lora_expand(void* y, int y_dtype, const void* v_part, const
   return mlora_launch_status("lora_expand");
 }
 
-extern "C" int mlora_gather_mm(void* y, int y_dtype, const void* x, const void* A, const void* B,
+extern "C" int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, const void* A, const void* B,
                                const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
                                void* workspace, size_t workspace_bytes, void* stream) {
   if (int e = check_lora_shape(T, K, N, r, n_ad)) return e;
@@ -304,7 +306,7 @@ extern "C" int mlora_gather_mm(void* y, int y_dtype, const void* x, const void* 
               "gather_mm: workspace of %zu bytes given, %zu needed", workspace_bytes,
               mlora_gather_mm_workspace_bytes(T, K, r));
   if (int e = mlora_lora_shrink(workspace, x, A, tok_adapter, T, K, r, n_ad, stream)) return e;
-  return mlora_lora_expand(y, y_dtype, workspace, B, tok_adapter, scaling, T, K, N, r, n_ad, stream);
+  return mlora_lora_expand(y, y_dtype, ldy, workspace, B, tok_adapter, scaling, T, K, N, r, n_ad, stream);
 }
 
 extern "C" int mlora_write_tensor_part(void* Z, const void* X, const void* Y, const int32_t* ids, int B, int A, int PH,

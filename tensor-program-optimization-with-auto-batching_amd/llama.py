@@ -1,0 +1,248 @@
+"""Llama-style decoder on the HIP operator set, with per-token adapter-indexed LoRA.
+
+Keeps the entry points the reference compiles into its VM (`tvm/llama_auto_batcher/compile_tvm.py:163-285`):
+    embed(input_ids) ; prefill_no_adapter(h, kv) ; prefill_a{i}(h, kv, wids) ;
+    decode_no_adapter(h, kv) ; decode_a{i}(h, kv, wids) ; mixed_decode_a{i}_a{j}...(h, kv, sids_i, wids_i, ...)
+each returning fp32 logits, reachable by name through `model[name]` the way the reference calls `vm[name]`.
+The layer graph follows `tvm/llama_auto_batcher/llama_for_causal_lm.py:79-84,95-100,121-144` and the
+patched attention of `compile_tvm.py:116-160`; the reference adds LoRA to q and v only (`:180-181`), here
+any subset of the seven linears can carry adapters, of several adapter types (rank / alpha) at once.
+
+Precision contract: fp16 weights and stored activations, fp32 accumulation everywhere, fp32 residual
+stream (the o_proj / down_proj kernels accumulate straight into it), fp32 logits.
+"""
+from __future__ import annotations
+
+import re
+
+import numpy as np
+import torch
+
+from . import ops
+from .kv_cache import PagedKVCache
+from .synth import LINEARS, LlamaShape, linear_dims
+
+
+class LoraType:
+    """One adapter type (rank, alpha): stacked tables per (layer, projection)."""
+
+    def __init__(self, r: int, scaling: float, n_adapters: int):
+        self.r, self.scaling, self.n_adapters = r, float(scaling), n_adapters
+        self.tables = {}     # (layer, proj) -> (A [n_ad, r, K], B [n_ad, N, r])
+
+    def add(self, layer: int, proj: str, A: torch.Tensor, B: torch.Tensor):
+        if A.shape[0] != self.n_adapters or A.shape[1] != self.r or B.shape[0] != self.n_adapters or B.shape[2] != self.r:
+            raise ValueError(f"LoRA table shape mismatch at layer {layer} {proj}: A{tuple(A.shape)} B{tuple(B.shape)}")
+        self.tables[(layer, proj)] = (A.contiguous(), B.contiguous())
+
+
+class LlamaForCausalLM:
+    def __init__(self, shape: LlamaShape, device="cuda:0"):
+        self.shape = shape
+        self.device = torch.device(device)
+        self.layers = []          # per layer dict: qkv, o, gate_up, down (PackedWeight), ln1, ln2 (fp16 [H])
+        self.embed_tokens = None
+        self.lm_head = None
+        self.norm = None
+        self.lora_types = []      # index = adapter type id
+        self._ws = None
+
+    # ------------------------------------------------------------------ weights
+    def load_layer(self, l: int, w: dict):
+        """w: the seven projection weights [N, K] fp16 and the two norm weights of layer l
+        (keys 'q_proj', ..., 'input_layernorm', 'post_attention_layernorm').  q/k/v and gate/up are fused
+        row-wise and stored in matrix-core fragment order."""
+        assert l == len(self.layers), "layers must be loaded in order"
+        dev = self.device
+        qkv = torch.cat([w["q_proj"], w["k_proj"], w["v_proj"]], 0).to(dev, torch.float16)
+        gu = torch.cat([w["gate_proj"], w["up_proj"]], 0).to(dev, torch.float16)
+        self.layers.append({
+            "qkv": ops.PackedWeight(qkv), "o": ops.PackedWeight(w["o_proj"].to(dev, torch.float16)),
+            "gate_up": ops.PackedWeight(gu), "down": ops.PackedWeight(w["down_proj"].to(dev, torch.float16)),
+            "ln1": w["input_layernorm"].to(dev, torch.float16).contiguous(),
+            "ln2": w["post_attention_layernorm"].to(dev, torch.float16).contiguous(),
+        })
+
+    def load_head(self, embed_tokens, lm_head, norm):
+        dev = self.device
+        self.embed_tokens = embed_tokens.to(dev, torch.float16).contiguous()
+        self.lm_head = ops.PackedWeight(lm_head.to(dev, torch.float16))
+        self.norm = norm.to(dev, torch.float16).contiguous()
+
+    def add_lora_type(self, lora_type: LoraType) -> int:
+        self.lora_types.append(lora_type)
+        return len(self.lora_types) - 1
+
+    @classmethod
+    def from_synthetic(cls, seed: int, shape: LlamaShape, lora_specs=(), device="cuda:0", synth=None):
+        """Random-init model generated on the device (bit-identical to the CPU generation of the same seed)."""
+        from . import synth as S
+        m = cls(shape, device)
+        for l in range(shape.num_hidden_layers):
+            w = S.layer_weights(seed, shape, l, torch.float16, device)
+            m.load_layer(l, {k.split(".", 2)[2]: v for k, v in w.items()})
+            del w
+        m.load_head(S.normal(seed, "embed_tokens", (shape.vocab_size, shape.hidden_size), 0.02, torch.float16, device),
+                    S.normal(seed, "lm_head", (shape.vocab_size, shape.hidden_size), 0.02, torch.float16, device),
+                    torch.ones(shape.hidden_size, dtype=torch.float16, device=device))
+        for tid, spec in enumerate(lora_specs):
+            lt = LoraType(spec.r, spec.scaling, spec.n_adapters)
+            lw = S.lora_weights(seed, shape, spec, torch.float16, device, tag=f"a{tid}")
+            for l in range(shape.num_hidden_layers):
+                for proj in spec.targets:
+                    lt.add(l, proj, lw[f"layers.{l}.{proj}.lora_A.a{tid}"], lw[f"layers.{l}.{proj}.lora_B.a{tid}"])
+            m.add_lora_type(lt)
+        return m
+
+    def create_paged_kv_cache(self, max_batch_size, max_total_seq_len, prefill_chunk_size, page_size,
+                              free_pages=None, max_seq_len=None):
+        """Same arguments as the reference's VM function (`llama_for_causal_lm.py:148-174`).  The pool holds
+        ceil(max_total_seq_len / page_size) + max_batch_size pages (one partial page per sequence)."""
+        s = self.shape
+        n_pages = -(-max_total_seq_len // page_size) + max_batch_size
+        if free_pages is not None:
+            n_pages = len(free_pages)
+        max_seq_len = max_seq_len or min(max_total_seq_len, n_pages * page_size)
+        max_blocks = -(-max_seq_len // page_size)
+        return PagedKVCache(s.num_hidden_layers, n_pages, s.num_key_value_heads, s.head_dim, max_seqs=max_batch_size,
+                            max_blocks=max_blocks, rope_theta=s.rope_theta, max_pos=max_blocks * page_size,
+                            device=self.device, free_pages=free_pages, page_size=page_size)
+
+    # ------------------------------------------------------------------ forward
+    def embed(self, input_ids: torch.Tensor) -> torch.Tensor:
+        """input_ids [T] or [b, s] int32 -> hidden [T, H] fp32 (the residual stream)."""
+        ids = input_ids.reshape(-1).to(self.device, torch.int32).contiguous()
+        return ops.embed(self.embed_tokens, ids, out_dtype=torch.float32)
+
+    def _workspace(self, T, K, r):
+        need = ops.lib().mlora_gather_mm_workspace_bytes(T, K, r) // 4 + 4
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.empty(need, dtype=torch.float32, device=self.device)
+        return self._ws
+
+    def _lora(self, y, x, l, proj, tok_adapter):
+        """y += delta for every adapter type that targets (l, proj); tok_adapter: {tid: ids [T] int32}."""
+        for tid, ids in tok_adapter.items():
+            lt = self.lora_types[tid]
+            tab = lt.tables.get((l, proj))
+            if tab is not None:
+                ops.gather_mm(y, x, tab[0], tab[1], ids, lt.scaling, self._workspace(x.shape[0], x.shape[1], lt.r))
+
+    def forward(self, hidden: torch.Tensor, kv: PagedKVCache, tok_adapter=None, logits_rows=None) -> torch.Tensor:
+        """hidden [T, H] fp32 (updated in place), tokens in kv.begin_forward order -> logits fp32."""
+        s = self.shape
+        tok_adapter = tok_adapter or {}
+        T = hidden.shape[0]
+        H, I = s.hidden_size, s.intermediate_size
+        q_sz, kv_sz = s.q_size, s.kv_size
+        resid = hidden
+        for l, L in enumerate(self.layers):
+            xn = ops.rmsnorm(resid, L["ln1"], s.rms_norm_eps)
+            qkv = ops.linear(xn, L["qkv"])
+            if tok_adapter:
+                self._lora(qkv[:, :q_sz], xn, l, "q_proj", tok_adapter)
+                self._lora(qkv[:, q_sz:q_sz + kv_sz], xn, l, "k_proj", tok_adapter)
+                self._lora(qkv[:, q_sz + kv_sz:], xn, l, "v_proj", tok_adapter)
+            attn = kv.attention_with_fused_qkv(l, qkv, s.num_attention_heads)
+            ops.linear(attn, L["o"], out=resid, accumulate=True)
+            if tok_adapter:
+                self._lora(resid, attn, l, "o_proj", tok_adapter)
+            xn = ops.rmsnorm(resid, L["ln2"], s.rms_norm_eps)
+            gu = ops.linear(xn, L["gate_up"])
+            if tok_adapter:
+                self._lora(gu[:, :I], xn, l, "gate_proj", tok_adapter)
+                self._lora(gu[:, I:], xn, l, "up_proj", tok_adapter)
+            act = ops.silu_mul(gu)
+            ops.linear(act, L["down"], out=resid, accumulate=True)
+            if tok_adapter:
+                self._lora(resid, act, l, "down_proj", tok_adapter)
+        if logits_rows is not None:
+            resid = resid[logits_rows].contiguous()
+        xn = ops.rmsnorm(resid, self.norm, s.rms_norm_eps)
+        return ops.linear(xn, self.lm_head, out_dtype=torch.float32)
+
+    # ------------------------------------------------------------------ reference entry points
+    def _ids(self, T, pairs):
+        """{tid: (positions | None, wids)} -> {tid: ids [T] int32 on device, -1 where the type is absent}."""
+        out = {}
+        for tid, (sids, wids) in pairs.items():
+            full = np.full(T, -1, dtype=np.int32)
+            w = _host_i32(wids)
+            lt = self.lora_types[tid]
+            if w.size and (w.min() < 0 or w.max() >= lt.n_adapters):
+                raise ValueError(f"adapter weight id out of range for type {tid}: {w.min()}..{w.max()} of {lt.n_adapters}")
+            if sids is None:
+                full[:] = np.broadcast_to(w, (T,)) if w.size in (1, T) else _bad(T, w)
+            else:
+                p = _host_i32(sids)
+                if p.size != w.size or (p.size and (p.min() < 0 or p.max() >= T)):
+                    raise ValueError("sids / wids mismatch")
+                full[p] = w
+            out[tid] = torch.from_numpy(full).to(self.device)
+        return out
+
+    def _last_rows(self, kv):
+        lens = kv._cur[1]
+        return torch.from_numpy(np.cumsum(lens).astype(np.int64) - 1).to(self.device)
+
+    def prefill_no_adapter(self, h, kv):
+        return self.forward(h, kv, None, self._last_rows(kv)), kv
+
+    def decode_no_adapter(self, h, kv):
+        return self.forward(h, kv, None), kv
+
+    def prefill_a(self, tid, h, kv, wids):
+        """Prefill of the sequences announced to kv.begin_forward; wids: one weight id per sequence
+        (the reference prefills one sequence per call: wids [1])."""
+        lens = kv._cur[1]
+        w = np.repeat(_host_i32(wids), lens)
+        return self.forward(h, kv, self._ids(h.shape[0], {tid: (None, w)}), self._last_rows(kv)), kv
+
+    def decode_a(self, tid, h, kv, wids):
+        return self.forward(h, kv, self._ids(h.shape[0], {tid: (None, wids)})), kv
+
+    def mixed_decode(self, tids, h, kv, *params):
+        """params = sids_i, wids_i, sids_j, wids_j, ... for the adapter types in `tids`
+        (`compile_tvm.py:135-155`: rows `sids` of the batch use that type with weight ids `wids`)."""
+        if len(params) != 2 * len(tids):
+            raise ValueError(f"mixed decode over {len(tids)} adapter types needs {2 * len(tids)} id arrays")
+        pairs = {tid: (params[2 * i], params[2 * i + 1]) for i, tid in enumerate(tids)}
+        return self.forward(h, kv, self._ids(h.shape[0], pairs)), kv
+
+    def __getitem__(self, name: str):
+        """Entry points by the reference's VM function names."""
+        if name in ("embed", "create_paged_kv_cache", "prefill_no_adapter", "decode_no_adapter"):
+            return getattr(self, name)
+        m = re.fullmatch(r"(prefill|decode)_a(\d+)", name)
+        if m:
+            tid = int(m.group(2))
+            self._check_tid(tid)
+            fn = self.prefill_a if m.group(1) == "prefill" else self.decode_a
+            return lambda h, kv, wids: fn(tid, h, kv, wids)
+        m = re.fullmatch(r"mixed_decode((?:_a\d+)+)", name)
+        if m:
+            tids = [int(t) for t in re.findall(r"_a(\d+)", m.group(1))]
+            for t in tids:
+                self._check_tid(t)
+            return lambda h, kv, *params: self.mixed_decode(tids, h, kv, *params)
+        raise KeyError(f"unknown entry point {name}")
+
+    def _check_tid(self, tid):
+        if not 0 <= tid < len(self.lora_types):
+            raise KeyError(f"adapter type a{tid} not loaded")
+
+    def weight_bytes_per_step(self):
+        """Algorithmic fp16 weight bytes one decode step streams (all layers + lm_head)."""
+        s = self.shape
+        per_layer = sum(np.prod(linear_dims(s, p)) for p in LINEARS)
+        return int(2 * (per_layer * s.num_hidden_layers + s.vocab_size * s.hidden_size))
+
+
+def _host_i32(a):
+    if isinstance(a, torch.Tensor):
+        a = a.detach().cpu().numpy()
+    return np.asarray(a, dtype=np.int32).reshape(-1)
+
+
+def _bad(T, w):
+    raise ValueError(f"expected 1 or {T} weight ids, got {w.size}")

@@ -1,0 +1,157 @@
+"""Execution of the auto-batching graph on the HIP model: prefill per sequence, batched greedy decode.
+
+Restates `tvm/llama_auto_batcher/llama_exec_graph.py:10-174`.  Differences that do not change results:
+the argmax runs on the device and only the token ids cross to the host (the reference copies the full
+fp32 logits and calls np.argmax, `:92,134-137`; ties resolve to the lowest index in both); prompts may be
+given as token-id arrays when no tokenizer is configured.
+"""
+from __future__ import annotations
+
+import dataclasses
+import os
+
+import numpy as np
+import torch
+
+from . import ops
+from .exec_graph import ExecGraph
+
+
+@dataclasses.dataclass
+class LlamaExecConfig:
+    max_prompt_len: int
+    max_gen_len: int
+    page_size: int
+
+
+class LlamaExecGraph(ExecGraph):
+    def __init__(self, batchable_op_types=("decode",)):
+        super().__init__(batchable_op_types)
+        self.measure = False
+        self.measure_file = None
+        self.step_ms = []
+
+    def set_exec_vars(self, vm, dev, params, tokenizer, seq_info, exec_config, eos_token_id=None, free_pages=None):
+        self.vm = vm                  # a LlamaForCausalLM: entry points by name
+        self.dev = dev
+        self.params = params          # kept for signature parity; weights live inside `vm`
+        self.tokenizer = tokenizer
+        self.seq_info = seq_info
+        self.exec_config = exec_config
+        self.eos_token_id = eos_token_id if eos_token_id is not None else getattr(tokenizer, "eos_token_id", None)
+        self.free_pages = free_pages
+        self.measure = False
+        self.kv_cache = None
+        self.set_kv_cache(False)
+
+    def set_kv_cache(self, delete_prev=True):
+        if delete_prev:
+            self.kv_cache = None
+        n = self.seq_info.get_num_sequences()
+        c = self.exec_config
+        self.kv_cache = self.vm["create_paged_kv_cache"](
+            n, n * (c.max_prompt_len + c.max_gen_len), c.max_prompt_len, c.page_size,
+            free_pages=self.free_pages, max_seq_len=c.max_prompt_len + c.max_gen_len)
+
+    def set_measuring(self, dest):
+        """One millisecond value per line, one line per prefill and per decode step (`:48-50,70-74,116-132`)."""
+        self.measure = True
+        self.measure_file = open(dest if os.path.isabs(dest) else os.path.join(os.path.expanduser("~"), dest), "w")
+
+    # ------------------------------------------------------------------ timing
+    def _tic(self):
+        if not self.measure:
+            return None
+        ev = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+        torch.cuda.synchronize()
+        ev[0].record()
+        return ev
+
+    def _toc(self, ev):
+        if ev is None:
+            return
+        ev[1].record()
+        torch.cuda.synchronize()
+        ms = ev[0].elapsed_time(ev[1])
+        self.step_ms.append(ms)
+        if self.measure_file is not None:
+            self.measure_file.write(f"{ms}\n")
+
+    # ------------------------------------------------------------------ operations
+    def execute_encode_prompt(self, op):
+        assert len(op.input_vars) == 1 and len(op.output_vars) == 1 and len(op.seqids) == 1, \
+            "encode_prompt node must have exactly 1 input var, 1 output var and 1 seqid"
+        prompt = op.input_vars[0].var
+        if isinstance(prompt, str):
+            assert self.tokenizer is not None, "a text prompt needs a tokenizer"
+            ids = np.asarray(self.tokenizer(prompt)["input_ids"], dtype=np.int32).reshape(1, -1)
+        else:
+            ids = np.asarray(prompt, dtype=np.int32).reshape(1, -1)
+        op.output_vars[0].var = ids
+
+    def execute_prefill(self, op):
+        assert len(op.input_vars) == 1 and len(op.output_vars) == 1 and len(op.seqids) == 1, \
+            "prefill node must have exactly 1 input var, 1 output var and 1 seqid"
+        sid = op.seqids[0]
+        tokens = op.input_vars[0].var
+        self.kv_cache.add_sequence(sid)
+        hidden = self.vm["embed"](torch.from_numpy(np.ascontiguousarray(tokens)))
+        adapter = self.seq_info.get_adapter_info(sid)
+        ev = self._tic()
+        self.kv_cache.begin_forward([sid], [tokens.shape[1]])
+        if adapter is None:
+            logits, _ = self.vm["prefill_no_adapter"](hidden, self.kv_cache)
+        else:
+            logits, _ = self.vm[f"prefill_a{adapter['tid']}"](hidden, self.kv_cache, [adapter["wid"]])
+        self.kv_cache.end_forward()
+        self._toc(ev)
+        op.output_vars[0].var = int(ops.argmax(logits).cpu()[0])
+
+    def check_seqs_finished(self, seqs_2_decode, outputs):
+        return [sid for sid in seqs_2_decode
+                if outputs[sid][-1] != self.eos_token_id and len(outputs[sid]) < self.seq_info.get_max_gen_len(sid)]
+
+    def execute_decode(self, op):
+        assert len(op.input_vars) == len(op.output_vars), "decode node needs as many output vars as input vars"
+        assert len(op.input_vars) == len(op.seqids), "decode node needs one sequence id per input var"
+        seqs, original_positions = self.seq_info.order_seqs(op.seqids)
+        outputs = {sid: [int(op.input_vars[original_positions[i]].var)] for i, sid in enumerate(seqs)}
+        ordered = list(seqs)
+        # the first token (from prefill) already counts towards max_gen_len (`:94-100`)
+        seqs = self.check_seqs_finished(seqs, outputs)
+        while seqs:
+            tokens = torch.tensor([outputs[sid][-1] for sid in seqs], dtype=torch.int32)
+            hidden = self.vm["embed"](tokens)
+            method, params = self.seq_info.get_decode_method(seqs)
+            ev = self._tic()
+            self.kv_cache.begin_forward(seqs, [1] * len(seqs))
+            logits, _ = self.vm[method](hidden, self.kv_cache, *params)
+            self.kv_cache.end_forward()
+            self._toc(ev)
+            nxt = ops.argmax(logits).cpu().numpy()
+            for i, sid in enumerate(seqs):
+                outputs[sid].append(int(nxt[i]))
+            seqs = self.check_seqs_finished(seqs, outputs)
+        for i, sid in enumerate(ordered):
+            op.output_vars[original_positions[i]].var = np.asarray(outputs[sid], dtype=np.int64)
+
+    def execute_decode_answer(self, op):
+        assert len(op.input_vars) == 1 and len(op.output_vars) == 1 and len(op.seqids) == 1, \
+            "decode_answer node must have exactly 1 input var, 1 output var and 1 seqid"
+        ids = op.input_vars[0].var
+        op.output_vars[0].var = self.tokenizer.decode(ids) if self.tokenizer is not None else ids
+
+    def execute_print(self, op):
+        if self.measure:
+            return
+        assert len(op.input_vars) == 1 and len(op.seqids) == 1, "print node must have exactly 1 input var and 1 seqid"
+        print(f"Answer for Sequence {op.seqids[0]} {op.input_vars[0].var}")
+
+    def execute_op(self, op):
+        fn = {"encode_prompt": self.execute_encode_prompt, "prefill": self.execute_prefill,
+              "decode": self.execute_decode, "decode_answer": self.execute_decode_answer,
+              "print": self.execute_print}.get(op.op_type)
+        if fn is None:
+            print(f"[ERROR] unknown op_type: {op.op_type}")
+            return
+        fn(op)

@@ -39,8 +39,9 @@ def gather_mm_workspace(T: int, K: int, r: int, device) -> torch.Tensor:
 
 
 def gather_mm(y, x, A, B, tok_adapter, scaling: float, workspace=None):
-    """y[t] += scaling * B[id_t] @ (A[id_t] @ x[t]) in place.  y [T,N] f16|f32, x [T,K] f16,
-    A [n_ad,r,K] f16, B [n_ad,N,r] f16, tok_adapter [T] int32 (-1 = no adapter)."""
+    """y[t] += scaling * B[id_t] @ (A[id_t] @ x[t]) in place.  y [T,N] f16|f32 (rows may be strided: a
+    column slice of a wider buffer), x [T,K] f16, A [n_ad,r,K] f16, B [n_ad,N,r] f16,
+    tok_adapter [T] int32 (-1 = no adapter)."""
     T, K = x.shape
     n_ad, r, K2 = A.shape
     N = B.shape[1]
@@ -49,7 +50,10 @@ def gather_mm(y, x, A, B, tok_adapter, scaling: float, workspace=None):
                          f"B{tuple(B.shape)} ids{tuple(tok_adapter.shape)}")
     if workspace is None:
         workspace = gather_mm_workspace(T, K, r, x.device)
-    check(lib().mlora_gather_mm(_dev(y, None, "y"), _dt(y), _dev(x, torch.float16, "x"), _dev(A, torch.float16, "A"),
+    if not y.is_cuda or y.stride(1) != 1:
+        raise ValueError("gather_mm: y must be a GPU tensor with unit inner stride")
+    ldy = y.stride(0) if T > 1 else max(N, y.stride(0))
+    check(lib().mlora_gather_mm(y.data_ptr(), _dt(y), ldy, _dev(x, torch.float16, "x"), _dev(A, torch.float16, "A"),
                                 _dev(B, torch.float16, "B"), _dev(tok_adapter, torch.int32, "tok_adapter"),
                                 float(scaling), T, K, N, r, n_ad, _dev(workspace, torch.float32, "workspace"),
                                 workspace.numel() * 4, _stream()))
@@ -67,7 +71,7 @@ def lora_shrink(v_part, x, A, tok_adapter):
 def lora_expand(y, v_part, B, tok_adapter, scaling: float, K: int):
     T, N = y.shape
     n_ad, _, r = B.shape
-    check(lib().mlora_lora_expand(_dev(y), _dt(y), _dev(v_part, torch.float32), _dev(B, torch.float16),
+    check(lib().mlora_lora_expand(_dev(y), _dt(y), N, _dev(v_part, torch.float32), _dev(B, torch.float16),
                                   _dev(tok_adapter, torch.int32), float(scaling), T, K, N, r, n_ad, _stream()))
     return y
 

@@ -65,11 +65,25 @@ def test_gather_mm_no_adapter_rows_untouched_and_index_exact(ops, synth):
     assert np.array_equal(_np(y)[ids < 0], ys[ids < 0])
 
 
+def test_gather_mm_into_column_slice(ops, synth):
+    """y may be a column slice of a fused projection output (row stride > N); other columns stay untouched."""
+    T, K, N, r, n_ad = 32, 1024, 256, 16, 4
+    c = synth.gather_mm_case(seed=2, T=T, K=K, N=N, r=r, n_ad=n_ad, device=DEV, tag="slice")
+    wide = synth.normal(2, "gmm.wide", (T, 3 * N), 1.0, torch.float16, DEV)
+    before = _np(wide).copy()
+    ops.gather_mm(wide[:, N:2 * N], c["x"], c["A"], c["B"], c["ids"], 0.5)
+    torch.cuda.synchronize()
+    ref = oracle.gather_mm_ref(before[:, N:2 * N], _np(c["x"]), _np(c["A"]), _np(c["B"]), c["ids"].cpu().numpy(), 0.5)
+    after = _np(wide)
+    assert max_rel_err(after[:, N:2 * N], ref) <= TOL
+    assert np.array_equal(after[:, :N], before[:, :N]) and np.array_equal(after[:, 2 * N:], before[:, 2 * N:])
+
+
 def test_gather_mm_rejects_bad_shapes(ops):
     lib = ops.lib()
-    assert lib.mlora_gather_mm(1, 0, 1, 1, 1, 1, 1.0, 4, 64, 64, 12, 2, 1, 1 << 20, None) == -2   # rank 12
+    assert lib.mlora_gather_mm(1, 0, 64, 1, 1, 1, 1, 1.0, 4, 64, 64, 12, 2, 1, 1 << 20, None) == -2   # rank 12
     assert b"rank" in lib.mlora_last_error()
-    assert lib.mlora_gather_mm(1, 0, 1, 1, 1, 1, 1.0, 4, 64, 64, 16, 2, 1, 8, None) == -3          # workspace
+    assert lib.mlora_gather_mm(1, 0, 64, 1, 1, 1, 1, 1.0, 4, 64, 64, 16, 2, 1, 8, None) == -3          # workspace
     assert lib.mlora_gemv(1, 0, 0, 1, 64, 1, 65, 64, 64, None) == -2                                 # T > 64
 
 
