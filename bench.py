@@ -1,0 +1,238 @@
+#!/usr/bin/env python3
+"""Headline benchmark: greedy decode of a Llama-2-7B-shape model, 32 requests x 16 rank-16 LoRA adapters
+(q/k/v/o), paged KV cache with 16-token pages in random page order, 512-token prompts.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the whole batch (32 new tokens).  Inputs are synthetic (seeded, generated on
+the device); weights and the KV cache are resident in HBM when the timed region starts.  Prints ONE JSON
+line: decode tok/s, the roofline of the dominant kernel (the weight-streaming GEMV, timed with events on
+the launch stream), the gather-matmul figures, and a CPU baseline (the numpy oracle on the host cores,
+bounded sample).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+PKG = "tensor-program-optimization-with-auto-batching_amd"
+HBM_PEAK_GBS = 8000.0
+
+
+def _mod(name):
+    return importlib.import_module(PKG + "." + name)
+
+
+def prefill_all(model, kv, prompts, adapter_ids, chunk=4):
+    """Prefill all sequences, `chunk` at a time; returns the first generated token of each."""
+    import torch
+    ops = _mod("ops")
+    B, P = prompts.shape
+    first = np.zeros(B, dtype=np.int32)
+    for s in range(B):
+        kv.add_sequence(s)
+    for lo in range(0, B, chunk):
+        sids = list(range(lo, min(B, lo + chunk)))
+        kv.begin_forward(sids, [P] * len(sids))
+        h = model.embed(torch.from_numpy(np.ascontiguousarray(prompts[sids].reshape(-1))))
+        logits, _ = model["prefill_a0"](h, kv, adapter_ids[sids])
+        kv.end_forward()
+        first[sids] = ops.argmax(logits).cpu().numpy()
+    return first
+
+
+def gemv_event_timing(model, T):
+    """Average duration of the weight-streaming GEMV over one decode step's worth of launches (the four
+    fused projections of every layer + lm_head), each launch bracketed by events on the launch stream."""
+    import torch
+    ops = _mod("ops")
+    s = model.shape
+    dev = model.device
+    x_h = torch.zeros((T, s.hidden_size), dtype=torch.float16, device=dev)
+    x_q = torch.zeros((T, s.q_size), dtype=torch.float16, device=dev)
+    x_i = torch.zeros((T, s.intermediate_size), dtype=torch.float16, device=dev)
+    resid = torch.zeros((T, s.hidden_size), dtype=torch.float32, device=dev)
+    qkv = torch.empty((T, s.q_size + 2 * s.kv_size), dtype=torch.float16, device=dev)
+    gu = torch.empty((T, 2 * s.intermediate_size), dtype=torch.float16, device=dev)
+    logits = torch.empty((T, s.vocab_size), dtype=torch.float32, device=dev)
+    launches = []
+    for L in model.layers:
+        launches += [(x_h, L["qkv"], qkv, False), (x_q, L["o"], resid, True),
+                     (x_h, L["gate_up"], gu, False), (x_i, L["down"], resid, True)]
+    launches.append((x_h, model.lm_head, logits, False))
+    for x, W, out, acc in launches[:8]:
+        ops.linear(x, W, out=out, accumulate=acc, kernel="gemv")
+    torch.cuda.synchronize()
+    evs = []
+    for x, W, out, acc in launches:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        ops.linear(x, W, out=out, accumulate=acc, kernel="gemv")
+        e1.record()
+        evs.append((e0, e1, W.N * W.K * 2 + T * W.K * 2 + T * W.N * (4 if out.dtype == torch.float32 else 2) * (2 if acc else 1)))
+    torch.cuda.synchronize()
+    ms = [a.elapsed_time(b) for a, b, _ in evs]
+    total_bytes = sum(b for _, _, b in evs)
+    return {"launches": len(evs), "avg_us": 1e3 * sum(ms) / len(ms), "bytes_per_launch": total_bytes / len(evs),
+            "gbs": total_bytes / (sum(ms) * 1e-3) / 1e9}
+
+
+def gather_mm_timing(n_sets=128):
+    """Isolated gather-matmul at the decode shape (T=64, K=N=4096, r=16, 32 adapters): n_sets distinct
+    operand sets (> 1 GiB, larger than the 256 MB last-level cache) issued back to back."""
+    import torch
+    ops, synth = _mod("ops"), _mod("synth")
+    dev = "cuda:0"
+    T, K, N, r, n_ad = 64, 4096, 4096, 16, 32
+    ids = synth.randint(1, "gmm.ids", (T,), n_ad, dev)
+    U = len(np.unique(ids.cpu().numpy()))
+    sets = []
+    for j in range(n_sets):
+        sets.append((synth.normal(1, f"b.x{j}", (T, K), 1.0, torch.float16, dev),
+                     synth.normal(1, f"b.A{j}", (n_ad, r, K), 0.02, torch.float16, dev),
+                     synth.normal(1, f"b.B{j}", (n_ad, N, r), 0.02, torch.float16, dev),
+                     synth.normal(1, f"b.y{j}", (T, N), 1.0, torch.float16, dev)))
+    ws = ops.gather_mm_workspace(T, K, r, dev)
+    for x, A, B, y in sets[:4]:
+        ops.gather_mm(y, x, A, B, ids, 1.0, ws)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for x, A, B, y in sets:
+        ops.gather_mm(y, x, A, B, ids, 1.0, ws)
+    e1.record()
+    torch.cuda.synchronize()
+    sec = e0.elapsed_time(e1) * 1e-3
+    by = 2 * T * K + U * 2 * r * K + U * 2 * N * r + 4 * T * N + 4 * T
+    return {"workload": "T=64 K=N=4096 r=16 n_ad=32", "distinct_adapters": U, "sets": n_sets,
+            "bytes_per_call": by, "us_per_call": sec / n_sets * 1e6, "gbs": by * n_sets / sec / 1e9,
+            "frac_of_hbm_peak": by * n_sets / sec / 1e9 / HBM_PEAK_GBS}
+
+
+def cpu_baseline(wl, ctx, layers=2, steps=3):
+    """The numpy oracle (fp32) on the host cores: `layers` of the 32 layers, `steps` decode steps of the
+    whole batch at context `ctx` with a pre-filled cache, plus lm_head; scaled to the full depth."""
+    import torch
+    import oracle
+    synth = _mod("synth")
+    shape = synth.LlamaShape(**{**wl.shape.__dict__, "num_hidden_layers": layers})
+    w = {k: v.float().numpy() for k, v in synth.base_weights(wl.seed, shape, torch.float16, "cpu").items()}
+    lw = {k: v.float().numpy() for k, v in synth.lora_weights(wl.seed, shape, wl.lora, torch.float16, "cpu", tag="a0").items()}
+    ref = oracle.LlamaRef(shape, w, lw, {"a0": wl.lora.scaling}, mode="fp32")
+    B = wl.batch
+    blocks = -(-(ctx + steps + 1) // 16)
+    kv = ref.new_cache(B * blocks, 16, ctx + steps + 2)
+    rng = np.random.default_rng(0)
+    kv.k[:] = rng.standard_normal(kv.k.shape, dtype=np.float32)
+    kv.v[:] = rng.standard_normal(kv.v.shape, dtype=np.float32)
+    for s in range(B):
+        kv.add_sequence(s)
+        kv.tables[s] = [kv.free.pop(0) for _ in range(blocks)]
+        kv.lens[s] = ctx
+    toks = rng.integers(0, shape.vocab_size, B)
+    ids = {"a0": wl.adapter_ids}
+    t_steps = []
+    for _ in range(steps):
+        t0 = time.perf_counter()
+        kv.begin_forward(list(range(B)), [1] * B)
+        logits = ref.forward(toks, kv, ids)
+        kv.end_forward()
+        toks = logits.argmax(-1)
+        t_steps.append(time.perf_counter() - t0)
+    # split one step into the per-layer part and the head (embedding + final norm + lm_head)
+    t0 = time.perf_counter()
+    xn = oracle.rmsnorm_ref(w["embed_tokens"][toks], w["norm"], shape.rms_norm_eps)
+    (xn @ w["lm_head"].T).argmax(-1)
+    t_head = time.perf_counter() - t0
+    t_step = float(np.median(t_steps))
+    t_full = (t_step - t_head) * (wl.shape.num_hidden_layers / layers) + t_head
+    return {"value": B / t_full, "unit": "tok/s", "cores": os.cpu_count(), "kind": "port",
+            "sample": f"numpy fp32 oracle, {layers} of {wl.shape.num_hidden_layers} layers x {steps} decode steps of the "
+                      f"32-request batch at context {ctx} (pre-filled cache) + lm_head, per-layer time scaled x"
+                      f"{wl.shape.num_hidden_layers // layers}; threads = BLAS default on {os.cpu_count()} cores"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=32, help="model depth (32 = the benchmark configuration)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel event timing and the gather-matmul stream")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (every box here has one GPU, and the "
+              f"path has no collective: requests would simply be partitioned over GPUs).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    synth, llama, dsm = _mod("synth"), _mod("llama"), _mod("decode_session")
+    wl = synth.config3(num_layers=args.layers)
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    t_setup = time.perf_counter()
+    model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, [wl.lora], dev)
+    prompts = synth.prompts(wl)
+    total_new = args.warmup + args.steps + 1
+    max_len = wl.prompt_len + total_new
+    blocks = -(-max_len // wl.page_size)
+    perm = synth.permutation(wl.seed, "c3.pages", wl.batch * blocks)
+    kv = model.create_paged_kv_cache(wl.batch, wl.batch * blocks * wl.page_size, wl.prompt_len, wl.page_size,
+                                     free_pages=perm, max_seq_len=blocks * wl.page_size)
+    first = prefill_all(model, kv, prompts, wl.adapter_ids)
+    sess = dsm.DecodeSession(model, kv, list(range(wl.batch)), {0: wl.adapter_ids}, first)
+    for _ in range(args.warmup):
+        sess.step()
+    torch.cuda.synchronize()
+    t_setup = time.perf_counter() - t_setup
+
+    ctx0 = wl.prompt_len + args.warmup
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        sess.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    tok_s = wl.batch * args.steps / dt
+
+    # algorithmic bytes of one step at the mean context of the timed region
+    mean_ctx = ctx0 + (args.steps + 1) / 2.0
+    kv_bytes = wl.batch * mean_ctx * wl.shape.num_hidden_layers * 2 * wl.shape.kv_size * 2
+    lora_bytes = wl.shape.num_hidden_layers * len(wl.lora.targets) * wl.lora.n_adapters * 2 * wl.lora.r * (2 * 4096)
+    step_bytes = model.weight_bytes_per_step() + kv_bytes + lora_bytes
+
+    out = {
+        "metric": "decode tok/s, Llama-7B-shape bs32×16 LoRAs; gather-matmul HBM GB/s %peak",
+        "value": tok_s, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": wl.name, "layers": wl.shape.num_hidden_layers, "hidden": wl.shape.hidden_size,
+                   "batch": wl.batch, "adapters": wl.lora.n_adapters, "rank": wl.lora.r, "lora_targets": list(wl.lora.targets),
+                   "prompt_len": wl.prompt_len, "context_at_start": ctx0, "page_size": wl.page_size, "page_order": "random"},
+        "step_algorithmic_gb": step_bytes / 1e9,
+        "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "setup_s": t_setup,
+    }
+    if not args.no_extras:
+        g = gemv_event_timing(model, wl.batch)
+        out["roofline"] = {"kernel": "gemv_kernel (packed weights, T=32)", "bound": "hbm", "achieved": g["gbs"],
+                           "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g["gbs"] / HBM_PEAK_GBS, "traffic": None,
+                           "launches_timed": g["launches"], "avg_launch_us": g["avg_us"],
+                           "algorithmic_bytes_per_launch": g["bytes_per_launch"]}
+        del sess, kv
+        torch.cuda.empty_cache()
+        out["gather_matmul"] = gather_mm_timing()
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wl, ctx0)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
