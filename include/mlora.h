@@ -38,6 +38,15 @@ extern "C" {
 #define MLORA_STORE       0
 #define MLORA_ACCUMULATE  1
 
+/* Activation layouts.  MLORA_ROWMAJOR: x[T, K], innermost contiguous.  MLORA_FRAG: the order in which the
+ * matrix cores consume the token block of a decode step (T <= 64),
+ *     Xf[k/32][t/16][(k%32)/8][t%16][k%8]     with TT = 1, 2 or 4 sixteen-token tiles for T <= 16, 32, 64,
+ * so that the 16-token x 32-k operand fragment is one contiguous 1 KiB block; mlora_frag_activation_elems
+ * gives the buffer size.  Producers (RMSNorm, SiLU*mul, decode attention) can write it directly, the decode
+ * GEMV (mlora_gemv_frag) and the LoRA shrink read it; rows t >= T of the last tile are never read back. */
+#define MLORA_ROWMAJOR 0
+#define MLORA_FRAG     1
+
 #define MLORA_PAGE_SIZE 16   /* tokens per KV page; the only page size the kernels accept */
 
 int mlora_version(void);
@@ -55,7 +64,8 @@ const char* mlora_last_error(void);
  *   token, the row gather/scatter around it in the mixed path (compile_tvm.py:147-153,
  *   tvm/custom/write_tensor_part.py:3-20).
  *
- * Layouts (PEFT orientation): x [T, K] f16; A [n_ad, r, K] f16; B [n_ad, N, r] f16;
+ * Layouts (PEFT orientation): x [T, K] f16 (x_layout: row-major, or fragment order when T <= 64);
+ *   A [n_ad, r, K] f16; B [n_ad, N, r] f16;
  *   y [T, N] f16 or f32 (y_dtype) with row stride ldy elements (y may be a column slice of a fused
  *   projection output); tok_adapter [T] int32.
  * Constraints: r in {8, 16, 32, 64}; K % 8 == 0; N % 8 == 0; ldy >= N, ldy % 8 == 0.
@@ -63,7 +73,7 @@ const char* mlora_last_error(void);
  *   contents need not be initialised.
  * ------------------------------------------------------------------------------------------- */
 size_t mlora_gather_mm_workspace_bytes(int T, int K, int r);
-int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, const void* A, const void* B,
+int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, int x_layout, const void* A, const void* B,
                     const int32_t* tok_adapter, float scaling,
                     int T, int K, int N, int r, int n_ad,
                     void* workspace, size_t workspace_bytes, void* stream);
@@ -72,7 +82,7 @@ int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, const void* A,
  *   shrink: v_part[c, t, :] = A[id_t][:, chunk c] . x[t, chunk c]   (fp32 partials per K-chunk)
  *   expand: y[t, :] += scaling * B[id_t] . sum_c v_part[c, t, :]
  * Same layouts and constraints; v_part is the workspace described above. */
-int mlora_lora_shrink(void* v_part, const void* x, const void* A, const int32_t* tok_adapter,
+int mlora_lora_shrink(void* v_part, const void* x, int x_layout, const void* A, const int32_t* tok_adapter,
                       int T, int K, int r, int n_ad, void* stream);
 int mlora_lora_expand(void* y, int y_dtype, int ldy, const void* v_part, const void* B, const int32_t* tok_adapter,
                       float scaling, int T, int K, int N, int r, int n_ad, void* stream);
@@ -118,15 +128,24 @@ int mlora_gemm_packed(void* y, int y_dtype, int mode, const void* x, int ldx, co
 int mlora_linear_packed(void* y, int y_dtype, int mode, const void* x, int ldx, const void* Wp,
                         int T, int K, int N, void* stream);
 
+/* Decode GEMV with both operands in fragment order: Wp as above, xf in MLORA_FRAG layout (T <= 64).  Every
+ * operand load of the kernel is then a contiguous 1 KiB block.  mlora_pack_activation converts a row-major
+ * x (row stride ldsrc) into fragment order for callers whose producer cannot write it directly. */
+size_t mlora_frag_activation_elems(int T, int K);
+int mlora_pack_activation(void* dst, const void* src, int ldsrc, int T, int K, void* stream);
+int mlora_gemv_frag(void* y, int y_dtype, int mode, const void* xf, const void* Wp,
+                    int T, int K, int N, void* stream);
+
 /* y[t, :] = f16( x[t, :] * rsqrt(mean(x[t, :]^2) + eps) * w )   row-wise, statistics in fp32.
  * Replaces: nn.RMSNorm(hidden, -1, eps, bias=False) (llama_for_causal_lm.py:76-77,93).
- * x [T, H] f16 or f32 (x_dtype), w [H] f16, y [T, H] f16.  H % 8 == 0, H <= 16384. */
-int mlora_rmsnorm(void* y, const void* x, int x_dtype, const void* w, float eps, int T, int H, void* stream);
+ * x [T, H] f16 or f32 (x_dtype), w [H] f16, y [T, H] f16 in y_layout.  H % 8 == 0, H <= 16384. */
+int mlora_rmsnorm(void* y, int y_layout, const void* x, int x_dtype, const void* w, float eps, int T, int H,
+                  void* stream);
 
 /* out[t, i] = f16( silu(gate[t, i]) * up[t, i] );  gate and up are column slices with row stride ld
  * (elements) so a fused [T, 2I] projection output can be passed as (p, p + I, 2I).
  * Replaces: op.silu(gate_proj(x)) * up_proj(x) (llama_for_causal_lm.py:35-36).  I % 8 == 0. */
-int mlora_silu_mul(void* out, const void* gate, const void* up, int ld, int T, int I, void* stream);
+int mlora_silu_mul(void* out, int out_layout, const void* gate, const void* up, int ld, int T, int I, void* stream);
 
 /* out[t, :] = table[ids[t], :] widened to out_dtype.  Replaces: nn.Embedding lookup
  * (llama_for_causal_lm.py:121-122).  table [V, H] f16; ids outside [0, V) produce a zero row. */
@@ -155,14 +174,15 @@ int mlora_argmax(int32_t* ids, const float* logits, int B, int V, void* stream);
  *   first ctx_len[b] cached positions of sequence seq_ids[b] (the new token already appended).
  * mlora_paged_attn_prefill: query token t (sequence tok_seq[t], position tok_pos[t]) attends to cached
  *   positions 0..tok_pos[t]; tokens of a sequence must be consecutive in t with increasing positions.
- * q is read from qkv (already rotated).  out [T, Hq, D] f16.  D in {64, 128}; Hq % Hkv == 0.
+ * q is read from qkv (already rotated).  out [T, Hq * D] f16 (decode: in out_layout).  D in {64, 128};
+ * Hq % Hkv == 0.
  * ------------------------------------------------------------------------------------------- */
 int mlora_rope_kv_append(void* qkv, void* k_cache, void* v_cache,
                          const int32_t* block_table, int max_blocks,
                          const int32_t* tok_seq, const int32_t* tok_pos,
                          const float* rope_cos, const float* rope_sin, int max_pos,
                          int T, int Hq, int Hkv, int D, int n_pages, int n_seq, void* stream);
-int mlora_paged_attn_decode(void* out, const void* qkv, const void* k_cache, const void* v_cache,
+int mlora_paged_attn_decode(void* out, int out_layout, const void* qkv, const void* k_cache, const void* v_cache,
                             const int32_t* block_table, int max_blocks,
                             const int32_t* seq_ids, const int32_t* ctx_len,
                             int B, int Hq, int Hkv, int D, int n_pages, int n_seq, void* stream);

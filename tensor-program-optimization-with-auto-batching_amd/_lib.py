@@ -11,6 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmlora_hip.so")
 
 F16, F32 = 0, 1
+ROWMAJOR, FRAG = 0, 1
 STORE, ACCUMULATE = 0, 1
 PAGE_SIZE = 16
 
@@ -21,8 +22,8 @@ SIGNATURES = {
     "mlora_version": (_i, []),
     "mlora_last_error": (C.c_char_p, []),
     "mlora_gather_mm_workspace_bytes": (_z, [_i, _i, _i]),
-    "mlora_gather_mm": (_i, [_p, _i, _i, _p, _p, _p, _p, _f, _i, _i, _i, _i, _i, _p, _z, _p]),
-    "mlora_lora_shrink": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),
+    "mlora_gather_mm": (_i, [_p, _i, _i, _p, _i, _p, _p, _p, _f, _i, _i, _i, _i, _i, _p, _z, _p]),
+    "mlora_lora_shrink": (_i, [_p, _p, _i, _p, _p, _i, _i, _i, _i, _p]),
     "mlora_lora_expand": (_i, [_p, _i, _i, _p, _p, _p, _f, _i, _i, _i, _i, _i, _p]),
     "mlora_write_tensor_part": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
     "mlora_gemv": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
@@ -33,12 +34,15 @@ SIGNATURES = {
     "mlora_gemv_packed": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
     "mlora_gemm_packed": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
     "mlora_linear_packed": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p]),
-    "mlora_rmsnorm": (_i, [_p, _p, _i, _p, _f, _i, _i, _p]),
-    "mlora_silu_mul": (_i, [_p, _p, _p, _i, _i, _i, _p]),
+    "mlora_frag_activation_elems": (_z, [_i, _i]),
+    "mlora_pack_activation": (_i, [_p, _p, _i, _i, _i, _p]),
+    "mlora_gemv_frag": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p]),
+    "mlora_rmsnorm": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _p]),
+    "mlora_silu_mul": (_i, [_p, _i, _p, _p, _i, _i, _i, _p]),
     "mlora_embed": (_i, [_p, _i, _p, _p, _i, _i, _i, _p]),
     "mlora_argmax": (_i, [_p, _p, _i, _i, _p]),
     "mlora_rope_kv_append": (_i, [_p, _p, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
-    "mlora_paged_attn_decode": (_i, [_p, _p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
+    "mlora_paged_attn_decode": (_i, [_p, _i, _p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "mlora_paged_attn_prefill": (_i, [_p, _p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
 }
 

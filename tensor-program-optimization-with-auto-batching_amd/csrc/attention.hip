@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void paged_attn_decode_kernel(f16* __restrict_
                                                                 const int32_t* __restrict__ block_table, int max_blocks,
                                                                 const int32_t* __restrict__ seq_ids,
                                                                 const int32_t* __restrict__ ctx_len, int Hq, int Hkv,
-                                                                int n_pages, int n_seq, float scale) {
+                                                                int n_pages, int n_seq, float scale, int frag_tt) {
   constexpr int LPT = D / 8;          // lanes sharing one token of a K load
   constexpr int TPL = WAVE / LPT;     // tokens per K load
   constexpr int NK = PAGE / TPL;      // K loads per page
@@ -165,7 +165,8 @@ __global__ __launch_bounds__(256) void paged_attn_decode_kernel(f16* __restrict_
       L += sl[w] * f;
       o += sacc[w][threadIdx.x] * f;
     }
-    out[((size_t)b * Hq + h) * D + threadIdx.x] = (f16)(L > 0.f ? o / L : 0.f);
+    const size_t oo = frag_tt ? frag_offset(b, h * D + threadIdx.x, frag_tt) : ((size_t)b * Hq + h) * D + threadIdx.x;
+    out[oo] = (f16)(L > 0.f ? o / L : 0.f);
   }
 }
 
@@ -316,22 +317,25 @@ extern "C" int mlora_rope_kv_append(void* qkv, void* k_cache, void* v_cache, con
   return mlora_launch_status("rope_kv_append");
 }
 
-extern "C" int mlora_paged_attn_decode(void* out, const void* qkv, const void* k_cache, const void* v_cache,
+extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qkv, const void* k_cache, const void* v_cache,
                                        const int32_t* block_table, int max_blocks, const int32_t* seq_ids,
                                        const int32_t* ctx_len, int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
                                        void* stream) {
   if (int e = check_attn("paged_attn_decode", Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
   MLORA_CHECK(out && qkv && k_cache && v_cache && block_table && seq_ids && ctx_len, MLORA_ERR_INVALID, "paged_attn_decode: null pointer");
   MLORA_CHECK(B >= 0, MLORA_ERR_INVALID, "paged_attn_decode: bad B=%d", B);
+  MLORA_CHECK(out_layout == MLORA_ROWMAJOR || (out_layout == MLORA_FRAG && B <= 64), MLORA_ERR_UNSUPPORTED,
+              "paged_attn_decode: fragment-ordered output needs B <= 64 (layout=%d B=%d)", out_layout, B);
+  const int frag_tt = out_layout == MLORA_FRAG ? mlora_frag_tiles(B) : 0;
   if (B == 0) return MLORA_OK;
   const float scale = 1.f / sqrtf((float)D);
   hipStream_t s = (hipStream_t)stream;
   if (D == 128)
     hipLaunchKernelGGL(paged_attn_decode_kernel<128>, dim3(B, Hq), dim3(256), 0, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
-                       (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale);
+                       (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale, frag_tt);
   else
     hipLaunchKernelGGL(paged_attn_decode_kernel<64>, dim3(B, Hq), dim3(256), 0, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
-                       (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale);
+                       (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale, frag_tt);
   return mlora_launch_status("paged_attn_decode");
 }
 

@@ -36,9 +36,19 @@ static inline int mlora_launch_status(const char* what) {
 
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// 16-token tiles of the fragment-ordered activation layout: the tile count the decode GEMV is compiled
+// for (1, 2 or 4), so that producer and consumer agree on the stride between k-steps.
+static inline int mlora_frag_tiles(int T) { return T <= 16 ? 1 : (T <= 32 ? 2 : 4); }
+
 // ---------------------------------------------------------------------------------------------
 // device side
 // ---------------------------------------------------------------------------------------------
+// Element offset of x[t, k] in the fragment-ordered activation layout with TT 16-token tiles:
+//   Xf[k/32][t/16][(k%32)/8][t%16][k%8]
+__device__ __forceinline__ size_t frag_offset(int t, int k, int TT) {
+  return ((((size_t)(k >> 5) * TT + (t >> 4)) * 4 + ((k >> 3) & 3)) * 16 + (t & 15)) * 8 + (k & 7);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);

@@ -53,7 +53,8 @@ __device__ __forceinline__ int reduce_transpose(float (&p)[G], int lane) {
 template <int R>
 __global__ __launch_bounds__(64) void lora_shrink_kernel(float* __restrict__ vpart, const f16* __restrict__ x,
                                                          const f16* __restrict__ A,
-                                                         const int32_t* __restrict__ ids, int T, int K, int CI) {
+                                                         const int32_t* __restrict__ ids, int T, int K, int CI,
+                                                         int frag_tt) {
   constexpr int G = R < 16 ? R : 16;   // A rows held in registers at once
   constexpr int TB = 4;                // tokens in flight
   const int a = blockIdx.x;
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(64) void lora_shrink_kernel(float* __restrict__ vpa
 #pragma unroll
           for (int u = 0; u < TB; ++u) {
             xv[u] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-            if (kin && tt[u] >= 0) xv[u] = ld8(x + (size_t)tt[u] * K + k);
+            if (kin && tt[u] >= 0) xv[u] = ld8(x + (frag_tt ? frag_offset(tt[u], k, frag_tt) : (size_t)tt[u] * K + k));
           }
           f16x8 areg[G];
 #pragma unroll
@@ -236,9 +237,10 @@ int check_lora_shape(int T, int K, int N, int r, int n_ad) {
 }
 
 template <int R>
-void launch_shrink(float* vpart, const f16* x, const f16* A, const int32_t* ids, int T, int K, int n_ad, hipStream_t s) {
+void launch_shrink(float* vpart, const f16* x, int frag_tt, const f16* A, const int32_t* ids, int T, int K, int n_ad,
+                   hipStream_t s) {
   const KSplit ks = k_split(K);
-  hipLaunchKernelGGL(lora_shrink_kernel<R>, dim3(n_ad, ks.kc), dim3(64), 0, s, vpart, x, A, ids, T, K, ks.ci);
+  hipLaunchKernelGGL(lora_shrink_kernel<R>, dim3(n_ad, ks.kc), dim3(64), 0, s, vpart, x, A, ids, T, K, ks.ci, frag_tt);
 }
 
 template <int R, typename YT>
@@ -256,9 +258,12 @@ extern "C" size_t mlora_gather_mm_workspace_bytes(int T, int K, int r) {
   return (size_t)k_split(K).kc * (size_t)T * (size_t)r * sizeof(float);
 }
 
-extern "C" int mlora_lora_shrink(void* v_part, const void* x, const void* A, const int32_t* tok_adapter, int T, int K,
-                                 int r, int n_ad, void* stream) {
+extern "C" int mlora_lora_shrink(void* v_part, const void* x, int x_layout, const void* A, const int32_t* tok_adapter,
+                                 int T, int K, int r, int n_ad, void* stream) {
   if (int e = check_lora_shape(T, K, 8, r, n_ad)) return e;
+  MLORA_CHECK(x_layout == MLORA_ROWMAJOR || (x_layout == MLORA_FRAG && T <= 64 && K % 32 == 0), MLORA_ERR_UNSUPPORTED,
+              "lora_shrink: fragment-ordered x needs T <= 64 and K %% 32 == 0 (layout=%d T=%d K=%d)", x_layout, T, K);
+  const int frag_tt = x_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   MLORA_CHECK(v_part && x && A && tok_adapter, MLORA_ERR_INVALID, "lora_shrink: null pointer");
   if (T == 0) return MLORA_OK;
   hipStream_t s = (hipStream_t)stream;
@@ -266,10 +271,10 @@ extern "C" int mlora_lora_shrink(void* v_part, const void* x, const void* A, con
   const f16* xp = (const f16*)x;
   const f16* Ap = (const f16*)A;
   switch (r) {
-    case 8: launch_shrink<8>(vp, xp, Ap, tok_adapter, T, K, n_ad, s); break;
-    case 16: launch_shrink<16>(vp, xp, Ap, tok_adapter, T, K, n_ad, s); break;
-    case 32: launch_shrink<32>(vp, xp, Ap, tok_adapter, T, K, n_ad, s); break;
-    default: launch_shrink<64>(vp, xp, Ap, tok_adapter, T, K, n_ad, s); break;
+    case 8: launch_shrink<8>(vp, xp, frag_tt, Ap, tok_adapter, T, K, n_ad, s); break;
+    case 16: launch_shrink<16>(vp, xp, frag_tt, Ap, tok_adapter, T, K, n_ad, s); break;
+    case 32: launch_shrink<32>(vp, xp, frag_tt, Ap, tok_adapter, T, K, n_ad, s); break;
+    default: launch_shrink<64>(vp, xp, frag_tt, Ap, tok_adapter, T, K, n_ad, s); break;
   }
   return mlora_launch_status("lora_shrink");
 }
@@ -298,14 +303,14 @@ extern "C" int mlora_lora_expand(void* y, int y_dtype, int ldy, const void* v_pa
   return mlora_launch_status("lora_expand");
 }
 
-extern "C" int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, const void* A, const void* B,
+extern "C" int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, int x_layout, const void* A, const void* B,
                                const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
                                void* workspace, size_t workspace_bytes, void* stream) {
   if (int e = check_lora_shape(T, K, N, r, n_ad)) return e;
   MLORA_CHECK(workspace && workspace_bytes >= mlora_gather_mm_workspace_bytes(T, K, r) || T == 0, MLORA_ERR_WORKSPACE,
               "gather_mm: workspace of %zu bytes given, %zu needed", workspace_bytes,
               mlora_gather_mm_workspace_bytes(T, K, r));
-  if (int e = mlora_lora_shrink(workspace, x, A, tok_adapter, T, K, r, n_ad, stream)) return e;
+  if (int e = mlora_lora_shrink(workspace, x, x_layout, A, tok_adapter, T, K, r, n_ad, stream)) return e;
   return mlora_lora_expand(y, y_dtype, ldy, workspace, B, tok_adapter, scaling, T, K, N, r, n_ad, stream);
 }
 

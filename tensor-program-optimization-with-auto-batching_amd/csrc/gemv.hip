@@ -23,7 +23,7 @@ constexpr int PIPE = 4;     // k-steps in flight per wave
 
 enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2 };
 
-template <int NT, int TT, int OUT, bool PACKED>
+template <int NT, int TT, int OUT, bool PACKED, bool XFRAG>
 __global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx,
                                                                 const f16* __restrict__ W, int T, int K, int N) {
   __shared__ f32x4 red[GEMV_WAVES][NT * TT][WAVE];
@@ -47,11 +47,16 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(void* __restrict
       wp[i] = W + (size_t)n * K + kg * 8;
     }
   }
+  constexpr int XSTEP = XFRAG ? TT * 512 : KSTEP;   // elements between consecutive k-steps of the x fragments
 #pragma unroll
   for (int j = 0; j < TT; ++j) {
-    int t = j * 16 + r16;
-    t = t < T ? t : T - 1;
-    xp[j] = x + (size_t)t * ldx + kg * 8;
+    if constexpr (XFRAG) {
+      xp[j] = x + j * 512 + lane * 8;
+    } else {
+      int t = j * 16 + r16;
+      t = t < T ? t : T - 1;
+      xp[j] = x + (size_t)t * ldx + kg * 8;
+    }
   }
 
   f32x4 acc[NT][TT];
@@ -73,7 +78,7 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(void* __restrict
       if (!in) a[u][i] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
 #pragma unroll
-    for (int j = 0; j < TT; ++j) b[u][j] = ld8(xp[j] + ks * KSTEP);
+    for (int j = 0; j < TT; ++j) b[u][j] = ld8(xp[j] + (size_t)ks * XSTEP);
   };
 #pragma unroll
   for (int u = 0; u < PIPE; ++u) load_stage(u, u);
@@ -134,15 +139,28 @@ __global__ __launch_bounds__(256) void pack_weight_kernel(f16* __restrict__ dst,
   st8(dst + c * 8, v);
 }
 
-template <int NT, int TT, bool PACKED>
-void launch_gemv(void* y, int out, const f16* x, int ldx, const f16* W, int T, int K, int N, hipStream_t s) {
-  const dim3 grid(ceil_div(N, 16 * NT)), block(GEMV_WAVES * WAVE);
-  if (out == OUT_F16) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F16, PACKED>), grid, block, 0, s, y, x, ldx, W, T, K, N);
-  else if (out == OUT_F32) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F32, PACKED>), grid, block, 0, s, y, x, ldx, W, T, K, N);
-  else hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_ACC_F32, PACKED>), grid, block, 0, s, y, x, ldx, W, T, K, N);
+// one thread per 16-byte chunk of the fragment-ordered activation block
+__global__ __launch_bounds__(256) void pack_activation_kernel(f16* __restrict__ dst, const f16* __restrict__ src, int ldsrc,
+                                                              int T, int K, int TT, int chunks) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= chunks) return;
+  const int t16 = c & 15, kg = (c >> 4) & 3, blk = c >> 6;
+  const int tt = blk % TT, ks = blk / TT;
+  const int t = tt * 16 + t16;
+  f16x8 v = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  if (t < T) v = ld8(src + (size_t)t * ldsrc + ks * KSTEP + kg * 8);
+  st8(dst + (size_t)c * 8, v);
 }
 
-template <bool PACKED>
+template <int NT, int TT, bool PACKED, bool XFRAG>
+void launch_gemv(void* y, int out, const f16* x, int ldx, const f16* W, int T, int K, int N, hipStream_t s) {
+  const dim3 grid(ceil_div(N, 16 * NT)), block(GEMV_WAVES * WAVE);
+  if (out == OUT_F16) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F16, PACKED, XFRAG>), grid, block, 0, s, y, x, ldx, W, T, K, N);
+  else if (out == OUT_F32) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F32, PACKED, XFRAG>), grid, block, 0, s, y, x, ldx, W, T, K, N);
+  else hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_ACC_F32, PACKED, XFRAG>), grid, block, 0, s, y, x, ldx, W, T, K, N);
+}
+
+template <bool PACKED, bool XFRAG>
 int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K, int N, void* stream) {
   const int out = mode == MLORA_ACCUMULATE ? OUT_ACC_F32 : (y_dtype == MLORA_F32 ? OUT_F32 : OUT_F16);
   hipStream_t s = (hipStream_t)stream;
@@ -153,13 +171,13 @@ int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const 
   const int tiles = ceil_div(N, 16);
   const bool wide = tiles >= 512 && (!PACKED || tiles % 2 == 0);
   if (T <= 16) {
-    if (wide) launch_gemv<2, 1, PACKED>(y, out, xp, ldx, Wp, T, K, N, s);
-    else launch_gemv<1, 1, PACKED>(y, out, xp, ldx, Wp, T, K, N, s);
+    if (wide) launch_gemv<2, 1, PACKED, XFRAG>(y, out, xp, ldx, Wp, T, K, N, s);
+    else launch_gemv<1, 1, PACKED, XFRAG>(y, out, xp, ldx, Wp, T, K, N, s);
   } else if (T <= 32) {
-    if (wide) launch_gemv<2, 2, PACKED>(y, out, xp, ldx, Wp, T, K, N, s);
-    else launch_gemv<1, 2, PACKED>(y, out, xp, ldx, Wp, T, K, N, s);
+    if (wide) launch_gemv<2, 2, PACKED, XFRAG>(y, out, xp, ldx, Wp, T, K, N, s);
+    else launch_gemv<1, 2, PACKED, XFRAG>(y, out, xp, ldx, Wp, T, K, N, s);
   } else {
-    launch_gemv<1, 4, PACKED>(y, out, xp, ldx, Wp, T, K, N, s);
+    launch_gemv<1, 4, PACKED, XFRAG>(y, out, xp, ldx, Wp, T, K, N, s);
   }
   return mlora_launch_status("gemv");
 }
@@ -183,7 +201,7 @@ extern "C" int mlora_gemv(void* y, int y_dtype, int mode, const void* x, int ldx
   if (int e = mlora_check_linear("gemv", y, y_dtype, mode, x, ldx, W, T, K, N)) return e;
   MLORA_CHECK(T <= 64, MLORA_ERR_UNSUPPORTED, "gemv: T=%d exceeds 64 (use mlora_gemm)", T);
   if (T == 0) return MLORA_OK;
-  return gemv_dispatch<false>(y, y_dtype, mode, x, ldx, W, T, K, N, stream);
+  return gemv_dispatch<false, false>(y, y_dtype, mode, x, ldx, W, T, K, N, stream);
 }
 
 extern "C" int mlora_gemv_packed(void* y, int y_dtype, int mode, const void* x, int ldx, const void* Wp, int T, int K,
@@ -191,7 +209,30 @@ extern "C" int mlora_gemv_packed(void* y, int y_dtype, int mode, const void* x, 
   if (int e = mlora_check_linear("gemv_packed", y, y_dtype, mode, x, ldx, Wp, T, K, N)) return e;
   MLORA_CHECK(T <= 64, MLORA_ERR_UNSUPPORTED, "gemv_packed: T=%d exceeds 64 (use mlora_gemm_packed)", T);
   if (T == 0) return MLORA_OK;
-  return gemv_dispatch<true>(y, y_dtype, mode, x, ldx, Wp, T, K, N, stream);
+  return gemv_dispatch<true, false>(y, y_dtype, mode, x, ldx, Wp, T, K, N, stream);
+}
+
+extern "C" int mlora_gemv_frag(void* y, int y_dtype, int mode, const void* xf, const void* Wp, int T, int K, int N,
+                               void* stream) {
+  if (int e = mlora_check_linear("gemv_frag", y, y_dtype, mode, xf, K, Wp, T, K, N)) return e;
+  MLORA_CHECK(T <= 64, MLORA_ERR_UNSUPPORTED, "gemv_frag: T=%d exceeds 64", T);
+  if (T == 0) return MLORA_OK;
+  return gemv_dispatch<true, true>(y, y_dtype, mode, xf, K, Wp, T, K, N, stream);
+}
+
+extern "C" size_t mlora_frag_activation_elems(int T, int K) {
+  if (T <= 0 || K <= 0) return 0;
+  return (size_t)mlora_frag_tiles(T) * 16 * (size_t)K;
+}
+
+extern "C" int mlora_pack_activation(void* dst, const void* src, int ldsrc, int T, int K, void* stream) {
+  MLORA_CHECK(dst && src && dst != src, MLORA_ERR_INVALID, "pack_activation: null or aliasing pointers");
+  MLORA_CHECK(T > 0 && T <= 64 && K > 0 && K % 32 == 0 && ldsrc >= K && ldsrc % 8 == 0, MLORA_ERR_UNSUPPORTED,
+              "pack_activation: need 0 < T <= 64, K %% 32 == 0, ldsrc >= K (T=%d K=%d ldsrc=%d)", T, K, ldsrc);
+  const int chunks = mlora_frag_tiles(T) * 16 * (K / 8);
+  hipLaunchKernelGGL(pack_activation_kernel, dim3(ceil_div(chunks, 256)), dim3(256), 0, (hipStream_t)stream, (f16*)dst,
+                     (const f16*)src, ldsrc, T, K, mlora_frag_tiles(T), chunks);
+  return mlora_launch_status("pack_activation");
 }
 
 extern "C" size_t mlora_packed_weight_elems(int N, int K) {

@@ -21,7 +21,7 @@ __device__ __forceinline__ float block_sum(float v, float* lds) {
 // One block per row; each thread keeps up to VPT 8-element vectors of the row in registers.
 template <typename XT, int VPT>
 __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(f16* __restrict__ y, const XT* __restrict__ x,
-                                                              const f16* __restrict__ w, float eps, int H) {
+                                                              const f16* __restrict__ w, float eps, int H, int frag_tt) {
   __shared__ float lds[ROW_THREADS / WAVE];
   const int row = blockIdx.x;
   const XT* xr = x + (size_t)row * H;
@@ -58,13 +58,13 @@ __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(f16* __restrict__ 
       f16x8 o;
 #pragma unroll
       for (int e = 0; e < 8; ++e) o[e] = (f16)(v[i][e] * inv * (float)wv[e]);
-      st8(y + (size_t)row * H + c, o);
+      st8(y + (frag_tt ? frag_offset(row, c, frag_tt) : (size_t)row * H + c), o);
     }
   }
 }
 
 __global__ __launch_bounds__(ROW_THREADS) void silu_mul_kernel(f16* __restrict__ out, const f16* __restrict__ gate,
-                                                               const f16* __restrict__ up, int ld, int I) {
+                                                               const f16* __restrict__ up, int ld, int I, int frag_tt) {
   const int row = blockIdx.y;
   const int c = (blockIdx.x * ROW_THREADS + threadIdx.x) * 8;
   if (c >= I) return;
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(ROW_THREADS) void silu_mul_kernel(f16* __restrict__
     const float gf = (float)g[e];
     o[e] = (f16)(gf / (1.f + expf(-gf)) * (float)u[e]);
   }
-  st8(out + (size_t)row * I + c, o);
+  st8(out + (frag_tt ? frag_offset(row, c, frag_tt) : (size_t)row * I + c), o);
 }
 
 template <typename OT>
@@ -134,7 +134,11 @@ __global__ __launch_bounds__(ROW_THREADS) void argmax_kernel(int32_t* __restrict
 
 }  // namespace
 
-extern "C" int mlora_rmsnorm(void* y, const void* x, int x_dtype, const void* w, float eps, int T, int H, void* stream) {
+extern "C" int mlora_rmsnorm(void* y, int y_layout, const void* x, int x_dtype, const void* w, float eps, int T, int H,
+                             void* stream) {
+  MLORA_CHECK(y_layout == MLORA_ROWMAJOR || (y_layout == MLORA_FRAG && T <= 64 && H % 32 == 0), MLORA_ERR_UNSUPPORTED,
+              "rmsnorm: fragment-ordered output needs T <= 64 and H %% 32 == 0 (layout=%d T=%d H=%d)", y_layout, T, H);
+  const int frag_tt = y_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   MLORA_CHECK(y && x && w, MLORA_ERR_INVALID, "rmsnorm: null pointer");
   MLORA_CHECK(T >= 0 && H > 0 && H % 8 == 0 && H <= 16384, MLORA_ERR_UNSUPPORTED, "rmsnorm: need H %% 8 == 0, H <= 16384 (T=%d H=%d)", T, H);
   MLORA_CHECK(x_dtype == MLORA_F16 || x_dtype == MLORA_F32, MLORA_ERR_INVALID, "rmsnorm: bad x_dtype %d", x_dtype);
@@ -142,7 +146,7 @@ extern "C" int mlora_rmsnorm(void* y, const void* x, int x_dtype, const void* w,
   hipStream_t s = (hipStream_t)stream;
   const int vpt = ceil_div(H, ROW_THREADS * 8);
 #define MLORA_RMS(XT, VPT) \
-  hipLaunchKernelGGL((rmsnorm_kernel<XT, VPT>), dim3(T), dim3(ROW_THREADS), 0, s, (f16*)y, (const XT*)x, (const f16*)w, eps, H)
+  hipLaunchKernelGGL((rmsnorm_kernel<XT, VPT>), dim3(T), dim3(ROW_THREADS), 0, s, (f16*)y, (const XT*)x, (const f16*)w, eps, H, frag_tt)
   if (x_dtype == MLORA_F16) {
     if (vpt <= 2) MLORA_RMS(f16, 2);
     else if (vpt <= 4) MLORA_RMS(f16, 4);
@@ -156,13 +160,17 @@ extern "C" int mlora_rmsnorm(void* y, const void* x, int x_dtype, const void* w,
   return mlora_launch_status("rmsnorm");
 }
 
-extern "C" int mlora_silu_mul(void* out, const void* gate, const void* up, int ld, int T, int I, void* stream) {
+extern "C" int mlora_silu_mul(void* out, int out_layout, const void* gate, const void* up, int ld, int T, int I,
+                              void* stream) {
+  MLORA_CHECK(out_layout == MLORA_ROWMAJOR || (out_layout == MLORA_FRAG && T <= 64 && I % 32 == 0), MLORA_ERR_UNSUPPORTED,
+              "silu_mul: fragment-ordered output needs T <= 64 and I %% 32 == 0 (layout=%d T=%d I=%d)", out_layout, T, I);
+  const int frag_tt = out_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   MLORA_CHECK(out && gate && up, MLORA_ERR_INVALID, "silu_mul: null pointer");
   MLORA_CHECK(T >= 0 && I > 0 && I % 8 == 0 && ld >= I && ld % 8 == 0, MLORA_ERR_UNSUPPORTED, "silu_mul: need I %% 8 == 0, ld >= I, ld %% 8 == 0 (T=%d I=%d ld=%d)", T, I, ld);
   MLORA_CHECK(T <= 65535, MLORA_ERR_UNSUPPORTED, "silu_mul: T=%d exceeds 65535", T);
   if (T == 0) return MLORA_OK;
   hipLaunchKernelGGL(silu_mul_kernel, dim3(ceil_div(I, ROW_THREADS * 8), T), dim3(ROW_THREADS), 0, (hipStream_t)stream,
-                     (f16*)out, (const f16*)gate, (const f16*)up, ld, I);
+                     (f16*)out, (const f16*)gate, (const f16*)up, ld, I, frag_tt);
   return mlora_launch_status("silu_mul");
 }
 

@@ -136,29 +136,31 @@ class LlamaForCausalLM:
         H, I = s.hidden_size, s.intermediate_size
         q_sz, kv_sz = s.q_size, s.kv_size
         resid = hidden
+        # a decode step (one token per sequence, T <= 64) keeps its activations in fragment order
+        frag = T <= 64 and kv._cur is not None and kv._cur[2]
         for l, L in enumerate(self.layers):
-            xn = ops.rmsnorm(resid, L["ln1"], s.rms_norm_eps)
+            xn = ops.rmsnorm(resid, L["ln1"], s.rms_norm_eps, frag=frag)
             qkv = ops.linear(xn, L["qkv"])
             if tok_adapter:
                 self._lora(qkv[:, :q_sz], xn, l, "q_proj", tok_adapter)
                 self._lora(qkv[:, q_sz:q_sz + kv_sz], xn, l, "k_proj", tok_adapter)
                 self._lora(qkv[:, q_sz + kv_sz:], xn, l, "v_proj", tok_adapter)
-            attn = kv.attention_with_fused_qkv(l, qkv, s.num_attention_heads)
+            attn = kv.attention_with_fused_qkv(l, qkv, s.num_attention_heads, frag=frag)
             ops.linear(attn, L["o"], out=resid, accumulate=True)
             if tok_adapter:
                 self._lora(resid, attn, l, "o_proj", tok_adapter)
-            xn = ops.rmsnorm(resid, L["ln2"], s.rms_norm_eps)
+            xn = ops.rmsnorm(resid, L["ln2"], s.rms_norm_eps, frag=frag)
             gu = ops.linear(xn, L["gate_up"])
             if tok_adapter:
                 self._lora(gu[:, :I], xn, l, "gate_proj", tok_adapter)
                 self._lora(gu[:, I:], xn, l, "up_proj", tok_adapter)
-            act = ops.silu_mul(gu)
+            act = ops.silu_mul(gu, frag=frag)
             ops.linear(act, L["down"], out=resid, accumulate=True)
             if tok_adapter:
                 self._lora(resid, act, l, "down_proj", tok_adapter)
         if logits_rows is not None:
             resid = resid[logits_rows].contiguous()
-        xn = ops.rmsnorm(resid, self.norm, s.rms_norm_eps)
+        xn = ops.rmsnorm(resid, self.norm, s.rms_norm_eps, frag=resid.shape[0] <= 64)
         return ops.linear(xn, self.lm_head, out_dtype=torch.float32)
 
     # ------------------------------------------------------------------ reference entry points

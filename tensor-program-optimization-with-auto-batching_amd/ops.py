@@ -8,7 +8,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from ._lib import F16, F32, STORE, ACCUMULATE, PAGE_SIZE, check, lib
+from ._lib import F16, F32, ROWMAJOR, FRAG, STORE, ACCUMULATE, PAGE_SIZE, check, lib
 
 
 def _stream() -> int:
@@ -33,6 +33,47 @@ def _dt(t: torch.Tensor) -> int:
     raise TypeError(f"expected float16 or float32, got {t.dtype}")
 
 
+class FragActivation:
+    """A [T, K] fp16 activation block (T <= 64) stored in matrix-core fragment order (MLORA_FRAG)."""
+
+    def __init__(self, T: int, K: int, device, data: torch.Tensor = None):
+        self.T, self.K = T, K
+        n = lib().mlora_frag_activation_elems(T, K)
+        self.data = torch.empty(n, dtype=torch.float16, device=device) if data is None else data
+        if self.data.numel() < n:
+            raise ValueError("FragActivation: buffer too small")
+
+    @property
+    def shape(self):
+        return (self.T, self.K)
+
+    @property
+    def device(self):
+        return self.data.device
+
+    @classmethod
+    def pack(cls, x: torch.Tensor, out: "FragActivation" = None):
+        """Row-major [T, K] fp16 (unit inner stride) -> fragment order."""
+        T, K = x.shape
+        out = cls(T, K, x.device) if out is None else out
+        ld = x.stride(0) if T > 1 else max(K, x.stride(0))
+        check(lib().mlora_pack_activation(out.data.data_ptr(), x.data_ptr(), ld, T, K, _stream()))
+        return out
+
+    def unpack(self) -> torch.Tensor:
+        """Back to row-major [T, K] (host-side index arithmetic on the device tensor; for tests)."""
+        TT = 1 if self.T <= 16 else (2 if self.T <= 32 else 4)
+        v = self.data[: TT * 16 * self.K].view(self.K // 32, TT, 4, 16, 8)
+        return v.permute(1, 3, 0, 2, 4).reshape(TT * 16, self.K)[: self.T].contiguous()
+
+
+def _x_arg(x, name="x"):
+    """(pointer, layout, T, K) of a row-major tensor or a FragActivation."""
+    if isinstance(x, FragActivation):
+        return x.data.data_ptr(), FRAG, x.T, x.K
+    return _dev(x, torch.float16, name), ROWMAJOR, x.shape[0], x.shape[1]
+
+
 def gather_mm_workspace(T: int, K: int, r: int, device) -> torch.Tensor:
     n = lib().mlora_gather_mm_workspace_bytes(T, K, r)
     return torch.empty(max(n, 16) // 4, dtype=torch.float32, device=device)
@@ -42,7 +83,7 @@ def gather_mm(y, x, A, B, tok_adapter, scaling: float, workspace=None):
     """y[t] += scaling * B[id_t] @ (A[id_t] @ x[t]) in place.  y [T,N] f16|f32 (rows may be strided: a
     column slice of a wider buffer), x [T,K] f16, A [n_ad,r,K] f16, B [n_ad,N,r] f16,
     tok_adapter [T] int32 (-1 = no adapter)."""
-    T, K = x.shape
+    xptr, xlay, T, K = _x_arg(x)
     n_ad, r, K2 = A.shape
     N = B.shape[1]
     if K2 != K or B.shape != (n_ad, N, r) or y.shape != (T, N) or tok_adapter.shape != (T,):
@@ -53,7 +94,7 @@ def gather_mm(y, x, A, B, tok_adapter, scaling: float, workspace=None):
     if not y.is_cuda or y.stride(1) != 1:
         raise ValueError("gather_mm: y must be a GPU tensor with unit inner stride")
     ldy = y.stride(0) if T > 1 else max(N, y.stride(0))
-    check(lib().mlora_gather_mm(y.data_ptr(), _dt(y), ldy, _dev(x, torch.float16, "x"), _dev(A, torch.float16, "A"),
+    check(lib().mlora_gather_mm(y.data_ptr(), _dt(y), ldy, xptr, xlay, _dev(A, torch.float16, "A"),
                                 _dev(B, torch.float16, "B"), _dev(tok_adapter, torch.int32, "tok_adapter"),
                                 float(scaling), T, K, N, r, n_ad, _dev(workspace, torch.float32, "workspace"),
                                 workspace.numel() * 4, _stream()))
@@ -61,9 +102,9 @@ def gather_mm(y, x, A, B, tok_adapter, scaling: float, workspace=None):
 
 
 def lora_shrink(v_part, x, A, tok_adapter):
-    T, K = x.shape
+    xptr, xlay, T, K = _x_arg(x)
     n_ad, r, _ = A.shape
-    check(lib().mlora_lora_shrink(_dev(v_part, torch.float32), _dev(x, torch.float16), _dev(A, torch.float16),
+    check(lib().mlora_lora_shrink(_dev(v_part, torch.float32), xptr, xlay, _dev(A, torch.float16),
                                   _dev(tok_adapter, torch.int32), T, K, r, n_ad, _stream()))
     return v_part
 
@@ -102,8 +143,10 @@ class PackedWeight:
 
 
 def linear(x, W, out=None, out_dtype=torch.float16, accumulate=False, kernel="auto"):
-    """y (=|+=) x @ W.T.  x [T,K] f16 (row stride may exceed K), W [N,K] f16 or a PackedWeight.
-    accumulate=True adds into the fp32 tensor `out`."""
+    """y (=|+=) x @ W.T.  x [T,K] f16 (row stride may exceed K) or a FragActivation, W [N,K] f16 or a
+    PackedWeight.  accumulate=True adds into the fp32 tensor `out`."""
+    if isinstance(x, FragActivation):
+        return _linear_frag(x, W, out, out_dtype, accumulate)
     T, K = x.shape
     packed = isinstance(W, PackedWeight)
     N, K2 = W.shape
@@ -128,22 +171,49 @@ def linear(x, W, out=None, out_dtype=torch.float16, accumulate=False, kernel="au
     return out
 
 
-def rmsnorm(x, w, eps: float, out=None):
-    T, H = x.shape
+def _linear_frag(x, W, out, out_dtype, accumulate):
+    if not isinstance(W, PackedWeight):
+        raise TypeError("a fragment-ordered activation needs a PackedWeight")
+    T, K = x.shape
+    N, K2 = W.shape
+    if K2 != K:
+        raise ValueError(f"linear: x{x.shape} vs W{W.shape}")
     if out is None:
-        out = torch.empty((T, H), dtype=torch.float16, device=x.device)
-    check(lib().mlora_rmsnorm(_dev(out, torch.float16), _dev(x), _dt(x), _dev(w, torch.float16), float(eps), T, H, _stream()))
+        if accumulate:
+            raise ValueError("linear: accumulate needs out")
+        out = torch.empty((T, N), dtype=out_dtype, device=x.device)
+    if out.shape != (T, N):
+        raise ValueError(f"linear: out{tuple(out.shape)} expected {(T, N)}")
+    check(lib().mlora_gemv_frag(_dev(out), _dt(out), ACCUMULATE if accumulate else STORE, x.data.data_ptr(),
+                                W.data.data_ptr(), T, K, N, _stream()))
     return out
 
 
-def silu_mul(gate_up, out=None):
+def _out_arg(out, T, H, frag, device):
+    """Output buffer of a producer: row-major tensor or FragActivation."""
+    if frag:
+        out = FragActivation(T, H, device) if out is None else out
+        return out, out.data.data_ptr(), FRAG
+    if out is None:
+        out = torch.empty((T, H), dtype=torch.float16, device=device)
+    return out, _dev(out, torch.float16, "out"), ROWMAJOR
+
+
+def rmsnorm(x, w, eps: float, out=None, frag=False):
+    """Row-wise RMSNorm of x [T, H] (f16 | f32); frag=True writes a FragActivation."""
+    T, H = x.shape
+    out, optr, lay = _out_arg(out, T, H, frag, x.device)
+    check(lib().mlora_rmsnorm(optr, lay, _dev(x), _dt(x), _dev(w, torch.float16), float(eps), T, H, _stream()))
+    return out
+
+
+def silu_mul(gate_up, out=None, frag=False):
     """gate_up [T, 2I] (gate columns first) -> silu(gate) * up [T, I]."""
     T, I2 = gate_up.shape
     I = I2 // 2
-    if out is None:
-        out = torch.empty((T, I), dtype=torch.float16, device=gate_up.device)
+    out, optr, lay = _out_arg(out, T, I, frag, gate_up.device)
     p = _dev(gate_up, torch.float16)
-    check(lib().mlora_silu_mul(_dev(out, torch.float16), p, p + I * 2, I2, T, I, _stream()))
+    check(lib().mlora_silu_mul(optr, lay, p, p + I * 2, I2, T, I, _stream()))
     return out
 
 
@@ -151,7 +221,7 @@ def silu_mul_split(gate, up, out=None):
     T, I = gate.shape
     if out is None:
         out = torch.empty((T, I), dtype=torch.float16, device=gate.device)
-    check(lib().mlora_silu_mul(_dev(out, torch.float16), _dev(gate, torch.float16), _dev(up, torch.float16), I, T, I, _stream()))
+    check(lib().mlora_silu_mul(_dev(out, torch.float16), ROWMAJOR, _dev(gate, torch.float16), _dev(up, torch.float16), I, T, I, _stream()))
     return out
 
 
@@ -184,12 +254,11 @@ def rope_kv_append(qkv, k_cache, v_cache, block_table, tok_seq, tok_pos, rope_co
                                      max_pos, T, Hq, Hkv, D, n_pages, n_seq, _stream()))
 
 
-def paged_attn_decode(qkv, k_cache, v_cache, block_table, seq_ids, ctx_len, Hq, Hkv, D, out=None):
+def paged_attn_decode(qkv, k_cache, v_cache, block_table, seq_ids, ctx_len, Hq, Hkv, D, out=None, frag=False):
     B = qkv.shape[0]
     n_seq, max_blocks = block_table.shape
-    if out is None:
-        out = torch.empty((B, Hq * D), dtype=torch.float16, device=qkv.device)
-    check(lib().mlora_paged_attn_decode(_dev(out, torch.float16), _dev(qkv, torch.float16), _dev(k_cache, torch.float16),
+    out, optr, lay = _out_arg(out, B, Hq * D, frag, qkv.device)
+    check(lib().mlora_paged_attn_decode(optr, lay, _dev(qkv, torch.float16), _dev(k_cache, torch.float16),
                                         _dev(v_cache, torch.float16), _dev(block_table, torch.int32), max_blocks,
                                         _dev(seq_ids, torch.int32), _dev(ctx_len, torch.int32), B, Hq, Hkv, D,
                                         k_cache.shape[0], n_seq, _stream()))

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 def test_argument_validation_without_gpu():
     """Shape checks happen on the host before any launch, so they can be exercised without a GPU."""
     lib = load_pkg("_lib").lib()
-    assert lib.mlora_gather_mm(1, 0, 64, 1, 1, 1, 1, 1.0, 4, 64, 64, 12, 2, 1, 1 << 20, None) == -2
+    assert lib.mlora_gather_mm(1, 0, 64, 1, 0, 1, 1, 1, 1.0, 4, 64, 64, 12, 2, 1, 1 << 20, None) == -2
     assert b"rank" in lib.mlora_last_error()
     assert lib.mlora_gather_mm_workspace_bytes(64, 4096, 16) == 8 * 64 * 16 * 4
     assert lib.mlora_gather_mm_workspace_bytes(32, 11008, 64) == 8 * 32 * 64 * 4
@@ -38,9 +38,11 @@ def test_argument_validation_without_gpu():
     assert lib.mlora_gemv(1, 0, 0, 1, 64, 1, 65, 64, 64, None) == -2
     assert lib.mlora_gemv(1, 0, 1, 1, 64, 1, 4, 64, 64, None) == -2          # accumulate into fp16
     assert lib.mlora_gemv(1, 1, 0, 1, 60, 1, 4, 64, 64, None) == -1          # ldx < K
-    assert lib.mlora_rmsnorm(1, 1, 0, 1, 1e-5, 4, 12, None) == -2
-    assert lib.mlora_paged_attn_decode(1, 1, 1, 1, 1, 4, 1, 1, 2, 8, 8, 96, 4, 2, None) == -2   # head_dim 96
-    assert lib.mlora_paged_attn_decode(1, 1, 1, 1, 1, 4, 1, 1, 2, 8, 3, 128, 4, 2, None) == -1  # Hq % Hkv
+    assert lib.mlora_rmsnorm(1, 0, 1, 0, 1, 1e-5, 4, 12, None) == -2
+    assert lib.mlora_rmsnorm(1, 1, 1, 0, 1, 1e-5, 65, 64, None) == -2        # fragment order needs T <= 64
+    assert lib.mlora_frag_activation_elems(17, 64) == 32 * 64 and lib.mlora_frag_activation_elems(33, 64) == 64 * 64
+    assert lib.mlora_paged_attn_decode(1, 0, 1, 1, 1, 1, 4, 1, 1, 2, 8, 8, 96, 4, 2, None) == -2   # head_dim 96
+    assert lib.mlora_paged_attn_decode(1, 0, 1, 1, 1, 1, 4, 1, 1, 2, 8, 3, 128, 4, 2, None) == -1  # Hq % Hkv
 
 
 def test_ops_refuse_cpu_tensors():

@@ -81,9 +81,9 @@ def test_gather_mm_into_column_slice(ops, synth):
 
 def test_gather_mm_rejects_bad_shapes(ops):
     lib = ops.lib()
-    assert lib.mlora_gather_mm(1, 0, 64, 1, 1, 1, 1, 1.0, 4, 64, 64, 12, 2, 1, 1 << 20, None) == -2   # rank 12
+    assert lib.mlora_gather_mm(1, 0, 64, 1, 0, 1, 1, 1, 1.0, 4, 64, 64, 12, 2, 1, 1 << 20, None) == -2   # rank 12
     assert b"rank" in lib.mlora_last_error()
-    assert lib.mlora_gather_mm(1, 0, 64, 1, 1, 1, 1, 1.0, 4, 64, 64, 16, 2, 1, 8, None) == -3          # workspace
+    assert lib.mlora_gather_mm(1, 0, 64, 1, 0, 1, 1, 1, 1.0, 4, 64, 64, 16, 2, 1, 8, None) == -3          # workspace
     assert lib.mlora_gemv(1, 0, 0, 1, 64, 1, 65, 64, 64, None) == -2                                 # T > 64
 
 
@@ -118,6 +118,52 @@ def test_linear_matches_oracle(ops, synth, T, K, N, kernel, packed):
     assert max_rel_err(_np(y16), ref) <= TOL
     assert max_rel_err(_np(y32), ref, floor=1e-2) <= 5e-4      # fp32 output: only summation-order noise
     assert max_rel_err(_np(racc), _np(r0) + ref, floor=1e-2) <= 5e-4
+
+
+@pytest.mark.parametrize("T,K,N", [(32, 4096, 4096), (32, 4096, 12288), (32, 11008, 4096), (64, 4096, 4096),
+                                   (16, 4096, 22016), (4, 1024, 3072), (1, 1024, 1024), (17, 2752, 1024), (5, 64, 36)])
+def test_gemv_fragment_ordered_activation(ops, synth, T, K, N):
+    """Both operands in fragment order: pack/unpack of x is an exact permutation, the product matches."""
+    print(f"case gemv_frag T={T} K={K} N={N}", flush=True)
+    x = synth.normal(7, f"lin.x.{T}.{K}", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(7, f"lin.W.{N}.{K}", (N, K), 0.02, torch.float16, DEV)
+    xf = ops.FragActivation.pack(x)
+    assert torch.equal(xf.unpack(), x)
+    ref = _np(x).astype(np.float64) @ _np(W).astype(np.float64).T
+    Wp = ops.PackedWeight(W)
+    y16 = ops.linear(xf, Wp)
+    r0 = synth.normal(7, f"lin.r.{T}.{N}", (T, N), 1.0, torch.float32, DEV)
+    racc = r0.clone()
+    ops.linear(xf, Wp, out=racc, accumulate=True)
+    torch.cuda.synchronize()
+    assert max_rel_err(_np(y16), ref) <= TOL
+    assert max_rel_err(_np(racc), _np(r0) + ref, floor=1e-2) <= 5e-4
+    # identical bits to the row-major-x kernel: same fragments, same accumulation order
+    assert torch.equal(y16, ops.linear(x, Wp))
+
+
+def test_producers_write_fragment_order(ops, synth):
+    """RMSNorm and SiLU*mul writing fragment order == their row-major output, packed."""
+    T, H, I = 32, 4096, 11008
+    x = synth.normal(11, "frag.x", (T, H), 1.5, torch.float32, DEV)
+    w = synth.normal(11, "frag.w", (H,), 1.0, torch.float16, DEV)
+    assert torch.equal(ops.rmsnorm(x, w, 1e-5, frag=True).unpack(), ops.rmsnorm(x, w, 1e-5))
+    gu = synth.normal(12, "frag.gu", (T, 2 * I), 2.0, torch.float16, DEV)
+    assert torch.equal(ops.silu_mul(gu, frag=True).unpack(), ops.silu_mul(gu))
+    for T2 in (1, 17, 64):
+        x2 = synth.normal(11, f"frag.x{T2}", (T2, 1024), 1.5, torch.float16, DEV)
+        w2 = synth.normal(11, "frag.w2", (1024,), 1.0, torch.float16, DEV)
+        assert torch.equal(ops.rmsnorm(x2, w2, 1e-5, frag=True).unpack(), ops.rmsnorm(x2, w2, 1e-5))
+
+
+def test_gather_mm_reads_fragment_order(ops, synth):
+    T, K, N, r, n_ad = 32, 4096, 4096, 16, 16
+    c = synth.gather_mm_case(seed=3, T=T, K=K, N=N, r=r, n_ad=n_ad, device=DEV, tag="frag")
+    y1, y2 = c["y"].clone(), c["y"].clone()
+    ops.gather_mm(y1, c["x"], c["A"], c["B"], c["ids"], 0.5)
+    ops.gather_mm(y2, ops.FragActivation.pack(c["x"]), c["A"], c["B"], c["ids"], 0.5)
+    torch.cuda.synchronize()
+    assert torch.equal(y1, y2)
 
 
 @pytest.mark.parametrize("packed", [False, True])
@@ -232,9 +278,11 @@ def test_paged_attention_prefill_then_decode(ops, synth, Hq, Hkv, D):
         exp = ref.attention_with_fused_qkv(0, _np(qkv), Hq)
         ref.end_forward()
         cache.begin_forward(sids, lens)
-        got = cache.attention_with_fused_qkv(0, qkv.clone(), Hq)
+        frag = it == 1                      # one of the decode steps writes fragment order
+        got = cache.attention_with_fused_qkv(0, qkv.clone(), Hq, frag=frag)
         cache.end_forward()
         torch.cuda.synchronize()
+        got = got.unpack() if frag else got
         assert max_rel_err(_np(got), exp) <= TOL, f"step {it}"
     # cache contents: rotated K and V, page by page, against the oracle's pages
     k_ref = oracle.f16(ref.k[0])                       # [n_pages, Hkv, 16, D]
