@@ -47,16 +47,19 @@ def prefill_all(model, kv, prompts, adapter_ids, chunk=4):
     return first
 
 
-def gemv_event_timing(model, T):
+def gemv_event_timing(model, T, reps=3):
     """Average duration of the weight-streaming GEMV over one decode step's worth of launches (the four
-    fused projections of every layer + lm_head), each launch bracketed by events on the launch stream."""
+    fused projections of every layer + lm_head, 129 launches on 129 distinct weight matrices), issued back to
+    back as in a decode step and bracketed by one event pair on the launch stream."""
     import torch
     ops = _mod("ops")
     s = model.shape
     dev = model.device
-    x_h = torch.zeros((T, s.hidden_size), dtype=torch.float16, device=dev)
-    x_q = torch.zeros((T, s.q_size), dtype=torch.float16, device=dev)
-    x_i = torch.zeros((T, s.intermediate_size), dtype=torch.float16, device=dev)
+    x_h = ops.FragActivation(T, s.hidden_size, dev)
+    x_q = ops.FragActivation(T, s.q_size, dev)
+    x_i = ops.FragActivation(T, s.intermediate_size, dev)
+    for x in (x_h, x_q, x_i):
+        x.data.zero_()
     resid = torch.zeros((T, s.hidden_size), dtype=torch.float32, device=dev)
     qkv = torch.empty((T, s.q_size + 2 * s.kv_size), dtype=torch.float16, device=dev)
     gu = torch.empty((T, 2 * s.intermediate_size), dtype=torch.float16, device=dev)
@@ -66,21 +69,20 @@ def gemv_event_timing(model, T):
         launches += [(x_h, L["qkv"], qkv, False), (x_q, L["o"], resid, True),
                      (x_h, L["gate_up"], gu, False), (x_i, L["down"], resid, True)]
     launches.append((x_h, model.lm_head, logits, False))
-    for x, W, out, acc in launches[:8]:
-        ops.linear(x, W, out=out, accumulate=acc, kernel="gemv")
-    torch.cuda.synchronize()
-    evs = []
-    for x, W, out, acc in launches:
+    total_bytes = sum(W.N * W.K * 2 + T * W.K * 2 + T * W.N * (4 if out.dtype == torch.float32 else 2) * (2 if acc else 1)
+                      for _, W, out, acc in launches)
+    best = None
+    for _ in range(reps + 1):          # first pass is a warm-up
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        ops.linear(x, W, out=out, accumulate=acc, kernel="gemv")
+        for x, W, out, acc in launches:
+            ops.linear(x, W, out=out, accumulate=acc)
         e1.record()
-        evs.append((e0, e1, W.N * W.K * 2 + T * W.K * 2 + T * W.N * (4 if out.dtype == torch.float32 else 2) * (2 if acc else 1)))
-    torch.cuda.synchronize()
-    ms = [a.elapsed_time(b) for a, b, _ in evs]
-    total_bytes = sum(b for _, _, b in evs)
-    return {"launches": len(evs), "avg_us": 1e3 * sum(ms) / len(ms), "bytes_per_launch": total_bytes / len(evs),
-            "gbs": total_bytes / (sum(ms) * 1e-3) / 1e9}
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        best = ms if best is None else min(best, ms)
+    return {"launches": len(launches), "avg_us": 1e3 * best / len(launches), "bytes_per_launch": total_bytes / len(launches),
+            "gbs": total_bytes / (best * 1e-3) / 1e9}
 
 
 def gather_mm_timing(n_sets=128):
@@ -166,6 +168,9 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="model depth (32 = the benchmark configuration)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel event timing and the gather-matmul stream")
+    ap.add_argument("--probe", action="store_true",
+                    help="counter probe: a few GEMV / gather-matmul launches and a plain 256 MiB copy of known size "
+                         "(the calibration for FETCH_SIZE / WRITE_SIZE), no decode loop")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (every box here has one GPU, and the "
@@ -174,9 +179,21 @@ def main():
 
     import torch
     synth, llama, dsm = _mod("synth"), _mod("llama"), _mod("decode_session")
-    wl = synth.config3(num_layers=args.layers)
     dev = "cuda:0"
     torch.cuda.set_device(0)
+    if args.probe:
+        wl = synth.config3(num_layers=2)
+        model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, [wl.lora], dev)
+        src = torch.zeros(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)                       # plain copy kernel: reads 256 MiB, writes 256 MiB
+        g = gemv_event_timing(model, wl.batch, reps=1)
+        gm = gather_mm_timing(n_sets=8)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": True, "copy_bytes_each_way": 256 << 20, "gemv": g, "gather_matmul": gm}))
+        return
+    wl = synth.config3(num_layers=args.layers)
     t_setup = time.perf_counter()
     model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, [wl.lora], dev)
     prompts = synth.prompts(wl)
@@ -222,7 +239,7 @@ def main():
     }
     if not args.no_extras:
         g = gemv_event_timing(model, wl.batch)
-        out["roofline"] = {"kernel": "gemv_kernel (packed weights, T=32)", "bound": "hbm", "achieved": g["gbs"],
+        out["roofline"] = {"kernel": "gemv_kernel (fragment-ordered weights and activations, T=32)", "bound": "hbm", "achieved": g["gbs"],
                            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g["gbs"] / HBM_PEAK_GBS, "traffic": None,
                            "launches_timed": g["launches"], "avg_launch_us": g["avg_us"],
                            "algorithmic_bytes_per_launch": g["bytes_per_launch"]}
