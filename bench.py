@@ -168,6 +168,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="model depth (32 = the benchmark configuration)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel event timing and the gather-matmul stream")
+    ap.add_argument("--python-loop", action="store_true", help="issue every kernel from Python instead of mlora_decode_step")
+    ap.add_argument("--no-graph", action="store_true", help="call mlora_decode_step every step instead of replaying a captured graph")
     ap.add_argument("--probe", action="store_true",
                     help="counter probe: a few GEMV / gather-matmul launches and a plain 256 MiB copy of known size "
                          "(the calibration for FETCH_SIZE / WRITE_SIZE), no decode loop")
@@ -204,7 +206,10 @@ def main():
     kv = model.create_paged_kv_cache(wl.batch, wl.batch * blocks * wl.page_size, wl.prompt_len, wl.page_size,
                                      free_pages=perm, max_seq_len=blocks * wl.page_size)
     first = prefill_all(model, kv, prompts, wl.adapter_ids)
-    sess = dsm.DecodeSession(model, kv, list(range(wl.batch)), {0: wl.adapter_ids}, first)
+    if args.python_loop:
+        sess = dsm.DecodeSession(model, kv, list(range(wl.batch)), {0: wl.adapter_ids}, first)
+    else:
+        sess = dsm.NativeDecodeSession(model, kv, list(range(wl.batch)), wl.adapter_ids, first, use_graph=not args.no_graph)
     for _ in range(args.warmup):
         sess.step()
     torch.cuda.synchronize()
@@ -232,7 +237,8 @@ def main():
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": wl.name, "layers": wl.shape.num_hidden_layers, "hidden": wl.shape.hidden_size,
                    "batch": wl.batch, "adapters": wl.lora.n_adapters, "rank": wl.lora.r, "lora_targets": list(wl.lora.targets),
-                   "prompt_len": wl.prompt_len, "context_at_start": ctx0, "page_size": wl.page_size, "page_order": "random"},
+                   "prompt_len": wl.prompt_len, "context_at_start": ctx0, "page_size": wl.page_size, "page_order": "random",
+                   "host_loop": "python" if args.python_loop else ("native" if args.no_graph else "native+graph")},
         "step_algorithmic_gb": step_bytes / 1e9,
         "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "setup_s": t_setup,

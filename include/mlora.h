@@ -191,6 +191,103 @@ int mlora_paged_attn_prefill(void* out, const void* qkv, const void* k_cache, co
                              const int32_t* tok_seq, const int32_t* tok_pos,
                              int T, int Hq, int Hkv, int D, int n_pages, int n_seq, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Decode-step variants that carry the LoRA work of a projection inside a neighbouring launch, so that the
+ * adapter delta adds no launches of its own (results are bit-identical to the separate calls):
+ *   mlora_gemv_frag_lora      - mlora_gemv_frag, plus the shrink partials of n_proj <= 3 projections that read
+ *                               the same xf (A[p] [n_ad, r, K], a NULL slot is skipped); v_part is [n_proj][kc][T][r] fp32,
+ *                               n_proj * mlora_gather_mm_workspace_bytes(T, K, r) bytes;
+ *   mlora_rope_kv_append_lora - mlora_rope_kv_append, after adding scaling * B[p][id_t] . v to the q, k, v
+ *                               rows of qkv (B[p] [n_ad, N_p, r] or NULL; v_part as written above with K);
+ *   mlora_lora_expand_rmsnorm - resid[t, :] += scaling * B[id_t] . v (B [n_ad, H, r], v_part [kc][T][r] of a
+ *                               shrink over K inputs), then y = RMSNorm(resid) as mlora_rmsnorm.
+ * These replace the same reference operators as mlora_gather_mm, mlora_rope_kv_append and mlora_rmsnorm.
+ * ------------------------------------------------------------------------------------------- */
+int mlora_gemv_frag_lora(void* y, int y_dtype, int mode, const void* xf, const void* Wp, int T, int K, int N,
+                         void* v_part, const void* const* A, int n_proj, const int32_t* tok_adapter, int r, int n_ad,
+                         void* stream);
+int mlora_rope_kv_append_lora(void* qkv, void* k_cache, void* v_cache,
+                              const int32_t* block_table, int max_blocks,
+                              const int32_t* tok_seq, const int32_t* tok_pos,
+                              const float* rope_cos, const float* rope_sin, int max_pos,
+                              int T, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                              const void* v_part, const void* const* B, const int32_t* tok_adapter, float scaling,
+                              int K, int r, int n_ad, void* stream);
+int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v_part, const void* B,
+                              const int32_t* tok_adapter, float scaling, const void* w, float eps,
+                              int T, int H, int K, int r, int n_ad, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * One decode step of the whole model, enqueued by one call.
+ * Replaces: the body of the reference's hot loop between kv_state_begin_forward and the argmax
+ *   (tvm/llama_auto_batcher/llama_exec_graph.py:110-137): vm["embed"], vm["decode_*"] over all layers
+ *   (llama_for_causal_lm.py:79-84,95-100,121-128 with the patched attention of compile_tvm.py:116-160) and
+ *   np.argmax.  The host keeps only the integer page bookkeeping (a new page per sequence every 16 steps).
+ *
+ * All pointers inside the structs are device pointers; the structs themselves and the `layers` array live in
+ * host memory and are read during the call only.  Weights are fragment-ordered (mlora_pack_weight), q/k/v and
+ * gate/up fused row-wise.  A LoRA projection with A == NULL is not adapted.  One adapter type (rank, scaling)
+ * per call; tok_adapter[t] < 0 = no adapter for that sequence.
+ * Per step: tokens[t] (in) is embedded, attends at position pos[t] of sequence row rows[t] (ctx[t] = pos[t] + 1
+ * positions visible), and tokens[t] (out) receives the greedy next token; pos and ctx are then incremented on the
+ * device, so the call can be replayed from a captured graph without host work while no new page is needed.
+ * Scratch buffers are caller-owned (sizes in elements):
+ *   resid f32 [T*H]; xn, attn: mlora_frag_activation_elems(T, H | Hq*D) f16; qkv f16 [T*(Hq+2Hkv)*D];
+ *   gate_up f16 [T*2I]; act: mlora_frag_activation_elems(T, I) f16; logits f32 [T*V];
+ *   lora_ws: 5 * mlora_gather_mm_workspace_bytes(T, max(H, I, Hq*D), r) bytes.
+ * ------------------------------------------------------------------------------------------- */
+typedef struct mlora_lora_proj {
+  const void* A;   /* [n_ad, r, K] f16 or NULL */
+  const void* B;   /* [n_ad, N, r] f16 */
+} mlora_lora_proj;
+
+enum { MLORA_Q = 0, MLORA_K = 1, MLORA_V = 2, MLORA_O = 3, MLORA_GATE = 4, MLORA_UP = 5, MLORA_DOWN = 6 };
+
+typedef struct mlora_layer {
+  const void* qkv_p;
+  const void* o_p;
+  const void* gate_up_p;
+  const void* down_p;
+  const void* ln1;
+  const void* ln2;
+  mlora_lora_proj lora[7];
+  void* k_cache;
+  void* v_cache;
+} mlora_layer;
+
+typedef struct mlora_decode_plan {
+  int n_layers, hidden, inter, n_q_heads, n_kv_heads, head_dim, vocab;
+  float eps;
+  int lora_r, lora_n_ad;
+  float lora_scaling;
+  const mlora_layer* layers;
+  const void* embed;
+  const void* norm;
+  const void* lm_head_p;
+  const float* rope_cos;
+  const float* rope_sin;
+  int max_pos;
+  const int32_t* block_table;
+  int max_blocks, n_pages, n_seq;
+  int T;
+  int32_t* tokens;
+  const int32_t* rows;
+  int32_t* pos;
+  int32_t* ctx;
+  const int32_t* tok_adapter;
+  float* resid;
+  void* xn;
+  void* qkv;
+  void* attn;
+  void* gate_up;
+  void* act;
+  float* logits;
+  void* lora_ws;
+  size_t lora_ws_bytes;
+} mlora_decode_plan;
+
+int mlora_decode_step(const mlora_decode_plan* plan, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -37,6 +37,9 @@ SIGNATURES = {
     "mlora_frag_activation_elems": (_z, [_i, _i]),
     "mlora_pack_activation": (_i, [_p, _p, _i, _i, _i, _p]),
     "mlora_gemv_frag": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p]),
+    "mlora_gemv_frag_lora": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _i, _p, _i, _i, _p]),
+    "mlora_rope_kv_append_lora": (_i, [_p, _p, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _f, _i, _i, _i, _p]),
+    "mlora_lora_expand_rmsnorm": (_i, [_p, _i, _p, _p, _p, _p, _f, _p, _f, _i, _i, _i, _i, _i, _p]),
     "mlora_rmsnorm": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _p]),
     "mlora_silu_mul": (_i, [_p, _i, _p, _p, _i, _i, _i, _p]),
     "mlora_embed": (_i, [_p, _i, _p, _p, _i, _i, _i, _p]),
@@ -45,6 +48,30 @@ SIGNATURES = {
     "mlora_paged_attn_decode": (_i, [_p, _i, _p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "mlora_paged_attn_prefill": (_i, [_p, _p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
 }
+
+
+
+class LoraProj(C.Structure):
+    _fields_ = [("A", _p), ("B", _p)]
+
+
+class Layer(C.Structure):
+    _fields_ = [("qkv_p", _p), ("o_p", _p), ("gate_up_p", _p), ("down_p", _p), ("ln1", _p), ("ln2", _p),
+                ("lora", LoraProj * 7), ("k_cache", _p), ("v_cache", _p)]
+
+
+class DecodePlan(C.Structure):
+    _fields_ = [("n_layers", _i), ("hidden", _i), ("inter", _i), ("n_q_heads", _i), ("n_kv_heads", _i), ("head_dim", _i),
+                ("vocab", _i), ("eps", _f), ("lora_r", _i), ("lora_n_ad", _i), ("lora_scaling", _f),
+                ("layers", C.POINTER(Layer)), ("embed", _p), ("norm", _p), ("lm_head_p", _p),
+                ("rope_cos", _p), ("rope_sin", _p), ("max_pos", _i),
+                ("block_table", _p), ("max_blocks", _i), ("n_pages", _i), ("n_seq", _i),
+                ("T", _i), ("tokens", _p), ("rows", _p), ("pos", _p), ("ctx", _p), ("tok_adapter", _p),
+                ("resid", _p), ("xn", _p), ("qkv", _p), ("attn", _p), ("gate_up", _p), ("act", _p), ("logits", _p),
+                ("lora_ws", _p), ("lora_ws_bytes", _z)]
+
+
+SIGNATURES["mlora_decode_step"] = (_i, [C.POINTER(DecodePlan), _p])
 
 _lib = None
 

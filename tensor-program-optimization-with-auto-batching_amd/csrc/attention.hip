@@ -7,11 +7,21 @@
 // The K layout gives the decode kernel and the MFMA prefill kernel 16-byte loads along D; the V
 // layout gives both of them the P.V contraction (over tokens) without an LDS transpose.
 // The page-table walk is integer-only: page = block_table[seq, pos / 16], slot = pos % 16.
-#include "common.h"
+#include "lora_device.h"
 
 namespace {
 
 constexpr int PAGE = MLORA_PAGE_SIZE;
+
+// LoRA expand of the q, k, v projections carried by the RoPE / append kernel: delta rows are added to the
+// projection output (and rounded to fp16, as the stand-alone expand does) before rotation and storage.
+struct LoraExpandQKV {
+  const float* vpart;        // [3][kc][T][r] partials of the q, k, v shrinks (nullptr = no LoRA in this launch)
+  const f16* B[3];           // [n_ad, N_p, r] per projection, nullptr = projection not adapted
+  const int32_t* ids;
+  float scaling;
+  int r, n_ad, kc;
+};
 
 // grid (T, Hq + 2 Hkv), 64 threads: thread i rotates the pair (i, i + D/2) of one head of one token
 __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qkv, f16* __restrict__ k_cache,
@@ -21,24 +31,46 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qk
                                                             const int32_t* __restrict__ tok_pos,
                                                             const float* __restrict__ rope_cos,
                                                             const float* __restrict__ rope_sin, int max_pos, int Hq,
-                                                            int Hkv, int D, int n_pages, int n_seq) {
+                                                            int Hkv, int D, int n_pages, int n_seq, int T,
+                                                            LoraExpandQKV lx) {
 #pragma clang fp contract(off)
+  __shared__ float lv[64];
   const int t = blockIdx.x, hh = blockIdx.y, i = threadIdx.x;
   const int half = D >> 1;
+  const int proj = hh < Hq ? 0 : (hh < Hq + Hkv ? 1 : 2);
+  const int head = hh - (proj == 0 ? 0 : (proj == 1 ? Hq : Hq + Hkv));
+  const f16* brow = nullptr;
+  if (lx.vpart != nullptr && lx.B[proj] != nullptr) {          // block-uniform
+    const int id = lx.ids[t];
+    if (id >= 0 && id < lx.n_ad) {
+      if (i < lx.r) lv[i] = lora_v(lx.vpart + (size_t)proj * lx.kc * T * lx.r, lx.kc, T, lx.r, t, i, lx.scaling);
+      __syncthreads();
+      const int n_rows = (proj == 0 ? Hq : Hkv) * D;
+      brow = lx.B[proj] + ((size_t)id * n_rows + (size_t)head * D) * lx.r;
+    }
+  }
   if (i >= half) return;
   const int seq = tok_seq[t], pos = tok_pos[t];
   if (seq < 0 || seq >= n_seq || pos < 0 || pos >= max_pos || pos / PAGE >= max_blocks) return;
   f16* src = qkv + ((size_t)t * (Hq + 2 * Hkv) + hh) * D;
+  f16 h1 = src[i], h2 = src[i + half];
+  if (brow != nullptr) {
+    {
+#pragma clang fp contract(fast)
+      h1 = (f16)((float)h1 + lora_row_dot(brow + (size_t)i * lx.r, lv, lx.r));
+      h2 = (f16)((float)h2 + lora_row_dot(brow + (size_t)(i + half) * lx.r, lv, lx.r));
+    }
+  }
   if (hh >= Hq + Hkv) {
     const int page = block_table[(size_t)seq * max_blocks + pos / PAGE];
     if (page < 0 || page >= n_pages) return;
     f16* dst = v_cache + ((size_t)page * Hkv + (hh - Hq - Hkv)) * D * PAGE + pos % PAGE;
-    dst[(size_t)i * PAGE] = src[i];
-    dst[(size_t)(i + half) * PAGE] = src[i + half];
+    dst[(size_t)i * PAGE] = h1;
+    dst[(size_t)(i + half) * PAGE] = h2;
     return;
   }
   const float c = rope_cos[(size_t)pos * half + i], s = rope_sin[(size_t)pos * half + i];
-  const float x1 = (float)src[i], x2 = (float)src[i + half];
+  const float x1 = (float)h1, x2 = (float)h2;
   // Separately rounded products (fp contraction is off in this kernel) and an fp32 result that is
   // materialised before the fp16 conversion (the empty asm keeps the compiler from fusing the add
   // and the convert into one single-rounding instruction): the rotation is then the same IEEE fp32
@@ -303,18 +335,44 @@ int check_attn(const char* who, int Hq, int Hkv, int D, int n_pages, int n_seq, 
 
 }  // namespace
 
+static int rope_kv_append_impl(const char* who, void* qkv, void* k_cache, void* v_cache, const int32_t* block_table,
+                               int max_blocks, const int32_t* tok_seq, const int32_t* tok_pos, const float* rope_cos,
+                               const float* rope_sin, int max_pos, int T, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                               const LoraExpandQKV& lx, void* stream) {
+  if (int e = check_attn(who, Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
+  MLORA_CHECK(qkv && k_cache && v_cache && block_table && tok_seq && tok_pos && rope_cos && rope_sin, MLORA_ERR_INVALID, "%s: null pointer", who);
+  MLORA_CHECK(T >= 0 && max_pos > 0, MLORA_ERR_INVALID, "%s: bad T=%d max_pos=%d", who, T, max_pos);
+  if (T == 0) return MLORA_OK;
+  hipLaunchKernelGGL(rope_kv_append_kernel, dim3(T, Hq + 2 * Hkv), dim3(64), 0, (hipStream_t)stream, (f16*)qkv,
+                     (f16*)k_cache, (f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, rope_cos, rope_sin,
+                     max_pos, Hq, Hkv, D, n_pages, n_seq, T, lx);
+  return mlora_launch_status(who);
+}
+
 extern "C" int mlora_rope_kv_append(void* qkv, void* k_cache, void* v_cache, const int32_t* block_table, int max_blocks,
                                     const int32_t* tok_seq, const int32_t* tok_pos, const float* rope_cos,
                                     const float* rope_sin, int max_pos, int T, int Hq, int Hkv, int D, int n_pages,
                                     int n_seq, void* stream) {
-  if (int e = check_attn("rope_kv_append", Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
-  MLORA_CHECK(qkv && k_cache && v_cache && block_table && tok_seq && tok_pos && rope_cos && rope_sin, MLORA_ERR_INVALID, "rope_kv_append: null pointer");
-  MLORA_CHECK(T >= 0 && max_pos > 0, MLORA_ERR_INVALID, "rope_kv_append: bad T=%d max_pos=%d", T, max_pos);
-  if (T == 0) return MLORA_OK;
-  hipLaunchKernelGGL(rope_kv_append_kernel, dim3(T, Hq + 2 * Hkv), dim3(64), 0, (hipStream_t)stream, (f16*)qkv,
-                     (f16*)k_cache, (f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, rope_cos, rope_sin,
-                     max_pos, Hq, Hkv, D, n_pages, n_seq);
-  return mlora_launch_status("rope_kv_append");
+  return rope_kv_append_impl("rope_kv_append", qkv, k_cache, v_cache, block_table, max_blocks, tok_seq, tok_pos, rope_cos,
+                             rope_sin, max_pos, T, Hq, Hkv, D, n_pages, n_seq, LoraExpandQKV(), stream);
+}
+
+extern "C" int mlora_rope_kv_append_lora(void* qkv, void* k_cache, void* v_cache, const int32_t* block_table,
+                                         int max_blocks, const int32_t* tok_seq, const int32_t* tok_pos,
+                                         const float* rope_cos, const float* rope_sin, int max_pos, int T, int Hq, int Hkv,
+                                         int D, int n_pages, int n_seq, const void* v_part, const void* const* B,
+                                         const int32_t* tok_adapter, float scaling, int K, int r, int n_ad, void* stream) {
+  MLORA_CHECK(v_part && B && tok_adapter, MLORA_ERR_INVALID, "rope_kv_append_lora: null LoRA argument");
+  MLORA_CHECK((r == 8 || r == 16 || r == 32 || r == 64) && n_ad > 0 && K > 0, MLORA_ERR_UNSUPPORTED,
+              "rope_kv_append_lora: rank %d not in {8,16,32,64} or bad n_ad/K", r);
+  LoraExpandQKV lx = {};
+  lx.vpart = (const float*)v_part;
+  for (int i = 0; i < 3; ++i) lx.B[i] = (const f16*)B[i];
+  lx.ids = tok_adapter;
+  lx.scaling = scaling;
+  lx.r = r; lx.n_ad = n_ad; lx.kc = lora_k_split(K).kc;
+  return rope_kv_append_impl("rope_kv_append_lora", qkv, k_cache, v_cache, block_table, max_blocks, tok_seq, tok_pos,
+                             rope_cos, rope_sin, max_pos, T, Hq, Hkv, D, n_pages, n_seq, lx, stream);
 }
 
 extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qkv, const void* k_cache, const void* v_cache,

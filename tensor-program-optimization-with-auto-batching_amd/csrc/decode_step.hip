@@ -1,0 +1,104 @@
+// One decode step of the whole model enqueued natively: the per-layer launch sequence of the decode hot
+// loop without any host work between kernels, so the step can be captured into a graph and replayed.
+#include "common.h"
+
+namespace {
+
+__global__ void advance_kernel(int32_t* __restrict__ pos, int32_t* __restrict__ ctx, int T) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < T) {
+    pos[t] += 1;
+    ctx[t] += 1;
+  }
+}
+
+#define STEP(call)                  \
+  do {                              \
+    if (int e_ = (call)) return e_; \
+  } while (0)
+
+}  // namespace
+
+extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
+  MLORA_CHECK(p && p->layers, MLORA_ERR_INVALID, "decode_step: null plan");
+  const int T = p->T, H = p->hidden, I = p->inter, Hq = p->n_q_heads, Hkv = p->n_kv_heads, D = p->head_dim;
+  MLORA_CHECK(T > 0 && T <= 64, MLORA_ERR_UNSUPPORTED, "decode_step: T=%d outside 1..64", T);
+  MLORA_CHECK(p->tokens && p->rows && p->pos && p->ctx && p->resid && p->xn && p->qkv && p->attn && p->gate_up && p->act &&
+                  p->logits && p->embed && p->norm && p->lm_head_p && p->block_table && p->rope_cos && p->rope_sin,
+              MLORA_ERR_INVALID, "decode_step: null buffer");
+  const int q_sz = Hq * D, kv_sz = Hkv * D, qkv_sz = q_sz + 2 * kv_sz;
+  const bool lora = p->tok_adapter != nullptr && p->lora_r > 0;
+  const int r = p->lora_r, n_ad = p->lora_n_ad;
+  const float sc = p->lora_scaling;
+  f16* qkv = (f16*)p->qkv;
+  f16* gu = (f16*)p->gate_up;
+  // LoRA scratch: slots 0-2 q/k/v partials, slot 3 o_proj, slot 4 down_proj / stand-alone calls
+  const int Kmax = H > I ? (H > q_sz ? H : q_sz) : (I > q_sz ? I : q_sz);
+  const size_t slot = lora ? mlora_gather_mm_workspace_bytes(T, Kmax, r) : 0;
+  MLORA_CHECK(!lora || (p->lora_ws && p->lora_ws_bytes >= 5 * slot), MLORA_ERR_WORKSPACE,
+              "decode_step: lora_ws of %zu bytes given, %zu needed", p->lora_ws_bytes, 5 * slot);
+  char* ws = (char*)p->lora_ws;
+  void* ws_qkv = ws;
+  void* ws_o = ws + 3 * slot;
+  void* ws_down = ws + 4 * slot;
+  auto delta = [&](void* y, int y_dtype, int ldy, const void* x, const mlora_lora_proj& lp, int K, int N) -> int {
+    if (!lora || !lp.A) return MLORA_OK;
+    return mlora_gather_mm(y, y_dtype, ldy, x, MLORA_FRAG, lp.A, lp.B, p->tok_adapter, sc, T, K, N, r, n_ad, ws_down, slot, stream);
+  };
+  // RMSNorm of the residual stream, applying a pending down_proj expand of the previous layer first
+  const void* pending_B = nullptr;
+  auto norm = [&](const void* w) -> int {
+    if (pending_B) {
+      const void* B = pending_B;
+      pending_B = nullptr;
+      return mlora_lora_expand_rmsnorm(p->xn, MLORA_FRAG, p->resid, ws_down, B, p->tok_adapter, sc, w, p->eps, T, H, I, r, n_ad, stream);
+    }
+    return mlora_rmsnorm(p->xn, MLORA_FRAG, p->resid, MLORA_F32, w, p->eps, T, H, stream);
+  };
+  STEP(mlora_embed(p->resid, MLORA_F32, p->embed, p->tokens, T, H, p->vocab, stream));
+  for (int l = 0; l < p->n_layers; ++l) {
+    const mlora_layer& L = p->layers[l];
+    STEP(norm(L.ln1));
+    const bool qkv_lora = lora && (L.lora[MLORA_Q].A || L.lora[MLORA_K].A || L.lora[MLORA_V].A);
+    if (qkv_lora) {
+      const void* A3[3] = {L.lora[MLORA_Q].A, L.lora[MLORA_K].A, L.lora[MLORA_V].A};
+      const void* B3[3] = {L.lora[MLORA_Q].A ? L.lora[MLORA_Q].B : nullptr, L.lora[MLORA_K].A ? L.lora[MLORA_K].B : nullptr,
+                           L.lora[MLORA_V].A ? L.lora[MLORA_V].B : nullptr};
+      STEP(mlora_gemv_frag_lora(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, ws_qkv, A3, 3, p->tok_adapter, r, n_ad, stream));
+      STEP(mlora_rope_kv_append_lora(qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos, p->rope_cos,
+                                     p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, ws_qkv, B3, p->tok_adapter,
+                                     sc, H, r, n_ad, stream));
+    } else {
+      STEP(mlora_gemv_frag(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, stream));
+      STEP(mlora_rope_kv_append(qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos, p->rope_cos,
+                                p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, stream));
+    }
+    STEP(mlora_paged_attn_decode(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows,
+                                 p->ctx, T, Hq, Hkv, D, p->n_pages, p->n_seq, stream));
+    if (lora && L.lora[MLORA_O].A) {
+      const void* A1[1] = {L.lora[MLORA_O].A};
+      STEP(mlora_gemv_frag_lora(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->attn, L.o_p, T, q_sz, H, ws_o, A1, 1, p->tok_adapter, r, n_ad, stream));
+      STEP(mlora_lora_expand_rmsnorm(p->xn, MLORA_FRAG, p->resid, ws_o, L.lora[MLORA_O].B, p->tok_adapter, sc, L.ln2, p->eps, T, H,
+                                     q_sz, r, n_ad, stream));
+    } else {
+      STEP(mlora_gemv_frag(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->attn, L.o_p, T, q_sz, H, stream));
+      STEP(mlora_rmsnorm(p->xn, MLORA_FRAG, p->resid, MLORA_F32, L.ln2, p->eps, T, H, stream));
+    }
+    STEP(mlora_gemv_frag(gu, MLORA_F16, MLORA_STORE, p->xn, L.gate_up_p, T, H, 2 * I, stream));
+    STEP(delta(gu, MLORA_F16, 2 * I, p->xn, L.lora[MLORA_GATE], H, I));
+    STEP(delta(gu + I, MLORA_F16, 2 * I, p->xn, L.lora[MLORA_UP], H, I));
+    STEP(mlora_silu_mul(p->act, MLORA_FRAG, gu, gu + I, 2 * I, T, I, stream));
+    if (lora && L.lora[MLORA_DOWN].A) {
+      const void* A1[1] = {L.lora[MLORA_DOWN].A};
+      STEP(mlora_gemv_frag_lora(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->act, L.down_p, T, I, H, ws_down, A1, 1, p->tok_adapter, r, n_ad, stream));
+      pending_B = L.lora[MLORA_DOWN].B;   // expanded inside the next RMSNorm launch
+    } else {
+      STEP(mlora_gemv_frag(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->act, L.down_p, T, I, H, stream));
+    }
+  }
+  STEP(norm(p->norm));
+  STEP(mlora_gemv_frag(p->logits, MLORA_F32, MLORA_STORE, p->xn, p->lm_head_p, T, H, p->vocab, stream));
+  STEP(mlora_argmax(p->tokens, p->logits, T, p->vocab, stream));
+  hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, p->pos, p->ctx, T);
+  return mlora_launch_status("decode_step");
+}

@@ -11,107 +11,11 @@
 //             through a small LDS transpose so every lane touches contiguous y elements.
 // The adapter table is never materialised per token: the index lookup happens inside the kernels,
 // which is the optimisation of tvm/custom/fuse_take_matmul.py:85-105 kept in hand-written form.
-#include "common.h"
+#include "lora_device.h"
 
 namespace {
 
-constexpr int KCHUNK = 512;   // K elements one wave covers per pass: 64 lanes x 8 fp16
-constexpr int MAX_KC = 8;     // K-slices (partials) per token
-
-struct KSplit { int ci; int kc; };
-
-KSplit k_split(int K) {
-  int ci = ceil_div(K, KCHUNK * MAX_KC);
-  if (ci < 1) ci = 1;
-  return {ci, ceil_div(K, KCHUNK * ci)};
-}
-
-// Reduce G per-lane partials across the 64 lanes.  On return every lane holds in p[0] the full sum
-// of partial index j (returned); lanes sharing j hold the same value.
-template <int G>
-__device__ __forceinline__ int reduce_transpose(float (&p)[G], int lane) {
-  int j = 0;
-  int off = 32;
-#pragma unroll
-  for (int n = G; n > 1; n >>= 1) {
-    const int half = n >> 1;
-    const bool hi = (lane & off) != 0;
-#pragma unroll
-    for (int i = 0; i < half; ++i) {
-      const float send = hi ? p[i] : p[i + half];
-      const float keep = hi ? p[i + half] : p[i];
-      p[i] = keep + __shfl_xor(send, off, WAVE);
-    }
-    j += hi ? half : 0;
-    off >>= 1;
-  }
-#pragma unroll
-  for (; off > 0; off >>= 1) p[0] += __shfl_xor(p[0], off, WAVE);
-  return j;
-}
-
-template <int R>
-__global__ __launch_bounds__(64) void lora_shrink_kernel(float* __restrict__ vpart, const f16* __restrict__ x,
-                                                         const f16* __restrict__ A,
-                                                         const int32_t* __restrict__ ids, int T, int K, int CI,
-                                                         int frag_tt) {
-  constexpr int G = R < 16 ? R : 16;   // A rows held in registers at once
-  constexpr int TB = 4;                // tokens in flight
-  const int a = blockIdx.x;
-  const int c = blockIdx.y;
-  const int lane = threadIdx.x;
-  const int kbase = c * CI * KCHUNK + lane * 8;
-
-  for (int t0 = 0; t0 < T; t0 += WAVE) {
-    const int id = (t0 + lane < T) ? ids[t0 + lane] : -1;
-    unsigned long long mask = __ballot(id == a);
-    while (mask) {
-      int tt[TB];
-#pragma unroll
-      for (int u = 0; u < TB; ++u) {
-        if (mask) {
-          tt[u] = t0 + __builtin_ctzll(mask);
-          mask &= mask - 1;
-        } else {
-          tt[u] = -1;
-        }
-      }
-      for (int jb = 0; jb < R; jb += G) {
-        float p[TB][G];
-#pragma unroll
-        for (int u = 0; u < TB; ++u)
-#pragma unroll
-          for (int j = 0; j < G; ++j) p[u][j] = 0.f;
-        for (int ci = 0; ci < CI; ++ci) {
-          const int k = kbase + ci * KCHUNK;
-          const bool kin = k < K;
-          f16x8 xv[TB];
-#pragma unroll
-          for (int u = 0; u < TB; ++u) {
-            xv[u] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-            if (kin && tt[u] >= 0) xv[u] = ld8(x + (frag_tt ? frag_offset(tt[u], k, frag_tt) : (size_t)tt[u] * K + k));
-          }
-          f16x8 areg[G];
-#pragma unroll
-          for (int j = 0; j < G; ++j) {
-            areg[j] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-            if (kin) areg[j] = ld8(A + ((size_t)a * R + jb + j) * K + k);
-          }
-#pragma unroll
-          for (int u = 0; u < TB; ++u)
-#pragma unroll
-            for (int j = 0; j < G; ++j) p[u][j] = dot8(areg[j], xv[u], p[u][j]);
-        }
-#pragma unroll
-        for (int u = 0; u < TB; ++u) {
-          if (tt[u] < 0) continue;   // wave-uniform
-          const int j = reduce_transpose<G>(p[u], lane);
-          if ((lane & (WAVE / G - 1)) == 0) vpart[((size_t)c * T + tt[u]) * R + jb + j] = p[u][0];
-        }
-      }
-    }
-  }
-}
+__global__ __launch_bounds__(64) void lora_shrink_kernel(LoraShrinkBatch b) { lora_shrink_unit(b, blockIdx.x, threadIdx.x); }
 
 template <typename YT, int N>
 struct YVec;
@@ -197,7 +101,7 @@ __global__ __launch_bounds__(64) void lora_expand_kernel(YT* __restrict__ y, con
 #pragma unroll
         for (int e = 0; e < 8; ++e) s = fmaf(bf[i][e], v[e], s);
 #pragma unroll
-        for (int o = LPR >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, WAVE);
+        for (int o = 1; o < LPR; o <<= 1) s += __shfl_xor(s, o, WAVE);   // neighbouring groups of 8 first
         if (sub == 0) stage[parity][i * RPI + rloc] = s;
       }
       __syncthreads();
@@ -232,15 +136,8 @@ int check_lora_shape(int T, int K, int N, int r, int n_ad) {
   MLORA_CHECK(T >= 0 && K > 0 && N > 0 && n_ad > 0, MLORA_ERR_INVALID, "gather_mm: bad shape T=%d K=%d N=%d n_ad=%d", T, K, N, n_ad);
   MLORA_CHECK(r == 8 || r == 16 || r == 32 || r == 64, MLORA_ERR_UNSUPPORTED, "gather_mm: rank %d not in {8,16,32,64}", r);
   MLORA_CHECK(K % 8 == 0 && N % 8 == 0, MLORA_ERR_UNSUPPORTED, "gather_mm: K=%d and N=%d must be multiples of 8", K, N);
-  MLORA_CHECK(n_ad <= 65535, MLORA_ERR_UNSUPPORTED, "gather_mm: n_ad=%d exceeds 65535", n_ad);
+  MLORA_CHECK(n_ad <= 65535 && T <= (1 << 20), MLORA_ERR_UNSUPPORTED, "gather_mm: n_ad=%d or T=%d too large", n_ad, T);
   return MLORA_OK;
-}
-
-template <int R>
-void launch_shrink(float* vpart, const f16* x, int frag_tt, const f16* A, const int32_t* ids, int T, int K, int n_ad,
-                   hipStream_t s) {
-  const KSplit ks = k_split(K);
-  hipLaunchKernelGGL(lora_shrink_kernel<R>, dim3(n_ad, ks.kc), dim3(64), 0, s, vpart, x, A, ids, T, K, ks.ci, frag_tt);
 }
 
 template <int R, typename YT>
@@ -248,14 +145,14 @@ void launch_expand(YT* y, int ldy, const float* vpart, const f16* B, const int32
                    int n_ad, hipStream_t s) {
   constexpr int CH = 8 * (WAVE / (R / 8));
   hipLaunchKernelGGL((lora_expand_kernel<R, YT>), dim3(n_ad, ceil_div(N, CH)), dim3(64), 0, s, y, vpart, B, ids, scaling,
-                     T, N, ldy, k_split(K).kc);
+                     T, N, ldy, lora_k_split(K).kc);
 }
 
 }  // namespace
 
 extern "C" size_t mlora_gather_mm_workspace_bytes(int T, int K, int r) {
   if (T <= 0 || K <= 0 || r <= 0) return 0;
-  return (size_t)k_split(K).kc * (size_t)T * (size_t)r * sizeof(float);
+  return (size_t)lora_k_split(K).kc * (size_t)T * (size_t)r * sizeof(float);
 }
 
 extern "C" int mlora_lora_shrink(void* v_part, const void* x, int x_layout, const void* A, const int32_t* tok_adapter,
@@ -263,19 +160,18 @@ extern "C" int mlora_lora_shrink(void* v_part, const void* x, int x_layout, cons
   if (int e = check_lora_shape(T, K, 8, r, n_ad)) return e;
   MLORA_CHECK(x_layout == MLORA_ROWMAJOR || (x_layout == MLORA_FRAG && T <= 64 && K % 32 == 0), MLORA_ERR_UNSUPPORTED,
               "lora_shrink: fragment-ordered x needs T <= 64 and K %% 32 == 0 (layout=%d T=%d K=%d)", x_layout, T, K);
-  const int frag_tt = x_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   MLORA_CHECK(v_part && x && A && tok_adapter, MLORA_ERR_INVALID, "lora_shrink: null pointer");
   if (T == 0) return MLORA_OK;
-  hipStream_t s = (hipStream_t)stream;
-  float* vp = (float*)v_part;
-  const f16* xp = (const f16*)x;
-  const f16* Ap = (const f16*)A;
-  switch (r) {
-    case 8: launch_shrink<8>(vp, xp, frag_tt, Ap, tok_adapter, T, K, n_ad, s); break;
-    case 16: launch_shrink<16>(vp, xp, frag_tt, Ap, tok_adapter, T, K, n_ad, s); break;
-    case 32: launch_shrink<32>(vp, xp, frag_tt, Ap, tok_adapter, T, K, n_ad, s); break;
-    default: launch_shrink<64>(vp, xp, frag_tt, Ap, tok_adapter, T, K, n_ad, s); break;
-  }
+  const LoraKSplit ks = lora_k_split(K);
+  LoraShrinkBatch b = {};
+  b.A[0] = (const f16*)A;
+  b.n_proj = 1;
+  b.vpart = (float*)v_part;
+  b.x = (const f16*)x;
+  b.ids = tok_adapter;
+  b.T = T; b.K = K; b.r = r; b.n_ad = n_ad; b.ci = ks.ci; b.kc = ks.kc;
+  b.frag_tt = x_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
+  hipLaunchKernelGGL(lora_shrink_kernel, dim3(lora_shrink_units(b)), dim3(64), 0, (hipStream_t)stream, b);
   return mlora_launch_status("lora_shrink");
 }
 

@@ -13,7 +13,7 @@
 //       Wp[n/16][k/32][(k%32)/8][n%16][k%8],
 //     so the fragment of (16 rows, 32 k) is one contiguous 1 KiB block and a wave streams consecutive
 //     blocks: every load is a full DRAM page and consecutive k-steps are consecutive addresses.
-#include "common.h"
+#include "lora_device.h"
 
 namespace {
 
@@ -23,15 +23,27 @@ constexpr int PIPE = 4;     // k-steps in flight per wave
 
 enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2 };
 
-template <int NT, int TT, int OUT, bool PACKED, bool XFRAG>
+// With SHRINK the first `shrink_blocks` workgroups of the launch do LoRA shrink units (one per wave) on the same
+// x instead of a GEMV tile: the adapter work rides in the GEMV launch and finishes long before it does.
+template <int NT, int TT, int OUT, bool PACKED, bool XFRAG, bool SHRINK>
 __global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx,
-                                                                const f16* __restrict__ W, int T, int K, int N) {
+                                                                const f16* __restrict__ W, int T, int K, int N,
+                                                                LoraShrinkBatch sb, int shrink_blocks) {
   __shared__ f32x4 red[GEMV_WAVES][NT * TT][WAVE];
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
+  int bid = blockIdx.x;
+  if constexpr (SHRINK) {
+    if (bid < shrink_blocks) {
+      const int unit = bid * GEMV_WAVES + wave;
+      if (unit < sb.n_proj * sb.n_ad * sb.kc) lora_shrink_unit(sb, unit, lane);
+      return;
+    }
+    bid -= shrink_blocks;
+  }
   const int r16 = lane & 15;
   const int kg = lane >> 4;
-  const int n0 = blockIdx.x * (16 * NT);
+  const int n0 = bid * (16 * NT);
   const int KB = K / KSTEP;
   constexpr int WSTEP = PACKED ? 512 : KSTEP;   // elements between consecutive k-steps of one fragment stream
 
@@ -40,7 +52,7 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(void* __restrict
 #pragma unroll
   for (int i = 0; i < NT; ++i) {
     if constexpr (PACKED) {
-      wp[i] = W + ((size_t)(blockIdx.x * NT + i) * KB) * 512 + lane * 8;
+      wp[i] = W + ((size_t)(bid * NT + i) * KB) * 512 + lane * 8;
     } else {
       int n = n0 + i * 16 + r16;
       n = n < N ? n : N - 1;
@@ -152,16 +164,19 @@ __global__ __launch_bounds__(256) void pack_activation_kernel(f16* __restrict__ 
   st8(dst + (size_t)c * 8, v);
 }
 
-template <int NT, int TT, bool PACKED, bool XFRAG>
-void launch_gemv(void* y, int out, const f16* x, int ldx, const f16* W, int T, int K, int N, hipStream_t s) {
-  const dim3 grid(ceil_div(N, 16 * NT)), block(GEMV_WAVES * WAVE);
-  if (out == OUT_F16) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F16, PACKED, XFRAG>), grid, block, 0, s, y, x, ldx, W, T, K, N);
-  else if (out == OUT_F32) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F32, PACKED, XFRAG>), grid, block, 0, s, y, x, ldx, W, T, K, N);
-  else hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_ACC_F32, PACKED, XFRAG>), grid, block, 0, s, y, x, ldx, W, T, K, N);
+template <int NT, int TT, bool PACKED, bool XFRAG, bool SHRINK>
+void launch_gemv(void* y, int out, const f16* x, int ldx, const f16* W, int T, int K, int N, hipStream_t s,
+                 const LoraShrinkBatch& sb) {
+  const int sblocks = SHRINK ? ceil_div(lora_shrink_units(sb), GEMV_WAVES) : 0;
+  const dim3 grid(ceil_div(N, 16 * NT) + sblocks), block(GEMV_WAVES * WAVE);
+  if (out == OUT_F16) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F16, PACKED, XFRAG, SHRINK>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks);
+  else if (out == OUT_F32) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F32, PACKED, XFRAG, SHRINK>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks);
+  else hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_ACC_F32, PACKED, XFRAG, SHRINK>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks);
 }
 
-template <bool PACKED, bool XFRAG>
-int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K, int N, void* stream) {
+template <bool PACKED, bool XFRAG, bool SHRINK = false>
+int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K, int N, void* stream,
+                  const LoraShrinkBatch& sb = LoraShrinkBatch()) {
   const int out = mode == MLORA_ACCUMULATE ? OUT_ACC_F32 : (y_dtype == MLORA_F32 ? OUT_F32 : OUT_F16);
   hipStream_t s = (hipStream_t)stream;
   const f16* xp = (const f16*)x;
@@ -171,13 +186,13 @@ int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const 
   const int tiles = ceil_div(N, 16);
   const bool wide = tiles >= 512 && (!PACKED || tiles % 2 == 0);
   if (T <= 16) {
-    if (wide) launch_gemv<2, 1, PACKED, XFRAG>(y, out, xp, ldx, Wp, T, K, N, s);
-    else launch_gemv<1, 1, PACKED, XFRAG>(y, out, xp, ldx, Wp, T, K, N, s);
+    if (wide) launch_gemv<2, 1, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb);
+    else launch_gemv<1, 1, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb);
   } else if (T <= 32) {
-    if (wide) launch_gemv<2, 2, PACKED, XFRAG>(y, out, xp, ldx, Wp, T, K, N, s);
-    else launch_gemv<1, 2, PACKED, XFRAG>(y, out, xp, ldx, Wp, T, K, N, s);
+    if (wide) launch_gemv<2, 2, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb);
+    else launch_gemv<1, 2, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb);
   } else {
-    launch_gemv<1, 4, PACKED, XFRAG>(y, out, xp, ldx, Wp, T, K, N, s);
+    launch_gemv<1, 4, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb);
   }
   return mlora_launch_status("gemv");
 }
@@ -218,6 +233,28 @@ extern "C" int mlora_gemv_frag(void* y, int y_dtype, int mode, const void* xf, c
   MLORA_CHECK(T <= 64, MLORA_ERR_UNSUPPORTED, "gemv_frag: T=%d exceeds 64", T);
   if (T == 0) return MLORA_OK;
   return gemv_dispatch<true, true>(y, y_dtype, mode, xf, K, Wp, T, K, N, stream);
+}
+
+extern "C" int mlora_gemv_frag_lora(void* y, int y_dtype, int mode, const void* xf, const void* Wp, int T, int K, int N,
+                                    void* v_part, const void* const* A, int n_proj, const int32_t* tok_adapter, int r,
+                                    int n_ad, void* stream) {
+  if (int e = mlora_check_linear("gemv_frag_lora", y, y_dtype, mode, xf, K, Wp, T, K, N)) return e;
+  MLORA_CHECK(T <= 64, MLORA_ERR_UNSUPPORTED, "gemv_frag_lora: T=%d exceeds 64", T);
+  MLORA_CHECK(n_proj >= 1 && n_proj <= LORA_MAX_PROJ && v_part && A && tok_adapter, MLORA_ERR_INVALID,
+              "gemv_frag_lora: need 1..%d projections and non-null LoRA arguments", LORA_MAX_PROJ);
+  MLORA_CHECK((r == 8 || r == 16 || r == 32 || r == 64) && n_ad > 0 && n_ad <= 65535, MLORA_ERR_UNSUPPORTED,
+              "gemv_frag_lora: rank %d not in {8,16,32,64} or bad n_ad %d", r, n_ad);
+  if (T == 0) return MLORA_OK;
+  const LoraKSplit ks = lora_k_split(K);
+  LoraShrinkBatch b = {};
+  for (int i = 0; i < n_proj; ++i) b.A[i] = (const f16*)A[i];   // a null slot is skipped
+  b.n_proj = n_proj;
+  b.vpart = (float*)v_part;
+  b.x = (const f16*)xf;
+  b.ids = tok_adapter;
+  b.T = T; b.K = K; b.r = r; b.n_ad = n_ad; b.ci = ks.ci; b.kc = ks.kc;
+  b.frag_tt = mlora_frag_tiles(T);
+  return gemv_dispatch<true, true, true>(y, y_dtype, mode, xf, K, Wp, T, K, N, stream, b);
 }
 
 extern "C" size_t mlora_frag_activation_elems(int T, int K) {

@@ -1,0 +1,136 @@
+// Device-side building blocks of the adapter-indexed LoRA delta, shared by the stand-alone gather-matmul
+// kernels and by the decode kernels that carry LoRA work inside their own launch.
+#pragma once
+#include "common.h"
+
+constexpr int LORA_KCHUNK = 512;   // K elements one wave covers per pass: 64 lanes x 8 fp16
+constexpr int LORA_MAX_KC = 8;     // K-slices (fp32 partials) per token
+constexpr int LORA_MAX_PROJ = 3;   // projections that share x in one batched shrink (q, k, v)
+
+struct LoraKSplit { int ci; int kc; };
+
+static inline LoraKSplit lora_k_split(int K) {
+  int ci = ceil_div(K, LORA_KCHUNK * LORA_MAX_KC);
+  if (ci < 1) ci = 1;
+  return {ci, ceil_div(K, LORA_KCHUNK * ci)};
+}
+
+// A batch of shrink problems that share x and the token->adapter table:
+//   v_part[p][c][t][:] = A[p][id_t][:, slice c] . x[t, slice c]        (fp32, one partial per K-slice c)
+struct LoraShrinkBatch {
+  const f16* A[LORA_MAX_PROJ];   // [n_ad, r, K] each
+  int n_proj;
+  float* vpart;                  // [n_proj][kc][T][r]
+  const f16* x;
+  const int32_t* ids;
+  int T, K, r, n_ad, ci, kc, frag_tt;
+};
+
+static inline int lora_shrink_units(const LoraShrinkBatch& b) { return b.n_proj * b.n_ad * b.kc; }
+
+// Reduce G per-lane partials across the 64 lanes.  On return every lane holds in p[0] the full sum
+// of partial index j (returned); lanes sharing j hold the same value.
+template <int G>
+__device__ __forceinline__ int reduce_transpose(float (&p)[G], int lane) {
+  int j = 0;
+  int off = 32;
+#pragma unroll
+  for (int n = G; n > 1; n >>= 1) {
+    const int half = n >> 1;
+    const bool hi = (lane & off) != 0;
+#pragma unroll
+    for (int i = 0; i < half; ++i) {
+      const float send = hi ? p[i] : p[i + half];
+      const float keep = hi ? p[i + half] : p[i];
+      p[i] = keep + __shfl_xor(send, off, WAVE);
+    }
+    j += hi ? half : 0;
+    off >>= 1;
+  }
+#pragma unroll
+  for (; off > 0; off >>= 1) p[0] += __shfl_xor(p[0], off, WAVE);
+  return j;
+}
+
+// One wave: adapter a of projection p, K-slice c.  Finds the tokens bound to a with ballots over the
+// token->adapter table, streams its slice of A[a] 8 rows at a time into registers (coalesced 1 KiB rows),
+// dots it against the tokens' x slices two at a time and writes the r partial sums per token.
+__device__ __forceinline__ void lora_shrink_unit(const LoraShrinkBatch& b, int unit, int lane) {
+  constexpr int G = 8, TB = 2;
+  const int c = unit % b.kc;
+  const int a = (unit / b.kc) % b.n_ad;
+  const int pj = unit / (b.kc * b.n_ad);
+  if (b.A[pj] == nullptr) return;   // projection slot not adapted
+  const f16* __restrict__ A = b.A[pj] + (size_t)a * b.r * b.K;
+  float* __restrict__ vp = b.vpart + ((size_t)pj * b.kc + c) * b.T * b.r;
+  const int kbase = c * b.ci * LORA_KCHUNK + lane * 8;
+  for (int t0 = 0; t0 < b.T; t0 += WAVE) {
+    const int id = (t0 + lane < b.T) ? b.ids[t0 + lane] : -1;
+    unsigned long long mask = __ballot(id == a);
+    while (mask) {
+      int tt[TB];
+#pragma unroll
+      for (int u = 0; u < TB; ++u) {
+        tt[u] = -1;
+        if (mask) {
+          tt[u] = t0 + __builtin_ctzll(mask);
+          mask &= mask - 1;
+        }
+      }
+      for (int jb = 0; jb < b.r; jb += G) {
+        float p[TB][G];
+#pragma unroll
+        for (int u = 0; u < TB; ++u)
+#pragma unroll
+          for (int j = 0; j < G; ++j) p[u][j] = 0.f;
+        for (int ci = 0; ci < b.ci; ++ci) {
+          const int k = kbase + ci * LORA_KCHUNK;
+          if (k < b.K) {
+            f16x8 xv[TB];
+#pragma unroll
+            for (int u = 0; u < TB; ++u) {
+              const int t = tt[u] >= 0 ? tt[u] : tt[0];
+              xv[u] = ld8(b.x + (b.frag_tt ? frag_offset(t, k, b.frag_tt) : (size_t)t * b.K + k));
+            }
+#pragma unroll
+            for (int j = 0; j < G; ++j) {
+              const f16x8 av = ld8(A + (size_t)(jb + j) * b.K + k);
+#pragma unroll
+              for (int u = 0; u < TB; ++u) p[u][j] = dot8(av, xv[u], p[u][j]);
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < TB; ++u) {
+          const int j = reduce_transpose<G>(p[u], lane);
+          if (tt[u] >= 0 && (lane & (WAVE / G - 1)) == 0) vp[(size_t)tt[u] * b.r + jb + j] = p[u][0];
+        }
+      }
+    }
+  }
+}
+
+// v[j] = scaling * sum_c v_part[c][t][j] for one token, summed in slice order (the order every consumer uses,
+// so fused and stand-alone expands agree bit for bit).
+__device__ __forceinline__ float lora_v(const float* __restrict__ vpart_proj, int kc, int T, int r, int t, int j, float scaling) {
+  float v = 0.f;
+  for (int c = 0; c < kc; ++c) v += vpart_proj[((size_t)c * T + t) * r + j];
+  return v * scaling;
+}
+
+// delta = B_row[0..r) . v[0..r) with the summation tree of the stand-alone expand kernel: an fma chain over each
+// group of 8, then pairwise sums of neighbouring groups.
+__device__ __forceinline__ float lora_row_dot(const f16* __restrict__ brow, const float* __restrict__ v, int r) {
+  float g[8];
+  const int ng = r >> 3;
+  for (int q = 0; q < ng; ++q) {
+    const f16x8 bv = ld8(brow + q * 8);
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s = fmaf((float)bv[e], v[q * 8 + e], s);
+    g[q] = s;
+  }
+  for (int n = ng; n > 1; n >>= 1)
+    for (int q = 0; q < n / 2; ++q) g[q] = g[2 * q] + g[2 * q + 1];
+  return g[0];
+}

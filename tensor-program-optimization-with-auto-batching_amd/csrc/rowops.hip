@@ -1,11 +1,20 @@
 // Row-wise operators for gfx950: RMSNorm, SiLU*mul, embedding gather, argmax.
 // All are a few hundred KiB per call at decode batch sizes - one pass over the row in registers,
 // 64-lane wave reductions, one LDS exchange between the waves of a block.
-#include "common.h"
+#include "lora_device.h"
 
 namespace {
 
 constexpr int ROW_THREADS = 256;
+
+// LoRA expand carried by the RMSNorm launch: resid[t, :] += scaling * B[id_t] . v[t] before the row is normed.
+struct LoraExpandRow {
+  const float* vpart;   // [kc][T][r] partials of the shrink (nullptr = plain RMSNorm)
+  const f16* B;         // [n_ad, H, r]
+  const int32_t* ids;
+  float scaling;
+  int r, n_ad, kc, T;
+};
 
 __device__ __forceinline__ float block_sum(float v, float* lds) {
   v = wave_sum(v);
@@ -20,11 +29,24 @@ __device__ __forceinline__ float block_sum(float v, float* lds) {
 
 // One block per row; each thread keeps up to VPT 8-element vectors of the row in registers.
 template <typename XT, int VPT>
-__global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(f16* __restrict__ y, const XT* __restrict__ x,
-                                                              const f16* __restrict__ w, float eps, int H, int frag_tt) {
+__global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(f16* __restrict__ y, XT* __restrict__ x,
+                                                              const f16* __restrict__ w, float eps, int H, int frag_tt,
+                                                              LoraExpandRow lx) {
   __shared__ float lds[ROW_THREADS / WAVE];
+  __shared__ float lv[64];
   const int row = blockIdx.x;
-  const XT* xr = x + (size_t)row * H;
+  XT* xr = x + (size_t)row * H;
+  const f16* brow = nullptr;
+  if constexpr (sizeof(XT) == 4) {
+    if (lx.vpart != nullptr) {                      // block-uniform
+      const int id = lx.ids[row];
+      if (id >= 0 && id < lx.n_ad) {
+        if (threadIdx.x < lx.r) lv[threadIdx.x] = lora_v(lx.vpart, lx.kc, lx.T, lx.r, row, threadIdx.x, lx.scaling);
+        __syncthreads();
+        brow = lx.B + (size_t)id * H * lx.r;
+      }
+    }
+  }
   float v[VPT][8];
   float ss = 0.f;
 #pragma unroll
@@ -42,6 +64,12 @@ __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(f16* __restrict__ 
         for (int e = 0; e < 4; ++e) {
           v[i][e] = lo[e];
           v[i][4 + e] = hi[e];
+        }
+        if (brow != nullptr) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[i][e] = v[i][e] + lora_row_dot(brow + (size_t)(c + e) * lx.r, lv, lx.r);
+          *reinterpret_cast<f32x4*>((float*)xr + c) = f32x4{v[i][0], v[i][1], v[i][2], v[i][3]};
+          *reinterpret_cast<f32x4*>((float*)xr + c + 4) = f32x4{v[i][4], v[i][5], v[i][6], v[i][7]};
         }
       }
 #pragma unroll
@@ -134,19 +162,19 @@ __global__ __launch_bounds__(ROW_THREADS) void argmax_kernel(int32_t* __restrict
 
 }  // namespace
 
-extern "C" int mlora_rmsnorm(void* y, int y_layout, const void* x, int x_dtype, const void* w, float eps, int T, int H,
-                             void* stream) {
+static int rmsnorm_impl(const char* who, void* y, int y_layout, void* x, int x_dtype, const void* w, float eps, int T,
+                        int H, const LoraExpandRow& lx, void* stream) {
   MLORA_CHECK(y_layout == MLORA_ROWMAJOR || (y_layout == MLORA_FRAG && T <= 64 && H % 32 == 0), MLORA_ERR_UNSUPPORTED,
-              "rmsnorm: fragment-ordered output needs T <= 64 and H %% 32 == 0 (layout=%d T=%d H=%d)", y_layout, T, H);
+              "%s: fragment-ordered output needs T <= 64 and H %% 32 == 0 (layout=%d T=%d H=%d)", who, y_layout, T, H);
   const int frag_tt = y_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
-  MLORA_CHECK(y && x && w, MLORA_ERR_INVALID, "rmsnorm: null pointer");
-  MLORA_CHECK(T >= 0 && H > 0 && H % 8 == 0 && H <= 16384, MLORA_ERR_UNSUPPORTED, "rmsnorm: need H %% 8 == 0, H <= 16384 (T=%d H=%d)", T, H);
-  MLORA_CHECK(x_dtype == MLORA_F16 || x_dtype == MLORA_F32, MLORA_ERR_INVALID, "rmsnorm: bad x_dtype %d", x_dtype);
+  MLORA_CHECK(y && x && w, MLORA_ERR_INVALID, "%s: null pointer", who);
+  MLORA_CHECK(T >= 0 && H > 0 && H % 8 == 0 && H <= 16384, MLORA_ERR_UNSUPPORTED, "%s: need H %% 8 == 0, H <= 16384 (T=%d H=%d)", who, T, H);
+  MLORA_CHECK(x_dtype == MLORA_F16 || x_dtype == MLORA_F32, MLORA_ERR_INVALID, "%s: bad x_dtype %d", who, x_dtype);
   if (T == 0) return MLORA_OK;
   hipStream_t s = (hipStream_t)stream;
   const int vpt = ceil_div(H, ROW_THREADS * 8);
 #define MLORA_RMS(XT, VPT) \
-  hipLaunchKernelGGL((rmsnorm_kernel<XT, VPT>), dim3(T), dim3(ROW_THREADS), 0, s, (f16*)y, (const XT*)x, (const f16*)w, eps, H, frag_tt)
+  hipLaunchKernelGGL((rmsnorm_kernel<XT, VPT>), dim3(T), dim3(ROW_THREADS), 0, s, (f16*)y, (XT*)x, (const f16*)w, eps, H, frag_tt, lx)
   if (x_dtype == MLORA_F16) {
     if (vpt <= 2) MLORA_RMS(f16, 2);
     else if (vpt <= 4) MLORA_RMS(f16, 4);
@@ -157,7 +185,27 @@ extern "C" int mlora_rmsnorm(void* y, int y_layout, const void* x, int x_dtype, 
     else MLORA_RMS(float, 8);
   }
 #undef MLORA_RMS
-  return mlora_launch_status("rmsnorm");
+  return mlora_launch_status(who);
+}
+
+extern "C" int mlora_rmsnorm(void* y, int y_layout, const void* x, int x_dtype, const void* w, float eps, int T, int H,
+                             void* stream) {
+  return rmsnorm_impl("rmsnorm", y, y_layout, const_cast<void*>(x), x_dtype, w, eps, T, H, LoraExpandRow(), stream);
+}
+
+extern "C" int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v_part, const void* B,
+                                         const int32_t* tok_adapter, float scaling, const void* w, float eps, int T, int H,
+                                         int K, int r, int n_ad, void* stream) {
+  MLORA_CHECK(v_part && B && tok_adapter, MLORA_ERR_INVALID, "lora_expand_rmsnorm: null LoRA argument");
+  MLORA_CHECK((r == 8 || r == 16 || r == 32 || r == 64) && n_ad > 0 && K > 0, MLORA_ERR_UNSUPPORTED,
+              "lora_expand_rmsnorm: rank %d not in {8,16,32,64} or bad n_ad/K", r);
+  LoraExpandRow lx = {};
+  lx.vpart = (const float*)v_part;
+  lx.B = (const f16*)B;
+  lx.ids = tok_adapter;
+  lx.scaling = scaling;
+  lx.r = r; lx.n_ad = n_ad; lx.kc = lora_k_split(K).kc; lx.T = T;
+  return rmsnorm_impl("lora_expand_rmsnorm", y, y_layout, resid, MLORA_F32, w, eps, T, H, lx, stream);
 }
 
 extern "C" int mlora_silu_mul(void* out, int out_layout, const void* gate, const void* up, int ld, int T, int I,

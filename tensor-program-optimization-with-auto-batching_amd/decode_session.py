@@ -42,3 +42,97 @@ class DecodeSession:
         if keep_history:
             self.history.append(nxt)
         return nxt
+
+
+class NativeDecodeSession:
+    """The same fixed-batch greedy decode, one `mlora_decode_step` call per step (one adapter type), optionally
+    replayed from a captured graph.  The graph is re-used as long as the batch does not change; the host only
+    grows the block table when a sequence crosses a page boundary."""
+
+    def __init__(self, model, kv, seq_ids, adapter_ids, first_tokens, tid=0, use_graph=True):
+        import ctypes as C
+        from . import _lib
+        self.model, self.kv = model, kv
+        self.seq_ids = list(seq_ids)
+        s = model.shape
+        dev = model.device
+        T = len(self.seq_ids)
+        if T > 64:
+            raise ValueError("NativeDecodeSession handles at most 64 sequences per step")
+        lt = model.lora_types[tid] if adapter_ids is not None and model.lora_types else None
+        i32 = lambda a: torch.as_tensor(np.asarray(a, dtype=np.int32)).to(dev)
+        self.tokens = i32(first_tokens)
+        self.rows = i32([kv.slot[q] for q in self.seq_ids])
+        self.pos = i32([kv.lens[q] for q in self.seq_ids])
+        self.ctx = self.pos + 1
+        self.tok_adapter = i32(adapter_ids) if lt is not None else None
+        H, I, V = s.hidden_size, s.intermediate_size, s.vocab_size
+        f16, f32 = torch.float16, torch.float32
+        fe = _lib.lib().mlora_frag_activation_elems
+        self.buf = {
+            "resid": torch.empty(T * H, dtype=f32, device=dev), "xn": torch.empty(fe(T, H), dtype=f16, device=dev),
+            "qkv": torch.empty(T * (s.q_size + 2 * s.kv_size), dtype=f16, device=dev),
+            "attn": torch.empty(fe(T, s.q_size), dtype=f16, device=dev),
+            "gate_up": torch.empty(T * 2 * I, dtype=f16, device=dev), "act": torch.empty(fe(T, I), dtype=f16, device=dev),
+            "logits": torch.empty(T * V, dtype=f32, device=dev),
+        }
+        r = lt.r if lt is not None else 0
+        ws_bytes = 5 * _lib.lib().mlora_gather_mm_workspace_bytes(T, max(H, I, s.q_size), max(r, 8))
+        self.buf["lora_ws"] = torch.empty(ws_bytes // 4, dtype=f32, device=dev)
+        layers = (_lib.Layer * s.num_hidden_layers)()
+        order = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")
+        for l, L in enumerate(model.layers):
+            layers[l].qkv_p, layers[l].o_p = L["qkv"].data.data_ptr(), L["o"].data.data_ptr()
+            layers[l].gate_up_p, layers[l].down_p = L["gate_up"].data.data_ptr(), L["down"].data.data_ptr()
+            layers[l].ln1, layers[l].ln2 = L["ln1"].data_ptr(), L["ln2"].data_ptr()
+            layers[l].k_cache, layers[l].v_cache = kv.k[l].data_ptr(), kv.v[l].data_ptr()
+            for j, proj in enumerate(order):
+                tab = lt.tables.get((l, proj)) if lt is not None else None
+                if tab is not None:
+                    layers[l].lora[j].A, layers[l].lora[j].B = tab[0].data_ptr(), tab[1].data_ptr()
+        p = _lib.DecodePlan()
+        p.n_layers, p.hidden, p.inter = s.num_hidden_layers, H, I
+        p.n_q_heads, p.n_kv_heads, p.head_dim, p.vocab, p.eps = s.num_attention_heads, s.num_key_value_heads, s.head_dim, V, s.rms_norm_eps
+        if lt is not None:
+            p.lora_r, p.lora_n_ad, p.lora_scaling = lt.r, lt.n_adapters, lt.scaling
+        p.layers = C.cast(layers, C.POINTER(_lib.Layer))
+        p.embed, p.norm, p.lm_head_p = model.embed_tokens.data_ptr(), model.norm.data_ptr(), model.lm_head.data.data_ptr()
+        p.rope_cos, p.rope_sin, p.max_pos = kv.rope_cos.data_ptr(), kv.rope_sin.data_ptr(), kv.max_pos
+        p.block_table, p.max_blocks, p.n_pages, p.n_seq = kv.block_table.data_ptr(), kv.max_blocks, kv.n_pages, kv.max_seqs
+        p.T = T
+        p.tokens, p.rows, p.pos, p.ctx = self.tokens.data_ptr(), self.rows.data_ptr(), self.pos.data_ptr(), self.ctx.data_ptr()
+        p.tok_adapter = self.tok_adapter.data_ptr() if self.tok_adapter is not None else None
+        for k in ("resid", "xn", "qkv", "attn", "gate_up", "act", "logits", "lora_ws"):
+            setattr(p, k, self.buf[k].data_ptr())
+        p.lora_ws_bytes = ws_bytes
+        self._layers, self.plan = layers, p
+        self._lib = _lib
+        self.use_graph = use_graph
+        self.graph = None
+        self.history = []
+
+    def _enqueue(self):
+        import ctypes as C
+        self._lib.check(self._lib.lib().mlora_decode_step(C.byref(self.plan), torch.cuda.current_stream().cuda_stream))
+
+    def step(self, keep_history=False):
+        kv = self.kv
+        # integer page bookkeeping on the host; copies the block table only when a page was added
+        kv.begin_forward(self.seq_ids, [1] * len(self.seq_ids), device_meta=(self.rows, self.pos, self.ctx))
+        if self.use_graph:
+            if self.graph is None:
+                # warm-up launch outside capture is not needed: kernels are plain launches; capture directly
+                g = torch.cuda.CUDAGraph()
+                snap = (self.tokens.clone(), self.pos.clone(), self.ctx.clone())
+                with torch.cuda.graph(g):
+                    self._enqueue()
+                # capture does not execute: restore nothing, just replay once for this step
+                self.tokens.copy_(snap[0]); self.pos.copy_(snap[1]); self.ctx.copy_(snap[2])
+                self.graph = g
+            self.graph.replay()
+        else:
+            self._enqueue()
+        kv.end_forward()
+        if keep_history:
+            self.history.append(self.tokens.clone())
+        return self.tokens
