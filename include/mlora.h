@@ -197,23 +197,33 @@ int mlora_paged_attn_prefill(void* out, const void* qkv, const void* k_cache, co
  *   mlora_gemv_frag_lora      - mlora_gemv_frag, plus the shrink partials of n_proj <= 3 projections that read
  *                               the same xf (A[p] [n_ad, r, K], a NULL slot is skipped); v_part is [n_proj][kc][T][r] fp32,
  *                               n_proj * mlora_gather_mm_workspace_bytes(T, K, r) bytes;
+ *   mlora_gemv_frag_split     - mlora_gemv_frag over a weight that has N_ext extra rows appended after its N_main
+ *                               rows: the stacked A tables of all adapters ([n_ad * r, K] per adapted projection,
+ *                               packed together with W).  Rows < N_main go to y as usual, the extra rows to
+ *                               y2 [T, N_ext] fp32: the shrink of every (token, adapter) pair, for the cost of the
+ *                               A bytes alone and with no dependence on the token->adapter table;
  *   mlora_rope_kv_append_lora - mlora_rope_kv_append, after adding scaling * B[p][id_t] . v to the q, k, v
- *                               rows of qkv (B[p] [n_ad, N_p, r] or NULL; v_part as written above with K);
- *   mlora_lora_expand_rmsnorm - resid[t, :] += scaling * B[id_t] . v (B [n_ad, H, r], v_part [kc][T][r] of a
- *                               shrink over K inputs), then y = RMSNorm(resid) as mlora_rmsnorm.
+ *                               rows of qkv (B[p] [n_ad, N_p, r] or NULL).  v_dense = 0: v_part holds the K-slice
+ *                               partials written by mlora_gemv_frag_lora with this K; v_dense = 1: v_part is
+ *                               y2 [T, 3 * n_ad * r] of mlora_gemv_frag_split (slot p = projection p);
+ *   mlora_lora_expand_rmsnorm - resid[t, :] += scaling * B[id_t] . v (B [n_ad, H, r]; v_part [kc][T][r] partials
+ *                               of a shrink over K inputs, or y2 [T, n_ad * r] when v_dense = 1), then
+ *                               y = RMSNorm(resid) as mlora_rmsnorm.
  * These replace the same reference operators as mlora_gather_mm, mlora_rope_kv_append and mlora_rmsnorm.
  * ------------------------------------------------------------------------------------------- */
 int mlora_gemv_frag_lora(void* y, int y_dtype, int mode, const void* xf, const void* Wp, int T, int K, int N,
                          void* v_part, const void* const* A, int n_proj, const int32_t* tok_adapter, int r, int n_ad,
                          void* stream);
+int mlora_gemv_frag_split(void* y, int y_dtype, int mode, float* y2, const void* xf, const void* Wp,
+                          int T, int K, int N_main, int N_ext, void* stream);
 int mlora_rope_kv_append_lora(void* qkv, void* k_cache, void* v_cache,
                               const int32_t* block_table, int max_blocks,
                               const int32_t* tok_seq, const int32_t* tok_pos,
                               const float* rope_cos, const float* rope_sin, int max_pos,
                               int T, int Hq, int Hkv, int D, int n_pages, int n_seq,
-                              const void* v_part, const void* const* B, const int32_t* tok_adapter, float scaling,
-                              int K, int r, int n_ad, void* stream);
-int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v_part, const void* B,
+                              const void* v_part, int v_dense, const void* const* B, const int32_t* tok_adapter,
+                              float scaling, int K, int r, int n_ad, void* stream);
+int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v_part, int v_dense, const void* B,
                               const int32_t* tok_adapter, float scaling, const void* w, float eps,
                               int T, int H, int K, int r, int n_ad, void* stream);
 
@@ -228,6 +238,9 @@ int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v
  * host memory and are read during the call only.  Weights are fragment-ordered (mlora_pack_weight), q/k/v and
  * gate/up fused row-wise.  A LoRA projection with A == NULL is not adapted.  One adapter type (rank, scaling)
  * per call; tok_adapter[t] < 0 = no adapter for that sequence.
+ * lora_dense != 0: qkv_p, o_p and down_p have the stacked A tables of their adapted projections appended as extra
+ * rows (q, k, v slots in that order, n_ad * r rows each, zero rows for a slot that is not adapted), and the shrink
+ * is part of the base GEMV; otherwise shrink units ride in the GEMV launch and read the A pointers.
  * Per step: tokens[t] (in) is embedded, attends at position pos[t] of sequence row rows[t] (ctx[t] = pos[t] + 1
  * positions visible), and tokens[t] (out) receives the greedy next token; pos and ctx are then incremented on the
  * device, so the call can be replayed from a captured graph without host work while no new page is needed.
@@ -260,6 +273,7 @@ typedef struct mlora_decode_plan {
   float eps;
   int lora_r, lora_n_ad;
   float lora_scaling;
+  int lora_dense;
   const mlora_layer* layers;
   const void* embed;
   const void* norm;

@@ -38,8 +38,9 @@ SIGNATURES = {
     "mlora_pack_activation": (_i, [_p, _p, _i, _i, _i, _p]),
     "mlora_gemv_frag": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p]),
     "mlora_gemv_frag_lora": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _i, _p, _i, _i, _p]),
-    "mlora_rope_kv_append_lora": (_i, [_p, _p, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _f, _i, _i, _i, _p]),
-    "mlora_lora_expand_rmsnorm": (_i, [_p, _i, _p, _p, _p, _p, _f, _p, _f, _i, _i, _i, _i, _i, _p]),
+    "mlora_gemv_frag_split": (_i, [_p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _p]),
+    "mlora_rope_kv_append_lora": (_i, [_p, _p, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p]),
+    "mlora_lora_expand_rmsnorm": (_i, [_p, _i, _p, _p, _i, _p, _p, _f, _p, _f, _i, _i, _i, _i, _i, _p]),
     "mlora_rmsnorm": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _p]),
     "mlora_silu_mul": (_i, [_p, _i, _p, _p, _i, _i, _i, _p]),
     "mlora_embed": (_i, [_p, _i, _p, _p, _i, _i, _i, _p]),
@@ -62,7 +63,7 @@ class Layer(C.Structure):
 
 class DecodePlan(C.Structure):
     _fields_ = [("n_layers", _i), ("hidden", _i), ("inter", _i), ("n_q_heads", _i), ("n_kv_heads", _i), ("head_dim", _i),
-                ("vocab", _i), ("eps", _f), ("lora_r", _i), ("lora_n_ad", _i), ("lora_scaling", _f),
+                ("vocab", _i), ("eps", _f), ("lora_r", _i), ("lora_n_ad", _i), ("lora_scaling", _f), ("lora_dense", _i),
                 ("layers", C.POINTER(Layer)), ("embed", _p), ("norm", _p), ("lm_head_p", _p),
                 ("rope_cos", _p), ("rope_sin", _p), ("max_pos", _i),
                 ("block_table", _p), ("max_blocks", _i), ("n_pages", _i), ("n_seq", _i),

@@ -16,11 +16,11 @@ constexpr int PAGE = MLORA_PAGE_SIZE;
 // LoRA expand of the q, k, v projections carried by the RoPE / append kernel: delta rows are added to the
 // projection output (and rounded to fp16, as the stand-alone expand does) before rotation and storage.
 struct LoraExpandQKV {
-  const float* vpart;        // [3][kc][T][r] partials of the q, k, v shrinks (nullptr = no LoRA in this launch)
+  LoraVSource src;           // shrink results of the q, k, v slots (src.v == nullptr: no LoRA in this launch)
   const f16* B[3];           // [n_ad, N_p, r] per projection, nullptr = projection not adapted
   const int32_t* ids;
   float scaling;
-  int r, n_ad, kc;
+  int r, n_ad;
 };
 
 // grid (T, Hq + 2 Hkv), 64 threads: thread i rotates the pair (i, i + D/2) of one head of one token
@@ -40,10 +40,10 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qk
   const int proj = hh < Hq ? 0 : (hh < Hq + Hkv ? 1 : 2);
   const int head = hh - (proj == 0 ? 0 : (proj == 1 ? Hq : Hq + Hkv));
   const f16* brow = nullptr;
-  if (lx.vpart != nullptr && lx.B[proj] != nullptr) {          // block-uniform
+  if (lx.src.v != nullptr && lx.B[proj] != nullptr) {          // block-uniform
     const int id = lx.ids[t];
     if (id >= 0 && id < lx.n_ad) {
-      if (i < lx.r) lv[i] = lora_v(lx.vpart + (size_t)proj * lx.kc * T * lx.r, lx.kc, T, lx.r, t, i, lx.scaling);
+      if (i < lx.r) lv[i] = lora_v_from(lx.src, proj, id, lx.r, t, i, lx.scaling);
       __syncthreads();
       const int n_rows = (proj == 0 ? Hq : Hkv) * D;
       brow = lx.B[proj] + ((size_t)id * n_rows + (size_t)head * D) * lx.r;
@@ -360,17 +360,20 @@ extern "C" int mlora_rope_kv_append(void* qkv, void* k_cache, void* v_cache, con
 extern "C" int mlora_rope_kv_append_lora(void* qkv, void* k_cache, void* v_cache, const int32_t* block_table,
                                          int max_blocks, const int32_t* tok_seq, const int32_t* tok_pos,
                                          const float* rope_cos, const float* rope_sin, int max_pos, int T, int Hq, int Hkv,
-                                         int D, int n_pages, int n_seq, const void* v_part, const void* const* B,
-                                         const int32_t* tok_adapter, float scaling, int K, int r, int n_ad, void* stream) {
+                                         int D, int n_pages, int n_seq, const void* v_part, int v_dense,
+                                         const void* const* B, const int32_t* tok_adapter, float scaling, int K, int r,
+                                         int n_ad, void* stream) {
   MLORA_CHECK(v_part && B && tok_adapter, MLORA_ERR_INVALID, "rope_kv_append_lora: null LoRA argument");
   MLORA_CHECK((r == 8 || r == 16 || r == 32 || r == 64) && n_ad > 0 && K > 0, MLORA_ERR_UNSUPPORTED,
               "rope_kv_append_lora: rank %d not in {8,16,32,64} or bad n_ad/K", r);
   LoraExpandQKV lx = {};
-  lx.vpart = (const float*)v_part;
+  lx.src.v = (const float*)v_part;
+  lx.src.kc = v_dense ? 0 : lora_k_split(K).kc;
+  lx.src.T = T; lx.src.n_ad = n_ad; lx.src.ld = 3 * n_ad * r;
   for (int i = 0; i < 3; ++i) lx.B[i] = (const f16*)B[i];
   lx.ids = tok_adapter;
   lx.scaling = scaling;
-  lx.r = r; lx.n_ad = n_ad; lx.kc = lora_k_split(K).kc;
+  lx.r = r; lx.n_ad = n_ad;
   return rope_kv_append_impl("rope_kv_append_lora", qkv, k_cache, v_cache, block_table, max_blocks, tok_seq, tok_pos,
                              rope_cos, rope_sin, max_pos, T, Hq, Hkv, D, n_pages, n_seq, lx, stream);
 }

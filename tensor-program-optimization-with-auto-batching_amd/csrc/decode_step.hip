@@ -12,9 +12,9 @@ __global__ void advance_kernel(int32_t* __restrict__ pos, int32_t* __restrict__ 
   }
 }
 
-#define STEP(call)                  \
-  do {                              \
-    if (int e_ = (call)) return e_; \
+#define STEP(call)                   \
+  do {                               \
+    if (int e_ = (call)) return e_;  \
   } while (0)
 
 }  // namespace
@@ -28,13 +28,15 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
               MLORA_ERR_INVALID, "decode_step: null buffer");
   const int q_sz = Hq * D, kv_sz = Hkv * D, qkv_sz = q_sz + 2 * kv_sz;
   const bool lora = p->tok_adapter != nullptr && p->lora_r > 0;
+  const bool dense = lora && p->lora_dense != 0;
   const int r = p->lora_r, n_ad = p->lora_n_ad;
   const float sc = p->lora_scaling;
   f16* qkv = (f16*)p->qkv;
   f16* gu = (f16*)p->gate_up;
   // LoRA scratch: slots 0-2 q/k/v partials, slot 3 o_proj, slot 4 down_proj / stand-alone calls
   const int Kmax = H > I ? (H > q_sz ? H : q_sz) : (I > q_sz ? I : q_sz);
-  const size_t slot = lora ? mlora_gather_mm_workspace_bytes(T, Kmax, r) : 0;
+  size_t slot = lora ? mlora_gather_mm_workspace_bytes(T, Kmax, r) : 0;
+  if (dense && slot < (size_t)T * n_ad * r * sizeof(float)) slot = (size_t)T * n_ad * r * sizeof(float);
   MLORA_CHECK(!lora || (p->lora_ws && p->lora_ws_bytes >= 5 * slot), MLORA_ERR_WORKSPACE,
               "decode_step: lora_ws of %zu bytes given, %zu needed", p->lora_ws_bytes, 5 * slot);
   char* ws = (char*)p->lora_ws;
@@ -51,7 +53,7 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
     if (pending_B) {
       const void* B = pending_B;
       pending_B = nullptr;
-      return mlora_lora_expand_rmsnorm(p->xn, MLORA_FRAG, p->resid, ws_down, B, p->tok_adapter, sc, w, p->eps, T, H, I, r, n_ad, stream);
+      return mlora_lora_expand_rmsnorm(p->xn, MLORA_FRAG, p->resid, ws_down, dense, B, p->tok_adapter, sc, w, p->eps, T, H, I, r, n_ad, stream);
     }
     return mlora_rmsnorm(p->xn, MLORA_FRAG, p->resid, MLORA_F32, w, p->eps, T, H, stream);
   };
@@ -64,10 +66,11 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
       const void* A3[3] = {L.lora[MLORA_Q].A, L.lora[MLORA_K].A, L.lora[MLORA_V].A};
       const void* B3[3] = {L.lora[MLORA_Q].A ? L.lora[MLORA_Q].B : nullptr, L.lora[MLORA_K].A ? L.lora[MLORA_K].B : nullptr,
                            L.lora[MLORA_V].A ? L.lora[MLORA_V].B : nullptr};
-      STEP(mlora_gemv_frag_lora(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, ws_qkv, A3, 3, p->tok_adapter, r, n_ad, stream));
+      if (dense) STEP(mlora_gemv_frag_split(qkv, MLORA_F16, MLORA_STORE, (float*)ws_qkv, p->xn, L.qkv_p, T, H, qkv_sz, 3 * n_ad * r, stream));
+      else STEP(mlora_gemv_frag_lora(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, ws_qkv, A3, 3, p->tok_adapter, r, n_ad, stream));
       STEP(mlora_rope_kv_append_lora(qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos, p->rope_cos,
-                                     p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, ws_qkv, B3, p->tok_adapter,
-                                     sc, H, r, n_ad, stream));
+                                     p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, ws_qkv, dense, B3,
+                                     p->tok_adapter, sc, H, r, n_ad, stream));
     } else {
       STEP(mlora_gemv_frag(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, stream));
       STEP(mlora_rope_kv_append(qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos, p->rope_cos,
@@ -77,8 +80,9 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
                                  p->ctx, T, Hq, Hkv, D, p->n_pages, p->n_seq, stream));
     if (lora && L.lora[MLORA_O].A) {
       const void* A1[1] = {L.lora[MLORA_O].A};
-      STEP(mlora_gemv_frag_lora(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->attn, L.o_p, T, q_sz, H, ws_o, A1, 1, p->tok_adapter, r, n_ad, stream));
-      STEP(mlora_lora_expand_rmsnorm(p->xn, MLORA_FRAG, p->resid, ws_o, L.lora[MLORA_O].B, p->tok_adapter, sc, L.ln2, p->eps, T, H,
+      if (dense) STEP(mlora_gemv_frag_split(p->resid, MLORA_F32, MLORA_ACCUMULATE, (float*)ws_o, p->attn, L.o_p, T, q_sz, H, n_ad * r, stream));
+      else STEP(mlora_gemv_frag_lora(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->attn, L.o_p, T, q_sz, H, ws_o, A1, 1, p->tok_adapter, r, n_ad, stream));
+      STEP(mlora_lora_expand_rmsnorm(p->xn, MLORA_FRAG, p->resid, ws_o, dense, L.lora[MLORA_O].B, p->tok_adapter, sc, L.ln2, p->eps, T, H,
                                      q_sz, r, n_ad, stream));
     } else {
       STEP(mlora_gemv_frag(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->attn, L.o_p, T, q_sz, H, stream));
@@ -90,7 +94,8 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
     STEP(mlora_silu_mul(p->act, MLORA_FRAG, gu, gu + I, 2 * I, T, I, stream));
     if (lora && L.lora[MLORA_DOWN].A) {
       const void* A1[1] = {L.lora[MLORA_DOWN].A};
-      STEP(mlora_gemv_frag_lora(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->act, L.down_p, T, I, H, ws_down, A1, 1, p->tok_adapter, r, n_ad, stream));
+      if (dense) STEP(mlora_gemv_frag_split(p->resid, MLORA_F32, MLORA_ACCUMULATE, (float*)ws_down, p->act, L.down_p, T, I, H, n_ad * r, stream));
+      else STEP(mlora_gemv_frag_lora(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->act, L.down_p, T, I, H, ws_down, A1, 1, p->tok_adapter, r, n_ad, stream));
       pending_B = L.lora[MLORA_DOWN].B;   // expanded inside the next RMSNorm launch
     } else {
       STEP(mlora_gemv_frag(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->act, L.down_p, T, I, H, stream));

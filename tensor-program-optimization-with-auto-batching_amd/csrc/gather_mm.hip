@@ -171,6 +171,7 @@ extern "C" int mlora_lora_shrink(void* v_part, const void* x, int x_layout, cons
   b.ids = tok_adapter;
   b.T = T; b.K = K; b.r = r; b.n_ad = n_ad; b.ci = ks.ci; b.kc = ks.kc;
   b.frag_tt = x_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
+  b.speculate = n_ad <= 2 * T;
   hipLaunchKernelGGL(lora_shrink_kernel, dim3(lora_shrink_units(b)), dim3(64), 0, (hipStream_t)stream, b);
   return mlora_launch_status("lora_shrink");
 }

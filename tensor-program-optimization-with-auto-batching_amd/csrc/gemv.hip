@@ -26,9 +26,10 @@ enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2 };
 // With SHRINK the first `shrink_blocks` workgroups of the launch do LoRA shrink units (one per wave) on the same
 // x instead of a GEMV tile: the adapter work rides in the GEMV launch and finishes long before it does.
 template <int NT, int TT, int OUT, bool PACKED, bool XFRAG, bool SHRINK>
-__global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx,
+__global__ __launch_bounds__(GEMV_WAVES* WAVE, 4) void gemv_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx,
                                                                 const f16* __restrict__ W, int T, int K, int N,
-                                                                LoraShrinkBatch sb, int shrink_blocks) {
+                                                                LoraShrinkBatch sb, int shrink_blocks, int n_main,
+                                                                float* __restrict__ y2) {
   __shared__ f32x4 red[GEMV_WAVES][NT * TT][WAVE];
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
@@ -120,8 +121,11 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(void* __restrict
     const int i = tile / TT, j = tile % TT;
     const int n = n0 + i * 16 + (sl >> 4) * 4;   // D[n][t]: lane holds rows 4*(lane/16)..+3, column lane%16
     const int t = j * 16 + (sl & 15);
-    if (t < T && n < N) {                         // N % 4 == 0: the 4 rows are inside together
-      const size_t o = (size_t)t * N + n;
+    if (t < T && n >= n_main && n < N) {
+      // rows past n_main are a second result block (adapter shrink rows appended to the weight): fp32, own buffer
+      *reinterpret_cast<f32x4*>(y2 + (size_t)t * (N - n_main) + (n - n_main)) = s;
+    } else if (t < T && n < N) {                  // N % 4 == 0: the 4 rows are inside together
+      const size_t o = (size_t)t * n_main + n;
       if constexpr (OUT == OUT_F16) {
         *reinterpret_cast<f16x4*>((f16*)yv + o) = f16x4{(f16)s[0], (f16)s[1], (f16)s[2], (f16)s[3]};
       } else if constexpr (OUT == OUT_F32) {
@@ -166,17 +170,18 @@ __global__ __launch_bounds__(256) void pack_activation_kernel(f16* __restrict__ 
 
 template <int NT, int TT, bool PACKED, bool XFRAG, bool SHRINK>
 void launch_gemv(void* y, int out, const f16* x, int ldx, const f16* W, int T, int K, int N, hipStream_t s,
-                 const LoraShrinkBatch& sb) {
+                 const LoraShrinkBatch& sb, int n_main, float* y2) {
   const int sblocks = SHRINK ? ceil_div(lora_shrink_units(sb), GEMV_WAVES) : 0;
   const dim3 grid(ceil_div(N, 16 * NT) + sblocks), block(GEMV_WAVES * WAVE);
-  if (out == OUT_F16) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F16, PACKED, XFRAG, SHRINK>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks);
-  else if (out == OUT_F32) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F32, PACKED, XFRAG, SHRINK>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks);
-  else hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_ACC_F32, PACKED, XFRAG, SHRINK>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks);
+  if (out == OUT_F16) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F16, PACKED, XFRAG, SHRINK>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2);
+  else if (out == OUT_F32) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F32, PACKED, XFRAG, SHRINK>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2);
+  else hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_ACC_F32, PACKED, XFRAG, SHRINK>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2);
 }
 
 template <bool PACKED, bool XFRAG, bool SHRINK = false>
 int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K, int N, void* stream,
-                  const LoraShrinkBatch& sb = LoraShrinkBatch()) {
+                  const LoraShrinkBatch& sb = LoraShrinkBatch(), int n_main = -1, float* y2 = nullptr) {
+  if (n_main < 0) n_main = N;
   const int out = mode == MLORA_ACCUMULATE ? OUT_ACC_F32 : (y_dtype == MLORA_F32 ? OUT_F32 : OUT_F16);
   hipStream_t s = (hipStream_t)stream;
   const f16* xp = (const f16*)x;
@@ -186,13 +191,13 @@ int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const 
   const int tiles = ceil_div(N, 16);
   const bool wide = tiles >= 512 && (!PACKED || tiles % 2 == 0);
   if (T <= 16) {
-    if (wide) launch_gemv<2, 1, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb);
-    else launch_gemv<1, 1, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb);
+    if (wide) launch_gemv<2, 1, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2);
+    else launch_gemv<1, 1, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2);
   } else if (T <= 32) {
-    if (wide) launch_gemv<2, 2, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb);
-    else launch_gemv<1, 2, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb);
+    if (wide) launch_gemv<2, 2, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2);
+    else launch_gemv<1, 2, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2);
   } else {
-    launch_gemv<1, 4, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb);
+    launch_gemv<1, 4, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2);
   }
   return mlora_launch_status("gemv");
 }
@@ -254,7 +259,18 @@ extern "C" int mlora_gemv_frag_lora(void* y, int y_dtype, int mode, const void* 
   b.ids = tok_adapter;
   b.T = T; b.K = K; b.r = r; b.n_ad = n_ad; b.ci = ks.ci; b.kc = ks.kc;
   b.frag_tt = mlora_frag_tiles(T);
+  b.speculate = n_ad <= 2 * T;
   return gemv_dispatch<true, true, true>(y, y_dtype, mode, xf, K, Wp, T, K, N, stream, b);
+}
+
+extern "C" int mlora_gemv_frag_split(void* y, int y_dtype, int mode, float* y2, const void* xf, const void* Wp, int T, int K,
+                                     int N_main, int N_ext, void* stream) {
+  if (int e = mlora_check_linear("gemv_frag_split", y, y_dtype, mode, xf, K, Wp, T, K, N_main)) return e;
+  MLORA_CHECK(T <= 64, MLORA_ERR_UNSUPPORTED, "gemv_frag_split: T=%d exceeds 64", T);
+  MLORA_CHECK(y2 && N_ext > 0 && N_ext % 4 == 0 && N_main % 16 == 0, MLORA_ERR_INVALID,
+              "gemv_frag_split: need y2, N_ext %% 4 == 0 and N_main %% 16 == 0 (N_main=%d N_ext=%d)", N_main, N_ext);
+  if (T == 0) return MLORA_OK;
+  return gemv_dispatch<true, true, false>(y, y_dtype, mode, xf, K, Wp, T, K, N_main + N_ext, stream, LoraShrinkBatch(), N_main, y2);
 }
 
 extern "C" size_t mlora_frag_activation_elems(int T, int K) {

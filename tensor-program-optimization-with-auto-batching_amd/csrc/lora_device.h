@@ -24,6 +24,7 @@ struct LoraShrinkBatch {
   const f16* x;
   const int32_t* ids;
   int T, K, r, n_ad, ci, kc, frag_tt;
+  int speculate;                 // request A before the adapter table is read (adapters expected to be in use)
 };
 
 static inline int lora_shrink_units(const LoraShrinkBatch& b) { return b.n_proj * b.n_ad * b.kc; }
@@ -52,11 +53,13 @@ __device__ __forceinline__ int reduce_transpose(float (&p)[G], int lane) {
   return j;
 }
 
-// One wave: adapter a of projection p, K-slice c.  Finds the tokens bound to a with ballots over the
-// token->adapter table, streams its slice of A[a] 8 rows at a time into registers (coalesced 1 KiB rows),
-// dots it against the tokens' x slices two at a time and writes the r partial sums per token.
+// One wave: adapter a of projection p, K-slice c.  The first 16 rows of its slice of A[a] are requested before the
+// token->adapter table has been read (when `speculate` is set: adapters are expected to be in use), so the wave
+// pays one memory round trip, not two, before it can start; that matters when the unit shares a launch with a
+// bandwidth-saturating GEMV and every round trip queues behind the weight stream.  Tokens bound to a are found
+// with ballots; A stays in registers across token pairs whenever the whole slice fits (r <= 16, one chunk).
 __device__ __forceinline__ void lora_shrink_unit(const LoraShrinkBatch& b, int unit, int lane) {
-  constexpr int G = 8, TB = 2;
+  constexpr int G = 16, TB = 2;
   const int c = unit % b.kc;
   const int a = (unit / b.kc) % b.n_ad;
   const int pj = unit / (b.kc * b.n_ad);
@@ -64,9 +67,23 @@ __device__ __forceinline__ void lora_shrink_unit(const LoraShrinkBatch& b, int u
   const f16* __restrict__ A = b.A[pj] + (size_t)a * b.r * b.K;
   float* __restrict__ vp = b.vpart + ((size_t)pj * b.kc + c) * b.T * b.r;
   const int kbase = c * b.ci * LORA_KCHUNK + lane * 8;
+  const bool resident = b.r <= G && b.ci == 1;   // the wave's whole slice of A fits the register file
+  const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  f16x8 areg[G];
+  int id = lane < b.T ? b.ids[lane] : -1;
+  if (resident && b.speculate) {
+#pragma unroll
+    for (int j = 0; j < G; ++j) areg[j] = (j < b.r && kbase < b.K) ? ld8(A + (size_t)j * b.K + kbase) : zero8;
+  }
+  bool loaded = resident && b.speculate;
   for (int t0 = 0; t0 < b.T; t0 += WAVE) {
-    const int id = (t0 + lane < b.T) ? b.ids[t0 + lane] : -1;
+    if (t0 > 0) id = (t0 + lane < b.T) ? b.ids[t0 + lane] : -1;
     unsigned long long mask = __ballot(id == a);
+    if (mask && resident && !loaded) {
+      loaded = true;
+#pragma unroll
+      for (int j = 0; j < G; ++j) areg[j] = (j < b.r && kbase < b.K) ? ld8(A + (size_t)j * b.K + kbase) : zero8;
+    }
     while (mask) {
       int tt[TB];
 #pragma unroll
@@ -85,25 +102,25 @@ __device__ __forceinline__ void lora_shrink_unit(const LoraShrinkBatch& b, int u
           for (int j = 0; j < G; ++j) p[u][j] = 0.f;
         for (int ci = 0; ci < b.ci; ++ci) {
           const int k = kbase + ci * LORA_KCHUNK;
-          if (k < b.K) {
-            f16x8 xv[TB];
+          f16x8 xv[TB];
 #pragma unroll
-            for (int u = 0; u < TB; ++u) {
-              const int t = tt[u] >= 0 ? tt[u] : tt[0];
-              xv[u] = ld8(b.x + (b.frag_tt ? frag_offset(t, k, b.frag_tt) : (size_t)t * b.K + k));
-            }
-#pragma unroll
-            for (int j = 0; j < G; ++j) {
-              const f16x8 av = ld8(A + (size_t)(jb + j) * b.K + k);
-#pragma unroll
-              for (int u = 0; u < TB; ++u) p[u][j] = dot8(av, xv[u], p[u][j]);
-            }
+          for (int u = 0; u < TB; ++u) {
+            const int t = tt[u] >= 0 ? tt[u] : tt[0];
+            xv[u] = k < b.K ? ld8(b.x + (b.frag_tt ? frag_offset(t, k, b.frag_tt) : (size_t)t * b.K + k)) : zero8;
           }
+          if (!resident) {
+#pragma unroll
+            for (int j = 0; j < G; ++j) areg[j] = (jb + j < b.r && k < b.K) ? ld8(A + (size_t)(jb + j) * b.K + k) : zero8;
+          }
+#pragma unroll
+          for (int j = 0; j < G; ++j)
+#pragma unroll
+            for (int u = 0; u < TB; ++u) p[u][j] = dot8(areg[j], xv[u], p[u][j]);
         }
 #pragma unroll
         for (int u = 0; u < TB; ++u) {
           const int j = reduce_transpose<G>(p[u], lane);
-          if (tt[u] >= 0 && (lane & (WAVE / G - 1)) == 0) vp[(size_t)tt[u] * b.r + jb + j] = p[u][0];
+          if (tt[u] >= 0 && jb + j < b.r && (lane & (WAVE / G - 1)) == 0) vp[(size_t)tt[u] * b.r + jb + j] = p[u][0];
         }
       }
     }
@@ -116,6 +133,20 @@ __device__ __forceinline__ float lora_v(const float* __restrict__ vpart_proj, in
   float v = 0.f;
   for (int c = 0; c < kc; ++c) v += vpart_proj[((size_t)c * T + t) * r + j];
   return v * scaling;
+}
+
+// Where an expand finds v for (token t, projection slot p, adapter id):
+//   kc > 0  : K-slice partials v_part[p][c][t][:]                    (written by the shrink units)
+//   kc == 0 : dense shrink results v_all[t][(p * n_ad + id) * r + :]  (written by a GEMV over weight rows that have the
+//             A tables of all adapters appended; the adapter is picked here, by index)
+struct LoraVSource {
+  const float* v;
+  int kc, T, n_ad, ld;
+};
+
+__device__ __forceinline__ float lora_v_from(const LoraVSource& s, int slot, int id, int r, int t, int j, float scaling) {
+  if (s.kc > 0) return lora_v(s.v + (size_t)slot * s.kc * s.T * r, s.kc, s.T, r, t, j, scaling);
+  return s.v[(size_t)t * s.ld + ((size_t)slot * s.n_ad + id) * r + j] * scaling;
 }
 
 // delta = B_row[0..r) . v[0..r) with the summation tree of the stand-alone expand kernel: an fma chain over each

@@ -9,13 +9,14 @@ constexpr int ROW_THREADS = 256;
 
 // LoRA expand carried by the RMSNorm launch: resid[t, :] += scaling * B[id_t] . v[t] before the row is normed.
 struct LoraExpandRow {
-  const float* vpart;   // [kc][T][r] partials of the shrink (nullptr = plain RMSNorm)
+  LoraVSource src;      // shrink results, one slot (src.v == nullptr: plain RMSNorm)
   const f16* B;         // [n_ad, H, r]
   const int32_t* ids;
   float scaling;
-  int r, n_ad, kc, T;
+  int r, n_ad;
 };
 
+template <int NTHREADS>
 __device__ __forceinline__ float block_sum(float v, float* lds) {
   v = wave_sum(v);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -23,27 +24,56 @@ __device__ __forceinline__ float block_sum(float v, float* lds) {
   __syncthreads();
   float s = 0.f;
 #pragma unroll
-  for (int w = 0; w < ROW_THREADS / WAVE; ++w) s += lds[w];
+  for (int w = 0; w < NTHREADS / WAVE; ++w) s += lds[w];
   return s;
 }
 
-// One block per row; each thread keeps up to VPT 8-element vectors of the row in registers.
+constexpr int NORM_THREADS = 512;
+
+// One block of 512 threads per row; each thread keeps up to VPT 8-element vectors of the row in registers.
+// With a LoRA expand attached (fp32 rows only) the block first streams B[id_row] ([H, r] fp16, coalesced 16-byte
+// chunks, r/8 lanes per output column combined by shuffles), stages the H deltas in LDS, adds them to the
+// residual row in place, and then norms the updated row.
 template <typename XT, int VPT>
-__global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(f16* __restrict__ y, XT* __restrict__ x,
-                                                              const f16* __restrict__ w, float eps, int H, int frag_tt,
-                                                              LoraExpandRow lx) {
-  __shared__ float lds[ROW_THREADS / WAVE];
+__global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(f16* __restrict__ y, XT* __restrict__ x,
+                                                               const f16* __restrict__ w, float eps, int H, int frag_tt,
+                                                               LoraExpandRow lx) {
+  __shared__ float lds[NORM_THREADS / WAVE];
   __shared__ float lv[64];
+  extern __shared__ float delta[];    // H floats when a LoRA expand is attached, otherwise empty
   const int row = blockIdx.x;
   XT* xr = x + (size_t)row * H;
-  const f16* brow = nullptr;
+  bool has_delta = false;
   if constexpr (sizeof(XT) == 4) {
-    if (lx.vpart != nullptr) {                      // block-uniform
+    if (lx.src.v != nullptr) {                      // block-uniform
       const int id = lx.ids[row];
       if (id >= 0 && id < lx.n_ad) {
-        if (threadIdx.x < lx.r) lv[threadIdx.x] = lora_v(lx.vpart, lx.kc, lx.T, lx.r, row, threadIdx.x, lx.scaling);
+        has_delta = true;
+        if (threadIdx.x < lx.r) lv[threadIdx.x] = lora_v_from(lx.src, 0, id, lx.r, row, threadIdx.x, lx.scaling);
         __syncthreads();
-        brow = lx.B + (size_t)id * H * lx.r;
+        const f16* __restrict__ B = lx.B + (size_t)id * H * lx.r;
+        const int lpr = lx.r >> 3;                  // lanes (16-byte chunks) per output column
+        const int chunks = H * lpr;
+        for (int q0 = 0; q0 < chunks; q0 += NORM_THREADS * 8) {
+          f16x8 bv[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const int q = q0 + u * NORM_THREADS + threadIdx.x;
+            bv[u] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (q < chunks) bv[u] = ld8(B + (size_t)q * 8);
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const int q = q0 + u * NORM_THREADS + threadIdx.x;
+            const int sub = q % lpr;
+            float s = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s = fmaf((float)bv[u][e], lv[sub * 8 + e], s);
+            for (int o = 1; o < lpr; o <<= 1) s += __shfl_xor(s, o, WAVE);   // neighbouring groups of 8 first
+            if (sub == 0 && q < chunks) delta[q / lpr] = s;
+          }
+        }
+        __syncthreads();
       }
     }
   }
@@ -51,7 +81,7 @@ __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(f16* __restrict__ 
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
-    const int c = (i * ROW_THREADS + threadIdx.x) * 8;
+    const int c = (i * NORM_THREADS + threadIdx.x) * 8;
     if (c < H) {
       if constexpr (sizeof(XT) == 2) {
         const f16x8 t = ld8((const f16*)xr + c);
@@ -65,9 +95,9 @@ __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(f16* __restrict__ 
           v[i][e] = lo[e];
           v[i][4 + e] = hi[e];
         }
-        if (brow != nullptr) {
+        if (has_delta) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) v[i][e] = v[i][e] + lora_row_dot(brow + (size_t)(c + e) * lx.r, lv, lx.r);
+          for (int e = 0; e < 8; ++e) v[i][e] = v[i][e] + delta[c + e];
           *reinterpret_cast<f32x4*>((float*)xr + c) = f32x4{v[i][0], v[i][1], v[i][2], v[i][3]};
           *reinterpret_cast<f32x4*>((float*)xr + c + 4) = f32x4{v[i][4], v[i][5], v[i][6], v[i][7]};
         }
@@ -76,11 +106,11 @@ __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(f16* __restrict__ 
       for (int e = 0; e < 8; ++e) ss = fmaf(v[i][e], v[i][e], ss);
     }
   }
-  ss = block_sum(ss, lds);
+  ss = block_sum<NORM_THREADS>(ss, lds);
   const float inv = rsqrtf(ss / (float)H + eps);
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
-    const int c = (i * ROW_THREADS + threadIdx.x) * 8;
+    const int c = (i * NORM_THREADS + threadIdx.x) * 8;
     if (c < H) {
       const f16x8 wv = ld8(w + c);
       f16x8 o;
@@ -172,17 +202,18 @@ static int rmsnorm_impl(const char* who, void* y, int y_layout, void* x, int x_d
   MLORA_CHECK(x_dtype == MLORA_F16 || x_dtype == MLORA_F32, MLORA_ERR_INVALID, "%s: bad x_dtype %d", who, x_dtype);
   if (T == 0) return MLORA_OK;
   hipStream_t s = (hipStream_t)stream;
-  const int vpt = ceil_div(H, ROW_THREADS * 8);
+  const int vpt = ceil_div(H, NORM_THREADS * 8);
+  const size_t dyn = lx.src.v ? (size_t)H * sizeof(float) : 0;   // LDS staging of the expand deltas
 #define MLORA_RMS(XT, VPT) \
-  hipLaunchKernelGGL((rmsnorm_kernel<XT, VPT>), dim3(T), dim3(ROW_THREADS), 0, s, (f16*)y, (XT*)x, (const f16*)w, eps, H, frag_tt, lx)
+  hipLaunchKernelGGL((rmsnorm_kernel<XT, VPT>), dim3(T), dim3(NORM_THREADS), dyn, s, (f16*)y, (XT*)x, (const f16*)w, eps, H, frag_tt, lx)
   if (x_dtype == MLORA_F16) {
-    if (vpt <= 2) MLORA_RMS(f16, 2);
-    else if (vpt <= 4) MLORA_RMS(f16, 4);
-    else MLORA_RMS(f16, 8);
+    if (vpt <= 1) MLORA_RMS(f16, 1);
+    else if (vpt <= 2) MLORA_RMS(f16, 2);
+    else MLORA_RMS(f16, 4);
   } else {
-    if (vpt <= 2) MLORA_RMS(float, 2);
-    else if (vpt <= 4) MLORA_RMS(float, 4);
-    else MLORA_RMS(float, 8);
+    if (vpt <= 1) MLORA_RMS(float, 1);
+    else if (vpt <= 2) MLORA_RMS(float, 2);
+    else MLORA_RMS(float, 4);
   }
 #undef MLORA_RMS
   return mlora_launch_status(who);
@@ -193,18 +224,20 @@ extern "C" int mlora_rmsnorm(void* y, int y_layout, const void* x, int x_dtype, 
   return rmsnorm_impl("rmsnorm", y, y_layout, const_cast<void*>(x), x_dtype, w, eps, T, H, LoraExpandRow(), stream);
 }
 
-extern "C" int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v_part, const void* B,
+extern "C" int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v_part, int v_dense, const void* B,
                                          const int32_t* tok_adapter, float scaling, const void* w, float eps, int T, int H,
                                          int K, int r, int n_ad, void* stream) {
   MLORA_CHECK(v_part && B && tok_adapter, MLORA_ERR_INVALID, "lora_expand_rmsnorm: null LoRA argument");
   MLORA_CHECK((r == 8 || r == 16 || r == 32 || r == 64) && n_ad > 0 && K > 0, MLORA_ERR_UNSUPPORTED,
               "lora_expand_rmsnorm: rank %d not in {8,16,32,64} or bad n_ad/K", r);
   LoraExpandRow lx = {};
-  lx.vpart = (const float*)v_part;
+  lx.src.v = (const float*)v_part;
+  lx.src.kc = v_dense ? 0 : lora_k_split(K).kc;
+  lx.src.T = T; lx.src.n_ad = n_ad; lx.src.ld = n_ad * r;
   lx.B = (const f16*)B;
   lx.ids = tok_adapter;
   lx.scaling = scaling;
-  lx.r = r; lx.n_ad = n_ad; lx.kc = lora_k_split(K).kc; lx.T = T;
+  lx.r = r; lx.n_ad = n_ad;
   return rmsnorm_impl("lora_expand_rmsnorm", y, y_layout, resid, MLORA_F32, w, eps, T, H, lx, stream);
 }
 

@@ -49,7 +49,7 @@ class NativeDecodeSession:
     replayed from a captured graph.  The graph is re-used as long as the batch does not change; the host only
     grows the block table when a sequence crosses a page boundary."""
 
-    def __init__(self, model, kv, seq_ids, adapter_ids, first_tokens, tid=0, use_graph=True):
+    def __init__(self, model, kv, seq_ids, adapter_ids, first_tokens, tid=0, use_graph=True, dense_lora=None):
         import ctypes as C
         from . import _lib
         self.model, self.kv = model, kv
@@ -77,13 +77,22 @@ class NativeDecodeSession:
             "logits": torch.empty(T * V, dtype=f32, device=dev),
         }
         r = lt.r if lt is not None else 0
-        ws_bytes = 5 * _lib.lib().mlora_gather_mm_workspace_bytes(T, max(H, I, s.q_size), max(r, 8))
+        ws_bytes = 5 * max(_lib.lib().mlora_gather_mm_workspace_bytes(T, max(H, I, s.q_size), max(r, 8)),
+                           4 * T * (lt.n_adapters if lt is not None else 0) * max(r, 8))
         self.buf["lora_ws"] = torch.empty(ws_bytes // 4, dtype=f32, device=dev)
         layers = (_lib.Layer * s.num_hidden_layers)()
         order = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")
+        # Dense shrink: the stacked A tables become extra weight rows of the base GEMV.  Worth it while the tables
+        # are small next to the base weight and most adapters are in use (the extra rows are read whether or not
+        # an adapter has a token in the batch).
+        if dense_lora is None:
+            dense_lora = lt is not None and lt.n_adapters <= 2 * T
+        self.dense_lora = bool(dense_lora and lt is not None)
+        ext = model.dense_lora_weights(tid) if self.dense_lora else None
         for l, L in enumerate(model.layers):
-            layers[l].qkv_p, layers[l].o_p = L["qkv"].data.data_ptr(), L["o"].data.data_ptr()
-            layers[l].gate_up_p, layers[l].down_p = L["gate_up"].data.data_ptr(), L["down"].data.data_ptr()
+            W = ext[l] if ext is not None else L
+            layers[l].qkv_p, layers[l].o_p = W["qkv"].data.data_ptr(), W["o"].data.data_ptr()
+            layers[l].gate_up_p, layers[l].down_p = L["gate_up"].data.data_ptr(), W["down"].data.data_ptr()
             layers[l].ln1, layers[l].ln2 = L["ln1"].data_ptr(), L["ln2"].data_ptr()
             layers[l].k_cache, layers[l].v_cache = kv.k[l].data_ptr(), kv.v[l].data_ptr()
             for j, proj in enumerate(order):
@@ -95,6 +104,7 @@ class NativeDecodeSession:
         p.n_q_heads, p.n_kv_heads, p.head_dim, p.vocab, p.eps = s.num_attention_heads, s.num_key_value_heads, s.head_dim, V, s.rms_norm_eps
         if lt is not None:
             p.lora_r, p.lora_n_ad, p.lora_scaling = lt.r, lt.n_adapters, lt.scaling
+            p.lora_dense = 1 if self.dense_lora else 0
         p.layers = C.cast(layers, C.POINTER(_lib.Layer))
         p.embed, p.norm, p.lm_head_p = model.embed_tokens.data_ptr(), model.norm.data_ptr(), model.lm_head.data.data_ptr()
         p.rope_cos, p.rope_sin, p.max_pos = kv.rope_cos.data_ptr(), kv.rope_sin.data_ptr(), kv.max_pos

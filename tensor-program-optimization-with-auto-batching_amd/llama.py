@@ -94,6 +94,38 @@ class LlamaForCausalLM:
             m.add_lora_type(lt)
         return m
 
+    def dense_lora_weights(self, tid: int = 0):
+        """Per layer, the qkv / o / down weights with the stacked A tables of adapter type `tid` appended as extra
+        rows ([n_ad * r, K] per adapted projection; q, k, v slots always present for qkv, zero when not adapted),
+        in fragment order.  Cached; costs one more copy of those matrices."""
+        cache = getattr(self, "_dense_cache", None)
+        if cache is None:
+            cache = self._dense_cache = {}
+        if tid in cache:
+            return cache[tid]
+        lt = self.lora_types[tid]
+        out = []
+        for l, L in enumerate(self.layers):
+            ent = {}
+            def slot(proj, K):
+                tab = lt.tables.get((l, proj))
+                if tab is None:
+                    return torch.zeros((lt.n_adapters * lt.r, K), dtype=torch.float16, device=self.device)
+                return tab[0].reshape(lt.n_adapters * lt.r, K)
+            H, I = self.shape.hidden_size, self.shape.intermediate_size
+            if any((l, p) in lt.tables for p in ("q_proj", "k_proj", "v_proj")):
+                ent["qkv"] = ops.PackedWeight(torch.cat([L["qkv"].unpack()] + [slot(p, H) for p in ("q_proj", "k_proj", "v_proj")]))
+            else:
+                ent["qkv"] = L["qkv"]
+            for key, proj, K in (("o", "o_proj", self.shape.q_size), ("down", "down_proj", I)):
+                if (l, proj) in lt.tables:
+                    ent[key] = ops.PackedWeight(torch.cat([L[key].unpack(), slot(proj, K)]))
+                else:
+                    ent[key] = L[key]
+            out.append(ent)
+        cache[tid] = out
+        return out
+
     def create_paged_kv_cache(self, max_batch_size, max_total_seq_len, prefill_chunk_size, page_size,
                               free_pages=None, max_seq_len=None):
         """Same arguments as the reference's VM function (`llama_for_causal_lm.py:148-174`).  The pool holds

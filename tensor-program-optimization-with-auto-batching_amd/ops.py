@@ -141,6 +141,12 @@ class PackedWeight:
     def shape(self):
         return (self.N, self.K)
 
+    def unpack(self) -> torch.Tensor:
+        """Back to row-major [N, K] (index arithmetic on the device tensor)."""
+        nt = (self.N + 15) // 16
+        v = self.data[: nt * 16 * self.K].view(nt, self.K // 32, 4, 16, 8)
+        return v.permute(0, 3, 1, 2, 4).reshape(nt * 16, self.K)[: self.N].contiguous()
+
 
 def linear(x, W, out=None, out_dtype=torch.float16, accumulate=False, kernel="auto"):
     """y (=|+=) x @ W.T.  x [T,K] f16 (row stride may exceed K) or a FragActivation, W [N,K] f16 or a
