@@ -203,7 +203,7 @@ class LlamaForCausalLM:
             full = np.full(T, -1, dtype=np.int32)
             w = _host_i32(wids)
             lt = self.lora_types[tid]
-            if w.size and (w.min() < 0 or w.max() >= lt.n_adapters):
+            if w.size and (w.min() < -1 or w.max() >= lt.n_adapters):      # -1 = no adapter for that row
                 raise ValueError(f"adapter weight id out of range for type {tid}: {w.min()}..{w.max()} of {lt.n_adapters}")
             if sids is None:
                 full[:] = np.broadcast_to(w, (T,)) if w.size in (1, T) else _bad(T, w)
