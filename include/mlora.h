@@ -214,6 +214,12 @@ int mlora_paged_attn_prefill(void* out, const void* qkv, const void* k_cache, co
 int mlora_gemv_frag_lora(void* y, int y_dtype, int mode, const void* xf, const void* Wp, int T, int K, int N,
                          void* v_part, const void* const* A, int n_proj, const int32_t* tok_adapter, int r, int n_ad,
                          void* stream);
+/* Gate/up projection with the SiLU product in its epilogue:  act = silu(f16(x . Wgate^T)) * f16(x . Wup^T), written
+ * in MLORA_FRAG order for the down projection (T <= 32).  Wil_p is the fragment-ordered [2I, K] matrix whose 16-row
+ * tiles alternate gate and up (tile 2j = gate rows 16j.., tile 2j+1 = up rows 16j..), so one workgroup holds both
+ * halves of a channel.  Replaces: gate_proj, up_proj, op.silu and the multiply (llama_for_causal_lm.py:35-36) in
+ * one launch; same result bits as mlora_gemv_frag followed by mlora_silu_mul. */
+int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p, int T, int K, int I, void* stream);
 int mlora_gemv_frag_split(void* y, int y_dtype, int mode, float* y2, const void* xf, const void* Wp,
                           int T, int K, int N_main, int N_ext, void* stream);
 int mlora_rope_kv_append_lora(void* qkv, void* k_cache, void* v_cache,
@@ -259,7 +265,8 @@ enum { MLORA_Q = 0, MLORA_K = 1, MLORA_V = 2, MLORA_O = 3, MLORA_GATE = 4, MLORA
 typedef struct mlora_layer {
   const void* qkv_p;
   const void* o_p;
-  const void* gate_up_p;
+  const void* gate_up_p;      /* [2I, K]: gate rows then up rows; may be NULL when gate_up_il_p is given and gate/up carry no LoRA */
+  const void* gate_up_il_p;   /* the same matrix with 16-row tiles of gate and up interleaved (mlora_gemv_frag_silu), or NULL */
   const void* down_p;
   const void* ln1;
   const void* ln2;

@@ -38,6 +38,7 @@ SIGNATURES = {
     "mlora_pack_activation": (_i, [_p, _p, _i, _i, _i, _p]),
     "mlora_gemv_frag": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p]),
     "mlora_gemv_frag_lora": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _i, _p, _i, _i, _p]),
+    "mlora_gemv_frag_silu": (_i, [_p, _p, _p, _i, _i, _i, _p]),
     "mlora_gemv_frag_split": (_i, [_p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _p]),
     "mlora_rope_kv_append_lora": (_i, [_p, _p, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p]),
     "mlora_lora_expand_rmsnorm": (_i, [_p, _i, _p, _p, _i, _p, _p, _f, _p, _f, _i, _i, _i, _i, _i, _p]),
@@ -57,7 +58,7 @@ class LoraProj(C.Structure):
 
 
 class Layer(C.Structure):
-    _fields_ = [("qkv_p", _p), ("o_p", _p), ("gate_up_p", _p), ("down_p", _p), ("ln1", _p), ("ln2", _p),
+    _fields_ = [("qkv_p", _p), ("o_p", _p), ("gate_up_p", _p), ("gate_up_il_p", _p), ("down_p", _p), ("ln1", _p), ("ln2", _p),
                 ("lora", LoraProj * 7), ("k_cache", _p), ("v_cache", _p)]
 
 

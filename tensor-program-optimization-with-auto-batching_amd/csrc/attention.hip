@@ -39,37 +39,54 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qk
   const int half = D >> 1;
   const int proj = hh < Hq ? 0 : (hh < Hq + Hkv ? 1 : 2);
   const int head = hh - (proj == 0 ? 0 : (proj == 1 ? Hq : Hq + Hkv));
-  const f16* brow = nullptr;
-  if (lx.src.v != nullptr && lx.B[proj] != nullptr) {          // block-uniform
-    const int id = lx.ids[t];
-    if (id >= 0 && id < lx.n_ad) {
-      if (i < lx.r) lv[i] = lora_v_from(lx.src, proj, id, lx.r, t, i, lx.scaling);
-      __syncthreads();
+  // Two dependent rounds of loads instead of five: the indices first, then everything they address.
+  const bool lora = lx.src.v != nullptr && lx.B[proj] != nullptr;          // block-uniform
+  const int seq = tok_seq[t], pos = tok_pos[t];
+  const int id = lora ? lx.ids[t] : -1;
+  const bool adapted = lora && id >= 0 && id < lx.n_ad;
+  const bool valid = !(seq < 0 || seq >= n_seq || pos < 0 || pos >= max_pos || pos / PAGE >= max_blocks);
+  const bool active = valid && i < half;
+  f16* src = qkv + ((size_t)t * (Hq + 2 * Hkv) + hh) * D;
+  f16 h1 = (f16)0.f, h2 = (f16)0.f;
+  float c = 0.f, s = 0.f;
+  int page = -1;
+  f16x8 b1[8], b2[8];
+  float lvv = 0.f;
+  if (adapted && i < lx.r) lvv = lora_v_from(lx.src, proj, id, lx.r, t, i, lx.scaling);
+  if (active) {
+    h1 = src[i];
+    h2 = src[i + half];
+    if (hh >= Hq) page = block_table[(size_t)seq * max_blocks + pos / PAGE];
+    if (hh < Hq + Hkv) {
+      c = rope_cos[(size_t)pos * half + i];
+      s = rope_sin[(size_t)pos * half + i];
+    }
+    if (adapted) {
       const int n_rows = (proj == 0 ? Hq : Hkv) * D;
-      brow = lx.B[proj] + ((size_t)id * n_rows + (size_t)head * D) * lx.r;
+      const f16* brow = lx.B[proj] + ((size_t)id * n_rows + (size_t)head * D) * lx.r;
+      lora_row_load(brow + (size_t)i * lx.r, lx.r, b1);
+      lora_row_load(brow + (size_t)(i + half) * lx.r, lx.r, b2);
     }
   }
-  if (i >= half) return;
-  const int seq = tok_seq[t], pos = tok_pos[t];
-  if (seq < 0 || seq >= n_seq || pos < 0 || pos >= max_pos || pos / PAGE >= max_blocks) return;
-  f16* src = qkv + ((size_t)t * (Hq + 2 * Hkv) + hh) * D;
-  f16 h1 = src[i], h2 = src[i + half];
-  if (brow != nullptr) {
+  if (adapted) {
+    if (i < lx.r) lv[i] = lvv;
+    __syncthreads();
+  }
+  if (!active) return;
+  if (adapted) {
     {
 #pragma clang fp contract(fast)
-      h1 = (f16)((float)h1 + lora_row_dot(brow + (size_t)i * lx.r, lv, lx.r));
-      h2 = (f16)((float)h2 + lora_row_dot(brow + (size_t)(i + half) * lx.r, lv, lx.r));
+      h1 = (f16)((float)h1 + lora_row_dot_regs(b1, lv, lx.r));
+      h2 = (f16)((float)h2 + lora_row_dot_regs(b2, lv, lx.r));
     }
   }
   if (hh >= Hq + Hkv) {
-    const int page = block_table[(size_t)seq * max_blocks + pos / PAGE];
     if (page < 0 || page >= n_pages) return;
     f16* dst = v_cache + ((size_t)page * Hkv + (hh - Hq - Hkv)) * D * PAGE + pos % PAGE;
     dst[(size_t)i * PAGE] = h1;
     dst[(size_t)(i + half) * PAGE] = h2;
     return;
   }
-  const float c = rope_cos[(size_t)pos * half + i], s = rope_sin[(size_t)pos * half + i];
   const float x1 = (float)h1, x2 = (float)h2;
   // Separately rounded products (fp contraction is off in this kernel) and an fp32 result that is
   // materialised before the fp16 conversion (the empty asm keeps the compiler from fusing the add
@@ -83,7 +100,6 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qk
     src[i] = o1;
     src[i + half] = o2;
   } else {
-    const int page = block_table[(size_t)seq * max_blocks + pos / PAGE];
     if (page < 0 || page >= n_pages) return;
     f16* dst = k_cache + (((size_t)page * Hkv + (hh - Hq)) * PAGE + pos % PAGE) * D;
     dst[i] = o1;

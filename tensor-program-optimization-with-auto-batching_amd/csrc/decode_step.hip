@@ -88,10 +88,16 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
       STEP(mlora_gemv_frag(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->attn, L.o_p, T, q_sz, H, stream));
       STEP(mlora_rmsnorm(p->xn, MLORA_FRAG, p->resid, MLORA_F32, L.ln2, p->eps, T, H, stream));
     }
-    STEP(mlora_gemv_frag(gu, MLORA_F16, MLORA_STORE, p->xn, L.gate_up_p, T, H, 2 * I, stream));
-    STEP(delta(gu, MLORA_F16, 2 * I, p->xn, L.lora[MLORA_GATE], H, I));
-    STEP(delta(gu + I, MLORA_F16, 2 * I, p->xn, L.lora[MLORA_UP], H, I));
-    STEP(mlora_silu_mul(p->act, MLORA_FRAG, gu, gu + I, 2 * I, T, I, stream));
+    const bool gu_lora = lora && (L.lora[MLORA_GATE].A || L.lora[MLORA_UP].A);
+    if (L.gate_up_il_p && !gu_lora && T <= 32) {
+      STEP(mlora_gemv_frag_silu(p->act, p->xn, L.gate_up_il_p, T, H, I, stream));
+    } else {
+      MLORA_CHECK(L.gate_up_p, MLORA_ERR_INVALID, "decode_step: layer %d needs gate_up_p", l);
+      STEP(mlora_gemv_frag(gu, MLORA_F16, MLORA_STORE, p->xn, L.gate_up_p, T, H, 2 * I, stream));
+      STEP(delta(gu, MLORA_F16, 2 * I, p->xn, L.lora[MLORA_GATE], H, I));
+      STEP(delta(gu + I, MLORA_F16, 2 * I, p->xn, L.lora[MLORA_UP], H, I));
+      STEP(mlora_silu_mul(p->act, MLORA_FRAG, gu, gu + I, 2 * I, T, I, stream));
+    }
     if (lora && L.lora[MLORA_DOWN].A) {
       const void* A1[1] = {L.lora[MLORA_DOWN].A};
       if (dense) STEP(mlora_gemv_frag_split(p->resid, MLORA_F32, MLORA_ACCUMULATE, (float*)ws_down, p->act, L.down_p, T, I, H, n_ad * r, stream));

@@ -21,7 +21,7 @@ constexpr int GEMV_WAVES = 8;
 constexpr int KSTEP = 32;   // k per MFMA
 constexpr int PIPE = 4;     // k-steps in flight per wave
 
-enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2 };
+enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2, OUT_SILU_FRAG = 3 };
 
 // With SHRINK the first `shrink_blocks` workgroups of the launch do LoRA shrink units (one per wave) on the same
 // x instead of a GEMV tile: the adapter work rides in the GEMV launch and finishes long before it does.
@@ -112,6 +112,32 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, 4) void gemv_kernel(void* __restr
     for (int j = 0; j < TT; ++j) red[wave][i * TT + j][lane] = acc[i][j];
   __syncthreads();
 
+  if constexpr (OUT == OUT_SILU_FRAG) {
+    // The weight interleaves 16-row tiles of gate and up, so this block's two tiles are gate rows c..c+15 and up
+    // rows c..c+15 of the same channels: out[t, c + ..] = silu(f16(gate)) * f16(up), written in fragment order.
+    static_assert(NT == 2 || OUT != OUT_SILU_FRAG, "the SiLU epilogue pairs a gate tile with an up tile");
+    for (int e = threadIdx.x; e < TT * WAVE; e += GEMV_WAVES * WAVE) {
+      const int j = e >> 6, sl = e & 63;
+      f32x4 sg = red[0][j][sl], su = red[0][TT + j][sl];
+#pragma unroll
+      for (int w = 1; w < GEMV_WAVES; ++w) {
+        sg += red[w][j][sl];
+        su += red[w][TT + j][sl];
+      }
+      const int c = bid * 16 + (sl >> 4) * 4;      // output channel of the first of this lane's 4 rows
+      const int t = j * 16 + (sl & 15);
+      if (t < T && c < N / 2) {
+        f16x4 o;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float gf = (float)(f16)sg[q];
+          o[q] = (f16)(gf / (1.f + expf(-gf)) * (float)(f16)su[q]);
+        }
+        *reinterpret_cast<f16x4*>((f16*)yv + frag_offset(t, c, TT)) = o;
+      }
+    }
+    return;
+  }
   // thread e < NT*TT*64 sums tile (e / 64), lane slot (e % 64) over the 8 waves in order
   for (int e = threadIdx.x; e < NT * TT * WAVE; e += GEMV_WAVES * WAVE) {
     const int tile = e >> 6, sl = e & 63;
@@ -130,7 +156,7 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, 4) void gemv_kernel(void* __restr
         *reinterpret_cast<f16x4*>((f16*)yv + o) = f16x4{(f16)s[0], (f16)s[1], (f16)s[2], (f16)s[3]};
       } else if constexpr (OUT == OUT_F32) {
         *reinterpret_cast<f32x4*>((float*)yv + o) = s;
-      } else {
+      } else if constexpr (OUT == OUT_ACC_F32) {
         f32x4* p = reinterpret_cast<f32x4*>((float*)yv + o);
         *p = *p + s;
       }
@@ -261,6 +287,20 @@ extern "C" int mlora_gemv_frag_lora(void* y, int y_dtype, int mode, const void* 
   b.frag_tt = mlora_frag_tiles(T);
   b.speculate = n_ad <= 2 * T;
   return gemv_dispatch<true, true, true>(y, y_dtype, mode, xf, K, Wp, T, K, N, stream, b);
+}
+
+extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p, int T, int K, int I, void* stream) {
+  MLORA_CHECK(act && xf && Wil_p, MLORA_ERR_INVALID, "gemv_frag_silu: null pointer");
+  MLORA_CHECK(T > 0 && T <= 32 && K > 0 && K % 32 == 0 && I > 0 && I % 32 == 0, MLORA_ERR_UNSUPPORTED,
+              "gemv_frag_silu: need 0 < T <= 32, K %% 32 == 0, I %% 32 == 0 (T=%d K=%d I=%d)", T, K, I);
+  const f16* xp = (const f16*)xf;
+  const f16* Wp = (const f16*)Wil_p;
+  hipStream_t s = (hipStream_t)stream;
+  const LoraShrinkBatch sb = LoraShrinkBatch();
+  const dim3 grid(I / 16), block(GEMV_WAVES * WAVE);
+  if (T <= 16) hipLaunchKernelGGL((gemv_kernel<2, 1, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr);
+  else hipLaunchKernelGGL((gemv_kernel<2, 2, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr);
+  return mlora_launch_status("gemv_frag_silu");
 }
 
 extern "C" int mlora_gemv_frag_split(void* y, int y_dtype, int mode, float* y2, const void* xf, const void* Wp, int T, int K,

@@ -149,6 +149,39 @@ __device__ __forceinline__ float lora_v_from(const LoraVSource& s, int slot, int
   return s.v[(size_t)t * s.ld + ((size_t)slot * s.n_ad + id) * r + j] * scaling;
 }
 
+// The same dot product in two halves, so that a caller can issue the row's loads before the v values are ready:
+// lora_row_load fetches up to 8 groups of 8 (r <= 64), lora_row_dot_regs consumes them in lora_row_dot's order.
+__device__ __forceinline__ void lora_row_load(const f16* __restrict__ brow, int r, f16x8 (&bv)[8]) {
+  const int ng = r >> 3;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    bv[q] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    if (q < ng) bv[q] = ld8(brow + q * 8);
+  }
+}
+
+__device__ __forceinline__ float lora_row_dot_regs(const f16x8 (&bv)[8], const float* __restrict__ v, int r) {
+  float g[8];
+  const int ng = r >> 3;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    float s = 0.f;
+    if (q < ng) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s = fmaf((float)bv[q][e], v[q * 8 + e], s);
+    }
+    g[q] = s;
+  }
+  if (ng > 4) {
+    g[0] = g[0] + g[1]; g[1] = g[2] + g[3]; g[2] = g[4] + g[5]; g[3] = g[6] + g[7];
+  }
+  if (ng > 2) {
+    g[0] = g[0] + g[1]; g[1] = g[2] + g[3];
+  }
+  if (ng > 1) g[0] = g[0] + g[1];
+  return g[0];
+}
+
 // delta = B_row[0..r) . v[0..r) with the summation tree of the stand-alone expand kernel: an fma chain over each
 // group of 8, then pairwise sums of neighbouring groups.
 __device__ __forceinline__ float lora_row_dot(const f16* __restrict__ brow, const float* __restrict__ v, int r) {

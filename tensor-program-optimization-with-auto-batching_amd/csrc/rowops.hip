@@ -43,46 +43,15 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(f16* __restrict__
   extern __shared__ float delta[];    // H floats when a LoRA expand is attached, otherwise empty
   const int row = blockIdx.x;
   XT* xr = x + (size_t)row * H;
-  bool has_delta = false;
-  if constexpr (sizeof(XT) == 4) {
-    if (lx.src.v != nullptr) {                      // block-uniform
-      const int id = lx.ids[row];
-      if (id >= 0 && id < lx.n_ad) {
-        has_delta = true;
-        if (threadIdx.x < lx.r) lv[threadIdx.x] = lora_v_from(lx.src, 0, id, lx.r, row, threadIdx.x, lx.scaling);
-        __syncthreads();
-        const f16* __restrict__ B = lx.B + (size_t)id * H * lx.r;
-        const int lpr = lx.r >> 3;                  // lanes (16-byte chunks) per output column
-        const int chunks = H * lpr;
-        for (int q0 = 0; q0 < chunks; q0 += NORM_THREADS * 8) {
-          f16x8 bv[8];
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            const int q = q0 + u * NORM_THREADS + threadIdx.x;
-            bv[u] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-            if (q < chunks) bv[u] = ld8(B + (size_t)q * 8);
-          }
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            const int q = q0 + u * NORM_THREADS + threadIdx.x;
-            const int sub = q % lpr;
-            float s = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) s = fmaf((float)bv[u][e], lv[sub * 8 + e], s);
-            for (int o = 1; o < lpr; o <<= 1) s += __shfl_xor(s, o, WAVE);   // neighbouring groups of 8 first
-            if (sub == 0 && q < chunks) delta[q / lpr] = s;
-          }
-        }
-        __syncthreads();
-      }
-    }
-  }
+  // The row and the norm weight are requested first: neither depends on the adapter id, so their latency
+  // overlaps the id -> (shrink results, B table) chain below.
   float v[VPT][8];
-  float ss = 0.f;
+  f16x8 wv[VPT];
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const int c = (i * NORM_THREADS + threadIdx.x) * 8;
     if (c < H) {
+      wv[i] = ld8(w + c);
       if constexpr (sizeof(XT) == 2) {
         const f16x8 t = ld8((const f16*)xr + c);
 #pragma unroll
@@ -95,6 +64,65 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(f16* __restrict__
           v[i][e] = lo[e];
           v[i][4 + e] = hi[e];
         }
+      }
+    }
+  }
+  bool has_delta = false;
+  if constexpr (sizeof(XT) == 4) {
+    if (lx.src.v != nullptr) {                      // block-uniform
+      const int id = lx.ids[row];
+      if (id >= 0 && id < lx.n_ad) {
+        has_delta = true;
+        const f16* __restrict__ B = lx.B + (size_t)id * H * lx.r;
+        const int lpr = lx.r >> 3;                  // lanes (16-byte chunks) per output column
+        const int chunks = H * lpr;
+        constexpr int NB = 8;
+        f16x8 bv[NB];
+        auto load_batch = [&](int q0) {
+#pragma unroll
+          for (int u = 0; u < NB; ++u) {
+            const int q = q0 + u * NORM_THREADS + threadIdx.x;
+            bv[u] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (q < chunks) bv[u] = ld8(B + (size_t)q * 8);
+          }
+        };
+        // the shrink results and the first batch of B go out together, before the barrier that publishes lv
+        float lvv = 0.f;
+        if (threadIdx.x < lx.r) lvv = lora_v_from(lx.src, 0, id, lx.r, row, threadIdx.x, lx.scaling);
+        load_batch(0);
+        if (threadIdx.x < lx.r) lv[threadIdx.x] = lvv;
+        __syncthreads();
+        for (int q0 = 0; q0 < chunks; q0 += NORM_THREADS * NB) {
+          float part[NB];
+#pragma unroll
+          for (int u = 0; u < NB; ++u) {
+            const int q = q0 + u * NORM_THREADS + threadIdx.x;
+            const int sub = q % lpr;
+            float s = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s = fmaf((float)bv[u][e], lv[sub * 8 + e], s);
+            part[u] = s;
+          }
+          if (q0 + NORM_THREADS * NB < chunks) load_batch(q0 + NORM_THREADS * NB);   // next batch flies during the reduce
+#pragma unroll
+          for (int u = 0; u < NB; ++u) {
+            const int q = q0 + u * NORM_THREADS + threadIdx.x;
+            const int sub = q % lpr;
+            float s = part[u];
+            for (int o = 1; o < lpr; o <<= 1) s += __shfl_xor(s, o, WAVE);   // neighbouring groups of 8 first
+            if (sub == 0 && q < chunks) delta[q / lpr] = s;
+          }
+        }
+        __syncthreads();
+      }
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = (i * NORM_THREADS + threadIdx.x) * 8;
+    if (c < H) {
+      if constexpr (sizeof(XT) == 4) {
         if (has_delta) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[i][e] = v[i][e] + delta[c + e];
@@ -112,10 +140,9 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(f16* __restrict__
   for (int i = 0; i < VPT; ++i) {
     const int c = (i * NORM_THREADS + threadIdx.x) * 8;
     if (c < H) {
-      const f16x8 wv = ld8(w + c);
       f16x8 o;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] = (f16)(v[i][e] * inv * (float)wv[e]);
+      for (int e = 0; e < 8; ++e) o[e] = (f16)(v[i][e] * inv * (float)wv[i][e]);
       st8(y + (frag_tt ? frag_offset(row, c, frag_tt) : (size_t)row * H + c), o);
     }
   }

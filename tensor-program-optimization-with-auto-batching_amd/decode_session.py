@@ -49,7 +49,7 @@ class NativeDecodeSession:
     replayed from a captured graph.  The graph is re-used as long as the batch does not change; the host only
     grows the block table when a sequence crosses a page boundary."""
 
-    def __init__(self, model, kv, seq_ids, adapter_ids, first_tokens, tid=0, use_graph=True, dense_lora=None):
+    def __init__(self, model, kv, seq_ids, adapter_ids, first_tokens, tid=0, use_graph=True, dense_lora=None, fuse_silu=True):
         import ctypes as C
         from . import _lib
         self.model, self.kv = model, kv
@@ -89,7 +89,10 @@ class NativeDecodeSession:
             dense_lora = lt is not None and lt.n_adapters <= 2 * T
         self.dense_lora = bool(dense_lora and lt is not None)
         ext = model.dense_lora_weights(tid) if self.dense_lora else None
+        il = model.interleaved_gate_up() if (fuse_silu and T <= 32 and s.intermediate_size % 32 == 0) else None
         for l, L in enumerate(model.layers):
+            if il is not None:
+                layers[l].gate_up_il_p = il[l].data.data_ptr()
             W = ext[l] if ext is not None else L
             layers[l].qkv_p, layers[l].o_p = W["qkv"].data.data_ptr(), W["o"].data.data_ptr()
             layers[l].gate_up_p, layers[l].down_p = L["gate_up"].data.data_ptr(), W["down"].data.data_ptr()

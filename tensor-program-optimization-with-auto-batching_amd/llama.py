@@ -94,6 +94,15 @@ class LlamaForCausalLM:
             m.add_lora_type(lt)
         return m
 
+    def interleaved_gate_up(self):
+        """Per layer, the gate/up matrix with 16-row tiles of gate and up alternating (for the GEMV whose epilogue
+        is the SiLU product).  Cached; one more copy of that matrix."""
+        cache = getattr(self, "_il_cache", None)
+        if cache is None:
+            cache = [ops.interleave_gate_up(L["gate_up"].unpack()) for L in self.layers]
+            self._il_cache = cache
+        return cache
+
     def dense_lora_weights(self, tid: int = 0):
         """Per layer, the qkv / o / down weights with the stacked A tables of adapter type `tid` appended as extra
         rows ([n_ad * r, K] per adapted projection; q, k, v slots always present for qkv, zero when not adapted),

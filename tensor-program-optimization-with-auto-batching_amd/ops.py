@@ -195,6 +195,26 @@ def _linear_frag(x, W, out, out_dtype, accumulate):
     return out
 
 
+def interleave_gate_up(gate_up: torch.Tensor) -> PackedWeight:
+    """[2I, K] (gate rows, then up rows) -> PackedWeight whose 16-row tiles alternate gate and up."""
+    I2, K = gate_up.shape
+    I = I2 // 2
+    if I % 16:
+        raise ValueError("interleave_gate_up: intermediate size must be a multiple of 16")
+    return PackedWeight(gate_up.view(2, I // 16, 16, K).permute(1, 0, 2, 3).reshape(I2, K).contiguous())
+
+
+def gate_up_silu(x: FragActivation, W_il: PackedWeight, out: FragActivation = None) -> FragActivation:
+    """silu(x @ Wgate.T) * (x @ Wup.T) in one launch; W_il from interleave_gate_up.  T <= 32."""
+    T, K = x.shape
+    I2, K2 = W_il.shape
+    if K2 != K:
+        raise ValueError(f"gate_up_silu: x{x.shape} vs W{W_il.shape}")
+    out = FragActivation(T, I2 // 2, x.device) if out is None else out
+    check(lib().mlora_gemv_frag_silu(out.data.data_ptr(), x.data.data_ptr(), W_il.data.data_ptr(), T, K, I2 // 2, _stream()))
+    return out
+
+
 def _out_arg(out, T, H, frag, device):
     """Output buffer of a producer: row-major tensor or FragActivation."""
     if frag:

@@ -339,3 +339,17 @@ def test_page_walk_bit_exact_with_integer_kv(ops, synth):
         for s in range(n_seq):
             for h in range(Hq):
                 assert np.all(o[s, h] == code[(s, sel[s], h)]), (probe, s, h, o[s, h, :4], code[(s, sel[s], h)])
+
+
+@pytest.mark.parametrize("T,K,I", [(1, 256, 64), (16, 512, 352), (32, 4096, 11008), (21, 1024, 96)])
+def test_gate_up_silu_epilogue_equals_two_launches(ops, synth, T, K, I):
+    """The GEMV whose epilogue is the SiLU product gives the bits of GEMV followed by silu_mul."""
+    x = synth.normal(5, "gus.x", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(5, "gus.w", (2 * I, K), 0.05, torch.float16, DEV)
+    xf = ops.FragActivation.pack(x)
+    gu = ops.linear(xf, ops.PackedWeight(W))
+    want = ops.silu_mul(gu)
+    got = ops.gate_up_silu(xf, ops.interleave_gate_up(W)).unpack()
+    assert torch.equal(got, want)
+    g = _np(x).astype(np.float64) @ _np(W).astype(np.float64).T
+    assert max_rel_err(_np(got), oracle.silu_mul_ref(g[:, :I], g[:, I:]), floor=1e-2) <= TOL
