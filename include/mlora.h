@@ -162,7 +162,8 @@ int mlora_argmax(int32_t* ids, const float* logits, int B, int V, void* stream);
  * (tvm/llama_auto_batcher/llama_exec_graph.py:75-85,121-127; llama_for_causal_lm.py:55-64).
  *
  * Layouts, per layer:
- *   k_cache [n_pages, Hkv, 16, D] f16   - rotated keys, one 16-token page of one head contiguous
+ *   k_cache [n_pages, Hkv, D/32, 4, 16, 8] f16 - rotated keys; a 16-token page of one head is contiguous and
+ *       in matrix-core fragment order: element (token, d) at ((d/32 * 4 + (d%32)/8) * 16 + token) * 8 + d%8
  *   v_cache [n_pages, Hkv, D, 16] f16   - values, token-minor inside a page
  *   block_table [n_seq, max_blocks] int32 - physical page of logical block j of sequence s
  *   qkv [T, Hq + 2 Hkv, D] f16 - fused projection output, token-major
@@ -175,7 +176,7 @@ int mlora_argmax(int32_t* ids, const float* logits, int B, int V, void* stream);
  * mlora_paged_attn_prefill: query token t (sequence tok_seq[t], position tok_pos[t]) attends to cached
  *   positions 0..tok_pos[t]; tokens of a sequence must be consecutive in t with increasing positions.
  * q is read from qkv (already rotated).  out [T, Hq * D] f16 (decode: in out_layout).  D in {64, 128};
- * Hq % Hkv == 0.
+ * Hq % Hkv == 0, Hq / Hkv <= 16 for decode.
  * ------------------------------------------------------------------------------------------- */
 int mlora_rope_kv_append(void* qkv, void* k_cache, void* v_cache,
                          const int32_t* block_table, int max_blocks,

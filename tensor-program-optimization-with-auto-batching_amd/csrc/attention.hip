@@ -1,17 +1,23 @@
 // Paged-KV attention for gfx950: RoPE + cache append, decode attention, prefill attention.
 //
 // Cache layout per layer (16-token pages):
-//   k_cache [n_pages, Hkv, 16, D]  rotated keys   - a page of one head is 16*D contiguous fp16
+//   k_cache [n_pages, Hkv, D/32, 4, 16, 8]  rotated keys in matrix-core fragment order: element (token, d) of a
+//                                   page sits at ((d/32 * 4 + (d%32)/8) * 16 + token) * 8 + d%8, so the
+//                                   16-token x 32-dim operand of one MFMA is a contiguous 1 KiB block
 //   v_cache [n_pages, Hkv, D, 16]  values         - token-minor, so a lane's 16-byte load holds 8
 //                                                   consecutive tokens of one dim
-// The K layout gives the decode kernel and the MFMA prefill kernel 16-byte loads along D; the V
-// layout gives both of them the P.V contraction (over tokens) without an LDS transpose.
+// Both attention kernels read K and V straight into MFMA operands: no LDS transpose, no shuffles.
 // The page-table walk is integer-only: page = block_table[seq, pos / 16], slot = pos % 16.
 #include "lora_device.h"
 
 namespace {
 
 constexpr int PAGE = MLORA_PAGE_SIZE;
+
+// element (token, d) inside one head's K page
+__device__ __forceinline__ int k_page_offset(int token, int d) {
+  return (((d >> 5) * 4 + ((d >> 3) & 3)) * PAGE + token) * 8 + (d & 7);
+}
 
 // LoRA expand of the q, k, v projections carried by the RoPE / append kernel: delta rows are added to the
 // projection output (and rounded to fp16, as the stand-alone expand does) before rotation and storage.
@@ -101,119 +107,137 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qk
     src[i + half] = o2;
   } else {
     if (page < 0 || page >= n_pages) return;
-    f16* dst = k_cache + (((size_t)page * Hkv + (hh - Hq)) * PAGE + pos % PAGE) * D;
-    dst[i] = o1;
-    dst[i + half] = o2;
+    f16* dst = k_cache + ((size_t)page * Hkv + (hh - Hq)) * PAGE * D;
+    dst[k_page_offset(pos % PAGE, i)] = o1;
+    dst[k_page_offset(pos % PAGE, i + half)] = o2;
   }
 }
 
 // ---------------------------------------------------------------------------------------------
-// Decode: one workgroup (4 waves) per (sequence, q head).  A wave takes pages w, w+4, ...; a page of
-// K is four (D=128) coalesced 1 KiB loads, as is a page of V.  Scores are reduced inside the group of
-// lanes that shares a token, broadcast with readlane, and folded into an fp32 online softmax; the
-// four waves' (max, sum, acc) states are merged through LDS.
+// Decode: one workgroup (4 waves) per (sequence, kv head); the G = Hq / Hkv <= 16 query heads that share the
+// kv head are the 16 columns of the matrix-core tiles, so K and V are read once per group.  A wave takes
+// pages w, w+4, ...  Per page:
+//   S^T = K . Q^T      4 (D=128) v_mfma_f32_16x16x32_f16, K fragments are contiguous 1 KiB loads;
+//                      accumulator rows are the page's tokens (lane group g holds tokens 4g..4g+3), columns
+//                      the query heads - a lane keeps the online-softmax state (m, l) of its own column
+//   O^T += V^T . P^T   one MFMA per 16 dims; the lane's four probabilities are already the B operand it
+//                      must supply (hi + lo fp16 halves in k-slots 0-3 / 4-7, V repeated in both, so P
+//                      enters with ~22 mantissa bits), and the rescale factor alpha is the lane's own.
+// The four waves' (m, l, O) states are merged through LDS.
 // ---------------------------------------------------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(256) void paged_attn_decode_kernel(f16* __restrict__ out, const f16* __restrict__ qkv,
-                                                                const f16* __restrict__ k_cache,
-                                                                const f16* __restrict__ v_cache,
-                                                                const int32_t* __restrict__ block_table, int max_blocks,
-                                                                const int32_t* __restrict__ seq_ids,
-                                                                const int32_t* __restrict__ ctx_len, int Hq, int Hkv,
-                                                                int n_pages, int n_seq, float scale, int frag_tt) {
-  constexpr int LPT = D / 8;          // lanes sharing one token of a K load
-  constexpr int TPL = WAVE / LPT;     // tokens per K load
-  constexpr int NK = PAGE / TPL;      // K loads per page
-  constexpr int NV = D * PAGE / 512;  // V loads per page (512 fp16 each)
-  constexpr int NW = 4;
-  __shared__ float sm[NW], sl[NW];
-  __shared__ float sacc[NW][D];
+constexpr int ATT_WAVES = 4;
 
-  const int b = blockIdx.x, h = blockIdx.y;
+template <int D>
+__global__ __launch_bounds__(ATT_WAVES * WAVE, 4) void paged_attn_decode_kernel(
+    f16* __restrict__ out, const f16* __restrict__ qkv, const f16* __restrict__ k_cache, const f16* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ seq_ids,
+    const int32_t* __restrict__ ctx_len, int Hq, int Hkv, int n_pages, int n_seq, float scale, int frag_tt) {
+  constexpr int NKB = D / 32;   // k-blocks of the QK^T product
+  constexpr int NDB = D / 16;   // dim blocks of the output
+  constexpr int NW = ATT_WAVES;
+  __shared__ float sm[NW][16], sl[NW][16];
+  extern __shared__ float sacc[];   // [NW][G][D]
+
+  const int b = blockIdx.x, kh = blockIdx.y;
+  const int G = Hq / Hkv;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int kh = h / (Hq / Hkv);
+  const int col = lane & 15, g = lane >> 4;
   const int seq = seq_ids[b];
   int ctx = ctx_len[b];
   if (seq < 0 || seq >= n_seq) ctx = 0;
   if (ctx > max_blocks * PAGE) ctx = max_blocks * PAGE;
   const int npages = (ctx + PAGE - 1) / PAGE;
+  const int32_t* __restrict__ bt = block_table + (size_t)(seq < 0 || seq >= n_seq ? 0 : seq) * max_blocks;
 
-  const f16x8 q8 = ld8(qkv + ((size_t)b * (Hq + 2 * Hkv) + h) * D + (lane % LPT) * 8);
+  // Q^T as the B operand: lane holds q[head kh*G + col][kb*32 + g*8 .. +8], zero for unused columns
+  f16x8 qf[NKB];
+#pragma unroll
+  for (int kb = 0; kb < NKB; ++kb) qf[kb] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  if (col < G) {
+    const f16* qp = qkv + ((size_t)b * (Hq + 2 * Hkv) + kh * G + col) * D + g * 8;
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) qf[kb] = ld8(qp + kb * 32);
+  }
 
   float m = -INFINITY, l = 0.f;
-  float acc[NV];
+  f32x4 O[NDB];
 #pragma unroll
-  for (int i = 0; i < NV; ++i) acc[i] = 0.f;
+  for (int db = 0; db < NDB; ++db) O[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  int page = wave < npages ? bt[wave] : -1;
   for (int pg = wave; pg < npages; pg += NW) {
-    const int page = block_table[(size_t)seq * max_blocks + pg];
-    if (page < 0 || page >= n_pages) continue;   // wave-uniform
-    const f16* kp = k_cache + ((size_t)page * Hkv + kh) * PAGE * D + lane * 8;
-    const f16* vp = v_cache + ((size_t)page * Hkv + kh) * D * PAGE + lane * 8;
-    f16x8 kf[NK], vf[NV];
+    const int next = pg + NW < npages ? bt[pg + NW] : -1;   // the next page id is requested one page ahead
+    if (page >= 0 && page < n_pages) {                      // wave-uniform
+      const f16* kp = k_cache + ((size_t)page * Hkv + kh) * PAGE * D + lane * 8;
+      const f16* vp = v_cache + (((size_t)page * Hkv + kh) * D + col) * PAGE + g * 4;   // dim col (+16 db), tokens 4g..
+      f16x8 kf[NKB];
+      f16x4 vf[NDB];
 #pragma unroll
-    for (int i = 0; i < NK; ++i) kf[i] = ld8(kp + i * 512);
+      for (int kb = 0; kb < NKB; ++kb) kf[kb] = ld8(kp + kb * 512);
 #pragma unroll
-    for (int i = 0; i < NV; ++i) vf[i] = ld8(vp + i * 512);
+      for (int db = 0; db < NDB; ++db) vf[db] = *reinterpret_cast<const f16x4*>(vp + db * 16 * PAGE);
 
-    float sc[PAGE];
+      f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f};   // st[r] = S[token 4g + r][head col]
 #pragma unroll
-    for (int i = 0; i < NK; ++i) {
-      float s = dot8(q8, kf[i], 0.f);
+      for (int kb = 0; kb < NKB; ++kb) st = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kb], qf[kb], st, 0, 0, 0);
+
+      float pm = -INFINITY;
 #pragma unroll
-      for (int o = LPT >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, WAVE);
-      s *= scale;
+      for (int r = 0; r < 4; ++r) {
+        st[r] = (pg * PAGE + 4 * g + r >= ctx) ? -INFINITY : st[r] * scale;
+        pm = fmaxf(pm, st[r]);
+      }
+      pm = fmaxf(pm, __shfl_xor(pm, 16, WAVE));
+      pm = fmaxf(pm, __shfl_xor(pm, 32, WAVE));
+      const float m_new = fmaxf(m, pm);       // finite: the first token of a visited page is < ctx
+      const float alpha = __expf(m - m_new);
+      f16x8 pa;
+      float ps = 0.f;
 #pragma unroll
-      for (int g = 0; g < TPL; ++g)
-        sc[i * TPL + g] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s), g * LPT));
+      for (int r = 0; r < 4; ++r) {
+        const float p = __expf(st[r] - m_new);
+        ps += p;
+        const f16 hi = (f16)p;
+        pa[r] = hi;
+        pa[4 + r] = (f16)(p - (float)hi);
+      }
+      l = l * alpha + ps;                     // per-lane share of the column's sum; lanes are combined at the end
+      m = m_new;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        O[db] *= alpha;
+        const f16x8 vv = f16x8{vf[db][0], vf[db][1], vf[db][2], vf[db][3], vf[db][0], vf[db][1], vf[db][2], vf[db][3]};
+        O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vv, pa, O[db], 0, 0, 0);   // O^T[dim 16db+4g+r][head col]
+      }
     }
-    float pm = -INFINITY;
-#pragma unroll
-    for (int tk = 0; tk < PAGE; ++tk) {
-      if (pg * PAGE + tk >= ctx) sc[tk] = -INFINITY;
-      pm = fmaxf(pm, sc[tk]);
-    }
-    const float m_new = fmaxf(m, pm);     // finite: the first token of a visited page is < ctx
-    const float alpha = __expf(m - m_new);
-    float ps = 0.f;
-#pragma unroll
-    for (int tk = 0; tk < PAGE; ++tk) {
-      sc[tk] = __expf(sc[tk] - m_new);
-      ps += sc[tk];
-    }
-    l = l * alpha + ps;
-    m = m_new;
-    const bool hi = lane & 1;
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      float a = acc[i] * alpha;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) a = fmaf(hi ? sc[8 + e] : sc[e], (float)vf[i][e], a);
-      acc[i] = a;
-    }
+    page = next;
   }
+  l += __shfl_xor(l, 16, WAVE);
+  l += __shfl_xor(l, 32, WAVE);
+  if (col < G) {
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    acc[i] += __shfl_xor(acc[i], 1, WAVE);
-    if ((lane & 1) == 0) sacc[wave][i * 32 + (lane >> 1)] = acc[i];
-  }
-  if (lane == 0) {
-    sm[wave] = m;
-    sl[wave] = l;
+    for (int db = 0; db < NDB; ++db)
+      *reinterpret_cast<f32x4*>(&sacc[((size_t)wave * G + col) * D + db * 16 + 4 * g]) = O[db];
+    if (g == 0) {
+      sm[wave][col] = m;
+      sl[wave][col] = l;
+    }
   }
   __syncthreads();
-  if (threadIdx.x < D) {
-    float M = sm[0];
+  for (int e = threadIdx.x; e < G * D; e += NW * WAVE) {
+    const int qh = e / D, d = e % D;
+    float M = sm[0][qh];
 #pragma unroll
-    for (int w = 1; w < NW; ++w) M = fmaxf(M, sm[w]);
+    for (int w = 1; w < NW; ++w) M = fmaxf(M, sm[w][qh]);
     float L = 0.f, o = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
-      const float f = sm[w] == -INFINITY ? 0.f : __expf(sm[w] - M);
-      L += sl[w] * f;
-      o += sacc[w][threadIdx.x] * f;
+      const float f = sm[w][qh] == -INFINITY ? 0.f : __expf(sm[w][qh] - M);
+      L += sl[w][qh] * f;
+      o += sacc[((size_t)w * G + qh) * D + d] * f;
     }
-    const size_t oo = frag_tt ? frag_offset(b, h * D + threadIdx.x, frag_tt) : ((size_t)b * Hq + h) * D + threadIdx.x;
+    const int h = kh * G + qh;
+    const size_t oo = frag_tt ? frag_offset(b, h * D + d, frag_tt) : ((size_t)b * Hq + h) * D + d;
     out[oo] = (f16)(L > 0.f ? o / L : 0.f);
   }
 }
@@ -274,12 +298,12 @@ __global__ __launch_bounds__(256) void paged_attn_prefill_kernel(f16* __restrict
     for (int pg = 0; pg < npages; ++pg) {
       const int page = block_table[(size_t)cur_seq * max_blocks + pg];
       if (page < 0 || page >= n_pages) continue;   // wave-uniform
-      const f16* kp = k_cache + (((size_t)page * Hkv + kh) * PAGE + qi) * D + g * 8;   // key qi of the page
+      const f16* kp = k_cache + ((size_t)page * Hkv + kh) * PAGE * D + lane * 8;       // key qi, dims 8g.. of each k-block
       const f16* vp = v_cache + (((size_t)page * Hkv + kh) * D + qi) * PAGE + g * 4;   // dim qi (+16 db), keys 4g..
       f16x8 kf[NKB];
       f16x4 vf[NDB];
 #pragma unroll
-      for (int kb = 0; kb < NKB; ++kb) kf[kb] = ld8(kp + kb * 32);
+      for (int kb = 0; kb < NKB; ++kb) kf[kb] = ld8(kp + kb * 512);
 #pragma unroll
       for (int db = 0; db < NDB; ++db) vf[db] = *reinterpret_cast<const f16x4*>(vp + db * 16 * PAGE);
 
@@ -407,11 +431,14 @@ extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qk
   if (B == 0) return MLORA_OK;
   const float scale = 1.f / sqrtf((float)D);
   hipStream_t s = (hipStream_t)stream;
+  const int G = Hq / Hkv;
+  MLORA_CHECK(G <= 16, MLORA_ERR_UNSUPPORTED, "paged_attn_decode: more than 16 query heads per kv head (%d)", G);
+  const size_t lds = (size_t)ATT_WAVES * G * D * sizeof(float);
   if (D == 128)
-    hipLaunchKernelGGL(paged_attn_decode_kernel<128>, dim3(B, Hq), dim3(256), 0, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
+    hipLaunchKernelGGL(paged_attn_decode_kernel<128>, dim3(B, Hkv), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
                        (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale, frag_tt);
   else
-    hipLaunchKernelGGL(paged_attn_decode_kernel<64>, dim3(B, Hq), dim3(256), 0, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
+    hipLaunchKernelGGL(paged_attn_decode_kernel<64>, dim3(B, Hkv), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
                        (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale, frag_tt);
   return mlora_launch_status("paged_attn_decode");
 }

@@ -36,7 +36,10 @@ class PagedKVCache:
         self.n_layers, self.n_pages, self.Hkv, self.D = n_layers, n_pages, n_kv_heads, head_dim
         self.max_seqs, self.max_blocks, self.max_pos = max_seqs, max_blocks, max_pos
         self.device = torch.device(device)
-        self.k = torch.zeros((n_layers, n_pages, n_kv_heads, PAGE, head_dim), dtype=torch.float16, device=self.device)
+        if head_dim % 32:
+            raise ValueError("head_dim must be a multiple of 32")
+        # keys in matrix-core fragment order: element (token, d) of a page at [d // 32, (d % 32) // 8, token, d % 8]
+        self.k = torch.zeros((n_layers, n_pages, n_kv_heads, head_dim // 32, 4, PAGE, 8), dtype=torch.float16, device=self.device)
         self.v = torch.zeros((n_layers, n_pages, n_kv_heads, head_dim, PAGE), dtype=torch.float16, device=self.device)
         cos, sin = rope_tables(head_dim, rope_theta, max_pos)
         self.rope_cos = torch.from_numpy(cos).to(self.device)
@@ -51,6 +54,11 @@ class PagedKVCache:
         self.block_table = torch.from_numpy(self.table_h.copy()).to(self.device)
         self._dirty = False
         self._cur = None
+
+    def k_rowmajor(self, layer: int) -> torch.Tensor:
+        """The layer's rotated keys as [n_pages, Hkv, 16, D] (a copy, for inspection)."""
+        k = self.k[layer]
+        return k.permute(0, 1, 4, 2, 3, 5).reshape(self.n_pages, self.Hkv, PAGE, self.D).contiguous()
 
     # ------------------------------------------------------------------ protocol
     def add_sequence(self, sid):

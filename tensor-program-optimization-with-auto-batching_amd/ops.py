@@ -269,7 +269,8 @@ def argmax(logits, out=None):
 
 
 def rope_kv_append(qkv, k_cache, v_cache, block_table, tok_seq, tok_pos, rope_cos, rope_sin, Hq, Hkv, D):
-    """qkv [T, Hq+2Hkv, D] f16 (q rotated in place); k_cache [n_pages,Hkv,16,D], v_cache [n_pages,Hkv,D,16]."""
+    """qkv [T, Hq+2Hkv, D] f16 (q rotated in place); k_cache [n_pages,Hkv,D/32,4,16,8] (fragment order),
+    v_cache [n_pages,Hkv,D,16]."""
     T = qkv.shape[0]
     n_pages = k_cache.shape[0]
     n_seq, max_blocks = block_table.shape

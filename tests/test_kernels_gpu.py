@@ -287,7 +287,7 @@ def test_paged_attention_prefill_then_decode(ops, synth, Hq, Hkv, D):
     # cache contents: rotated K and V, page by page, against the oracle's pages
     k_ref = oracle.f16(ref.k[0])                       # [n_pages, Hkv, 16, D]
     v_ref = oracle.f16(ref.v[0]).transpose(0, 1, 3, 2)  # -> [n_pages, Hkv, D, 16]
-    assert max_rel_err(_np(cache.k[0]), k_ref) <= TOL
+    assert max_rel_err(_np(cache.k_rowmajor(0)), k_ref) <= TOL
     assert np.array_equal(_np(cache.v[0]), v_ref)
 
 
