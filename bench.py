@@ -47,6 +47,19 @@ def prefill_all(model, kv, prompts, adapter_ids, chunk=4):
     return first
 
 
+def profiled_gemv_traffic():
+    """HBM bytes per GEMV launch from the committed rocprofv3 counter summary (FETCH_SIZE and WRITE_SIZE runs of
+    `bench.py --probe`, each scaled by what the counter reads for a plain 256 MiB copy), weighted over the launch
+    mix of one decode step; None when the summary is not there."""
+    import re
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "gemv_gather_mm_pmc_fetch_write.txt")
+    try:
+        m = re.search(r"gemv_mix_hbm_bytes_per_launch=(\d+)", open(path).read())
+    except OSError:
+        return None
+    return int(m.group(1)) if m else None
+
+
 def gemv_event_timing(model, T, reps=3):
     """Average duration of the weight-streaming GEMV over one decode step's worth of launches (the four
     fused projections of every layer + lm_head, 129 launches on 129 distinct weight matrices), issued back to
@@ -246,7 +259,7 @@ def main():
     if not args.no_extras:
         g = gemv_event_timing(model, wl.batch)
         out["roofline"] = {"kernel": "gemv_kernel (fragment-ordered weights and activations, T=32)", "bound": "hbm", "achieved": g["gbs"],
-                           "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g["gbs"] / HBM_PEAK_GBS, "traffic": None,
+                           "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g["gbs"] / HBM_PEAK_GBS, "traffic": profiled_gemv_traffic(),
                            "launches_timed": g["launches"], "avg_launch_us": g["avg_us"],
                            "algorithmic_bytes_per_launch": g["bytes_per_launch"]}
         del sess, kv
