@@ -77,6 +77,14 @@ int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, int x_layout, 
                     const int32_t* tok_adapter, float scaling,
                     int T, int K, int N, int r, int n_ad,
                     void* workspace, size_t workspace_bytes, void* stream);
+/* Several independent gather-matmul problems of one shape and one token->adapter table in ONE launch (decode
+ * shapes: T <= 64 and (K-slices + 1) * T * r * 4 <= 48 KiB of LDS, else MLORA_ERR_UNSUPPORTED).
+ * sets: DEVICE array of n_sets records of four pointers {y, x, A, B}, laid out as above.  This is how a decode step
+ * meets the op: every layer and projection has its own A / B / x / y, and the ~2 us of work per problem is far below
+ * the cost of a launch.  Same result bits as n_sets calls of mlora_gather_mm.  Replaces the same reference code. */
+int mlora_gather_mm_batch(const void* const* sets, int n_sets, int y_dtype, int ldy, int x_layout,
+                          const int32_t* tok_adapter, float scaling,
+                          int T, int K, int N, int r, int n_ad, void* stream);
 
 /* The two halves of the above, for callers that fuse differently:
  *   shrink: v_part[c, t, :] = A[id_t][:, chunk c] . x[t, chunk c]   (fp32 partials per K-chunk)

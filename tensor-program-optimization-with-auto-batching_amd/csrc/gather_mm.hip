@@ -117,6 +117,165 @@ __global__ __launch_bounds__(64) void lora_expand_kernel(YT* __restrict__ y, con
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Decode-shaped gather-matmul (T <= 64) in ONE launch.  A workgroup of 8 waves owns (adapter a, slice p of the
+// output rows):
+//   1. wave c runs the shrink unit of K-slice c of A[a] for the tokens bound to a (found with ballots) and leaves
+//      its fp32 partials in LDS - the P workgroups of an adapter repeat this, which costs L2 reads of A[a] but no
+//      grid-wide dependency; the workgroup index is laid out so that all slices of an adapter run on the same XCD
+//      (index % 8) and share that XCD's L2;
+//   2. the partials are summed in slice order and scaled (LDS);
+//   3. every thread owns output rows n of the slice: it loads row n of B[a] once and read-modify-writes y[t, n]
+//      for each token of the adapter.
+// Same arithmetic, in the same order, as lora_shrink_kernel followed by lora_expand_kernel.
+// A launch can cover several independent problems (sets of y, x, A, B with a common shape and adapter table):
+// blockIdx.y selects the set.
+// ---------------------------------------------------------------------------------------------
+struct GmmSet {
+  void* y;
+  const f16* x;
+  const f16* A;
+  const f16* B;
+};
+
+constexpr int GMM_WAVES = 8;
+constexpr int GMM_THREADS = GMM_WAVES * WAVE;
+
+// B[n, 0..R) . v[0..R): an fma chain over each group of 8, then pairwise sums of neighbouring groups
+// (the order of lora_expand_kernel and lora_row_dot).
+template <int R>
+__device__ __forceinline__ float row_dot(const f16x8 (&bv)[R / 8], const float* __restrict__ v) {
+  constexpr int NG = R / 8;
+  float g[NG];
+#pragma unroll
+  for (int q = 0; q < NG; ++q) {
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s = fmaf((float)bv[q][e], v[q * 8 + e], s);
+    g[q] = s;
+  }
+#pragma unroll
+  for (int n = NG; n > 1; n >>= 1)
+#pragma unroll
+    for (int q = 0; q < n / 2; ++q) g[q] = g[2 * q] + g[2 * q + 1];
+  return g[0];
+}
+
+template <int R, typename YT>
+__global__ __launch_bounds__(GMM_THREADS) void gather_mm_decode_kernel(GmmSet one, const GmmSet* __restrict__ sets,
+                                                                        const int32_t* __restrict__ ids, float scaling,
+                                                                        int T, int K, int N, int n_ad, int ldy,
+                                                                        int frag_tt, int P, int ci_n, int kc) {
+  constexpr int G = R < 16 ? R : 16;         // rows of A reduced together
+  constexpr int NG = R / 8;
+  extern __shared__ float lds[];             // part [kc][T][R], then v [T][R]
+  float* part = lds;
+  float* vfin = lds + (size_t)kc * T * R;
+  const int wg = blockIdx.x;
+  const int a = (wg & 7) + 8 * (wg / (8 * P));
+  const int p = (wg >> 3) % P;
+  if (a >= n_ad) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int id = lane < T ? ids[lane] : -1;            // T <= 64: one table row per lane
+  const unsigned long long mine = __ballot(id == a);
+  if (!mine) return;                                    // workgroup-uniform
+  const GmmSet s = sets ? sets[blockIdx.y] : one;
+  const f16* __restrict__ A = s.A + (size_t)a * R * K;
+  const f16* __restrict__ B = s.B + (size_t)a * N * R;
+  YT* __restrict__ y = (YT*)s.y;
+  const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+
+  // Requests that depend on the adapter table only go out first, ahead of the shrink: the thread's first row of B
+  // and the y elements of that row for the first two tokens of the adapter.
+  const int NS = ((N + P - 1) / P + 7) & ~7;            // rows per slice
+  const int n1 = min(N, (p + 1) * NS);
+  const int nf = p * NS + threadIdx.x;
+  const int ta = __builtin_ctzll(mine);
+  const unsigned long long rest1 = mine & (mine - 1);
+  const int tb = rest1 ? __builtin_ctzll(rest1) : -1;
+  f16x8 bfirst[NG];
+  float ya = 0.f, yb = 0.f;
+  if (nf < n1) {
+#pragma unroll
+    for (int q = 0; q < NG; ++q) bfirst[q] = ld8(B + (size_t)nf * R + q * 8);
+    ya = (float)y[(size_t)ta * ldy + nf];
+    if (tb >= 0) yb = (float)y[(size_t)tb * ldy + nf];
+  }
+
+  // ---- shrink: wave c owns K-slice c; tokens two at a time; same arithmetic as lora_shrink_unit
+  if (wave < kc) {
+    const int kbase = wave * ci_n * LORA_KCHUNK + lane * 8;
+    float* __restrict__ vp = part + (size_t)wave * T * R;
+    unsigned long long m = mine;
+    while (m) {
+      int tt[2];
+      tt[0] = __builtin_ctzll(m);
+      m &= m - 1;
+      tt[1] = -1;
+      if (m) {
+        tt[1] = __builtin_ctzll(m);
+        m &= m - 1;
+      }
+      const int t1 = tt[1] >= 0 ? tt[1] : tt[0];
+#pragma unroll
+      for (int jb = 0; jb < R; jb += G) {
+        float acc0[G], acc1[G];
+#pragma unroll
+        for (int j = 0; j < G; ++j) acc0[j] = acc1[j] = 0.f;
+        for (int ci = 0; ci < ci_n; ++ci) {
+          const int k = kbase + ci * LORA_KCHUNK;
+          const bool in = k < K;
+          const f16x8 x0 = in ? ld8(s.x + (frag_tt ? frag_offset(tt[0], k, frag_tt) : (size_t)tt[0] * K + k)) : zero8;
+          const f16x8 x1 = in ? ld8(s.x + (frag_tt ? frag_offset(t1, k, frag_tt) : (size_t)t1 * K + k)) : zero8;
+          f16x8 areg[G];
+#pragma unroll
+          for (int j = 0; j < G; ++j) areg[j] = in ? ld8(A + (size_t)(jb + j) * K + k) : zero8;
+#pragma unroll
+          for (int j = 0; j < G; ++j) {
+            acc0[j] = dot8(areg[j], x0, acc0[j]);
+            acc1[j] = dot8(areg[j], x1, acc1[j]);
+          }
+        }
+        const int j0 = reduce_transpose<G>(acc0, lane);
+        if ((lane & (WAVE / G - 1)) == 0) vp[(size_t)tt[0] * R + jb + j0] = acc0[0];
+        const int j1 = reduce_transpose<G>(acc1, lane);
+        if (tt[1] >= 0 && (lane & (WAVE / G - 1)) == 0) vp[(size_t)tt[1] * R + jb + j1] = acc1[0];
+      }
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < T * R; e += GMM_THREADS) {
+    const int t = e / R, j = e % R;
+    if ((mine >> t) & 1) vfin[e] = lora_v(part, kc, T, R, t, j, scaling);
+  }
+  __syncthreads();
+
+  // ---- expand: the thread's rows of the slice, every token of the adapter
+  if (nf < n1) {
+    y[(size_t)ta * ldy + nf] = (YT)(ya + row_dot<R>(bfirst, vfin + ta * R));
+    if (tb >= 0) y[(size_t)tb * ldy + nf] = (YT)(yb + row_dot<R>(bfirst, vfin + tb * R));
+    unsigned long long m = tb >= 0 ? rest1 & (rest1 - 1) : 0ull;
+    while (m) {
+      const int t = __builtin_ctzll(m);
+      m &= m - 1;
+      YT* yp = y + (size_t)t * ldy + nf;
+      *yp = (YT)((float)*yp + row_dot<R>(bfirst, vfin + t * R));
+    }
+  }
+  for (int n = nf + GMM_THREADS; n < n1; n += GMM_THREADS) {
+    f16x8 bv[NG];
+#pragma unroll
+    for (int q = 0; q < NG; ++q) bv[q] = ld8(B + (size_t)n * R + q * 8);
+    unsigned long long m = mine;
+    while (m) {
+      const int t = __builtin_ctzll(m);
+      m &= m - 1;
+      YT* yp = y + (size_t)t * ldy + n;
+      *yp = (YT)((float)*yp + row_dot<R>(bv, vfin + t * R));
+    }
+  }
+}
+
 __global__ void write_tensor_part_kernel(f16* __restrict__ Z, const f16* __restrict__ X, const f16* __restrict__ Y,
                                          const int32_t* __restrict__ ids, int B, int A, int PH) {
   // Phase split by blockIdx.y: 0 copies X -> Z (skipped when Z aliases X), 1 scatters Y rows.
@@ -200,13 +359,76 @@ extern "C" int mlora_lora_expand(void* y, int y_dtype, int ldy, const void* v_pa
   return mlora_launch_status("lora_expand");
 }
 
+// The one-launch kernel applies when the table fits one wave (T <= 64) and the partials fit LDS.
+static bool gmm_one_launch_fits(int T, int K, int r) {
+  return T > 0 && T <= 64 && (size_t)(lora_k_split(K).kc + 1) * T * r * sizeof(float) <= 48 * 1024;
+}
+
+template <int R>
+static void gmm_launch_r(const GmmSet& one, const GmmSet* sets, dim3 grid, size_t lds, int y_dtype, const int32_t* ids,
+                         float scaling, int T, int K, int N, int n_ad, int ldy, int frag_tt, int P, LoraKSplit ks, hipStream_t s) {
+  const dim3 block(GMM_THREADS);
+  if (y_dtype == MLORA_F16)
+    hipLaunchKernelGGL((gather_mm_decode_kernel<R, f16>), grid, block, lds, s, one, sets, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks.ci, ks.kc);
+  else
+    hipLaunchKernelGGL((gather_mm_decode_kernel<R, float>), grid, block, lds, s, one, sets, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks.ci, ks.kc);
+}
+
+static int gmm_one_launch(const GmmSet& one, const GmmSet* sets, int n_sets, int y_dtype, int ldy, int x_layout,
+                          const int32_t* ids, float scaling, int T, int K, int N, int r, int n_ad, hipStream_t s) {
+  const LoraKSplit ks = lora_k_split(K);
+  const int groups = ceil_div(n_ad, 8);                 // adapters are dealt to the 8 XCDs in groups of 8
+  // Output-row slices per adapter: enough workgroups to cover the chip when the launch holds one problem, one slice
+  // (no repeated shrink) once the problems themselves supply the parallelism.
+  int P = 256 / (groups * 8 * n_sets);
+  const int pmax = ceil_div(N, GMM_THREADS);
+  if (P > pmax) P = pmax;
+  if (P < 1) P = 1;
+  const size_t lds = (size_t)(ks.kc + 1) * T * r * sizeof(float);
+  const int frag_tt = x_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
+  const dim3 grid(groups * 8 * P, n_sets);
+  switch (r) {
+    case 8: gmm_launch_r<8>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s); break;
+    case 16: gmm_launch_r<16>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s); break;
+    case 32: gmm_launch_r<32>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s); break;
+    default: gmm_launch_r<64>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s); break;
+  }
+  return mlora_launch_status("gather_mm");
+}
+
+extern "C" int mlora_gather_mm_batch(const void* const* sets, int n_sets, int y_dtype, int ldy, int x_layout,
+                                     const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
+                                     void* stream) {
+  if (int e = check_lora_shape(T, K, N, r, n_ad)) return e;
+  MLORA_CHECK(sets && tok_adapter && n_sets >= 0 && n_sets <= 65535, MLORA_ERR_INVALID, "gather_mm_batch: null pointer or bad n_sets=%d", n_sets);
+  MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "gather_mm_batch: bad y_dtype %d", y_dtype);
+  MLORA_CHECK(ldy >= N, MLORA_ERR_INVALID, "gather_mm_batch: need ldy >= N (ldy=%d N=%d)", ldy, N);
+  MLORA_CHECK(x_layout == MLORA_ROWMAJOR || (x_layout == MLORA_FRAG && K % 32 == 0), MLORA_ERR_UNSUPPORTED,
+              "gather_mm_batch: fragment-ordered x needs K %% 32 == 0");
+  if (T == 0 || n_sets == 0) return MLORA_OK;
+  MLORA_CHECK(gmm_one_launch_fits(T, K, r), MLORA_ERR_UNSUPPORTED,
+              "gather_mm_batch: decode shapes only (T <= 64 and (kc + 1) * T * r * 4 <= 48 KiB; T=%d K=%d r=%d)", T, K, r);
+  return gmm_one_launch(GmmSet(), (const GmmSet*)sets, n_sets, y_dtype, ldy, x_layout, tok_adapter, scaling, T, K, N, r, n_ad,
+                        (hipStream_t)stream);
+}
+
 extern "C" int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, int x_layout, const void* A, const void* B,
                                const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
                                void* workspace, size_t workspace_bytes, void* stream) {
   if (int e = check_lora_shape(T, K, N, r, n_ad)) return e;
+  // the workspace is part of the contract whichever kernel runs (the one-launch kernel keeps its partials in LDS)
   MLORA_CHECK(workspace && workspace_bytes >= mlora_gather_mm_workspace_bytes(T, K, r) || T == 0, MLORA_ERR_WORKSPACE,
               "gather_mm: workspace of %zu bytes given, %zu needed", workspace_bytes,
               mlora_gather_mm_workspace_bytes(T, K, r));
+  if (gmm_one_launch_fits(T, K, r)) {
+    MLORA_CHECK(y && x && A && B && tok_adapter, MLORA_ERR_INVALID, "gather_mm: null pointer");
+    MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "gather_mm: bad y_dtype %d", y_dtype);
+    MLORA_CHECK(ldy >= N, MLORA_ERR_INVALID, "gather_mm: need ldy >= N (ldy=%d N=%d)", ldy, N);
+    MLORA_CHECK(x_layout == MLORA_ROWMAJOR || (x_layout == MLORA_FRAG && K % 32 == 0), MLORA_ERR_UNSUPPORTED,
+                "gather_mm: fragment-ordered x needs T <= 64 and K %% 32 == 0 (layout=%d T=%d K=%d)", x_layout, T, K);
+    const GmmSet one = {y, (const f16*)x, (const f16*)A, (const f16*)B};
+    return gmm_one_launch(one, nullptr, 1, y_dtype, ldy, x_layout, tok_adapter, scaling, T, K, N, r, n_ad, (hipStream_t)stream);
+  }
   if (int e = mlora_lora_shrink(workspace, x, x_layout, A, tok_adapter, T, K, r, n_ad, stream)) return e;
   return mlora_lora_expand(y, y_dtype, ldy, workspace, B, tok_adapter, scaling, T, K, N, r, n_ad, stream);
 }

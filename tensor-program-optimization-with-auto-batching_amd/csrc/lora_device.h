@@ -41,8 +41,13 @@ __device__ __forceinline__ int reduce_transpose(float (&p)[G], int lane) {
     const bool hi = (lane & off) != 0;
 #pragma unroll
     for (int i = 0; i < half; ++i) {
-      const float send = hi ? p[i] : p[i + half];
-      const float keep = hi ? p[i + half] : p[i];
+      // The two candidates are pinned in registers of their own (empty asm): left to itself the compiler folds the
+      // selects of all levels into one dynamically indexed read of p[], which it lowers to a 16-way compare/select
+      // chain per element - hundreds of instructions instead of two.
+      float a = p[i], b = p[i + half];
+      asm volatile("" : "+v"(a), "+v"(b));
+      const float send = hi ? a : b;
+      const float keep = hi ? b : a;
       p[i] = keep + __shfl_xor(send, off, WAVE);
     }
     j += hi ? half : 0;

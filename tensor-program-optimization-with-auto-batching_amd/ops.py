@@ -101,6 +101,36 @@ def gather_mm(y, x, A, B, tok_adapter, scaling: float, workspace=None):
     return y
 
 
+class GatherMMBatch:
+    """Several gather-matmul problems of one shape and one token->adapter table, issued as one launch.
+    sets: list of (y, x, A, B) as for gather_mm (x row-major); the tensors are kept alive by this object."""
+
+    def __init__(self, sets, tok_adapter, scaling: float):
+        y0, x0, A0, B0 = sets[0]
+        self.T, self.K = x0.shape
+        self.n_ad, self.r, _ = A0.shape
+        self.N = B0.shape[1]
+        self.ldy = y0.stride(0) if self.T > 1 else max(self.N, y0.stride(0))
+        self.ydt = _dt(y0)
+        ptrs = []
+        for y, x, A, B in sets:
+            if (x.shape != (self.T, self.K) or A.shape != (self.n_ad, self.r, self.K) or B.shape != (self.n_ad, self.N, self.r)
+                    or y.shape != (self.T, self.N) or _dt(y) != self.ydt or y.stride(1) != 1
+                    or (self.T > 1 and y.stride(0) != self.ldy)):
+                raise ValueError("GatherMMBatch: all sets must share shape, dtype and row stride")
+            ptrs += [y.data_ptr(), _dev(x, torch.float16, "x"), _dev(A, torch.float16, "A"), _dev(B, torch.float16, "B")]
+        self.sets = list(sets)
+        self.ids = tok_adapter
+        _dev(tok_adapter, torch.int32, "tok_adapter")
+        self.scaling = float(scaling)
+        self.table = torch.tensor(ptrs, dtype=torch.int64, device=x0.device)
+
+    def run(self):
+        check(lib().mlora_gather_mm_batch(self.table.data_ptr(), len(self.sets), self.ydt, self.ldy, ROWMAJOR,
+                                          self.ids.data_ptr(), self.scaling, self.T, self.K, self.N, self.r, self.n_ad,
+                                          _stream()))
+
+
 def lora_shrink(v_part, x, A, tok_adapter):
     xptr, xlay, T, K = _x_arg(x)
     n_ad, r, _ = A.shape

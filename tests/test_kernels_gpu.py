@@ -353,3 +353,43 @@ def test_gate_up_silu_epilogue_equals_two_launches(ops, synth, T, K, I):
     assert torch.equal(got, want)
     g = _np(x).astype(np.float64) @ _np(W).astype(np.float64).T
     assert max_rel_err(_np(got), oracle.silu_mul_ref(g[:, :I], g[:, I:]), floor=1e-2) <= TOL
+
+
+@pytest.mark.parametrize("T,K,N,r,n_ad,ydt", [
+    (64, 4096, 4096, 16, 32, torch.float16),     # the isolated-op benchmark shape
+    (32, 4096, 4096, 16, 16, torch.float32),
+    (17, 11008, 4096, 8, 5, torch.float16),      # three K-chunks per slice
+    (64, 1024, 264, 32, 70, torch.float16),      # more adapters than tokens, ragged N
+    (3, 512, 4096, 64, 2, torch.float16),
+])
+def test_gather_mm_one_launch_equals_shrink_then_expand(ops, synth, T, K, N, r, n_ad, ydt):
+    """Decode shapes take the single-launch kernel; its result has the bits of the two-kernel path (which the
+    larger shapes use and which the oracle tests cover)."""
+    c = synth.gather_mm_case(seed=7, T=T, K=K, N=N, r=r, n_ad=n_ad, device=DEV, tag=f"one{T}.{K}.{N}.{r}")
+    ids = c["ids"].clone()
+    ids[T // 2] = -1
+    y1 = c["y"].to(ydt).clone()
+    y2 = y1.clone()
+    ops.gather_mm(y1, c["x"], c["A"], c["B"], ids, 0.5)
+    vp = ops.gather_mm_workspace(T, K, r, DEV)
+    ops.lora_shrink(vp, c["x"], c["A"], ids)
+    ops.lora_expand(y2, vp, c["B"], ids, 0.5, K)
+    assert torch.equal(y1, y2)
+    ref = oracle.gather_mm_ref(_np(c["y"].to(ydt)), _np(c["x"]), _np(c["A"]), _np(c["B"]), ids.cpu().numpy(), 0.5)
+    assert max_rel_err(_np(y1), ref) <= TOL
+
+
+def test_gather_mm_batch_equals_separate_calls(ops, synth):
+    """Five problems with their own x, A, B, y in one launch: same bits as five calls."""
+    T, K, N, r, n_ad = 48, 2048, 1024, 16, 12
+    ids = synth.randint(9, "gmb.ids", (T,), n_ad, DEV)
+    sets, want = [], []
+    for j in range(5):
+        c = synth.gather_mm_case(seed=9, T=T, K=K, N=N, r=r, n_ad=n_ad, device=DEV, tag=f"gmb{j}")
+        y = c["y"].clone()
+        ops.gather_mm(y, c["x"], c["A"], c["B"], ids, 0.25)
+        want.append(y)
+        sets.append((c["y"].clone(), c["x"], c["A"], c["B"]))
+    ops.GatherMMBatch(sets, ids, 0.25).run()
+    for (y, _, _, _), w in zip(sets, want):
+        assert torch.equal(y, w)
