@@ -78,6 +78,14 @@ class LlamaAutoBatcherClass:
             self.current["generated"] = False
         self.seq_info.set_adapter(self.current["sid"], config, wid)
 
+    def load_adapters(self, cache_dir):
+        """Load the adapter types the registered requests use from `{cache_dir}/lora_adapters/r{rank}_a{wid}.safetensors`
+        (`compile_tvm.py:296-314`); call after the requests are registered and before compile()."""
+        from .adapter_files import load_adapters_for
+        if self.model is None:
+            raise RuntimeError("set_model() must be called before load_adapters()")
+        load_adapters_for(self.seq_info, self.model, cache_dir)
+
     def compile(self, fuse_decode=True):
         if fuse_decode:
             self.graph.fuse_batchable_ops()

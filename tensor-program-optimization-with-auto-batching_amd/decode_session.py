@@ -65,7 +65,7 @@ class NativeDecodeSession:
         self.rows = i32([kv.slot[q] for q in self.seq_ids])
         self.pos = i32([kv.lens[q] for q in self.seq_ids])
         self.ctx = self.pos + 1
-        self.tok_adapter = i32(adapter_ids) if lt is not None else None
+        self.tok_adapter = i32(lt.rows(np.asarray(adapter_ids, dtype=np.int32).reshape(-1))) if lt is not None else None
         H, I, V = s.hidden_size, s.intermediate_size, s.vocab_size
         f16, f32 = torch.float16, torch.float32
         fe = _lib.lib().mlora_frag_activation_elems

@@ -29,6 +29,23 @@ class LoraType:
     def __init__(self, r: int, scaling: float, n_adapters: int):
         self.r, self.scaling, self.n_adapters = r, float(scaling), n_adapters
         self.tables = {}     # (layer, proj) -> (A [n_ad, r, K], B [n_ad, N, r])
+        self.row_of = None   # weight id -> table row when the two differ (adapters loaded from files), else None
+
+    def rows(self, wids: np.ndarray) -> np.ndarray:
+        """Table rows of the weight ids `wids` (-1 stays -1); raises on an id that is not loaded."""
+        if self.row_of is None:
+            if wids.size and (wids.min() < -1 or wids.max() >= self.n_adapters):
+                raise ValueError(f"adapter weight id out of range: {wids.min()}..{wids.max()} of {self.n_adapters}")
+            return wids
+        out = np.full(wids.shape, -1, dtype=np.int32)
+        for i, w in enumerate(wids.tolist()):
+            if w >= 0:
+                if w not in self.row_of:
+                    raise ValueError(f"adapter weight id {w} is not loaded (loaded: {sorted(self.row_of)})")
+                out[i] = self.row_of[w]
+            elif w != -1:
+                raise ValueError(f"bad adapter weight id {w}")
+        return out
 
     def add(self, layer: int, proj: str, A: torch.Tensor, B: torch.Tensor):
         if A.shape[0] != self.n_adapters or A.shape[1] != self.r or B.shape[0] != self.n_adapters or B.shape[2] != self.r:
@@ -210,10 +227,7 @@ class LlamaForCausalLM:
         out = {}
         for tid, (sids, wids) in pairs.items():
             full = np.full(T, -1, dtype=np.int32)
-            w = _host_i32(wids)
-            lt = self.lora_types[tid]
-            if w.size and (w.min() < -1 or w.max() >= lt.n_adapters):      # -1 = no adapter for that row
-                raise ValueError(f"adapter weight id out of range for type {tid}: {w.min()}..{w.max()} of {lt.n_adapters}")
+            w = self.lora_types[tid].rows(_host_i32(wids))      # -1 = no adapter for that row
             if sids is None:
                 full[:] = np.broadcast_to(w, (T,)) if w.size in (1, T) else _bad(T, w)
             else:

@@ -117,3 +117,32 @@ def test_workload_configs():
     assert counts[0] == counts.max() and counts[0] > 20          # Zipf: adapter 0 is the most popular
     c4 = synth.config4()
     assert c4.lora.r == 64 and len(c4.lora.targets) == 7
+
+
+def test_adapter_files_round_trip_and_wid_translation(tmp_path):
+    """Adapters written in the reference's file layout (`r{rank}_a{wid}.safetensors`, PEFT-oriented fp32 tensors) load
+    into stacked tables; weight ids that are not 0..n-1 in order are translated to table rows (the reference indexes
+    the stack with the raw id, `compile_tvm.py:298-313` vs `llama_exec_graph.py:83`)."""
+    import torch
+    from safetensors.torch import load_file
+    synth, af = load_pkg("synth"), load_pkg("adapter_files")
+    shape = synth.LlamaShape(hidden_size=64, intermediate_size=96, num_attention_heads=4, num_key_value_heads=2,
+                             num_hidden_layers=2, head_dim=16, vocab_size=50)
+    d = str(tmp_path / "lora_adapters")
+    af.write_synthetic_adapters(d, shape, ranks=(8, 16), n_adapters=5, targets=("q_proj", "v_proj"), seed=3)
+    f = load_file(af.adapter_path(d, 16, 4))
+    assert sorted(f) == sorted(f"layers.{l}.self_attn.{p}.lora_{w}.weight" for l in range(2) for p in ("q_proj", "v_proj") for w in "AB")
+    assert f["layers.1.self_attn.v_proj.lora_B.weight"].shape == (32, 16) and f["layers.0.self_attn.q_proj.lora_A.weight"].dtype == torch.float32
+    lt = af.load_lora_type(d, 16, 8.0, [4, 0, 2], shape, device="cpu")
+    assert lt.n_adapters == 3 and lt.scaling == 0.5 and lt.row_of == {4: 0, 0: 1, 2: 2}
+    A, B = lt.tables[(1, "v_proj")]
+    assert A.shape == (3, 16, 64) and B.shape == (3, 32, 16) and A.dtype == torch.float16
+    want = load_file(af.adapter_path(d, 16, 2))["layers.1.self_attn.v_proj.lora_A.weight"].half()
+    assert torch.equal(A[2], want)
+    assert list(lt.rows(np.array([2, -1, 4, 0], dtype=np.int32))) == [2, -1, 0, 1]
+    with pytest.raises(ValueError):
+        lt.rows(np.array([3], dtype=np.int32))
+    with pytest.raises(FileNotFoundError):
+        af.load_lora_type(d, 16, 8.0, [7], shape, device="cpu")
+    with pytest.raises(ValueError):
+        af.load_lora_type(d, 16, 8.0, [1, 1], shape, device="cpu")

@@ -152,3 +152,60 @@ def test_per_request_max_gen_len_and_eos(c1):
             assert got[b] == exp, b
         else:
             assert len(got[b]) <= lens[b]
+
+
+def test_adapters_loaded_from_files_and_weight_id_translation(tmp_path):
+    """Adapters stored as `lora_adapters/r{rank}_a{wid}.safetensors` are loaded for the types and weight ids the
+    registered requests use (two ranks, weight ids out of order); tokens equal the oracle's, which indexes full
+    per-rank tables by the raw weight id."""
+    from safetensors.torch import load_file
+    synth, af, ab, lora, xg = (load_pkg(m) for m in ("synth", "adapter_files", "auto_batcher", "lora", "llama_exec_graph"))
+    shape = synth.LlamaShape(hidden_size=256, intermediate_size=704, num_attention_heads=4, num_key_value_heads=4,
+                             num_hidden_layers=2, head_dim=64, vocab_size=1000)
+    cache_dir = str(tmp_path)
+    d = cache_dir + "/lora_adapters"
+    n_files = 5
+    af.write_synthetic_adapters(d, shape, ranks=(8, 16), n_adapters=n_files, targets=("q_proj", "v_proj"), seed=6, std=0.05)
+    wl = synth.Workload("files", 6, shape, synth.LoraSpec(), batch=5, prompt_len=12, gen_len=5)
+    # request -> (rank, weight id); None = no adapter.  Type a0 = rank 16 (first seen), a1 = rank 8.
+    reqs = [(16, 4), None, (8, 2), (16, 1), (16, 4)]
+    P, max_gen_len = 12, 5
+    prompts = synth.randint(6, "files.prompts", (len(reqs), P), shape.vocab_size).numpy()
+    model = hip_model(wl, lora_specs=[])
+    batcher = ab.LlamaAutoBatcherClass()
+    batcher.set_model(model)
+    batcher.set_exec_config(xg.LlamaExecConfig(max_prompt_len=P, max_gen_len=max_gen_len, page_size=16))
+    results = []
+    for i, rq in enumerate(reqs):
+        var = batcher.create_var(np.asarray(prompts[i], dtype=np.int32))
+        if rq is not None:
+            batcher.set_adapter(lora.LoraConfig(r=rq[0], alpha=rq[0] / 2), wid=rq[1])
+        results.append(batcher.generate(var))
+    batcher.load_adapters(cache_dir)
+    assert [lt.r for lt in model.lora_types] == [16, 8]
+    assert set(model.lora_types[0].row_of) == {4, 1} and model.lora_types[1].row_of == {2: 0}
+    batcher.compile()
+    batcher.execute()
+    got = [list(map(int, r.var)) for r in results]
+
+    # oracle: full tables indexed by the raw weight id
+    w = {k: v.float().numpy() for k, v in synth.base_weights(wl.seed, shape, torch.float16, "cpu").items()}
+    lw, scaling = {}, {}
+    for tid, r in enumerate((16, 8)):
+        files = [load_file(af.adapter_path(d, r, wid)) for wid in range(n_files)]
+        for l in range(shape.num_hidden_layers):
+            for proj in ("q_proj", "v_proj"):
+                for which in "AB":
+                    lw[f"layers.{l}.{proj}.lora_{which}.a{tid}"] = np.stack(
+                        [f[af.tensor_key(l, proj, which)].half().float().numpy() for f in files])
+        scaling[f"a{tid}"] = 0.5
+    ref = oracle.LlamaRef(shape, w, lw, scaling, mode="mixed")
+    ids = {"a0": np.array([4, -1, -1, 1, 4], dtype=np.int32), "a1": np.array([-1, -1, 2, -1, -1], dtype=np.int32)}
+    n_pages = len(reqs) * 3
+    exp, margins, scales = oracle.greedy_generate_ref(ref, prompts, ids, max_gen_len, n_pages, 16, None, return_logits=True)
+    for b in range(len(reqs)):
+        i = next((i for i in range(max_gen_len) if got[b][i] != exp[b][i]), None)
+        assert i is None or margins[b][i] < 2e-2 * scales[b][i], (b, i, got[b], exp[b])
+    # the adapters must matter: dropping them changes at least one request's tokens
+    base, _, _ = oracle.greedy_generate_ref(ref, prompts, {}, max_gen_len, n_pages, 16, None, return_logits=True)
+    assert any(base[b] != exp[b] for b in (0, 2, 3, 4))
