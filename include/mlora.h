@@ -82,6 +82,30 @@ int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, int x_layout, 
  * sets: DEVICE array of n_sets records of four pointers {y, x, A, B}, laid out as above.  This is how a decode step
  * meets the op: every layer and projection has its own A / B / x / y, and the ~2 us of work per problem is far below
  * the cost of a launch.  Same result bits as n_sets calls of mlora_gather_mm.  Replaces the same reference code. */
+/* Adapters of several ranks in one batch.  Bucket b holds the adapters of one rank and scaling,
+ *   A [n_ad, r, K], B [n_ad, N, r]; token t uses adapter tok_adapter[t] of bucket tok_bucket[t]; a token whose
+ *   bucket is outside [0, n_buckets) or whose adapter id is outside [0, n_ad) of its bucket is left untouched.
+ * Every table is read at its own rank: nothing is padded to the largest rank and no rank is split into chunks, and
+ * rows are addressed by token, so there is no gather of x rows nor scatter of results.  Same result bits as one
+ * mlora_gather_mm call per bucket with the other buckets' tokens masked to -1.  workspace: the largest
+ * mlora_gather_mm_workspace_bytes(T, K, r) over the buckets; the launches of the buckets are ordered on `stream`.
+ * All buckets are validated before the first launch.  `buckets` is a HOST array; a bucket with A == B == NULL is
+ * skipped (its adapters do not target this projection) and its tokens are left untouched.
+ *
+ * Replaces: the per-type loop of the mixed decode (tvm/llama_auto_batcher/compile_tvm.py:135-155: take rows, delta,
+ * write_tensor_part scatter, add) and the padded / splitted / sequential multi-rank strategies of the case study
+ * (tvm/lora_only/case_study/multiple_ranks.py:21-151), which all compute this sum. */
+typedef struct mlora_lora_bucket {
+  const void* A;
+  const void* B;
+  int r;
+  int n_ad;
+  float scaling;
+} mlora_lora_bucket;
+int mlora_gather_mm_multi(void* y, int y_dtype, int ldy, const void* x, int x_layout,
+                          const mlora_lora_bucket* buckets, int n_buckets,
+                          const int32_t* tok_bucket, const int32_t* tok_adapter,
+                          int T, int K, int N, void* workspace, size_t workspace_bytes, void* stream);
 int mlora_gather_mm_batch(const void* const* sets, int n_sets, int y_dtype, int ldy, int x_layout,
                           const int32_t* tok_adapter, float scaling,
                           int T, int K, int N, int r, int n_ad, void* stream);

@@ -23,6 +23,7 @@ SIGNATURES = {
     "mlora_last_error": (C.c_char_p, []),
     "mlora_gather_mm_workspace_bytes": (_z, [_i, _i, _i]),
     "mlora_gather_mm": (_i, [_p, _i, _i, _p, _i, _p, _p, _p, _f, _i, _i, _i, _i, _i, _p, _z, _p]),
+    "mlora_gather_mm_multi": (_i, [_p, _i, _i, _p, _i, _p, _i, _p, _p, _i, _i, _i, _p, _z, _p]),
     "mlora_gather_mm_batch": (_i, [_p, _i, _i, _i, _i, _p, _f, _i, _i, _i, _i, _i, _p]),
     "mlora_lora_shrink": (_i, [_p, _p, _i, _p, _p, _i, _i, _i, _i, _p]),
     "mlora_lora_expand": (_i, [_p, _i, _i, _p, _p, _p, _f, _i, _i, _i, _i, _i, _p]),
@@ -52,6 +53,10 @@ SIGNATURES = {
     "mlora_paged_attn_prefill": (_i, [_p, _p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
 }
 
+
+
+class LoraBucket(C.Structure):
+    _fields_ = [("A", _p), ("B", _p), ("r", _i), ("n_ad", _i), ("scaling", _f)]
 
 
 class LoraProj(C.Structure):

@@ -46,7 +46,8 @@ template <int R, typename YT>
 __global__ __launch_bounds__(64) void lora_expand_kernel(YT* __restrict__ y, const float* __restrict__ vpart,
                                                          const f16* __restrict__ B,
                                                          const int32_t* __restrict__ ids, float scaling,
-                                                         int T, int N, int ldy, int KC) {
+                                                         int T, int N, int ldy, int KC,
+                                                         const int32_t* __restrict__ bucket_of, int bucket) {
   constexpr int LPR = R / 8;           // lanes sharing one row of B
   constexpr int RPI = WAVE / LPR;      // rows per load instruction
   constexpr int NI = 8;                // load instructions (1 KiB each) per wave
@@ -65,7 +66,7 @@ __global__ __launch_bounds__(64) void lora_expand_kernel(YT* __restrict__ y, con
   int parity = 0;
 
   for (int t0 = 0; t0 < T; t0 += WAVE) {
-    const int id = (t0 + lane < T) ? ids[t0 + lane] : -1;
+    const int id = lora_token_id(ids, bucket_of, bucket, t0 + lane, T);
     unsigned long long mask = __ballot(id == a);
     if (mask && !loaded) {
       loaded = true;
@@ -165,7 +166,8 @@ template <int R, typename YT>
 __global__ __launch_bounds__(GMM_THREADS) void gather_mm_decode_kernel(GmmSet one, const GmmSet* __restrict__ sets,
                                                                         const int32_t* __restrict__ ids, float scaling,
                                                                         int T, int K, int N, int n_ad, int ldy,
-                                                                        int frag_tt, int P, int ci_n, int kc) {
+                                                                        int frag_tt, int P, int ci_n, int kc,
+                                                                        const int32_t* __restrict__ bucket_of, int bucket) {
   constexpr int G = R < 16 ? R : 16;         // rows of A reduced together
   constexpr int NG = R / 8;
   extern __shared__ float lds[];             // part [kc][T][R], then v [T][R]
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(GMM_THREADS) void gather_mm_decode_kernel(GmmSet on
   const int p = (wg >> 3) % P;
   if (a >= n_ad) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int id = lane < T ? ids[lane] : -1;            // T <= 64: one table row per lane
+  const int id = lora_token_id(ids, bucket_of, bucket, lane, T);   // T <= 64: one table row per lane
   const unsigned long long mine = __ballot(id == a);
   if (!mine) return;                                    // workgroup-uniform
   const GmmSet s = sets ? sets[blockIdx.y] : one;
@@ -301,10 +303,10 @@ int check_lora_shape(int T, int K, int N, int r, int n_ad) {
 
 template <int R, typename YT>
 void launch_expand(YT* y, int ldy, const float* vpart, const f16* B, const int32_t* ids, float scaling, int T, int K, int N,
-                   int n_ad, hipStream_t s) {
+                   int n_ad, hipStream_t s, const int32_t* bucket_of, int bucket) {
   constexpr int CH = 8 * (WAVE / (R / 8));
   hipLaunchKernelGGL((lora_expand_kernel<R, YT>), dim3(n_ad, ceil_div(N, CH)), dim3(64), 0, s, y, vpart, B, ids, scaling,
-                     T, N, ldy, lora_k_split(K).kc);
+                     T, N, ldy, lora_k_split(K).kc, bucket_of, bucket);
 }
 
 }  // namespace
@@ -314,8 +316,14 @@ extern "C" size_t mlora_gather_mm_workspace_bytes(int T, int K, int r) {
   return (size_t)lora_k_split(K).kc * (size_t)T * (size_t)r * sizeof(float);
 }
 
-extern "C" int mlora_lora_shrink(void* v_part, const void* x, int x_layout, const void* A, const int32_t* tok_adapter,
-                                 int T, int K, int r, int n_ad, void* stream) {
+// A rank bucket restricts a launch to the tokens whose bucket_of[t] equals `bucket` (bucket_of == nullptr: all tokens).
+struct BucketFilter {
+  const int32_t* bucket_of;
+  int bucket;
+};
+
+static int shrink_impl(void* v_part, const void* x, int x_layout, const void* A, const int32_t* tok_adapter,
+                       int T, int K, int r, int n_ad, BucketFilter bf, void* stream) {
   if (int e = check_lora_shape(T, K, 8, r, n_ad)) return e;
   MLORA_CHECK(x_layout == MLORA_ROWMAJOR || (x_layout == MLORA_FRAG && T <= 64 && K % 32 == 0), MLORA_ERR_UNSUPPORTED,
               "lora_shrink: fragment-ordered x needs T <= 64 and K %% 32 == 0 (layout=%d T=%d K=%d)", x_layout, T, K);
@@ -331,13 +339,19 @@ extern "C" int mlora_lora_shrink(void* v_part, const void* x, int x_layout, cons
   b.T = T; b.K = K; b.r = r; b.n_ad = n_ad; b.ci = ks.ci; b.kc = ks.kc;
   b.frag_tt = x_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   b.speculate = n_ad <= 2 * T;
+  b.bucket_of = bf.bucket_of;
+  b.bucket = bf.bucket;
   hipLaunchKernelGGL(lora_shrink_kernel, dim3(lora_shrink_units(b)), dim3(64), 0, (hipStream_t)stream, b);
   return mlora_launch_status("lora_shrink");
 }
 
-extern "C" int mlora_lora_expand(void* y, int y_dtype, int ldy, const void* v_part, const void* B,
-                                 const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
-                                 void* stream) {
+extern "C" int mlora_lora_shrink(void* v_part, const void* x, int x_layout, const void* A, const int32_t* tok_adapter,
+                                 int T, int K, int r, int n_ad, void* stream) {
+  return shrink_impl(v_part, x, x_layout, A, tok_adapter, T, K, r, n_ad, BucketFilter{nullptr, 0}, stream);
+}
+
+static int expand_impl(void* y, int y_dtype, int ldy, const void* v_part, const void* B, const int32_t* tok_adapter,
+                       float scaling, int T, int K, int N, int r, int n_ad, BucketFilter bf, void* stream) {
   if (int e = check_lora_shape(T, K, N, r, n_ad)) return e;
   MLORA_CHECK(ldy >= N && ldy % 8 == 0, MLORA_ERR_INVALID, "lora_expand: need ldy >= N and ldy %% 8 == 0 (ldy=%d N=%d)", ldy, N);
   MLORA_CHECK(y && v_part && B && tok_adapter, MLORA_ERR_INVALID, "lora_expand: null pointer");
@@ -347,8 +361,8 @@ extern "C" int mlora_lora_expand(void* y, int y_dtype, int ldy, const void* v_pa
   const float* vp = (const float*)v_part;
   const f16* Bp = (const f16*)B;
 #define MLORA_EXPAND(R)                                                                                   \
-  if (y_dtype == MLORA_F16) launch_expand<R, f16>((f16*)y, ldy, vp, Bp, tok_adapter, scaling, T, K, N, n_ad, s); \
-  else launch_expand<R, float>((float*)y, ldy, vp, Bp, tok_adapter, scaling, T, K, N, n_ad, s)
+  if (y_dtype == MLORA_F16) launch_expand<R, f16>((f16*)y, ldy, vp, Bp, tok_adapter, scaling, T, K, N, n_ad, s, bf.bucket_of, bf.bucket); \
+  else launch_expand<R, float>((float*)y, ldy, vp, Bp, tok_adapter, scaling, T, K, N, n_ad, s, bf.bucket_of, bf.bucket)
   switch (r) {
     case 8: MLORA_EXPAND(8); break;
     case 16: MLORA_EXPAND(16); break;
@@ -359,6 +373,12 @@ extern "C" int mlora_lora_expand(void* y, int y_dtype, int ldy, const void* v_pa
   return mlora_launch_status("lora_expand");
 }
 
+extern "C" int mlora_lora_expand(void* y, int y_dtype, int ldy, const void* v_part, const void* B,
+                                 const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
+                                 void* stream) {
+  return expand_impl(y, y_dtype, ldy, v_part, B, tok_adapter, scaling, T, K, N, r, n_ad, BucketFilter{nullptr, 0}, stream);
+}
+
 // The one-launch kernel applies when the table fits one wave (T <= 64) and the partials fit LDS.
 static bool gmm_one_launch_fits(int T, int K, int r) {
   return T > 0 && T <= 64 && (size_t)(lora_k_split(K).kc + 1) * T * r * sizeof(float) <= 48 * 1024;
@@ -366,16 +386,18 @@ static bool gmm_one_launch_fits(int T, int K, int r) {
 
 template <int R>
 static void gmm_launch_r(const GmmSet& one, const GmmSet* sets, dim3 grid, size_t lds, int y_dtype, const int32_t* ids,
-                         float scaling, int T, int K, int N, int n_ad, int ldy, int frag_tt, int P, LoraKSplit ks, hipStream_t s) {
+                         float scaling, int T, int K, int N, int n_ad, int ldy, int frag_tt, int P, LoraKSplit ks, hipStream_t s,
+                         BucketFilter bf) {
   const dim3 block(GMM_THREADS);
   if (y_dtype == MLORA_F16)
-    hipLaunchKernelGGL((gather_mm_decode_kernel<R, f16>), grid, block, lds, s, one, sets, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks.ci, ks.kc);
+    hipLaunchKernelGGL((gather_mm_decode_kernel<R, f16>), grid, block, lds, s, one, sets, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks.ci, ks.kc, bf.bucket_of, bf.bucket);
   else
-    hipLaunchKernelGGL((gather_mm_decode_kernel<R, float>), grid, block, lds, s, one, sets, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks.ci, ks.kc);
+    hipLaunchKernelGGL((gather_mm_decode_kernel<R, float>), grid, block, lds, s, one, sets, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks.ci, ks.kc, bf.bucket_of, bf.bucket);
 }
 
 static int gmm_one_launch(const GmmSet& one, const GmmSet* sets, int n_sets, int y_dtype, int ldy, int x_layout,
-                          const int32_t* ids, float scaling, int T, int K, int N, int r, int n_ad, hipStream_t s) {
+                          const int32_t* ids, float scaling, int T, int K, int N, int r, int n_ad, hipStream_t s,
+                          BucketFilter bf = BucketFilter{nullptr, 0}) {
   const LoraKSplit ks = lora_k_split(K);
   const int groups = ceil_div(n_ad, 8);                 // adapters are dealt to the 8 XCDs in groups of 8
   // Output-row slices per adapter: enough workgroups to cover the chip when the launch holds one problem, one slice
@@ -388,10 +410,10 @@ static int gmm_one_launch(const GmmSet& one, const GmmSet* sets, int n_sets, int
   const int frag_tt = x_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   const dim3 grid(groups * 8 * P, n_sets);
   switch (r) {
-    case 8: gmm_launch_r<8>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s); break;
-    case 16: gmm_launch_r<16>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s); break;
-    case 32: gmm_launch_r<32>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s); break;
-    default: gmm_launch_r<64>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s); break;
+    case 8: gmm_launch_r<8>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s, bf); break;
+    case 16: gmm_launch_r<16>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s, bf); break;
+    case 32: gmm_launch_r<32>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s, bf); break;
+    default: gmm_launch_r<64>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s, bf); break;
   }
   return mlora_launch_status("gather_mm");
 }
@@ -412,9 +434,9 @@ extern "C" int mlora_gather_mm_batch(const void* const* sets, int n_sets, int y_
                         (hipStream_t)stream);
 }
 
-extern "C" int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, int x_layout, const void* A, const void* B,
-                               const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
-                               void* workspace, size_t workspace_bytes, void* stream) {
+static int gather_mm_impl(void* y, int y_dtype, int ldy, const void* x, int x_layout, const void* A, const void* B,
+                          const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
+                          void* workspace, size_t workspace_bytes, BucketFilter bf, void* stream) {
   if (int e = check_lora_shape(T, K, N, r, n_ad)) return e;
   // the workspace is part of the contract whichever kernel runs (the one-launch kernel keeps its partials in LDS)
   MLORA_CHECK(workspace && workspace_bytes >= mlora_gather_mm_workspace_bytes(T, K, r) || T == 0, MLORA_ERR_WORKSPACE,
@@ -427,10 +449,41 @@ extern "C" int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, int
     MLORA_CHECK(x_layout == MLORA_ROWMAJOR || (x_layout == MLORA_FRAG && K % 32 == 0), MLORA_ERR_UNSUPPORTED,
                 "gather_mm: fragment-ordered x needs T <= 64 and K %% 32 == 0 (layout=%d T=%d K=%d)", x_layout, T, K);
     const GmmSet one = {y, (const f16*)x, (const f16*)A, (const f16*)B};
-    return gmm_one_launch(one, nullptr, 1, y_dtype, ldy, x_layout, tok_adapter, scaling, T, K, N, r, n_ad, (hipStream_t)stream);
+    return gmm_one_launch(one, nullptr, 1, y_dtype, ldy, x_layout, tok_adapter, scaling, T, K, N, r, n_ad, (hipStream_t)stream, bf);
   }
-  if (int e = mlora_lora_shrink(workspace, x, x_layout, A, tok_adapter, T, K, r, n_ad, stream)) return e;
-  return mlora_lora_expand(y, y_dtype, ldy, workspace, B, tok_adapter, scaling, T, K, N, r, n_ad, stream);
+  if (int e = shrink_impl(workspace, x, x_layout, A, tok_adapter, T, K, r, n_ad, bf, stream)) return e;
+  return expand_impl(y, y_dtype, ldy, workspace, B, tok_adapter, scaling, T, K, N, r, n_ad, bf, stream);
+}
+
+extern "C" int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, int x_layout, const void* A, const void* B,
+                               const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+  return gather_mm_impl(y, y_dtype, ldy, x, x_layout, A, B, tok_adapter, scaling, T, K, N, r, n_ad, workspace, workspace_bytes,
+                        BucketFilter{nullptr, 0}, stream);
+}
+
+extern "C" int mlora_gather_mm_multi(void* y, int y_dtype, int ldy, const void* x, int x_layout,
+                                     const mlora_lora_bucket* buckets, int n_buckets, const int32_t* tok_bucket,
+                                     const int32_t* tok_adapter, int T, int K, int N, void* workspace,
+                                     size_t workspace_bytes, void* stream) {
+  MLORA_CHECK(buckets && n_buckets > 0 && n_buckets <= 64, MLORA_ERR_INVALID, "gather_mm_multi: bad bucket list (n_buckets=%d)", n_buckets);
+  MLORA_CHECK(tok_bucket && tok_adapter, MLORA_ERR_INVALID, "gather_mm_multi: null id array");
+  // validate every bucket before the first launch, so that an error leaves y untouched
+  for (int b = 0; b < n_buckets; ++b) {
+    if (!buckets[b].A && !buckets[b].B) continue;       // this bucket's adapters do not target the projection
+    if (int e = check_lora_shape(T, K, N, buckets[b].r, buckets[b].n_ad)) return e;
+    MLORA_CHECK(buckets[b].A && buckets[b].B, MLORA_ERR_INVALID, "gather_mm_multi: bucket %d has one null table", b);
+    MLORA_CHECK(T == 0 || (workspace && workspace_bytes >= mlora_gather_mm_workspace_bytes(T, K, buckets[b].r)), MLORA_ERR_WORKSPACE,
+                "gather_mm_multi: workspace of %zu bytes given, %zu needed for bucket %d (rank %d)", workspace_bytes,
+                mlora_gather_mm_workspace_bytes(T, K, buckets[b].r), b, buckets[b].r);
+  }
+  for (int b = 0; b < n_buckets; ++b) {
+    if (!buckets[b].A) continue;
+    if (int e = gather_mm_impl(y, y_dtype, ldy, x, x_layout, buckets[b].A, buckets[b].B, tok_adapter, buckets[b].scaling, T, K, N,
+                               buckets[b].r, buckets[b].n_ad, workspace, workspace_bytes, BucketFilter{tok_bucket, b}, stream))
+      return e;
+  }
+  return MLORA_OK;
 }
 
 extern "C" int mlora_write_tensor_part(void* Z, const void* X, const void* Y, const int32_t* ids, int B, int A, int PH,

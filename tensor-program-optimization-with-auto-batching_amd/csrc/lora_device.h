@@ -25,7 +25,17 @@ struct LoraShrinkBatch {
   const int32_t* ids;
   int T, K, r, n_ad, ci, kc, frag_tt;
   int speculate;                 // request A before the adapter table is read (adapters expected to be in use)
+  const int32_t* bucket_of;      // optional [T]: rank bucket of each token; tokens of other buckets count as unadapted
+  int bucket;
 };
+
+// Adapter id of token t as this launch sees it: -1 outside the table and for tokens of another rank bucket.
+__device__ __forceinline__ int lora_token_id(const int32_t* __restrict__ ids, const int32_t* __restrict__ bucket_of,
+                                             int bucket, int t, int T) {
+  if (t >= T) return -1;
+  if (bucket_of != nullptr && bucket_of[t] != bucket) return -1;
+  return ids[t];
+}
 
 static inline int lora_shrink_units(const LoraShrinkBatch& b) { return b.n_proj * b.n_ad * b.kc; }
 
@@ -75,14 +85,14 @@ __device__ __forceinline__ void lora_shrink_unit(const LoraShrinkBatch& b, int u
   const bool resident = b.r <= G && b.ci == 1;   // the wave's whole slice of A fits the register file
   const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
   f16x8 areg[G];
-  int id = lane < b.T ? b.ids[lane] : -1;
+  int id = lora_token_id(b.ids, b.bucket_of, b.bucket, lane, b.T);
   if (resident && b.speculate) {
 #pragma unroll
     for (int j = 0; j < G; ++j) areg[j] = (j < b.r && kbase < b.K) ? ld8(A + (size_t)j * b.K + kbase) : zero8;
   }
   bool loaded = resident && b.speculate;
   for (int t0 = 0; t0 < b.T; t0 += WAVE) {
-    if (t0 > 0) id = (t0 + lane < b.T) ? b.ids[t0 + lane] : -1;
+    if (t0 > 0) id = lora_token_id(b.ids, b.bucket_of, b.bucket, t0 + lane, b.T);
     unsigned long long mask = __ballot(id == a);
     if (mask && resident && !loaded) {
       loaded = true;

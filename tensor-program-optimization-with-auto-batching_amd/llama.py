@@ -179,17 +179,47 @@ class LlamaForCausalLM:
         return self._ws
 
     def _lora(self, y, x, l, proj, tok_adapter):
-        """y += delta for every adapter type that targets (l, proj); tok_adapter: {tid: ids [T] int32}."""
+        """y += delta for every adapter type that targets (l, proj); tok_adapter: {tid: ids [T] int32}, or the merged
+        form {"multi": (tok_bucket, tok_adapter)} in which a token names its adapter type and weight row."""
+        if "multi" in tok_adapter:
+            tb, ta = tok_adapter["multi"]
+            buckets = []
+            for lt in self.lora_types:
+                tab = lt.tables.get((l, proj))
+                buckets.append(None if tab is None else (tab[0], tab[1], lt.scaling))
+            if any(b is not None for b in buckets):
+                rmax = max(lt.r for lt in self.lora_types)
+                ops.gather_mm_multi(y, x, buckets, tb, ta, self._workspace(x.shape[0], x.shape[1], rmax))
+            return
         for tid, ids in tok_adapter.items():
             lt = self.lora_types[tid]
             tab = lt.tables.get((l, proj))
             if tab is not None:
                 ops.gather_mm(y, x, tab[0], tab[1], ids, lt.scaling, self._workspace(x.shape[0], x.shape[1], lt.r))
 
+    @staticmethod
+    def _merge_types(tok_adapter):
+        """{tid: ids} with at most one adapter per token -> per-token (type, weight row) arrays for the multi-rank call."""
+        tids = sorted(tok_adapter)
+        first = tok_adapter[tids[0]]
+        tb = torch.full_like(first, -1)
+        ta = torch.full_like(first, -1)
+        taken = torch.zeros_like(first, dtype=torch.bool)
+        for tid in tids:
+            has = tok_adapter[tid] >= 0
+            if bool((has & taken).any()):
+                raise ValueError("a token is bound to adapters of two types")
+            taken |= has
+            tb = torch.where(has, torch.full_like(tb, tid), tb)
+            ta = torch.where(has, tok_adapter[tid], ta)
+        return {"multi": (tb, ta)}
+
     def forward(self, hidden: torch.Tensor, kv: PagedKVCache, tok_adapter=None, logits_rows=None) -> torch.Tensor:
         """hidden [T, H] fp32 (updated in place), tokens in kv.begin_forward order -> logits fp32."""
         s = self.shape
         tok_adapter = tok_adapter or {}
+        if len(tok_adapter) > 1:            # several adapter types (ranks) in the batch: one multi-rank call per projection
+            tok_adapter = self._merge_types(tok_adapter)
         T = hidden.shape[0]
         H, I = s.hidden_size, s.intermediate_size
         q_sz, kv_sz = s.q_size, s.kv_size

@@ -77,3 +77,34 @@ class GatherMMLinear:
         return y.view(*shp[:-1], self.out_features)
 
     __call__ = forward
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Multi-rank table transforms of the reference's case study (`tvm/lora_only/case_study/multiple_ranks.py`): the
+# same delta can be computed from tables padded to the largest rank (`:165-178`, PaddedLora `:66-95`) or split into
+# chunks of the smallest rank whose partial deltas are summed (`:180-194`, SplittedLora `:98-151`).  The kernels do
+# not need either (mlora_gather_mm_multi reads every table at its own rank); these are kept for the equivalence
+# checks and for callers that hold padded or splitted tables already.
+# ---------------------------------------------------------------------------------------------------------------
+def pad_rank(A: torch.Tensor, B: torch.Tensor, r_to: int):
+    """A [n, r, K], B [n, N, r] -> zero-padded to rank r_to.  The padded rows contribute exact zeros."""
+    n, r, K = A.shape
+    if r_to < r:
+        raise ValueError(f"cannot pad rank {r} down to {r_to}")
+    Ap = torch.zeros((n, r_to, K), dtype=A.dtype, device=A.device)
+    Bp = torch.zeros((n, B.shape[1], r_to), dtype=B.dtype, device=B.device)
+    Ap[:, :r] = A
+    Bp[:, :, :r] = B
+    return Ap, Bp
+
+
+def split_rank(A: torch.Tensor, B: torch.Tensor, r_chunk: int):
+    """A [n, r, K], B [n, N, r] -> [n * r/r_chunk, r_chunk, K], [n * r/r_chunk, N, r_chunk]; adapter i becomes rows
+    i*m .. i*m+m-1 (m = r / r_chunk), and its delta is the sum of the m chunk deltas."""
+    n, r, K = A.shape
+    if r % r_chunk:
+        raise ValueError(f"rank {r} is not a multiple of {r_chunk}")
+    m = r // r_chunk
+    As = A.reshape(n, m, r_chunk, K).reshape(n * m, r_chunk, K).contiguous()
+    Bs = B.reshape(n, B.shape[1], m, r_chunk).permute(0, 2, 1, 3).reshape(n * m, B.shape[1], r_chunk).contiguous()
+    return As, Bs

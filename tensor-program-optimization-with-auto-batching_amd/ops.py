@@ -101,6 +101,39 @@ def gather_mm(y, x, A, B, tok_adapter, scaling: float, workspace=None):
     return y
 
 
+def gather_mm_multi(y, x, buckets, tok_bucket, tok_adapter, workspace=None):
+    """Adapters of several ranks in one batch: buckets = [(A [n_ad,r,K], B [n_ad,N,r], scaling) | None, ...]; token t uses
+    adapter tok_adapter[t] of bucket tok_bucket[t] (-1 = none).  y is updated in place."""
+    import ctypes
+    from ._lib import LoraBucket
+    xptr, xlay, T, K = _x_arg(x)
+    N = y.shape[1]
+    if y.shape[0] != T or tok_bucket.shape != (T,) or tok_adapter.shape != (T,):
+        raise ValueError("gather_mm_multi: inconsistent shapes")
+    arr = (LoraBucket * len(buckets))()
+    rmax = 8
+    for i, bk in enumerate(buckets):
+        if bk is None:                      # the bucket's adapters do not target this projection
+            arr[i].A = arr[i].B = None
+            continue
+        A, B, scaling = bk
+        n_ad, r, K2 = A.shape
+        if K2 != K or B.shape != (n_ad, N, r):
+            raise ValueError(f"gather_mm_multi: bucket {i} has A{tuple(A.shape)} B{tuple(B.shape)} for K={K} N={N}")
+        arr[i].A, arr[i].B = _dev(A, torch.float16, "A"), _dev(B, torch.float16, "B")
+        arr[i].r, arr[i].n_ad, arr[i].scaling = r, n_ad, float(scaling)
+        rmax = max(rmax, r)
+    if workspace is None:
+        workspace = gather_mm_workspace(T, K, rmax, x.device)
+    if not y.is_cuda or y.stride(1) != 1:
+        raise ValueError("gather_mm_multi: y must be a GPU tensor with unit inner stride")
+    ldy = y.stride(0) if T > 1 else max(N, y.stride(0))
+    check(lib().mlora_gather_mm_multi(y.data_ptr(), _dt(y), ldy, xptr, xlay, ctypes.cast(arr, ctypes.c_void_p), len(buckets),
+                                      _dev(tok_bucket, torch.int32, "tok_bucket"), _dev(tok_adapter, torch.int32, "tok_adapter"),
+                                      T, K, N, _dev(workspace, torch.float32, "workspace"), workspace.numel() * 4, _stream()))
+    return y
+
+
 class GatherMMBatch:
     """Several gather-matmul problems of one shape and one token->adapter table, issued as one launch.
     sets: list of (y, x, A, B) as for gather_mm (x row-major); the tensors are kept alive by this object."""

@@ -10,6 +10,7 @@ import torch
 
 import oracle
 from oracle import max_rel_err
+from conftest import load_pkg
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-3
@@ -393,3 +394,53 @@ def test_gather_mm_batch_equals_separate_calls(ops, synth):
     ops.GatherMMBatch(sets, ids, 0.25).run()
     for (y, _, _, _), w in zip(sets, want):
         assert torch.equal(y, w)
+
+
+@pytest.mark.parametrize("T,K,N", [(48, 1024, 512), (150, 2048, 1024)])
+def test_gather_mm_multi_rank_strategies_agree(ops, synth, T, K, N):
+    """Three rank buckets (8, 16, 64) in one call: equal, bit for bit, to one masked call per bucket (the reference's
+    sequential strategy, `multiple_ranks.py:21-63`) and to tables zero-padded to rank 64 (`:66-95`); equal within
+    tolerance to rank-8 chunks summed (`:98-151`) and to the oracle.  Covers both the one-launch (T <= 64) and the
+    two-kernel path."""
+    lora = load_pkg("lora")
+    ranks, n_ads, scal = (8, 16, 64), (3, 5, 2), (0.5, 0.25, 1.0)
+    x = synth.normal(21, "mr.x", (T, K), 1.0, torch.float16, DEV)
+    y0 = synth.normal(21, "mr.y", (T, N), 1.0, torch.float16, DEV)
+    tabs = [(synth.normal(21, f"mr.A{i}", (n, r, K), 0.05, torch.float16, DEV),
+             synth.normal(21, f"mr.B{i}", (n, N, r), 0.05, torch.float16, DEV)) for i, (r, n) in enumerate(zip(ranks, n_ads))]
+    tb = synth.randint(21, "mr.bucket", (T,), 4, DEV) - 1            # -1 = no adapter
+    ta = torch.stack([synth.randint(21, f"mr.ad{i}", (T,), n, DEV) for i, n in enumerate(n_ads)])
+    tok_adapter = torch.where(tb >= 0, ta.gather(0, tb.clamp(min=0).long()[None])[0], torch.full_like(tb, -1)).to(torch.int32)
+    tb = tb.to(torch.int32)
+    multi = ops.gather_mm_multi(y0.clone(), x, [(A, B, s) for (A, B), s in zip(tabs, scal)], tb, tok_adapter)
+    # sequential: one call per bucket, other tokens masked
+    seq = y0.clone()
+    for i, ((A, B), s) in enumerate(zip(tabs, scal)):
+        ops.gather_mm(seq, x, A, B, torch.where(tb == i, tok_adapter, torch.full_like(tb, -1)), s)
+    assert torch.equal(multi, seq)
+    # padded: one table of rank 64 holding all adapters; scaling differs per bucket, so it is folded into B here
+    offs = np.concatenate([[0], np.cumsum(n_ads)])
+    padded = [lora.pad_rank(A, (B.float() * s).half(), 64) for (A, B), s in zip(tabs, scal)]
+    Ap, Bp = torch.cat([p[0] for p in padded]), torch.cat([p[1] for p in padded])
+    pid = torch.where(tb >= 0, tok_adapter + torch.tensor(offs[:-1], device=DEV, dtype=torch.int32)[tb.clamp(min=0).long()],
+                      torch.full_like(tb, -1))
+    pad = ops.gather_mm(y0.clone(), x, Ap, Bp, pid, 1.0)
+    ref = _np(y0).astype(np.float64)
+    xs = _np(x).astype(np.float64)
+    for t in range(T):
+        b = int(tb[t])
+        if b >= 0:
+            A, B = tabs[b]
+            a = int(tok_adapter[t])
+            ref[t] += scal[b] * (_np(B[a]).astype(np.float64) @ (_np(A[a]).astype(np.float64) @ xs[t]))
+    assert max_rel_err(_np(multi), ref) <= TOL
+    assert max_rel_err(_np(pad), ref) <= TOL            # scaling folded into fp16 B: one more rounding than `multi`
+    # splitted: rank-64 bucket as 8 chunks of rank 8, chunk deltas summed (fp32 y keeps the chunk sums unrounded)
+    A64, B64 = tabs[2]
+    As, Bs = lora.split_rank(A64, B64, 8)
+    only64 = torch.where(tb == 2, tok_adapter, torch.full_like(tb, -1))
+    full = ops.gather_mm(torch.zeros((T, N), dtype=torch.float32, device=DEV), x, A64, B64, only64, 1.0)
+    chunks = torch.zeros((T, N), dtype=torch.float32, device=DEV)
+    for c in range(8):
+        ops.gather_mm(chunks, x, As, Bs, torch.where(only64 >= 0, only64 * 8 + c, only64), 1.0)
+    assert max_rel_err(_np(chunks), _np(full).astype(np.float64), floor=1e-2) <= 1e-4
