@@ -278,6 +278,149 @@ __global__ __launch_bounds__(GMM_THREADS) void gather_mm_decode_kernel(GmmSet on
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Prefill-sized gather-matmul (T > 64) on the matrix cores.  Tokens arrive grouped in adapter segments, so a tile
+// of 16 consecutive tokens holds one adapter, two at a segment boundary; a tile is processed once per distinct
+// adapter in it and rows of other adapters are masked at the store.
+//   shrink: workgroup per token tile, 4 waves split K;  V^T[r, 16 tok] = A[a] . X^T  with A[a] as the A operand
+//           (rows = rank index) and the token tile as the B operand, so a lane ends up with 4 consecutive rank
+//           entries of one token (one 16-byte store of v[t, 4g..4g+3]); fixed-order LDS sum of the 4 waves.
+//   expand: wave per (token tile, 64 output columns);  D[n, tok] = B[a] . V^T with v split into fp16 hi + lo halves
+//           (two MFMAs, ~22 mantissa bits of v); a lane read-modify-writes 4 consecutive y elements of one token.
+// v is [T, r] fp32 (one full sum per token, no K-slices).
+// ---------------------------------------------------------------------------------------------
+constexpr int SEG_WAVES = 4;
+
+// adapter of the first unprocessed token of the tile and the mask of tile rows bound to it; lanes 0..15 hold ids
+__device__ __forceinline__ bool next_tile_adapter(int id, unsigned& todo, int& a, unsigned& rows) {
+  if (!todo) return false;
+  const int first = __builtin_ctz(todo);
+  a = __shfl(id, first, WAVE);
+  rows = (unsigned)__ballot(id == a) & 0xffffu & todo;
+  todo &= ~rows;
+  return true;
+}
+
+template <int R>
+__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(float* __restrict__ v, const f16* __restrict__ x,
+                                                                            const f16* __restrict__ A,
+                                                                            const int32_t* __restrict__ ids, int T, int K,
+                                                                            int n_ad, const int32_t* __restrict__ bucket_of,
+                                                                            int bucket) {
+  constexpr int NT = (R + 15) / 16;     // 16-row tiles of A[a]; rank 8 uses half a tile
+  __shared__ f32x4 red[SEG_WAVES][NT][WAVE];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t0 = blockIdx.x * 16;
+  const int col = lane & 15, g = lane >> 4;
+  const int tl = min(t0 + col, T - 1);                          // token whose x row this lane supplies
+  const int raw = lora_token_id(ids, bucket_of, bucket, t0 + col, T);
+  const int id = (raw >= 0 && raw < n_ad) ? raw : -1;
+  unsigned todo = (unsigned)__ballot(id >= 0) & 0xffffu;
+  const f16* __restrict__ xr = x + (size_t)tl * K + g * 8;
+  const int KB = K / 32;
+  int a;
+  unsigned rows;
+  while (next_tile_adapter(id, todo, a, rows)) {
+    const f16* __restrict__ Aa = A + (size_t)a * R * K + g * 8;
+    f32x4 acc[NT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int kb = wave; kb < KB; kb += SEG_WAVES) {
+      const f16x8 xf = ld8(xr + kb * 32);
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        const int row = i * 16 + col;
+        const f16x8 af = row < R ? ld8(Aa + (size_t)row * K + kb * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, xf, acc[i], 0, 0, 0);   // rows: rank index, cols: tokens
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NT; ++i) red[wave][i][lane] = acc[i];
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        f32x4 s = red[0][i][lane];
+#pragma unroll
+        for (int w = 1; w < SEG_WAVES; ++w) s += red[w][i][lane];
+        const int j = i * 16 + 4 * g;                              // first of this lane's 4 rank entries
+        if (((rows >> col) & 1u) && j < R) *reinterpret_cast<f32x4*>(v + (size_t)(t0 + col) * R + j) = s;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <int R, typename YT>
+__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* __restrict__ y, const float* __restrict__ v,
+                                                                            const f16* __restrict__ B,
+                                                                            const int32_t* __restrict__ ids, float scaling,
+                                                                            int T, int N, int ldy, int n_ad,
+                                                                            const int32_t* __restrict__ bucket_of, int bucket) {
+  constexpr int KS = (R + 31) / 32;     // k-steps of 32 rank entries (ranks 8 and 16: one partly filled step)
+  constexpr int CT = 4;                 // 16-column tiles per wave
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t0 = blockIdx.x * 16;
+  const int n0 = (blockIdx.y * SEG_WAVES + wave) * 16 * CT;
+  if (n0 >= N) return;
+  const int col = lane & 15, g = lane >> 4;
+  const int tl = min(t0 + col, T - 1);
+  const int raw = lora_token_id(ids, bucket_of, bucket, t0 + col, T);
+  const int id = (raw >= 0 && raw < n_ad) ? raw : -1;
+  unsigned todo = (unsigned)__ballot(id >= 0) & 0xffffu;
+  if (!todo) return;
+  // the token tile of v as the B operand, hi and lo halves: lane holds v[token col][ks*32 + 8g .. +7]
+  f16x8 vh[KS], vl[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int j = ks * 32 + g * 8;
+    float f[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = 0.f;
+    if (j < R) {
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(v + (size_t)tl * R + j);
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(v + (size_t)tl * R + j + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        f[e] = lo[e] * scaling;
+        f[4 + e] = hi[e] * scaling;
+      }
+    }
+    if (id < 0) {                        // rows of unadapted tokens may hold anything: keep NaNs out of the product
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const f16 h = (f16)f[e];
+      vh[ks][e] = h;
+      vl[ks][e] = (f16)(f[e] - (float)h);
+    }
+  }
+  int a;
+  unsigned rows;
+  while (next_tile_adapter(id, todo, a, rows)) {
+    const f16* __restrict__ Ba = B + (size_t)a * N * R + g * 8;
+#pragma unroll
+    for (int c = 0; c < CT; ++c) {
+      const int nb = n0 + c * 16;
+      if (nb >= N) break;                                          // wave-uniform
+      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int j = ks * 32 + g * 8;
+        const f16x8 bf = j < R ? ld8(Ba + (size_t)(nb + col) * R + ks * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf, vh[ks], acc, 0, 0, 0);      // rows: output column, cols: tokens
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf, vl[ks], acc, 0, 0, 0);
+      }
+      if ((rows >> col) & 1u) {
+        float d[4] = {acc[0], acc[1], acc[2], acc[3]};
+        rmw_add<YT, 4>(y + (size_t)(t0 + col) * ldy + nb + 4 * g, d);
+      }
+    }
+  }
+}
+
 __global__ void write_tensor_part_kernel(f16* __restrict__ Z, const f16* __restrict__ X, const f16* __restrict__ Y,
                                          const int32_t* __restrict__ ids, int B, int A, int PH) {
   // Phase split by blockIdx.y: 0 copies X -> Z (skipped when Z aliases X), 1 scatters Y rows.
@@ -434,6 +577,33 @@ extern "C" int mlora_gather_mm_batch(const void* const* sets, int n_sets, int y_
                         (hipStream_t)stream);
 }
 
+template <int R>
+static void gmm_segments_r(void* y, int y_dtype, int ldy, const f16* x, const f16* A, const f16* B, const int32_t* ids,
+                           float scaling, int T, int K, int N, int n_ad, float* v, BucketFilter bf, hipStream_t s) {
+  const int tiles = ceil_div(T, 16);
+  hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles), dim3(SEG_WAVES * WAVE), 0, s, v, x, A, ids, T, K, n_ad,
+                     bf.bucket_of, bf.bucket);
+  const dim3 grid(tiles, ceil_div(N, SEG_WAVES * 64));
+  if (y_dtype == MLORA_F16)
+    hipLaunchKernelGGL((lora_expand_mfma_kernel<R, f16>), grid, dim3(SEG_WAVES * WAVE), 0, s, (f16*)y, v, B, ids, scaling, T, N,
+                       ldy, n_ad, bf.bucket_of, bf.bucket);
+  else
+    hipLaunchKernelGGL((lora_expand_mfma_kernel<R, float>), grid, dim3(SEG_WAVES * WAVE), 0, s, (float*)y, v, B, ids, scaling, T,
+                       N, ldy, n_ad, bf.bucket_of, bf.bucket);
+}
+
+// shrink + expand on the matrix cores; v = workspace viewed as [T, r] fp32
+static int gmm_segments(void* y, int y_dtype, int ldy, const f16* x, const f16* A, const f16* B, const int32_t* ids,
+                        float scaling, int T, int K, int N, int r, int n_ad, float* v, BucketFilter bf, hipStream_t s) {
+  switch (r) {
+    case 8: gmm_segments_r<8>(y, y_dtype, ldy, x, A, B, ids, scaling, T, K, N, n_ad, v, bf, s); break;
+    case 16: gmm_segments_r<16>(y, y_dtype, ldy, x, A, B, ids, scaling, T, K, N, n_ad, v, bf, s); break;
+    case 32: gmm_segments_r<32>(y, y_dtype, ldy, x, A, B, ids, scaling, T, K, N, n_ad, v, bf, s); break;
+    default: gmm_segments_r<64>(y, y_dtype, ldy, x, A, B, ids, scaling, T, K, N, n_ad, v, bf, s); break;
+  }
+  return mlora_launch_status("gather_mm");
+}
+
 static int gather_mm_impl(void* y, int y_dtype, int ldy, const void* x, int x_layout, const void* A, const void* B,
                           const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
                           void* workspace, size_t workspace_bytes, BucketFilter bf, void* stream) {
@@ -450,6 +620,13 @@ static int gather_mm_impl(void* y, int y_dtype, int ldy, const void* x, int x_la
                 "gather_mm: fragment-ordered x needs T <= 64 and K %% 32 == 0 (layout=%d T=%d K=%d)", x_layout, T, K);
     const GmmSet one = {y, (const f16*)x, (const f16*)A, (const f16*)B};
     return gmm_one_launch(one, nullptr, 1, y_dtype, ldy, x_layout, tok_adapter, scaling, T, K, N, r, n_ad, (hipStream_t)stream, bf);
+  }
+  if (x_layout == MLORA_ROWMAJOR && T > 64 && K % 32 == 0 && N % 16 == 0 && ldy % 4 == 0 && (uintptr_t)y % 16 == 0) {
+    MLORA_CHECK(y && x && A && B && tok_adapter, MLORA_ERR_INVALID, "gather_mm: null pointer");
+    MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "gather_mm: bad y_dtype %d", y_dtype);
+    MLORA_CHECK(ldy >= N, MLORA_ERR_INVALID, "gather_mm: need ldy >= N (ldy=%d N=%d)", ldy, N);
+    return gmm_segments(y, y_dtype, ldy, (const f16*)x, (const f16*)A, (const f16*)B, tok_adapter, scaling, T, K, N, r, n_ad,
+                        (float*)workspace, bf, (hipStream_t)stream);
   }
   if (int e = shrink_impl(workspace, x, x_layout, A, tok_adapter, T, K, r, n_ad, bf, stream)) return e;
   return expand_impl(y, y_dtype, ldy, workspace, B, tok_adapter, scaling, T, K, N, r, n_ad, bf, stream);

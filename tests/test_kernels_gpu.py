@@ -444,3 +444,45 @@ def test_gather_mm_multi_rank_strategies_agree(ops, synth, T, K, N):
     for c in range(8):
         ops.gather_mm(chunks, x, As, Bs, torch.where(only64 >= 0, only64 * 8 + c, only64), 1.0)
     assert max_rel_err(_np(chunks), _np(full).astype(np.float64), floor=1e-2) <= 1e-4
+
+
+@pytest.mark.parametrize("T,K,N,r,n_ad,ydt", [
+    (512, 4096, 4096, 64, 8, torch.float16),      # prefill segments, rank 64
+    (200, 1024, 528, 16, 6, torch.float32),       # T not a multiple of 16, N a multiple of 16 only
+    (97, 2048, 256, 8, 3, torch.float16),
+    (160, 11008, 1024, 32, 4, torch.float16),     # down_proj-like K
+])
+@pytest.mark.parametrize("pattern", ["segments", "random"])
+def test_gather_mm_prefill_sizes_on_matrix_cores(ops, synth, T, K, N, r, n_ad, ydt, pattern):
+    """T > 64 takes the matrix-core shrink/expand pair: adapter segments (with unadapted gaps and boundaries inside
+    a 16-token tile) and fully random ids, against the oracle; unadapted rows stay bit-identical."""
+    c = synth.gather_mm_case(seed=11, T=T, K=K, N=N, r=r, n_ad=n_ad, device=DEV, tag=f"pf{T}.{K}.{N}.{r}")
+    if pattern == "segments":
+        cuts = np.sort(synth.randint(11, f"pf.cuts{T}", (n_ad + 1,), T).numpy())
+        ids = np.full(T, -1, dtype=np.int32)
+        order = synth.permutation(11, f"pf.order{T}", n_ad)
+        for i in range(n_ad):
+            ids[cuts[i]:cuts[i + 1]] = order[i]
+        ids[:cuts[0] // 2] = order[0]
+    else:
+        ids = synth.randint(11, f"pf.ids{T}", (T,), n_ad + 1).numpy().astype(np.int32) - 1
+    y0 = c["y"].to(ydt)
+    y = y0.clone()
+    ops.gather_mm(y, c["x"], c["A"], c["B"], torch.tensor(ids, device=DEV), 0.5)
+    ref = oracle.gather_mm_ref(_np(y0), _np(c["x"]), _np(c["A"]), _np(c["B"]), ids, 0.5)
+    assert max_rel_err(_np(y), ref) <= TOL
+    none = ids < 0
+    assert none.any() and torch.equal(y[torch.tensor(none, device=DEV)], y0[torch.tensor(none, device=DEV)])
+
+
+def test_gather_mm_prefill_column_slice(ops, synth):
+    """The matrix-core pair writes into a column slice of a fused projection output and leaves the rest alone."""
+    T, K, N, r, n_ad = 130, 1024, 256, 64, 4
+    c = synth.gather_mm_case(seed=12, T=T, K=K, N=N, r=r, n_ad=n_ad, device=DEV, tag="pfslice")
+    wide = synth.normal(12, "pf.wide", (T, 3 * N), 1.0, torch.float16, DEV)
+    before = _np(wide).copy()
+    ops.gather_mm(wide[:, N:2 * N], c["x"], c["A"], c["B"], c["ids"], 0.5)
+    after = _np(wide)
+    ref = oracle.gather_mm_ref(before[:, N:2 * N], _np(c["x"]), _np(c["A"]), _np(c["B"]), c["ids"].cpu().numpy(), 0.5)
+    assert max_rel_err(after[:, N:2 * N], ref) <= TOL
+    assert np.array_equal(after[:, :N], before[:, :N]) and np.array_equal(after[:, 2 * N:], before[:, 2 * N:])
