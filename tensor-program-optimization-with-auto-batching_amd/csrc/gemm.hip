@@ -99,6 +99,139 @@ __global__ __launch_bounds__(256) void gemm_kernel(void* __restrict__ yv, const 
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Large-T variant for fragment-ordered weights: a workgroup of 4 waves owns a 256-token x 256-column output block,
+// a wave 128 x 128 of it (8 x 8 MFMA tiles; the 256 accumulator registers live in the accumulation half of the
+// register file at one wave per SIMD).  A stage is 64 k of both operands (2 x 32 KiB) staged through LDS in
+// fragment order, double buffered: while the matrix cores work on one buffer, the next stage's global loads are in
+// flight and are written to the other buffer, one barrier per stage.  Weight fragments are copied as they lie in
+// memory (contiguous 1 KiB); the token fragments are transposed on the way in (lane = token of the tile, so the LDS
+// writes are contiguous) - every LDS read and write is a conflict-free 16-byte access at lane * 16.
+// Per stage and CU: 64 KiB from L2 for 2 x 64 x 4 MFMAs (2048 MFMA cycles per SIMD): 32 B/clk, half the L1 rate;
+// LDS traffic 64 KiB written + 128 KiB read.
+// ---------------------------------------------------------------------------------------------
+constexpr int LB = 256;              // block edge (tokens and columns)
+constexpr int LBK = 64;              // k per stage
+constexpr int LFR = LB / 16;         // 16-row fragments per operand per 32-k step
+constexpr int LSTAGE = 2 * (LBK / 32) * LFR * 512;   // fp16 elements per stage: W then x
+
+template <int OUT>
+__global__ __launch_bounds__(256) void gemm_lds_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx,
+                                                       const f16* __restrict__ Wp, int T, int K, int N) {
+  extern __shared__ __align__(16) f16 smem[];       // [2][LSTAGE]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int n0 = blockIdx.x * LB, t0 = blockIdx.y * LB;
+  const int wn = wave & 1, wt = wave >> 1;
+  const int KB = K / 32;
+  const int tiles = (N + 15) / 16;
+  constexpr int KS = LBK / 32;                      // 32-k steps per stage
+  constexpr int CH = KS * LFR * WAVE / 256;         // 16-byte chunks per thread, per operand and stage (8)
+
+  // chunk c = threadIdx.x + 256 j of a stage: fragment f = c / 64 = ks * LFR + tile, lane slot l = c % 64
+  const f16* wsrc[CH];
+  const f16* xsrc[CH];
+#pragma unroll
+  for (int j = 0; j < CH; ++j) {
+    const int c = threadIdx.x + 256 * j;
+    const int f = c >> 6, l = c & 63;
+    const int ks = f / LFR, tile = f % LFR;
+    int nt = n0 / 16 + tile;
+    nt = nt < tiles ? nt : tiles - 1;               // columns past N: a valid fragment, results dropped
+    wsrc[j] = Wp + ((size_t)nt * KB + ks) * 512 + l * 8;
+    int t = t0 + tile * 16 + (l & 15);
+    t = t < T ? t : T - 1;
+    xsrc[j] = x + (size_t)t * ldx + ks * 32 + (l >> 4) * 8;
+  }
+  f16x8 wst[CH], xst[CH];
+  auto load_stage = [&](int s) {                    // s: stage index; k-steps 2s, 2s+1 (the last may be past K)
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int ks = (threadIdx.x + 256 * j) / (64 * LFR);
+      const int kb = s * KS + ks;
+      const int kc = kb < KB ? kb : KB - 1;         // past K: a valid address; that step is not multiplied
+      wst[j] = ld8(wsrc[j] + (size_t)(kc - ks) * 512);
+      xst[j] = ld8(xsrc[j] + (kc - ks) * 32);
+    }
+  };
+  auto store_stage = [&](int buf) {
+    f16* dst = smem + buf * LSTAGE;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int c = threadIdx.x + 256 * j;
+      st8(dst + c * 8, wst[j]);
+      st8(dst + LSTAGE / 2 + c * 8, xst[j]);
+    }
+  };
+
+  f32x4 acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int S = (KB + KS - 1) / KS;
+  load_stage(0);
+  store_stage(0);
+  __syncthreads();
+  for (int s = 0; s < S; ++s) {
+    if (s + 1 < S) load_stage(s + 1);
+    const f16* ws = smem + (s & 1) * LSTAGE;
+    const f16* xs = ws + LSTAGE / 2;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (s * KS + ks < KB) {                        // workgroup-uniform
+        f16x8 a[8], b[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          a[i] = ld8(ws + (ks * LFR + wn * 8 + i) * 512 + lane * 8);
+          b[i] = ld8(xs + (ks * LFR + wt * 8 + i) * 512 + lane * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+      }
+    }
+    if (s + 1 < S) store_stage((s + 1) & 1);
+    __syncthreads();
+  }
+
+  const int r16 = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int t = t0 + wt * 128 + j * 16 + r16;
+    if (t >= T) continue;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int n = n0 + wn * 128 + i * 16 + g * 4;
+      if (n >= N) continue;
+      const size_t o = (size_t)t * N + n;
+      const f32x4 sacc = acc[i][j];
+      if constexpr (OUT == OUT_F16) {
+        *reinterpret_cast<f16x4*>((f16*)yv + o) = f16x4{(f16)sacc[0], (f16)sacc[1], (f16)sacc[2], (f16)sacc[3]};
+      } else if constexpr (OUT == OUT_F32) {
+        *reinterpret_cast<f32x4*>((float*)yv + o) = sacc;
+      } else {
+        f32x4* p = reinterpret_cast<f32x4*>((float*)yv + o);
+        *p = *p + sacc;
+      }
+    }
+  }
+}
+
+template <int OUT>
+int launch_gemm_lds(void* y, const f16* x, int ldx, const f16* Wp, int T, int K, int N, hipStream_t s) {
+  constexpr size_t lds = 2 * LSTAGE * sizeof(f16);
+  static bool configured = false;                    // the attribute is per kernel, set once per process
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_lds_kernel<OUT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return mlora_set_error(MLORA_ERR_LAUNCH, "gemm_packed: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    configured = true;
+  }
+  hipLaunchKernelGGL((gemm_lds_kernel<OUT>), dim3(ceil_div(N, LB), ceil_div(T, LB)), dim3(256), lds, s, y, x, ldx, Wp, T, K, N);
+  return MLORA_OK;
+}
+
 template <bool PACKED>
 int gemm_dispatch(const char* who, void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K,
                   int N, void* stream) {
@@ -109,6 +242,15 @@ int gemm_dispatch(const char* who, void* y, int y_dtype, int mode, const void* x
   hipStream_t s = (hipStream_t)stream;
   const f16* xp = (const f16*)x;
   const f16* Wp = (const f16*)W;
+  if constexpr (PACKED) {
+    if (T >= 512) {                                   // enough token blocks for the 256 x 256 kernel
+      int e;
+      if (mode == MLORA_ACCUMULATE) e = launch_gemm_lds<OUT_ACC_F32>(y, xp, ldx, Wp, T, K, N, s);
+      else if (y_dtype == MLORA_F32) e = launch_gemm_lds<OUT_F32>(y, xp, ldx, Wp, T, K, N, s);
+      else e = launch_gemm_lds<OUT_F16>(y, xp, ldx, Wp, T, K, N, s);
+      return e ? e : mlora_launch_status(who);
+    }
+  }
   if (mode == MLORA_ACCUMULATE) hipLaunchKernelGGL((gemm_kernel<OUT_ACC_F32, PACKED>), grid, block, 0, s, y, xp, ldx, Wp, T, K, N);
   else if (y_dtype == MLORA_F32) hipLaunchKernelGGL((gemm_kernel<OUT_F32, PACKED>), grid, block, 0, s, y, xp, ldx, Wp, T, K, N);
   else hipLaunchKernelGGL((gemm_kernel<OUT_F16, PACKED>), grid, block, 0, s, y, xp, ldx, Wp, T, K, N);

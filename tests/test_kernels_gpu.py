@@ -177,6 +177,27 @@ def test_gemm_large_T(ops, synth, packed):
     assert max_rel_err(_np(y), _np(x).astype(np.float64) @ _np(W).astype(np.float64).T, floor=1e-2) <= 5e-4
 
 
+@pytest.mark.parametrize("T,K,N", [(700, 1056, 1000), (512, 4096, 4096), (1300, 64, 36), (2048, 2752, 1024)])
+def test_gemm_lds_staged_block_kernel(ops, synth, T, K, N):
+    """T >= 512 with fragment-ordered weights takes the 256 x 256 LDS-staged kernel: odd number of 32-k steps, ragged
+    token and column edges, all three epilogues; and the same bits for x given as a strided column slice."""
+    x = synth.normal(9, f"gl.x.{T}.{K}", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(9, f"gl.W.{N}.{K}", (N, K), 0.02, torch.float16, DEV)
+    ref = _np(x).astype(np.float64) @ _np(W).astype(np.float64).T
+    Wp = ops.PackedWeight(W)
+    y16 = ops.linear(x, Wp)
+    y32 = ops.linear(x, Wp, out_dtype=torch.float32)
+    r0 = synth.normal(9, f"gl.r.{T}.{N}", (T, N), 1.0, torch.float32, DEV)
+    racc = r0.clone()
+    ops.linear(x, Wp, out=racc, accumulate=True)
+    assert max_rel_err(_np(y16), ref) <= TOL
+    assert max_rel_err(_np(y32), ref, floor=1e-2) <= 5e-4
+    assert max_rel_err(_np(racc), _np(r0) + ref, floor=1e-2) <= 5e-4
+    wide = torch.zeros((T, K + 64), dtype=torch.float16, device=DEV)
+    wide[:, 32:32 + K] = x
+    assert torch.equal(ops.linear(wide[:, 32:32 + K], Wp, out_dtype=torch.float32), y32)
+
+
 def test_pack_weight_is_a_permutation(ops, synth):
     """Bit-exact: every element of W appears at its fragment-order position, padding rows are zero."""
     N, K = 40, 64
