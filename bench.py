@@ -200,12 +200,123 @@ def cpu_baseline(wl, ctx, layers=2, steps=3):
                       f"{wl.shape.num_hidden_layers // layers}; threads = BLAS default on {os.cpu_count()} cores"}
 
 
+def bench_c4_prefill(args, synth, llama):
+    """BASELINE configs[3]: prefill of 8 x 512 tokens grouped in adapter segments, 64 rank-64 adapters on all seven
+    linears.  A step = one batched prefill pass over the whole model (fresh cache slots each step)."""
+    import torch
+    ops = _mod("ops")
+    dev = "cuda:0"
+    wl = synth.config4(num_layers=args.layers)
+    s = wl.shape
+    model = llama.LlamaForCausalLM.from_synthetic(wl.seed, s, [wl.lora], dev)
+    prompts = synth.prompts(wl)
+    B, P = prompts.shape
+    order = np.argsort(wl.adapter_ids, kind="stable")             # requests grouped into adapter segments
+    tokens = torch.from_numpy(np.ascontiguousarray(prompts[order].reshape(-1)))
+    wids = wl.adapter_ids[order]
+    blocks = -(-P // wl.page_size)
+    n_steps = args.warmup + args.steps
+    kv = model.create_paged_kv_cache(B, B * blocks * wl.page_size, P, wl.page_size,
+                                     free_pages=synth.permutation(wl.seed, "c4.pages", B * blocks), max_seq_len=blocks * wl.page_size)
+    for b in range(B):
+        kv.add_sequence(b)
+
+    def step():
+        for b in range(B):                                          # same pages again: every pass starts from empty sequences
+            kv.lens[b] = 0
+        kv.begin_forward(list(range(B)), [P] * B)
+        logits, _ = model["prefill_a0"](model.embed(tokens), kv, wids)
+        kv.end_forward()
+        return logits
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    T = B * P
+    L = s.num_hidden_layers
+    per_layer = sum(int(np.prod(synth.linear_dims(s, p))) for p in synth.LINEARS)
+    flops_base = 2.0 * T * per_layer * L
+    flops_lora = sum(2.0 * T * wl.lora.r * sum(synth.linear_dims(s, p)) for p in wl.lora.targets) * L
+    flops_attn = 2.0 * 2 * P * P / 2 * s.q_size * B * L            # causal QK^T and PV
+    flops = flops_base + flops_lora + flops_attn + 2.0 * B * s.hidden_size * s.vocab_size
+    print(json.dumps({
+        "metric": "prefill tok/s, Llama-7B-shape 8x512 tokens, 64 rank-64 adapters on 7 linears", "value": T / dt, "unit": "tok/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": wl.name, "layers": L, "tokens": T, "segments": int(len(np.unique(wids))), "rank": wl.lora.r,
+                   "lora_targets": list(wl.lora.targets)},
+        "roofline": {"kernel": "whole prefill pass (base GEMMs 97 % of the flops)", "bound": "mfma", "achieved": flops / dt / 1e12,
+                     "peak": 2500.0, "unit": "TFLOP/s", "frac": flops / dt / 1e12 / 2500.0, "traffic": None,
+                     "flops_base": flops_base, "flops_lora": flops_lora, "flops_attention": flops_attn}}))
+
+
+def bench_c5_decode(args, synth, llama):
+    """BASELINE configs[4]: 256 concurrent requests, Zipf(1.1) over 256 rank-16 adapters, context lengths uniform in
+    128..2048 in a shuffled paged cache pre-filled with N(0,1) values; a step = one decode step of all 256 requests
+    (per-operator path: the token count exceeds the 64-token decode tile of the native step)."""
+    import torch
+    dsm = _mod("decode_session")
+    dev = "cuda:0"
+    wl = synth.config5(num_layers=args.layers)
+    s = wl.shape
+    model = llama.LlamaForCausalLM.from_synthetic(wl.seed, s, [wl.lora], dev)
+    B = wl.batch
+    n_steps = args.warmup + args.steps
+    # requests in adapter order, as the front end batches them (`llama_seq_info.py:61-75` sorts by adapter type and weight id)
+    order = np.argsort(wl.adapter_ids, kind="stable")
+    adapter_ids = wl.adapter_ids[order]
+    ctx = wl.ctx_lens[order].astype(np.int64)
+    blocks = [int(-(-(c + n_steps + 1) // wl.page_size)) for c in ctx]
+    n_pages = sum(blocks)
+    kv = model.create_paged_kv_cache(B, n_pages * wl.page_size, 1, wl.page_size,
+                                     free_pages=synth.permutation(wl.seed, "c5.pages", n_pages), max_seq_len=max(blocks) * wl.page_size)
+    for l in range(s.num_hidden_layers):
+        kv.k[l].normal_()
+        kv.v[l].normal_()
+    for b in range(B):
+        kv.add_sequence(b)
+    kv.begin_forward(list(range(B)), [int(c) for c in ctx])          # claims the pages of the pre-filled contexts
+    kv.end_forward()
+    first = synth.randint(wl.seed, "c5.first", (B,), s.vocab_size).numpy()
+    sess = dsm.DecodeSession(model, kv, list(range(B)), {0: adapter_ids}, first)
+    for _ in range(args.warmup):
+        sess.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        sess.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    mean_ctx = float(ctx.sum()) + B * (args.warmup + (args.steps + 1) / 2.0)
+    kv_bytes = mean_ctx * s.num_hidden_layers * 2 * s.kv_size * 2
+    used = len(np.unique(wl.adapter_ids))
+    lora_bytes = s.num_hidden_layers * len(wl.lora.targets) * used * 2 * wl.lora.r * (2 * 4096)
+    step_bytes = model.weight_bytes_per_step() + kv_bytes + lora_bytes
+    print(json.dumps({
+        "metric": "decode tok/s, Llama-7B-shape 256 requests, Zipf over 256 rank-16 adapters, ctx 128-2048", "value": B / dt,
+        "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": wl.name, "layers": s.num_hidden_layers, "batch": B, "adapters_in_use": used,
+                   "total_context": int(ctx.sum()), "host_loop": "python"},
+        "roofline": {"kernel": "whole decode step (paged attention 91 % of the bytes)", "bound": "hbm",
+                     "achieved": step_bytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": step_bytes / dt / 1e9 / HBM_PEAK_GBS, "traffic": None, "step_algorithmic_gb": step_bytes / 1e9}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--layers", type=int, default=32, help="model depth (32 = the benchmark configuration)")
+    ap.add_argument("--workload", default="c3_decode", choices=["c3_decode", "c4_prefill", "c5_decode"],
+                    help="c3_decode is the benchmark the metric is quoted on; the other two time the prefill and the "
+                         "256-request stress configurations with the same harness")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel event timing and the gather-matmul stream")
     ap.add_argument("--python-loop", action="store_true", help="issue every kernel from Python instead of mlora_decode_step")
@@ -223,6 +334,10 @@ def main():
     synth, llama, dsm = _mod("synth"), _mod("llama"), _mod("decode_session")
     dev = "cuda:0"
     torch.cuda.set_device(0)
+    if args.workload == "c4_prefill":
+        return bench_c4_prefill(args, synth, llama)
+    if args.workload == "c5_decode":
+        return bench_c5_decode(args, synth, llama)
     if args.probe:
         wl = synth.config3(num_layers=2)
         model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, [wl.lora], dev)

@@ -307,6 +307,7 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(floa
                                                                             const int32_t* __restrict__ ids, int T, int K,
                                                                             int n_ad, const int32_t* __restrict__ bucket_of,
                                                                             int bucket) {
+  // blockIdx.y selects one of gridDim.y contiguous ranges of 32-k steps; its partial sums go to v[blockIdx.y][T][R]
   constexpr int NT = (R + 15) / 16;     // 16-row tiles of A[a]; rank 8 uses half a tile
   __shared__ f32x4 red[SEG_WAVES][NT][WAVE];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -318,6 +319,9 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(floa
   unsigned todo = (unsigned)__ballot(id >= 0) & 0xffffu;
   const f16* __restrict__ xr = x + (size_t)tl * K + g * 8;
   const int KB = K / 32;
+  const int per = (KB + gridDim.y - 1) / gridDim.y;
+  const int kb0 = blockIdx.y * per, kb1 = min(KB, kb0 + per);
+  v += (size_t)blockIdx.y * T * R;
   int a;
   unsigned rows;
   while (next_tile_adapter(id, todo, a, rows)) {
@@ -325,7 +329,7 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(floa
     f32x4 acc[NT];
 #pragma unroll
     for (int i = 0; i < NT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int kb = wave; kb < KB; kb += SEG_WAVES) {
+    for (int kb = kb0 + wave; kb < kb1; kb += SEG_WAVES) {
       const f16x8 xf = ld8(xr + kb * 32);
 #pragma unroll
       for (int i = 0; i < NT; ++i) {
@@ -356,7 +360,8 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* 
                                                                             const f16* __restrict__ B,
                                                                             const int32_t* __restrict__ ids, float scaling,
                                                                             int T, int N, int ldy, int n_ad,
-                                                                            const int32_t* __restrict__ bucket_of, int bucket) {
+                                                                            const int32_t* __restrict__ bucket_of, int bucket,
+                                                                            int splits) {
   constexpr int KS = (R + 31) / 32;     // k-steps of 32 rank entries (ranks 8 and 16: one partly filled step)
   constexpr int CT = 4;                 // 16-column tiles per wave
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -377,19 +382,19 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* 
     float f[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) f[e] = 0.f;
-    if (j < R) {
-      const f32x4 lo = *reinterpret_cast<const f32x4*>(v + (size_t)tl * R + j);
-      const f32x4 hi = *reinterpret_cast<const f32x4*>(v + (size_t)tl * R + j + 4);
+    if (j < R && id >= 0) {
+      f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
+      for (int sp = 0; sp < splits; ++sp) {           // the K-range partials of the shrink, summed in range order
+        lo += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + tl) * R + j);
+        hi += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + tl) * R + j + 4);
+      }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         f[e] = lo[e] * scaling;
         f[4 + e] = hi[e] * scaling;
       }
     }
-    if (id < 0) {                        // rows of unadapted tokens may hold anything: keep NaNs out of the product
-#pragma unroll
-      for (int e = 0; e < 8; ++e) f[e] = 0.f;
-    }
+    // rows of unadapted tokens are never read (their v holds nothing) and enter the product as zeros
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const f16 h = (f16)f[e];
@@ -581,15 +586,22 @@ template <int R>
 static void gmm_segments_r(void* y, int y_dtype, int ldy, const f16* x, const f16* A, const f16* B, const int32_t* ids,
                            float scaling, int T, int K, int N, int n_ad, float* v, BucketFilter bf, hipStream_t s) {
   const int tiles = ceil_div(T, 16);
-  hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles), dim3(SEG_WAVES * WAVE), 0, s, v, x, A, ids, T, K, n_ad,
+  // few token tiles: split K over workgroups so that the shrink still covers the chip (partials fit the workspace,
+  // which holds lora_k_split(K).kc slices of [T, r])
+  int splits = 512 / tiles;
+  const int kc = lora_k_split(K).kc;
+  if (splits > kc) splits = kc;
+  if (splits > K / 128) splits = K / 128;
+  if (splits < 1) splits = 1;
+  hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles, splits), dim3(SEG_WAVES * WAVE), 0, s, v, x, A, ids, T, K, n_ad,
                      bf.bucket_of, bf.bucket);
   const dim3 grid(tiles, ceil_div(N, SEG_WAVES * 64));
   if (y_dtype == MLORA_F16)
     hipLaunchKernelGGL((lora_expand_mfma_kernel<R, f16>), grid, dim3(SEG_WAVES * WAVE), 0, s, (f16*)y, v, B, ids, scaling, T, N,
-                       ldy, n_ad, bf.bucket_of, bf.bucket);
+                       ldy, n_ad, bf.bucket_of, bf.bucket, splits);
   else
     hipLaunchKernelGGL((lora_expand_mfma_kernel<R, float>), grid, dim3(SEG_WAVES * WAVE), 0, s, (float*)y, v, B, ids, scaling, T,
-                       N, ldy, n_ad, bf.bucket_of, bf.bucket);
+                       N, ldy, n_ad, bf.bucket_of, bf.bucket, splits);
 }
 
 // shrink + expand on the matrix cores; v = workspace viewed as [T, r] fp32

@@ -243,7 +243,8 @@ int gemm_dispatch(const char* who, void* y, int y_dtype, int mode, const void* x
   const f16* xp = (const f16*)x;
   const f16* Wp = (const f16*)W;
   if constexpr (PACKED) {
-    if (T >= 512) {                                   // enough token blocks for the 256 x 256 kernel
+    if (T >= 512) {                                   // enough token blocks for the 256 x 256 kernel (slower than the
+                                                      // register-tile kernel at T = 256: too few workgroups)
       int e;
       if (mode == MLORA_ACCUMULATE) e = launch_gemm_lds<OUT_ACC_F32>(y, xp, ldx, Wp, T, K, N, s);
       else if (y_dtype == MLORA_F32) e = launch_gemm_lds<OUT_F32>(y, xp, ldx, Wp, T, K, N, s);
