@@ -100,96 +100,115 @@ __global__ __launch_bounds__(256) void gemm_kernel(void* __restrict__ yv, const 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Large-T variant for fragment-ordered weights: a workgroup of 4 waves owns a 256-token x 256-column output block,
-// a wave 128 x 128 of it (8 x 8 MFMA tiles; the 256 accumulator registers live in the accumulation half of the
-// register file at one wave per SIMD).  A stage is 64 k of both operands (2 x 32 KiB) staged through LDS in
+// LDS-staged variant for fragment-ordered weights.  In its large shape a workgroup of 4 waves owns a 256-token x
+// 256-column output block, a wave 128 x 128 of it (8 x 8 MFMA tiles; the 256 accumulator registers live in the
+// accumulation half of the register file at one wave per SIMD).  A stage is 64 k of both operands (2 x 32 KiB) staged through LDS in
 // fragment order, double buffered: while the matrix cores work on one buffer, the next stage's global loads are in
 // flight and are written to the other buffer, one barrier per stage.  Weight fragments are copied as they lie in
-// memory (contiguous 1 KiB); the token fragments are transposed on the way in (lane = token of the tile, so the LDS
-// writes are contiguous) - every LDS read and write is a conflict-free 16-byte access at lane * 16.
+// memory (contiguous 1 KiB); the token rows are read 64 contiguous bytes at a time and transposed into fragment
+// order by the LDS write (with an XOR on the token slot that keeps every quarter-wave write conflict-free).
 // Per stage and CU: 64 KiB from L2 for 2 x 64 x 4 MFMAs (2048 MFMA cycles per SIMD): 32 B/clk, half the L1 rate;
 // LDS traffic 64 KiB written + 128 KiB read.
 // ---------------------------------------------------------------------------------------------
-constexpr int LB = 256;              // block edge (tokens and columns)
 constexpr int LBK = 64;              // k per stage
-constexpr int LFR = LB / 16;         // 16-row fragments per operand per 32-k step
-constexpr int LSTAGE = 2 * (LBK / 32) * LFR * 512;   // fp16 elements per stage: W then x
 
-template <int OUT>
+// FT x FN: 16-row fragments of tokens / of weight rows per block; WT x WN: MFMA tiles of a wave (FT/WT * FN/WN == 4 waves)
+template <int OUT, int FT, int FN, int WT_, int WN_>
 __global__ __launch_bounds__(256) void gemm_lds_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx,
                                                        const f16* __restrict__ Wp, int T, int K, int N) {
-  extern __shared__ __align__(16) f16 smem[];       // [2][LSTAGE]
+  static_assert((FT / WT_) * (FN / WN_) == 4, "four waves cover the block");
+  constexpr int KS = LBK / 32;                      // 32-k steps per stage
+  constexpr int WELEMS = KS * FN * 512, XELEMS = KS * FT * 512;   // fp16 elements of a stage: W, then x
+  constexpr int STAGE = WELEMS + XELEMS;
+  constexpr int WCH = KS * FN * WAVE / 256, XCH = KS * FT * WAVE / 256;   // 16-byte chunks per thread and stage
+  static_assert(WCH >= 1 && XCH >= 1, "a stage gives every thread at least one chunk of each operand");
+  extern __shared__ __align__(16) f16 smem[];       // [2][STAGE]
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int n0 = blockIdx.x * LB, t0 = blockIdx.y * LB;
-  const int wn = wave & 1, wt = wave >> 1;
+  const int n0 = blockIdx.x * FN * 16, t0 = blockIdx.y * FT * 16;
+  constexpr int WAVES_N = FN / WN_;
+  const int wn = wave % WAVES_N, wt = wave / WAVES_N;
   const int KB = K / 32;
   const int tiles = (N + 15) / 16;
-  constexpr int KS = LBK / 32;                      // 32-k steps per stage
-  constexpr int CH = KS * LFR * WAVE / 256;         // 16-byte chunks per thread, per operand and stage (8)
 
-  // chunk c = threadIdx.x + 256 j of a stage: fragment f = c / 64 = ks * LFR + tile, lane slot l = c % 64
-  const f16* wsrc[CH];
-  const f16* xsrc[CH];
+  // chunk c = threadIdx.x + 256 j of an operand's stage: fragment f = c / 64 = ks * F + tile, lane slot l = c % 64
+  const f16* wsrc[WCH];
+  const f16* xsrc[XCH];
 #pragma unroll
-  for (int j = 0; j < CH; ++j) {
+  for (int j = 0; j < WCH; ++j) {
     const int c = threadIdx.x + 256 * j;
     const int f = c >> 6, l = c & 63;
-    const int ks = f / LFR, tile = f % LFR;
+    const int ks = f / FN, tile = f % FN;
     int nt = n0 / 16 + tile;
     nt = nt < tiles ? nt : tiles - 1;               // columns past N: a valid fragment, results dropped
     wsrc[j] = Wp + ((size_t)nt * KB + ks) * 512 + l * 8;
-    int t = t0 + tile * 16 + (l & 15);
-    t = t < T ? t : T - 1;
-    xsrc[j] = x + (size_t)t * ldx + ks * 32 + (l >> 4) * 8;
   }
-  f16x8 wst[CH], xst[CH];
-  auto load_stage = [&](int s) {                    // s: stage index; k-steps 2s, 2s+1 (the last may be past K)
+  // x chunks: 4 consecutive lanes read the 64 contiguous bytes (one 32-k step) of one token row, so a quarter-wave
+  // covers 4 rows x 4 lane groups g.  The LDS slot of a token inside its 16-token fragment is XORed with 4 g: the 16
+  // lanes of a quarter-wave then write 16 different slots (no bank conflict), and a read of a fragment stays a
+  // permutation inside each 16-lane group.
+  int xdst[XCH];
 #pragma unroll
-    for (int j = 0; j < CH; ++j) {
-      const int ks = (threadIdx.x + 256 * j) / (64 * LFR);
+  for (int j = 0; j < XCH; ++j) {
+    const int c2 = threadIdx.x + 256 * j;
+    const int ks = c2 / (FT * 64), c = c2 % (FT * 64);
+    const int row = c >> 2, gq = c & 3;
+    int t = t0 + row;
+    t = t < T ? t : T - 1;
+    xsrc[j] = x + (size_t)t * ldx + ks * 32 + gq * 8;
+    xdst[j] = ((ks * FT + (row >> 4)) * 64 + gq * 16 + ((row & 15) ^ (gq << 2))) * 8;
+  }
+  f16x8 wst[WCH], xst[XCH];
+  auto load_stage = [&](int s) {                    // s: stage index; k-steps KS*s .. (the last may be past K)
+#pragma unroll
+    for (int j = 0; j < WCH; ++j) {
+      const int ks = (threadIdx.x + 256 * j) / (64 * FN);
       const int kb = s * KS + ks;
       const int kc = kb < KB ? kb : KB - 1;         // past K: a valid address; that step is not multiplied
       wst[j] = ld8(wsrc[j] + (size_t)(kc - ks) * 512);
+    }
+#pragma unroll
+    for (int j = 0; j < XCH; ++j) {
+      const int ks = (threadIdx.x + 256 * j) / (FT * 64);
+      const int kb = s * KS + ks;
+      const int kc = kb < KB ? kb : KB - 1;
       xst[j] = ld8(xsrc[j] + (kc - ks) * 32);
     }
   };
   auto store_stage = [&](int buf) {
-    f16* dst = smem + buf * LSTAGE;
+    f16* dst = smem + buf * STAGE;
 #pragma unroll
-    for (int j = 0; j < CH; ++j) {
-      const int c = threadIdx.x + 256 * j;
-      st8(dst + c * 8, wst[j]);
-      st8(dst + LSTAGE / 2 + c * 8, xst[j]);
-    }
+    for (int j = 0; j < WCH; ++j) st8(dst + (threadIdx.x + 256 * j) * 8, wst[j]);
+#pragma unroll
+    for (int j = 0; j < XCH; ++j) st8(dst + WELEMS + xdst[j], xst[j]);
   };
 
-  f32x4 acc[8][8];
+  f32x4 acc[WN_][WT_];
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
+  for (int i = 0; i < WN_; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < WT_; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  const int xslot = (lane & 48) + ((lane & 15) ^ ((lane >> 4) << 2));   // lane's token slot after the write-side XOR
   const int S = (KB + KS - 1) / KS;
   load_stage(0);
   store_stage(0);
   __syncthreads();
   for (int s = 0; s < S; ++s) {
     if (s + 1 < S) load_stage(s + 1);
-    const f16* ws = smem + (s & 1) * LSTAGE;
-    const f16* xs = ws + LSTAGE / 2;
+    const f16* ws = smem + (s & 1) * STAGE;
+    const f16* xs = ws + WELEMS;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (s * KS + ks < KB) {                        // workgroup-uniform
-        f16x8 a[8], b[8];
+        f16x8 a[WN_], b[WT_];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          a[i] = ld8(ws + (ks * LFR + wn * 8 + i) * 512 + lane * 8);
-          b[i] = ld8(xs + (ks * LFR + wt * 8 + i) * 512 + lane * 8);
-        }
+        for (int i = 0; i < WN_; ++i) a[i] = ld8(ws + (ks * FN + wn * WN_ + i) * 512 + lane * 8);
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int j = 0; j < WT_; ++j) b[j] = ld8(xs + (ks * FT + wt * WT_ + j) * 512 + xslot * 8);
 #pragma unroll
-          for (int j = 0; j < 8; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int i = 0; i < WN_; ++i)
+#pragma unroll
+          for (int j = 0; j < WT_; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], b[j], acc[i][j], 0, 0, 0);
       }
     }
     if (s + 1 < S) store_stage((s + 1) & 1);
@@ -198,12 +217,12 @@ __global__ __launch_bounds__(256) void gemm_lds_kernel(void* __restrict__ yv, co
 
   const int r16 = lane & 15, g = lane >> 4;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int t = t0 + wt * 128 + j * 16 + r16;
+  for (int j = 0; j < WT_; ++j) {
+    const int t = t0 + (wt * WT_ + j) * 16 + r16;
     if (t >= T) continue;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int n = n0 + wn * 128 + i * 16 + g * 4;
+    for (int i = 0; i < WN_; ++i) {
+      const int n = n0 + (wn * WN_ + i) * 16 + g * 4;
       if (n >= N) continue;
       const size_t o = (size_t)t * N + n;
       const f32x4 sacc = acc[i][j];
@@ -219,17 +238,27 @@ __global__ __launch_bounds__(256) void gemm_lds_kernel(void* __restrict__ yv, co
   }
 }
 
-template <int OUT>
+template <int OUT, int FT, int FN, int WT_, int WN_>
 int launch_gemm_lds(void* y, const f16* x, int ldx, const f16* Wp, int T, int K, int N, hipStream_t s) {
-  constexpr size_t lds = 2 * LSTAGE * sizeof(f16);
+  constexpr size_t lds = 2 * (LBK / 32) * (FT + FN) * 512 * sizeof(f16);
   static bool configured = false;                    // the attribute is per kernel, set once per process
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_lds_kernel<OUT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (!configured && lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_lds_kernel<OUT, FT, FN, WT_, WN_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return mlora_set_error(MLORA_ERR_LAUNCH, "gemm_packed: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     configured = true;
   }
-  hipLaunchKernelGGL((gemm_lds_kernel<OUT>), dim3(ceil_div(N, LB), ceil_div(T, LB)), dim3(256), lds, s, y, x, ldx, Wp, T, K, N);
+  hipLaunchKernelGGL((gemm_lds_kernel<OUT, FT, FN, WT_, WN_>), dim3(ceil_div(N, FN * 16), ceil_div(T, FT * 16)), dim3(256), lds, s,
+                     y, x, ldx, Wp, T, K, N);
   return MLORA_OK;
+}
+
+// Block shape by problem size: 256 x 256 (wave 128 x 128) when there are enough blocks to fill the chip, else
+// 256 tokens x 64 columns (wave 64 x 64, several workgroups per CU) so that a few hundred tokens still spread
+// over all CUs.
+template <int OUT>
+int launch_gemm_lds_auto(void* y, const f16* x, int ldx, const f16* Wp, int T, int K, int N, hipStream_t s) {
+  if ((long)ceil_div(T, 256) * ceil_div(N, 256) >= 256) return launch_gemm_lds<OUT, 16, 16, 8, 8>(y, x, ldx, Wp, T, K, N, s);
+  return launch_gemm_lds<OUT, 16, 4, 4, 4>(y, x, ldx, Wp, T, K, N, s);
 }
 
 template <bool PACKED>
@@ -243,12 +272,11 @@ int gemm_dispatch(const char* who, void* y, int y_dtype, int mode, const void* x
   const f16* xp = (const f16*)x;
   const f16* Wp = (const f16*)W;
   if constexpr (PACKED) {
-    if (T >= 512) {                                   // enough token blocks for the 256 x 256 kernel (slower than the
-                                                      // register-tile kernel at T = 256: too few workgroups)
+    if (T > 128) {
       int e;
-      if (mode == MLORA_ACCUMULATE) e = launch_gemm_lds<OUT_ACC_F32>(y, xp, ldx, Wp, T, K, N, s);
-      else if (y_dtype == MLORA_F32) e = launch_gemm_lds<OUT_F32>(y, xp, ldx, Wp, T, K, N, s);
-      else e = launch_gemm_lds<OUT_F16>(y, xp, ldx, Wp, T, K, N, s);
+      if (mode == MLORA_ACCUMULATE) e = launch_gemm_lds_auto<OUT_ACC_F32>(y, xp, ldx, Wp, T, K, N, s);
+      else if (y_dtype == MLORA_F32) e = launch_gemm_lds_auto<OUT_F32>(y, xp, ldx, Wp, T, K, N, s);
+      else e = launch_gemm_lds_auto<OUT_F16>(y, xp, ldx, Wp, T, K, N, s);
       return e ? e : mlora_launch_status(who);
     }
   }

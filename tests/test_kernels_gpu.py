@@ -177,10 +177,12 @@ def test_gemm_large_T(ops, synth, packed):
     assert max_rel_err(_np(y), _np(x).astype(np.float64) @ _np(W).astype(np.float64).T, floor=1e-2) <= 5e-4
 
 
-@pytest.mark.parametrize("T,K,N", [(700, 1056, 1000), (512, 4096, 4096), (1300, 64, 36), (2048, 2752, 1024)])
+@pytest.mark.parametrize("T,K,N", [(700, 1056, 1000), (512, 4096, 4096), (1300, 64, 36), (2048, 2752, 1024),
+                                   (4096, 288, 4096), (4100, 96, 4104), (200, 512, 264)])
 def test_gemm_lds_staged_block_kernel(ops, synth, T, K, N):
-    """T >= 512 with fragment-ordered weights takes the 256 x 256 LDS-staged kernel: odd number of 32-k steps, ragged
-    token and column edges, all three epilogues; and the same bits for x given as a strided column slice."""
+    """T > 128 with fragment-ordered weights takes the LDS-staged kernel (256 x 64 blocks, or 256 x 256 once there are
+    256 of those): odd number of 32-k steps, ragged token and column edges, all three epilogues; and the same bits
+    for x given as a strided column slice."""
     x = synth.normal(9, f"gl.x.{T}.{K}", (T, K), 1.0, torch.float16, DEV)
     W = synth.normal(9, f"gl.W.{N}.{K}", (N, K), 0.02, torch.float16, DEV)
     ref = _np(x).astype(np.float64) @ _np(W).astype(np.float64).T
