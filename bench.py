@@ -201,7 +201,7 @@ def cpu_baseline(wl, ctx, layers=2, steps=3):
 
 
 def bench_c4_prefill(args, synth, llama):
-    """BASELINE configs[3]: prefill of 8 x 512 tokens grouped in adapter segments, 64 rank-64 adapters on all seven
+    """The prefill configuration: 8 x 512 tokens grouped in adapter segments, 64 rank-64 adapters on all seven
     linears.  A step = one batched prefill pass over the whole model (fresh cache slots each step)."""
     import torch
     ops = _mod("ops")
@@ -256,7 +256,7 @@ def bench_c4_prefill(args, synth, llama):
 
 
 def bench_c5_decode(args, synth, llama):
-    """BASELINE configs[4]: 256 concurrent requests, Zipf(1.1) over 256 rank-16 adapters, context lengths uniform in
+    """The auto-batching stress configuration: 256 concurrent requests, Zipf(1.1) over 256 rank-16 adapters, context lengths uniform in
     128..2048 in a shuffled paged cache pre-filled with N(0,1) values; a step = one decode step of all 256 requests
     (per-operator path: the token count exceeds the 64-token decode tile of the native step)."""
     import torch
