@@ -364,16 +364,17 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* 
                                                                             int splits) {
   constexpr int KS = (R + 31) / 32;     // k-steps of 32 rank entries (ranks 8 and 16: one partly filled step)
   constexpr int CT = 4;                 // 16-column tiles per wave
+  constexpr int LD = 16 * CT + 4;       // padded row of the transposition buffer (floats): conflict-free both ways
+  __shared__ float stage[SEG_WAVES][16][LD];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t0 = blockIdx.x * 16;
   const int n0 = (blockIdx.y * SEG_WAVES + wave) * 16 * CT;
-  if (n0 >= N) return;
   const int col = lane & 15, g = lane >> 4;
   const int tl = min(t0 + col, T - 1);
   const int raw = lora_token_id(ids, bucket_of, bucket, t0 + col, T);
   const int id = (raw >= 0 && raw < n_ad) ? raw : -1;
   unsigned todo = (unsigned)__ballot(id >= 0) & 0xffffu;
-  if (!todo) return;
+  if (!todo) return;                    // the same for every wave of the workgroup
   // the token tile of v as the B operand, hi and lo halves: lane holds v[token col][ks*32 + 8g .. +7]
   f16x8 vh[KS], vl[KS];
 #pragma unroll
@@ -382,6 +383,7 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* 
     float f[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) f[e] = 0.f;
+    // rows of unadapted tokens are never read (their v holds nothing) and enter the product as zeros
     if (j < R && id >= 0) {
       f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
       for (int sp = 0; sp < splits; ++sp) {           // the K-range partials of the shrink, summed in range order
@@ -394,7 +396,6 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* 
         f[4 + e] = hi[e] * scaling;
       }
     }
-    // rows of unadapted tokens are never read (their v holds nothing) and enter the product as zeros
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const f16 h = (f16)f[e];
@@ -402,6 +403,10 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* 
       vl[ks][e] = (f16)(f[e] - (float)h);
     }
   }
+  // write-back role of the lane: token lane / 4, the 16 columns of column tile lane % 4 (contiguous in y)
+  const int wt = lane >> 2, wc = lane & 3;
+  const int nw = n0 + wc * 16;
+  YT* __restrict__ yrow = y + (size_t)(t0 + wt) * ldy + nw;
   int a;
   unsigned rows;
   while (next_tile_adapter(id, todo, a, rows)) {
@@ -409,20 +414,35 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* 
 #pragma unroll
     for (int c = 0; c < CT; ++c) {
       const int nb = n0 + c * 16;
-      if (nb >= N) break;                                          // wave-uniform
-      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (nb < N) {                                                // wave-uniform
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int j = ks * 32 + g * 8;
-        const f16x8 bf = j < R ? ld8(Ba + (size_t)(nb + col) * R + ks * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf, vh[ks], acc, 0, 0, 0);      // rows: output column, cols: tokens
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf, vl[ks], acc, 0, 0, 0);
-      }
-      if ((rows >> col) & 1u) {
-        float d[4] = {acc[0], acc[1], acc[2], acc[3]};
-        rmw_add<YT, 4>(y + (size_t)(t0 + col) * ldy + nb + 4 * g, d);
+        for (int ks = 0; ks < KS; ++ks) {
+          const int j = ks * 32 + g * 8;
+          const f16x8 bf = j < R ? ld8(Ba + (size_t)(nb + col) * R + ks * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf, vh[ks], acc, 0, 0, 0);    // rows: output column, cols: tokens
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf, vl[ks], acc, 0, 0, 0);
+        }
+        *reinterpret_cast<f32x4*>(&stage[wave][col][c * 16 + 4 * g]) = acc;           // D[n = 4g.., token col]
       }
     }
+    __syncthreads();
+    if (nw < N && ((rows >> wt) & 1u)) {
+      float d[16];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const f32x4 s4 = *reinterpret_cast<const f32x4*>(&stage[wave][wt][wc * 16 + 4 * q]);
+        d[4 * q] = s4[0]; d[4 * q + 1] = s4[1]; d[4 * q + 2] = s4[2]; d[4 * q + 3] = s4[3];
+      }
+      if constexpr (sizeof(YT) == 2) {
+        rmw_add<YT, 8>(yrow, d);
+        rmw_add<YT, 8>(yrow + 8, d + 8);
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) rmw_add<YT, 4>(yrow + 4 * q, d + 4 * q);
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -633,7 +653,7 @@ static int gather_mm_impl(void* y, int y_dtype, int ldy, const void* x, int x_la
     const GmmSet one = {y, (const f16*)x, (const f16*)A, (const f16*)B};
     return gmm_one_launch(one, nullptr, 1, y_dtype, ldy, x_layout, tok_adapter, scaling, T, K, N, r, n_ad, (hipStream_t)stream, bf);
   }
-  if (x_layout == MLORA_ROWMAJOR && T > 64 && K % 32 == 0 && N % 16 == 0 && ldy % 4 == 0 && (uintptr_t)y % 16 == 0) {
+  if (x_layout == MLORA_ROWMAJOR && T > 64 && K % 32 == 0 && N % 16 == 0 && ldy % 8 == 0 && (uintptr_t)y % 16 == 0) {
     MLORA_CHECK(y && x && A && B && tok_adapter, MLORA_ERR_INVALID, "gather_mm: null pointer");
     MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "gather_mm: bad y_dtype %d", y_dtype);
     MLORA_CHECK(ldy >= N, MLORA_ERR_INVALID, "gather_mm: need ldy >= N (ldy=%d N=%d)", ldy, N);
