@@ -262,6 +262,20 @@ int mlora_rope_kv_append_lora(void* qkv, void* k_cache, void* v_cache,
                               int T, int Hq, int Hkv, int D, int n_pages, int n_seq,
                               const void* v_part, int v_dense, const void* const* B, const int32_t* tok_adapter,
                               float scaling, int K, int r, int n_ad, void* stream);
+/* RoPE + cache append + decode attention (+ the LoRA expand of q, k, v) in ONE launch, for a decode step in which
+ * row b of qkv is the new token of sequence seq_ids[b] at position tok_pos[b] and ctx_len[b] = tok_pos[b] + 1.
+ * Results equal mlora_rope_kv_append[_lora] followed by mlora_paged_attn_decode bit for bit (out and both caches),
+ * except that the q rows of qkv are left unrotated.  v_part == NULL: no LoRA (B, tok_adapter ignored); otherwise
+ * the LoRA arguments are those of mlora_rope_kv_append_lora.  Replaces: attention_with_fused_qkv
+ * (tvm/llama_auto_batcher/llama_for_causal_lm.py:55-64) for the decode entry points, with the q/v adapter deltas of
+ * compile_tvm.py:126-134 applied inside. */
+int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv, void* k_cache, void* v_cache,
+                           const int32_t* block_table, int max_blocks,
+                           const int32_t* seq_ids, const int32_t* tok_pos, const int32_t* ctx_len,
+                           const float* rope_cos, const float* rope_sin, int max_pos,
+                           int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                           const void* v_part, int v_dense, const void* const* Bmat, const int32_t* tok_adapter,
+                           float scaling, int K, int r, int n_ad, void* stream);
 int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v_part, int v_dense, const void* B,
                               const int32_t* tok_adapter, float scaling, const void* w, float eps,
                               int T, int H, int K, int r, int n_ad, void* stream);

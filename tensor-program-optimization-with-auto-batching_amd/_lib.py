@@ -43,6 +43,7 @@ SIGNATURES = {
     "mlora_gemv_frag_silu": (_i, [_p, _p, _p, _i, _i, _i, _p]),
     "mlora_gemv_frag_split": (_i, [_p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _p]),
     "mlora_rope_kv_append_lora": (_i, [_p, _p, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p]),
+    "mlora_rope_attn_decode": (_i, [_p, _i, _p, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p]),
     "mlora_lora_expand_rmsnorm": (_i, [_p, _i, _p, _p, _i, _p, _p, _f, _p, _f, _i, _i, _i, _i, _i, _p]),
     "mlora_rmsnorm": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _p]),
     "mlora_silu_mul": (_i, [_p, _i, _p, _p, _i, _i, _i, _p]),

@@ -243,6 +243,248 @@ __global__ __launch_bounds__(ATT_WAVES * WAVE, 4) void paged_attn_decode_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
+// Decode step in one launch: RoPE + cache append (+ LoRA expand of q, k, v) + attention.  Same workgroup shape
+// and page loop as paged_attn_decode_kernel.  The workgroup first finishes the new token of its sequence for its
+// own heads - projection output + LoRA delta, rotation of q and k exactly as rope_kv_append_kernel does it - keeps
+// the rotated q, the new k and the new v in LDS and stores k, v to their page slot.  In the page loop the wave that
+// meets the page of the new token overwrites that token's lanes of the K / V fragments from LDS, so it never
+// depends on reading back what the workgroup has just stored.  Results are those of the two separate kernels,
+// bit for bit; the q rows of qkv are left unrotated.
+// ---------------------------------------------------------------------------------------------
+template <int D, int RG>   // RG: 8-wide rank groups the B-row registers hold (rank <= 8 RG)
+__global__ __launch_bounds__(ATT_WAVES * WAVE, 4) void rope_attn_decode_kernel(
+    f16* __restrict__ out, const f16* __restrict__ qkv, f16* __restrict__ k_cache, f16* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ seq_ids,
+    const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ ctx_len, const float* __restrict__ rope_cos,
+    const float* __restrict__ rope_sin, int max_pos, int Hq, int Hkv, int n_pages, int n_seq, float scale, int frag_tt,
+    LoraExpandQKV lx) {
+  constexpr int NKB = D / 32;
+  constexpr int NDB = D / 16;
+  constexpr int NW = ATT_WAVES;
+  constexpr int half = D / 2;
+  __shared__ float sm[NW][16], sl[NW][16];
+  __shared__ float lv[3][64];
+  __shared__ __align__(16) f16 qs[16 * D];       // rotated q of the group's heads
+  __shared__ __align__(16) f16 knew[D], vnew[D];   // the new token's rotated key and its value
+  extern __shared__ float sacc[];                  // [NW][G][D]
+
+  const int b = blockIdx.x, kh = blockIdx.y;
+  const int G = Hq / Hkv;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int col = lane & 15, g = lane >> 4;
+  const int seq = seq_ids[b];
+  const int pos = tok_pos[b];
+  int ctx = ctx_len[b];
+  const bool seq_ok = seq >= 0 && seq < n_seq;
+  if (!seq_ok) ctx = 0;
+  if (ctx > max_blocks * PAGE) ctx = max_blocks * PAGE;
+  const int npages = (ctx + PAGE - 1) / PAGE;
+  const int32_t* __restrict__ bt = block_table + (size_t)(seq_ok ? seq : 0) * max_blocks;
+  const bool pos_ok = seq_ok && pos >= 0 && pos < max_pos && pos / PAGE < max_blocks;   // the append condition of rope_kv_append
+  const int new_pg = pos_ok ? pos / PAGE : -1, new_slot = pos & (PAGE - 1);
+  const int new_page = pos_ok ? bt[new_pg] : -1;
+  const bool lora = lx.src.v != nullptr;
+  const int id = lora ? lx.ids[b] : -1;
+  const bool adapted = lora && id >= 0 && id < lx.n_ad;
+
+  // The wave's first page is requested before anything else, so that its latency overlaps the work on the new token.
+  int page = wave < npages ? bt[wave] : -1;
+  f16x8 kf[NKB];
+  f16x4 vf[NDB];
+  auto load_page = [&](int pgid) {
+    const f16* kp = k_cache + ((size_t)pgid * Hkv + kh) * PAGE * D + lane * 8;
+    const f16* vp = v_cache + (((size_t)pgid * Hkv + kh) * D + col) * PAGE + g * 4;   // dim col (+16 db), tokens 4g..
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) kf[kb] = ld8(kp + kb * 512);
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) vf[db] = *reinterpret_cast<const f16x4*>(vp + db * 16 * PAGE);
+  };
+  if (page >= 0 && page < n_pages) load_page(page);
+
+  // ---- the new token: heads kh*G .. kh*G+G-1 of q, head kh of k and of v; one (head, pair) item per thread and pass.
+  // An item's loads (projection output, rows of B, rotation factors) do not depend on the shrink results, so the
+  // first pass issues them before the barrier that publishes lv.
+  const int items = (G + 2) * half;
+  f16 h1, h2;
+  f16x8 b1[RG], b2[RG];
+  float rc, rs;
+  int hl, pi, proj;
+  bool with_delta;
+  auto issue = [&](int it) {
+    hl = it / half;                                              // local head: 0..G-1 q, G k, G+1 v
+    pi = it % half;
+    proj = hl < G ? 0 : (hl == G ? 1 : 2);
+    const int hh = proj == 0 ? kh * G + hl : (proj == 1 ? Hq + kh : Hq + Hkv + kh);   // head index inside qkv
+    const int head = proj == 0 ? kh * G + hl : kh;               // head index inside its projection
+    const f16* src = qkv + ((size_t)b * (Hq + 2 * Hkv) + hh) * D;
+    h1 = src[pi];
+    h2 = src[pi + half];
+    with_delta = adapted && lx.B[proj] != nullptr;
+    if (with_delta) {
+      const int n_rows = (proj == 0 ? Hq : Hkv) * D;
+      const f16* brow = lx.B[proj] + ((size_t)id * n_rows + (size_t)head * D) * lx.r;
+      lora_row_load(brow + (size_t)pi * lx.r, lx.r, b1);
+      lora_row_load(brow + (size_t)(pi + half) * lx.r, lx.r, b2);
+    }
+    rc = 1.f;
+    rs = 0.f;
+    if (proj != 2 && pos >= 0 && pos < max_pos) {
+      rc = rope_cos[(size_t)pos * half + pi];
+      rs = rope_sin[(size_t)pos * half + pi];
+    }
+  };
+  auto finish = [&]() {
+    if (with_delta) {
+      h1 = (f16)((float)h1 + lora_row_dot_regs(b1, lv[proj], lx.r));
+      h2 = (f16)((float)h2 + lora_row_dot_regs(b2, lv[proj], lx.r));
+    }
+    if (proj == 2) {
+      vnew[pi] = h1;
+      vnew[pi + half] = h2;
+      if (new_page >= 0 && new_page < n_pages) {
+        f16* dst = v_cache + ((size_t)new_page * Hkv + kh) * D * PAGE + new_slot;
+        dst[(size_t)pi * PAGE] = h1;
+        dst[(size_t)(pi + half) * PAGE] = h2;
+      }
+    } else {
+      const float x1 = (float)h1, x2 = (float)h2;
+      float r1, r2;
+      {
+#pragma clang fp contract(off)
+        r1 = x1 * rc - x2 * rs;                    // separately rounded products, as in rope_kv_append_kernel
+        r2 = x2 * rc + x1 * rs;
+      }
+      asm volatile("" : "+v"(r1), "+v"(r2));     // the fp32 result exists before the conversion
+      const f16 o1 = (f16)r1, o2 = (f16)r2;
+      if (proj == 0) {
+        qs[hl * D + pi] = o1;
+        qs[hl * D + pi + half] = o2;
+      } else {
+        knew[pi] = o1;
+        knew[pi + half] = o2;
+        if (new_page >= 0 && new_page < n_pages) {
+          f16* dst = k_cache + ((size_t)new_page * Hkv + kh) * PAGE * D;
+          dst[k_page_offset(new_slot, pi)] = o1;
+          dst[k_page_offset(new_slot, pi + half)] = o2;
+        }
+      }
+    }
+  };
+  const bool first = threadIdx.x < items;
+  if (first) issue(threadIdx.x);
+  if (adapted) {
+    for (int e = threadIdx.x; e < 3 * lx.r; e += NW * WAVE) {
+      const int pj = e / lx.r, j = e % lx.r;
+      lv[pj][j] = lx.B[pj] != nullptr ? lora_v_from(lx.src, pj, id, lx.r, b, j, lx.scaling) : 0.f;
+    }
+    __syncthreads();
+  }
+  if (first) finish();
+  for (int it = threadIdx.x + NW * WAVE; it < items; it += NW * WAVE) {
+    issue(it);
+    finish();
+  }
+  __syncthreads();
+
+  // Q^T as the B operand, from LDS: lane holds q[head col][kb*32 + g*8 .. +8], zero for unused columns
+  f16x8 qf[NKB];
+#pragma unroll
+  for (int kb = 0; kb < NKB; ++kb)
+    qf[kb] = col < G ? *reinterpret_cast<const f16x8*>(&qs[col * D + kb * 32 + g * 8]) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+
+  float m = -INFINITY, l = 0.f;
+  f32x4 O[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) O[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int pg = wave; pg < npages; pg += NW) {
+    const int next = pg + NW < npages ? bt[pg + NW] : -1;
+    if (page >= 0 && page < n_pages) {                      // wave-uniform
+      if (pg != wave) load_page(page);                      // the first page is already on its way
+      if (pg == new_pg) {                                   // wave-uniform: this page holds the token appended above
+        if (col == new_slot) {
+#pragma unroll
+          for (int kb = 0; kb < NKB; ++kb) kf[kb] = *reinterpret_cast<const f16x8*>(&knew[kb * 32 + g * 8]);
+        }
+        if ((new_slot >> 2) == g) {
+#pragma unroll
+          for (int db = 0; db < NDB; ++db) {
+            const f16 nv = vnew[db * 16 + col];
+            const int e = new_slot & 3;
+            vf[db][0] = e == 0 ? nv : vf[db][0];
+            vf[db][1] = e == 1 ? nv : vf[db][1];
+            vf[db][2] = e == 2 ? nv : vf[db][2];
+            vf[db][3] = e == 3 ? nv : vf[db][3];
+          }
+        }
+      }
+
+      f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) st = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kb], qf[kb], st, 0, 0, 0);
+
+      float pm = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        st[r] = (pg * PAGE + 4 * g + r >= ctx) ? -INFINITY : st[r] * scale;
+        pm = fmaxf(pm, st[r]);
+      }
+      pm = fmaxf(pm, __shfl_xor(pm, 16, WAVE));
+      pm = fmaxf(pm, __shfl_xor(pm, 32, WAVE));
+      const float m_new = fmaxf(m, pm);
+      const float alpha = __expf(m - m_new);
+      f16x8 pa;
+      float ps = 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = __expf(st[r] - m_new);
+        ps += p;
+        const f16 hi = (f16)p;
+        pa[r] = hi;
+        pa[4 + r] = (f16)(p - (float)hi);
+      }
+      l = l * alpha + ps;
+      m = m_new;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        O[db] *= alpha;
+        const f16x8 vv = f16x8{vf[db][0], vf[db][1], vf[db][2], vf[db][3], vf[db][0], vf[db][1], vf[db][2], vf[db][3]};
+        O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vv, pa, O[db], 0, 0, 0);
+      }
+    }
+    page = next;
+  }
+  l += __shfl_xor(l, 16, WAVE);
+  l += __shfl_xor(l, 32, WAVE);
+  if (col < G) {
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+      *reinterpret_cast<f32x4*>(&sacc[((size_t)wave * G + col) * D + db * 16 + 4 * g]) = O[db];
+    if (g == 0) {
+      sm[wave][col] = m;
+      sl[wave][col] = l;
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < G * D; e += NW * WAVE) {
+    const int qh = e / D, d = e % D;
+    float M = sm[0][qh];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) M = fmaxf(M, sm[w][qh]);
+    float L = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const float f = sm[w][qh] == -INFINITY ? 0.f : __expf(sm[w][qh] - M);
+      L += sl[w][qh] * f;
+      o += sacc[((size_t)w * G + qh) * D + d] * f;
+    }
+    const int h = kh * G + qh;
+    const size_t oo = frag_tt ? frag_offset(b, h * D + d, frag_tt) : ((size_t)b * Hq + h) * D + d;
+    out[oo] = (f16)(L > 0.f ? o / L : 0.f);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Prefill: a wave owns 16 consecutive query tokens of one head and walks the pages of their
 // sequence.  S^T = K . Q^T on v_mfma_f32_16x16x32_f16 puts key index on the accumulator rows, which
 // is exactly the A-operand layout the matrix core wants for P in O = P . V (a lane's four
@@ -441,6 +683,54 @@ extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qk
     hipLaunchKernelGGL(paged_attn_decode_kernel<64>, dim3(B, Hkv), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
                        (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale, frag_tt);
   return mlora_launch_status("paged_attn_decode");
+}
+
+extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv, void* k_cache, void* v_cache,
+                                      const int32_t* block_table, int max_blocks, const int32_t* seq_ids,
+                                      const int32_t* tok_pos, const int32_t* ctx_len, const float* rope_cos,
+                                      const float* rope_sin, int max_pos, int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                                      const void* v_part, int v_dense, const void* const* Bmat, const int32_t* tok_adapter,
+                                      float scaling, int K, int r, int n_ad, void* stream) {
+  if (int e = check_attn("rope_attn_decode", Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
+  MLORA_CHECK(out && qkv && k_cache && v_cache && block_table && seq_ids && tok_pos && ctx_len && rope_cos && rope_sin,
+              MLORA_ERR_INVALID, "rope_attn_decode: null pointer");
+  MLORA_CHECK(B >= 0 && max_pos > 0, MLORA_ERR_INVALID, "rope_attn_decode: bad B=%d max_pos=%d", B, max_pos);
+  MLORA_CHECK(out_layout == MLORA_ROWMAJOR || (out_layout == MLORA_FRAG && B <= 64), MLORA_ERR_UNSUPPORTED,
+              "rope_attn_decode: fragment-ordered output needs B <= 64 (layout=%d B=%d)", out_layout, B);
+  const int G = Hq / Hkv;
+  MLORA_CHECK(G <= 16, MLORA_ERR_UNSUPPORTED, "rope_attn_decode: more than 16 query heads per kv head (%d)", G);
+  LoraExpandQKV lx = {};
+  if (v_part != nullptr) {
+    MLORA_CHECK(Bmat && tok_adapter, MLORA_ERR_INVALID, "rope_attn_decode: null LoRA argument");
+    MLORA_CHECK((r == 8 || r == 16 || r == 32 || r == 64) && n_ad > 0 && K > 0, MLORA_ERR_UNSUPPORTED,
+                "rope_attn_decode: rank %d not in {8,16,32,64} or bad n_ad/K", r);
+    lx.src.v = (const float*)v_part;
+    lx.src.kc = v_dense ? 0 : lora_k_split(K).kc;
+    lx.src.T = B; lx.src.n_ad = n_ad; lx.src.ld = 3 * n_ad * r;
+    for (int i = 0; i < 3; ++i) lx.B[i] = (const f16*)Bmat[i];
+    lx.ids = tok_adapter;
+    lx.scaling = scaling;
+    lx.r = r; lx.n_ad = n_ad;
+  }
+  if (B == 0) return MLORA_OK;
+  const int frag_tt = out_layout == MLORA_FRAG ? mlora_frag_tiles(B) : 0;
+  const float scale = 1.f / sqrtf((float)D);
+  const size_t lds = (size_t)ATT_WAVES * G * D * sizeof(float);
+  hipStream_t s = (hipStream_t)stream;
+#define MLORA_ROPE_ATTN(DD, RG)                                                                                              \
+  hipLaunchKernelGGL((rope_attn_decode_kernel<DD, RG>), dim3(B, Hkv), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, \
+                     (f16*)k_cache, (f16*)v_cache, block_table, max_blocks, seq_ids, tok_pos, ctx_len, rope_cos, rope_sin,       \
+                     max_pos, Hq, Hkv, n_pages, n_seq, scale, frag_tt, lx)
+  const bool small_rank = v_part == nullptr || r <= 16;
+  if (D == 128) {
+    if (small_rank) MLORA_ROPE_ATTN(128, 2);
+    else MLORA_ROPE_ATTN(128, 8);
+  } else {
+    if (small_rank) MLORA_ROPE_ATTN(64, 2);
+    else MLORA_ROPE_ATTN(64, 8);
+  }
+#undef MLORA_ROPE_ATTN
+  return mlora_launch_status("rope_attn_decode");
 }
 
 extern "C" int mlora_paged_attn_prefill(void* out, const void* qkv, const void* k_cache, const void* v_cache,

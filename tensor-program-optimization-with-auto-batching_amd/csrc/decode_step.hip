@@ -68,16 +68,15 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
                            L.lora[MLORA_V].A ? L.lora[MLORA_V].B : nullptr};
       if (dense) STEP(mlora_gemv_frag_split(qkv, MLORA_F16, MLORA_STORE, (float*)ws_qkv, p->xn, L.qkv_p, T, H, qkv_sz, 3 * n_ad * r, stream));
       else STEP(mlora_gemv_frag_lora(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, ws_qkv, A3, 3, p->tok_adapter, r, n_ad, stream));
-      STEP(mlora_rope_kv_append_lora(qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos, p->rope_cos,
-                                     p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, ws_qkv, dense, B3,
-                                     p->tok_adapter, sc, H, r, n_ad, stream));
+      STEP(mlora_rope_attn_decode(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos,
+                                  p->ctx, p->rope_cos, p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, ws_qkv, dense,
+                                  B3, p->tok_adapter, sc, H, r, n_ad, stream));
     } else {
       STEP(mlora_gemv_frag(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, stream));
-      STEP(mlora_rope_kv_append(qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos, p->rope_cos,
-                                p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, stream));
+      STEP(mlora_rope_attn_decode(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos,
+                                  p->ctx, p->rope_cos, p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, nullptr, 0,
+                                  nullptr, nullptr, 0.f, 0, 0, 0, stream));
     }
-    STEP(mlora_paged_attn_decode(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows,
-                                 p->ctx, T, Hq, Hkv, D, p->n_pages, p->n_seq, stream));
     if (lora && L.lora[MLORA_O].A) {
       const void* A1[1] = {L.lora[MLORA_O].A};
       if (dense) STEP(mlora_gemv_frag_split(p->resid, MLORA_F32, MLORA_ACCUMULATE, (float*)ws_o, p->attn, L.o_p, T, q_sz, H, n_ad * r, stream));

@@ -166,24 +166,28 @@ __device__ __forceinline__ float lora_v_from(const LoraVSource& s, int slot, int
 
 // The same dot product in two halves, so that a caller can issue the row's loads before the v values are ready:
 // lora_row_load fetches up to 8 groups of 8 (r <= 64), lora_row_dot_regs consumes them in lora_row_dot's order.
-__device__ __forceinline__ void lora_row_load(const f16* __restrict__ brow, int r, f16x8 (&bv)[8]) {
+template <int NGMAX>
+__device__ __forceinline__ void lora_row_load(const f16* __restrict__ brow, int r, f16x8 (&bv)[NGMAX]) {
   const int ng = r >> 3;
 #pragma unroll
-  for (int q = 0; q < 8; ++q) {
+  for (int q = 0; q < NGMAX; ++q) {
     bv[q] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     if (q < ng) bv[q] = ld8(brow + q * 8);
   }
 }
 
-__device__ __forceinline__ float lora_row_dot_regs(const f16x8 (&bv)[8], const float* __restrict__ v, int r) {
-  float g[8];
+template <int NGMAX>
+__device__ __forceinline__ float lora_row_dot_regs(const f16x8 (&bv)[NGMAX], const float* __restrict__ v, int r) {
+  float g[8];                           // r <= 8 * NGMAX; groups past NGMAX are empty
   const int ng = r >> 3;
 #pragma unroll
   for (int q = 0; q < 8; ++q) {
     float s = 0.f;
-    if (q < ng) {
+    if (q < NGMAX) {
+      if (q < ng) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) s = fmaf((float)bv[q][e], v[q * 8 + e], s);
+        for (int e = 0; e < 8; ++e) s = fmaf((float)bv[q < NGMAX ? q : 0][e], v[q * 8 + e], s);
+      }
     }
     g[q] = s;
   }

@@ -198,7 +198,26 @@ __global__ __launch_bounds__(ROW_THREADS) void argmax_kernel(int32_t* __restrict
   const float* p = logits + (size_t)row * V;
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  for (int c = threadIdx.x; c < V; c += ROW_THREADS) amax_merge(bv, bi, p[c], c);
+  // 16-byte loads, four in flight per thread; elements are merged in increasing index order within a thread and the
+  // merge keeps the lower index on ties, so the result is the first maximum whatever the traversal order
+  const int V4 = ((size_t)p % 16 == 0) ? V / 4 : 0;
+  for (int c0 = threadIdx.x; c0 < V4; c0 += ROW_THREADS * 4) {
+    f32x4 q[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = c0 + u * ROW_THREADS;
+      q[u] = c < V4 ? *reinterpret_cast<const f32x4*>(p + 4 * (size_t)c) : f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = c0 + u * ROW_THREADS;
+      if (c < V4) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) amax_merge(bv, bi, q[u][e], 4 * c + e);
+      }
+    }
+  }
+  for (int c = 4 * V4 + threadIdx.x; c < V; c += ROW_THREADS) amax_merge(bv, bi, p[c], c);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     const float ov = __shfl_xor(bv, o, WAVE);

@@ -355,6 +355,20 @@ def paged_attn_decode(qkv, k_cache, v_cache, block_table, seq_ids, ctx_len, Hq, 
     return out
 
 
+def rope_attn_decode(qkv, k_cache, v_cache, block_table, seq_ids, tok_pos, ctx_len, rope_cos, rope_sin, Hq, Hkv, D,
+                     out=None, frag=False):
+    """rope_kv_append + paged_attn_decode of one decode step in one launch (no LoRA); qkv is left unrotated."""
+    B = qkv.shape[0]
+    n_seq, max_blocks = block_table.shape
+    out, optr, lay = _out_arg(out, B, Hq * D, frag, qkv.device)
+    check(lib().mlora_rope_attn_decode(optr, lay, _dev(qkv, torch.float16), _dev(k_cache, torch.float16),
+                                       _dev(v_cache, torch.float16), _dev(block_table, torch.int32), max_blocks,
+                                       _dev(seq_ids, torch.int32), _dev(tok_pos, torch.int32), _dev(ctx_len, torch.int32),
+                                       _dev(rope_cos, torch.float32), _dev(rope_sin, torch.float32), rope_cos.shape[0],
+                                       B, Hq, Hkv, D, k_cache.shape[0], n_seq, None, 0, None, None, 0.0, 0, 0, 0, _stream()))
+    return out
+
+
 def paged_attn_prefill(qkv, k_cache, v_cache, block_table, tok_seq, tok_pos, Hq, Hkv, D, out=None):
     T = qkv.shape[0]
     n_seq, max_blocks = block_table.shape

@@ -509,3 +509,41 @@ def test_gather_mm_prefill_column_slice(ops, synth):
     ref = oracle.gather_mm_ref(before[:, N:2 * N], _np(c["x"]), _np(c["A"]), _np(c["B"]), c["ids"].cpu().numpy(), 0.5)
     assert max_rel_err(after[:, N:2 * N], ref) <= TOL
     assert np.array_equal(after[:, :N], before[:, :N]) and np.array_equal(after[:, 2 * N:], before[:, 2 * N:])
+
+
+@pytest.mark.parametrize("Hq,Hkv,D", [(4, 4, 128), (8, 2, 64), (16, 1, 128), (6, 3, 64)])
+def test_rope_attn_decode_one_launch_equals_two(ops, synth, Hq, Hkv, D):
+    """RoPE + append + decode attention in one launch: output and both caches equal, bit for bit, those of
+    rope_kv_append followed by paged_attn_decode.  New tokens at the first and last slot of a page, in a fresh
+    sequence (context 1) and deep into a sequence; MHA and grouped heads; an out-of-range sequence row."""
+    kvm = load_pkg("kv_cache")
+    pos = [0, 15, 16, 31, 37, 100, 5]
+    B = len(pos)
+    n_pages, max_blocks = 40, 8
+    perm = synth.permutation(13, "ra.pages", n_pages)
+    table = np.full((B, max_blocks), -1, dtype=np.int32)
+    o = 0
+    for b, p in enumerate(pos):
+        nb = p // 16 + 1
+        table[b, :nb] = perm[o:o + nb]
+        o += nb
+    cos, sin = kvm.rope_tables(D, 10000.0, max_blocks * 16)
+    cos, sin = torch.from_numpy(cos).to(DEV), torch.from_numpy(sin).to(DEV)
+    table = torch.tensor(table, device=DEV)
+    k0 = synth.normal(13, f"ra.k{D}", (n_pages, Hkv, D // 32, 4, 16, 8), 1.0, torch.float16, DEV)
+    v0 = synth.normal(13, f"ra.v{D}", (n_pages, Hkv, D, 16), 1.0, torch.float16, DEV)
+    qkv = synth.normal(13, f"ra.q{D}.{Hq}", (B, Hq + 2 * Hkv, D), 1.0, torch.float16, DEV)
+    seqs = torch.tensor([0, 1, 2, 3, 4, 5, 99], dtype=torch.int32, device=DEV)      # the last row names no sequence
+    tpos = torch.tensor(pos, dtype=torch.int32, device=DEV)
+    ctx = tpos + 1
+    for frag in (False, True):
+        k1, v1, q1 = k0.clone(), v0.clone(), qkv.clone()
+        ops.rope_kv_append(q1, k1, v1, table, seqs, tpos, cos, sin, Hq, Hkv, D)
+        want = ops.paged_attn_decode(q1, k1, v1, table, seqs, ctx, Hq, Hkv, D, frag=frag)
+        k2, v2, q2 = k0.clone(), v0.clone(), qkv.clone()
+        got = ops.rope_attn_decode(q2, k2, v2, table, seqs, tpos, ctx, cos, sin, Hq, Hkv, D, frag=frag)
+        assert torch.equal(k1, k2) and torch.equal(v1, v2)
+        assert torch.equal(q2, qkv)
+        a, b_ = (got.unpack(), want.unpack()) if frag else (got, want)
+        assert torch.equal(a, b_)
+        assert float(a[:6].abs().max()) > 0 and float(a[6].abs().max()) == 0
