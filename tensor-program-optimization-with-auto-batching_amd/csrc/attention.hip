@@ -113,6 +113,59 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qk
   }
 }
 
+// Prefill-sized variant without LoRA: one workgroup of 256 threads per token walks all (head, pair) items of the
+// token, instead of one 64-thread workgroup per (token, head) - 96 times fewer workgroups at the 7B shape.  Same
+// arithmetic per element as rope_kv_append_kernel.
+__global__ __launch_bounds__(256) void rope_kv_append_rows_kernel(f16* __restrict__ qkv, f16* __restrict__ k_cache,
+                                                                  f16* __restrict__ v_cache,
+                                                                  const int32_t* __restrict__ block_table, int max_blocks,
+                                                                  const int32_t* __restrict__ tok_seq,
+                                                                  const int32_t* __restrict__ tok_pos,
+                                                                  const float* __restrict__ rope_cos,
+                                                                  const float* __restrict__ rope_sin, int max_pos, int Hq,
+                                                                  int Hkv, int D, int n_pages, int n_seq) {
+  const int t = blockIdx.x;
+  const int half = D >> 1;
+  const int seq = tok_seq[t], pos = tok_pos[t];
+  if (seq < 0 || seq >= n_seq || pos < 0 || pos >= max_pos || pos / PAGE >= max_blocks) return;
+  const int page = block_table[(size_t)seq * max_blocks + pos / PAGE];
+  const bool page_ok = page >= 0 && page < n_pages;
+  const int slot = pos % PAGE;
+  f16* row = qkv + (size_t)t * (Hq + 2 * Hkv) * D;
+  const int items = (Hq + 2 * Hkv) * half;
+  for (int it = threadIdx.x; it < items; it += 256) {
+    const int hh = it / half, i = it % half;
+    f16* src = row + (size_t)hh * D;
+    const f16 h1 = src[i], h2 = src[i + half];
+    if (hh >= Hq + Hkv) {
+      if (page_ok) {
+        f16* dst = v_cache + ((size_t)page * Hkv + (hh - Hq - Hkv)) * D * PAGE + slot;
+        dst[(size_t)i * PAGE] = h1;
+        dst[(size_t)(i + half) * PAGE] = h2;
+      }
+      continue;
+    }
+    const float c = rope_cos[(size_t)pos * half + i], s = rope_sin[(size_t)pos * half + i];
+    const float x1 = (float)h1, x2 = (float)h2;
+    float r1, r2;
+    {
+#pragma clang fp contract(off)
+      r1 = x1 * c - x2 * s;
+      r2 = x2 * c + x1 * s;
+    }
+    asm volatile("" : "+v"(r1), "+v"(r2));
+    const f16 o1 = (f16)r1, o2 = (f16)r2;
+    if (hh < Hq) {
+      src[i] = o1;
+      src[i + half] = o2;
+    } else if (page_ok) {
+      f16* dst = k_cache + ((size_t)page * Hkv + (hh - Hq)) * PAGE * D;
+      dst[k_page_offset(slot, i)] = o1;
+      dst[k_page_offset(slot, i + half)] = o2;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Decode: one workgroup (4 waves) per (sequence, kv head); the G = Hq / Hkv <= 16 query heads that share the
 // kv head are the 16 columns of the matrix-core tiles, so K and V are read once per group.  A wave takes
@@ -625,6 +678,12 @@ static int rope_kv_append_impl(const char* who, void* qkv, void* k_cache, void* 
   MLORA_CHECK(qkv && k_cache && v_cache && block_table && tok_seq && tok_pos && rope_cos && rope_sin, MLORA_ERR_INVALID, "%s: null pointer", who);
   MLORA_CHECK(T >= 0 && max_pos > 0, MLORA_ERR_INVALID, "%s: bad T=%d max_pos=%d", who, T, max_pos);
   if (T == 0) return MLORA_OK;
+  if (T > 64 && lx.src.v == nullptr) {
+    hipLaunchKernelGGL(rope_kv_append_rows_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, (f16*)qkv, (f16*)k_cache,
+                       (f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, rope_cos, rope_sin, max_pos, Hq, Hkv, D, n_pages,
+                       n_seq);
+    return mlora_launch_status(who);
+  }
   hipLaunchKernelGGL(rope_kv_append_kernel, dim3(T, Hq + 2 * Hkv), dim3(64), 0, (hipStream_t)stream, (f16*)qkv,
                      (f16*)k_cache, (f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, rope_cos, rope_sin,
                      max_pos, Hq, Hkv, D, n_pages, n_seq, T, lx);
