@@ -45,6 +45,46 @@ def test_argument_validation_without_gpu():
     assert lib.mlora_paged_attn_decode(1, 0, 1, 1, 1, 1, 4, 1, 1, 2, 8, 3, 128, 4, 2, None) == -1  # Hq % Hkv
 
 
+def test_argument_validation_of_fused_and_batched_entry_points():
+    """Every error below is detected on the host before a launch (pointers are dummies)."""
+    import ctypes as C
+    lm = load_pkg("_lib")
+    lib = lm.lib()
+    # multi-rank: bad rank in the second bucket is reported before the first bucket runs; workspace sized by the largest rank
+    bk = (lm.LoraBucket * 2)()
+    bk[0].A, bk[0].B, bk[0].r, bk[0].n_ad, bk[0].scaling = 1, 1, 16, 4, 0.5
+    bk[1].A, bk[1].B, bk[1].r, bk[1].n_ad, bk[1].scaling = 1, 1, 12, 4, 0.5
+    args = (1, 0, 64, 1, 0, C.cast(bk, C.c_void_p), 2, 1, 1, 8, 64, 64, 1, 1 << 20, None)
+    assert lib.mlora_gather_mm_multi(*args) == -2 and b"rank" in lib.mlora_last_error()
+    bk[1].r = 64
+    small = lib.mlora_gather_mm_workspace_bytes(8, 64, 16)
+    assert lib.mlora_gather_mm_multi(1, 0, 64, 1, 0, C.cast(bk, C.c_void_p), 2, 1, 1, 8, 64, 64, 1, small, None) == -3
+    bk[1].A = None
+    assert lib.mlora_gather_mm_multi(1, 0, 64, 1, 0, C.cast(bk, C.c_void_p), 2, 1, 1, 8, 64, 64, 1, 1 << 20, None) == -1   # one null table
+    assert lib.mlora_gather_mm_multi(1, 0, 64, 1, 0, None, 2, 1, 1, 8, 64, 64, 1, 1 << 20, None) == -1
+    # batched gather-matmul: decode shapes only
+    assert lib.mlora_gather_mm_batch(1, 4, 0, 64, 0, 1, 1.0, 65, 64, 64, 16, 2, None) == -2
+    assert lib.mlora_gather_mm_batch(None, 4, 0, 64, 0, 1, 1.0, 8, 64, 64, 16, 2, None) == -1
+    assert lib.mlora_gather_mm_batch(1, 0, 0, 64, 0, 1, 1.0, 8, 64, 64, 16, 2, None) == 0           # nothing to do
+    # fused decode attention
+    ra = lambda Hq, Hkv, D, B, lay: lib.mlora_rope_attn_decode(1, lay, 1, 1, 1, 1, 4, 1, 1, 1, 1, 1, 64, B, Hq, Hkv, D, 4, 2,
+                                                               None, 0, None, None, 0.0, 0, 0, 0, None)
+    assert ra(8, 8, 96, 2, 0) == -2                    # head_dim
+    assert ra(34, 2, 128, 2, 0) == -2                  # 17 query heads per kv head
+    assert ra(8, 8, 128, 65, 1) == -2                  # fragment-ordered output needs B <= 64
+    assert ra(8, 8, 128, 0, 0) == 0
+    assert lib.mlora_rope_attn_decode(1, 0, 1, 1, 1, 1, 4, 1, 1, 1, 1, 1, 64, 2, 8, 8, 128, 4, 2,
+                                      1, 1, None, None, 0.5, 64, 16, 2, None) == -1     # LoRA without B / ids
+    # SiLU epilogue GEMV and split GEMV
+    assert lib.mlora_gemv_frag_silu(1, 1, 1, 33, 64, 64, None) == -2
+    assert lib.mlora_gemv_frag_silu(1, 1, 1, 8, 64, 48, None) == -2
+    assert lib.mlora_gemv_frag_silu(None, 1, 1, 8, 64, 64, None) == -1
+    # decode step: a plan without layers / with a token count beyond the decode tile
+    plan = lm.DecodePlan()
+    assert lib.mlora_decode_step(C.byref(plan), None) < 0
+    assert lib.mlora_decode_step(None, None) == -1
+
+
 def test_ops_refuse_cpu_tensors():
     import torch
     ops = load_pkg("ops")
