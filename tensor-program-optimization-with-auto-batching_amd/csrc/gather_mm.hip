@@ -361,14 +361,15 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* 
                                                                             const int32_t* __restrict__ ids, float scaling,
                                                                             int T, int N, int ldy, int n_ad,
                                                                             const int32_t* __restrict__ bucket_of, int bucket,
-                                                                            int splits) {
+                                                                            int splits, int nit) {
   constexpr int KS = (R + 31) / 32;     // k-steps of 32 rank entries (ranks 8 and 16: one partly filled step)
   constexpr int CT = 4;                 // 16-column tiles per wave
   constexpr int LD = 16 * CT + 4;       // padded row of the transposition buffer (floats): conflict-free both ways
   __shared__ float stage[SEG_WAVES][16][LD];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t0 = blockIdx.x * 16;
-  const int n0 = (blockIdx.y * SEG_WAVES + wave) * 16 * CT;
+  // a workgroup covers nit consecutive blocks of 4 waves x 64 columns; the token tile of v stays in registers
+  const int nbase = blockIdx.y * nit * SEG_WAVES * 16 * CT + wave * 16 * CT;
   const int col = lane & 15, g = lane >> 4;
   const int tl = min(t0 + col, T - 1);
   const int raw = lora_token_id(ids, bucket_of, bucket, t0 + col, T);
@@ -405,12 +406,14 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* 
   }
   // write-back role of the lane: token lane / 4, the 16 columns of column tile lane % 4 (contiguous in y)
   const int wt = lane >> 2, wc = lane & 3;
-  const int nw = n0 + wc * 16;
-  YT* __restrict__ yrow = y + (size_t)(t0 + wt) * ldy + nw;
   int a;
   unsigned rows;
   while (next_tile_adapter(id, todo, a, rows)) {
     const f16* __restrict__ Ba = B + (size_t)a * N * R + g * 8;
+   for (int it = 0; it < nit; ++it) {
+    const int n0 = nbase + it * SEG_WAVES * 16 * CT;
+    const int nw = n0 + wc * 16;
+    YT* __restrict__ yrow = y + (size_t)(t0 + wt) * ldy + nw;
 #pragma unroll
     for (int c = 0; c < CT; ++c) {
       const int nb = n0 + c * 16;
@@ -443,6 +446,7 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* 
       }
     }
     __syncthreads();
+   }
   }
 }
 
@@ -615,13 +619,16 @@ static void gmm_segments_r(void* y, int y_dtype, int ldy, const f16* x, const f1
   if (splits < 1) splits = 1;
   hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles, splits), dim3(SEG_WAVES * WAVE), 0, s, v, x, A, ids, T, K, n_ad,
                      bf.bucket_of, bf.bucket);
-  const dim3 grid(tiles, ceil_div(N, SEG_WAVES * 64));
+  // column blocks per workgroup: as many as leave about a thousand workgroups (per-workgroup set-up amortised)
+  int nit = (int)(((long)tiles * ceil_div(N, SEG_WAVES * 64)) / 1024);
+  nit = nit < 1 ? 1 : (nit > 8 ? 8 : nit);
+  const dim3 grid(tiles, ceil_div(N, SEG_WAVES * 64 * nit));
   if (y_dtype == MLORA_F16)
     hipLaunchKernelGGL((lora_expand_mfma_kernel<R, f16>), grid, dim3(SEG_WAVES * WAVE), 0, s, (f16*)y, v, B, ids, scaling, T, N,
-                       ldy, n_ad, bf.bucket_of, bf.bucket, splits);
+                       ldy, n_ad, bf.bucket_of, bf.bucket, splits, nit);
   else
     hipLaunchKernelGGL((lora_expand_mfma_kernel<R, float>), grid, dim3(SEG_WAVES * WAVE), 0, s, (float*)y, v, B, ids, scaling, T,
-                       N, ldy, n_ad, bf.bucket_of, bf.bucket, splits);
+                       N, ldy, n_ad, bf.bucket_of, bf.bucket, splits, nit);
 }
 
 // shrink + expand on the matrix cores; v = workspace viewed as [T, r] fp32
