@@ -113,56 +113,115 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qk
   }
 }
 
-// Prefill-sized variant without LoRA: one workgroup of 256 threads per token walks all (head, pair) items of the
-// token, instead of one 64-thread workgroup per (token, head) - 96 times fewer workgroups at the 7B shape.  Same
-// arithmetic per element as rope_kv_append_kernel.
-__global__ __launch_bounds__(256) void rope_kv_append_rows_kernel(f16* __restrict__ qkv, f16* __restrict__ k_cache,
+// Prefill-sized variant that writes whole page rows: one workgroup per (16 consecutive tokens, head).  When the 16
+// tokens are slots 0..15 of one page (prompts that start on a page boundary), a K fragment row (16 tokens x 16 B) and
+// a V row (16 tokens of one dim, 32 B) are written as contiguous pieces instead of 2 bytes at a time; other tiles fall
+// back to element-wise writes.  Same arithmetic per element as rope_kv_append_kernel.
+template <int D>
+__global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restrict__ qkv, f16* __restrict__ k_cache,
                                                                   f16* __restrict__ v_cache,
                                                                   const int32_t* __restrict__ block_table, int max_blocks,
                                                                   const int32_t* __restrict__ tok_seq,
                                                                   const int32_t* __restrict__ tok_pos,
                                                                   const float* __restrict__ rope_cos,
                                                                   const float* __restrict__ rope_sin, int max_pos, int Hq,
-                                                                  int Hkv, int D, int n_pages, int n_seq) {
-  const int t = blockIdx.x;
-  const int half = D >> 1;
-  const int seq = tok_seq[t], pos = tok_pos[t];
-  if (seq < 0 || seq >= n_seq || pos < 0 || pos >= max_pos || pos / PAGE >= max_blocks) return;
-  const int page = block_table[(size_t)seq * max_blocks + pos / PAGE];
-  const bool page_ok = page >= 0 && page < n_pages;
-  const int slot = pos % PAGE;
-  f16* row = qkv + (size_t)t * (Hq + 2 * Hkv) * D;
-  const int items = (Hq + 2 * Hkv) * half;
-  for (int it = threadIdx.x; it < items; it += 256) {
-    const int hh = it / half, i = it % half;
-    f16* src = row + (size_t)hh * D;
-    const f16 h1 = src[i], h2 = src[i + half];
-    if (hh >= Hq + Hkv) {
-      if (page_ok) {
-        f16* dst = v_cache + ((size_t)page * Hkv + (hh - Hq - Hkv)) * D * PAGE + slot;
-        dst[(size_t)i * PAGE] = h1;
-        dst[(size_t)(i + half) * PAGE] = h2;
-      }
-      continue;
+                                                                  int Hkv, int n_pages, int n_seq, int T) {
+  constexpr int half = D / 2;
+  __shared__ int s_seq[16], s_pos[16];
+  __shared__ int s_aligned, s_page;
+  const int t0 = blockIdx.x * 16, hh = blockIdx.y;            // hh < Hq: a q head; else kv head hh - Hq (k and v)
+  const int HH = Hq + 2 * Hkv;
+  if (threadIdx.x < 16) {
+    const int t = t0 + threadIdx.x;
+    int seq = -1, pos = -1;
+    if (t < T) {
+      seq = tok_seq[t];
+      pos = tok_pos[t];
+      if (seq < 0 || seq >= n_seq || pos < 0 || pos >= max_pos || pos / PAGE >= max_blocks) seq = -1;
     }
-    const float c = rope_cos[(size_t)pos * half + i], s = rope_sin[(size_t)pos * half + i];
-    const float x1 = (float)h1, x2 = (float)h2;
-    float r1, r2;
+    s_seq[threadIdx.x] = seq;
+    s_pos[threadIdx.x] = pos;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    bool al = s_seq[0] >= 0 && (s_pos[0] % PAGE) == 0;
+    for (int i = 1; i < 16 && al; ++i) al = s_seq[i] == s_seq[0] && s_pos[i] == s_pos[0] + i;
+    int page = -1;
+    if (al) {
+      page = block_table[(size_t)s_seq[0] * max_blocks + s_pos[0] / PAGE];
+      if (page < 0 || page >= n_pages) al = false;
+    }
+    s_aligned = al;
+    s_page = page;
+  }
+  __syncthreads();
+  // rotation of one element d of a head row (x1 = first-half element, x2 = its partner in the second half)
+  auto rot = [&](float x1, float x2, float c, float s, bool second) -> f16 {
+    float r;
     {
 #pragma clang fp contract(off)
-      r1 = x1 * c - x2 * s;
-      r2 = x2 * c + x1 * s;
+      r = second ? x2 * c + x1 * s : x1 * c - x2 * s;
     }
-    asm volatile("" : "+v"(r1), "+v"(r2));
-    const f16 o1 = (f16)r1, o2 = (f16)r2;
-    if (hh < Hq) {
-      src[i] = o1;
-      src[i + half] = o2;
-    } else if (page_ok) {
-      f16* dst = k_cache + ((size_t)page * Hkv + (hh - Hq)) * PAGE * D;
-      dst[k_page_offset(slot, i)] = o1;
-      dst[k_page_offset(slot, i + half)] = o2;
+    asm volatile("" : "+v"(r));
+    return (f16)r;
+  };
+  if (hh < Hq) {                                              // q: rotate in place, 16 tokens x D/2 pairs
+    for (int it = threadIdx.x; it < 16 * half; it += 256) {
+      const int tk = it / half, i = it % half;
+      if (s_seq[tk] < 0) continue;
+      f16* src = qkv + ((size_t)(t0 + tk) * HH + hh) * D;
+      const float c = rope_cos[(size_t)s_pos[tk] * half + i], s = rope_sin[(size_t)s_pos[tk] * half + i];
+      const float x1 = (float)src[i], x2 = (float)src[i + half];
+      src[i] = rot(x1, x2, c, s, false);
+      src[i + half] = rot(x1, x2, c, s, true);
     }
+    return;
+  }
+  const int kh = hh - Hq;
+  if (s_aligned) {
+    const int page = s_page;
+    // K: one 16-byte fragment chunk (8 dims of one token) per item; 16 tokens of a chunk row are contiguous
+    for (int it = threadIdx.x; it < (D / 8) * 16; it += 256) {
+      const int tk = it & 15, ch = it >> 4;                   // ch = ks * 4 + g: dims 8 ch .. 8 ch + 7
+      const int d0 = ch * 8;
+      const bool second = d0 >= half;
+      const int p0 = second ? d0 - half : d0;                 // pair index of the first of the 8 dims
+      const f16* src = qkv + ((size_t)(t0 + tk) * HH + Hq + kh) * D;
+      const f16x8 lo = ld8(src + p0), hi = ld8(src + p0 + half);
+      const float* cp = rope_cos + (size_t)s_pos[tk] * half + p0;
+      const float* sp = rope_sin + (size_t)s_pos[tk] * half + p0;
+      f16x8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = rot((float)lo[e], (float)hi[e], cp[e], sp[e], second);
+      st8(k_cache + ((size_t)page * Hkv + kh) * PAGE * D + ((size_t)ch * 16 + tk) * 8, o);
+    }
+    // V: 8 tokens of one dim per item (16 bytes of the dim's 32-byte row)
+    for (int it = threadIdx.x; it < D * 2; it += 256) {
+      const int d = it % D, tg = it / D;
+      f16x8 o;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = qkv[((size_t)(t0 + tg * 8 + j) * HH + Hq + Hkv + kh) * D + d];
+      st8(v_cache + (((size_t)page * Hkv + kh) * D + d) * PAGE + tg * 8, o);
+    }
+    return;
+  }
+  for (int it = threadIdx.x; it < 16 * half; it += 256) {      // element-wise: tokens of several pages or sequences
+    const int tk = it / half, i = it % half;
+    if (s_seq[tk] < 0) continue;
+    const int pos = s_pos[tk];
+    const int page = block_table[(size_t)s_seq[tk] * max_blocks + pos / PAGE];
+    if (page < 0 || page >= n_pages) continue;
+    const int slot = pos % PAGE;
+    const f16* ksrc = qkv + ((size_t)(t0 + tk) * HH + Hq + kh) * D;
+    const f16* vsrc = qkv + ((size_t)(t0 + tk) * HH + Hq + Hkv + kh) * D;
+    const float c = rope_cos[(size_t)pos * half + i], s = rope_sin[(size_t)pos * half + i];
+    const float x1 = (float)ksrc[i], x2 = (float)ksrc[i + half];
+    f16* kd = k_cache + ((size_t)page * Hkv + kh) * PAGE * D;
+    kd[k_page_offset(slot, i)] = rot(x1, x2, c, s, false);
+    kd[k_page_offset(slot, i + half)] = rot(x1, x2, c, s, true);
+    f16* vd = v_cache + ((size_t)page * Hkv + kh) * D * PAGE + slot;
+    vd[(size_t)i * PAGE] = vsrc[i];
+    vd[(size_t)(i + half) * PAGE] = vsrc[i + half];
   }
 }
 
@@ -679,9 +738,15 @@ static int rope_kv_append_impl(const char* who, void* qkv, void* k_cache, void* 
   MLORA_CHECK(T >= 0 && max_pos > 0, MLORA_ERR_INVALID, "%s: bad T=%d max_pos=%d", who, T, max_pos);
   if (T == 0) return MLORA_OK;
   if (T > 64 && lx.src.v == nullptr) {
-    hipLaunchKernelGGL(rope_kv_append_rows_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, (f16*)qkv, (f16*)k_cache,
-                       (f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, rope_cos, rope_sin, max_pos, Hq, Hkv, D, n_pages,
-                       n_seq);
+    const dim3 grid(ceil_div(T, 16), Hq + Hkv);
+    if (D == 128)
+      hipLaunchKernelGGL(rope_kv_append_tile_kernel<128>, grid, dim3(256), 0, (hipStream_t)stream, (f16*)qkv, (f16*)k_cache,
+                         (f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, rope_cos, rope_sin, max_pos, Hq, Hkv, n_pages,
+                         n_seq, T);
+    else
+      hipLaunchKernelGGL(rope_kv_append_tile_kernel<64>, grid, dim3(256), 0, (hipStream_t)stream, (f16*)qkv, (f16*)k_cache,
+                         (f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, rope_cos, rope_sin, max_pos, Hq, Hkv, n_pages,
+                         n_seq, T);
     return mlora_launch_status(who);
   }
   hipLaunchKernelGGL(rope_kv_append_kernel, dim3(T, Hq + 2 * Hkv), dim3(64), 0, (hipStream_t)stream, (f16*)qkv,

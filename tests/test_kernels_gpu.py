@@ -547,3 +547,41 @@ def test_rope_attn_decode_one_launch_equals_two(ops, synth, Hq, Hkv, D):
         a, b_ = (got.unpack(), want.unpack()) if frag else (got, want)
         assert torch.equal(a, b_)
         assert float(a[:6].abs().max()) > 0 and float(a[6].abs().max()) == 0
+
+
+@pytest.mark.parametrize("Hq,Hkv,D", [(4, 4, 128), (8, 2, 64)])
+def test_rope_append_page_row_writer_equals_per_token_kernel(ops, synth, Hq, Hkv, D):
+    """T > 64 takes the kernel that writes whole page rows for page-aligned token tiles: q, K cache and V cache are
+    bit-identical to the per-token kernel run over chunks of at most 64 tokens.  Sequences start on and off a
+    16-token boundary, one ends inside a tile, one token row is invalid."""
+    kvm = load_pkg("kv_cache")
+    lens = [64, 36, 21, 48]                       # token offsets 0, 64, 100, 121: the last two are not tile-aligned
+    T = sum(lens)
+    n_pages, max_blocks = 16, 4
+    perm = synth.permutation(17, "rw.pages", n_pages)
+    table = np.full((len(lens), max_blocks), -1, dtype=np.int32)
+    o = 0
+    for s, n in enumerate(lens):
+        nb = -(-n // 16)
+        table[s, :nb] = perm[o:o + nb]
+        o += nb
+    tseq = np.repeat(np.arange(len(lens)), lens).astype(np.int32)
+    tpos = np.concatenate([np.arange(n) for n in lens]).astype(np.int32)
+    tseq[70] = -1                                 # a token that belongs to no sequence
+    cos, sin = kvm.rope_tables(D, 10000.0, max_blocks * 16)
+    cos, sin = torch.from_numpy(cos).to(DEV), torch.from_numpy(sin).to(DEV)
+    table = torch.tensor(table, device=DEV)
+    qkv = synth.normal(17, f"rw.qkv{D}", (T, Hq + 2 * Hkv, D), 1.0, torch.float16, DEV)
+    k0 = torch.zeros((n_pages, Hkv, D // 32, 4, 16, 8), dtype=torch.float16, device=DEV)
+    v0 = torch.zeros((n_pages, Hkv, D, 16), dtype=torch.float16, device=DEV)
+    q1, k1, v1 = qkv.clone(), k0.clone(), v0.clone()
+    ops.rope_kv_append(q1, k1, v1, table, torch.tensor(tseq, device=DEV), torch.tensor(tpos, device=DEV), cos, sin, Hq, Hkv, D)
+    q2, k2, v2 = qkv.clone(), k0.clone(), v0.clone()
+    for lo in range(0, T, 50):
+        hi = min(T, lo + 50)
+        part = q2[lo:hi].clone()
+        ops.rope_kv_append(part, k2, v2, table, torch.tensor(tseq[lo:hi], device=DEV), torch.tensor(tpos[lo:hi], device=DEV),
+                           cos, sin, Hq, Hkv, D)
+        q2[lo:hi] = part
+    assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    assert torch.equal(q1[70], qkv[70]) and float(k1.abs().sum()) > 0
