@@ -162,13 +162,15 @@ __device__ __forceinline__ float row_dot(const f16x8 (&bv)[R / 8], const float* 
   return g[0];
 }
 
-template <int R, typename YT>
-__global__ __launch_bounds__(GMM_THREADS) void gather_mm_decode_kernel(GmmSet one, const GmmSet* __restrict__ sets,
+// GR: rows of A a wave reduces together.  16 reads x once per 16 rows (shortest single problem); 8 keeps the kernel
+// under 128 VGPRs, i.e. two workgroups per CU, which is what a launch over many problems wants.  Same result bits.
+template <int R, typename YT, int GR>
+__global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_decode_kernel(GmmSet one, const GmmSet* __restrict__ sets,
                                                                         const int32_t* __restrict__ ids, float scaling,
                                                                         int T, int K, int N, int n_ad, int ldy,
                                                                         int frag_tt, int P, int ci_n, int kc,
                                                                         const int32_t* __restrict__ bucket_of, int bucket) {
-  constexpr int G = R < 16 ? R : 16;         // rows of A reduced together
+  constexpr int G = R < GR ? R : GR;         // rows of A reduced together
   constexpr int NG = R / 8;
   extern __shared__ float lds[];             // part [kc][T][R], then v [T][R]
   float* part = lds;
@@ -561,10 +563,18 @@ static void gmm_launch_r(const GmmSet& one, const GmmSet* sets, dim3 grid, size_
                          float scaling, int T, int K, int N, int n_ad, int ldy, int frag_tt, int P, LoraKSplit ks, hipStream_t s,
                          BucketFilter bf) {
   const dim3 block(GMM_THREADS);
-  if (y_dtype == MLORA_F16)
-    hipLaunchKernelGGL((gather_mm_decode_kernel<R, f16>), grid, block, lds, s, one, sets, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks.ci, ks.kc, bf.bucket_of, bf.bucket);
-  else
-    hipLaunchKernelGGL((gather_mm_decode_kernel<R, float>), grid, block, lds, s, one, sets, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks.ci, ks.kc, bf.bucket_of, bf.bucket);
+#define MLORA_GMM_LAUNCH(YT, GR)                                                                                              \
+  hipLaunchKernelGGL((gather_mm_decode_kernel<R, YT, GR>), grid, block, lds, s, one, sets, ids, scaling, T, K, N, n_ad, ldy, \
+                     frag_tt, P, ks.ci, ks.kc, bf.bucket_of, bf.bucket)
+  const bool many = grid.y > 1;
+  if (y_dtype == MLORA_F16) {
+    if (many) MLORA_GMM_LAUNCH(f16, 8);
+    else MLORA_GMM_LAUNCH(f16, 16);
+  } else {
+    if (many) MLORA_GMM_LAUNCH(float, 8);
+    else MLORA_GMM_LAUNCH(float, 16);
+  }
+#undef MLORA_GMM_LAUNCH
 }
 
 static int gmm_one_launch(const GmmSet& one, const GmmSet* sets, int n_sets, int y_dtype, int ldy, int x_layout,
