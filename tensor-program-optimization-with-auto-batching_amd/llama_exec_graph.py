@@ -3,7 +3,8 @@
 Restates `tvm/llama_auto_batcher/llama_exec_graph.py:10-174`.  Differences that do not change results:
 the argmax runs on the device and only the token ids cross to the host (the reference copies the full
 fp32 logits and calls np.argmax, `:92,134-137`; ties resolve to the lowest index in both); prompts may be
-given as token-id arrays when no tokenizer is configured.
+given as token-id arrays when no tokenizer is configured; decode batches of a single adapter type run through the
+native decode step (bit-identical tokens, see LlamaExecConfig.native_decode).
 """
 from __future__ import annotations
 
@@ -22,6 +23,10 @@ class LlamaExecConfig:
     max_prompt_len: int
     max_gen_len: int
     page_size: int
+    # Run decode batches of one adapter type (or none) and at most 64 sequences through the native decode step (one
+    # C call per step, graph replay when several steps lie ahead) instead of one call per operator.  Same tokens:
+    # the native step with ids-based LoRA shrink is bit-identical to the per-operator path.
+    native_decode: bool = True
 
 
 class LlamaExecGraph(ExecGraph):
@@ -120,9 +125,13 @@ class LlamaExecGraph(ExecGraph):
         # the first token (from prefill) already counts towards max_gen_len (`:94-100`)
         seqs = self.check_seqs_finished(seqs, outputs)
         while seqs:
+            method, params = self.seq_info.get_decode_method(seqs)
+            single = method == "decode_no_adapter" or method.startswith("decode_a")
+            if getattr(self.exec_config, "native_decode", False) and single and len(seqs) <= 64:
+                seqs = self._decode_native(seqs, outputs, method, params)
+                continue
             tokens = torch.tensor([outputs[sid][-1] for sid in seqs], dtype=torch.int32)
             hidden = self.vm["embed"](tokens)
-            method, params = self.seq_info.get_decode_method(seqs)
             ev = self._tic()
             self.kv_cache.begin_forward(seqs, [1] * len(seqs))
             logits, _ = self.vm[method](hidden, self.kv_cache, *params)
@@ -134,6 +143,34 @@ class LlamaExecGraph(ExecGraph):
             seqs = self.check_seqs_finished(seqs, outputs)
         for i, sid in enumerate(ordered):
             op.output_vars[original_positions[i]].var = np.asarray(outputs[sid], dtype=np.int64)
+
+    def _decode_native(self, seqs, outputs, method, params):
+        """Decode this batch with the native step until its composition changes (a sequence reaches its length
+        limit or emits EOS); returns the sequences still running.  Without an EOS id the number of steps until
+        the next length limit is known in advance and the tokens come back in one copy."""
+        from .decode_session import NativeDecodeSession
+        tid = int(method[len("decode_a"):]) if method != "decode_no_adapter" else 0
+        wids = params[0] if params else None
+        last = [outputs[sid][-1] for sid in seqs]
+        ahead = min(self.seq_info.get_max_gen_len(sid) - len(outputs[sid]) for sid in seqs)
+        sess = NativeDecodeSession(self.vm, self.kv_cache, seqs, wids, last, tid=tid, use_graph=ahead >= 8, dense_lora=False)
+        if self.eos_token_id is None and not self.measure:
+            for _ in range(ahead):
+                sess.step(keep_history=True)
+            toks = torch.stack(sess.history).cpu().numpy()             # [ahead, batch]
+            for i, sid in enumerate(seqs):
+                outputs[sid].extend(int(t) for t in toks[:, i])
+            return self.check_seqs_finished(seqs, outputs)
+        while True:
+            ev = self._tic()
+            nxt = sess.step()
+            self._toc(ev)
+            nxt = nxt.cpu().numpy()
+            for i, sid in enumerate(seqs):
+                outputs[sid].append(int(nxt[i]))
+            left = self.check_seqs_finished(seqs, outputs)
+            if len(left) != len(seqs):
+                return left
 
     def execute_decode_answer(self, op):
         assert len(op.input_vars) == 1 and len(op.output_vars) == 1 and len(op.seqids) == 1, \

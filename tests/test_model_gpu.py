@@ -209,3 +209,27 @@ def test_adapters_loaded_from_files_and_weight_id_translation(tmp_path):
     # the adapters must matter: dropping them changes at least one request's tokens
     base, _, _ = oracle.greedy_generate_ref(ref, prompts, {}, max_gen_len, n_pages, 16, None, return_logits=True)
     assert any(base[b] != exp[b] for b in (0, 2, 3, 4))
+
+
+def test_front_end_native_decode_equals_per_operator_decode(c1):
+    """The auto-batching front end gives the same token ids whether a decode batch runs through the native decode
+    step or through one call per operator: with and without an EOS id, with per-request length limits (the batch
+    shrinks and a new native session starts), and with a batch that holds requests without adapter."""
+    wl, model, prompts = c1
+    synth = load_pkg("synth")
+    perm = synth.permutation(9, "c1.pages.native", n_pages_for(wl, 12))
+    ids = wl.adapter_ids
+    for kwargs in ({}, {"max_gen_lens": [12, 5, 9, 3]}, {"eos_token_id": None, "max_gen_lens": [4, 4, 11, 11]}):
+        a, _ = run_hip_generate(model, wl, prompts, ids, 12, perm, native_decode=False, **kwargs)
+        b, _ = run_hip_generate(model, wl, prompts, ids, 12, perm, native_decode=True, **kwargs)
+        assert a == b
+    # an EOS id that one request emits early: take it from the free-running output
+    base, _ = run_hip_generate(model, wl, prompts, ids, 12, perm, native_decode=False)
+    eos = base[2][4]
+    a, _ = run_hip_generate(model, wl, prompts, ids, 12, perm, native_decode=False, eos_token_id=eos)
+    b, _ = run_hip_generate(model, wl, prompts, ids, 12, perm, native_decode=True, eos_token_id=eos)
+    assert a == b and len(a[2]) <= 5
+    none = np.array([-1, -1, -1, -1], dtype=np.int32)
+    a, _ = run_hip_generate(model, wl, prompts, none, 8, perm, native_decode=False)
+    b, _ = run_hip_generate(model, wl, prompts, none, 8, perm, native_decode=True)
+    assert a == b
