@@ -157,6 +157,30 @@ def gather_mm_timing(n_sets=128):
                                         "frac_of_hbm_peak": by * n_sets / bsec / 1e9 / HBM_PEAK_GBS}}
 
 
+def gather_mm_cpu_baseline(reps=20):
+    """The isolated gather-matmul on the host cores, in the reference's two forms (fp32, the oracle's restatements):
+    GatherBMM (stack the per-request A and scaled B, two batched matmuls, add - `lora_gatherbmm_linear_layer.py:14-20`)
+    and sequential (requests sorted by adapter, one matmul pair per adapter - `single_rank.py:39-50`)."""
+    import torch
+    import oracle
+    synth = _mod("synth")
+    c = synth.gather_mm_case(seed=1, T=64, K=4096, N=4096, r=16, n_ad=32, device="cpu")
+    x, A, B, y = (c[k].float().numpy() for k in ("x", "A", "B", "y"))
+    ids = c["ids"].numpy()
+    order = np.argsort(ids, kind="stable")
+    out = {}
+    for name, fn in (("gather_bmm", lambda: oracle.gather_bmm_hf_ref(y[:, None, :], x[:, None, :], A, B, ids, 1.0)),
+                     ("sequential", lambda: oracle.lora_sequential_ref(y[order], x[order], A, B, ids[order], 1.0))):
+        fn()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        out[name + "_us_per_call"] = (time.perf_counter() - t0) / reps * 1e6
+    out["cores"] = os.cpu_count()
+    out["kind"] = "port"
+    return out
+
+
 def cpu_baseline(wl, ctx, layers=2, steps=3):
     """The numpy oracle (fp32) on the host cores: `layers` of the 32 layers, `steps` decode steps of the
     whole batch at context `ctx` with a pre-filled cache, plus lm_head; scaled to the full depth."""
@@ -409,6 +433,8 @@ def main():
         out["gather_matmul"] = gather_mm_timing()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl, ctx0)
+        if "gather_matmul" in out:
+            out["gather_matmul"]["cpu_baseline"] = gather_mm_cpu_baseline()
     print(json.dumps(out))
 
 
