@@ -63,8 +63,8 @@ def profiled_gemv_traffic():
 def gemv_event_timing(model, T, reps=3):
     """Average duration of the weight-streaming GEMV over exactly the launches of one decode step (per layer: qkv with
     the adapters' A rows appended, o with A rows appended accumulating into the residual, gate/up with the SiLU
-    epilogue, down accumulating; then lm_head: 129 launches on 129 distinct matrices), issued back to back as in a
-    decode step and bracketed by one event pair on the launch stream."""
+    epilogue, down accumulating - o and down with their K split; then lm_head: 129 launches on 129 distinct matrices),
+    issued back to back as in a decode step and bracketed by one event pair on the launch stream."""
     import torch
     ops, lm = _mod("ops"), _mod("_lib")
     lib = lm.lib()
@@ -88,6 +88,9 @@ def gemv_event_timing(model, T, reps=3):
     H, I, Q, QKV = s.hidden_size, s.intermediate_size, s.q_size, s.q_size + 2 * s.kv_size
     launches, total_bytes = [], 0
     st = torch.cuda.current_stream().cuda_stream        # the stream the events below are recorded on
+    # o and down split K over several workgroups as in the decode step; the partial results go to `part`
+    ks_o, ks_d = lib.mlora_gemv_ksplit(T, Q, H + n_ext), lib.mlora_gemv_ksplit(T, I, H)
+    part = torch.empty(3 * T * (H + n_ext), dtype=torch.float32, device=dev)
 
     def add(fn, rows, K, out_bytes):
         nonlocal total_bytes
@@ -101,12 +104,14 @@ def gemv_event_timing(model, T, reps=3):
         add(lambda wq=wq, q_ext=q_ext: lib.mlora_gemv_frag_split(qkv.data_ptr(), F16, STORE, y2.data_ptr(), x_h.data.data_ptr(),
                                                                  wq.data.data_ptr(), T, H, QKV, q_ext, st),
             wq.N, H, T * QKV * 2 + T * q_ext * 4)
-        add(lambda wo=wo, o_ext=o_ext: lib.mlora_gemv_frag_split(resid.data_ptr(), F32, ACC, y2.data_ptr(), x_q.data.data_ptr(),
-                                                                 wo.data.data_ptr(), T, Q, H, o_ext, st),
+        add(lambda wo=wo, o_ext=o_ext: lib.mlora_gemv_frag_acc_ksplit(resid.data_ptr(), y2.data_ptr(), part.data_ptr(), ks_o,
+                                                                      x_q.data.data_ptr(), wo.data.data_ptr(), T, Q, H, o_ext,
+                                                                      None, None, 0, None, 0, 0, st),
             wo.N, Q, T * H * 8 + T * o_ext * 4)
         add(lambda wg=wg: lib.mlora_gemv_frag_silu(act.data.data_ptr(), x_h.data.data_ptr(), wg.data.data_ptr(), T, H, I, st),
             2 * I, H, T * I * 2)
-        add(lambda wd=wd: lib.mlora_gemv_frag(resid.data_ptr(), F32, ACC, x_i.data.data_ptr(), wd.data.data_ptr(), T, I, H, st),
+        add(lambda wd=wd: lib.mlora_gemv_frag_acc_ksplit(resid.data_ptr(), None, part.data_ptr(), ks_d, x_i.data.data_ptr(),
+                                                         wd.data.data_ptr(), T, I, H, 0, None, None, 0, None, 0, 0, st),
             H, I, T * H * 8)
     add(lambda: lib.mlora_gemv_frag(logits.data_ptr(), F32, STORE, x_h.data.data_ptr(), model.lm_head.data.data_ptr(), T, H,
                                     s.vocab_size, st), s.vocab_size, H, T * s.vocab_size * 4)

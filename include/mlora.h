@@ -281,6 +281,38 @@ int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v
                               int T, int H, int K, int r, int n_ad, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * K split of the accumulating decode GEMV over a narrow weight (o_proj, down_proj: 256 row tiles give one
+ * workgroup per compute unit only at one tile each, which makes every workgroup read the whole token block for 16
+ * rows).  With a split, a workgroup takes four row tiles and 1/ks of K; slice 0 accumulates into y as usual and
+ * slices 1..ks-1 store fp32 partial results that the next reader of y adds in slice order - in the decoder layer
+ * that reader is always an RMSNorm, so the sum is formed there and no extra pass or atomics are needed
+ * (results do not depend on scheduling).
+ *   mlora_gemv_ksplit          - the number of slices (1..4) this library uses for (T, K, N_total); 1 = no split;
+ *   mlora_gemv_ksplit_bytes    - size of the partials buffer, part [ks-1][T][N_total] fp32;
+ *   mlora_gemv_frag_acc_ksplit - y[T, N_main] (fp32) += xf . Wp^T over slice 0, partials of the other slices to
+ *                                `part`.  N_ext > 0: appended rows as in mlora_gemv_frag_split (their slice-0 result
+ *                                goes to y2 [T, N_ext], their partials to columns N_main.. of `part`).  A != NULL
+ *                                (N_ext must be 0): shrink partials of n_proj projections as in
+ *                                mlora_gemv_frag_lora.  ks = 1 needs no `part` and equals the unsplit calls.
+ *   mlora_rmsnorm_ksplit       - resid[t, :] (+= LoRA expand as in mlora_lora_expand_rmsnorm when B != NULL)
+ *                                += part[0][t, :H] + ... + part[ks-2][t, :H], stored back, then y = RMSNorm(resid).
+ *                                ld_part = N_total of the GEMV that wrote `part`; with v_dense = 1 the shrink results
+ *                                are y2 plus columns H.. of the partials.
+ * These replace the same reference operators as mlora_gemv_frag (llama_for_causal_lm.py:31-33,44-47, the o_proj and
+ * down_proj linears with the residual add of :79-84) and mlora_rmsnorm (:76-77).
+ * ------------------------------------------------------------------------------------------- */
+int mlora_gemv_ksplit(int T, int K, int N_total);
+size_t mlora_gemv_ksplit_bytes(int T, int N_total, int ks);
+int mlora_gemv_frag_acc_ksplit(float* y, float* y2, float* part, int ks, const void* xf, const void* Wp,
+                               int T, int K, int N_main, int N_ext,
+                               void* v_part, const void* const* A, int n_proj, const int32_t* tok_adapter, int r, int n_ad,
+                               void* stream);
+int mlora_rmsnorm_ksplit(void* y, int y_layout, float* resid, const float* part, int ks, int ld_part,
+                         const void* w, float eps, int T, int H,
+                         const void* v_part, int v_dense, const void* B, const int32_t* tok_adapter, float scaling,
+                         int K, int r, int n_ad, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * One decode step of the whole model, enqueued by one call.
  * Replaces: the body of the reference's hot loop between kv_state_begin_forward and the argmax
  *   (tvm/llama_auto_batcher/llama_exec_graph.py:110-137): vm["embed"], vm["decode_*"] over all layers
@@ -352,6 +384,8 @@ typedef struct mlora_decode_plan {
   float* logits;
   void* lora_ws;
   size_t lora_ws_bytes;
+  float* ksplit_ws;           /* partials of the K-split o_proj / down_proj GEMVs, or NULL (no split) */
+  size_t ksplit_ws_bytes;     /* >= mlora_gemv_ksplit_bytes over both projections (with their appended rows) */
 } mlora_decode_plan;
 
 int mlora_decode_step(const mlora_decode_plan* plan, void* stream);

@@ -44,6 +44,10 @@ SIGNATURES = {
     "mlora_gemv_frag_split": (_i, [_p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _p]),
     "mlora_rope_kv_append_lora": (_i, [_p, _p, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p]),
     "mlora_rope_attn_decode": (_i, [_p, _i, _p, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p]),
+    "mlora_gemv_ksplit": (_i, [_i, _i, _i]),
+    "mlora_gemv_ksplit_bytes": (_z, [_i, _i, _i]),
+    "mlora_gemv_frag_acc_ksplit": (_i, [_p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _p, _p, _i, _p, _i, _i, _p]),
+    "mlora_rmsnorm_ksplit": (_i, [_p, _i, _p, _p, _i, _i, _p, _f, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p]),
     "mlora_lora_expand_rmsnorm": (_i, [_p, _i, _p, _p, _i, _p, _p, _f, _p, _f, _i, _i, _i, _i, _i, _p]),
     "mlora_rmsnorm": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _p]),
     "mlora_silu_mul": (_i, [_p, _i, _p, _p, _i, _i, _i, _p]),
@@ -77,7 +81,7 @@ class DecodePlan(C.Structure):
                 ("block_table", _p), ("max_blocks", _i), ("n_pages", _i), ("n_seq", _i),
                 ("T", _i), ("tokens", _p), ("rows", _p), ("pos", _p), ("ctx", _p), ("tok_adapter", _p),
                 ("resid", _p), ("xn", _p), ("qkv", _p), ("attn", _p), ("gate_up", _p), ("act", _p), ("logits", _p),
-                ("lora_ws", _p), ("lora_ws_bytes", _z)]
+                ("lora_ws", _p), ("lora_ws_bytes", _z), ("ksplit_ws", _p), ("ksplit_ws_bytes", _z)]
 
 
 SIGNATURES["mlora_decode_step"] = (_i, [C.POINTER(DecodePlan), _p])

@@ -47,20 +47,39 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
     if (!lora || !lp.A) return MLORA_OK;
     return mlora_gather_mm(y, y_dtype, ldy, x, MLORA_FRAG, lp.A, lp.B, p->tok_adapter, sc, T, K, N, r, n_ad, ws_down, slot, stream);
   };
-  // RMSNorm of the residual stream, applying a pending down_proj expand of the previous layer first
-  const void* pending_B = nullptr;
-  auto norm = [&](const void* w) -> int {
-    if (pending_B) {
-      const void* B = pending_B;
-      pending_B = nullptr;
-      return mlora_lora_expand_rmsnorm(p->xn, MLORA_FRAG, p->resid, ws_down, dense, B, p->tok_adapter, sc, w, p->eps, T, H, I, r, n_ad, stream);
-    }
+  // K split of the two narrow accumulating GEMVs: the slices' partials are summed by the RMSNorm that reads the
+  // residual next.  N_total counts the appended adapter rows of the dense shrink.
+  auto ksplit_of = [&](int K, bool has_lora) -> int {
+    const int n_total = H + (dense && has_lora ? n_ad * r : 0);
+    const int ks = p->ksplit_ws ? mlora_gemv_ksplit(T, K, n_total) : 1;
+    return ks > 1 && mlora_gemv_ksplit_bytes(T, n_total, ks) <= p->ksplit_ws_bytes ? ks : 1;
+  };
+  // o_proj / down_proj: resid += x . W^T with the adapter's shrink riding along (dense: appended rows; else shrink units)
+  auto acc_gemv = [&](const void* x, const void* Wp, int K, const mlora_lora_proj& lp, void* v_ws, int ks) -> int {
+    const bool has = lora && lp.A;
+    const void* A1[1] = {lp.A};
+    if (has && dense)
+      return mlora_gemv_frag_acc_ksplit(p->resid, (float*)v_ws, p->ksplit_ws, ks, x, Wp, T, K, H, n_ad * r, nullptr, nullptr, 0,
+                                        nullptr, 0, 0, stream);
+    if (has)
+      return mlora_gemv_frag_acc_ksplit(p->resid, nullptr, p->ksplit_ws, ks, x, Wp, T, K, H, 0, v_ws, A1, 1, p->tok_adapter, r, n_ad,
+                                        stream);
+    return mlora_gemv_frag_acc_ksplit(p->resid, nullptr, p->ksplit_ws, ks, x, Wp, T, K, H, 0, nullptr, nullptr, 0, nullptr, 0, 0, stream);
+  };
+  // RMSNorm of the residual stream, first applying the pending expand and K-split partials of the GEMV before it
+  auto norm = [&](const void* w, const void* B, const void* v_ws, int K, int ks) -> int {
+    const int ld_part = H + (dense && B ? n_ad * r : 0);
+    if (B || ks > 1)
+      return mlora_rmsnorm_ksplit(p->xn, MLORA_FRAG, p->resid, p->ksplit_ws, ks, ld_part, w, p->eps, T, H, B ? v_ws : nullptr, dense, B,
+                                  p->tok_adapter, sc, K, r, n_ad, stream);
     return mlora_rmsnorm(p->xn, MLORA_FRAG, p->resid, MLORA_F32, w, p->eps, T, H, stream);
   };
+  const void* pending_B = nullptr;    // down_proj expand and partials of the previous layer
+  int pending_ks = 1;
   STEP(mlora_embed(p->resid, MLORA_F32, p->embed, p->tokens, T, H, p->vocab, stream));
   for (int l = 0; l < p->n_layers; ++l) {
     const mlora_layer& L = p->layers[l];
-    STEP(norm(L.ln1));
+    STEP(norm(L.ln1, pending_B, ws_down, I, pending_ks));
     const bool qkv_lora = lora && (L.lora[MLORA_Q].A || L.lora[MLORA_K].A || L.lora[MLORA_V].A);
     if (qkv_lora) {
       const void* A3[3] = {L.lora[MLORA_Q].A, L.lora[MLORA_K].A, L.lora[MLORA_V].A};
@@ -77,16 +96,10 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
                                   p->ctx, p->rope_cos, p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, nullptr, 0,
                                   nullptr, nullptr, 0.f, 0, 0, 0, stream));
     }
-    if (lora && L.lora[MLORA_O].A) {
-      const void* A1[1] = {L.lora[MLORA_O].A};
-      if (dense) STEP(mlora_gemv_frag_split(p->resid, MLORA_F32, MLORA_ACCUMULATE, (float*)ws_o, p->attn, L.o_p, T, q_sz, H, n_ad * r, stream));
-      else STEP(mlora_gemv_frag_lora(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->attn, L.o_p, T, q_sz, H, ws_o, A1, 1, p->tok_adapter, r, n_ad, stream));
-      STEP(mlora_lora_expand_rmsnorm(p->xn, MLORA_FRAG, p->resid, ws_o, dense, L.lora[MLORA_O].B, p->tok_adapter, sc, L.ln2, p->eps, T, H,
-                                     q_sz, r, n_ad, stream));
-    } else {
-      STEP(mlora_gemv_frag(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->attn, L.o_p, T, q_sz, H, stream));
-      STEP(mlora_rmsnorm(p->xn, MLORA_FRAG, p->resid, MLORA_F32, L.ln2, p->eps, T, H, stream));
-    }
+    const bool o_lora = lora && L.lora[MLORA_O].A;
+    const int ks_o = ksplit_of(q_sz, o_lora);
+    STEP(acc_gemv(p->attn, L.o_p, q_sz, L.lora[MLORA_O], ws_o, ks_o));
+    STEP(norm(L.ln2, o_lora ? L.lora[MLORA_O].B : nullptr, ws_o, q_sz, ks_o));
     const bool gu_lora = lora && (L.lora[MLORA_GATE].A || L.lora[MLORA_UP].A);
     if (L.gate_up_il_p && !gu_lora && T <= 32) {
       STEP(mlora_gemv_frag_silu(p->act, p->xn, L.gate_up_il_p, T, H, I, stream));
@@ -97,16 +110,12 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
       STEP(delta(gu + I, MLORA_F16, 2 * I, p->xn, L.lora[MLORA_UP], H, I));
       STEP(mlora_silu_mul(p->act, MLORA_FRAG, gu, gu + I, 2 * I, T, I, stream));
     }
-    if (lora && L.lora[MLORA_DOWN].A) {
-      const void* A1[1] = {L.lora[MLORA_DOWN].A};
-      if (dense) STEP(mlora_gemv_frag_split(p->resid, MLORA_F32, MLORA_ACCUMULATE, (float*)ws_down, p->act, L.down_p, T, I, H, n_ad * r, stream));
-      else STEP(mlora_gemv_frag_lora(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->act, L.down_p, T, I, H, ws_down, A1, 1, p->tok_adapter, r, n_ad, stream));
-      pending_B = L.lora[MLORA_DOWN].B;   // expanded inside the next RMSNorm launch
-    } else {
-      STEP(mlora_gemv_frag(p->resid, MLORA_F32, MLORA_ACCUMULATE, p->act, L.down_p, T, I, H, stream));
-    }
+    const bool down_lora = lora && L.lora[MLORA_DOWN].A;
+    pending_ks = ksplit_of(I, down_lora);
+    STEP(acc_gemv(p->act, L.down_p, I, L.lora[MLORA_DOWN], ws_down, pending_ks));
+    pending_B = down_lora ? L.lora[MLORA_DOWN].B : nullptr;   // expanded inside the next RMSNorm launch
   }
-  STEP(norm(p->norm));
+  STEP(norm(p->norm, pending_B, ws_down, I, pending_ks));
   STEP(mlora_gemv_frag(p->logits, MLORA_F32, MLORA_STORE, p->xn, p->lm_head_p, T, H, p->vocab, stream));
   STEP(mlora_argmax(p->tokens, p->logits, T, p->vocab, stream));
   hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, p->pos, p->ctx, T);

@@ -19,19 +19,18 @@ namespace {
 
 constexpr int GEMV_WAVES = 8;
 constexpr int KSTEP = 32;   // k per MFMA
-constexpr int PIPE = 4;     // k-steps in flight per wave
 
 enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2, OUT_SILU_FRAG = 3 };
 
 // With SHRINK the first `shrink_blocks` workgroups of the launch do LoRA shrink units (one per wave) on the same
 // x instead of a GEMV tile: the adapter work rides in the GEMV launch and finishes long before it does.
-template <int NT, int TT, int OUT, bool PACKED, bool XFRAG, bool SHRINK>
+template <int NT, int TT, int OUT, bool PACKED, bool XFRAG, bool SHRINK, int PIPE = 4>   // PIPE: k-steps in flight per wave
 __global__ __launch_bounds__(GEMV_WAVES* WAVE, 4) void gemv_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx,
                                                                 const f16* __restrict__ W, int T, int K, int N,
                                                                 LoraShrinkBatch sb, int shrink_blocks, int n_main,
-                                                                float* __restrict__ y2) {
+                                                                float* __restrict__ y2, int ksplit, float* __restrict__ part) {
   __shared__ f32x4 red[GEMV_WAVES][NT * TT][WAVE];
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps the k-loop control scalar
   const int lane = threadIdx.x & 63;
   int bid = blockIdx.x;
   if constexpr (SHRINK) {
@@ -42,19 +41,30 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, 4) void gemv_kernel(void* __restr
     }
     bid -= shrink_blocks;
   }
+  // K split over `ksplit` consecutive workgroups: slice 0 runs the normal epilogue, slice s > 0 stores its fp32
+  // partial tile to part[s - 1][t][n]; whoever reads y next adds the partials in slice order.
+  int slice = 0;
+  if (ksplit > 1) {
+    slice = bid % ksplit;
+    bid /= ksplit;
+  }
   const int r16 = lane & 15;
   const int kg = lane >> 4;
   const int n0 = bid * (16 * NT);
   const int KB = K / KSTEP;
   constexpr int WSTEP = PACKED ? 512 : KSTEP;   // elements between consecutive k-steps of one fragment stream
 
-  const f16* wp[NT];
+  const f16* wp[PACKED ? 1 : NT];
+  int woff[NT];                                    // packed: element offset of tile i from the block's first tile (uniform)
   const f16* xp[TT];
+  if constexpr (PACKED) wp[0] = W + ((size_t)bid * NT * KB) * 512 + lane * 8;
 #pragma unroll
   for (int i = 0; i < NT; ++i) {
     if constexpr (PACKED) {
-      wp[i] = W + ((size_t)(bid * NT + i) * KB) * 512 + lane * 8;
+      // a tile past the end repeats the block's first tile and is not stored
+      woff[i] = ((bid * NT + i) * 16 < N ? i : 0) * KB * 512;
     } else {
+      woff[i] = 0;
       int n = n0 + i * 16 + r16;
       n = n < N ? n : N - 1;
       wp[i] = W + (size_t)n * K + kg * 8;
@@ -80,14 +90,16 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, 4) void gemv_kernel(void* __restr
 
   // wave w takes k-steps w, w + 8, w + 16, ...; stage s of this wave is k-step w + 8 s.
   // PIPE stages are always in flight: each buffer is refilled right after it is consumed.
-  const int S = (KB - wave + GEMV_WAVES - 1) / GEMV_WAVES;
+  const int kb0 = ksplit > 1 ? (int)((long)slice * KB / ksplit) : 0;
+  const int kb1 = ksplit > 1 ? (int)((long)(slice + 1) * KB / ksplit) : KB;
+  const int S = (kb1 - kb0 - wave + GEMV_WAVES - 1) / GEMV_WAVES;
   f16x8 a[PIPE][NT], b[PIPE][TT];
   auto load_stage = [&](int u, int s) {
     const bool in = s < S;
-    const int ks = in ? wave + GEMV_WAVES * s : 0;
+    const int ks = in ? kb0 + wave + GEMV_WAVES * s : 0;
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
-      a[u][i] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(wp[i] + (size_t)ks * WSTEP));
+      a[u][i] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(wp[PACKED ? 0 : i] + (woff[i] + ks * WSTEP)));
       if (!in) a[u][i] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
 #pragma unroll
@@ -112,19 +124,32 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, 4) void gemv_kernel(void* __restr
     for (int j = 0; j < TT; ++j) red[wave][i * TT + j][lane] = acc[i][j];
   __syncthreads();
 
+  if (slice > 0) {
+    for (int e = threadIdx.x; e < NT * TT * WAVE; e += GEMV_WAVES * WAVE) {
+      const int tile = e >> 6, sl = e & 63;
+      f32x4 s = red[0][tile][sl];
+#pragma unroll
+      for (int w = 1; w < GEMV_WAVES; ++w) s += red[w][tile][sl];
+      const int n = n0 + (tile / TT) * 16 + (sl >> 4) * 4;
+      const int t = (tile % TT) * 16 + (sl & 15);
+      if (t < T && n < N) *reinterpret_cast<f32x4*>(part + ((size_t)(slice - 1) * T + t) * N + n) = s;
+    }
+    return;
+  }
   if constexpr (OUT == OUT_SILU_FRAG) {
     // The weight interleaves 16-row tiles of gate and up, so this block's two tiles are gate rows c..c+15 and up
     // rows c..c+15 of the same channels: out[t, c + ..] = silu(f16(gate)) * f16(up), written in fragment order.
-    static_assert(NT == 2 || OUT != OUT_SILU_FRAG, "the SiLU epilogue pairs a gate tile with an up tile");
-    for (int e = threadIdx.x; e < TT * WAVE; e += GEMV_WAVES * WAVE) {
-      const int j = e >> 6, sl = e & 63;
-      f32x4 sg = red[0][j][sl], su = red[0][TT + j][sl];
+    static_assert(NT % 2 == 0 || OUT != OUT_SILU_FRAG, "the SiLU epilogue pairs a gate tile with an up tile");
+    for (int e = threadIdx.x; e < (NT / 2) * TT * WAVE; e += GEMV_WAVES * WAVE) {
+      const int pj = e >> 6, sl = e & 63;
+      const int p = pj / TT, j = pj % TT;         // tile pair (gate tile 2p, up tile 2p + 1), token tile j
+      f32x4 sg = red[0][2 * p * TT + j][sl], su = red[0][(2 * p + 1) * TT + j][sl];
 #pragma unroll
       for (int w = 1; w < GEMV_WAVES; ++w) {
-        sg += red[w][j][sl];
-        su += red[w][TT + j][sl];
+        sg += red[w][2 * p * TT + j][sl];
+        su += red[w][(2 * p + 1) * TT + j][sl];
       }
-      const int c = bid * 16 + (sl >> 4) * 4;      // output channel of the first of this lane's 4 rows
+      const int c = (bid * (NT / 2) + p) * 16 + (sl >> 4) * 4;   // output channel of the first of this lane's 4 rows
       const int t = j * 16 + (sl & 15);
       if (t < T && c < N / 2) {
         f16x4 o;
@@ -194,27 +219,39 @@ __global__ __launch_bounds__(256) void pack_activation_kernel(f16* __restrict__ 
   st8(dst + (size_t)c * 8, v);
 }
 
-template <int NT, int TT, bool PACKED, bool XFRAG, bool SHRINK>
+template <int NT, int TT, bool PACKED, bool XFRAG, bool SHRINK, int PIPE = 4>
 void launch_gemv(void* y, int out, const f16* x, int ldx, const f16* W, int T, int K, int N, hipStream_t s,
-                 const LoraShrinkBatch& sb, int n_main, float* y2) {
+                 const LoraShrinkBatch& sb, int n_main, float* y2, int ksplit = 1, float* part = nullptr) {
   const int sblocks = SHRINK ? ceil_div(lora_shrink_units(sb), GEMV_WAVES) : 0;
-  const dim3 grid(ceil_div(N, 16 * NT) + sblocks), block(GEMV_WAVES * WAVE);
-  if (out == OUT_F16) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F16, PACKED, XFRAG, SHRINK>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2);
-  else if (out == OUT_F32) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F32, PACKED, XFRAG, SHRINK>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2);
-  else hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_ACC_F32, PACKED, XFRAG, SHRINK>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2);
+  const dim3 grid(ceil_div(N, 16 * NT) * ksplit + sblocks), block(GEMV_WAVES * WAVE);
+  if (out == OUT_F16) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F16, PACKED, XFRAG, SHRINK, PIPE>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2, ksplit, part);
+  else if (out == OUT_F32) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F32, PACKED, XFRAG, SHRINK, PIPE>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2, ksplit, part);
+  else hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_ACC_F32, PACKED, XFRAG, SHRINK, PIPE>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2, ksplit, part);
 }
 
+// Rows per workgroup.  Every workgroup reads the whole token block, so its L2 traffic is T / (16 NT) of the weight
+// traffic and the time of a launch follows the most loaded compute unit: wide matrices (>= 768 tiles) take four tiles
+// per wave, which keeps one or two equal workgroups on every unit; narrow ones one tile (or, with a partials buffer,
+// four tiles and a K split - see mlora_gemv_ksplit).
 template <bool PACKED, bool XFRAG, bool SHRINK = false>
 int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K, int N, void* stream,
-                  const LoraShrinkBatch& sb = LoraShrinkBatch(), int n_main = -1, float* y2 = nullptr) {
+                  const LoraShrinkBatch& sb = LoraShrinkBatch(), int n_main = -1, float* y2 = nullptr, int ksplit = 1,
+                  float* part = nullptr) {
   if (n_main < 0) n_main = N;
   const int out = mode == MLORA_ACCUMULATE ? OUT_ACC_F32 : (y_dtype == MLORA_F32 ? OUT_F32 : OUT_F16);
   hipStream_t s = (hipStream_t)stream;
   const f16* xp = (const f16*)x;
   const f16* Wp = (const f16*)W;
+  const int tiles = ceil_div(N, 16);
+  if constexpr (PACKED && XFRAG) {
+    if (T <= 32 && (ksplit > 1 || tiles >= 768)) {
+      if (T <= 16) launch_gemv<4, 1, PACKED, XFRAG, SHRINK, 4>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part);
+      else launch_gemv<4, 2, PACKED, XFRAG, SHRINK, 3>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part);
+      return mlora_launch_status("gemv");
+    }
+  }
   // two 16-row tiles per wave once there are enough rows to give every CU a workgroup; the packed
   // layout pads N to a multiple of 16, so an odd tile count keeps one tile per wave
-  const int tiles = ceil_div(N, 16);
   const bool wide = tiles >= 512 && (!PACKED || tiles % 2 == 0);
   if (T <= 16) {
     if (wide) launch_gemv<2, 1, PACKED, XFRAG, SHRINK>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2);
@@ -266,16 +303,17 @@ extern "C" int mlora_gemv_frag(void* y, int y_dtype, int mode, const void* xf, c
   return gemv_dispatch<true, true>(y, y_dtype, mode, xf, K, Wp, T, K, N, stream);
 }
 
-extern "C" int mlora_gemv_frag_lora(void* y, int y_dtype, int mode, const void* xf, const void* Wp, int T, int K, int N,
-                                    void* v_part, const void* const* A, int n_proj, const int32_t* tok_adapter, int r,
-                                    int n_ad, void* stream) {
-  if (int e = mlora_check_linear("gemv_frag_lora", y, y_dtype, mode, xf, K, Wp, T, K, N)) return e;
-  MLORA_CHECK(T <= 64, MLORA_ERR_UNSUPPORTED, "gemv_frag_lora: T=%d exceeds 64", T);
+static int check_shrink_args(const char* who, const void* v_part, const void* const* A, int n_proj, const int32_t* tok_adapter,
+                             int r, int n_ad) {
   MLORA_CHECK(n_proj >= 1 && n_proj <= LORA_MAX_PROJ && v_part && A && tok_adapter, MLORA_ERR_INVALID,
-              "gemv_frag_lora: need 1..%d projections and non-null LoRA arguments", LORA_MAX_PROJ);
+              "%s: need 1..%d projections and non-null LoRA arguments", who, LORA_MAX_PROJ);
   MLORA_CHECK((r == 8 || r == 16 || r == 32 || r == 64) && n_ad > 0 && n_ad <= 65535, MLORA_ERR_UNSUPPORTED,
-              "gemv_frag_lora: rank %d not in {8,16,32,64} or bad n_ad %d", r, n_ad);
-  if (T == 0) return MLORA_OK;
+              "%s: rank %d not in {8,16,32,64} or bad n_ad %d", who, r, n_ad);
+  return MLORA_OK;
+}
+
+static LoraShrinkBatch shrink_batch(const void* xf, void* v_part, const void* const* A, int n_proj, const int32_t* tok_adapter,
+                                    int T, int K, int r, int n_ad) {
   const LoraKSplit ks = lora_k_split(K);
   LoraShrinkBatch b = {};
   for (int i = 0; i < n_proj; ++i) b.A[i] = (const f16*)A[i];   // a null slot is skipped
@@ -286,7 +324,58 @@ extern "C" int mlora_gemv_frag_lora(void* y, int y_dtype, int mode, const void* 
   b.T = T; b.K = K; b.r = r; b.n_ad = n_ad; b.ci = ks.ci; b.kc = ks.kc;
   b.frag_tt = mlora_frag_tiles(T);
   b.speculate = n_ad <= 2 * T;
-  return gemv_dispatch<true, true, true>(y, y_dtype, mode, xf, K, Wp, T, K, N, stream, b);
+  return b;
+}
+
+extern "C" int mlora_gemv_frag_lora(void* y, int y_dtype, int mode, const void* xf, const void* Wp, int T, int K, int N,
+                                    void* v_part, const void* const* A, int n_proj, const int32_t* tok_adapter, int r,
+                                    int n_ad, void* stream) {
+  if (int e = mlora_check_linear("gemv_frag_lora", y, y_dtype, mode, xf, K, Wp, T, K, N)) return e;
+  MLORA_CHECK(T <= 64, MLORA_ERR_UNSUPPORTED, "gemv_frag_lora: T=%d exceeds 64", T);
+  if (int e = check_shrink_args("gemv_frag_lora", v_part, A, n_proj, tok_adapter, r, n_ad)) return e;
+  if (T == 0) return MLORA_OK;
+  return gemv_dispatch<true, true, true>(y, y_dtype, mode, xf, K, Wp, T, K, N, stream,
+                                         shrink_batch(xf, v_part, A, n_proj, tok_adapter, T, K, r, n_ad));
+}
+
+// A narrow weight (fewer than 512 row tiles) gives too few workgroups for four tiles each; splitting K over up to four
+// workgroups restores one equal workgroup per compute unit.  At least 24 k-steps per slice keep every wave's pipeline full.
+extern "C" int mlora_gemv_ksplit(int T, int K, int N_total) {
+  if (T <= 0 || T > 32 || K <= 0 || K % 32 || N_total <= 0) return 1;
+  const int tiles = ceil_div(N_total, 16);
+  if (tiles >= 512) return 1;
+  const int groups = ceil_div(tiles, 4);
+  int ks = 256 / groups;
+  const int by_k = (K / KSTEP) / 24;
+  if (ks > by_k) ks = by_k;
+  if (ks > 4) ks = 4;
+  return ks < 1 ? 1 : ks;
+}
+
+extern "C" size_t mlora_gemv_ksplit_bytes(int T, int N_total, int ks) {
+  if (T <= 0 || N_total <= 0 || ks <= 1) return 0;
+  return (size_t)(ks - 1) * T * N_total * sizeof(float);
+}
+
+extern "C" int mlora_gemv_frag_acc_ksplit(float* y, float* y2, float* part, int ks, const void* xf, const void* Wp, int T, int K,
+                                          int N_main, int N_ext, void* v_part, const void* const* A, int n_proj,
+                                          const int32_t* tok_adapter, int r, int n_ad, void* stream) {
+  if (int e = mlora_check_linear("gemv_frag_acc_ksplit", y, MLORA_F32, MLORA_ACCUMULATE, xf, K, Wp, T, K, N_main)) return e;
+  MLORA_CHECK(T <= 64 && (ks == 1 || T <= 32), MLORA_ERR_UNSUPPORTED, "gemv_frag_acc_ksplit: T=%d exceeds 64 (32 with a K split)", T);
+  MLORA_CHECK(N_ext >= 0 && N_ext % 4 == 0 && (N_ext == 0 || (y2 && N_main % 16 == 0)), MLORA_ERR_INVALID,
+              "gemv_frag_acc_ksplit: appended rows need y2, N_ext %% 4 == 0 and N_main %% 16 == 0 (N_main=%d N_ext=%d)", N_main, N_ext);
+  MLORA_CHECK(!(A && N_ext), MLORA_ERR_INVALID, "gemv_frag_acc_ksplit: shrink units and appended rows are exclusive");
+  MLORA_CHECK(ks >= 1 && ks <= 4 && (ks == 1 || part) && (K / KSTEP) / ks >= 8, MLORA_ERR_INVALID,
+              "gemv_frag_acc_ksplit: ks=%d outside 1..4, too many slices for K=%d, or no partials buffer", ks, K);
+  if (A)
+    if (int e = check_shrink_args("gemv_frag_acc_ksplit", v_part, A, n_proj, tok_adapter, r, n_ad)) return e;
+  if (T == 0) return MLORA_OK;
+  const int N = N_main + N_ext;
+  if (A)
+    return gemv_dispatch<true, true, true>(y, MLORA_F32, MLORA_ACCUMULATE, xf, K, Wp, T, K, N, stream,
+                                           shrink_batch(xf, v_part, A, n_proj, tok_adapter, T, K, r, n_ad), N_main, y2, ks, part);
+  return gemv_dispatch<true, true, false>(y, MLORA_F32, MLORA_ACCUMULATE, xf, K, Wp, T, K, N, stream, LoraShrinkBatch(), N_main, y2,
+                                          ks, part);
 }
 
 extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p, int T, int K, int I, void* stream) {
@@ -298,8 +387,8 @@ extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p
   hipStream_t s = (hipStream_t)stream;
   const LoraShrinkBatch sb = LoraShrinkBatch();
   const dim3 grid(I / 16), block(GEMV_WAVES * WAVE);
-  if (T <= 16) hipLaunchKernelGGL((gemv_kernel<2, 1, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr);
-  else hipLaunchKernelGGL((gemv_kernel<2, 2, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr);
+  if (T <= 16) hipLaunchKernelGGL((gemv_kernel<2, 1, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);
+  else hipLaunchKernelGGL((gemv_kernel<2, 2, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);
   return mlora_launch_status("gemv_frag_silu");
 }
 

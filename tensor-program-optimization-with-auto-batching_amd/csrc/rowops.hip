@@ -16,6 +16,15 @@ struct LoraExpandRow {
   int r, n_ad;
 };
 
+// Partial results of a K-split GEMV that accumulated into the row being normed: n blocks [T][ld] fp32, `stride`
+// elements apart; columns 0..H-1 belong to the row, columns from H on to the appended adapter rows (dense shrink).
+constexpr int MAX_PARTS = 3;
+struct KSplitParts {
+  const float* p;
+  int n, ld;
+  size_t stride;
+};
+
 template <int NTHREADS>
 __device__ __forceinline__ float block_sum(float v, float* lds) {
   v = wave_sum(v);
@@ -34,10 +43,11 @@ constexpr int NORM_THREADS = 512;
 // With a LoRA expand attached (fp32 rows only) the block first streams B[id_row] ([H, r] fp16, coalesced 16-byte
 // chunks, r/8 lanes per output column combined by shuffles), stages the H deltas in LDS, adds them to the
 // residual row in place, and then norms the updated row.
-template <typename XT, int VPT>
+// With PARTS the K-split partials of the row are added after the expand, in slice order, and the row is stored back.
+template <typename XT, int VPT, bool PARTS = false>
 __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(f16* __restrict__ y, XT* __restrict__ x,
                                                                const f16* __restrict__ w, float eps, int H, int frag_tt,
-                                                               LoraExpandRow lx) {
+                                                               LoraExpandRow lx, KSplitParts kp) {
   __shared__ float lds[NORM_THREADS / WAVE];
   __shared__ float lv[64];
   extern __shared__ float delta[];    // H floats when a LoRA expand is attached, otherwise empty
@@ -67,6 +77,26 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(f16* __restrict__
       }
     }
   }
+  float pv[PARTS ? MAX_PARTS : 1][VPT][8];
+  if constexpr (PARTS) {
+#pragma unroll
+    for (int q = 0; q < MAX_PARTS; ++q)
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        const int c = (i * NORM_THREADS + threadIdx.x) * 8;
+        f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
+        if (q < kp.n && c < H) {
+          const float* pr = kp.p + q * kp.stride + (size_t)row * kp.ld + c;
+          lo = *reinterpret_cast<const f32x4*>(pr);
+          hi = *reinterpret_cast<const f32x4*>(pr + 4);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          pv[q][i][e] = lo[e];
+          pv[q][i][4 + e] = hi[e];
+        }
+      }
+  }
   bool has_delta = false;
   if constexpr (sizeof(XT) == 4) {
     if (lx.src.v != nullptr) {                      // block-uniform
@@ -88,7 +118,16 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(f16* __restrict__
         };
         // the shrink results and the first batch of B go out together, before the barrier that publishes lv
         float lvv = 0.f;
-        if (threadIdx.x < lx.r) lvv = lora_v_from(lx.src, 0, id, lx.r, row, threadIdx.x, lx.scaling);
+        if (threadIdx.x < lx.r) {
+          if (PARTS && lx.src.kc == 0) {            // dense shrink rows were K-split with the matrix: add their partials
+            const size_t col = (size_t)id * lx.r + threadIdx.x;
+            float a = lx.src.v[(size_t)row * lx.src.ld + col];
+            for (int q = 0; q < kp.n; ++q) a += kp.p[q * kp.stride + (size_t)row * kp.ld + H + col];
+            lvv = a * lx.scaling;
+          } else {
+            lvv = lora_v_from(lx.src, 0, id, lx.r, row, threadIdx.x, lx.scaling);
+          }
+        }
         load_batch(0);
         if (threadIdx.x < lx.r) lv[threadIdx.x] = lvv;
         __syncthreads();
@@ -126,6 +165,16 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(f16* __restrict__
         if (has_delta) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[i][e] = v[i][e] + delta[c + e];
+        }
+        if constexpr (PARTS) {
+#pragma unroll
+          for (int q = 0; q < MAX_PARTS; ++q)
+            if (q < kp.n) {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) v[i][e] = v[i][e] + pv[q][i][e];
+            }
+        }
+        if (has_delta || PARTS) {
           *reinterpret_cast<f32x4*>((float*)xr + c) = f32x4{v[i][0], v[i][1], v[i][2], v[i][3]};
           *reinterpret_cast<f32x4*>((float*)xr + c + 4) = f32x4{v[i][4], v[i][5], v[i][6], v[i][7]};
         }
@@ -239,7 +288,7 @@ __global__ __launch_bounds__(ROW_THREADS) void argmax_kernel(int32_t* __restrict
 }  // namespace
 
 static int rmsnorm_impl(const char* who, void* y, int y_layout, void* x, int x_dtype, const void* w, float eps, int T,
-                        int H, const LoraExpandRow& lx, void* stream) {
+                        int H, const LoraExpandRow& lx, void* stream, const KSplitParts& kp = KSplitParts()) {
   MLORA_CHECK(y_layout == MLORA_ROWMAJOR || (y_layout == MLORA_FRAG && T <= 64 && H % 32 == 0), MLORA_ERR_UNSUPPORTED,
               "%s: fragment-ordered output needs T <= 64 and H %% 32 == 0 (layout=%d T=%d H=%d)", who, y_layout, T, H);
   const int frag_tt = y_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
@@ -251,8 +300,13 @@ static int rmsnorm_impl(const char* who, void* y, int y_layout, void* x, int x_d
   const int vpt = ceil_div(H, NORM_THREADS * 8);
   const size_t dyn = lx.src.v ? (size_t)H * sizeof(float) : 0;   // LDS staging of the expand deltas
 #define MLORA_RMS(XT, VPT) \
-  hipLaunchKernelGGL((rmsnorm_kernel<XT, VPT>), dim3(T), dim3(NORM_THREADS), dyn, s, (f16*)y, (XT*)x, (const f16*)w, eps, H, frag_tt, lx)
-  if (x_dtype == MLORA_F16) {
+  hipLaunchKernelGGL((rmsnorm_kernel<XT, VPT>), dim3(T), dim3(NORM_THREADS), dyn, s, (f16*)y, (XT*)x, (const f16*)w, eps, H, frag_tt, lx, kp)
+  if (kp.n > 0) {
+    MLORA_CHECK(x_dtype == MLORA_F32 && vpt <= 2 && kp.n <= MAX_PARTS && kp.p, MLORA_ERR_UNSUPPORTED,
+                "%s: K-split partials need an fp32 row, H <= 8192 and at most %d partial blocks (H=%d n=%d)", who, H, MAX_PARTS, kp.n);
+    if (vpt <= 1) hipLaunchKernelGGL((rmsnorm_kernel<float, 1, true>), dim3(T), dim3(NORM_THREADS), dyn, s, (f16*)y, (float*)x, (const f16*)w, eps, H, frag_tt, lx, kp);
+    else hipLaunchKernelGGL((rmsnorm_kernel<float, 2, true>), dim3(T), dim3(NORM_THREADS), dyn, s, (f16*)y, (float*)x, (const f16*)w, eps, H, frag_tt, lx, kp);
+  } else if (x_dtype == MLORA_F16) {
     if (vpt <= 1) MLORA_RMS(f16, 1);
     else if (vpt <= 2) MLORA_RMS(f16, 2);
     else MLORA_RMS(f16, 4);
@@ -285,6 +339,33 @@ extern "C" int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, co
   lx.scaling = scaling;
   lx.r = r; lx.n_ad = n_ad;
   return rmsnorm_impl("lora_expand_rmsnorm", y, y_layout, resid, MLORA_F32, w, eps, T, H, lx, stream);
+}
+
+extern "C" int mlora_rmsnorm_ksplit(void* y, int y_layout, float* resid, const float* part, int ks, int ld_part, const void* w,
+                                    float eps, int T, int H, const void* v_part, int v_dense, const void* B,
+                                    const int32_t* tok_adapter, float scaling, int K, int r, int n_ad, void* stream) {
+  MLORA_CHECK(ks >= 1 && ks <= MAX_PARTS + 1 && (ks == 1 || (part && ld_part >= H && ld_part % 4 == 0)), MLORA_ERR_INVALID,
+              "rmsnorm_ksplit: ks=%d outside 1..%d, or bad partials (ld_part=%d H=%d)", ks, MAX_PARTS + 1, ld_part, H);
+  LoraExpandRow lx = {};
+  if (B) {
+    MLORA_CHECK(v_part && tok_adapter, MLORA_ERR_INVALID, "rmsnorm_ksplit: null LoRA argument");
+    MLORA_CHECK((r == 8 || r == 16 || r == 32 || r == 64) && n_ad > 0 && K > 0, MLORA_ERR_UNSUPPORTED,
+                "rmsnorm_ksplit: rank %d not in {8,16,32,64} or bad n_ad/K", r);
+    MLORA_CHECK(!v_dense || ks == 1 || ld_part >= H + n_ad * r, MLORA_ERR_INVALID,
+                "rmsnorm_ksplit: partials of a dense shrink need ld_part >= H + n_ad * r (ld_part=%d)", ld_part);
+    lx.src.v = (const float*)v_part;
+    lx.src.kc = v_dense ? 0 : lora_k_split(K).kc;
+    lx.src.T = T; lx.src.n_ad = n_ad; lx.src.ld = n_ad * r;
+    lx.B = (const f16*)B;
+    lx.ids = tok_adapter;
+    lx.scaling = scaling;
+    lx.r = r; lx.n_ad = n_ad;
+  }
+  KSplitParts kp = {};
+  if (ks > 1) {
+    kp.p = part; kp.n = ks - 1; kp.ld = ld_part; kp.stride = (size_t)T * ld_part;
+  }
+  return rmsnorm_impl("rmsnorm_ksplit", y, y_layout, resid, MLORA_F32, w, eps, T, H, lx, stream, kp);
 }
 
 extern "C" int mlora_silu_mul(void* out, int out_layout, const void* gate, const void* up, int ld, int T, int I,

@@ -49,7 +49,7 @@ class NativeDecodeSession:
     replayed from a captured graph.  The graph is re-used as long as the batch does not change; the host only
     grows the block table when a sequence crosses a page boundary."""
 
-    def __init__(self, model, kv, seq_ids, adapter_ids, first_tokens, tid=0, use_graph=True, dense_lora=None, fuse_silu=True):
+    def __init__(self, model, kv, seq_ids, adapter_ids, first_tokens, tid=0, use_graph=True, dense_lora=None, fuse_silu=True, ksplit=True):
         import ctypes as C
         from . import _lib
         self.model, self.kv = model, kv
@@ -80,6 +80,9 @@ class NativeDecodeSession:
         ws_bytes = 5 * max(_lib.lib().mlora_gather_mm_workspace_bytes(T, max(H, I, s.q_size), max(r, 8)),
                            4 * T * (lt.n_adapters if lt is not None else 0) * max(r, 8))
         self.buf["lora_ws"] = torch.empty(ws_bytes // 4, dtype=f32, device=dev)
+        # partials of the K-split o_proj / down_proj GEMVs (up to 3 slices of [T, H + appended adapter rows])
+        ks_elems = 3 * T * (H + (lt.n_adapters * r if lt is not None else 0)) if ksplit else 0
+        self.buf["ksplit_ws"] = torch.empty(max(ks_elems, 1), dtype=f32, device=dev)
         layers = (_lib.Layer * s.num_hidden_layers)()
         order = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")
         # Dense shrink: the stacked A tables become extra weight rows of the base GEMV.  Worth it while the tables
@@ -118,6 +121,8 @@ class NativeDecodeSession:
         for k in ("resid", "xn", "qkv", "attn", "gate_up", "act", "logits", "lora_ws"):
             setattr(p, k, self.buf[k].data_ptr())
         p.lora_ws_bytes = ws_bytes
+        if ksplit:
+            p.ksplit_ws, p.ksplit_ws_bytes = self.buf["ksplit_ws"].data_ptr(), 4 * ks_elems
         self._layers, self.plan = layers, p
         self._lib = _lib
         self.use_graph = use_graph

@@ -226,30 +226,50 @@ class LlamaForCausalLM:
         resid = hidden
         # a decode step (one token per sequence, T <= 64) keeps its activations in fragment order
         frag = T <= 64 and kv._cur is not None and kv._cur[2]
+        # a decode step splits K of the two narrow accumulating GEMVs; the RMSNorm that reads the residual next adds
+        # the partial results (the same kernels and slice counts as the native decode step)
+        ks_ws = self._ksplit_ws(T) if frag else None
+        parts = None
         for l, L in enumerate(self.layers):
-            xn = ops.rmsnorm(resid, L["ln1"], s.rms_norm_eps, frag=frag)
+            xn = ops.rmsnorm(resid, L["ln1"], s.rms_norm_eps, frag=frag, parts=parts)
             qkv = ops.linear(xn, L["qkv"])
             if tok_adapter:
                 self._lora(qkv[:, :q_sz], xn, l, "q_proj", tok_adapter)
                 self._lora(qkv[:, q_sz:q_sz + kv_sz], xn, l, "k_proj", tok_adapter)
                 self._lora(qkv[:, q_sz + kv_sz:], xn, l, "v_proj", tok_adapter)
             attn = kv.attention_with_fused_qkv(l, qkv, s.num_attention_heads, frag=frag)
-            ops.linear(attn, L["o"], out=resid, accumulate=True)
+            parts = self._linear_acc(attn, L["o"], resid, ks_ws)
             if tok_adapter:
                 self._lora(resid, attn, l, "o_proj", tok_adapter)
-            xn = ops.rmsnorm(resid, L["ln2"], s.rms_norm_eps, frag=frag)
+            xn = ops.rmsnorm(resid, L["ln2"], s.rms_norm_eps, frag=frag, parts=parts)
             gu = ops.linear(xn, L["gate_up"])
             if tok_adapter:
                 self._lora(gu[:, :I], xn, l, "gate_proj", tok_adapter)
                 self._lora(gu[:, I:], xn, l, "up_proj", tok_adapter)
             act = ops.silu_mul(gu, frag=frag)
-            ops.linear(act, L["down"], out=resid, accumulate=True)
+            parts = self._linear_acc(act, L["down"], resid, ks_ws)
             if tok_adapter:
                 self._lora(resid, act, l, "down_proj", tok_adapter)
         if logits_rows is not None:
-            resid = resid[logits_rows].contiguous()
-        xn = ops.rmsnorm(resid, self.norm, s.rms_norm_eps, frag=resid.shape[0] <= 64)
+            resid = resid[logits_rows].contiguous()       # prefill: never K-split (parts is None)
+        xn = ops.rmsnorm(resid, self.norm, s.rms_norm_eps, frag=resid.shape[0] <= 64, parts=parts)
         return ops.linear(xn, self.lm_head, out_dtype=torch.float32)
+
+    def _ksplit_ws(self, T):
+        """fp32 scratch for the K-split partials of o_proj / down_proj at T tokens (grown on demand, reused)."""
+        s = self.shape
+        need = 3 * T * s.hidden_size
+        ws = getattr(self, "_ksplit_buf", None)
+        if ws is None or ws.numel() < need:
+            ws = self._ksplit_buf = torch.empty(need, dtype=torch.float32, device=self.device)
+        return ws
+
+    @staticmethod
+    def _linear_acc(x, W, resid, ks_ws):
+        if isinstance(x, ops.FragActivation) and isinstance(W, ops.PackedWeight):
+            return ops.linear_acc_ksplit(x, W, resid, ks_ws)
+        ops.linear(x, W, out=resid, accumulate=True)
+        return None
 
     # ------------------------------------------------------------------ reference entry points
     def _ids(self, T, pairs):

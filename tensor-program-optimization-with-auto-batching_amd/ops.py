@@ -288,10 +288,39 @@ def _out_arg(out, T, H, frag, device):
     return out, _dev(out, torch.float16, "out"), ROWMAJOR
 
 
-def rmsnorm(x, w, eps: float, out=None, frag=False):
-    """Row-wise RMSNorm of x [T, H] (f16 | f32); frag=True writes a FragActivation."""
+class KSplitParts:
+    """Partial results of a K-split accumulating GEMV (slices 1..ks-1), to be added by the next RMSNorm of the row."""
+
+    def __init__(self, part: torch.Tensor, ks: int, ld: int):
+        self.part, self.ks, self.ld = part, ks, ld
+
+
+def linear_acc_ksplit(x: FragActivation, W: PackedWeight, resid: torch.Tensor, ws: torch.Tensor = None):
+    """resid [T, N] fp32 += x @ W.T as `linear(..., accumulate=True)`, with K split over several workgroups when the
+    library recommends it for this shape and `ws` (fp32 scratch) is large enough: slice 0 lands in resid, the other
+    slices in the returned KSplitParts, which the caller hands to the next `rmsnorm(resid, ..., parts=...)`.
+    Returns None when the GEMV ran unsplit."""
+    T, K = x.shape
+    N, K2 = W.shape
+    if K2 != K or resid.shape != (T, N) or resid.dtype != torch.float32:
+        raise ValueError(f"linear_acc_ksplit: x{x.shape} W{W.shape} resid{tuple(resid.shape)}")
+    ks = lib().mlora_gemv_ksplit(T, K, N) if ws is not None else 1
+    if ks > 1 and ws.numel() * 4 < lib().mlora_gemv_ksplit_bytes(T, N, ks):
+        ks = 1
+    check(lib().mlora_gemv_frag_acc_ksplit(_dev(resid, torch.float32), None, _dev(ws, torch.float32) if ks > 1 else None, ks,
+                                           x.data.data_ptr(), W.data.data_ptr(), T, K, N, 0, None, None, 0, None, 0, 0, _stream()))
+    return KSplitParts(ws, ks, N) if ks > 1 else None
+
+
+def rmsnorm(x, w, eps: float, out=None, frag=False, parts: KSplitParts = None):
+    """Row-wise RMSNorm of x [T, H] (f16 | f32); frag=True writes a FragActivation.  With `parts` (x fp32) the K-split
+    partials are first added to x in place."""
     T, H = x.shape
     out, optr, lay = _out_arg(out, T, H, frag, x.device)
+    if parts is not None:
+        check(lib().mlora_rmsnorm_ksplit(optr, lay, _dev(x, torch.float32), _dev(parts.part, torch.float32), parts.ks, parts.ld,
+                                         _dev(w, torch.float16), float(eps), T, H, None, 0, None, None, 0.0, 0, 0, 0, _stream()))
+        return out
     check(lib().mlora_rmsnorm(optr, lay, _dev(x), _dt(x), _dev(w, torch.float16), float(eps), T, H, _stream()))
     return out
 

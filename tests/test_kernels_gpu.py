@@ -585,3 +585,89 @@ def test_rope_append_page_row_writer_equals_per_token_kernel(ops, synth, Hq, Hkv
         q2[lo:hi] = part
     assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(v1, v2)
     assert torch.equal(q1[70], qkv[70]) and float(k1.abs().sum()) > 0
+
+
+# ------------------------------------------------------------------ K-split accumulating GEMV + RMSNorm that sums the partials
+@pytest.mark.parametrize("T,K,N,ks_expected", [(32, 11008, 4096, 4), (32, 4096, 4096, 4), (9, 4096, 4096, 4), (32, 4096, 4352, 3),
+                                               (32, 2048, 1024, 2), (40, 4096, 4096, 1), (32, 1024, 1024, 1)])
+def test_gemv_ksplit_partials_summed_by_rmsnorm(ops, synth, T, K, N, ks_expected):
+    """o_proj / down_proj shapes: slice 0 accumulates into the residual, the RMSNorm adds the other slices in order and
+    stores the row back.  Checked against the fp64 product and against the unsplit kernels."""
+    print(f"case gemv_ksplit T={T} K={K} N={N}", flush=True)
+    lib = load_pkg("_lib").lib()
+    assert lib.mlora_gemv_ksplit(T, K, N) == ks_expected
+    x = synth.normal(23, f"ks.x.{T}.{K}", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(23, f"ks.W.{N}.{K}", (N, K), 0.02, torch.float16, DEV)
+    w = synth.normal(23, f"ks.w.{N}", (N,), 1.0, torch.float16, DEV)
+    r0 = synth.normal(23, f"ks.r.{T}.{N}", (T, N), 1.0, torch.float32, DEV)
+    xf, Wp = ops.FragActivation.pack(x), ops.PackedWeight(W)
+    ws = torch.full((3 * T * N,), float("nan"), dtype=torch.float32, device=DEV)
+    racc = r0.clone()
+    parts = ops.linear_acc_ksplit(xf, Wp, racc, ws)
+    assert (parts is not None) == (ks_expected > 1)
+    y = ops.rmsnorm(racc, w, 1e-5, parts=parts)
+    r1 = r0.clone()
+    ops.linear(xf, Wp, out=r1, accumulate=True)
+    y1 = ops.rmsnorm(r1, w, 1e-5)
+    torch.cuda.synchronize()
+    ref = _np(r0).astype(np.float64) + _np(x).astype(np.float64) @ _np(W).astype(np.float64).T
+    assert max_rel_err(_np(racc), ref, floor=1e-2) <= 5e-4
+    assert max_rel_err(_np(y), oracle.rmsnorm_ref(ref, _np(w), 1e-5)) <= TOL
+    assert float((racc - r1).abs().max()) <= 1e-4          # only the fp32 summation order differs
+    assert max_rel_err(_np(y), _np(y1)) <= TOL
+    if ks_expected == 1:
+        assert torch.equal(racc, r1) and torch.equal(y, y1)
+    # without scratch the same call runs unsplit, bit-identical to linear(accumulate=True)
+    r2 = r0.clone()
+    assert ops.linear_acc_ksplit(xf, Wp, r2, None) is None
+    assert torch.equal(r2, r1)
+
+
+@pytest.mark.parametrize("T,K,r,n_ad", [(32, 4096, 16, 16), (20, 11008, 8, 4)])
+def test_gemv_ksplit_with_appended_adapter_rows(ops, synth, T, K, r, n_ad):
+    """Dense shrink riding in a K-split GEMV: the appended A rows are split with the matrix and the fused expand +
+    RMSNorm adds their partials before it applies B.  Against the unsplit pair of calls."""
+    L = load_pkg("_lib")
+    lib = L.lib()
+    H = 4096
+    n_ext = n_ad * r
+    x = synth.normal(29, f"kx.x.{T}.{K}", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(29, f"kx.W.{K}", (H, K), 0.02, torch.float16, DEV)
+    A = synth.normal(29, f"kx.A.{K}.{r}", (n_ad, r, K), 0.02, torch.float16, DEV)
+    B = synth.normal(29, f"kx.B.{K}.{r}", (n_ad, H, r), 0.05, torch.float16, DEV)
+    w = synth.normal(29, "kx.w", (H,), 1.0, torch.float16, DEV)
+    ids = synth.randint(29, f"kx.ids.{T}", (T,), n_ad, DEV)
+    ids[1] = -1
+    r0 = synth.normal(29, f"kx.r.{T}", (T, H), 1.0, torch.float32, DEV)
+    xf = ops.FragActivation.pack(x)
+    Wp = ops.PackedWeight(torch.cat([W, A.reshape(n_ext, K)], 0))
+    ks = lib.mlora_gemv_ksplit(T, K, H + n_ext)
+    assert ks > 1
+    part = torch.full((lib.mlora_gemv_ksplit_bytes(T, H + n_ext, ks) // 4,), float("nan"), dtype=torch.float32, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    out = []
+    for split in (True, False):
+        resid = r0.clone()
+        y2 = torch.empty((T, n_ext), dtype=torch.float32, device=DEV)
+        y = ops.FragActivation(T, H, DEV)
+        if split:
+            L.check(lib.mlora_gemv_frag_acc_ksplit(resid.data_ptr(), y2.data_ptr(), part.data_ptr(), ks, xf.data.data_ptr(),
+                                                   Wp.data.data_ptr(), T, K, H, n_ext, None, None, 0, None, 0, 0, st))
+            L.check(lib.mlora_rmsnorm_ksplit(y.data.data_ptr(), L.FRAG, resid.data_ptr(), part.data_ptr(), ks, H + n_ext, w.data_ptr(),
+                                             1e-5, T, H, y2.data_ptr(), 1, B.data_ptr(), ids.data_ptr(), 0.5, K, r, n_ad, st))
+        else:
+            L.check(lib.mlora_gemv_frag_split(resid.data_ptr(), L.F32, L.ACCUMULATE, y2.data_ptr(), xf.data.data_ptr(),
+                                              Wp.data.data_ptr(), T, K, H, n_ext, st))
+            L.check(lib.mlora_lora_expand_rmsnorm(y.data.data_ptr(), L.FRAG, resid.data_ptr(), y2.data_ptr(), 1, B.data_ptr(),
+                                                  ids.data_ptr(), 0.5, w.data_ptr(), 1e-5, T, H, K, r, n_ad, st))
+        out.append((resid, y.unpack()))
+    torch.cuda.synchronize()
+    x64, idn = _np(x).astype(np.float64), ids.cpu().numpy()
+    ref = _np(r0).astype(np.float64) + x64 @ _np(W).astype(np.float64).T
+    for t in range(T):
+        if idn[t] >= 0:
+            ref[t] += 0.5 * (_np(B[idn[t]]).astype(np.float64) @ (_np(A[idn[t]]).astype(np.float64) @ x64[t]))
+    for resid, y in out:
+        assert max_rel_err(_np(resid), ref, floor=1e-2) <= 5e-4
+        assert max_rel_err(_np(y), oracle.rmsnorm_ref(ref, _np(w), 1e-5)) <= TOL
+    assert float((out[0][0] - out[1][0]).abs().max()) <= 1e-4
