@@ -189,22 +189,32 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
   YT* __restrict__ y = (YT*)s.y;
   const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
 
-  // Requests that depend on the adapter table only go out first, ahead of the shrink: the thread's first row of B
-  // and the y elements of that row for the first two tokens of the adapter.
+  // Requests that depend on the adapter table only go out first, ahead of the shrink: the thread's first row(s) of B
+  // and the y elements of those rows for the first two tokens of the adapter.
+  constexpr int EB = (GR == 8 && R <= 16) ? 4 : 1;      // rows per thread whose loads are in flight together
   const int NS = ((N + P - 1) / P + 7) & ~7;            // rows per slice
   const int n1 = min(N, (p + 1) * NS);
   const int nf = p * NS + threadIdx.x;
   const int ta = __builtin_ctzll(mine);
   const unsigned long long rest1 = mine & (mine - 1);
   const int tb = rest1 ? __builtin_ctzll(rest1) : -1;
-  f16x8 bfirst[NG];
-  float ya = 0.f, yb = 0.f;
-  if (nf < n1) {
+  const unsigned long long rest2 = tb >= 0 ? rest1 & (rest1 - 1) : 0ull;   // tokens beyond the first two
+  f16x8 bpre[EB][NG];
+  float ya[EB], yb[EB];
+  auto request = [&](int nbase) {
 #pragma unroll
-    for (int q = 0; q < NG; ++q) bfirst[q] = ld8(B + (size_t)nf * R + q * 8);
-    ya = (float)y[(size_t)ta * ldy + nf];
-    if (tb >= 0) yb = (float)y[(size_t)tb * ldy + nf];
-  }
+    for (int i = 0; i < EB; ++i) {
+      const int n = nbase + i * GMM_THREADS;
+      ya[i] = yb[i] = 0.f;
+      if (n < n1) {
+#pragma unroll
+        for (int q = 0; q < NG; ++q) bpre[i][q] = ld8(B + (size_t)n * R + q * 8);
+        ya[i] = (float)y[(size_t)ta * ldy + n];
+        if (tb >= 0) yb[i] = (float)y[(size_t)tb * ldy + n];
+      }
+    }
+  };
+  request(nf);
 
   // ---- shrink: wave c owns K-slice c; tokens two at a time; same arithmetic as lora_shrink_unit
   if (wave < kc) {
@@ -255,27 +265,60 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
   __syncthreads();
 
   // ---- expand: the thread's rows of the slice, every token of the adapter
-  if (nf < n1) {
-    y[(size_t)ta * ldy + nf] = (YT)(ya + row_dot<R>(bfirst, vfin + ta * R));
-    if (tb >= 0) y[(size_t)tb * ldy + nf] = (YT)(yb + row_dot<R>(bfirst, vfin + tb * R));
-    unsigned long long m = tb >= 0 ? rest1 & (rest1 - 1) : 0ull;
-    while (m) {
-      const int t = __builtin_ctzll(m);
-      m &= m - 1;
-      YT* yp = y + (size_t)t * ldy + nf;
-      *yp = (YT)((float)*yp + row_dot<R>(bfirst, vfin + t * R));
-    }
-  }
-  for (int n = nf + GMM_THREADS; n < n1; n += GMM_THREADS) {
-    f16x8 bv[NG];
+  if constexpr (EB > 1) {
+    // EB rows per pass; the next pass's loads are requested before this pass's remaining tokens are worked off
+    for (int nbase = nf; nbase < n1; nbase += EB * GMM_THREADS) {
+      f16x8 bcur[EB][NG];
 #pragma unroll
-    for (int q = 0; q < NG; ++q) bv[q] = ld8(B + (size_t)n * R + q * 8);
-    unsigned long long m = mine;
-    while (m) {
-      const int t = __builtin_ctzll(m);
-      m &= m - 1;
-      YT* yp = y + (size_t)t * ldy + n;
-      *yp = (YT)((float)*yp + row_dot<R>(bv, vfin + t * R));
+      for (int i = 0; i < EB; ++i) {
+        const int n = nbase + i * GMM_THREADS;
+        if (n < n1) {
+#pragma unroll
+          for (int q = 0; q < NG; ++q) bcur[i][q] = bpre[i][q];
+          y[(size_t)ta * ldy + n] = (YT)(ya[i] + row_dot<R>(bcur[i], vfin + ta * R));
+          if (tb >= 0) y[(size_t)tb * ldy + n] = (YT)(yb[i] + row_dot<R>(bcur[i], vfin + tb * R));
+        }
+      }
+      if (nbase + EB * GMM_THREADS < n1) request(nbase + EB * GMM_THREADS);
+      if (rest2) {
+#pragma unroll
+        for (int i = 0; i < EB; ++i) {
+          const int n = nbase + i * GMM_THREADS;
+          if (n < n1) {
+            unsigned long long m = rest2;
+            while (m) {
+              const int t = __builtin_ctzll(m);
+              m &= m - 1;
+              YT* yp = y + (size_t)t * ldy + n;
+              *yp = (YT)((float)*yp + row_dot<R>(bcur[i], vfin + t * R));
+            }
+          }
+        }
+      }
+    }
+  } else {
+    if (nf < n1) {
+      y[(size_t)ta * ldy + nf] = (YT)(ya[0] + row_dot<R>(bpre[0], vfin + ta * R));
+      if (tb >= 0) y[(size_t)tb * ldy + nf] = (YT)(yb[0] + row_dot<R>(bpre[0], vfin + tb * R));
+      unsigned long long m = rest2;
+      while (m) {
+        const int t = __builtin_ctzll(m);
+        m &= m - 1;
+        YT* yp = y + (size_t)t * ldy + nf;
+        *yp = (YT)((float)*yp + row_dot<R>(bpre[0], vfin + t * R));
+      }
+    }
+    for (int n = nf + GMM_THREADS; n < n1; n += GMM_THREADS) {
+      f16x8 bv[NG];
+#pragma unroll
+      for (int q = 0; q < NG; ++q) bv[q] = ld8(B + (size_t)n * R + q * 8);
+      unsigned long long m = mine;
+      while (m) {
+        const int t = __builtin_ctzll(m);
+        m &= m - 1;
+        YT* yp = y + (size_t)t * ldy + n;
+        *yp = (YT)((float)*yp + row_dot<R>(bv, vfin + t * R));
+      }
     }
   }
 }
