@@ -180,10 +180,13 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
   const int p = (wg >> 3) % P;
   if (a >= n_ad) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // the problem's pointers and the table row are independent requests: both are in flight before either is awaited
+  // (the empty asm keeps the pointer load in this block, ahead of the early exit)
+  const GmmSet s = sets ? sets[blockIdx.y] : one;
   const int id = lora_token_id(ids, bucket_of, bucket, lane, T);   // T <= 64: one table row per lane
+  asm volatile("" ::"s"(s.A), "s"(s.B), "s"(s.x), "s"(s.y));
   const unsigned long long mine = __ballot(id == a);
   if (!mine) return;                                    // workgroup-uniform
-  const GmmSet s = sets ? sets[blockIdx.y] : one;
   const f16* __restrict__ A = s.A + (size_t)a * R * K;
   const f16* __restrict__ B = s.B + (size_t)a * N * R;
   YT* __restrict__ y = (YT*)s.y;
@@ -220,40 +223,75 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
   if (wave < kc) {
     const int kbase = wave * ci_n * LORA_KCHUNK + lane * 8;
     float* __restrict__ vp = part + (size_t)wave * T * R;
-    unsigned long long m = mine;
-    while (m) {
-      int tt[2];
-      tt[0] = __builtin_ctzll(m);
-      m &= m - 1;
-      tt[1] = -1;
-      if (m) {
-        tt[1] = __builtin_ctzll(m);
-        m &= m - 1;
-      }
-      const int t1 = tt[1] >= 0 ? tt[1] : tt[0];
+    if (GR == 16 && ci_n == 1) {
+      // the slice is one 512-wide chunk: a group of G rows of A stays in registers over all tokens of the adapter
+      // (the single-problem variant; the many-problem variant has no registers to spare for it)
+      const bool in = kbase < K;
 #pragma unroll
       for (int jb = 0; jb < R; jb += G) {
-        float acc0[G], acc1[G];
+        f16x8 areg[G];
 #pragma unroll
-        for (int j = 0; j < G; ++j) acc0[j] = acc1[j] = 0.f;
-        for (int ci = 0; ci < ci_n; ++ci) {
-          const int k = kbase + ci * LORA_KCHUNK;
-          const bool in = k < K;
-          const f16x8 x0 = in ? ld8(s.x + (frag_tt ? frag_offset(tt[0], k, frag_tt) : (size_t)tt[0] * K + k)) : zero8;
-          const f16x8 x1 = in ? ld8(s.x + (frag_tt ? frag_offset(t1, k, frag_tt) : (size_t)t1 * K + k)) : zero8;
-          f16x8 areg[G];
-#pragma unroll
-          for (int j = 0; j < G; ++j) areg[j] = in ? ld8(A + (size_t)(jb + j) * K + k) : zero8;
+        for (int j = 0; j < G; ++j) areg[j] = in ? ld8(A + (size_t)(jb + j) * K + kbase) : zero8;
+        unsigned long long m = mine;
+        while (m) {
+          const int t0 = __builtin_ctzll(m);
+          m &= m - 1;
+          int t1 = -1;
+          if (m) {
+            t1 = __builtin_ctzll(m);
+            m &= m - 1;
+          }
+          const int t1x = t1 >= 0 ? t1 : t0;
+          const f16x8 x0 = in ? ld8(s.x + (frag_tt ? frag_offset(t0, kbase, frag_tt) : (size_t)t0 * K + kbase)) : zero8;
+          const f16x8 x1 = in ? ld8(s.x + (frag_tt ? frag_offset(t1x, kbase, frag_tt) : (size_t)t1x * K + kbase)) : zero8;
+          float acc0[G], acc1[G];
 #pragma unroll
           for (int j = 0; j < G; ++j) {
-            acc0[j] = dot8(areg[j], x0, acc0[j]);
-            acc1[j] = dot8(areg[j], x1, acc1[j]);
+            acc0[j] = dot8(areg[j], x0, 0.f);
+            acc1[j] = dot8(areg[j], x1, 0.f);
           }
+          const int j0 = reduce_transpose<G>(acc0, lane);
+          if ((lane & (WAVE / G - 1)) == 0) vp[(size_t)t0 * R + jb + j0] = acc0[0];
+          const int j1 = reduce_transpose<G>(acc1, lane);
+          if (t1 >= 0 && (lane & (WAVE / G - 1)) == 0) vp[(size_t)t1 * R + jb + j1] = acc1[0];
         }
-        const int j0 = reduce_transpose<G>(acc0, lane);
-        if ((lane & (WAVE / G - 1)) == 0) vp[(size_t)tt[0] * R + jb + j0] = acc0[0];
-        const int j1 = reduce_transpose<G>(acc1, lane);
-        if (tt[1] >= 0 && (lane & (WAVE / G - 1)) == 0) vp[(size_t)tt[1] * R + jb + j1] = acc1[0];
+      }
+    } else {
+      unsigned long long m = mine;
+      while (m) {
+        int tt[2];
+        tt[0] = __builtin_ctzll(m);
+        m &= m - 1;
+        tt[1] = -1;
+        if (m) {
+          tt[1] = __builtin_ctzll(m);
+          m &= m - 1;
+        }
+        const int t1 = tt[1] >= 0 ? tt[1] : tt[0];
+#pragma unroll
+        for (int jb = 0; jb < R; jb += G) {
+          float acc0[G], acc1[G];
+#pragma unroll
+          for (int j = 0; j < G; ++j) acc0[j] = acc1[j] = 0.f;
+          for (int ci = 0; ci < ci_n; ++ci) {
+            const int k = kbase + ci * LORA_KCHUNK;
+            const bool in = k < K;
+            const f16x8 x0 = in ? ld8(s.x + (frag_tt ? frag_offset(tt[0], k, frag_tt) : (size_t)tt[0] * K + k)) : zero8;
+            const f16x8 x1 = in ? ld8(s.x + (frag_tt ? frag_offset(t1, k, frag_tt) : (size_t)t1 * K + k)) : zero8;
+            f16x8 areg[G];
+#pragma unroll
+            for (int j = 0; j < G; ++j) areg[j] = in ? ld8(A + (size_t)(jb + j) * K + k) : zero8;
+#pragma unroll
+            for (int j = 0; j < G; ++j) {
+              acc0[j] = dot8(areg[j], x0, acc0[j]);
+              acc1[j] = dot8(areg[j], x1, acc1[j]);
+            }
+          }
+          const int j0 = reduce_transpose<G>(acc0, lane);
+          if ((lane & (WAVE / G - 1)) == 0) vp[(size_t)tt[0] * R + jb + j0] = acc0[0];
+          const int j1 = reduce_transpose<G>(acc1, lane);
+          if (tt[1] >= 0 && (lane & (WAVE / G - 1)) == 0) vp[(size_t)tt[1] * R + jb + j1] = acc1[0];
+        }
       }
     }
   }
