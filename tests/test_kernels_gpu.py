@@ -671,3 +671,33 @@ def test_gemv_ksplit_with_appended_adapter_rows(ops, synth, T, K, r, n_ad):
         assert max_rel_err(_np(resid), ref, floor=1e-2) <= 5e-4
         assert max_rel_err(_np(y), oracle.rmsnorm_ref(ref, _np(w), 1e-5)) <= TOL
     assert float((out[0][0] - out[1][0]).abs().max()) <= 1e-4
+
+
+# ------------------------------------------------------------------ plain prefill GEMM through the vendor library
+@pytest.mark.parametrize("T,K,N", [(256, 4096, 4096), (300, 1024, 1000), (1024, 2752, 1024), (130, 64, 40)])
+def test_library_gemm_matches_oracle(ops, synth, T, K, N):
+    """mlora_gemm_library (row-major W, hipBLASLt): store fp16 / fp32 and accumulate into an fp32 residual, against the
+    fp64 product; `linear` picks it by itself for T >= 129 on a PackedWeight that kept its row-major matrix."""
+    print(f"case library_gemm T={T} K={K} N={N}", flush=True)
+    x = synth.normal(41, f"lg.x.{T}.{K}", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(41, f"lg.W.{N}.{K}", (N, K), 0.02, torch.float16, DEV)
+    ref = _np(x).astype(np.float64) @ _np(W).astype(np.float64).T
+    y16 = ops.linear(x, W, kernel="library")
+    y32 = ops.linear(x, W, out_dtype=torch.float32, kernel="library")
+    r0 = synth.normal(41, f"lg.r.{T}.{N}", (T, N), 1.0, torch.float32, DEV)
+    racc = r0.clone()
+    ops.linear(x, W, out=racc, accumulate=True, kernel="library")
+    Wp = ops.PackedWeight(W, keep_rowmajor=True)
+    auto = ops.linear(x, Wp)
+    own = ops.linear(x, Wp, kernel="gemm")
+    torch.cuda.synchronize()
+    assert max_rel_err(_np(y16), ref) <= TOL
+    assert max_rel_err(_np(y32), ref) <= 5e-4
+    assert max_rel_err(_np(racc), _np(r0) + ref, floor=1e-2) <= 5e-4
+    assert torch.equal(auto, y16)                     # the same library call
+    assert max_rel_err(_np(own), ref) <= TOL          # and this package's GEMM agrees with both to tolerance
+    # a strided x (column slice of a wider buffer)
+    xw = synth.normal(41, f"lg.xw.{T}.{K}", (T, K + 64), 1.0, torch.float16, DEV)
+    ys = ops.linear(xw[:, :K], W, kernel="library")
+    torch.cuda.synchronize()
+    assert max_rel_err(_np(ys), _np(xw[:, :K]).astype(np.float64) @ _np(W).astype(np.float64).T) <= TOL
