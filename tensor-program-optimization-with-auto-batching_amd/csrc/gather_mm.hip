@@ -11,6 +11,8 @@
 //             through a small LDS transpose so every lane touches contiguous y elements.
 // The adapter table is never materialised per token: the index lookup happens inside the kernels,
 // which is the optimisation of tvm/custom/fuse_take_matmul.py:85-105 kept in hand-written form.
+#include <type_traits>
+
 #include "lora_device.h"
 
 namespace {
@@ -374,6 +376,118 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
 // ---------------------------------------------------------------------------------------------
 constexpr int SEG_WAVES = 4;
 
+// The distinct adapters of a 16-token tile (lanes 0..15 hold the tokens' ids, -1 = none) and, per adapter, the mask of
+// tile rows bound to it.  Everything is wave-uniform and lives in scalar registers; the loops over the list are fully
+// unrolled with a uniform `i < n` guard, so the list is never indexed dynamically.
+struct TileAdapters {
+  int a[16];
+  unsigned rows[16];
+  int n;
+  unsigned all;     // rows with any adapter
+};
+
+__device__ __forceinline__ TileAdapters tile_adapters(int id) {
+  TileAdapters ta;
+  unsigned todo = (unsigned)__ballot(id >= 0) & 0xffffu;
+  ta.all = todo;
+  ta.n = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    ta.a[i] = -1;
+    ta.rows[i] = 0u;
+    if (todo) {
+      const int first = __builtin_ctz(todo);
+      const int a = __builtin_amdgcn_readfirstlane(__shfl(id, first, WAVE));
+      const unsigned rows = (unsigned)__ballot(id == a) & 0xffffu & todo;
+      todo &= ~rows;
+      ta.a[i] = a;
+      ta.rows[i] = rows;
+      ta.n = i + 1;
+    }
+  }
+  return ta;
+}
+
+// Shrink.  The adapters of the tile are worked GA at a time inside ONE pass over K: per 32-k step the token fragment is
+// loaded once and every adapter of the group contributes one A fragment and one MFMA - a decode batch, where a tile of
+// 16 tokens holds up to 16 adapters, costs one K loop instead of 16, with all the groups' loads in flight together.
+template <int R>
+__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(float* __restrict__ v, const f16* __restrict__ x,
+                                                                            const f16* __restrict__ A,
+                                                                            const int32_t* __restrict__ ids, int T, int K,
+                                                                            int n_ad, const int32_t* __restrict__ bucket_of,
+                                                                            int bucket) {
+  // blockIdx.y selects one of gridDim.y contiguous ranges of 32-k steps; its partial sums go to v[blockIdx.y][T][R]
+  constexpr int NT = (R + 15) / 16;     // 16-row tiles of A[a]; rank 8 uses half a tile
+  constexpr int GA = 8 / NT;            // adapters per pass: 32 accumulator registers
+  __shared__ f32x4 red[SEG_WAVES][GA * NT][WAVE];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t0 = blockIdx.x * 16;
+  const int col = lane & 15, g = lane >> 4;
+  const int tl = min(t0 + col, T - 1);                          // token whose x row this lane supplies
+  const int raw = lora_token_id(ids, bucket_of, bucket, t0 + col, T);
+  const int id = (raw >= 0 && raw < n_ad) ? raw : -1;
+  const TileAdapters ta = tile_adapters(id);
+  const f16* __restrict__ xr = x + (size_t)tl * K + g * 8;
+  const int KB = K / 32;
+  const int per = (KB + gridDim.y - 1) / gridDim.y;
+  const int kb0 = blockIdx.y * per, kb1 = min(KB, kb0 + per);
+  v += (size_t)blockIdx.y * T * R;
+#pragma unroll
+  for (int g0 = 0; g0 < 16; g0 += GA) {
+    if (g0 < ta.n) {                                             // uniform
+      f32x4 acc[GA][NT];
+#pragma unroll
+      for (int u = 0; u < GA; ++u)
+#pragma unroll
+        for (int i = 0; i < NT; ++i) acc[u][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int kb = kb0 + wave; kb < kb1; kb += SEG_WAVES) {
+        const f16x8 xf = ld8(xr + kb * 32);
+        f16x8 af[GA][NT];
+#pragma unroll
+        for (int u = 0; u < GA; ++u) {
+          if (g0 + u < ta.n) {
+            const f16* __restrict__ Aa = A + (size_t)ta.a[g0 + u] * R * K + g * 8;
+#pragma unroll
+            for (int i = 0; i < NT; ++i) {
+              const int row = i * 16 + col;
+              af[u][i] = row < R ? ld8(Aa + (size_t)row * K + kb * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < GA; ++u) {
+          if (g0 + u < ta.n) {
+#pragma unroll
+            for (int i = 0; i < NT; ++i)
+              acc[u][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[u][i], xf, acc[u][i], 0, 0, 0);   // rows: rank index, cols: tokens
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < GA; ++u)
+#pragma unroll
+        for (int i = 0; i < NT; ++i) red[wave][u * NT + i][lane] = acc[u][i];
+      __syncthreads();
+      // wave w sums and stores the adapters u = w, w + 4, ... of the group (fixed order over the four K parts)
+#pragma unroll
+      for (int u = 0; u < GA; ++u) {
+        if (g0 + u < ta.n && (u % SEG_WAVES) == wave) {
+#pragma unroll
+          for (int i = 0; i < NT; ++i) {
+            f32x4 sum = red[0][u * NT + i][lane];
+#pragma unroll
+            for (int w = 1; w < SEG_WAVES; ++w) sum += red[w][u * NT + i][lane];
+            const int j = i * 16 + 4 * g;                          // first of this lane's 4 rank entries
+            if (((ta.rows[g0 + u] >> col) & 1u) && j < R) *reinterpret_cast<f32x4*>(v + (size_t)(t0 + col) * R + j) = sum;
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
 // adapter of the first unprocessed token of the tile and the mask of tile rows bound to it; lanes 0..15 hold ids
 __device__ __forceinline__ bool next_tile_adapter(int id, unsigned& todo, int& a, unsigned& rows) {
   if (!todo) return false;
@@ -384,60 +498,8 @@ __device__ __forceinline__ bool next_tile_adapter(int id, unsigned& todo, int& a
   return true;
 }
 
-template <int R>
-__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(float* __restrict__ v, const f16* __restrict__ x,
-                                                                            const f16* __restrict__ A,
-                                                                            const int32_t* __restrict__ ids, int T, int K,
-                                                                            int n_ad, const int32_t* __restrict__ bucket_of,
-                                                                            int bucket) {
-  // blockIdx.y selects one of gridDim.y contiguous ranges of 32-k steps; its partial sums go to v[blockIdx.y][T][R]
-  constexpr int NT = (R + 15) / 16;     // 16-row tiles of A[a]; rank 8 uses half a tile
-  __shared__ f32x4 red[SEG_WAVES][NT][WAVE];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int t0 = blockIdx.x * 16;
-  const int col = lane & 15, g = lane >> 4;
-  const int tl = min(t0 + col, T - 1);                          // token whose x row this lane supplies
-  const int raw = lora_token_id(ids, bucket_of, bucket, t0 + col, T);
-  const int id = (raw >= 0 && raw < n_ad) ? raw : -1;
-  unsigned todo = (unsigned)__ballot(id >= 0) & 0xffffu;
-  const f16* __restrict__ xr = x + (size_t)tl * K + g * 8;
-  const int KB = K / 32;
-  const int per = (KB + gridDim.y - 1) / gridDim.y;
-  const int kb0 = blockIdx.y * per, kb1 = min(KB, kb0 + per);
-  v += (size_t)blockIdx.y * T * R;
-  int a;
-  unsigned rows;
-  while (next_tile_adapter(id, todo, a, rows)) {
-    const f16* __restrict__ Aa = A + (size_t)a * R * K + g * 8;
-    f32x4 acc[NT];
-#pragma unroll
-    for (int i = 0; i < NT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int kb = kb0 + wave; kb < kb1; kb += SEG_WAVES) {
-      const f16x8 xf = ld8(xr + kb * 32);
-#pragma unroll
-      for (int i = 0; i < NT; ++i) {
-        const int row = i * 16 + col;
-        const f16x8 af = row < R ? ld8(Aa + (size_t)row * K + kb * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, xf, acc[i], 0, 0, 0);   // rows: rank index, cols: tokens
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < NT; ++i) red[wave][i][lane] = acc[i];
-    __syncthreads();
-    if (wave == 0) {
-#pragma unroll
-      for (int i = 0; i < NT; ++i) {
-        f32x4 s = red[0][i][lane];
-#pragma unroll
-        for (int w = 1; w < SEG_WAVES; ++w) s += red[w][i][lane];
-        const int j = i * 16 + 4 * g;                              // first of this lane's 4 rank entries
-        if (((rows >> col) & 1u) && j < R) *reinterpret_cast<f32x4*>(v + (size_t)(t0 + col) * R + j) = s;
-      }
-    }
-    __syncthreads();
-  }
-}
-
+// Expand for segment-ordered tokens (prefill): one pass per distinct adapter of the tile - one, two at a segment boundary.
+// Lean in registers (seven waves per SIMD), which is what this latency-bound kernel lives on.
 template <int R, typename YT>
 __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* __restrict__ y, const float* __restrict__ v,
                                                                             const f16* __restrict__ B,
@@ -531,6 +593,149 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* 
     __syncthreads();
    }
   }
+}
+
+// Expand for token tiles that mix many adapters (decode batches).  Per block of 16 output columns every adapter of the tile contributes B[a] . v^T (two MFMAs: hi and lo half of
+// v); a token's column of the result is taken from the product of its own adapter, so all adapters are worked off before
+// the one read-modify-write of y.  The B fragments of up to GB adapters are requested together.
+template <int R, typename YT>
+__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mixed_mfma_kernel(YT* __restrict__ y, const float* __restrict__ v,
+                                                                            const f16* __restrict__ B,
+                                                                            const int32_t* __restrict__ ids, float scaling,
+                                                                            int T, int N, int ldy, int n_ad,
+                                                                            const int32_t* __restrict__ bucket_of, int bucket,
+                                                                            int splits, int nit) {
+  constexpr int KS = (R + 31) / 32;     // k-steps of 32 rank entries (ranks 8 and 16: one partly filled step)
+  constexpr int GB = 8 / KS;            // adapters whose fragments are in flight together: 32 registers
+  constexpr int CT = 4;                 // 16-column tiles per wave
+  constexpr int LD = 16 * CT + 4;       // padded row of the transposition buffer (floats): conflict-free both ways
+  __shared__ float stage[SEG_WAVES][16][LD];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t0 = blockIdx.x * 16;
+  // a workgroup covers nit consecutive blocks of 4 waves x 64 columns; the token tile of v stays in registers
+  const int nbase = blockIdx.y * nit * SEG_WAVES * 16 * CT + wave * 16 * CT;
+  const int col = lane & 15, g = lane >> 4;
+  const int tl = min(t0 + col, T - 1);
+  const int raw = lora_token_id(ids, bucket_of, bucket, t0 + col, T);
+  const int id = (raw >= 0 && raw < n_ad) ? raw : -1;
+  const unsigned all = (unsigned)__ballot(id >= 0) & 0xffffu;    // tile rows with an adapter
+  if (!all) return;                     // the same for every wave of the workgroup
+  const int a_first = __builtin_amdgcn_readfirstlane(__shfl(id, __builtin_ctz(all), WAVE));
+  const bool one_adapter = ((unsigned)__ballot(id == a_first) & 0xffffu) == all;
+  // the token tile of v as the B operand, hi and lo halves: lane holds v[token col][ks*32 + 8g .. +7]
+  f16x8 vh[KS], vl[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int j = ks * 32 + g * 8;
+    float f[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = 0.f;
+    // rows of unadapted tokens are never read (their v holds nothing) and enter the product as zeros
+    if (j < R && id >= 0) {
+      f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
+      for (int sp = 0; sp < splits; ++sp) {           // the K-range partials of the shrink, summed in range order
+        lo += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + tl) * R + j);
+        hi += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + tl) * R + j + 4);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        f[e] = lo[e] * scaling;
+        f[4 + e] = hi[e] * scaling;
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const f16 h = (f16)f[e];
+      vh[ks][e] = h;
+      vl[ks][e] = (f16)(f[e] - (float)h);
+    }
+  }
+  // write-back role of the lane: token lane / 4, the 16 columns of column tile lane % 4 (contiguous in y)
+  const int wt = lane >> 2, wc = lane & 3;
+  // SINGLE: the tile holds one adapter (a prefill segment) - the products accumulate directly, no per-token selection
+  auto run = [&](auto single) {
+    constexpr bool SINGLE = decltype(single)::value;
+    for (int it = 0; it < nit; ++it) {
+      const int n0 = nbase + it * SEG_WAVES * 16 * CT;
+      const int nw = n0 + wc * 16;
+      YT* __restrict__ yrow = y + (size_t)(t0 + wt) * ldy + nw;
+#pragma unroll
+      for (int c = 0; c < CT; ++c) {
+        const int nb = n0 + c * 16;
+        if (nb < N) {                                                // wave-uniform
+          f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};                     // D[n = nb + 4g.., token col] of the token's own adapter
+          if constexpr (SINGLE) {
+            const f16* __restrict__ Ba = B + (size_t)a_first * N * R + g * 8;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+              const int j = ks * 32 + g * 8;
+              const f16x8 bf = j < R ? ld8(Ba + (size_t)(nb + col) * R + ks * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+              acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf, vh[ks], acc, 0, 0, 0);    // rows: output column, cols: tokens
+              acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf, vl[ks], acc, 0, 0, 0);
+            }
+          } else {
+            unsigned todo = all;
+            while (todo) {                                             // uniform: GB adapters of the tile per round
+              int ga[GB];
+              unsigned grows[GB];
+#pragma unroll
+              for (int u = 0; u < GB; ++u) {
+                ga[u] = -1;
+                grows[u] = 0u;
+                if (todo) {
+                  ga[u] = __builtin_amdgcn_readfirstlane(__shfl(id, __builtin_ctz(todo), WAVE));
+                  grows[u] = (unsigned)__ballot(id == ga[u]) & 0xffffu & todo;
+                  todo &= ~grows[u];
+                }
+              }
+              f16x8 bf[GB][KS];
+#pragma unroll
+              for (int u = 0; u < GB; ++u) {
+                if (ga[u] >= 0) {
+                  const f16* __restrict__ Ba = B + (size_t)ga[u] * N * R + g * 8;
+#pragma unroll
+                  for (int ks = 0; ks < KS; ++ks)
+                    bf[u][ks] = (ks * 32 + g * 8) < R ? ld8(Ba + (size_t)(nb + col) * R + ks * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                }
+              }
+#pragma unroll
+              for (int u = 0; u < GB; ++u) {
+                if (ga[u] >= 0) {
+                  f32x4 d = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                  for (int ks = 0; ks < KS; ++ks) {
+                    d = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf[u][ks], vh[ks], d, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf[u][ks], vl[ks], d, 0, 0, 0);
+                  }
+                  if ((grows[u] >> col) & 1u) acc = d;
+                }
+              }
+            }
+          }
+          *reinterpret_cast<f32x4*>(&stage[wave][col][c * 16 + 4 * g]) = acc;
+        }
+      }
+      __syncthreads();
+      if (nw < N && ((all >> wt) & 1u)) {
+        float d[16];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const f32x4 s4 = *reinterpret_cast<const f32x4*>(&stage[wave][wt][wc * 16 + 4 * q]);
+          d[4 * q] = s4[0]; d[4 * q + 1] = s4[1]; d[4 * q + 2] = s4[2]; d[4 * q + 3] = s4[3];
+        }
+        if constexpr (sizeof(YT) == 2) {
+          rmw_add<YT, 8>(yrow, d);
+          rmw_add<YT, 8>(yrow + 8, d + 8);
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) rmw_add<YT, 4>(yrow + 4 * q, d + 4 * q);
+        }
+      }
+      __syncthreads();
+    }
+  };
+  if (one_adapter) run(std::true_type{});
+  else run(std::false_type{});
 }
 
 __global__ void write_tensor_part_kernel(f16* __restrict__ Z, const f16* __restrict__ X, const f16* __restrict__ Y,
@@ -714,12 +919,20 @@ static void gmm_segments_r(void* y, int y_dtype, int ldy, const f16* x, const f1
   int nit = (int)(((long)tiles * ceil_div(N, SEG_WAVES * 64)) / 1024);
   nit = nit < 1 ? 1 : (nit > 8 ? 8 : nit);
   const dim3 grid(tiles, ceil_div(N, SEG_WAVES * 64 * nit));
-  if (y_dtype == MLORA_F16)
-    hipLaunchKernelGGL((lora_expand_mfma_kernel<R, f16>), grid, dim3(SEG_WAVES * WAVE), 0, s, (f16*)y, v, B, ids, scaling, T, N,
-                       ldy, n_ad, bf.bucket_of, bf.bucket, splits, nit);
-  else
-    hipLaunchKernelGGL((lora_expand_mfma_kernel<R, float>), grid, dim3(SEG_WAVES * WAVE), 0, s, (float*)y, v, B, ids, scaling, T,
-                       N, ldy, n_ad, bf.bucket_of, bf.bucket, splits, nit);
+  // Up to 1024 tokens the call is taken to be a decode batch (one token per sequence, tiles that mix many adapters);
+  // beyond that a prefill whose tokens come in adapter segments.  Either kernel is correct for either input.
+  const bool mixed = T <= 1024;
+#define MLORA_EXPAND_MFMA(KERNEL, YT)                                                                                       \
+  hipLaunchKernelGGL((KERNEL<R, YT>), grid, dim3(SEG_WAVES * WAVE), 0, s, (YT*)y, v, B, ids, scaling, T, N, ldy, n_ad, \
+                     bf.bucket_of, bf.bucket, splits, nit)
+  if (y_dtype == MLORA_F16) {
+    if (mixed) MLORA_EXPAND_MFMA(lora_expand_mixed_mfma_kernel, f16);
+    else MLORA_EXPAND_MFMA(lora_expand_mfma_kernel, f16);
+  } else {
+    if (mixed) MLORA_EXPAND_MFMA(lora_expand_mixed_mfma_kernel, float);
+    else MLORA_EXPAND_MFMA(lora_expand_mfma_kernel, float);
+  }
+#undef MLORA_EXPAND_MFMA
 }
 
 // shrink + expand on the matrix cores; v = workspace viewed as [T, r] fp32

@@ -474,6 +474,9 @@ def test_gather_mm_multi_rank_strategies_agree(ops, synth, T, K, N):
     (200, 1024, 528, 16, 6, torch.float32),       # T not a multiple of 16, N a multiple of 16 only
     (97, 2048, 256, 8, 3, torch.float16),
     (160, 11008, 1024, 32, 4, torch.float16),     # down_proj-like K
+    (256, 1024, 512, 16, 40, torch.float16),      # decode batch: up to 16 adapters in a 16-token tile (two groups of 8)
+    (1100, 1024, 256, 16, 5, torch.float16),      # beyond 1024 tokens: the segment-ordered expand kernel
+    (1200, 512, 128, 64, 3, torch.float32),
 ])
 @pytest.mark.parametrize("pattern", ["segments", "random"])
 def test_gather_mm_prefill_sizes_on_matrix_cores(ops, synth, T, K, N, r, n_ad, ydt, pattern):
