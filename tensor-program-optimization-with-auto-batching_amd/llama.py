@@ -55,7 +55,7 @@ class LoraType:
 
 class LlamaForCausalLM:
     def __init__(self, shape: LlamaShape, device="cuda:0", library_gemm: bool = False):
-        """library_gemm: keep a row-major copy of the four layer matrices so that prefill-sized base linears (T > 128)
+        """library_gemm: keep a row-major copy of the four layer matrices so that prefill-sized base linears (T > 64)
         go to the vendor GEMM library; decode-sized ones always use this package's kernels."""
         self.shape = shape
         self.device = torch.device(device)

@@ -194,7 +194,7 @@ class PackedWeight:
     """A [N, K] fp16 weight stored in matrix-core fragment order (see mlora_pack_weight)."""
 
     def __init__(self, W: torch.Tensor, keep_rowmajor: bool = False):
-        """keep_rowmajor: also keep the row-major matrix, which lets `linear` hand prefill-sized products (T > 128) to
+        """keep_rowmajor: also keep the row-major matrix, which lets `linear` hand prefill-sized products (T > 64) to
         the vendor GEMM library (one more copy of the weight)."""
         N, K = W.shape
         self.N, self.K = N, K
@@ -214,7 +214,7 @@ class PackedWeight:
         return v.permute(0, 3, 1, 2, 4).reshape(nt * 16, self.K)[: self.N].contiguous()
 
 
-LIBRARY_GEMM_MIN_T = 129      # below this the weight-streaming / small-tile kernels of this package are used
+LIBRARY_GEMM_MIN_T = 65       # up to 64 tokens the weight-streaming decode kernel of this package is used
 _lib_ws = {}
 
 
@@ -228,7 +228,7 @@ def _library_workspace(device) -> torch.Tensor:
 def linear(x, W, out=None, out_dtype=torch.float16, accumulate=False, kernel="auto"):
     """y (=|+=) x @ W.T.  x [T,K] f16 (row stride may exceed K) or a FragActivation, W [N,K] f16 or a
     PackedWeight.  accumulate=True adds into the fp32 tensor `out`.  kernel: "auto" | "gemv" | "gemm" | "library"
-    (the vendor GEMM library on a row-major W; "auto" picks it for T >= 129 when W is row-major-capable, i.e. a
+    (the vendor GEMM library on a row-major W; "auto" picks it for T >= 65 when W is row-major-capable, i.e. a
     PackedWeight built with keep_rowmajor=True)."""
     if isinstance(x, FragActivation):
         return _linear_frag(x, W, out, out_dtype, accumulate)
