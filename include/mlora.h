@@ -293,7 +293,7 @@ int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v
 /* ---------------------------------------------------------------------------------------------
  * K split of the accumulating decode GEMV over a narrow weight (o_proj, down_proj: 256 row tiles give one
  * workgroup per compute unit only at one tile each, which makes every workgroup read the whole token block for 16
- * rows).  With a split, a workgroup takes four row tiles and 1/ks of K; slice 0 accumulates into y as usual and
+ * rows).  With a split, a workgroup takes four row tiles (two beyond 32 tokens) and 1/ks of K; slice 0 accumulates into y as usual and
  * slices 1..ks-1 store fp32 partial results that the next reader of y adds in slice order - in the decoder layer
  * that reader is always an RMSNorm, so the sum is formed there and no extra pass or atomics are needed
  * (results do not depend on scheduling).

@@ -252,9 +252,13 @@ def linear(x, W, out=None, out_dtype=torch.float16, accumulate=False, kernel="au
             raise ValueError(f"linear: out{tuple(out.shape)} expected {(T, N)}")
         ws = _library_workspace(x.device)
         ldx = x.stride(0) if T > 1 else max(K, x.stride(0))
-        check(lib().mlora_gemm_library(_dev(out), _dt(out), ACCUMULATE if accumulate else STORE, x.data_ptr(), ldx,
-                                       _dev(rm, torch.float16, "W"), T, K, N, ws.data_ptr(), ws.numel(), _stream()))
-        return out
+        rc = lib().mlora_gemm_library(_dev(out), _dt(out), ACCUMULATE if accumulate else STORE, x.data_ptr(), ldx,
+                                      _dev(rm, torch.float16, "W"), T, K, N, ws.data_ptr(), ws.numel(), _stream())
+        if rc == -2 and kernel == "auto" and packed:      # the vendor library has no algorithm for this shape: own GEMM
+            kernel = "gemm"
+        else:
+            check(rc)
+            return out
     if not x.is_cuda or x.dtype != torch.float16 or x.stride(1) != 1:
         raise ValueError("linear: x must be a GPU fp16 tensor with unit inner stride")
     ldx = x.stride(0) if T > 1 else max(K, x.stride(0))
