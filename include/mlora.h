@@ -258,7 +258,7 @@ int mlora_gemv_frag_lora(void* y, int y_dtype, int mode, const void* xf, const v
                          void* v_part, const void* const* A, int n_proj, const int32_t* tok_adapter, int r, int n_ad,
                          void* stream);
 /* Gate/up projection with the SiLU product in its epilogue:  act = silu(f16(x . Wgate^T)) * f16(x . Wup^T), written
- * in MLORA_FRAG order for the down projection (T <= 32).  Wil_p is the fragment-ordered [2I, K] matrix whose 16-row
+ * in MLORA_FRAG order for the down projection (T <= 64).  Wil_p is the fragment-ordered [2I, K] matrix whose 16-row
  * tiles alternate gate and up (tile 2j = gate rows 16j.., tile 2j+1 = up rows 16j..), so one workgroup holds both
  * halves of a channel.  Replaces: gate_proj, up_proj, op.silu and the multiply (llama_for_causal_lm.py:35-36) in
  * one launch; same result bits as mlora_gemv_frag followed by mlora_silu_mul. */

@@ -101,7 +101,7 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
     STEP(acc_gemv(p->attn, L.o_p, q_sz, L.lora[MLORA_O], ws_o, ks_o));
     STEP(norm(L.ln2, o_lora ? L.lora[MLORA_O].B : nullptr, ws_o, q_sz, ks_o));
     const bool gu_lora = lora && (L.lora[MLORA_GATE].A || L.lora[MLORA_UP].A);
-    if (L.gate_up_il_p && !gu_lora && T <= 32) {
+    if (L.gate_up_il_p && !gu_lora) {
       STEP(mlora_gemv_frag_silu(p->act, p->xn, L.gate_up_il_p, T, H, I, stream));
     } else {
       MLORA_CHECK(L.gate_up_p, MLORA_ERR_INVALID, "decode_step: layer %d needs gate_up_p", l);

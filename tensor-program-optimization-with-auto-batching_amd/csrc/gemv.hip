@@ -389,15 +389,16 @@ extern "C" int mlora_gemv_frag_acc_ksplit(float* y, float* y2, float* part, int 
 
 extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p, int T, int K, int I, void* stream) {
   MLORA_CHECK(act && xf && Wil_p, MLORA_ERR_INVALID, "gemv_frag_silu: null pointer");
-  MLORA_CHECK(T > 0 && T <= 32 && K > 0 && K % 32 == 0 && I > 0 && I % 32 == 0, MLORA_ERR_UNSUPPORTED,
-              "gemv_frag_silu: need 0 < T <= 32, K %% 32 == 0, I %% 32 == 0 (T=%d K=%d I=%d)", T, K, I);
+  MLORA_CHECK(T > 0 && T <= 64 && K > 0 && K % 32 == 0 && I > 0 && I % 32 == 0, MLORA_ERR_UNSUPPORTED,
+              "gemv_frag_silu: need 0 < T <= 64, K %% 32 == 0, I %% 32 == 0 (T=%d K=%d I=%d)", T, K, I);
   const f16* xp = (const f16*)xf;
   const f16* Wp = (const f16*)Wil_p;
   hipStream_t s = (hipStream_t)stream;
   const LoraShrinkBatch sb = LoraShrinkBatch();
   const dim3 grid(I / 16), block(GEMV_WAVES * WAVE);
   if (T <= 16) hipLaunchKernelGGL((gemv_kernel<2, 1, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);
-  else hipLaunchKernelGGL((gemv_kernel<2, 2, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);
+  else if (T <= 32) hipLaunchKernelGGL((gemv_kernel<2, 2, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);
+  else hipLaunchKernelGGL((gemv_kernel<2, 4, OUT_SILU_FRAG, true, true, false, 2>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);
   return mlora_launch_status("gemv_frag_silu");
 }
 

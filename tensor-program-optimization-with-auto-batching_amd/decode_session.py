@@ -92,7 +92,7 @@ class NativeDecodeSession:
             dense_lora = lt is not None and lt.n_adapters <= 2 * T
         self.dense_lora = bool(dense_lora and lt is not None)
         ext = model.dense_lora_weights(tid) if self.dense_lora else None
-        il = model.interleaved_gate_up() if (fuse_silu and T <= 32 and s.intermediate_size % 32 == 0) else None
+        il = model.interleaved_gate_up() if (fuse_silu and s.intermediate_size % 32 == 0) else None
         for l, L in enumerate(model.layers):
             if il is not None:
                 layers[l].gate_up_il_p = il[l].data.data_ptr()

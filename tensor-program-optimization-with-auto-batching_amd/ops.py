@@ -306,7 +306,7 @@ def interleave_gate_up(gate_up: torch.Tensor) -> PackedWeight:
 
 
 def gate_up_silu(x: FragActivation, W_il: PackedWeight, out: FragActivation = None) -> FragActivation:
-    """silu(x @ Wgate.T) * (x @ Wup.T) in one launch; W_il from interleave_gate_up.  T <= 32."""
+    """silu(x @ Wgate.T) * (x @ Wup.T) in one launch; W_il from interleave_gate_up.  T <= 64."""
     T, K = x.shape
     I2, K2 = W_il.shape
     if K2 != K:

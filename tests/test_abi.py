@@ -76,7 +76,7 @@ def test_argument_validation_of_fused_and_batched_entry_points():
     assert lib.mlora_rope_attn_decode(1, 0, 1, 1, 1, 1, 4, 1, 1, 1, 1, 1, 64, 2, 8, 8, 128, 4, 2,
                                       1, 1, None, None, 0.5, 64, 16, 2, None) == -1     # LoRA without B / ids
     # SiLU epilogue GEMV and split GEMV
-    assert lib.mlora_gemv_frag_silu(1, 1, 1, 33, 64, 64, None) == -2
+    assert lib.mlora_gemv_frag_silu(1, 1, 1, 65, 64, 64, None) == -2
     assert lib.mlora_gemv_frag_silu(1, 1, 1, 8, 64, 48, None) == -2
     assert lib.mlora_gemv_frag_silu(None, 1, 1, 8, 64, 64, None) == -1
     # K-split GEMV: slice counts, partials buffer, argument checks

@@ -136,3 +136,21 @@ def test_full_depth_benchmark_model_native_equals_per_operator():
     margin = torch.topk(lg, 2, dim=-1).values
     decided = ((margin[:, 0] - margin[:, 1]) >= 2e-2 * lg.std(dim=-1)).cpu().numpy()
     assert np.array_equal(d[1][decided], c[1][decided])
+
+
+def test_native_step_between_33_and_64_requests():
+    """48 requests (four token tiles: two row tiles per wave in the GEMV, K split at two rows tiles, SiLU epilogue at
+    four token tiles): the native step reproduces the per-operator path bit for bit, tokens and K cache."""
+    synth, llama = load_pkg("synth"), load_pkg("llama")
+    wl = synth.config3(num_layers=2, batch=48, prompt_len=30)
+    ids = wl.adapter_ids.copy()
+    ids[11] = -1
+    model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, [wl.lora], DEV)
+    prompts = synth.prompts(wl)
+    a, ka, _ = _run(model, wl, prompts, ids, "py", 5, synth)
+    c, kc, lg = _run(model, wl, prompts, ids, "graph", 5, synth)
+    assert np.array_equal(a, c)
+    assert torch.equal(ka, kc)
+    d, _, ld = _run(model, wl, prompts, ids, "dense", 5, synth, run_steps=1)
+    err = float((ld - lg).abs().max() / lg.std())
+    assert err <= 1e-2, err
