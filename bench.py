@@ -373,6 +373,8 @@ def main():
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--layers", type=int, default=32, help="model depth (32 = the benchmark configuration)")
+    ap.add_argument("--batch", type=int, default=32,
+                    help="c3_decode: concurrent requests (32 = the benchmark configuration; up to 64 run the native step)")
     ap.add_argument("--workload", default="c3_decode", choices=["c3_decode", "c4_prefill", "c5_decode"],
                     help="c3_decode is the benchmark the metric is quoted on; the other two time the prefill and the "
                          "256-request stress configurations with the same harness")
@@ -411,7 +413,7 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"probe": True, "copy_bytes_each_way": 256 << 20, "gemv": g, "gather_matmul": gm}))
         return
-    wl = synth.config3(num_layers=args.layers)
+    wl = synth.config3(num_layers=args.layers, batch=args.batch)
     t_setup = time.perf_counter()
     model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, [wl.lora], dev)
     prompts = synth.prompts(wl)
