@@ -189,6 +189,93 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, 4) void gemv_kernel(void* __restr
   }
 }
 
+// Gate/up GEMV with the SiLU epilogue as ONE workgroup per compute unit.  A unit takes in first-level-cache fills at a
+// bounded rate, weights and token block together, so a launch is as fast as its most loaded unit: here every unit gets
+// an equal share of the (gate tile, up tile) pairs - NP or NP - 1 of them - and reads the token block once for all of
+// them, instead of once per pair.  Same k-split over the 8 waves and the same fixed-order reduction as gemv_kernel, so
+// the result bits are the same.  The reduction goes through LDS one pair at a time.
+template <int NP, int TT, int PIPE>
+__global__ __launch_bounds__(GEMV_WAVES* WAVE, 2) void gemv_silu_cu_kernel(f16* __restrict__ act, const f16* __restrict__ x,
+                                                                        const f16* __restrict__ W, int T, int K, int I,
+                                                                        int base, int rem) {
+  constexpr int NT = 2 * NP;
+  __shared__ f32x4 red[GEMV_WAVES][2 * TT][WAVE];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int wg = blockIdx.x;
+  const int p0 = wg * base + (wg < rem ? wg : rem);    // first pair of this workgroup
+  const int np = base + (wg < rem ? 1 : 0);            // and how many it has
+  const int KB = K / KSTEP;
+  const f16* wp = W + ((size_t)(2 * p0) * KB) * 512 + lane * 8;
+  int woff[NT];                                        // a missing last pair repeats the first tile (cache hits) and is not stored
+#pragma unroll
+  for (int i = 0; i < NT; ++i) woff[i] = (i < 2 * np ? i : 0) * KB * 512;
+  const f16* xp = x + lane * 8;
+  constexpr int XSTEP = TT * 512;
+
+  f32x4 acc[NT][TT];
+#pragma unroll
+  for (int i = 0; i < NT; ++i)
+#pragma unroll
+    for (int j = 0; j < TT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int S = (KB - wave + GEMV_WAVES - 1) / GEMV_WAVES;
+  f16x8 a[PIPE][NT], b[PIPE][TT];
+  auto load_stage = [&](int u, int s) {
+    const bool in = s < S;
+    const int ks = in ? wave + GEMV_WAVES * s : 0;
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      a[u][i] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(wp + (woff[i] + ks * 512)));
+      if (!in) a[u][i] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int j = 0; j < TT; ++j) b[u][j] = ld8(xp + j * 512 + (size_t)ks * XSTEP);
+  };
+#pragma unroll
+  for (int u = 0; u < PIPE; ++u) load_stage(u, u);
+  for (int s0 = 0; s0 < S; s0 += PIPE) {
+#pragma unroll
+    for (int u = 0; u < PIPE; ++u) {
+#pragma unroll
+      for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int j = 0; j < TT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][i], b[u][j], acc[i][j], 0, 0, 0);
+      load_stage(u, s0 + u + PIPE);
+    }
+  }
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    if (p < np) {                                      // workgroup-uniform
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < TT; ++j) red[wave][h * TT + j][lane] = acc[2 * p + h][j];
+      __syncthreads();
+      for (int e = threadIdx.x; e < TT * WAVE; e += GEMV_WAVES * WAVE) {
+        const int j = e >> 6, sl = e & 63;
+        f32x4 sg = red[0][j][sl], su = red[0][TT + j][sl];
+#pragma unroll
+        for (int w = 1; w < GEMV_WAVES; ++w) {
+          sg += red[w][j][sl];
+          su += red[w][TT + j][sl];
+        }
+        const int c = (p0 + p) * 16 + (sl >> 4) * 4;   // output channel of the first of this lane's 4 rows
+        const int t = j * 16 + (sl & 15);
+        if (t < T && c < I) {
+          f16x4 o;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float gf = (float)(f16)sg[q];
+            o[q] = (f16)(gf / (1.f + expf(-gf)) * (float)(f16)su[q]);
+          }
+          *reinterpret_cast<f16x4*>(act + frag_offset(t, c, TT)) = o;
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
 // one thread per 16-byte chunk of the packed array
 __global__ __launch_bounds__(256) void pack_weight_kernel(f16* __restrict__ dst, const f16* __restrict__ src, int N, int K,
                                                           size_t chunks) {
@@ -396,6 +483,22 @@ extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p
   hipStream_t s = (hipStream_t)stream;
   const LoraShrinkBatch sb = LoraShrinkBatch();
   const dim3 grid(I / 16), block(GEMV_WAVES * WAVE);
+  // enough pairs for two or more per compute unit: one workgroup per unit with an equal share of the pairs
+  static const int n_cu = [] {
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cu = 0;
+    return cu;
+  }();
+  const int pairs = I / 16;
+  const int per = n_cu > 0 ? ceil_div(pairs, n_cu) : 0;
+  if (T > 16 && T <= 32 && n_cu > 0 && pairs >= 2 * n_cu && per <= 4) {
+    const int base = pairs / n_cu, rem = pairs % n_cu;
+    const dim3 g(n_cu);
+    if (per <= 2) hipLaunchKernelGGL((gemv_silu_cu_kernel<2, 2, 4>), g, block, 0, s, (f16*)act, xp, Wp, T, K, I, base, rem);
+    else if (per == 3) hipLaunchKernelGGL((gemv_silu_cu_kernel<3, 2, 3>), g, block, 0, s, (f16*)act, xp, Wp, T, K, I, base, rem);
+    else hipLaunchKernelGGL((gemv_silu_cu_kernel<4, 2, 2>), g, block, 0, s, (f16*)act, xp, Wp, T, K, I, base, rem);
+    return mlora_launch_status("gemv_frag_silu");
+  }
   if (T <= 16) hipLaunchKernelGGL((gemv_kernel<2, 1, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);
   else if (T <= 32) hipLaunchKernelGGL((gemv_kernel<2, 2, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);
   else hipLaunchKernelGGL((gemv_kernel<2, 4, OUT_SILU_FRAG, true, true, false, 2>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);
