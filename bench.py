@@ -463,7 +463,7 @@ def main():
     }
     if not args.no_extras:
         g = gemv_event_timing(model, wl.batch)
-        out["roofline"] = {"kernel": "gemv_kernel (fragment-ordered weights and activations, T=32; the 129 launches of one decode step, with the adapter A rows appended to qkv / o and the SiLU epilogue on gate/up)", "bound": "hbm", "achieved": g["gbs"],
+        out["roofline"] = {"kernel": "gemv_kernel / gemv_silu_cu_kernel (fragment-ordered weights and activations, T=32; the 129 GEMV launches of one decode step: adapter A rows appended to qkv / o, K split on o / down, SiLU epilogue on gate/up)", "bound": "hbm", "achieved": g["gbs"],
                            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g["gbs"] / HBM_PEAK_GBS, "traffic": profiled_gemv_traffic(),
                            "launches_timed": g["launches"], "avg_launch_us": g["avg_us"],
                            "algorithmic_bytes_per_launch": g["bytes_per_launch"]}
