@@ -89,6 +89,8 @@ def gather_mm(y, x, A, B, tok_adapter, scaling: float, workspace=None):
     if K2 != K or B.shape != (n_ad, N, r) or y.shape != (T, N) or tok_adapter.shape != (T,):
         raise ValueError(f"gather_mm: inconsistent shapes y{tuple(y.shape)} x{tuple(x.shape)} A{tuple(A.shape)} "
                          f"B{tuple(B.shape)} ids{tuple(tok_adapter.shape)}")
+    if T == 0:
+        return y                                   # an empty batch: nothing to add (an empty tensor has no device pointer)
     if workspace is None:
         workspace = gather_mm_workspace(T, K, r, x.device)
     if not y.is_cuda or y.stride(1) != 1:
@@ -237,6 +239,10 @@ def linear(x, W, out=None, out_dtype=torch.float16, accumulate=False, kernel="au
     N, K2 = W.shape
     if K2 != K:
         raise ValueError(f"linear: x{tuple(x.shape)} vs W{tuple(W.shape)}")
+    if T == 0:                                     # an empty batch
+        if out is None:
+            out = torch.empty((0, N), dtype=torch.float32 if accumulate else out_dtype, device=x.device)
+        return out
     rm = W.rowmajor if packed else W
     if kernel == "library" or (kernel == "auto" and packed and rm is not None and T >= LIBRARY_GEMM_MIN_T
                                and K % 8 == 0 and N % 8 == 0):
@@ -354,6 +360,8 @@ def rmsnorm(x, w, eps: float, out=None, frag=False, parts: KSplitParts = None):
     """Row-wise RMSNorm of x [T, H] (f16 | f32); frag=True writes a FragActivation.  With `parts` (x fp32) the K-split
     partials are first added to x in place."""
     T, H = x.shape
+    if T == 0 and not frag:
+        return torch.empty((0, H), dtype=torch.float16, device=x.device) if out is None else out
     out, optr, lay = _out_arg(out, T, H, frag, x.device)
     if parts is not None:
         check(lib().mlora_rmsnorm_ksplit(optr, lay, _dev(x, torch.float32), _dev(parts.part, torch.float32), parts.ks, parts.ld,
@@ -367,6 +375,8 @@ def silu_mul(gate_up, out=None, frag=False):
     """gate_up [T, 2I] (gate columns first) -> silu(gate) * up [T, I]."""
     T, I2 = gate_up.shape
     I = I2 // 2
+    if T == 0 and not frag:
+        return torch.empty((0, I), dtype=torch.float16, device=gate_up.device) if out is None else out
     out, optr, lay = _out_arg(out, T, I, frag, gate_up.device)
     p = _dev(gate_up, torch.float16)
     check(lib().mlora_silu_mul(optr, lay, p, p + I * 2, I2, T, I, _stream()))
@@ -386,6 +396,8 @@ def embed(table, ids, out_dtype=torch.float32, out=None):
     V, H = table.shape
     if out is None:
         out = torch.empty((T, H), dtype=out_dtype, device=table.device)
+    if T == 0:
+        return out
     check(lib().mlora_embed(_dev(out), _dt(out), _dev(table, torch.float16), _dev(ids, torch.int32), T, H, V, _stream()))
     return out
 
@@ -394,6 +406,8 @@ def argmax(logits, out=None):
     B, V = logits.shape
     if out is None:
         out = torch.empty((B,), dtype=torch.int32, device=logits.device)
+    if B == 0:
+        return out
     check(lib().mlora_argmax(_dev(out, torch.int32), _dev(logits, torch.float32), B, V, _stream()))
     return out
 

@@ -704,3 +704,21 @@ def test_library_gemm_matches_oracle(ops, synth, T, K, N):
     ys = ops.linear(xw[:, :K], W, kernel="library")
     torch.cuda.synchronize()
     assert max_rel_err(_np(ys), _np(xw[:, :K]).astype(np.float64) @ _np(W).astype(np.float64).T) <= TOL
+
+
+def test_empty_batches(ops, synth):
+    """Zero tokens: every row-wise operator returns an empty result and touches nothing."""
+    K, N, r = 64, 48, 8
+    x = torch.empty((0, K), dtype=torch.float16, device=DEV)
+    W = synth.normal(43, "e.W", (N, K), 0.02, torch.float16, DEV)
+    assert ops.linear(x, W).shape == (0, N)
+    assert ops.linear(x, ops.PackedWeight(W, keep_rowmajor=True)).shape == (0, N)
+    y = torch.empty((0, N), dtype=torch.float16, device=DEV)
+    A = synth.normal(43, "e.A", (2, r, K), 0.02, torch.float16, DEV)
+    B = synth.normal(43, "e.B", (2, N, r), 0.02, torch.float16, DEV)
+    assert ops.gather_mm(y, x, A, B, torch.empty((0,), dtype=torch.int32, device=DEV), 0.5) is y
+    assert ops.rmsnorm(torch.empty((0, K), dtype=torch.float32, device=DEV), W[0, :K].contiguous(), 1e-5).shape == (0, K)
+    assert ops.silu_mul(torch.empty((0, 2 * N), dtype=torch.float16, device=DEV)).shape == (0, N)
+    assert ops.embed(W, torch.empty((0,), dtype=torch.int32, device=DEV)).shape == (0, K)
+    assert ops.argmax(torch.empty((0, 100), dtype=torch.float32, device=DEV)).shape == (0,)
+    torch.cuda.synchronize()
