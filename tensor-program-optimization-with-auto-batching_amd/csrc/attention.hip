@@ -399,19 +399,27 @@ __global__ __launch_bounds__(ATT_WAVES * WAVE, 4) void rope_attn_decode_kernel(
   const int id = lora ? lx.ids[b] : -1;
   const bool adapted = lora && id >= 0 && id < lx.n_ad;
 
-  // The wave's first page is requested before anything else, so that its latency overlaps the work on the new token.
+  // The wave's first TWO pages are requested before anything else: together with the other waves' that is enough traffic
+  // to keep the memory system busy for the whole time the new token takes (the second buffer lives in registers the
+  // accumulators only need later, and is gone after the second page).
+  constexpr bool PF2 = RG <= 2;      // the wide-rank variant has no registers to spare for the second buffer
   int page = wave < npages ? bt[wave] : -1;
-  f16x8 kf[NKB];
-  f16x4 vf[NDB];
-  auto load_page = [&](int pgid) {
+  const int page2 = PF2 && wave + NW < npages ? bt[wave + NW] : -1;
+  f16x8 kf[NKB], kf2[PF2 ? NKB : 1];
+  f16x4 vf[NDB], vf2[PF2 ? NDB : 1];
+  auto load_into = [&](f16x8 (&k)[NKB], f16x4 (&v)[NDB], int pgid) {
     const f16* kp = k_cache + ((size_t)pgid * Hkv + kh) * PAGE * D + lane * 8;
     const f16* vp = v_cache + (((size_t)pgid * Hkv + kh) * D + col) * PAGE + g * 4;   // dim col (+16 db), tokens 4g..
 #pragma unroll
-    for (int kb = 0; kb < NKB; ++kb) kf[kb] = ld8(kp + kb * 512);
+    for (int kb = 0; kb < NKB; ++kb) k[kb] = ld8(kp + kb * 512);
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) vf[db] = *reinterpret_cast<const f16x4*>(vp + db * 16 * PAGE);
+    for (int db = 0; db < NDB; ++db) v[db] = *reinterpret_cast<const f16x4*>(vp + db * 16 * PAGE);
   };
+  auto load_page = [&](int pgid) { load_into(kf, vf, pgid); };
   if (page >= 0 && page < n_pages) load_page(page);
+  if constexpr (PF2) {
+    if (page2 >= 0 && page2 < n_pages) load_into(kf2, vf2, page2);
+  }
 
   // ---- the new token: heads kh*G .. kh*G+G-1 of q, head kh of k and of v; one (head, pair) item per thread and pass.
   // An item's loads (projection output, rows of B, rotation factors) do not depend on the shrink results, so the
@@ -498,71 +506,79 @@ __global__ __launch_bounds__(ATT_WAVES * WAVE, 4) void rope_attn_decode_kernel(
   }
   __syncthreads();
 
-  // Q^T as the B operand, from LDS: lane holds q[head col][kb*32 + g*8 .. +8], zero for unused columns
-  f16x8 qf[NKB];
-#pragma unroll
-  for (int kb = 0; kb < NKB; ++kb)
-    qf[kb] = col < G ? *reinterpret_cast<const f16x8*>(&qs[col * D + kb * 32 + g * 8]) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-
   float m = -INFINITY, l = 0.f;
   f32x4 O[NDB];
 #pragma unroll
   for (int db = 0; db < NDB; ++db) O[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int pg = wave; pg < npages; pg += NW) {
-    const int next = pg + NW < npages ? bt[pg + NW] : -1;
+  // one page: scores against the rotated queries (Q^T as the B operand, read from LDS: lane holds
+  // q[head col][kb*32 + g*8 .. +8], zero for unused columns), online softmax, value accumulation
+  auto process = [&](f16x8 (&k)[NKB], f16x4 (&v)[NDB], int pg) {
+    if (pg == new_pg) {                                   // wave-uniform: this page holds the token appended above
+      if (col == new_slot) {
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb) k[kb] = *reinterpret_cast<const f16x8*>(&knew[kb * 32 + g * 8]);
+      }
+      if ((new_slot >> 2) == g) {
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+          const f16 nv = vnew[db * 16 + col];
+          const int e = new_slot & 3;
+          v[db][0] = e == 0 ? nv : v[db][0];
+          v[db][1] = e == 1 ? nv : v[db][1];
+          v[db][2] = e == 2 ? nv : v[db][2];
+          v[db][3] = e == 3 ? nv : v[db][3];
+        }
+      }
+    }
+    f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) {
+      const f16x8 qf = col < G ? *reinterpret_cast<const f16x8*>(&qs[col * D + kb * 32 + g * 8]) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      st = __builtin_amdgcn_mfma_f32_16x16x32_f16(k[kb], qf, st, 0, 0, 0);
+    }
+    float pm = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      st[r] = (pg * PAGE + 4 * g + r >= ctx) ? -INFINITY : st[r] * scale;
+      pm = fmaxf(pm, st[r]);
+    }
+    pm = fmaxf(pm, __shfl_xor(pm, 16, WAVE));
+    pm = fmaxf(pm, __shfl_xor(pm, 32, WAVE));
+    const float m_new = fmaxf(m, pm);
+    const float alpha = __expf(m - m_new);
+    f16x8 pa;
+    float ps = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float p = __expf(st[r] - m_new);
+      ps += p;
+      const f16 hi = (f16)p;
+      pa[r] = hi;
+      pa[4 + r] = (f16)(p - (float)hi);
+    }
+    l = l * alpha + ps;
+    m = m_new;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+      O[db] *= alpha;
+      const f16x8 vv = f16x8{v[db][0], v[db][1], v[db][2], v[db][3], v[db][0], v[db][1], v[db][2], v[db][3]};
+      O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vv, pa, O[db], 0, 0, 0);
+    }
+  };
+  // the two pages requested at the start, then one page at a time with the next page id requested one page ahead
+  constexpr int AHEAD = PF2 ? 2 : 1;
+  int next = wave + AHEAD * NW < npages ? bt[wave + AHEAD * NW] : -1;
+  if (page >= 0 && page < n_pages) process(kf, vf, wave);
+  if constexpr (PF2) {
+    if (page2 >= 0 && page2 < n_pages) process(kf2, vf2, wave + NW);
+  }
+  page = next;
+  for (int pg = wave + AHEAD * NW; pg < npages; pg += NW) {
+    next = pg + NW < npages ? bt[pg + NW] : -1;
     if (page >= 0 && page < n_pages) {                      // wave-uniform
-      if (pg != wave) load_page(page);                      // the first page is already on its way
-      if (pg == new_pg) {                                   // wave-uniform: this page holds the token appended above
-        if (col == new_slot) {
-#pragma unroll
-          for (int kb = 0; kb < NKB; ++kb) kf[kb] = *reinterpret_cast<const f16x8*>(&knew[kb * 32 + g * 8]);
-        }
-        if ((new_slot >> 2) == g) {
-#pragma unroll
-          for (int db = 0; db < NDB; ++db) {
-            const f16 nv = vnew[db * 16 + col];
-            const int e = new_slot & 3;
-            vf[db][0] = e == 0 ? nv : vf[db][0];
-            vf[db][1] = e == 1 ? nv : vf[db][1];
-            vf[db][2] = e == 2 ? nv : vf[db][2];
-            vf[db][3] = e == 3 ? nv : vf[db][3];
-          }
-        }
-      }
-
-      f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kb = 0; kb < NKB; ++kb) st = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kb], qf[kb], st, 0, 0, 0);
-
-      float pm = -INFINITY;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        st[r] = (pg * PAGE + 4 * g + r >= ctx) ? -INFINITY : st[r] * scale;
-        pm = fmaxf(pm, st[r]);
-      }
-      pm = fmaxf(pm, __shfl_xor(pm, 16, WAVE));
-      pm = fmaxf(pm, __shfl_xor(pm, 32, WAVE));
-      const float m_new = fmaxf(m, pm);
-      const float alpha = __expf(m - m_new);
-      f16x8 pa;
-      float ps = 0.f;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float p = __expf(st[r] - m_new);
-        ps += p;
-        const f16 hi = (f16)p;
-        pa[r] = hi;
-        pa[4 + r] = (f16)(p - (float)hi);
-      }
-      l = l * alpha + ps;
-      m = m_new;
-#pragma unroll
-      for (int db = 0; db < NDB; ++db) {
-        O[db] *= alpha;
-        const f16x8 vv = f16x8{vf[db][0], vf[db][1], vf[db][2], vf[db][3], vf[db][0], vf[db][1], vf[db][2], vf[db][3]};
-        O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vv, pa, O[db], 0, 0, 0);
-      }
+      load_page(page);
+      process(kf, vf, pg);
     }
     page = next;
   }
