@@ -113,10 +113,12 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qk
   }
 }
 
-// Prefill-sized variant that writes whole page rows: one workgroup per (16 consecutive tokens, head).  When the 16
-// tokens are slots 0..15 of one page (prompts that start on a page boundary), a K fragment row (16 tokens x 16 B) and
-// a V row (16 tokens of one dim, 32 B) are written as contiguous pieces instead of 2 bytes at a time; other tiles fall
-// back to element-wise writes.  Same arithmetic per element as rope_kv_append_kernel.
+// Prefill-sized variant that moves 16 bytes at a time: one WAVE per (16 consecutive tokens, head), four heads per
+// workgroup, no barriers and no LDS.  Lane l works on token l % 16 of the tile throughout, so its sequence and
+// position stay in its own registers.  q heads are rotated in place in chunks of 8 pairs.  When the 16 tokens are
+// slots 0..15 of one page (prompts that start on a page boundary), a K fragment row (16 tokens x 16 B) and a V row
+// (16 tokens of one dim, 32 B) are written as contiguous pieces; other tiles fall back to element-wise writes.
+// Same arithmetic per element as rope_kv_append_kernel.  rope_cos / rope_sin must be 16-byte aligned.
 template <int D>
 __global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restrict__ qkv, f16* __restrict__ k_cache,
                                                                   f16* __restrict__ v_cache,
@@ -127,34 +129,19 @@ __global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restric
                                                                   const float* __restrict__ rope_sin, int max_pos, int Hq,
                                                                   int Hkv, int n_pages, int n_seq, int T) {
   constexpr int half = D / 2;
-  __shared__ int s_seq[16], s_pos[16];
-  __shared__ int s_aligned, s_page;
-  const int t0 = blockIdx.x * 16, hh = blockIdx.y;            // hh < Hq: a q head; else kv head hh - Hq (k and v)
+  constexpr int NCH = half / 8;                               // 8-pair chunks of a head row
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int t0 = blockIdx.x * 16;
+  const int hh = blockIdx.y * 4 + wave;                       // hh < Hq: a q head; else kv head hh - Hq (k and v)
   const int HH = Hq + 2 * Hkv;
-  if (threadIdx.x < 16) {
-    const int t = t0 + threadIdx.x;
-    int seq = -1, pos = -1;
-    if (t < T) {
-      seq = tok_seq[t];
-      pos = tok_pos[t];
-      if (seq < 0 || seq >= n_seq || pos < 0 || pos >= max_pos || pos / PAGE >= max_blocks) seq = -1;
-    }
-    s_seq[threadIdx.x] = seq;
-    s_pos[threadIdx.x] = pos;
+  if (hh >= Hq + Hkv) return;
+  const int tk = lane & 15, t = t0 + tk;
+  int seq = -1, pos = -1;
+  if (t < T) {
+    seq = tok_seq[t];
+    pos = tok_pos[t];
+    if (seq < 0 || seq >= n_seq || pos < 0 || pos >= max_pos || pos / PAGE >= max_blocks) seq = -1;
   }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    bool al = s_seq[0] >= 0 && (s_pos[0] % PAGE) == 0;
-    for (int i = 1; i < 16 && al; ++i) al = s_seq[i] == s_seq[0] && s_pos[i] == s_pos[0] + i;
-    int page = -1;
-    if (al) {
-      page = block_table[(size_t)s_seq[0] * max_blocks + s_pos[0] / PAGE];
-      if (page < 0 || page >= n_pages) al = false;
-    }
-    s_aligned = al;
-    s_page = page;
-  }
-  __syncthreads();
   // rotation of one element d of a head row (x1 = first-half element, x2 = its partner in the second half)
   auto rot = [&](float x1, float x2, float c, float s, bool second) -> f16 {
     float r;
@@ -165,61 +152,76 @@ __global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restric
     asm volatile("" : "+v"(r));
     return (f16)r;
   };
-  if (hh < Hq) {                                              // q: rotate in place, 16 tokens x D/2 pairs
-    for (int it = threadIdx.x; it < 16 * half; it += 256) {
-      const int tk = it / half, i = it % half;
-      if (s_seq[tk] < 0) continue;
-      f16* src = qkv + ((size_t)(t0 + tk) * HH + hh) * D;
-      const float c = rope_cos[(size_t)s_pos[tk] * half + i], s = rope_sin[(size_t)s_pos[tk] * half + i];
-      const float x1 = (float)src[i], x2 = (float)src[i + half];
-      src[i] = rot(x1, x2, c, s, false);
-      src[i + half] = rot(x1, x2, c, s, true);
+  // chunk ch of the lane's token: pairs 8 ch .. 8 ch + 7 of a head row at src, rotated
+  auto rot_chunk = [&](const f16* src, int ch, f16x8& o_lo, f16x8& o_hi) {
+    const int p0 = ch * 8;
+    const f16x8 lo = ld8(src + p0), hi = ld8(src + p0 + half);
+    const float* cp = rope_cos + (size_t)pos * half + p0;
+    const float* sp = rope_sin + (size_t)pos * half + p0;
+    const f32x4 c0 = *reinterpret_cast<const f32x4*>(cp), c1 = *reinterpret_cast<const f32x4*>(cp + 4);
+    const f32x4 s0 = *reinterpret_cast<const f32x4*>(sp), s1 = *reinterpret_cast<const f32x4*>(sp + 4);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float c = e < 4 ? c0[e & 3] : c1[e & 3], sn = e < 4 ? s0[e & 3] : s1[e & 3];
+      o_lo[e] = rot((float)lo[e], (float)hi[e], c, sn, false);
+      o_hi[e] = rot((float)lo[e], (float)hi[e], c, sn, true);
+    }
+  };
+  if (hh < Hq) {                                              // q: rotate in place
+    if (seq < 0) return;
+    f16* src = qkv + ((size_t)t * HH + hh) * D;
+    for (int ch = lane >> 4; ch < NCH; ch += 4) {
+      f16x8 o_lo, o_hi;
+      rot_chunk(src, ch, o_lo, o_hi);
+      st8(src + ch * 8, o_lo);
+      st8(src + ch * 8 + half, o_hi);
     }
     return;
   }
   const int kh = hh - Hq;
-  if (s_aligned) {
-    const int page = s_page;
-    // K: one 16-byte fragment chunk (8 dims of one token) per item; 16 tokens of a chunk row are contiguous
-    for (int it = threadIdx.x; it < (D / 8) * 16; it += 256) {
-      const int tk = it & 15, ch = it >> 4;                   // ch = ks * 4 + g: dims 8 ch .. 8 ch + 7
-      const int d0 = ch * 8;
-      const bool second = d0 >= half;
-      const int p0 = second ? d0 - half : d0;                 // pair index of the first of the 8 dims
-      const f16* src = qkv + ((size_t)(t0 + tk) * HH + Hq + kh) * D;
-      const f16x8 lo = ld8(src + p0), hi = ld8(src + p0 + half);
-      const float* cp = rope_cos + (size_t)s_pos[tk] * half + p0;
-      const float* sp = rope_sin + (size_t)s_pos[tk] * half + p0;
-      f16x8 o;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] = rot((float)lo[e], (float)hi[e], cp[e], sp[e], second);
-      st8(k_cache + ((size_t)page * Hkv + kh) * PAGE * D + ((size_t)ch * 16 + tk) * 8, o);
+  const int seq0 = __shfl(seq, 0, WAVE), pos0 = __shfl(pos, 0, WAVE);
+  bool al = __ballot(seq >= 0 && seq == seq0 && pos == pos0 + tk) == ~0ull && (pos0 % PAGE) == 0;   // wave-uniform
+  int page = -1;
+  if (al) {
+    page = block_table[(size_t)seq0 * max_blocks + pos0 / PAGE];
+    if (page < 0 || page >= n_pages) al = false;
+  }
+  if (al) {
+    // K: the 16 tokens of a fragment chunk row are contiguous (16 B each)
+    const f16* ksrc = qkv + ((size_t)t * HH + Hq + kh) * D;
+    f16* kd = k_cache + ((size_t)page * Hkv + kh) * PAGE * D;
+    for (int ch = lane >> 4; ch < NCH; ch += 4) {
+      f16x8 o_lo, o_hi;
+      rot_chunk(ksrc, ch, o_lo, o_hi);
+      st8(kd + ((size_t)ch * 16 + tk) * 8, o_lo);
+      st8(kd + ((size_t)(ch + NCH) * 16 + tk) * 8, o_hi);
     }
-    // V: 8 tokens of one dim per item (16 bytes of the dim's 32-byte row)
-    for (int it = threadIdx.x; it < D * 2; it += 256) {
-      const int d = it % D, tg = it / D;
+    // V: 8 tokens of one dim per item; a pair of lanes writes the dim's 32-byte row
+    f16* vd = v_cache + ((size_t)page * Hkv + kh) * D * PAGE;
+    for (int it = lane; it < D * 2; it += WAVE) {
+      const int d = it >> 1, tg = it & 1;
       f16x8 o;
 #pragma unroll
       for (int j = 0; j < 8; ++j) o[j] = qkv[((size_t)(t0 + tg * 8 + j) * HH + Hq + Hkv + kh) * D + d];
-      st8(v_cache + (((size_t)page * Hkv + kh) * D + d) * PAGE + tg * 8, o);
+      st8(vd + (size_t)d * PAGE + tg * 8, o);
     }
     return;
   }
-  for (int it = threadIdx.x; it < 16 * half; it += 256) {      // element-wise: tokens of several pages or sequences
-    const int tk = it / half, i = it % half;
-    if (s_seq[tk] < 0) continue;
-    const int pos = s_pos[tk];
-    const int page = block_table[(size_t)s_seq[tk] * max_blocks + pos / PAGE];
-    if (page < 0 || page >= n_pages) continue;
-    const int slot = pos % PAGE;
-    const f16* ksrc = qkv + ((size_t)(t0 + tk) * HH + Hq + kh) * D;
-    const f16* vsrc = qkv + ((size_t)(t0 + tk) * HH + Hq + Hkv + kh) * D;
-    const float c = rope_cos[(size_t)pos * half + i], s = rope_sin[(size_t)pos * half + i];
+  for (int it = lane; it < 16 * half; it += WAVE) {           // element-wise: tokens of several pages or sequences
+    const int tke = it / half, i = it % half;
+    const int seq_e = __shfl(seq, tke, WAVE), pos_e = __shfl(pos, tke, WAVE);
+    if (seq_e < 0) continue;
+    const int pg = block_table[(size_t)seq_e * max_blocks + pos_e / PAGE];
+    if (pg < 0 || pg >= n_pages) continue;
+    const int slot = pos_e % PAGE;
+    const f16* ksrc = qkv + ((size_t)(t0 + tke) * HH + Hq + kh) * D;
+    const f16* vsrc = qkv + ((size_t)(t0 + tke) * HH + Hq + Hkv + kh) * D;
+    const float c = rope_cos[(size_t)pos_e * half + i], s = rope_sin[(size_t)pos_e * half + i];
     const float x1 = (float)ksrc[i], x2 = (float)ksrc[i + half];
-    f16* kd = k_cache + ((size_t)page * Hkv + kh) * PAGE * D;
+    f16* kd = k_cache + ((size_t)pg * Hkv + kh) * PAGE * D;
     kd[k_page_offset(slot, i)] = rot(x1, x2, c, s, false);
     kd[k_page_offset(slot, i + half)] = rot(x1, x2, c, s, true);
-    f16* vd = v_cache + ((size_t)page * Hkv + kh) * D * PAGE + slot;
+    f16* vd = v_cache + ((size_t)pg * Hkv + kh) * D * PAGE + slot;
     vd[(size_t)i * PAGE] = vsrc[i];
     vd[(size_t)(i + half) * PAGE] = vsrc[i + half];
   }
@@ -753,8 +755,8 @@ static int rope_kv_append_impl(const char* who, void* qkv, void* k_cache, void* 
   MLORA_CHECK(qkv && k_cache && v_cache && block_table && tok_seq && tok_pos && rope_cos && rope_sin, MLORA_ERR_INVALID, "%s: null pointer", who);
   MLORA_CHECK(T >= 0 && max_pos > 0, MLORA_ERR_INVALID, "%s: bad T=%d max_pos=%d", who, T, max_pos);
   if (T == 0) return MLORA_OK;
-  if (T > 64 && lx.src.v == nullptr) {
-    const dim3 grid(ceil_div(T, 16), Hq + Hkv);
+  if (T > 64 && lx.src.v == nullptr && (((uintptr_t)rope_cos | (uintptr_t)rope_sin) & 15) == 0) {
+    const dim3 grid(ceil_div(T, 16), ceil_div(Hq + Hkv, 4));
     if (D == 128)
       hipLaunchKernelGGL(rope_kv_append_tile_kernel<128>, grid, dim3(256), 0, (hipStream_t)stream, (f16*)qkv, (f16*)k_cache,
                          (f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, rope_cos, rope_sin, max_pos, Hq, Hkv, n_pages,
