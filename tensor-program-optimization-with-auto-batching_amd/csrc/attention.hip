@@ -252,7 +252,7 @@ __global__ __launch_bounds__(ATT_WAVES * WAVE, 4) void paged_attn_decode_kernel(
   __shared__ float sm[NW][16], sl[NW][16];
   extern __shared__ float sacc[];   // [NW][G][D]
 
-  const int b = blockIdx.x, kh = blockIdx.y;
+  const int b = blockIdx.y, kh = blockIdx.x;
   const int G = Hq / Hkv;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
@@ -382,7 +382,7 @@ __global__ __launch_bounds__(ATT_WAVES * WAVE, 4) void rope_attn_decode_kernel(
   __shared__ __align__(16) f16 knew[D], vnew[D];   // the new token's rotated key and its value
   extern __shared__ float sacc[];                  // [NW][G][D]
 
-  const int b = blockIdx.x, kh = blockIdx.y;
+  const int b = blockIdx.y, kh = blockIdx.x;
   const int G = Hq / Hkv;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
@@ -808,7 +808,7 @@ extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qk
                                        void* stream) {
   if (int e = check_attn("paged_attn_decode", Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
   MLORA_CHECK(out && qkv && k_cache && v_cache && block_table && seq_ids && ctx_len, MLORA_ERR_INVALID, "paged_attn_decode: null pointer");
-  MLORA_CHECK(B >= 0, MLORA_ERR_INVALID, "paged_attn_decode: bad B=%d", B);
+  MLORA_CHECK(B >= 0 && B <= 65535, MLORA_ERR_INVALID, "paged_attn_decode: bad B=%d (0..65535)", B);
   MLORA_CHECK(out_layout == MLORA_ROWMAJOR || (out_layout == MLORA_FRAG && B <= 64), MLORA_ERR_UNSUPPORTED,
               "paged_attn_decode: fragment-ordered output needs B <= 64 (layout=%d B=%d)", out_layout, B);
   const int frag_tt = out_layout == MLORA_FRAG ? mlora_frag_tiles(B) : 0;
@@ -819,10 +819,10 @@ extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qk
   MLORA_CHECK(G <= 16, MLORA_ERR_UNSUPPORTED, "paged_attn_decode: more than 16 query heads per kv head (%d)", G);
   const size_t lds = (size_t)ATT_WAVES * G * D * sizeof(float);
   if (D == 128)
-    hipLaunchKernelGGL(paged_attn_decode_kernel<128>, dim3(B, Hkv), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
+    hipLaunchKernelGGL(paged_attn_decode_kernel<128>, dim3(Hkv, B), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
                        (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale, frag_tt);
   else
-    hipLaunchKernelGGL(paged_attn_decode_kernel<64>, dim3(B, Hkv), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
+    hipLaunchKernelGGL(paged_attn_decode_kernel<64>, dim3(Hkv, B), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
                        (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale, frag_tt);
   return mlora_launch_status("paged_attn_decode");
 }
@@ -860,7 +860,7 @@ extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv
   const size_t lds = (size_t)ATT_WAVES * G * D * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
 #define MLORA_ROPE_ATTN(DD, RG)                                                                                              \
-  hipLaunchKernelGGL((rope_attn_decode_kernel<DD, RG>), dim3(B, Hkv), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, \
+  hipLaunchKernelGGL((rope_attn_decode_kernel<DD, RG>), dim3(Hkv, B), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, \
                      (f16*)k_cache, (f16*)v_cache, block_table, max_blocks, seq_ids, tok_pos, ctx_len, rope_cos, rope_sin,       \
                      max_pos, Hq, Hkv, n_pages, n_seq, scale, frag_tt, lx)
   const bool small_rank = v_part == nullptr || r <= 16;
