@@ -218,7 +218,7 @@ int mlora_argmax(int32_t* ids, const float* logits, int B, int V, void* stream);
  * mlora_paged_attn_prefill: query token t (sequence tok_seq[t], position tok_pos[t]) attends to cached
  *   positions 0..tok_pos[t]; tokens of a sequence must be consecutive in t with increasing positions.
  * q is read from qkv (already rotated).  out [T, Hq * D] f16 (decode: in out_layout).  D in {64, 128};
- * Hq % Hkv == 0, Hq / Hkv <= 16 for decode.
+ * Hq % Hkv == 0, Hq / Hkv <= 16 and B <= 65535 for decode.
  * ------------------------------------------------------------------------------------------- */
 int mlora_rope_kv_append(void* qkv, void* k_cache, void* v_cache,
                          const int32_t* block_table, int max_blocks,

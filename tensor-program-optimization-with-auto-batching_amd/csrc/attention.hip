@@ -836,7 +836,7 @@ extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv
   if (int e = check_attn("rope_attn_decode", Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
   MLORA_CHECK(out && qkv && k_cache && v_cache && block_table && seq_ids && tok_pos && ctx_len && rope_cos && rope_sin,
               MLORA_ERR_INVALID, "rope_attn_decode: null pointer");
-  MLORA_CHECK(B >= 0 && max_pos > 0, MLORA_ERR_INVALID, "rope_attn_decode: bad B=%d max_pos=%d", B, max_pos);
+  MLORA_CHECK(B >= 0 && B <= 65535 && max_pos > 0, MLORA_ERR_INVALID, "rope_attn_decode: bad B=%d (0..65535) max_pos=%d", B, max_pos);
   MLORA_CHECK(out_layout == MLORA_ROWMAJOR || (out_layout == MLORA_FRAG && B <= 64), MLORA_ERR_UNSUPPORTED,
               "rope_attn_decode: fragment-ordered output needs B <= 64 (layout=%d B=%d)", out_layout, B);
   const int G = Hq / Hkv;
