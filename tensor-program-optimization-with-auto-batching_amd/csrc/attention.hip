@@ -241,14 +241,23 @@ __global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restric
 // ---------------------------------------------------------------------------------------------
 constexpr int ATT_WAVES = 4;
 
-template <int D>
-__global__ __launch_bounds__(ATT_WAVES * WAVE, 4) void paged_attn_decode_kernel(
+// Waves per workgroup of the decode kernels: four when the launch has workgroups enough to fill the chip four deep
+// (every CU then holds 16 waves, one page each in flight), more when sequences x kv heads are few (small batches,
+// grouped-query models), so that a CU still has 16 pages in flight.  Limited by the LDS merge buffer [NW][G][D].
+int attn_waves(int B, int Hkv, int G, int D) {
+  const long wgs = (long)B * Hkv;
+  int nw = wgs > 512 ? ATT_WAVES : wgs > 256 ? 8 : 16;
+  while (nw > ATT_WAVES && (size_t)nw * G * D * sizeof(float) > 48 * 1024) nw >>= 1;
+  return nw;
+}
+
+template <int D, int NW>   // NW waves per workgroup share the pages of one (sequence, kv head)
+__global__ __launch_bounds__(NW * WAVE, 4) void paged_attn_decode_kernel(
     f16* __restrict__ out, const f16* __restrict__ qkv, const f16* __restrict__ k_cache, const f16* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ seq_ids,
     const int32_t* __restrict__ ctx_len, int Hq, int Hkv, int n_pages, int n_seq, float scale, int frag_tt) {
   constexpr int NKB = D / 32;   // k-blocks of the QK^T product
   constexpr int NDB = D / 16;   // dim blocks of the output
-  constexpr int NW = ATT_WAVES;
   __shared__ float sm[NW][16], sl[NW][16];
   extern __shared__ float sacc[];   // [NW][G][D]
 
@@ -365,8 +374,8 @@ __global__ __launch_bounds__(ATT_WAVES * WAVE, 4) void paged_attn_decode_kernel(
 // depends on reading back what the workgroup has just stored.  Results are those of the two separate kernels,
 // bit for bit; the q rows of qkv are left unrotated.
 // ---------------------------------------------------------------------------------------------
-template <int D, int RG>   // RG: 8-wide rank groups the B-row registers hold (rank <= 8 RG)
-__global__ __launch_bounds__(ATT_WAVES * WAVE, 4) void rope_attn_decode_kernel(
+template <int D, int RG, int NW>   // RG: 8-wide rank groups the B-row registers hold (rank <= 8 RG); NW: waves per workgroup
+__global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
     f16* __restrict__ out, const f16* __restrict__ qkv, f16* __restrict__ k_cache, f16* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ seq_ids,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ ctx_len, const float* __restrict__ rope_cos,
@@ -374,7 +383,6 @@ __global__ __launch_bounds__(ATT_WAVES * WAVE, 4) void rope_attn_decode_kernel(
     LoraExpandQKV lx) {
   constexpr int NKB = D / 32;
   constexpr int NDB = D / 16;
-  constexpr int NW = ATT_WAVES;
   constexpr int half = D / 2;
   __shared__ float sm[NW][16], sl[NW][16];
   __shared__ float lv[3][64];
@@ -817,13 +825,22 @@ extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qk
   hipStream_t s = (hipStream_t)stream;
   const int G = Hq / Hkv;
   MLORA_CHECK(G <= 16, MLORA_ERR_UNSUPPORTED, "paged_attn_decode: more than 16 query heads per kv head (%d)", G);
-  const size_t lds = (size_t)ATT_WAVES * G * D * sizeof(float);
-  if (D == 128)
-    hipLaunchKernelGGL(paged_attn_decode_kernel<128>, dim3(Hkv, B), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
-                       (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale, frag_tt);
-  else
-    hipLaunchKernelGGL(paged_attn_decode_kernel<64>, dim3(Hkv, B), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
-                       (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages, n_seq, scale, frag_tt);
+  const int nw = attn_waves(B, Hkv, G, D);
+  const size_t lds = (size_t)nw * G * D * sizeof(float);
+#define MLORA_ATTN(DD, NWV)                                                                                                   \
+  hipLaunchKernelGGL((paged_attn_decode_kernel<DD, NWV>), dim3(Hkv, B), dim3(NWV * WAVE), lds, s, (f16*)out, (const f16*)qkv, \
+                     (const f16*)k_cache, (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages,   \
+                     n_seq, scale, frag_tt)
+  if (D == 128) {
+    if (nw == 16) MLORA_ATTN(128, 16);
+    else if (nw == 8) MLORA_ATTN(128, 8);
+    else MLORA_ATTN(128, 4);
+  } else {
+    if (nw == 16) MLORA_ATTN(64, 16);
+    else if (nw == 8) MLORA_ATTN(64, 8);
+    else MLORA_ATTN(64, 4);
+  }
+#undef MLORA_ATTN
   return mlora_launch_status("paged_attn_decode");
 }
 
@@ -857,20 +874,28 @@ extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv
   if (B == 0) return MLORA_OK;
   const int frag_tt = out_layout == MLORA_FRAG ? mlora_frag_tiles(B) : 0;
   const float scale = 1.f / sqrtf((float)D);
-  const size_t lds = (size_t)ATT_WAVES * G * D * sizeof(float);
+  const int nw = attn_waves(B, Hkv, G, D);
+  const size_t lds = (size_t)nw * G * D * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
-#define MLORA_ROPE_ATTN(DD, RG)                                                                                              \
-  hipLaunchKernelGGL((rope_attn_decode_kernel<DD, RG>), dim3(Hkv, B), dim3(ATT_WAVES * WAVE), lds, s, (f16*)out, (const f16*)qkv, \
+#define MLORA_ROPE_ATTN(DD, RG, NWV)                                                                                             \
+  hipLaunchKernelGGL((rope_attn_decode_kernel<DD, RG, NWV>), dim3(Hkv, B), dim3(NWV * WAVE), lds, s, (f16*)out, (const f16*)qkv, \
                      (f16*)k_cache, (f16*)v_cache, block_table, max_blocks, seq_ids, tok_pos, ctx_len, rope_cos, rope_sin,       \
                      max_pos, Hq, Hkv, n_pages, n_seq, scale, frag_tt, lx)
+#define MLORA_ROPE_ATTN_NW(DD, RG)             \
+  do {                                         \
+    if (nw == 16) MLORA_ROPE_ATTN(DD, RG, 16); \
+    else if (nw == 8) MLORA_ROPE_ATTN(DD, RG, 8); \
+    else MLORA_ROPE_ATTN(DD, RG, 4);           \
+  } while (0)
   const bool small_rank = v_part == nullptr || r <= 16;
   if (D == 128) {
-    if (small_rank) MLORA_ROPE_ATTN(128, 2);
-    else MLORA_ROPE_ATTN(128, 8);
+    if (small_rank) MLORA_ROPE_ATTN_NW(128, 2);
+    else MLORA_ROPE_ATTN_NW(128, 8);
   } else {
-    if (small_rank) MLORA_ROPE_ATTN(64, 2);
-    else MLORA_ROPE_ATTN(64, 8);
+    if (small_rank) MLORA_ROPE_ATTN_NW(64, 2);
+    else MLORA_ROPE_ATTN_NW(64, 8);
   }
+#undef MLORA_ROPE_ATTN_NW
 #undef MLORA_ROPE_ATTN
   return mlora_launch_status("rope_attn_decode");
 }
