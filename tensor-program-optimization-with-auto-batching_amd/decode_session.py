@@ -14,34 +14,56 @@ from . import ops
 
 
 class DecodeSession:
-    def __init__(self, model, kv, seq_ids, tok_adapter, first_tokens):
-        """seq_ids: sequences already prefilled in `kv`; tok_adapter: {tid: ids [B] int32 (host)};
-        first_tokens [B]: the tokens produced by prefill."""
+    """Fixed-batch greedy decode through the per-operator path (any mix of adapter types and ranks).  With
+    use_graph the launch sequence of a step is captured once - after one eager step, which also sizes the model's
+    scratch buffers outside the graph's memory pool - and replayed, so the interpreter is out of the loop; the
+    kernels and their order are those of the eager step, hence the same tokens bit for bit."""
+
+    def __init__(self, model, kv, seq_ids, tok_adapter, first_tokens, use_graph=False):
+        """seq_ids: sequences already prefilled in `kv`; tok_adapter: {tid: ids [B] int32 (host or device), -1 = the
+        row does not use that type}; first_tokens [B]: the tokens produced by prefill."""
         self.model, self.kv = model, kv
         self.seq_ids = list(seq_ids)
         B = len(self.seq_ids)
         dev = model.device
-        self.tok_adapter = {tid: torch.as_tensor(np.asarray(ids, dtype=np.int32)).to(dev) for tid, ids in tok_adapter.items()}
-        self.tokens = torch.as_tensor(np.asarray(first_tokens, dtype=np.int32)).to(dev)
-        self.rows = torch.as_tensor(np.asarray([kv.slot[s] for s in self.seq_ids], dtype=np.int32)).to(dev)
-        self.pos = torch.as_tensor(np.asarray([kv.lens[s] for s in self.seq_ids], dtype=np.int32)).to(dev)
+        i32 = lambda a: (a if isinstance(a, torch.Tensor) else torch.as_tensor(np.asarray(a, dtype=np.int32))).to(dev, torch.int32)
+        self.tok_adapter = {tid: i32(ids) for tid, ids in tok_adapter.items()}
+        if len(self.tok_adapter) > 1:         # several adapter types: merged once here (the check reads back to the host)
+            self.tok_adapter = model._merge_types(self.tok_adapter)
+        self.tokens = i32(first_tokens).clone()
+        self.rows = i32([kv.slot[s] for s in self.seq_ids])
+        self.pos = i32([kv.lens[s] for s in self.seq_ids])
         self.ctx = self.pos + 1
+        self.use_graph = use_graph and B <= 64     # larger batches may call into the vendor GEMM library: not captured
+        self.graph = None
+        self._eager_steps = 0
         self.history = []
 
+    def _enqueue(self):
+        m = self.model
+        logits = m.forward(m.embed(self.tokens), self.kv, self.tok_adapter)
+        self.tokens.copy_(ops.argmax(logits))
+        self.pos.add_(1)
+        self.ctx.add_(1)
+
     def step(self, keep_history=False):
-        """One decode step for the whole batch; returns the device tensor of new token ids."""
-        m, kv = self.model, self.kv
-        hidden = m.embed(self.tokens)
+        """One decode step for the whole batch; returns the device tensor of new token ids (updated in place)."""
+        kv = self.kv
         kv.begin_forward(self.seq_ids, [1] * len(self.seq_ids), device_meta=(self.rows, self.pos, self.ctx))
-        logits = m.forward(hidden, kv, self.tok_adapter)
+        if self.use_graph and self._eager_steps >= 1:
+            if self.graph is None:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):         # records, does not run
+                    self._enqueue()
+                self.graph = g
+            self.graph.replay()
+        else:
+            self._enqueue()
+            self._eager_steps += 1
         kv.end_forward()
-        nxt = ops.argmax(logits)
-        self.tokens = nxt
-        self.pos += 1
-        self.ctx += 1
         if keep_history:
-            self.history.append(nxt)
-        return nxt
+            self.history.append(self.tokens.clone())
+        return self.tokens
 
 
 class NativeDecodeSession:

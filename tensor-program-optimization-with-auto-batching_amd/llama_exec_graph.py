@@ -4,12 +4,14 @@ Restates `tvm/llama_auto_batcher/llama_exec_graph.py:10-174`.  Differences that 
 the argmax runs on the device and only the token ids cross to the host (the reference copies the full
 fp32 logits and calls np.argmax, `:92,134-137`; ties resolve to the lowest index in both); prompts may be
 given as token-id arrays when no tokenizer is configured; decode batches of a single adapter type run through the
-native decode step (bit-identical tokens, see LlamaExecConfig.native_decode).
+native decode step and batches that mix adapter types through a graph-replayed per-operator step (bit-identical
+tokens either way, see LlamaExecConfig.native_decode).
 """
 from __future__ import annotations
 
 import dataclasses
 import os
+import re
 
 import numpy as np
 import torch
@@ -24,8 +26,9 @@ class LlamaExecConfig:
     max_gen_len: int
     page_size: int
     # Run decode batches of one adapter type (or none) and at most 64 sequences through the native decode step (one
-    # C call per step, graph replay when several steps lie ahead) instead of one call per operator.  Same tokens:
-    # the native step with ids-based LoRA shrink is bit-identical to the per-operator path.
+    # C call per step, graph replay when several steps lie ahead) instead of one call per operator, and batches that
+    # mix adapter types through the per-operator step recorded into a graph.  Same tokens: the native step with
+    # ids-based LoRA shrink is bit-identical to the per-operator path.
     native_decode: bool = True
 
 
@@ -127,8 +130,9 @@ class LlamaExecGraph(ExecGraph):
         while seqs:
             method, params = self.seq_info.get_decode_method(seqs)
             single = method == "decode_no_adapter" or method.startswith("decode_a")
-            if getattr(self.exec_config, "native_decode", False) and single and len(seqs) <= 64:
-                seqs = self._decode_native(seqs, outputs, method, params)
+            if getattr(self.exec_config, "native_decode", False) and len(seqs) <= 64:
+                seqs = self._decode_native(seqs, outputs, method, params) if single \
+                    else self._decode_session(seqs, outputs, method, params)
                 continue
             tokens = torch.tensor([outputs[sid][-1] for sid in seqs], dtype=torch.int32)
             hidden = self.vm["embed"](tokens)
@@ -154,6 +158,34 @@ class LlamaExecGraph(ExecGraph):
         last = [outputs[sid][-1] for sid in seqs]
         ahead = min(self.seq_info.get_max_gen_len(sid) - len(outputs[sid]) for sid in seqs)
         sess = NativeDecodeSession(self.vm, self.kv_cache, seqs, wids, last, tid=tid, use_graph=ahead >= 8, dense_lora=False)
+        if self.eos_token_id is None and not self.measure:
+            for _ in range(ahead):
+                sess.step(keep_history=True)
+            toks = torch.stack(sess.history).cpu().numpy()             # [ahead, batch]
+            for i, sid in enumerate(seqs):
+                outputs[sid].extend(int(t) for t in toks[:, i])
+            return self.check_seqs_finished(seqs, outputs)
+        while True:
+            ev = self._tic()
+            nxt = sess.step()
+            self._toc(ev)
+            nxt = nxt.cpu().numpy()
+            for i, sid in enumerate(seqs):
+                outputs[sid].append(int(nxt[i]))
+            left = self.check_seqs_finished(seqs, outputs)
+            if len(left) != len(seqs):
+                return left
+
+    def _decode_session(self, seqs, outputs, method, params):
+        """A batch that mixes adapter types (`mixed_decode_a{i}_a{j}...`): the per-operator step with the tokens,
+        positions and context lengths kept on the device, replayed from a graph when enough steps lie ahead.  Same
+        kernels in the same order as the call-per-step path, so the same tokens."""
+        from .decode_session import DecodeSession
+        tids = [int(t) for t in re.findall(r"_a(\d+)", method)]
+        pairs = {tid: (params[2 * i], params[2 * i + 1]) for i, tid in enumerate(tids)}
+        last = [outputs[sid][-1] for sid in seqs]
+        ahead = min(self.seq_info.get_max_gen_len(sid) - len(outputs[sid]) for sid in seqs)
+        sess = DecodeSession(self.vm, self.kv_cache, seqs, self.vm._ids(len(seqs), pairs), last, use_graph=ahead >= 8)
         if self.eos_token_id is None and not self.measure:
             for _ in range(ahead):
                 sess.step(keep_history=True)

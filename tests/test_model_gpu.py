@@ -130,6 +130,29 @@ def test_mixed_adapter_types_and_no_adapter(c1):
     assert name == "mixed_decode_a0_a1"
 
 
+def test_mixed_adapter_types_graph_replayed_session_equals_call_per_step(c1):
+    """A batch that mixes two adapter types and adapter-less requests decodes through the per-operator step recorded
+    into a graph (tokens and counters stay on the device); the tokens are those of the call-per-step loop, which
+    runs the same kernels.  24 generated tokens from a 24-token prompt: every sequence crosses a page boundary."""
+    wl, _, _ = c1
+    synth = load_pkg("synth")
+    spec1 = synth.LoraSpec(r=16, alpha=8.0, n_adapters=3, targets=("q_proj", "v_proj", "o_proj"))
+    model = hip_model(wl, [wl.lora, spec1])
+    B, P, max_gen_len = 6, 24, 24
+    prompts = synth.randint(12, "mixedg.prompts", (B, P), wl.shape.vocab_size).numpy()
+    tids = [0, 1, -1, 1, 0, -1]
+    wids = np.array([2, 0, -1, 2, 3, -1], dtype=np.int32)
+    n_pages = B * 5
+    perm = synth.permutation(12, "mixedg.pages", n_pages)
+    wl2 = synth.Workload("mixedg", 12, wl.shape, wl.lora, batch=B, prompt_len=P, gen_len=max_gen_len)
+    got, batcher = run_hip_generate(model, wl2, prompts, wids, max_gen_len, perm, tids=[max(t, 0) for t in tids])
+    name, _ = batcher.seq_info.get_decode_method(batcher.seq_info.order_seqs(list(range(B)))[0])
+    assert name == "mixed_decode_a0_a1"
+    want, _ = run_hip_generate(model, wl2, prompts, wids, max_gen_len, perm, tids=[max(t, 0) for t in tids], native_decode=False)
+    assert all(len(g) == max_gen_len for g in got)
+    assert got == want
+
+
 def test_per_request_max_gen_len_and_eos(c1):
     """The batch shrinks as sequences hit their own max_gen_len or EOS; outputs keep request order."""
     wl, model, prompts = c1
