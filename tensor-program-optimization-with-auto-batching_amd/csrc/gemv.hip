@@ -491,12 +491,21 @@ extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p
   }();
   const int pairs = I / 16;
   const int per = n_cu > 0 ? ceil_div(pairs, n_cu) : 0;
-  if (T > 16 && T <= 32 && n_cu > 0 && pairs >= 2 * n_cu && per <= 4) {
+  if (T <= 32 && n_cu > 0 && pairs >= 2 * n_cu && per <= 4) {
     const int base = pairs / n_cu, rem = pairs % n_cu;
     const dim3 g(n_cu);
-    if (per <= 2) hipLaunchKernelGGL((gemv_silu_cu_kernel<2, 2, 4>), g, block, 0, s, (f16*)act, xp, Wp, T, K, I, base, rem);
-    else if (per == 3) hipLaunchKernelGGL((gemv_silu_cu_kernel<3, 2, 3>), g, block, 0, s, (f16*)act, xp, Wp, T, K, I, base, rem);
-    else hipLaunchKernelGGL((gemv_silu_cu_kernel<4, 2, 2>), g, block, 0, s, (f16*)act, xp, Wp, T, K, I, base, rem);
+#define MLORA_SILU_CU(NP, TT, PIPE) \
+  hipLaunchKernelGGL((gemv_silu_cu_kernel<NP, TT, PIPE>), g, block, 0, s, (f16*)act, xp, Wp, T, K, I, base, rem)
+    if (T <= 16) {
+      if (per <= 2) MLORA_SILU_CU(2, 1, 4);
+      else if (per == 3) MLORA_SILU_CU(3, 1, 4);
+      else MLORA_SILU_CU(4, 1, 3);
+    } else {
+      if (per <= 2) MLORA_SILU_CU(2, 2, 4);
+      else if (per == 3) MLORA_SILU_CU(3, 2, 3);
+      else MLORA_SILU_CU(4, 2, 2);
+    }
+#undef MLORA_SILU_CU
     return mlora_launch_status("gemv_frag_silu");
   }
   if (T <= 16) hipLaunchKernelGGL((gemv_kernel<2, 1, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);

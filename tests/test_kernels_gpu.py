@@ -365,7 +365,8 @@ def test_page_walk_bit_exact_with_integer_kv(ops, synth):
                 assert np.all(o[s, h] == code[(s, sel[s], h)]), (probe, s, h, o[s, h, :4], code[(s, sel[s], h)])
 
 
-@pytest.mark.parametrize("T,K,I", [(1, 256, 64), (16, 512, 352), (32, 4096, 11008), (21, 1024, 96), (48, 1024, 352), (64, 4096, 11008)])
+@pytest.mark.parametrize("T,K,I", [(1, 256, 64), (16, 512, 352), (32, 4096, 11008), (21, 1024, 96), (48, 1024, 352), (64, 4096, 11008),
+                                   (8, 4096, 11008), (16, 4096, 14336), (5, 2048, 8192)])
 def test_gate_up_silu_epilogue_equals_two_launches(ops, synth, T, K, I):
     """The GEMV whose epilogue is the SiLU product gives the bits of GEMV followed by silu_mul."""
     x = synth.normal(5, "gus.x", (T, K), 1.0, torch.float16, DEV)
