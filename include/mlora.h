@@ -88,7 +88,9 @@ int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, int x_layout, 
  * Every table is read at its own rank: nothing is padded to the largest rank and no rank is split into chunks, and
  * rows are addressed by token, so there is no gather of x rows nor scatter of results.  Same result bits as one
  * mlora_gather_mm call per bucket with the other buckets' tokens masked to -1.  workspace: the largest
- * mlora_gather_mm_workspace_bytes(T, K, r) over the buckets; the launches of the buckets are ordered on `stream`.
+ * mlora_gather_mm_workspace_bytes(T, K, r) over the buckets.  A decode-sized batch (T <= 64) with at most four
+ * buckets is ONE launch: the kernel is built for the largest rank and a workgroup (one adapter) runs at its own
+ * bucket's rank; otherwise one launch sequence per bucket, ordered on `stream`.
  * All buckets are validated before the first launch.  `buckets` is a HOST array; a bucket with A == B == NULL is
  * skipped (its adapters do not target this projection) and its tokens are left untouched.
  *

@@ -144,6 +144,21 @@ struct GmmSet {
 constexpr int GMM_WAVES = 8;
 constexpr int GMM_THREADS = GMM_WAVES * WAVE;
 
+// Adapter tables of several ranks served by ONE launch (MULTI): bucket b holds adapters first[b] .. first[b+1]-1 of the
+// launch's global adapter numbering; a token names its bucket and its adapter inside the bucket.  The kernel is
+// instantiated for the largest rank; a workgroup (one adapter) runs with its bucket's rank, and the rank entries it
+// does not have enter every sum as zeros - which leaves the bits of the single-rank kernel: the reduction trees only
+// gain exact zero terms.
+constexpr int GMM_MAX_BUCKETS = 4;
+struct GmmBuckets {
+  const f16* A[GMM_MAX_BUCKETS];
+  const f16* B[GMM_MAX_BUCKETS];
+  int r[GMM_MAX_BUCKETS];
+  int first[GMM_MAX_BUCKETS + 1];
+  float scaling[GMM_MAX_BUCKETS];
+  int n;
+};
+
 // B[n, 0..R) . v[0..R): an fma chain over each group of 8, then pairwise sums of neighbouring groups
 // (the order of lora_expand_kernel and lora_row_dot).
 template <int R>
@@ -166,31 +181,50 @@ __device__ __forceinline__ float row_dot(const f16x8 (&bv)[R / 8], const float* 
 
 // GR: rows of A a wave reduces together.  16 reads x once per 16 rows (shortest single problem); 8 keeps the kernel
 // under 128 VGPRs, i.e. two workgroups per CU, which is what a launch over many problems wants.  Same result bits.
-template <int R, typename YT, int GR>
+template <int R, typename YT, int GR, bool MULTI = false>
 __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_decode_kernel(GmmSet one, const GmmSet* __restrict__ sets,
                                                                         const int32_t* __restrict__ ids, float scaling,
                                                                         int T, int K, int N, int n_ad, int ldy,
                                                                         int frag_tt, int P, int ci_n, int kc,
-                                                                        const int32_t* __restrict__ bucket_of, int bucket) {
+                                                                        const int32_t* __restrict__ bucket_of, int bucket,
+                                                                        GmmBuckets mb) {
   constexpr int G = R < GR ? R : GR;         // rows of A reduced together
   constexpr int NG = R / 8;
   extern __shared__ float lds[];             // part [kc][T][R], then v [T][R]
   float* part = lds;
   float* vfin = lds + (size_t)kc * T * R;
   const int wg = blockIdx.x;
-  const int a = (wg & 7) + 8 * (wg / (8 * P));
+  int a = (wg & 7) + 8 * (wg / (8 * P));                // MULTI: numbered over all buckets, n_ad their total
   const int p = (wg >> 3) % P;
   if (a >= n_ad) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   // the problem's pointers and the table row are independent requests: both are in flight before either is awaited
   // (the empty asm keeps the pointer load in this block, ahead of the early exit)
-  const GmmSet s = sets ? sets[blockIdx.y] : one;
+  GmmSet s = sets ? sets[blockIdx.y] : one;
+  int ra = R;                                           // rank of this workgroup's adapter
+  if constexpr (MULTI) {
+    int b = 0;
+#pragma unroll
+    for (int i = 1; i < GMM_MAX_BUCKETS; ++i)
+      if (i < mb.n && a >= mb.first[i]) b = i;
+#pragma unroll
+    for (int i = 0; i < GMM_MAX_BUCKETS; ++i)
+      if (i == b) {                                     // uniform selects: the struct is never indexed dynamically
+        s.A = mb.A[i];
+        s.B = mb.B[i];
+        ra = mb.r[i];
+        scaling = mb.scaling[i];
+        a -= mb.first[i];
+      }
+    bucket = b;
+    if (s.A == nullptr) return;                         // the bucket's adapters do not target this projection
+  }
   const int id = lora_token_id(ids, bucket_of, bucket, lane, T);   // T <= 64: one table row per lane
   asm volatile("" ::"s"(s.A), "s"(s.B), "s"(s.x), "s"(s.y));
   const unsigned long long mine = __ballot(id == a);
   if (!mine) return;                                    // workgroup-uniform
-  const f16* __restrict__ A = s.A + (size_t)a * R * K;
-  const f16* __restrict__ B = s.B + (size_t)a * N * R;
+  const f16* __restrict__ A = s.A + (size_t)a * ra * K;
+  const f16* __restrict__ B = s.B + (size_t)a * N * ra;
   YT* __restrict__ y = (YT*)s.y;
   const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
 
@@ -213,7 +247,7 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
       ya[i] = yb[i] = 0.f;
       if (n < n1) {
 #pragma unroll
-        for (int q = 0; q < NG; ++q) bpre[i][q] = ld8(B + (size_t)n * R + q * 8);
+        for (int q = 0; q < NG; ++q) bpre[i][q] = q * 8 < ra ? ld8(B + (size_t)n * ra + q * 8) : zero8;
         ya[i] = (float)y[(size_t)ta * ldy + n];
         if (tb >= 0) yb[i] = (float)y[(size_t)tb * ldy + n];
       }
@@ -231,9 +265,10 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
       const bool in = kbase < K;
 #pragma unroll
       for (int jb = 0; jb < R; jb += G) {
+        if (jb >= ra) break;                              // uniform; the rank entries beyond ra are zeroed below
         f16x8 areg[G];
 #pragma unroll
-        for (int j = 0; j < G; ++j) areg[j] = in ? ld8(A + (size_t)(jb + j) * K + kbase) : zero8;
+        for (int j = 0; j < G; ++j) areg[j] = (in && jb + j < ra) ? ld8(A + (size_t)(jb + j) * K + kbase) : zero8;
         unsigned long long m = mine;
         while (m) {
           const int t0 = __builtin_ctzll(m);
@@ -272,6 +307,7 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
         const int t1 = tt[1] >= 0 ? tt[1] : tt[0];
 #pragma unroll
         for (int jb = 0; jb < R; jb += G) {
+          if (jb >= ra) break;                            // uniform
           float acc0[G], acc1[G];
 #pragma unroll
           for (int j = 0; j < G; ++j) acc0[j] = acc1[j] = 0.f;
@@ -282,7 +318,7 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
             const f16x8 x1 = in ? ld8(s.x + (frag_tt ? frag_offset(t1, k, frag_tt) : (size_t)t1 * K + k)) : zero8;
             f16x8 areg[G];
 #pragma unroll
-            for (int j = 0; j < G; ++j) areg[j] = in ? ld8(A + (size_t)(jb + j) * K + k) : zero8;
+            for (int j = 0; j < G; ++j) areg[j] = (in && jb + j < ra) ? ld8(A + (size_t)(jb + j) * K + k) : zero8;
 #pragma unroll
             for (int j = 0; j < G; ++j) {
               acc0[j] = dot8(areg[j], x0, acc0[j]);
@@ -300,7 +336,7 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
   __syncthreads();
   for (int e = threadIdx.x; e < T * R; e += GMM_THREADS) {
     const int t = e / R, j = e % R;
-    if ((mine >> t) & 1) vfin[e] = lora_v(part, kc, T, R, t, j, scaling);
+    if ((mine >> t) & 1) vfin[e] = j < ra ? lora_v(part, kc, T, R, t, j, scaling) : 0.f;
   }
   __syncthreads();
 
@@ -351,7 +387,7 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
     for (int n = nf + GMM_THREADS; n < n1; n += GMM_THREADS) {
       f16x8 bv[NG];
 #pragma unroll
-      for (int q = 0; q < NG; ++q) bv[q] = ld8(B + (size_t)n * R + q * 8);
+      for (int q = 0; q < NG; ++q) bv[q] = q * 8 < ra ? ld8(B + (size_t)n * ra + q * 8) : zero8;
       unsigned long long m = mine;
       while (m) {
         const int t = __builtin_ctzll(m);
@@ -847,11 +883,20 @@ static bool gmm_one_launch_fits(int T, int K, int r) {
 template <int R>
 static void gmm_launch_r(const GmmSet& one, const GmmSet* sets, dim3 grid, size_t lds, int y_dtype, const int32_t* ids,
                          float scaling, int T, int K, int N, int n_ad, int ldy, int frag_tt, int P, LoraKSplit ks, hipStream_t s,
-                         BucketFilter bf) {
+                         BucketFilter bf, const GmmBuckets* mb) {
   const dim3 block(GMM_THREADS);
+  if (mb != nullptr) {     // adapters of several ranks: R is the largest, bf.bucket_of the per-token bucket
+#define MLORA_GMM_MULTI(YT)                                                                                                      \
+  hipLaunchKernelGGL((gather_mm_decode_kernel<R, YT, 16, true>), grid, block, lds, s, one, sets, ids, scaling, T, K, N, n_ad, ldy, \
+                     frag_tt, P, ks.ci, ks.kc, bf.bucket_of, 0, *mb)
+    if (y_dtype == MLORA_F16) MLORA_GMM_MULTI(f16);
+    else MLORA_GMM_MULTI(float);
+#undef MLORA_GMM_MULTI
+    return;
+  }
 #define MLORA_GMM_LAUNCH(YT, GR)                                                                                              \
   hipLaunchKernelGGL((gather_mm_decode_kernel<R, YT, GR>), grid, block, lds, s, one, sets, ids, scaling, T, K, N, n_ad, ldy, \
-                     frag_tt, P, ks.ci, ks.kc, bf.bucket_of, bf.bucket)
+                     frag_tt, P, ks.ci, ks.kc, bf.bucket_of, bf.bucket, GmmBuckets())
   const bool many = grid.y > 1;
   if (y_dtype == MLORA_F16) {
     if (many) MLORA_GMM_LAUNCH(f16, 8);
@@ -865,7 +910,7 @@ static void gmm_launch_r(const GmmSet& one, const GmmSet* sets, dim3 grid, size_
 
 static int gmm_one_launch(const GmmSet& one, const GmmSet* sets, int n_sets, int y_dtype, int ldy, int x_layout,
                           const int32_t* ids, float scaling, int T, int K, int N, int r, int n_ad, hipStream_t s,
-                          BucketFilter bf = BucketFilter{nullptr, 0}) {
+                          BucketFilter bf = BucketFilter{nullptr, 0}, const GmmBuckets* mb = nullptr) {
   const LoraKSplit ks = lora_k_split(K);
   const int groups = ceil_div(n_ad, 8);                 // adapters are dealt to the 8 XCDs in groups of 8
   // Output-row slices per adapter: enough workgroups to cover the chip when the launch holds one problem, one slice
@@ -878,10 +923,10 @@ static int gmm_one_launch(const GmmSet& one, const GmmSet* sets, int n_sets, int
   const int frag_tt = x_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   const dim3 grid(groups * 8 * P, n_sets);
   switch (r) {
-    case 8: gmm_launch_r<8>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s, bf); break;
-    case 16: gmm_launch_r<16>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s, bf); break;
-    case 32: gmm_launch_r<32>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s, bf); break;
-    default: gmm_launch_r<64>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s, bf); break;
+    case 8: gmm_launch_r<8>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s, bf, mb); break;
+    case 16: gmm_launch_r<16>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s, bf, mb); break;
+    case 32: gmm_launch_r<32>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s, bf, mb); break;
+    default: gmm_launch_r<64>(one, sets, grid, lds, y_dtype, ids, scaling, T, K, N, n_ad, ldy, frag_tt, P, ks, s, bf, mb); break;
   }
   return mlora_launch_status("gather_mm");
 }
@@ -996,6 +1041,37 @@ extern "C" int mlora_gather_mm_multi(void* y, int y_dtype, int ldy, const void* 
     MLORA_CHECK(T == 0 || (workspace && workspace_bytes >= mlora_gather_mm_workspace_bytes(T, K, buckets[b].r)), MLORA_ERR_WORKSPACE,
                 "gather_mm_multi: workspace of %zu bytes given, %zu needed for bucket %d (rank %d)", workspace_bytes,
                 mlora_gather_mm_workspace_bytes(T, K, buckets[b].r), b, buckets[b].r);
+  }
+  // Decode-sized batches with up to GMM_MAX_BUCKETS buckets: ONE launch serves all ranks (same bits as a launch per bucket)
+  int rmax = 0, total = 0, live = 0;
+  for (int b = 0; b < n_buckets; ++b) {
+    total += buckets[b].n_ad > 0 ? buckets[b].n_ad : 0;
+    if (buckets[b].A) {
+      ++live;
+      if (buckets[b].r > rmax) rmax = buckets[b].r;
+    }
+  }
+  if (live > 1 && n_buckets <= GMM_MAX_BUCKETS && gmm_one_launch_fits(T, K, rmax)) {
+    MLORA_CHECK(y && x, MLORA_ERR_INVALID, "gather_mm_multi: null pointer");
+    MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "gather_mm_multi: bad y_dtype %d", y_dtype);
+    MLORA_CHECK(ldy >= N, MLORA_ERR_INVALID, "gather_mm_multi: need ldy >= N (ldy=%d N=%d)", ldy, N);
+    MLORA_CHECK(x_layout == MLORA_ROWMAJOR || (x_layout == MLORA_FRAG && K % 32 == 0), MLORA_ERR_UNSUPPORTED,
+                "gather_mm_multi: fragment-ordered x needs K %% 32 == 0");
+    GmmBuckets mb = {};
+    mb.n = n_buckets;
+    int first = 0;
+    for (int b = 0; b < n_buckets; ++b) {
+      mb.A[b] = (const f16*)buckets[b].A;
+      mb.B[b] = (const f16*)buckets[b].B;
+      mb.r[b] = buckets[b].A ? buckets[b].r : rmax;
+      mb.scaling[b] = buckets[b].scaling;
+      mb.first[b] = first;
+      first += buckets[b].n_ad > 0 ? buckets[b].n_ad : 0;
+    }
+    for (int b = n_buckets; b <= GMM_MAX_BUCKETS; ++b) mb.first[b] = first;
+    GmmSet one = {y, (const f16*)x, nullptr, nullptr};
+    return gmm_one_launch(one, nullptr, 1, y_dtype, ldy, x_layout, tok_adapter, 1.f, T, K, N, rmax, total, (hipStream_t)stream,
+                          BucketFilter{tok_bucket, 0}, &mb);
   }
   for (int b = 0; b < n_buckets; ++b) {
     if (!buckets[b].A) continue;

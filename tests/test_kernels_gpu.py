@@ -420,6 +420,31 @@ def test_gather_mm_batch_equals_separate_calls(ops, synth):
         assert torch.equal(y, w)
 
 
+@pytest.mark.parametrize("ydt", [torch.float16, torch.float32])
+def test_gather_mm_multi_one_launch_with_absent_bucket_and_fragment_input(ops, synth, ydt):
+    """Decode-sized multi-rank call (one launch for all buckets): a bucket whose adapters do not target the projection,
+    an fp32 y (the residual stream), fragment-ordered x.  Bit-identical to one masked call per bucket."""
+    T, K, N = 32, 2048, 768
+    ranks, n_ads, scal = (32, 8, 16), (4, 3, 9), (0.5, 2.0, 0.125)
+    x = synth.normal(22, "mro.x", (T, K), 1.0, torch.float16, DEV)
+    y0 = synth.normal(22, "mro.y", (T, N), 1.0, ydt, DEV)
+    tabs = [(synth.normal(22, f"mro.A{i}", (n, r, K), 0.05, torch.float16, DEV),
+             synth.normal(22, f"mro.B{i}", (n, N, r), 0.05, torch.float16, DEV)) for i, (r, n) in enumerate(zip(ranks, n_ads))]
+    tb = (synth.randint(22, "mro.bucket", (T,), 4, DEV) - 1).to(torch.int32)
+    ta = torch.stack([synth.randint(22, f"mro.ad{i}", (T,), n, DEV) for i, n in enumerate(n_ads)])
+    tok_adapter = torch.where(tb >= 0, ta.gather(0, tb.clamp(min=0).long()[None])[0], torch.full_like(tb, -1)).to(torch.int32)
+    xf = ops.FragActivation.pack(x)
+    for absent in (None, 1):
+        buckets = [None if i == absent else (A, B, s) for i, ((A, B), s) in enumerate(zip(tabs, scal))]
+        multi = ops.gather_mm_multi(y0.clone(), xf, buckets, tb, tok_adapter)
+        seq = y0.clone()
+        for i, bk in enumerate(buckets):
+            if bk is not None:
+                ops.gather_mm(seq, xf, bk[0], bk[1], torch.where(tb == i, tok_adapter, torch.full_like(tb, -1)), bk[2])
+        assert torch.equal(multi, seq)
+        assert not torch.equal(multi, y0)
+
+
 @pytest.mark.parametrize("T,K,N", [(48, 1024, 512), (150, 2048, 1024)])
 def test_gather_mm_multi_rank_strategies_agree(ops, synth, T, K, N):
     """Three rank buckets (8, 16, 64) in one call: equal, bit for bit, to one masked call per bucket (the reference's
