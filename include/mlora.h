@@ -108,6 +108,18 @@ int mlora_gather_mm_multi(void* y, int y_dtype, int ldy, const void* x, int x_la
                           const mlora_lora_bucket* buckets, int n_buckets,
                           const int32_t* tok_bucket, const int32_t* tok_adapter,
                           int T, int K, int N, void* workspace, size_t workspace_bytes, void* stream);
+/* The same for n_proj projections that read the same x and write disjoint column ranges of one y (q, k, v inside the
+ * fused qkv row; gate and up): projection p adds to columns col_offset[p] .. col_offset[p] + n_cols[p] - 1 of y
+ * (col_offset[p] % 8 == 0) with the tables buckets[p * n_buckets + b] (B [n_ad, n_cols[p], r]).  A decode-sized batch
+ * with at most eight non-null (projection, bucket) entries is ONE launch; otherwise one mlora_gather_mm_multi per
+ * projection.  Same result bits as those calls.  buckets, col_offset and n_cols are HOST arrays.
+ * Replaces: q_ft_proj + v_ft_proj of the patched attention forward, one take-matmul pair each
+ * (tvm/llama_auto_batcher/compile_tvm.py:126-155). */
+int mlora_gather_mm_multi_proj(void* y, int y_dtype, int ldy, const void* x, int x_layout,
+                               const mlora_lora_bucket* buckets, int n_buckets, int n_proj,
+                               const int32_t* col_offset, const int32_t* n_cols,
+                               const int32_t* tok_bucket, const int32_t* tok_adapter,
+                               int T, int K, void* workspace, size_t workspace_bytes, void* stream);
 int mlora_gather_mm_batch(const void* const* sets, int n_sets, int y_dtype, int ldy, int x_layout,
                           const int32_t* tok_adapter, float scaling,
                           int T, int K, int N, int r, int n_ad, void* stream);

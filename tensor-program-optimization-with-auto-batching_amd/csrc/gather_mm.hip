@@ -144,18 +144,22 @@ struct GmmSet {
 constexpr int GMM_WAVES = 8;
 constexpr int GMM_THREADS = GMM_WAVES * WAVE;
 
-// Adapter tables of several ranks served by ONE launch (MULTI): bucket b holds adapters first[b] .. first[b+1]-1 of the
-// launch's global adapter numbering; a token names its bucket and its adapter inside the bucket.  The kernel is
-// instantiated for the largest rank; a workgroup (one adapter) runs with its bucket's rank, and the rank entries it
-// does not have enter every sum as zeros - which leaves the bits of the single-rank kernel: the reduction trees only
-// gain exact zero terms.
-constexpr int GMM_MAX_BUCKETS = 4;
+// Adapter tables of several ranks - and of several projections that read the same x - served by ONE launch (MULTI).
+// Entry e is one (projection, rank bucket) pair: its tables, rank and scaling, the token bucket it serves, and the
+// column range of y it adds to; it holds adapters first[e] .. first[e+1]-1 of the launch's global adapter numbering.
+// A token names its bucket and its adapter inside the bucket.  The kernel is instantiated for the largest rank; a
+// workgroup (one adapter of one entry) runs with its entry's rank, and the rank entries it does not have enter every
+// sum as zeros - which leaves the bits of the single-rank kernel: the reduction trees only gain exact zero terms.
+constexpr int GMM_MAX_BUCKETS = 8;
 struct GmmBuckets {
   const f16* A[GMM_MAX_BUCKETS];
   const f16* B[GMM_MAX_BUCKETS];
   int r[GMM_MAX_BUCKETS];
   int first[GMM_MAX_BUCKETS + 1];
   float scaling[GMM_MAX_BUCKETS];
+  int tok_bucket[GMM_MAX_BUCKETS];   // value of the per-token bucket array this entry serves
+  int ycol[GMM_MAX_BUCKETS];         // first column of y and number of columns (rows of B) of the entry's projection
+  int ncols[GMM_MAX_BUCKETS];
   int n;
 };
 
@@ -202,6 +206,7 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
   // (the empty asm keeps the pointer load in this block, ahead of the early exit)
   GmmSet s = sets ? sets[blockIdx.y] : one;
   int ra = R;                                           // rank of this workgroup's adapter
+  int ycol = 0;
   if constexpr (MULTI) {
     int b = 0;
 #pragma unroll
@@ -215,8 +220,10 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
         ra = mb.r[i];
         scaling = mb.scaling[i];
         a -= mb.first[i];
+        bucket = mb.tok_bucket[i];
+        ycol = mb.ycol[i];
+        N = mb.ncols[i];
       }
-    bucket = b;
     if (s.A == nullptr) return;                         // the bucket's adapters do not target this projection
   }
   const int id = lora_token_id(ids, bucket_of, bucket, lane, T);   // T <= 64: one table row per lane
@@ -225,7 +232,7 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
   if (!mine) return;                                    // workgroup-uniform
   const f16* __restrict__ A = s.A + (size_t)a * ra * K;
   const f16* __restrict__ B = s.B + (size_t)a * N * ra;
-  YT* __restrict__ y = (YT*)s.y;
+  YT* __restrict__ y = (YT*)s.y + ycol;
   const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
 
   // Requests that depend on the adapter table only go out first, ahead of the shrink: the thread's first row(s) of B
@@ -1027,6 +1034,52 @@ extern "C" int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, int
                         BucketFilter{nullptr, 0}, stream);
 }
 
+// One launch for n_proj projections that share x (columns col_offset[p] .. + n_cols[p] of y) and n_buckets rank buckets
+// each; buckets is [n_proj][n_buckets].  Returns 1 when the launch was made, 0 when the shapes do not allow it (the
+// caller then falls back to a launch sequence per bucket), < 0 on an argument error.
+static int gmm_multi_one_launch(void* y, int y_dtype, int ldy, const void* x, int x_layout, const mlora_lora_bucket* buckets,
+                                int n_buckets, int n_proj, const int32_t* col_offset, const int32_t* n_cols,
+                                const int32_t* tok_bucket, const int32_t* tok_adapter, int T, int K, hipStream_t stream) {
+  int rmax = 0, total = 0, live = 0, nmax = 0;
+  for (int e = 0; e < n_proj * n_buckets; ++e) {
+    if (!buckets[e].A) continue;
+    ++live;
+    total += buckets[e].n_ad;
+    if (buckets[e].r > rmax) rmax = buckets[e].r;
+    if (n_cols[e / n_buckets] > nmax) nmax = n_cols[e / n_buckets];
+  }
+  if (live < 2 || live > GMM_MAX_BUCKETS || !gmm_one_launch_fits(T, K, rmax)) return 0;
+  MLORA_CHECK(y && x, MLORA_ERR_INVALID, "gather_mm_multi: null pointer");
+  MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "gather_mm_multi: bad y_dtype %d", y_dtype);
+  MLORA_CHECK(x_layout == MLORA_ROWMAJOR || (x_layout == MLORA_FRAG && K % 32 == 0), MLORA_ERR_UNSUPPORTED,
+              "gather_mm_multi: fragment-ordered x needs K %% 32 == 0");
+  GmmBuckets mb = {};
+  int first = 0, n = 0;
+  for (int e = 0; e < n_proj * n_buckets; ++e) {
+    if (!buckets[e].A) continue;           // absent entries take no workgroups
+    const int p = e / n_buckets;
+    MLORA_CHECK(col_offset[p] >= 0 && n_cols[p] > 0 && col_offset[p] + n_cols[p] <= ldy, MLORA_ERR_INVALID,
+                "gather_mm_multi: columns %d..%d of projection %d outside a row of %d", col_offset[p], col_offset[p] + n_cols[p], p, ldy);
+    mb.A[n] = (const f16*)buckets[e].A;
+    mb.B[n] = (const f16*)buckets[e].B;
+    mb.r[n] = buckets[e].r;
+    mb.scaling[n] = buckets[e].scaling;
+    mb.tok_bucket[n] = e % n_buckets;
+    mb.ycol[n] = col_offset[p];
+    mb.ncols[n] = n_cols[p];
+    mb.first[n] = first;
+    first += buckets[e].n_ad;
+    ++n;
+  }
+  for (int e = n; e <= GMM_MAX_BUCKETS; ++e) mb.first[e] = first;
+  mb.n = n;
+  GmmSet one = {y, (const f16*)x, nullptr, nullptr};
+  if (int rc = gmm_one_launch(one, nullptr, 1, y_dtype, ldy, x_layout, tok_adapter, 1.f, T, K, nmax, rmax, total, stream,
+                              BucketFilter{tok_bucket, 0}, &mb))
+    return rc;
+  return 1;
+}
+
 extern "C" int mlora_gather_mm_multi(void* y, int y_dtype, int ldy, const void* x, int x_layout,
                                      const mlora_lora_bucket* buckets, int n_buckets, const int32_t* tok_bucket,
                                      const int32_t* tok_adapter, int T, int K, int N, void* workspace,
@@ -1043,42 +1096,51 @@ extern "C" int mlora_gather_mm_multi(void* y, int y_dtype, int ldy, const void* 
                 mlora_gather_mm_workspace_bytes(T, K, buckets[b].r), b, buckets[b].r);
   }
   // Decode-sized batches with up to GMM_MAX_BUCKETS buckets: ONE launch serves all ranks (same bits as a launch per bucket)
-  int rmax = 0, total = 0, live = 0;
-  for (int b = 0; b < n_buckets; ++b) {
-    total += buckets[b].n_ad > 0 ? buckets[b].n_ad : 0;
-    if (buckets[b].A) {
-      ++live;
-      if (buckets[b].r > rmax) rmax = buckets[b].r;
-    }
-  }
-  if (live > 1 && n_buckets <= GMM_MAX_BUCKETS && gmm_one_launch_fits(T, K, rmax)) {
-    MLORA_CHECK(y && x, MLORA_ERR_INVALID, "gather_mm_multi: null pointer");
-    MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "gather_mm_multi: bad y_dtype %d", y_dtype);
-    MLORA_CHECK(ldy >= N, MLORA_ERR_INVALID, "gather_mm_multi: need ldy >= N (ldy=%d N=%d)", ldy, N);
-    MLORA_CHECK(x_layout == MLORA_ROWMAJOR || (x_layout == MLORA_FRAG && K % 32 == 0), MLORA_ERR_UNSUPPORTED,
-                "gather_mm_multi: fragment-ordered x needs K %% 32 == 0");
-    GmmBuckets mb = {};
-    mb.n = n_buckets;
-    int first = 0;
-    for (int b = 0; b < n_buckets; ++b) {
-      mb.A[b] = (const f16*)buckets[b].A;
-      mb.B[b] = (const f16*)buckets[b].B;
-      mb.r[b] = buckets[b].A ? buckets[b].r : rmax;
-      mb.scaling[b] = buckets[b].scaling;
-      mb.first[b] = first;
-      first += buckets[b].n_ad > 0 ? buckets[b].n_ad : 0;
-    }
-    for (int b = n_buckets; b <= GMM_MAX_BUCKETS; ++b) mb.first[b] = first;
-    GmmSet one = {y, (const f16*)x, nullptr, nullptr};
-    return gmm_one_launch(one, nullptr, 1, y_dtype, ldy, x_layout, tok_adapter, 1.f, T, K, N, rmax, total, (hipStream_t)stream,
-                          BucketFilter{tok_bucket, 0}, &mb);
-  }
+  const int32_t zero = 0;
+  if (int rc = gmm_multi_one_launch(y, y_dtype, ldy, x, x_layout, buckets, n_buckets, 1, &zero, &N, tok_bucket, tok_adapter, T, K,
+                                    (hipStream_t)stream))
+    return rc < 0 ? rc : MLORA_OK;   // > 0: launched
   for (int b = 0; b < n_buckets; ++b) {
     if (!buckets[b].A) continue;
     if (int e = gather_mm_impl(y, y_dtype, ldy, x, x_layout, buckets[b].A, buckets[b].B, tok_adapter, buckets[b].scaling, T, K, N,
                                buckets[b].r, buckets[b].n_ad, workspace, workspace_bytes, BucketFilter{tok_bucket, b}, stream))
       return e;
   }
+  return MLORA_OK;
+}
+
+extern "C" int mlora_gather_mm_multi_proj(void* y, int y_dtype, int ldy, const void* x, int x_layout,
+                                          const mlora_lora_bucket* buckets, int n_buckets, int n_proj,
+                                          const int32_t* col_offset, const int32_t* n_cols, const int32_t* tok_bucket,
+                                          const int32_t* tok_adapter, int T, int K, void* workspace, size_t workspace_bytes,
+                                          void* stream) {
+  MLORA_CHECK(buckets && n_buckets > 0 && n_buckets <= 64 && n_proj > 0 && n_proj <= 8, MLORA_ERR_INVALID,
+              "gather_mm_multi_proj: bad bucket list (n_buckets=%d n_proj=%d)", n_buckets, n_proj);
+  MLORA_CHECK(y && x && col_offset && n_cols && tok_bucket && tok_adapter, MLORA_ERR_INVALID, "gather_mm_multi_proj: null pointer");
+  MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "gather_mm_multi_proj: bad y_dtype %d", y_dtype);
+  // validate everything before the first launch, so that an error leaves y untouched
+  for (int p = 0; p < n_proj; ++p) {
+    MLORA_CHECK(col_offset[p] >= 0 && col_offset[p] % 8 == 0 && n_cols[p] > 0 && col_offset[p] + n_cols[p] <= ldy, MLORA_ERR_INVALID,
+                "gather_mm_multi_proj: projection %d: columns %d..%d (offset must be a multiple of 8, row of %d)", p, col_offset[p],
+                col_offset[p] + n_cols[p], ldy);
+    for (int b = 0; b < n_buckets; ++b) {
+      const mlora_lora_bucket& bk = buckets[p * n_buckets + b];
+      if (!bk.A && !bk.B) continue;
+      if (int e = check_lora_shape(T, K, n_cols[p], bk.r, bk.n_ad)) return e;
+      MLORA_CHECK(bk.A && bk.B, MLORA_ERR_INVALID, "gather_mm_multi_proj: projection %d bucket %d has one null table", p, b);
+      MLORA_CHECK(T == 0 || (workspace && workspace_bytes >= mlora_gather_mm_workspace_bytes(T, K, bk.r)), MLORA_ERR_WORKSPACE,
+                  "gather_mm_multi_proj: workspace of %zu bytes given, %zu needed (rank %d)", workspace_bytes,
+                  mlora_gather_mm_workspace_bytes(T, K, bk.r), bk.r);
+    }
+  }
+  if (int rc = gmm_multi_one_launch(y, y_dtype, ldy, x, x_layout, buckets, n_buckets, n_proj, col_offset, n_cols, tok_bucket,
+                                    tok_adapter, T, K, (hipStream_t)stream))
+    return rc < 0 ? rc : MLORA_OK;
+  const size_t esz = y_dtype == MLORA_F16 ? 2 : 4;
+  for (int p = 0; p < n_proj; ++p)
+    if (int e = mlora_gather_mm_multi((char*)y + (size_t)col_offset[p] * esz, y_dtype, ldy, x, x_layout, buckets + p * n_buckets,
+                                      n_buckets, tok_bucket, tok_adapter, T, K, n_cols[p], workspace, workspace_bytes, stream))
+      return e;
   return MLORA_OK;
 }
 

@@ -201,6 +201,28 @@ class LlamaForCausalLM:
             if tab is not None:
                 ops.gather_mm(y, x, tab[0], tab[1], ids, lt.scaling, self._workspace(x.shape[0], x.shape[1], lt.r))
 
+    def _lora_group(self, y, x, l, projs, tok_adapter):
+        """The deltas of projections that read the same x and own column ranges of one fused output row:
+        projs = ((name, first column, columns), ...).  Batches that mix adapter types issue one call for the group."""
+        if "multi" in tok_adapter:
+            tb, ta = tok_adapter["multi"]
+            live, offs, cols = [], [], []
+            for proj, c0, n in projs:
+                buckets = []
+                for lt in self.lora_types:
+                    tab = lt.tables.get((l, proj))
+                    buckets.append(None if tab is None else (tab[0], tab[1], lt.scaling))
+                if any(b is not None for b in buckets):
+                    live.append(buckets)
+                    offs.append(c0)
+                    cols.append(n)
+            if live:
+                rmax = max(lt.r for lt in self.lora_types)
+                ops.gather_mm_multi_proj(y, x, live, offs, cols, tb, ta, self._workspace(x.shape[0], x.shape[1], rmax))
+            return
+        for proj, c0, n in projs:
+            self._lora(y[:, c0:c0 + n], x, l, proj, tok_adapter)
+
     @staticmethod
     def _merge_types(tok_adapter):
         """{tid: ids} with at most one adapter per token -> per-token (type, weight row) arrays for the multi-rank call."""
@@ -238,9 +260,8 @@ class LlamaForCausalLM:
             xn = ops.rmsnorm(resid, L["ln1"], s.rms_norm_eps, frag=frag, parts=parts)
             qkv = ops.linear(xn, L["qkv"])
             if tok_adapter:
-                self._lora(qkv[:, :q_sz], xn, l, "q_proj", tok_adapter)
-                self._lora(qkv[:, q_sz:q_sz + kv_sz], xn, l, "k_proj", tok_adapter)
-                self._lora(qkv[:, q_sz + kv_sz:], xn, l, "v_proj", tok_adapter)
+                self._lora_group(qkv, xn, l, (("q_proj", 0, q_sz), ("k_proj", q_sz, kv_sz), ("v_proj", q_sz + kv_sz, kv_sz)),
+                                 tok_adapter)
             attn = kv.attention_with_fused_qkv(l, qkv, s.num_attention_heads, frag=frag)
             parts = self._linear_acc(attn, L["o"], resid, ks_ws)
             if tok_adapter:
@@ -248,8 +269,7 @@ class LlamaForCausalLM:
             xn = ops.rmsnorm(resid, L["ln2"], s.rms_norm_eps, frag=frag, parts=parts)
             gu = ops.linear(xn, L["gate_up"])
             if tok_adapter:
-                self._lora(gu[:, :I], xn, l, "gate_proj", tok_adapter)
-                self._lora(gu[:, I:], xn, l, "up_proj", tok_adapter)
+                self._lora_group(gu, xn, l, (("gate_proj", 0, I), ("up_proj", I, I)), tok_adapter)
             act = ops.silu_mul(gu, frag=frag)
             parts = self._linear_acc(act, L["down"], resid, ks_ws)
             if tok_adapter:

@@ -136,6 +136,50 @@ def gather_mm_multi(y, x, buckets, tok_bucket, tok_adapter, workspace=None):
     return y
 
 
+def gather_mm_multi_proj(y, x, proj_buckets, col_offsets, n_cols, tok_bucket, tok_adapter, workspace=None):
+    """gather_mm_multi for several projections that read the same x and own disjoint column ranges of y (q, k, v in the
+    fused qkv row; gate and up): proj_buckets[p] is the bucket list of projection p (as for gather_mm_multi, all of the
+    same length), whose delta goes to y[:, col_offsets[p] : col_offsets[p] + n_cols[p]].  One launch at decode sizes."""
+    import ctypes
+    from ._lib import LoraBucket
+    xptr, xlay, T, K = _x_arg(x)
+    n_proj = len(proj_buckets)
+    n_buckets = len(proj_buckets[0])
+    if y.shape[0] != T or tok_bucket.shape != (T,) or tok_adapter.shape != (T,) or len(col_offsets) != n_proj or len(n_cols) != n_proj \
+            or any(len(b) != n_buckets for b in proj_buckets):
+        raise ValueError("gather_mm_multi_proj: inconsistent shapes")
+    if T == 0:
+        return y
+    arr = (LoraBucket * (n_proj * n_buckets))()
+    rmax = 8
+    for p, buckets in enumerate(proj_buckets):
+        for i, bk in enumerate(buckets):
+            e = arr[p * n_buckets + i]
+            if bk is None:                      # the bucket's adapters do not target this projection
+                e.A = e.B = None
+                continue
+            A, B, scaling = bk
+            n_ad, r, K2 = A.shape
+            if K2 != K or B.shape != (n_ad, n_cols[p], r):
+                raise ValueError(f"gather_mm_multi_proj: projection {p} bucket {i} has A{tuple(A.shape)} B{tuple(B.shape)} "
+                                 f"for K={K} N={n_cols[p]}")
+            e.A, e.B = _dev(A, torch.float16, "A"), _dev(B, torch.float16, "B")
+            e.r, e.n_ad, e.scaling = r, n_ad, float(scaling)
+            rmax = max(rmax, r)
+    if workspace is None:
+        workspace = gather_mm_workspace(T, K, rmax, x.device)
+    if not y.is_cuda or y.stride(1) != 1:
+        raise ValueError("gather_mm_multi_proj: y must be a GPU tensor with unit inner stride")
+    ldy = y.stride(0) if T > 1 else max(y.shape[1], y.stride(0))
+    co = (ctypes.c_int32 * n_proj)(*[int(c) for c in col_offsets])
+    nc = (ctypes.c_int32 * n_proj)(*[int(c) for c in n_cols])
+    check(lib().mlora_gather_mm_multi_proj(y.data_ptr(), _dt(y), ldy, xptr, xlay, ctypes.cast(arr, ctypes.c_void_p), n_buckets, n_proj,
+                                           ctypes.cast(co, ctypes.c_void_p), ctypes.cast(nc, ctypes.c_void_p),
+                                           _dev(tok_bucket, torch.int32, "tok_bucket"), _dev(tok_adapter, torch.int32, "tok_adapter"),
+                                           T, K, _dev(workspace, torch.float32, "workspace"), workspace.numel() * 4, _stream()))
+    return y
+
+
 class GatherMMBatch:
     """Several gather-matmul problems of one shape and one token->adapter table, issued as one launch.
     sets: list of (y, x, A, B) as for gather_mm (x row-major); the tensors are kept alive by this object."""

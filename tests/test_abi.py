@@ -62,6 +62,20 @@ def test_argument_validation_of_fused_and_batched_entry_points():
     bk[1].A = None
     assert lib.mlora_gather_mm_multi(1, 0, 64, 1, 0, C.cast(bk, C.c_void_p), 2, 1, 1, 8, 64, 64, 1, 1 << 20, None) == -1   # one null table
     assert lib.mlora_gather_mm_multi(1, 0, 64, 1, 0, None, 2, 1, 1, 8, 64, 64, 1, 1 << 20, None) == -1
+    # several projections in one call: column ranges and every bucket are checked before anything is launched
+    bk4 = (lm.LoraBucket * 4)()
+    for e in bk4:
+        e.A, e.B, e.r, e.n_ad, e.scaling = 1, 1, 16, 4, 0.5
+    co, nc = (C.c_int32 * 2)(0, 64), (C.c_int32 * 2)(64, 64)
+    mp = lambda ldy=128, r3=16, co=co: lib.mlora_gather_mm_multi_proj(1, 0, ldy, 1, 0, C.cast(bk4, C.c_void_p), 2, 2, C.cast(co, C.c_void_p),
+                                                                      C.cast(nc, C.c_void_p), 1, 1, 8, 64, 1, 1 << 20, None)
+    assert mp(ldy=120) == -1 and b"columns" in lib.mlora_last_error()               # second projection ends past the row
+    assert mp(co=(C.c_int32 * 2)(0, 60)) == -1                                         # offset not a multiple of 8
+    bk4[3].r = 12
+    assert mp() == -2 and b"rank" in lib.mlora_last_error()
+    bk4[3].r = 16
+    assert lib.mlora_gather_mm_multi_proj(1, 0, 128, 1, 0, C.cast(bk4, C.c_void_p), 2, 9, C.cast(co, C.c_void_p), C.cast(nc, C.c_void_p),
+                                          1, 1, 8, 64, 1, 1 << 20, None) == -1         # more than 8 projections
     # batched gather-matmul: decode shapes only
     assert lib.mlora_gather_mm_batch(1, 4, 0, 64, 0, 1, 1.0, 65, 64, 64, 16, 2, None) == -2
     assert lib.mlora_gather_mm_batch(None, 4, 0, 64, 0, 1, 1.0, 8, 64, 64, 16, 2, None) == -1

@@ -445,6 +445,38 @@ def test_gather_mm_multi_one_launch_with_absent_bucket_and_fragment_input(ops, s
         assert not torch.equal(multi, y0)
 
 
+@pytest.mark.parametrize("T", [32, 100])
+def test_gather_mm_multi_proj_equals_one_call_per_projection(ops, synth, T):
+    """q, k, v of a grouped-query layer (column ranges of different widths of one fused row) with two rank buckets, one
+    of which does not target k: one call for the group gives the bits of one multi-rank call per projection.
+    T = 32 is one launch, T = 100 the per-projection fallback."""
+    K, cols = 1024, (512, 128, 128)
+    offs = (0, 512, 640)
+    ranks, n_ads, scal = (16, 32), (5, 3), (0.5, 0.25)
+    x = synth.normal(24, "mp.x", (T, K), 1.0, torch.float16, DEV)
+    y0 = synth.normal(24, "mp.y", (T, sum(cols)), 1.0, torch.float16, DEV)
+    tb = (synth.randint(24, "mp.bucket", (T,), 3, DEV) - 1).to(torch.int32)
+    ta = torch.stack([synth.randint(24, f"mp.ad{i}", (T,), n, DEV) for i, n in enumerate(n_ads)])
+    tok_adapter = torch.where(tb >= 0, ta.gather(0, tb.clamp(min=0).long()[None])[0], torch.full_like(tb, -1)).to(torch.int32)
+    projs = []
+    for p, n in enumerate(cols):
+        bks = []
+        for i, (r, na, s) in enumerate(zip(ranks, n_ads, scal)):
+            if p == 1 and i == 1:
+                bks.append(None)
+            else:
+                bks.append((synth.normal(24, f"mp.A{p}{i}", (na, r, K), 0.05, torch.float16, DEV),
+                            synth.normal(24, f"mp.B{p}{i}", (na, n, r), 0.05, torch.float16, DEV), s))
+        projs.append(bks)
+    xin = ops.FragActivation.pack(x) if T <= 64 else x
+    got = ops.gather_mm_multi_proj(y0.clone(), xin, projs, offs, cols, tb, tok_adapter)
+    want = y0.clone()
+    for p, (c0, n) in enumerate(zip(offs, cols)):
+        ops.gather_mm_multi(want[:, c0:c0 + n], xin, projs[p], tb, tok_adapter)
+    assert torch.equal(got, want)
+    assert not torch.equal(got, y0)
+
+
 @pytest.mark.parametrize("T,K,N", [(48, 1024, 512), (150, 2048, 1024)])
 def test_gather_mm_multi_rank_strategies_agree(ops, synth, T, K, N):
     """Three rank buckets (8, 16, 64) in one call: equal, bit for bit, to one masked call per bucket (the reference's
