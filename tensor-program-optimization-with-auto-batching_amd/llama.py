@@ -201,6 +201,10 @@ class LlamaForCausalLM:
             if tab is not None:
                 ops.gather_mm(y, x, tab[0], tab[1], ids, lt.scaling, self._workspace(x.shape[0], x.shape[1], lt.r))
 
+    def _targets(self, l, *projs):
+        """Does any loaded adapter type carry tables for one of these projections of layer l?"""
+        return any(lt.tables.get((l, p)) is not None for lt in self.lora_types for p in projs)
+
     def _lora_group(self, y, x, l, projs, tok_adapter):
         """The deltas of projections that read the same x and own column ranges of one fused output row:
         projs = ((name, first column, columns), ...).  Batches that mix adapter types issue one call for the group."""
@@ -267,10 +271,14 @@ class LlamaForCausalLM:
             if tok_adapter:
                 self._lora(resid, attn, l, "o_proj", tok_adapter)
             xn = ops.rmsnorm(resid, L["ln2"], s.rms_norm_eps, frag=frag, parts=parts)
-            gu = ops.linear(xn, L["gate_up"])
-            if tok_adapter:
-                self._lora_group(gu, xn, l, (("gate_proj", 0, I), ("up_proj", I, I)), tok_adapter)
-            act = ops.silu_mul(gu, frag=frag)
+            if frag and I % 32 == 0 and not (tok_adapter and self._targets(l, "gate_proj", "up_proj")):
+                # decode step without an adapter on gate / up: the SiLU product is the epilogue of the GEMV (same bits)
+                act = ops.gate_up_silu(xn, self.interleaved_gate_up()[l])
+            else:
+                gu = ops.linear(xn, L["gate_up"])
+                if tok_adapter:
+                    self._lora_group(gu, xn, l, (("gate_proj", 0, I), ("up_proj", I, I)), tok_adapter)
+                act = ops.silu_mul(gu, frag=frag)
             parts = self._linear_acc(act, L["down"], resid, ks_ws)
             if tok_adapter:
                 self._lora(resid, act, l, "down_proj", tok_adapter)
