@@ -341,7 +341,7 @@ def bench_c5_decode(args, synth, llama):
     kv.begin_forward(list(range(B)), [int(c) for c in ctx])          # claims the pages of the pre-filled contexts
     kv.end_forward()
     first = synth.randint(wl.seed, "c5.first", (B,), s.vocab_size).numpy()
-    sess = dsm.DecodeSession(model, kv, list(range(B)), {0: adapter_ids}, first)
+    sess = dsm.DecodeSession(model, kv, list(range(B)), {0: adapter_ids}, first, longest_first=not args.batch_order)
     for _ in range(args.warmup):
         sess.step()
     torch.cuda.synchronize()
@@ -379,6 +379,7 @@ def main():
                     help="c3_decode is the benchmark the metric is quoted on; the other two time the prefill and the "
                          "256-request stress configurations with the same harness")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--batch-order", action="store_true", help="c5_decode: keep the request order inside the batch (default: longest context first)")
     ap.add_argument("--own-gemm", action="store_true",
                     help="c4_prefill / c5_decode: base linears on this package's LDS GEMM instead of the vendor GEMM library")
     ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel event timing and the gather-matmul stream")

@@ -19,14 +19,26 @@ class DecodeSession:
     scratch buffers outside the graph's memory pool - and replayed, so the interpreter is out of the loop; the
     kernels and their order are those of the eager step, hence the same tokens bit for bit."""
 
-    def __init__(self, model, kv, seq_ids, tok_adapter, first_tokens, use_graph=False):
+    def __init__(self, model, kv, seq_ids, tok_adapter, first_tokens, use_graph=False, longest_first=False):
         """seq_ids: sequences already prefilled in `kv`; tok_adapter: {tid: ids [B] int32 (host or device), -1 = the
-        row does not use that type}; first_tokens [B]: the tokens produced by prefill."""
+        row does not use that type}; first_tokens [B]: the tokens produced by prefill.
+        longest_first: run the batch internally in order of decreasing context length, so that the attention
+        workgroups of the longest sequences start first and the short ones fill the tail of the launch (every
+        operator treats rows independently: a sequence's results do not depend on its row); step() still returns
+        the tokens in the caller's order."""
         self.model, self.kv = model, kv
-        self.seq_ids = list(seq_ids)
-        B = len(self.seq_ids)
+        B = len(seq_ids)
         dev = model.device
         i32 = lambda a: (a if isinstance(a, torch.Tensor) else torch.as_tensor(np.asarray(a, dtype=np.int32))).to(dev, torch.int32)
+        self._inv = None
+        if longest_first and B > 1:
+            order = np.argsort(-np.asarray([kv.lens[s] for s in seq_ids], dtype=np.int64), kind="stable")
+            od = torch.from_numpy(order).to(dev)
+            seq_ids = [seq_ids[i] for i in order]
+            tok_adapter = {tid: i32(ids).index_select(0, od) for tid, ids in tok_adapter.items()}
+            first_tokens = i32(first_tokens).index_select(0, od)
+            self._inv = torch.from_numpy(np.argsort(order)).to(dev)
+        self.seq_ids = list(seq_ids)
         self.tok_adapter = {tid: i32(ids) for tid, ids in tok_adapter.items()}
         if len(self.tok_adapter) > 1:         # several adapter types: merged once here (the check reads back to the host)
             self.tok_adapter = model._merge_types(self.tok_adapter)
@@ -61,9 +73,10 @@ class DecodeSession:
             self._enqueue()
             self._eager_steps += 1
         kv.end_forward()
+        out = self.tokens if self._inv is None else self.tokens.index_select(0, self._inv)
         if keep_history:
-            self.history.append(self.tokens.clone())
-        return self.tokens
+            self.history.append(out.clone() if self._inv is None else out)
+        return out
 
 
 class NativeDecodeSession:

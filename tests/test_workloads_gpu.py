@@ -127,3 +127,36 @@ def test_decode_more_than_64_requests_zipf_adapters_ragged_contexts():
     for s in range(B):
         n_blk = -(-(lens[s] + steps) // 16)
         assert list(kvh.table_h[kvh.slot[s], :n_blk]) == list(kvr.tables[s])[:n_blk]
+
+
+@pytest.mark.parametrize("B,use_graph", [(70, False), (12, True)])
+def test_decode_session_longest_context_first_keeps_tokens_and_request_order(B, use_graph):
+    """The session may run its batch internally in order of decreasing context length (the long sequences' attention
+    workgroups start first); every operator treats rows independently, so each request's tokens and cache pages are
+    those of the batch in request order, bit for bit, and come back in request order."""
+    synth = load_pkg("synth")
+    dsm = load_pkg("decode_session")
+    shape = _small_shape(synth)
+    n_ad = 6
+    lora = synth.LoraSpec(r=16, alpha=8.0, n_adapters=n_ad, targets=("q_proj", "k_proj", "v_proj", "o_proj"))
+    ids = synth.randint(6, f"lf.ids{B}", (B,), n_ad + 1).numpy().astype(np.int32) - 1        # -1 = no adapter
+    wl = synth.Workload("lf_small", 6, shape, lora, batch=B, prompt_len=90, gen_len=6, adapter_ids=ids)
+    lens = (5 + synth.randint(6, f"lf.ctx{B}", (B,), 86).numpy()).tolist()
+    prompts = [synth.randint(6, f"lf.prompt{B}.{i}", (n,), shape.vocab_size).numpy() for i, n in enumerate(lens)]
+    steps = 6
+    n_pages = sum(-(-(n + steps + 1) // 16) for n in lens) + 4
+    perm = synth.permutation(6, f"lf.pages{B}", n_pages)
+    model = hip_model(wl)
+    runs = []
+    for longest_first in (False, True):
+        kv, logits = _hip_prefill(model, prompts, ids, n_pages, 16, perm, 112)
+        first = logits.argmax(-1).astype(np.int32)
+        sess = dsm.DecodeSession(model, kv, list(range(B)), {0: ids}, first, use_graph=use_graph, longest_first=longest_first)
+        toks = np.stack([sess.step().cpu().numpy().copy() for _ in range(steps)])
+        rows = [[kv.k[0][p].clone() for p in kv.pages_of(s)] for s in range(B)]
+        runs.append((toks, rows, [kv.lens[s] for s in range(B)]))
+    (t0, r0, l0), (t1, r1, l1) = runs
+    assert np.array_equal(t0, t1)
+    assert l0 == l1 == [n + steps for n in lens]
+    for s in range(B):
+        assert len(r0[s]) == len(r1[s]) and all(torch.equal(a, b) for a, b in zip(r0[s], r1[s])), s
