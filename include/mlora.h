@@ -111,8 +111,11 @@ int mlora_gather_mm_multi(void* y, int y_dtype, int ldy, const void* x, int x_la
 /* The same for n_proj projections that read the same x and write disjoint column ranges of one y (q, k, v inside the
  * fused qkv row; gate and up): projection p adds to columns col_offset[p] .. col_offset[p] + n_cols[p] - 1 of y
  * (col_offset[p] % 8 == 0) with the tables buckets[p * n_buckets + b] (B [n_ad, n_cols[p], r]).  A decode-sized batch
- * with at most eight non-null (projection, bucket) entries is ONE launch; otherwise one mlora_gather_mm_multi per
- * projection.  Same result bits as those calls.  buckets, col_offset and n_cols are HOST arrays.
+ * with at most eight non-null (projection, bucket) entries is ONE launch.  Larger batches: per bucket, up to three
+ * projections that carry it with the same rank, table size and scaling share one shrink and one expand launch on the
+ * matrix cores, provided the workspace holds one slice of mlora_gather_mm_workspace_bytes(T, K, r) per projection
+ * (otherwise, and for everything else, one mlora_gather_mm per projection and bucket).  Same result bits as one
+ * mlora_gather_mm_multi call per projection.  buckets, col_offset and n_cols are HOST arrays.
  * Replaces: q_ft_proj + v_ft_proj of the patched attention forward, one take-matmul pair each
  * (tvm/llama_auto_batcher/compile_tvm.py:126-155). */
 int mlora_gather_mm_multi_proj(void* y, int y_dtype, int ldy, const void* x, int x_layout,

@@ -419,6 +419,17 @@ __global__ __launch_bounds__(GMM_THREADS, (GR == 8 ? 4 : 2)) void gather_mm_deco
 // ---------------------------------------------------------------------------------------------
 constexpr int SEG_WAVES = 4;
 
+// Projections that share x, the token table, the rank and the scaling (q, k, v; gate, up): blockIdx.z selects one.
+// Projection z keeps its shrink results in slice z of the workspace.
+constexpr int SEG_MAX_PROJ = 3;
+struct SegProjs {
+  const f16* A[SEG_MAX_PROJ];
+  const f16* B[SEG_MAX_PROJ];
+  void* y[SEG_MAX_PROJ];
+  int N[SEG_MAX_PROJ];
+  int n;
+};
+
 // The distinct adapters of a 16-token tile (lanes 0..15 hold the tokens' ids, -1 = none) and, per adapter, the mask of
 // tile rows bound to it.  Everything is wave-uniform and lives in scalar registers; the loops over the list are fully
 // unrolled with a uniform `i < n` guard, so the list is never indexed dynamically.
@@ -456,10 +467,14 @@ __device__ __forceinline__ TileAdapters tile_adapters(int id) {
 // 16 tokens holds up to 16 adapters, costs one K loop instead of 16, with all the groups' loads in flight together.
 template <int R>
 __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(float* __restrict__ v, const f16* __restrict__ x,
-                                                                            const f16* __restrict__ A,
+                                                                            SegProjs pj,
                                                                             const int32_t* __restrict__ ids, int T, int K,
                                                                             int n_ad, const int32_t* __restrict__ bucket_of,
                                                                             int bucket) {
+  const f16* __restrict__ A = pj.A[0];
+#pragma unroll
+  for (int i = 1; i < SEG_MAX_PROJ; ++i)
+    if (i == blockIdx.z) A = pj.A[i];                    // uniform select: the struct is never indexed dynamically
   // blockIdx.y selects one of gridDim.y contiguous ranges of 32-k steps; its partial sums go to v[blockIdx.y][T][R]
   constexpr int NT = (R + 15) / 16;     // 16-row tiles of A[a]; rank 8 uses half a tile
   constexpr int GA = 8 / NT;            // adapters per pass: 32 accumulator registers
@@ -475,7 +490,7 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(floa
   const int KB = K / 32;
   const int per = (KB + gridDim.y - 1) / gridDim.y;
   const int kb0 = blockIdx.y * per, kb1 = min(KB, kb0 + per);
-  v += (size_t)blockIdx.y * T * R;
+  v += ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * T * R;
 #pragma unroll
   for (int g0 = 0; g0 < 16; g0 += GA) {
     if (g0 < ta.n) {                                             // uniform
@@ -544,12 +559,22 @@ __device__ __forceinline__ bool next_tile_adapter(int id, unsigned& todo, int& a
 // Expand for segment-ordered tokens (prefill): one pass per distinct adapter of the tile - one, two at a segment boundary.
 // Lean in registers (seven waves per SIMD), which is what this latency-bound kernel lives on.
 template <int R, typename YT>
-__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* __restrict__ y, const float* __restrict__ v,
-                                                                            const f16* __restrict__ B,
+__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(SegProjs pj, const float* __restrict__ v,
                                                                             const int32_t* __restrict__ ids, float scaling,
-                                                                            int T, int N, int ldy, int n_ad,
+                                                                            int T, int ldy, int n_ad,
                                                                             const int32_t* __restrict__ bucket_of, int bucket,
                                                                             int splits, int nit) {
+  YT* __restrict__ y = (YT*)pj.y[0];
+  const f16* __restrict__ B = pj.B[0];
+  int N = pj.N[0];
+#pragma unroll
+  for (int i = 1; i < SEG_MAX_PROJ; ++i)
+    if (i == blockIdx.z) {                               // uniform select: the struct is never indexed dynamically
+      y = (YT*)pj.y[i];
+      B = pj.B[i];
+      N = pj.N[i];
+    }
+  v += (size_t)blockIdx.z * splits * T * R;
   constexpr int KS = (R + 31) / 32;     // k-steps of 32 rank entries (ranks 8 and 16: one partly filled step)
   constexpr int CT = 4;                 // 16-column tiles per wave
   constexpr int LD = 16 * CT + 4;       // padded row of the transposition buffer (floats): conflict-free both ways
@@ -642,12 +667,22 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(YT* 
 // v); a token's column of the result is taken from the product of its own adapter, so all adapters are worked off before
 // the one read-modify-write of y.  The B fragments of up to GB adapters are requested together.
 template <int R, typename YT>
-__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mixed_mfma_kernel(YT* __restrict__ y, const float* __restrict__ v,
-                                                                            const f16* __restrict__ B,
+__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mixed_mfma_kernel(SegProjs pj, const float* __restrict__ v,
                                                                             const int32_t* __restrict__ ids, float scaling,
-                                                                            int T, int N, int ldy, int n_ad,
+                                                                            int T, int ldy, int n_ad,
                                                                             const int32_t* __restrict__ bucket_of, int bucket,
                                                                             int splits, int nit) {
+  YT* __restrict__ y = (YT*)pj.y[0];
+  const f16* __restrict__ B = pj.B[0];
+  int N = pj.N[0];
+#pragma unroll
+  for (int i = 1; i < SEG_MAX_PROJ; ++i)
+    if (i == blockIdx.z) {                               // uniform select: the struct is never indexed dynamically
+      y = (YT*)pj.y[i];
+      B = pj.B[i];
+      N = pj.N[i];
+    }
+  v += (size_t)blockIdx.z * splits * T * R;
   constexpr int KS = (R + 31) / 32;     // k-steps of 32 rank entries (ranks 8 and 16: one partly filled step)
   constexpr int GB = 8 / KS;            // adapters whose fragments are in flight together: 32 registers
   constexpr int CT = 4;                 // 16-column tiles per wave
@@ -955,27 +990,30 @@ extern "C" int mlora_gather_mm_batch(const void* const* sets, int n_sets, int y_
 }
 
 template <int R>
-static void gmm_segments_r(void* y, int y_dtype, int ldy, const f16* x, const f16* A, const f16* B, const int32_t* ids,
-                           float scaling, int T, int K, int N, int n_ad, float* v, BucketFilter bf, hipStream_t s) {
+static void gmm_segments_r(const SegProjs& pj, int y_dtype, int ldy, const f16* x, const int32_t* ids, float scaling, int T, int K,
+                           int n_ad, float* v, BucketFilter bf, hipStream_t s) {
   const int tiles = ceil_div(T, 16);
+  int N = 0;
+  for (int i = 0; i < pj.n; ++i) N = pj.N[i] > N ? pj.N[i] : N;
   // few token tiles: split K over workgroups so that the shrink still covers the chip (partials fit the workspace,
-  // which holds lora_k_split(K).kc slices of [T, r])
+  // which holds lora_k_split(K).kc slices of [T, r] per projection); the same split whatever the number of
+  // projections, so that a projection's sums do not depend on what shares its launch
   int splits = 512 / tiles;
   const int kc = lora_k_split(K).kc;
   if (splits > kc) splits = kc;
   if (splits > K / 128) splits = K / 128;
   if (splits < 1) splits = 1;
-  hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles, splits), dim3(SEG_WAVES * WAVE), 0, s, v, x, A, ids, T, K, n_ad,
+  hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles, splits, pj.n), dim3(SEG_WAVES * WAVE), 0, s, v, x, pj, ids, T, K, n_ad,
                      bf.bucket_of, bf.bucket);
   // column blocks per workgroup: as many as leave about a thousand workgroups (per-workgroup set-up amortised)
-  int nit = (int)(((long)tiles * ceil_div(N, SEG_WAVES * 64)) / 1024);
+  int nit = (int)(((long)tiles * pj.n * ceil_div(N, SEG_WAVES * 64)) / 1024);
   nit = nit < 1 ? 1 : (nit > 8 ? 8 : nit);
-  const dim3 grid(tiles, ceil_div(N, SEG_WAVES * 64 * nit));
+  const dim3 grid(tiles, ceil_div(N, SEG_WAVES * 64 * nit), pj.n);
   // Up to 1024 tokens the call is taken to be a decode batch (one token per sequence, tiles that mix many adapters);
   // beyond that a prefill whose tokens come in adapter segments.  Either kernel is correct for either input.
   const bool mixed = T <= 1024;
 #define MLORA_EXPAND_MFMA(KERNEL, YT)                                                                                       \
-  hipLaunchKernelGGL((KERNEL<R, YT>), grid, dim3(SEG_WAVES * WAVE), 0, s, (YT*)y, v, B, ids, scaling, T, N, ldy, n_ad, \
+  hipLaunchKernelGGL((KERNEL<R, YT>), grid, dim3(SEG_WAVES * WAVE), 0, s, pj, v, ids, scaling, T, ldy, n_ad, \
                      bf.bucket_of, bf.bucket, splits, nit)
   if (y_dtype == MLORA_F16) {
     if (mixed) MLORA_EXPAND_MFMA(lora_expand_mixed_mfma_kernel, f16);
@@ -987,16 +1025,21 @@ static void gmm_segments_r(void* y, int y_dtype, int ldy, const f16* x, const f1
 #undef MLORA_EXPAND_MFMA
 }
 
-// shrink + expand on the matrix cores; v = workspace viewed as [T, r] fp32
-static int gmm_segments(void* y, int y_dtype, int ldy, const f16* x, const f16* A, const f16* B, const int32_t* ids,
-                        float scaling, int T, int K, int N, int r, int n_ad, float* v, BucketFilter bf, hipStream_t s) {
+// shrink + expand on the matrix cores for pj.n projections; v = workspace viewed as [pj.n][splits][T, r] fp32
+static int gmm_segments(const SegProjs& pj, int y_dtype, int ldy, const f16* x, const int32_t* ids, float scaling, int T, int K,
+                        int r, int n_ad, float* v, BucketFilter bf, hipStream_t s) {
   switch (r) {
-    case 8: gmm_segments_r<8>(y, y_dtype, ldy, x, A, B, ids, scaling, T, K, N, n_ad, v, bf, s); break;
-    case 16: gmm_segments_r<16>(y, y_dtype, ldy, x, A, B, ids, scaling, T, K, N, n_ad, v, bf, s); break;
-    case 32: gmm_segments_r<32>(y, y_dtype, ldy, x, A, B, ids, scaling, T, K, N, n_ad, v, bf, s); break;
-    default: gmm_segments_r<64>(y, y_dtype, ldy, x, A, B, ids, scaling, T, K, N, n_ad, v, bf, s); break;
+    case 8: gmm_segments_r<8>(pj, y_dtype, ldy, x, ids, scaling, T, K, n_ad, v, bf, s); break;
+    case 16: gmm_segments_r<16>(pj, y_dtype, ldy, x, ids, scaling, T, K, n_ad, v, bf, s); break;
+    case 32: gmm_segments_r<32>(pj, y_dtype, ldy, x, ids, scaling, T, K, n_ad, v, bf, s); break;
+    default: gmm_segments_r<64>(pj, y_dtype, ldy, x, ids, scaling, T, K, n_ad, v, bf, s); break;
   }
   return mlora_launch_status("gather_mm");
+}
+
+// the matrix-core kernels need row-major x, 16-byte aligned rows of y and whole 16-column tiles
+static bool gmm_segments_fit(const void* y, int ldy, int x_layout, int T, int K, int N) {
+  return x_layout == MLORA_ROWMAJOR && T > 64 && K % 32 == 0 && N % 16 == 0 && ldy % 8 == 0 && (uintptr_t)y % 16 == 0;
 }
 
 static int gather_mm_impl(void* y, int y_dtype, int ldy, const void* x, int x_layout, const void* A, const void* B,
@@ -1016,12 +1059,14 @@ static int gather_mm_impl(void* y, int y_dtype, int ldy, const void* x, int x_la
     const GmmSet one = {y, (const f16*)x, (const f16*)A, (const f16*)B};
     return gmm_one_launch(one, nullptr, 1, y_dtype, ldy, x_layout, tok_adapter, scaling, T, K, N, r, n_ad, (hipStream_t)stream, bf);
   }
-  if (x_layout == MLORA_ROWMAJOR && T > 64 && K % 32 == 0 && N % 16 == 0 && ldy % 8 == 0 && (uintptr_t)y % 16 == 0) {
+  if (gmm_segments_fit(y, ldy, x_layout, T, K, N)) {
     MLORA_CHECK(y && x && A && B && tok_adapter, MLORA_ERR_INVALID, "gather_mm: null pointer");
     MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "gather_mm: bad y_dtype %d", y_dtype);
     MLORA_CHECK(ldy >= N, MLORA_ERR_INVALID, "gather_mm: need ldy >= N (ldy=%d N=%d)", ldy, N);
-    return gmm_segments(y, y_dtype, ldy, (const f16*)x, (const f16*)A, (const f16*)B, tok_adapter, scaling, T, K, N, r, n_ad,
-                        (float*)workspace, bf, (hipStream_t)stream);
+    SegProjs pj = {};
+    pj.A[0] = (const f16*)A; pj.B[0] = (const f16*)B; pj.y[0] = y; pj.N[0] = N; pj.n = 1;
+    return gmm_segments(pj, y_dtype, ldy, (const f16*)x, tok_adapter, scaling, T, K, r, n_ad, (float*)workspace, bf,
+                        (hipStream_t)stream);
   }
   if (int e = shrink_impl(workspace, x, x_layout, A, tok_adapter, T, K, r, n_ad, bf, stream)) return e;
   return expand_impl(y, y_dtype, ldy, workspace, B, tok_adapter, scaling, T, K, N, r, n_ad, bf, stream);
@@ -1137,10 +1182,38 @@ extern "C" int mlora_gather_mm_multi_proj(void* y, int y_dtype, int ldy, const v
                                     tok_adapter, T, K, (hipStream_t)stream))
     return rc < 0 ? rc : MLORA_OK;
   const size_t esz = y_dtype == MLORA_F16 ? 2 : 4;
+  if (T == 0) return MLORA_OK;
+  // Larger batches: per rank bucket, the projections that carry it (same rank, table size and scaling) share one
+  // shrink launch and one expand launch on the matrix cores when the workspace holds a slice for each of them.
+  bool done[8 * 64] = {};
+  for (int b = 0; b < n_buckets; ++b) {
+    SegProjs pj = {};
+    int members[SEG_MAX_PROJ];
+    const mlora_lora_bucket* lead = nullptr;
+    for (int p = 0; p < n_proj && pj.n < SEG_MAX_PROJ; ++p) {
+      const mlora_lora_bucket& bk = buckets[p * n_buckets + b];
+      void* yp = (char*)y + (size_t)col_offset[p] * esz;
+      if (!bk.A || !gmm_segments_fit(yp, ldy, x_layout, T, K, n_cols[p])) continue;
+      if (lead && (bk.r != lead->r || bk.n_ad != lead->n_ad || bk.scaling != lead->scaling)) continue;
+      if (!lead) lead = &bk;
+      pj.A[pj.n] = (const f16*)bk.A; pj.B[pj.n] = (const f16*)bk.B; pj.y[pj.n] = yp; pj.N[pj.n] = n_cols[p];
+      members[pj.n++] = p;
+    }
+    if (pj.n >= 2 && workspace_bytes >= (size_t)pj.n * mlora_gather_mm_workspace_bytes(T, K, lead->r)) {
+      if (int e = gmm_segments(pj, y_dtype, ldy, (const f16*)x, tok_adapter, lead->scaling, T, K, lead->r, lead->n_ad,
+                               (float*)workspace, BucketFilter{tok_bucket, b}, (hipStream_t)stream))
+        return e;
+      for (int i = 0; i < pj.n; ++i) done[members[i] * n_buckets + b] = true;
+    }
+  }
   for (int p = 0; p < n_proj; ++p)
-    if (int e = mlora_gather_mm_multi((char*)y + (size_t)col_offset[p] * esz, y_dtype, ldy, x, x_layout, buckets + p * n_buckets,
-                                      n_buckets, tok_bucket, tok_adapter, T, K, n_cols[p], workspace, workspace_bytes, stream))
-      return e;
+    for (int b = 0; b < n_buckets; ++b) {
+      const mlora_lora_bucket& bk = buckets[p * n_buckets + b];
+      if (!bk.A || done[p * n_buckets + b]) continue;
+      if (int e = gather_mm_impl((char*)y + (size_t)col_offset[p] * esz, y_dtype, ldy, x, x_layout, bk.A, bk.B, tok_adapter, bk.scaling,
+                                 T, K, n_cols[p], bk.r, bk.n_ad, workspace, workspace_bytes, BucketFilter{tok_bucket, b}, stream))
+        return e;
+    }
   return MLORA_OK;
 }
 

@@ -177,7 +177,8 @@ class LlamaForCausalLM:
         return ops.embed(self.embed_tokens, ids, out_dtype=torch.float32)
 
     def _workspace(self, T, K, r):
-        need = ops.lib().mlora_gather_mm_workspace_bytes(T, K, r) // 4 + 4
+        # three slices: projections that share an input (q, k, v) keep their shrink results side by side
+        need = 3 * (ops.lib().mlora_gather_mm_workspace_bytes(T, K, r) // 4) + 4
         if self._ws is None or self._ws.numel() < need:
             self._ws = torch.empty(need, dtype=torch.float32, device=self.device)
         return self._ws
@@ -223,6 +224,17 @@ class LlamaForCausalLM:
             if live:
                 rmax = max(lt.r for lt in self.lora_types)
                 ops.gather_mm_multi_proj(y, x, live, offs, cols, tb, ta, self._workspace(x.shape[0], x.shape[1], rmax))
+            return
+        (tid, ids), = tok_adapter.items()            # one adapter type: a single bucket that every token names
+        lt = self.lora_types[tid]
+        live = [(lt.tables.get((l, proj)), c0, n) for proj, c0, n in projs]
+        live = [(tab, c0, n) for tab, c0, n in live if tab is not None]
+        if len(live) >= 2:
+            zeros = getattr(self, "_zero_bucket", None)
+            if zeros is None or zeros.numel() < ids.numel():
+                zeros = self._zero_bucket = torch.zeros(max(ids.numel(), 64), dtype=torch.int32, device=self.device)
+            ops.gather_mm_multi_proj(y, x, [[(tab[0], tab[1], lt.scaling)] for tab, _, _ in live], [c0 for _, c0, _ in live],
+                                     [n for _, _, n in live], zeros[:ids.numel()], ids, self._workspace(x.shape[0], x.shape[1], lt.r))
             return
         for proj, c0, n in projs:
             self._lora(y[:, c0:c0 + n], x, l, proj, tok_adapter)

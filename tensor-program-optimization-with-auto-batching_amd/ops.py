@@ -167,7 +167,8 @@ def gather_mm_multi_proj(y, x, proj_buckets, col_offsets, n_cols, tok_bucket, to
             e.r, e.n_ad, e.scaling = r, n_ad, float(scaling)
             rmax = max(rmax, r)
     if workspace is None:
-        workspace = gather_mm_workspace(T, K, rmax, x.device)
+        one = gather_mm_workspace(T, K, rmax, x.device).numel()
+        workspace = torch.empty(3 * one, dtype=torch.float32, device=x.device)     # a slice per projection sharing a launch
     if not y.is_cuda or y.stride(1) != 1:
         raise ValueError("gather_mm_multi_proj: y must be a GPU tensor with unit inner stride")
     ldy = y.stride(0) if T > 1 else max(y.shape[1], y.stride(0))

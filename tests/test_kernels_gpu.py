@@ -445,11 +445,12 @@ def test_gather_mm_multi_one_launch_with_absent_bucket_and_fragment_input(ops, s
         assert not torch.equal(multi, y0)
 
 
-@pytest.mark.parametrize("T", [32, 100])
+@pytest.mark.parametrize("T", [32, 100, 300, 1100])
 def test_gather_mm_multi_proj_equals_one_call_per_projection(ops, synth, T):
     """q, k, v of a grouped-query layer (column ranges of different widths of one fused row) with two rank buckets, one
     of which does not target k: one call for the group gives the bits of one multi-rank call per projection.
-    T = 32 is one launch, T = 100 the per-projection fallback."""
+    T = 32 is one launch; larger batches run the matrix-core kernels with the projections of a bucket sharing the
+    shrink and the expand launch."""
     K, cols = 1024, (512, 128, 128)
     offs = (0, 512, 640)
     ranks, n_ads, scal = (16, 32), (5, 3), (0.5, 0.25)
