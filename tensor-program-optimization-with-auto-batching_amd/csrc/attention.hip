@@ -113,7 +113,7 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qk
   }
 }
 
-// Prefill-sized variant that moves 16 bytes at a time: one WAVE per (16 consecutive tokens, head), four heads per
+// Prefill-sized variant that moves 16 bytes at a time: one WAVE per (16 consecutive tokens, head of q / k / v), four heads per
 // workgroup, no barriers and no LDS.  Lane l works on token l % 16 of the tile throughout, so its sequence and
 // position stay in its own registers.  q heads are rotated in place in chunks of 8 pairs.  When the 16 tokens are
 // slots 0..15 of one page (prompts that start on a page boundary), a K fragment row (16 tokens x 16 B) and a V row
@@ -132,9 +132,9 @@ __global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restric
   constexpr int NCH = half / 8;                               // 8-pair chunks of a head row
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int t0 = blockIdx.x * 16;
-  const int hh = blockIdx.y * 4 + wave;                       // hh < Hq: a q head; else kv head hh - Hq (k and v)
+  const int hh = blockIdx.y * 4 + wave;                       // a head of the fused row: q heads, then k heads, then v heads
   const int HH = Hq + 2 * Hkv;
-  if (hh >= Hq + Hkv) return;
+  if (hh >= HH) return;
   const int tk = lane & 15, t = t0 + tk;
   int seq = -1, pos = -1;
   if (t < T) {
@@ -178,7 +178,8 @@ __global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restric
     }
     return;
   }
-  const int kh = hh - Hq;
+  const bool is_v = hh >= Hq + Hkv;                           // wave-uniform
+  const int kh = is_v ? hh - Hq - Hkv : hh - Hq;
   const int seq0 = __shfl(seq, 0, WAVE), pos0 = __shfl(pos, 0, WAVE);
   bool al = __ballot(seq >= 0 && seq == seq0 && pos == pos0 + tk) == ~0ull && (pos0 % PAGE) == 0;   // wave-uniform
   int page = -1;
@@ -186,7 +187,7 @@ __global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restric
     page = block_table[(size_t)seq0 * max_blocks + pos0 / PAGE];
     if (page < 0 || page >= n_pages) al = false;
   }
-  if (al) {
+  if (al && !is_v) {
     // K: the 16 tokens of a fragment chunk row are contiguous (16 B each)
     const f16* ksrc = qkv + ((size_t)t * HH + Hq + kh) * D;
     f16* kd = k_cache + ((size_t)page * Hkv + kh) * PAGE * D;
@@ -196,6 +197,9 @@ __global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restric
       st8(kd + ((size_t)ch * 16 + tk) * 8, o_lo);
       st8(kd + ((size_t)(ch + NCH) * 16 + tk) * 8, o_hi);
     }
+    return;
+  }
+  if (al) {
     // V: 8 tokens of one dim per item; a pair of lanes writes the dim's 32-byte row
     f16* vd = v_cache + ((size_t)page * Hkv + kh) * D * PAGE;
     for (int it = lane; it < D * 2; it += WAVE) {
@@ -214,16 +218,19 @@ __global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restric
     const int pg = block_table[(size_t)seq_e * max_blocks + pos_e / PAGE];
     if (pg < 0 || pg >= n_pages) continue;
     const int slot = pos_e % PAGE;
-    const f16* ksrc = qkv + ((size_t)(t0 + tke) * HH + Hq + kh) * D;
-    const f16* vsrc = qkv + ((size_t)(t0 + tke) * HH + Hq + Hkv + kh) * D;
-    const float c = rope_cos[(size_t)pos_e * half + i], s = rope_sin[(size_t)pos_e * half + i];
-    const float x1 = (float)ksrc[i], x2 = (float)ksrc[i + half];
-    f16* kd = k_cache + ((size_t)pg * Hkv + kh) * PAGE * D;
-    kd[k_page_offset(slot, i)] = rot(x1, x2, c, s, false);
-    kd[k_page_offset(slot, i + half)] = rot(x1, x2, c, s, true);
-    f16* vd = v_cache + ((size_t)pg * Hkv + kh) * D * PAGE + slot;
-    vd[(size_t)i * PAGE] = vsrc[i];
-    vd[(size_t)(i + half) * PAGE] = vsrc[i + half];
+    if (is_v) {
+      const f16* vsrc = qkv + ((size_t)(t0 + tke) * HH + Hq + Hkv + kh) * D;
+      f16* vd = v_cache + ((size_t)pg * Hkv + kh) * D * PAGE + slot;
+      vd[(size_t)i * PAGE] = vsrc[i];
+      vd[(size_t)(i + half) * PAGE] = vsrc[i + half];
+    } else {
+      const f16* ksrc = qkv + ((size_t)(t0 + tke) * HH + Hq + kh) * D;
+      const float c = rope_cos[(size_t)pos_e * half + i], s = rope_sin[(size_t)pos_e * half + i];
+      const float x1 = (float)ksrc[i], x2 = (float)ksrc[i + half];
+      f16* kd = k_cache + ((size_t)pg * Hkv + kh) * PAGE * D;
+      kd[k_page_offset(slot, i)] = rot(x1, x2, c, s, false);
+      kd[k_page_offset(slot, i + half)] = rot(x1, x2, c, s, true);
+    }
   }
 }
 
@@ -764,7 +771,7 @@ static int rope_kv_append_impl(const char* who, void* qkv, void* k_cache, void* 
   MLORA_CHECK(T >= 0 && max_pos > 0, MLORA_ERR_INVALID, "%s: bad T=%d max_pos=%d", who, T, max_pos);
   if (T == 0) return MLORA_OK;
   if (T > 64 && lx.src.v == nullptr && (((uintptr_t)rope_cos | (uintptr_t)rope_sin) & 15) == 0) {
-    const dim3 grid(ceil_div(T, 16), ceil_div(Hq + Hkv, 4));
+    const dim3 grid(ceil_div(T, 16), ceil_div(Hq + 2 * Hkv, 4));
     if (D == 128)
       hipLaunchKernelGGL(rope_kv_append_tile_kernel<128>, grid, dim3(256), 0, (hipStream_t)stream, (f16*)qkv, (f16*)k_cache,
                          (f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, rope_cos, rope_sin, max_pos, Hq, Hkv, n_pages,
