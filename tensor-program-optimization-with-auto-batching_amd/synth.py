@@ -221,11 +221,22 @@ def config1() -> Workload:
                     adapter_ids=np.arange(4, dtype=np.int32))
 
 
-def config3(num_layers: int = 32, batch: int = 32, prompt_len: int = 512, gen_len: int = 128) -> Workload:
-    """Llama-2-7B-shape decode: rank-16 adapters on q/k/v/o, 16 adapters round-robin over 32 requests."""
-    shape = LlamaShape(num_hidden_layers=num_layers)
+def llama31_8b_shape(num_layers: int = 32) -> LlamaShape:
+    """The reference's default model shape (`tvm/llama_auto_batcher/llama_for_causal_lm.py:12-21`): grouped-query
+    attention with 8 kv heads, intermediate size 14336, vocabulary 128256, rope theta 5e5."""
+    return LlamaShape(intermediate_size=14336, num_key_value_heads=8, num_hidden_layers=num_layers, vocab_size=128256,
+                      rope_theta=500000.0)
+
+
+def config3(num_layers: int = 32, batch: int = 32, prompt_len: int = 512, gen_len: int = 128, shape: str = "llama2_7b") -> Workload:
+    """Llama-2-7B-shape decode: rank-16 adapters on q/k/v/o, 16 adapters round-robin over 32 requests
+    (shape="llama31_8b": the same workload on the reference's default model shape)."""
+    if shape == "llama31_8b":
+        sh, name = llama31_8b_shape(num_layers), "c3_llama31_8b_decode"
+    else:
+        sh, name = LlamaShape(num_hidden_layers=num_layers), "c3_llama7b_decode"
     lora = LoraSpec(r=16, alpha=8.0, n_adapters=16, targets=("q_proj", "k_proj", "v_proj", "o_proj"))
-    return Workload("c3_llama7b_decode", 2, shape, lora, batch=batch, prompt_len=prompt_len, gen_len=gen_len,
+    return Workload(name, 2, sh, lora, batch=batch, prompt_len=prompt_len, gen_len=gen_len,
                     adapter_ids=(np.arange(batch) % 16).astype(np.int32))
 
 
