@@ -1,102 +1,114 @@
-"""Per-sequence adapter bookkeeping and decode-method selection (integer host logic).
+"""What the front end knows about each request: its adapter (type and weight id) and its generation limit; and,
+from that, the order of a decode batch and the entry point that serves it.  Integer host logic only.
 
-Restates `tvm/llama_auto_batcher/llama_seq_info.py:1-104`: adapter *types* are distinct `LoraConfig`s in
-first-seen order; `order_seqs` is a stable sort by (has adapter, type id, weight id) so that sequences
-without adapter come first; `get_decode_method` names the compiled entry point and builds the per-type
-position / weight-id lists.
+Behaviour of `tvm/llama_auto_batcher/llama_seq_info.py:1-104`:
+  * an adapter *type* is a distinct `LoraConfig` (rank, alpha); types are numbered in the order they are first seen;
+  * a decode batch is ordered by (has an adapter, type, weight id), stably, so adapter-less requests come first and
+    the rows of one type are contiguous;
+  * the entry point is `decode_no_adapter`, `decode_a{t}` (one type, every row adapted: parameter = weight ids) or
+    `mixed_decode_a{i}_a{j}...` (parameters per present type: row positions inside the batch, weight ids).
 """
 from __future__ import annotations
 
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+
+@dataclass
+class _Request:
+    max_gen_len: int
+    tid: Optional[int] = None     # adapter type, None = no adapter
+    wid: Optional[int] = None     # weight id inside the type
+
 
 class LlamaSeqInfo:
-    def __init__(self, max_gen_len):
-        self.sid_2_info = {}      # sid -> {"adapter": {"tid", "wid"} | None, "max_gen_len": int}
-        self.adapter_types = []
+    def __init__(self, max_gen_len: int):
+        self.max_gen_len = max_gen_len
+        self._requests: Dict[int, _Request] = {}
+        self._types: list = []                    # LoraConfig of type t at index t
+
+    # ------------------------------------------------------------------ registration
+    def add_sequence(self, sid: int) -> None:
+        assert sid not in self._requests, f"sequence with id {sid} has already been added"
+        self._requests[sid] = _Request(self.max_gen_len)
+
+    def update_max_gen_len(self, max_gen_len: int) -> None:
         self.max_gen_len = max_gen_len
 
-    def add_sequence(self, sid):
-        assert sid not in self.sid_2_info, f"sequence with id {sid} has already been added"
-        self.sid_2_info[sid] = {"adapter": None, "max_gen_len": self.max_gen_len}
+    def set_max_gen_len(self, sid: int, max_gen_len: Optional[int]) -> None:
+        """Per-request limit, clipped to the global one (None = the global one)."""
+        limit = self.max_gen_len if max_gen_len is None else max_gen_len
+        if limit > self.max_gen_len:
+            print(f"[WARN] max_gen_len {limit} requested for sequence {sid} exceeds the maximum {self.max_gen_len}; "
+                  f"using {self.max_gen_len}.")
+            limit = self.max_gen_len
+        self._requests[sid].max_gen_len = limit
 
-    def set_max_gen_len(self, sid, max_gen_len):
-        if max_gen_len is None:
-            max_gen_len = self.max_gen_len
-        if max_gen_len > self.max_gen_len:
-            print(f"[WARN] you are trying to set a max_gen_len of {max_gen_len} for sequence {sid} which is bigger "
-                  f"than the maximum {self.max_gen_len}. Setting max_gen_len to {self.max_gen_len}.")
-            max_gen_len = self.max_gen_len
-        self.sid_2_info[sid]["max_gen_len"] = max_gen_len
+    def set_adapter(self, sid: int, config, wid: int) -> None:
+        try:
+            tid = self._types.index(config)
+        except ValueError:
+            tid = len(self._types)
+            self._types.append(config)
+        req = self._requests[sid]
+        if req.tid is not None:
+            print(f"[WARN] sequence {sid} already has adapter {self.get_adapter_info(sid)}; replacing it with "
+                  f"{{'tid': {tid}, 'wid': {int(wid)}}}")
+        req.tid, req.wid = tid, int(wid)
 
-    def set_adapter(self, sid, config, wid):
-        if config in self.adapter_types:
-            tid = self.adapter_types.index(config)
-        else:
-            tid = len(self.adapter_types)
-            self.adapter_types.append(config)
-        adapter = {"tid": tid, "wid": int(wid)}
-        prev = self.sid_2_info[sid]["adapter"]
-        if prev is not None:
-            print(f"[WARN] you are setting adapter {adapter} for sequence {sid} but it has already been set to {prev}")
-        self.sid_2_info[sid]["adapter"] = adapter
+    # ------------------------------------------------------------------ queries
+    def get_num_sequences(self) -> int:
+        return len(self._requests)
 
-    def get_adapter_configs(self):
-        return self.adapter_types
+    def get_max_gen_len(self, sid: int) -> int:
+        return self._requests[sid].max_gen_len
 
-    def get_wids_per_type(self):
-        out = [set() for _ in self.adapter_types]
-        for info in self.sid_2_info.values():
-            if info["adapter"] is not None:
-                out[info["adapter"]["tid"]].add(info["adapter"]["wid"])
-        return out
+    def get_adapter_info(self, sid: int) -> Optional[dict]:
+        req = self._requests[sid]
+        return None if req.tid is None else {"tid": req.tid, "wid": req.wid}
 
-    def get_num_adapters_per_type(self):
-        return [len(s) for s in self.get_wids_per_type()]
+    def get_adapter_configs(self) -> list:
+        return self._types
 
-    def get_num_sequences(self):
-        return len(self.sid_2_info)
+    def get_wids_per_type(self) -> List[set]:
+        """The weight ids in use, per adapter type."""
+        used: List[set] = [set() for _ in self._types]
+        for req in self._requests.values():
+            if req.tid is not None:
+                used[req.tid].add(req.wid)
+        return used
 
-    def update_max_gen_len(self, max_gen_len):
-        self.max_gen_len = max_gen_len
+    def get_num_adapters_per_type(self) -> List[int]:
+        return [len(w) for w in self.get_wids_per_type()]
 
-    def get_max_gen_len(self, sid):
-        return self.sid_2_info[sid]["max_gen_len"]
+    # ------------------------------------------------------------------ batch order and entry point
+    def order_seqs(self, sids: Sequence[int]) -> Tuple[List[int], List[int]]:
+        """-> (the sequence ids in batch order, for each of them its position in `sids`)."""
+        positions = list(range(len(sids)))
+        if self._types:
+            def rank(pos: int):
+                req = self._requests[sids[pos]]
+                return (0, 0, 0) if req.tid is None else (1, req.tid, req.wid)
+            positions.sort(key=rank)                  # list.sort is stable: ties keep the caller's order
+        return [sids[p] for p in positions], positions
 
-    def get_adapter_info(self, sid):
-        return self.sid_2_info[sid]["adapter"]
-
-    def order_seqs(self, sids):
-        """-> (ordered sids, original position of each ordered sid)."""
-        if not self.adapter_types:
-            return list(sids), list(range(len(sids)))
-        inf = float("inf")
-
-        def key(item):
-            ad = self.sid_2_info[item[1]]["adapter"]
-            return (ad is not None, ad["tid"] if ad else inf, ad["wid"] if ad else inf)
-
-        ordered = sorted(enumerate(sids), key=key)      # sorted() is stable
-        return [sid for _, sid in ordered], [pos for pos, _ in ordered]
-
-    def get_decode_method(self, sids):
-        """-> (entry-point name, parameter lists).  `decode_a{t}` takes [wids]; `mixed_decode_a{i}_a{j}...`
-        takes [sids_i, wids_i, sids_j, wids_j, ...] where sids are positions inside this batch."""
-        no_adapter = False
-        a_sids = [[] for _ in self.adapter_types]
-        a_wids = [[] for _ in self.adapter_types]
-        for i, sid in enumerate(sids):
-            ad = self.sid_2_info[sid]["adapter"]
-            if ad is None:
-                no_adapter = True
-                continue
-            a_sids[ad["tid"]].append(i)
-            a_wids[ad["tid"]].append(ad["wid"])
-        present = [t for t, lst in enumerate(a_sids) if lst]
-        if no_adapter and not present:
+    def get_decode_method(self, sids: Sequence[int]) -> Tuple[str, list]:
+        """-> (entry-point name, parameter lists) for a batch whose rows are `sids` in this order."""
+        rows_of: Dict[int, List[int]] = {}            # type -> rows of the batch that use it
+        bare = 0
+        for row, sid in enumerate(sids):
+            tid = self._requests[sid].tid
+            if tid is None:
+                bare += 1
+            else:
+                rows_of.setdefault(tid, []).append(row)
+        present = sorted(rows_of)
+        wids = {t: [self._requests[sids[row]].wid for row in rows_of[t]] for t in present}
+        if not present:
             return "decode_no_adapter", []
-        if not no_adapter and len(present) == 1:
-            return f"decode_a{present[0]}", [a_wids[present[0]]]
-        name = "mixed_decode_" + "_".join(f"a{t}" for t in present)
-        params = []
+        if len(present) == 1 and bare == 0:
+            return f"decode_a{present[0]}", [wids[present[0]]]
+        params: list = []
         for t in present:
-            params += [a_sids[t], a_wids[t]]
-        return name, params
+            params.extend((rows_of[t], wids[t]))
+        return "mixed_decode_" + "_".join(f"a{t}" for t in present), params
