@@ -491,7 +491,7 @@ extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p
   }();
   const int pairs = I / 16;
   const int per = n_cu > 0 ? ceil_div(pairs, n_cu) : 0;
-  if (T <= 32 && n_cu > 0 && pairs >= 2 * n_cu && per <= 4) {
+  if ((T <= 32 || per <= 3) && n_cu > 0 && pairs >= 2 * n_cu && per <= 4) {
     const int base = pairs / n_cu, rem = pairs % n_cu;
     const dim3 g(n_cu);
 #define MLORA_SILU_CU(NP, TT, PIPE) \
@@ -500,10 +500,13 @@ extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p
       if (per <= 2) MLORA_SILU_CU(2, 1, 4);
       else if (per == 3) MLORA_SILU_CU(3, 1, 4);
       else MLORA_SILU_CU(4, 1, 3);
-    } else {
+    } else if (T <= 32) {
       if (per <= 2) MLORA_SILU_CU(2, 2, 4);
       else if (per == 3) MLORA_SILU_CU(3, 2, 3);
       else MLORA_SILU_CU(4, 2, 2);
+    } else {                                   // 33..64 tokens: four token tiles, at most three pairs fit the registers
+      if (per <= 2) MLORA_SILU_CU(2, 4, 2);
+      else MLORA_SILU_CU(3, 4, 2);
     }
 #undef MLORA_SILU_CU
     return mlora_launch_status("gemv_frag_silu");
