@@ -25,11 +25,13 @@ enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2, OUT_SILU_FRAG = 3 };
 // With SHRINK the first `shrink_blocks` workgroups of the launch do LoRA shrink units (one per wave) on the same
 // x instead of a GEMV tile: the adapter work rides in the GEMV launch and finishes long before it does.
 template <int NT, int TT, int OUT, bool PACKED, bool XFRAG, bool SHRINK, int PIPE = 4>   // PIPE: k-steps in flight per wave
-__global__ __launch_bounds__(GEMV_WAVES* WAVE, 4) void gemv_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx,
+__global__ __launch_bounds__(GEMV_WAVES* WAVE, (NT * TT > 8 ? 2 : 4)) void gemv_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx,
                                                                 const f16* __restrict__ W, int T, int K, int N,
                                                                 LoraShrinkBatch sb, int shrink_blocks, int n_main,
                                                                 float* __restrict__ y2, int ksplit, float* __restrict__ part) {
-  __shared__ f32x4 red[GEMV_WAVES][NT * TT][WAVE];
+  constexpr int TILES = NT * TT;
+  constexpr int HT = TILES > 8 ? TILES / 2 : TILES;   // accumulator tiles summed per pass through LDS (64 KiB holds 8)
+  __shared__ f32x4 red[GEMV_WAVES][HT][WAVE];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps the k-loop control scalar
   const int lane = threadIdx.x & 63;
   int bid = blockIdx.x;
@@ -118,28 +120,15 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, 4) void gemv_kernel(void* __restr
     }
   }
 
-#pragma unroll
-  for (int i = 0; i < NT; ++i)
-#pragma unroll
-    for (int j = 0; j < TT; ++j) red[wave][i * TT + j][lane] = acc[i][j];
-  __syncthreads();
-
-  if (slice > 0) {
-    for (int e = threadIdx.x; e < NT * TT * WAVE; e += GEMV_WAVES * WAVE) {
-      const int tile = e >> 6, sl = e & 63;
-      f32x4 s = red[0][tile][sl];
-#pragma unroll
-      for (int w = 1; w < GEMV_WAVES; ++w) s += red[w][tile][sl];
-      const int n = n0 + (tile / TT) * 16 + (sl >> 4) * 4;
-      const int t = (tile % TT) * 16 + (sl & 15);
-      if (t < T && n < N) *reinterpret_cast<f32x4*>(part + ((size_t)(slice - 1) * T + t) * N + n) = s;
-    }
-    return;
-  }
   if constexpr (OUT == OUT_SILU_FRAG) {
     // The weight interleaves 16-row tiles of gate and up, so this block's two tiles are gate rows c..c+15 and up
     // rows c..c+15 of the same channels: out[t, c + ..] = silu(f16(gate)) * f16(up), written in fragment order.
-    static_assert(NT % 2 == 0 || OUT != OUT_SILU_FRAG, "the SiLU epilogue pairs a gate tile with an up tile");
+    static_assert(NT % 2 == 0 && TILES <= 8, "the SiLU epilogue pairs a gate tile with an up tile and sums all tiles in one pass");
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+#pragma unroll
+      for (int j = 0; j < TT; ++j) red[wave][i * TT + j][lane] = acc[i][j];
+    __syncthreads();
     for (int e = threadIdx.x; e < (NT / 2) * TT * WAVE; e += GEMV_WAVES * WAVE) {
       const int pj = e >> 6, sl = e & 63;
       const int p = pj / TT, j = pj % TT;         // tile pair (gate tile 2p, up tile 2p + 1), token tile j
@@ -163,27 +152,42 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, 4) void gemv_kernel(void* __restr
     }
     return;
   }
-  // thread e < NT*TT*64 sums tile (e / 64), lane slot (e % 64) over the 8 waves in order
-  for (int e = threadIdx.x; e < NT * TT * WAVE; e += GEMV_WAVES * WAVE) {
-    const int tile = e >> 6, sl = e & 63;
-    f32x4 s = red[0][tile][sl];
+  // The waves' partial tiles are summed through LDS, in wave order, HT tiles per pass: thread e sums tile h0 + e / 64,
+  // lane slot e % 64.
+  for (int h0 = 0; h0 < TILES; h0 += HT) {
+    if (h0 > 0) __syncthreads();
 #pragma unroll
-    for (int w = 1; w < GEMV_WAVES; ++w) s += red[w][tile][sl];
-    const int i = tile / TT, j = tile % TT;
-    const int n = n0 + i * 16 + (sl >> 4) * 4;   // D[n][t]: lane holds rows 4*(lane/16)..+3, column lane%16
-    const int t = j * 16 + (sl & 15);
-    if (t < T && n >= n_main && n < N) {
-      // rows past n_main are a second result block (adapter shrink rows appended to the weight): fp32, own buffer
-      *reinterpret_cast<f32x4*>(y2 + (size_t)t * (N - n_main) + (n - n_main)) = s;
-    } else if (t < T && n < N) {                  // N % 4 == 0: the 4 rows are inside together
-      const size_t o = (size_t)t * n_main + n;
-      if constexpr (OUT == OUT_F16) {
-        *reinterpret_cast<f16x4*>((f16*)yv + o) = f16x4{(f16)s[0], (f16)s[1], (f16)s[2], (f16)s[3]};
-      } else if constexpr (OUT == OUT_F32) {
-        *reinterpret_cast<f32x4*>((float*)yv + o) = s;
-      } else if constexpr (OUT == OUT_ACC_F32) {
-        f32x4* p = reinterpret_cast<f32x4*>((float*)yv + o);
-        *p = *p + s;
+    for (int i = 0; i < NT; ++i)
+#pragma unroll
+      for (int j = 0; j < TT; ++j) {
+        const int tile = i * TT + j;               // compile-time
+        if (tile >= h0 && tile < h0 + HT) red[wave][tile - h0][lane] = acc[i][j];
+      }
+    __syncthreads();
+    for (int e = threadIdx.x; e < HT * WAVE; e += GEMV_WAVES * WAVE) {
+      const int lt = e >> 6, sl = e & 63;
+      f32x4 s = red[0][lt][sl];
+#pragma unroll
+      for (int w = 1; w < GEMV_WAVES; ++w) s += red[w][lt][sl];
+      const int tile = h0 + lt;
+      const int i = tile / TT, j = tile % TT;
+      const int n = n0 + i * 16 + (sl >> 4) * 4;   // D[n][t]: lane holds rows 4*(lane/16)..+3, column lane%16
+      const int t = j * 16 + (sl & 15);
+      if (slice > 0) {                             // a K slice other than the first: fp32 partial, summed by the reader of y
+        if (t < T && n < N) *reinterpret_cast<f32x4*>(part + ((size_t)(slice - 1) * T + t) * N + n) = s;
+      } else if (t < T && n >= n_main && n < N) {
+        // rows past n_main are a second result block (adapter shrink rows appended to the weight): fp32, own buffer
+        *reinterpret_cast<f32x4*>(y2 + (size_t)t * (N - n_main) + (n - n_main)) = s;
+      } else if (t < T && n < N) {                 // N % 4 == 0: the 4 rows are inside together
+        const size_t o = (size_t)t * n_main + n;
+        if constexpr (OUT == OUT_F16) {
+          *reinterpret_cast<f16x4*>((f16*)yv + o) = f16x4{(f16)s[0], (f16)s[1], (f16)s[2], (f16)s[3]};
+        } else if constexpr (OUT == OUT_F32) {
+          *reinterpret_cast<f32x4*>((float*)yv + o) = s;
+        } else if constexpr (OUT == OUT_ACC_F32) {
+          f32x4* p = reinterpret_cast<f32x4*>((float*)yv + o);
+          *p = *p + s;
+        }
       }
     }
   }
@@ -351,7 +355,11 @@ int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const 
     // 33..64 tokens: four token tiles leave registers for two row tiles per wave (x traffic is then twice the weight
     // traffic instead of four times): 5.3 -> 4.4 ms of GEMV per decode step at T = 64
     if constexpr (PACKED && XFRAG) {
-      if (ksplit > 1 || tiles > 256) {            // 257..511 tiles as one-tile workgroups would need a second, thin round
+      if (ksplit > 1 || tiles >= 768) {           // one workgroup per unit with four row tiles: the token block is read once per unit
+        launch_gemv<4, 4, PACKED, XFRAG, SHRINK, 2>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part);
+        return mlora_launch_status("gemv");
+      }
+      if (tiles > 256) {                          // 257..511 tiles as one-tile workgroups would need a second, thin round
         launch_gemv<2, 4, PACKED, XFRAG, SHRINK, 2>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part);
         return mlora_launch_status("gemv");
       }
@@ -440,7 +448,7 @@ extern "C" int mlora_gemv_ksplit(int T, int K, int N_total) {
   if (T <= 0 || T > 64 || K <= 0 || K % 32 || N_total <= 0) return 1;
   const int tiles = ceil_div(N_total, 16);
   if (tiles >= 512) return 1;
-  const int groups = ceil_div(tiles, T <= 32 ? 4 : 2);   // row tiles per workgroup of the split kernel (see gemv_dispatch)
+  const int groups = ceil_div(tiles, 4);      // row tiles per workgroup of the split kernel (see gemv_dispatch)
   int ks = 256 / groups;
   const int by_k = (K / KSTEP) / 24;
   if (ks > by_k) ks = by_k;

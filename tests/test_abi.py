@@ -95,8 +95,8 @@ def test_argument_validation_of_fused_and_batched_entry_points():
     assert lib.mlora_gemv_frag_silu(None, 1, 1, 8, 64, 64, None) == -1
     # K-split GEMV: slice counts, partials buffer, argument checks
     assert lib.mlora_gemv_ksplit(32, 11008, 4096) == 4 and lib.mlora_gemv_ksplit(32, 4096, 4352) == 3
-    assert lib.mlora_gemv_ksplit(33, 11008, 4096) == 2 and lib.mlora_gemv_ksplit(32, 4096, 12288) == 1
-    assert lib.mlora_gemv_ksplit(65, 11008, 4096) == 1 and lib.mlora_gemv_ksplit(64, 4096, 4352) == 1
+    assert lib.mlora_gemv_ksplit(33, 11008, 4096) == 4 and lib.mlora_gemv_ksplit(32, 4096, 12288) == 1
+    assert lib.mlora_gemv_ksplit(65, 11008, 4096) == 1 and lib.mlora_gemv_ksplit(64, 4096, 4352) == 3
     assert lib.mlora_gemv_ksplit_bytes(32, 4096, 4) == 3 * 32 * 4096 * 4 and lib.mlora_gemv_ksplit_bytes(32, 4096, 1) == 0
     ksg = lambda ks, part, T=32, n_ext=0, y2=None, A=None: lib.mlora_gemv_frag_acc_ksplit(1, y2, part, ks, 1, 1, T, 4096, 4096, n_ext,
                                                                                          None, A, 1 if A else 0, None, 16, 4, None)
