@@ -682,8 +682,11 @@ __global__ __launch_bounds__(256) void paged_attn_prefill_kernel(f16* __restrict
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) maxpos = max(maxpos, __shfl_xor(maxpos, o, WAVE));
     const int npages = maxpos / PAGE + 1;
+    const int32_t* __restrict__ bt = block_table + (size_t)cur_seq * max_blocks;
+    int page_next = bt[0];                           // the page id is requested one page ahead
     for (int pg = 0; pg < npages; ++pg) {
-      const int page = block_table[(size_t)cur_seq * max_blocks + pg];
+      const int page = page_next;
+      page_next = pg + 1 < npages ? bt[pg + 1] : -1;
       if (page < 0 || page >= n_pages) continue;   // wave-uniform
       const f16* kp = k_cache + ((size_t)page * Hkv + kh) * PAGE * D + lane * 8;       // key qi, dims 8g.. of each k-block
       const f16* vp = v_cache + (((size_t)page * Hkv + kh) * D + qi) * PAGE + g * 4;   // dim qi (+16 db), keys 4g..
