@@ -7,8 +7,7 @@ from __future__ import annotations
 
 import torch
 
-from . import _lib
-from ._lib import F16, F32, ROWMAJOR, FRAG, STORE, ACCUMULATE, PAGE_SIZE, check, lib
+from ._lib import F16, F32, ROWMAJOR, FRAG, STORE, ACCUMULATE, check, lib
 
 
 def _stream() -> int:

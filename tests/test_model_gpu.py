@@ -9,7 +9,6 @@ import pytest
 import torch
 
 import oracle
-from oracle import max_rel_err
 from conftest import load_pkg
 from helpers import (check_tokens_against_oracle, hip_model, n_pages_for, oracle_model, run_hip_generate,
                      teacher_forced_hip)

@@ -3,7 +3,6 @@ dense-library special cases and integer exactness.  The reference holds no golde
 its only checks are `np.allclose` between batching strategies on unseeded data
 (`tvm/lora_only/single_rank.py:254` atol 1e-4, `tvm/lora_only/case_study/multiple_ranks.py:382-383` atol 1e-5)."""
 import numpy as np
-import pytest
 
 import oracle
 from oracle import gather_mm_ref, max_rel_err

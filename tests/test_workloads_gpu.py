@@ -10,7 +10,6 @@ import numpy as np
 import pytest
 import torch
 
-import oracle
 from conftest import load_pkg
 from helpers import NEAR_TIE, hip_model, oracle_model
 
