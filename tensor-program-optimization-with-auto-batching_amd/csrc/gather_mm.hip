@@ -556,14 +556,18 @@ __device__ __forceinline__ bool next_tile_adapter(int id, unsigned& todo, int& a
   return true;
 }
 
-// Expand for segment-ordered tokens (prefill): one pass per distinct adapter of the tile - one, two at a segment boundary.
-// Lean in registers (seven waves per SIMD), which is what this latency-bound kernel lives on.
+// Expand for segment-ordered tokens (prefill): TWO token tiles per workgroup and 256 registers per lane (two workgroups
+// per CU, which is what a prefill-sized launch fills the chip with anyway).  In the common case - both tiles belong to
+// one adapter segment - a B fragment serves 32 tokens, the next column block's fragments are requested a block ahead
+// and the y rows at the top of the block, so a block costs one memory round.  Tiles that hold several adapters, or
+// different ones, are worked off one tile and one adapter at a time (one pass per distinct adapter of the tile, rows of
+// other adapters masked at the store).
 template <int R, typename YT>
-__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(SegProjs pj, const float* __restrict__ v,
-                                                                            const int32_t* __restrict__ ids, float scaling,
-                                                                            int T, int ldy, int n_ad,
-                                                                            const int32_t* __restrict__ bucket_of, int bucket,
-                                                                            int splits, int nit) {
+__global__ __launch_bounds__(SEG_WAVES * WAVE, 2) void lora_expand_pair_mfma_kernel(SegProjs pj, const float* __restrict__ v,
+                                                                                   const int32_t* __restrict__ ids, float scaling,
+                                                                                   int T, int ldy, int n_ad,
+                                                                                   const int32_t* __restrict__ bucket_of, int bucket,
+                                                                                   int splits, int nit) {
   YT* __restrict__ y = (YT*)pj.y[0];
   const f16* __restrict__ B = pj.B[0];
   int N = pj.N[0];
@@ -578,88 +582,155 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mfma_kernel(SegP
   constexpr int KS = (R + 31) / 32;     // k-steps of 32 rank entries (ranks 8 and 16: one partly filled step)
   constexpr int CT = 4;                 // 16-column tiles per wave
   constexpr int LD = 16 * CT + 4;       // padded row of the transposition buffer (floats): conflict-free both ways
-  __shared__ float stage[SEG_WAVES][16][LD];
+  typedef typename YVec<YT, sizeof(YT) == 2 ? 8 : 4>::type YV;      // 16 bytes of y
+  constexpr int NYV = sizeof(YT) == 2 ? 2 : 4;                       // ... of which a lane's 16 columns take 2 or 4
+  constexpr int EPV = 16 / NYV;
+  __shared__ float stage[2][SEG_WAVES][16][LD];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int t0 = blockIdx.x * 16;
-  // a workgroup covers nit consecutive blocks of 4 waves x 64 columns; the token tile of v stays in registers
   const int nbase = blockIdx.y * nit * SEG_WAVES * 16 * CT + wave * 16 * CT;
   const int col = lane & 15, g = lane >> 4;
-  const int tl = min(t0 + col, T - 1);
-  const int raw = lora_token_id(ids, bucket_of, bucket, t0 + col, T);
-  const int id = (raw >= 0 && raw < n_ad) ? raw : -1;
-  unsigned todo = (unsigned)__ballot(id >= 0) & 0xffffu;
-  if (!todo) return;                    // the same for every wave of the workgroup
-  // the token tile of v as the B operand, hi and lo halves: lane holds v[token col][ks*32 + 8g .. +7]
-  f16x8 vh[KS], vl[KS];
+  const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  int t0[2], id[2];
+  unsigned todo[2];
+  f16x8 vh[2][KS], vl[2][KS];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    const int j = ks * 32 + g * 8;
-    float f[8];
+  for (int u = 0; u < 2; ++u) {
+    t0[u] = (blockIdx.x * 2 + u) * 16;
+    const int raw = lora_token_id(ids, bucket_of, bucket, t0[u] + col, T);
+    id[u] = (raw >= 0 && raw < n_ad) ? raw : -1;
+    todo[u] = (unsigned)__ballot(id[u] >= 0) & 0xffffu;
+    const int tl = min(t0[u] + col, T - 1);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) f[e] = 0.f;
-    // rows of unadapted tokens are never read (their v holds nothing) and enter the product as zeros
-    if (j < R && id >= 0) {
-      f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
-      for (int sp = 0; sp < splits; ++sp) {           // the K-range partials of the shrink, summed in range order
-        lo += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + tl) * R + j);
-        hi += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + tl) * R + j + 4);
+    for (int ks = 0; ks < KS; ++ks) {
+      const int j = ks * 32 + g * 8;
+      float f[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = 0.f;
+      // rows of unadapted tokens are never read (their v holds nothing) and enter the product as zeros
+      if (j < R && id[u] >= 0) {
+        f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
+        for (int sp = 0; sp < splits; ++sp) {           // the K-range partials of the shrink, summed in range order
+          lo += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + tl) * R + j);
+          hi += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + tl) * R + j + 4);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          f[e] = lo[e] * scaling;
+          f[4 + e] = hi[e] * scaling;
+        }
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        f[e] = lo[e] * scaling;
-        f[4 + e] = hi[e] * scaling;
+      for (int e = 0; e < 8; ++e) {
+        const f16 h = (f16)f[e];
+        vh[u][ks][e] = h;
+        vl[u][ks][e] = (f16)(f[e] - (float)h);
       }
-    }
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const f16 h = (f16)f[e];
-      vh[ks][e] = h;
-      vl[ks][e] = (f16)(f[e] - (float)h);
     }
   }
+  if (!(todo[0] | todo[1])) return;     // the same for every wave of the workgroup
   // write-back role of the lane: token lane / 4, the 16 columns of column tile lane % 4 (contiguous in y)
   const int wt = lane >> 2, wc = lane & 3;
-  int a;
-  unsigned rows;
-  while (next_tile_adapter(id, todo, a, rows)) {
-    const f16* __restrict__ Ba = B + (size_t)a * N * R + g * 8;
-   for (int it = 0; it < nit; ++it) {
+  // the B fragments of column block `it` of adapter a
+  auto load_b = [&](f16x8 (&bf)[CT][KS], const f16* __restrict__ Ba, int it) {
     const int n0 = nbase + it * SEG_WAVES * 16 * CT;
-    const int nw = n0 + wc * 16;
-    YT* __restrict__ yrow = y + (size_t)(t0 + wt) * ldy + nw;
+#pragma unroll
+    for (int c = 0; c < CT; ++c)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int nb = n0 + c * 16;
+        bf[c][ks] = (nb < N && ks * 32 + g * 8 < R) ? ld8(Ba + (size_t)(nb + col) * R + ks * 32) : zero8;
+      }
+  };
+  // products of tile u with the fragments bf, into the tile's transposition buffer
+  auto products = [&](int u, const f16x8 (&bf)[CT][KS], int it) {
+    const int n0 = nbase + it * SEG_WAVES * 16 * CT;
 #pragma unroll
     for (int c = 0; c < CT; ++c) {
-      const int nb = n0 + c * 16;
-      if (nb < N) {                                                // wave-uniform
+      if (n0 + c * 16 < N) {                                          // wave-uniform
         f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          const int j = ks * 32 + g * 8;
-          const f16x8 bf = j < R ? ld8(Ba + (size_t)(nb + col) * R + ks * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf, vh[ks], acc, 0, 0, 0);    // rows: output column, cols: tokens
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf, vl[ks], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf[c][ks], vh[u][ks], acc, 0, 0, 0);    // rows: output column, cols: tokens
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf[c][ks], vl[u][ks], acc, 0, 0, 0);
         }
-        *reinterpret_cast<f32x4*>(&stage[wave][col][c * 16 + 4 * g]) = acc;           // D[n = 4g.., token col]
+        *reinterpret_cast<f32x4*>(&stage[u][wave][col][c * 16 + 4 * g]) = acc;           // D[n = 4g.., token col]
       }
     }
-    __syncthreads();
-    if (nw < N && ((rows >> wt) & 1u)) {
-      float d[16];
+  };
+  // y rows of tile u (already loaded into yv) plus the tile's products, stored
+  auto add_store = [&](int u, YV (&yv)[NYV], YT* __restrict__ yrow) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const f32x4 s4 = *reinterpret_cast<const f32x4*>(&stage[wave][wt][wc * 16 + 4 * q]);
-        d[4 * q] = s4[0]; d[4 * q + 1] = s4[1]; d[4 * q + 2] = s4[2]; d[4 * q + 3] = s4[3];
+    for (int q = 0; q < NYV; ++q) {
+#pragma unroll
+      for (int e4 = 0; e4 < EPV / 4; ++e4) {
+        const f32x4 s4 = *reinterpret_cast<const f32x4*>(&stage[u][wave][wt][wc * 16 + q * EPV + 4 * e4]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) yv[q][4 * e4 + e] = (YT)((float)yv[q][4 * e4 + e] + s4[e]);
       }
-      if constexpr (sizeof(YT) == 2) {
-        rmw_add<YT, 8>(yrow, d);
-        rmw_add<YT, 8>(yrow + 8, d + 8);
-      } else {
+      *reinterpret_cast<YV*>(yrow + q * EPV) = yv[q];
+    }
+  };
+  // one adapter for every adapted row of both tiles?
+  const int a_first = todo[0] ? __shfl(id[0], __builtin_ctz(todo[0] | 0x10000u) & 15, WAVE) : __shfl(id[1], __builtin_ctz(todo[1] | 0x10000u) & 15, WAVE);
+  const bool same = (((unsigned)__ballot(id[0] == a_first) & 0xffffu) == todo[0]) && (((unsigned)__ballot(id[1] == a_first) & 0xffffu) == todo[1]);
+  if (same) {
+    const f16* __restrict__ Ba = B + (size_t)a_first * N * R + g * 8;
+    auto block = [&](int it, f16x8 (&cur)[CT][KS], f16x8 (&nxt)[CT][KS]) {
+      const int nw = nbase + it * SEG_WAVES * 16 * CT + wc * 16;
+      YV yv[2][NYV];
+      bool wr[2];
+      YT* yrow[2];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) rmw_add<YT, 4>(yrow + 4 * q, d + 4 * q);
+      for (int u = 0; u < 2; ++u) {
+        yrow[u] = y + (size_t)(t0[u] + wt) * ldy + nw;
+        wr[u] = nw < N && ((todo[u] >> wt) & 1u);
+        if (wr[u]) {
+#pragma unroll
+          for (int q = 0; q < NYV; ++q) yv[u][q] = *reinterpret_cast<const YV*>(yrow[u] + q * EPV);
+        }
+      }
+      if (it + 1 < nit) load_b(nxt, Ba, it + 1);
+      if (todo[0]) products(0, cur, it);
+      if (todo[1]) products(1, cur, it);
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+        if (wr[u]) add_store(u, yv[u], yrow[u]);
+      __syncthreads();
+    };
+    f16x8 b0[CT][KS], b1[CT][KS];
+    load_b(b0, Ba, 0);
+    for (int it = 0; it < nit; it += 2) {
+      block(it, b0, b1);
+      if (it + 1 < nit) block(it + 1, b1, b0);
+    }
+    return;
+  }
+  // general case: tile by tile, adapter by adapter
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    int a;
+    unsigned rows;
+    unsigned left = todo[u];
+    while (next_tile_adapter(id[u], left, a, rows)) {
+      const f16* __restrict__ Ba = B + (size_t)a * N * R + g * 8;
+      for (int it = 0; it < nit; ++it) {
+        const int nw = nbase + it * SEG_WAVES * 16 * CT + wc * 16;
+        YT* __restrict__ yrow = y + (size_t)(t0[u] + wt) * ldy + nw;
+        const bool wr = nw < N && ((rows >> wt) & 1u);
+        f16x8 bf[CT][KS];
+        load_b(bf, Ba, it);
+        YV yv[NYV];
+        if (wr) {
+#pragma unroll
+          for (int q = 0; q < NYV; ++q) yv[q] = *reinterpret_cast<const YV*>(yrow + q * EPV);
+        }
+        products(u, bf, it);
+        __syncthreads();
+        if (wr) add_store(u, yv, yrow);
+        __syncthreads();
       }
     }
-    __syncthreads();
-   }
   }
 }
 
@@ -1008,19 +1079,25 @@ static void gmm_segments_r(const SegProjs& pj, int y_dtype, int ldy, const f16* 
   // column blocks per workgroup: as many as leave about a thousand workgroups (per-workgroup set-up amortised)
   int nit = (int)(((long)tiles * pj.n * ceil_div(N, SEG_WAVES * 64)) / 1024);
   nit = nit < 1 ? 1 : (nit > 8 ? 8 : nit);
-  const dim3 grid(tiles, ceil_div(N, SEG_WAVES * 64 * nit), pj.n);
   // Up to 1024 tokens the call is taken to be a decode batch (one token per sequence, tiles that mix many adapters);
-  // beyond that a prefill whose tokens come in adapter segments.  Either kernel is correct for either input.
+  // beyond that a prefill whose tokens come in adapter segments, two token tiles per workgroup and about two
+  // workgroups per compute unit.  Either kernel is correct for either input.
   const bool mixed = T <= 1024;
+  if (!mixed) {
+    const int pairs = ceil_div(tiles, 2);
+    nit = (int)(((long)pairs * pj.n * ceil_div(N, SEG_WAVES * 64)) / 512);
+    nit = nit < 1 ? 1 : (nit > 8 ? 8 : nit);
+  }
+  const dim3 grid(mixed ? tiles : ceil_div(tiles, 2), ceil_div(N, SEG_WAVES * 64 * nit), pj.n);
 #define MLORA_EXPAND_MFMA(KERNEL, YT)                                                                                       \
   hipLaunchKernelGGL((KERNEL<R, YT>), grid, dim3(SEG_WAVES * WAVE), 0, s, pj, v, ids, scaling, T, ldy, n_ad, \
                      bf.bucket_of, bf.bucket, splits, nit)
   if (y_dtype == MLORA_F16) {
     if (mixed) MLORA_EXPAND_MFMA(lora_expand_mixed_mfma_kernel, f16);
-    else MLORA_EXPAND_MFMA(lora_expand_mfma_kernel, f16);
+    else MLORA_EXPAND_MFMA(lora_expand_pair_mfma_kernel, f16);
   } else {
     if (mixed) MLORA_EXPAND_MFMA(lora_expand_mixed_mfma_kernel, float);
-    else MLORA_EXPAND_MFMA(lora_expand_mfma_kernel, float);
+    else MLORA_EXPAND_MFMA(lora_expand_pair_mfma_kernel, float);
   }
 #undef MLORA_EXPAND_MFMA
 }
