@@ -465,32 +465,22 @@ __device__ __forceinline__ TileAdapters tile_adapters(int id) {
 // Shrink.  The adapters of the tile are worked GA at a time inside ONE pass over K: per 32-k step the token fragment is
 // loaded once and every adapter of the group contributes one A fragment and one MFMA - a decode batch, where a tile of
 // 16 tokens holds up to 16 adapters, costs one K loop instead of 16, with all the groups' loads in flight together.
+// Shrink of one 16-token tile by the four waves of a workgroup: K steps kb0 .. kb1-1 dealt to the waves in turn, the
+// waves' sums added in wave order through `red`, partial result rows written to v [T][R].
 template <int R>
-__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(float* __restrict__ v, const f16* __restrict__ x,
-                                                                            SegProjs pj,
-                                                                            const int32_t* __restrict__ ids, int T, int K,
-                                                                            int n_ad, const int32_t* __restrict__ bucket_of,
-                                                                            int bucket) {
-  const f16* __restrict__ A = pj.A[0];
-#pragma unroll
-  for (int i = 1; i < SEG_MAX_PROJ; ++i)
-    if (i == blockIdx.z) A = pj.A[i];                    // uniform select: the struct is never indexed dynamically
-  // blockIdx.y selects one of gridDim.y contiguous ranges of 32-k steps; its partial sums go to v[blockIdx.y][T][R]
+__device__ __forceinline__ void shrink_tile_mfma(float* __restrict__ v, const f16* __restrict__ x, const f16* __restrict__ A,
+                                                 const int32_t* __restrict__ ids, int T, int K, int n_ad,
+                                                 const int32_t* __restrict__ bucket_of, int bucket, int t0, int kb0, int kb1,
+                                                 f32x4 (*red)[8][WAVE]) {
   constexpr int NT = (R + 15) / 16;     // 16-row tiles of A[a]; rank 8 uses half a tile
   constexpr int GA = 8 / NT;            // adapters per pass: 32 accumulator registers
-  __shared__ f32x4 red[SEG_WAVES][GA * NT][WAVE];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int t0 = blockIdx.x * 16;
   const int col = lane & 15, g = lane >> 4;
   const int tl = min(t0 + col, T - 1);                          // token whose x row this lane supplies
   const int raw = lora_token_id(ids, bucket_of, bucket, t0 + col, T);
   const int id = (raw >= 0 && raw < n_ad) ? raw : -1;
   const TileAdapters ta = tile_adapters(id);
   const f16* __restrict__ xr = x + (size_t)tl * K + g * 8;
-  const int KB = K / 32;
-  const int per = (KB + gridDim.y - 1) / gridDim.y;
-  const int kb0 = blockIdx.y * per, kb1 = min(KB, kb0 + per);
-  v += ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * T * R;
 #pragma unroll
   for (int g0 = 0; g0 < 16; g0 += GA) {
     if (g0 < ta.n) {                                             // uniform
@@ -543,6 +533,104 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(floa
       }
       __syncthreads();
     }
+  }
+}
+
+template <int R>
+__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(float* __restrict__ v, const f16* __restrict__ x,
+                                                                            SegProjs pj,
+                                                                            const int32_t* __restrict__ ids, int T, int K,
+                                                                            int n_ad, const int32_t* __restrict__ bucket_of,
+                                                                            int bucket) {
+  // blockIdx.y selects one of gridDim.y contiguous ranges of 32-k steps; its partial sums go to v[blockIdx.y][T][R]
+  __shared__ f32x4 red[SEG_WAVES][8][WAVE];
+  const f16* __restrict__ A = pj.A[0];
+#pragma unroll
+  for (int i = 1; i < SEG_MAX_PROJ; ++i)
+    if (i == blockIdx.z) A = pj.A[i];                    // uniform select: the struct is never indexed dynamically
+  const int KB = K / 32;
+  const int per = (KB + gridDim.y - 1) / gridDim.y;
+  const int kb0 = blockIdx.y * per, kb1 = min(KB, kb0 + per);
+  v += ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * T * R;
+  shrink_tile_mfma<R>(v, x, A, ids, T, K, n_ad, bucket_of, bucket, blockIdx.x * 16, kb0, kb1, red);
+}
+
+// Prefill-sized shrink: FOUR token tiles per workgroup.  When all adapted tokens of the four tiles use one adapter (an
+// adapter segment of 64 tokens or more), an A fragment is loaded once per 64 tokens instead of once per 16; otherwise
+// the tiles are worked off one after the other as above.  Same sums, in the same order, either way.
+template <int R>
+__global__ __launch_bounds__(SEG_WAVES * WAVE, 2) void lora_shrink_quad_mfma_kernel(float* __restrict__ v, const f16* __restrict__ x,
+                                                                                   SegProjs pj,
+                                                                                   const int32_t* __restrict__ ids, int T, int K,
+                                                                                   int n_ad, const int32_t* __restrict__ bucket_of,
+                                                                                   int bucket) {
+  constexpr int NT = (R + 15) / 16;
+  constexpr int QT = 4;
+  __shared__ f32x4 red[SEG_WAVES][8][WAVE];
+  const f16* __restrict__ A = pj.A[0];
+#pragma unroll
+  for (int i = 1; i < SEG_MAX_PROJ; ++i)
+    if (i == blockIdx.z) A = pj.A[i];                    // uniform select: the struct is never indexed dynamically
+  const int KB = K / 32;
+  const int per = (KB + gridDim.y - 1) / gridDim.y;
+  const int kb0 = blockIdx.y * per, kb1 = min(KB, kb0 + per);
+  v += ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * T * R;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int col = lane & 15, g = lane >> 4;
+  const int tq = blockIdx.x * 16 * QT;
+  // lane l looks at token tq + l: do all adapted tokens of the four tiles name the same adapter?
+  const int raw = lora_token_id(ids, bucket_of, bucket, tq + lane, T);
+  const int idl = (raw >= 0 && raw < n_ad) ? raw : -1;
+  const unsigned long long have = __ballot(idl >= 0);
+  if (!have) return;                                     // the same for every wave
+  const int a = __shfl(idl, __builtin_ctzll(have), WAVE);
+  const bool same = __ballot(idl == a) == have;
+  if (!same) {
+    for (int u = 0; u < QT; ++u)
+      if (tq + u * 16 < T) shrink_tile_mfma<R>(v, x, A, ids, T, K, n_ad, bucket_of, bucket, tq + u * 16, kb0, kb1, red);
+    return;
+  }
+  const f16* __restrict__ Aa = A + (size_t)a * R * K + g * 8;
+  const f16* xr[QT];
+#pragma unroll
+  for (int u = 0; u < QT; ++u) xr[u] = x + (size_t)min(tq + u * 16 + col, T - 1) * K + g * 8;
+  f32x4 acc[QT][NT];
+#pragma unroll
+  for (int u = 0; u < QT; ++u)
+#pragma unroll
+    for (int i = 0; i < NT; ++i) acc[u][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int kb = kb0 + wave; kb < kb1; kb += SEG_WAVES) {
+    f16x8 af[NT], xf[QT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      const int row = i * 16 + col;
+      af[i] = row < R ? ld8(Aa + (size_t)row * K + kb * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int u = 0; u < QT; ++u) xf[u] = ld8(xr[u] + kb * 32);
+#pragma unroll
+    for (int u = 0; u < QT; ++u)
+#pragma unroll
+      for (int i = 0; i < NT; ++i) acc[u][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], xf[u], acc[u][i], 0, 0, 0);
+  }
+  // the four waves' sums, tile by tile, added in wave order; wave w stores A-tile i = w, w + 4, ... of the token tile
+#pragma unroll
+  for (int u = 0; u < QT; ++u) {
+#pragma unroll
+    for (int i = 0; i < NT; ++i) red[wave][i][lane] = acc[u][i];
+    __syncthreads();
+    const unsigned rows = (unsigned)(have >> (16 * u)) & 0xffffu;
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      if ((i % SEG_WAVES) == wave) {
+        f32x4 sum = red[0][i][lane];
+#pragma unroll
+        for (int w = 1; w < SEG_WAVES; ++w) sum += red[w][i][lane];
+        const int j = i * 16 + 4 * g;
+        if (((rows >> col) & 1u) && j < R) *reinterpret_cast<f32x4*>(v + (size_t)(tq + u * 16 + col) * R + j) = sum;
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -1074,15 +1162,25 @@ static void gmm_segments_r(const SegProjs& pj, int y_dtype, int ldy, const f16* 
   if (splits > kc) splits = kc;
   if (splits > K / 128) splits = K / 128;
   if (splits < 1) splits = 1;
-  hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles, splits, pj.n), dim3(SEG_WAVES * WAVE), 0, s, v, x, pj, ids, T, K, n_ad,
-                     bf.bucket_of, bf.bucket);
+  // Up to 1024 tokens the call is taken to be a decode batch (one token per sequence, tiles that mix many adapters);
+  // beyond that a prefill whose tokens come in adapter segments: four token tiles per shrink workgroup, two per expand
+  // workgroup, about two workgroups per compute unit.  Either set of kernels is correct for either input.
+  const bool mixed = T <= 1024;
+  if (mixed) {
+    hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles, splits, pj.n), dim3(SEG_WAVES * WAVE), 0, s, v, x, pj, ids, T, K, n_ad,
+                       bf.bucket_of, bf.bucket);
+  } else {
+    const int quads = ceil_div(tiles, 4);
+    splits = 256 / quads;                        // few K ranges: the expand adds the ranges' partial sums per token
+    if (splits > kc) splits = kc;
+    if (splits > K / 128) splits = K / 128;
+    if (splits < 1) splits = 1;
+    hipLaunchKernelGGL((lora_shrink_quad_mfma_kernel<R>), dim3(quads, splits, pj.n), dim3(SEG_WAVES * WAVE), 0, s, v, x, pj, ids, T, K,
+                       n_ad, bf.bucket_of, bf.bucket);
+  }
   // column blocks per workgroup: as many as leave about a thousand workgroups (per-workgroup set-up amortised)
   int nit = (int)(((long)tiles * pj.n * ceil_div(N, SEG_WAVES * 64)) / 1024);
   nit = nit < 1 ? 1 : (nit > 8 ? 8 : nit);
-  // Up to 1024 tokens the call is taken to be a decode batch (one token per sequence, tiles that mix many adapters);
-  // beyond that a prefill whose tokens come in adapter segments, two token tiles per workgroup and about two
-  // workgroups per compute unit.  Either kernel is correct for either input.
-  const bool mixed = T <= 1024;
   if (!mixed) {
     const int pairs = ceil_div(tiles, 2);
     nit = (int)(((long)pairs * pj.n * ceil_div(N, SEG_WAVES * 64)) / 512);
