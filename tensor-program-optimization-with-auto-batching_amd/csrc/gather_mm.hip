@@ -687,24 +687,40 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE, 2) void lora_expand_pair_mfma_ker
     const int raw = lora_token_id(ids, bucket_of, bucket, t0[u] + col, T);
     id[u] = (raw >= 0 && raw < n_ad) ? raw : -1;
     todo[u] = (unsigned)__ballot(id[u] >= 0) & 0xffffu;
-    const int tl = min(t0[u] + col, T - 1);
+  }
+  // v of the two token tiles, once per workgroup: thread e sums four rank entries of one token over the K-range
+  // partials of the shrink (in range order), scales them and leaves them in LDS; rows of unadapted tokens are never
+  // read (their v holds nothing) and enter the products as zeros
+  float* __restrict__ vs = &stage[0][0][0][0];           // [2][16][R] floats, before the buffer serves the transposition
+  static_assert(2 * 16 * R <= 2 * SEG_WAVES * 16 * LD, "v of two token tiles fits the transposition buffer");
+  for (int e = threadIdx.x; e < 2 * 16 * (R / 4); e += SEG_WAVES * WAVE) {
+    const int u = e / (16 * (R / 4)), tok = (e / (R / 4)) % 16, j = (e % (R / 4)) * 4;
+    f32x4 sum = f32x4{0.f, 0.f, 0.f, 0.f};
+    if ((todo[u] >> tok) & 1u) {
+      const int t = t0[u] + tok;
+      for (int sp = 0; sp < splits; ++sp) sum += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + t) * R + j);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) sum[q] *= scaling;
+    }
+    *reinterpret_cast<f32x4*>(vs + ((size_t)u * 16 + tok) * R + j) = sum;
+  }
+  __syncthreads();
+  // the token tiles of v as the B operand, hi and lo halves: lane holds v[token col][ks*32 + 8g .. +7]
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int j = ks * 32 + g * 8;
       float f[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) f[e] = 0.f;
-      // rows of unadapted tokens are never read (their v holds nothing) and enter the product as zeros
-      if (j < R && id[u] >= 0) {
-        f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
-        for (int sp = 0; sp < splits; ++sp) {           // the K-range partials of the shrink, summed in range order
-          lo += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + tl) * R + j);
-          hi += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + tl) * R + j + 4);
-        }
+      if (j < R) {
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(vs + ((size_t)u * 16 + col) * R + j);
+        const f32x4 hi = *reinterpret_cast<const f32x4*>(vs + ((size_t)u * 16 + col) * R + j + 4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          f[e] = lo[e] * scaling;
-          f[4 + e] = hi[e] * scaling;
+          f[e] = lo[e];
+          f[4 + e] = hi[e];
         }
       }
 #pragma unroll
@@ -714,7 +730,7 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE, 2) void lora_expand_pair_mfma_ker
         vl[u][ks][e] = (f16)(f[e] - (float)h);
       }
     }
-  }
+  __syncthreads();                                       // vs is dead: the buffer goes back to the transposition
   if (!(todo[0] | todo[1])) return;     // the same for every wave of the workgroup
   // write-back role of the lane: token lane / 4, the 16 columns of column tile lane % 4 (contiguous in y)
   const int wt = lane >> 2, wc = lane & 3;
