@@ -573,15 +573,15 @@ def test_gather_mm_prefill_column_slice(ops, synth):
     assert np.array_equal(after[:, :N], before[:, :N]) and np.array_equal(after[:, 2 * N:], before[:, 2 * N:])
 
 
-@pytest.mark.parametrize("Hq,Hkv,D", [(4, 4, 128), (8, 2, 64), (16, 1, 128), (6, 3, 64)])
-def test_rope_attn_decode_one_launch_equals_two(ops, synth, Hq, Hkv, D):
+@pytest.mark.parametrize("Hq,Hkv,D,rep", [(4, 4, 128, 1), (8, 2, 64, 1), (16, 1, 128, 1), (6, 3, 64, 1), (8, 8, 128, 6), (16, 16, 64, 9)])
+def test_rope_attn_decode_one_launch_equals_two(ops, synth, Hq, Hkv, D, rep):
     """RoPE + append + decode attention in one launch: output and both caches equal, bit for bit, those of
     rope_kv_append followed by paged_attn_decode.  New tokens at the first and last slot of a page, in a fresh
     sequence (context 1) and deep into a sequence; MHA and grouped heads; an out-of-range sequence row."""
     kvm = load_pkg("kv_cache")
-    pos = [0, 15, 16, 31, 37, 100, 5]
+    pos = [0, 15, 16, 31, 37, 100, 5] * rep          # rep > 1: enough (sequence, kv head) pairs for the 8- and 4-wave workgroups
     B = len(pos)
-    n_pages, max_blocks = 40, 8
+    n_pages, max_blocks = 40 * rep, 8
     perm = synth.permutation(13, "ra.pages", n_pages)
     table = np.full((B, max_blocks), -1, dtype=np.int32)
     o = 0
@@ -595,7 +595,7 @@ def test_rope_attn_decode_one_launch_equals_two(ops, synth, Hq, Hkv, D):
     k0 = synth.normal(13, f"ra.k{D}", (n_pages, Hkv, D // 32, 4, 16, 8), 1.0, torch.float16, DEV)
     v0 = synth.normal(13, f"ra.v{D}", (n_pages, Hkv, D, 16), 1.0, torch.float16, DEV)
     qkv = synth.normal(13, f"ra.q{D}.{Hq}", (B, Hq + 2 * Hkv, D), 1.0, torch.float16, DEV)
-    seqs = torch.tensor([0, 1, 2, 3, 4, 5, 99], dtype=torch.int32, device=DEV)      # the last row names no sequence
+    seqs = torch.tensor(list(range(B - 1)) + [B + 92], dtype=torch.int32, device=DEV)      # the last row names no sequence
     tpos = torch.tensor(pos, dtype=torch.int32, device=DEV)
     ctx = tpos + 1
     for frag in (False, True):
@@ -608,7 +608,7 @@ def test_rope_attn_decode_one_launch_equals_two(ops, synth, Hq, Hkv, D):
         assert torch.equal(q2, qkv)
         a, b_ = (got.unpack(), want.unpack()) if frag else (got, want)
         assert torch.equal(a, b_)
-        assert float(a[:6].abs().max()) > 0 and float(a[6].abs().max()) == 0
+        assert float(a[:B - 1].abs().max()) > 0 and float(a[B - 1].abs().max()) == 0
 
 
 @pytest.mark.parametrize("Hq,Hkv,D", [(4, 4, 128), (8, 2, 64)])
