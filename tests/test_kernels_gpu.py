@@ -122,7 +122,8 @@ def test_linear_matches_oracle(ops, synth, T, K, N, kernel, packed):
 
 
 @pytest.mark.parametrize("T,K,N", [(32, 4096, 4096), (32, 4096, 12288), (32, 11008, 4096), (64, 4096, 4096),
-                                   (16, 4096, 22016), (4, 1024, 3072), (1, 1024, 1024), (17, 2752, 1024), (5, 64, 36)])
+                                   (16, 4096, 22016), (4, 1024, 3072), (1, 1024, 1024), (17, 2752, 1024), (5, 64, 36),
+                                   (48, 4096, 12288), (64, 1024, 13072), (33, 512, 32000)])
 def test_gemv_fragment_ordered_activation(ops, synth, T, K, N):
     """Both operands in fragment order: pack/unpack of x is an exact permutation, the product matches."""
     print(f"case gemv_frag T={T} K={K} N={N}", flush=True)
@@ -133,11 +134,13 @@ def test_gemv_fragment_ordered_activation(ops, synth, T, K, N):
     ref = _np(x).astype(np.float64) @ _np(W).astype(np.float64).T
     Wp = ops.PackedWeight(W)
     y16 = ops.linear(xf, Wp)
+    y32 = ops.linear(xf, Wp, out_dtype=torch.float32)
     r0 = synth.normal(7, f"lin.r.{T}.{N}", (T, N), 1.0, torch.float32, DEV)
     racc = r0.clone()
     ops.linear(xf, Wp, out=racc, accumulate=True)
     torch.cuda.synchronize()
     assert max_rel_err(_np(y16), ref) <= TOL
+    assert max_rel_err(_np(y32), ref, floor=1e-2) <= 5e-4
     assert max_rel_err(_np(racc), _np(r0) + ref, floor=1e-2) <= 5e-4
     # identical bits to the row-major-x kernel: same fragments, same accumulation order
     assert torch.equal(y16, ops.linear(x, Wp))
