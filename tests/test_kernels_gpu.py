@@ -688,7 +688,7 @@ def test_gemv_ksplit_partials_summed_by_rmsnorm(ops, synth, T, K, N, ks_expected
     assert torch.equal(r2, r1)
 
 
-@pytest.mark.parametrize("T,K,r,n_ad", [(32, 4096, 16, 16), (20, 11008, 8, 4)])
+@pytest.mark.parametrize("T,K,r,n_ad", [(32, 4096, 16, 16), (20, 11008, 8, 4), (48, 4096, 16, 16), (64, 2048, 32, 6)])
 def test_gemv_ksplit_with_appended_adapter_rows(ops, synth, T, K, r, n_ad):
     """Dense shrink riding in a K-split GEMV: the appended A rows are split with the matrix and the fused expand +
     RMSNorm adds their partials before it applies B.  Against the unsplit pair of calls."""
