@@ -139,8 +139,9 @@ def test_full_depth_benchmark_model_native_equals_per_operator():
 
 
 def test_native_step_between_33_and_64_requests():
-    """48 requests (four token tiles: two row tiles per wave in the GEMV, K split at two rows tiles, SiLU epilogue at
-    four token tiles): the native step reproduces the per-operator path bit for bit, tokens and K cache."""
+    """48 requests (four token tiles: four row tiles per wave in the GEMV with the reduction in two passes, K split,
+    the per-unit SiLU kernel at four token tiles): the native step reproduces the per-operator path bit for bit,
+    tokens and K cache."""
     synth, llama = load_pkg("synth"), load_pkg("llama")
     wl = synth.config3(num_layers=2, batch=48, prompt_len=30)
     ids = wl.adapter_ids.copy()
