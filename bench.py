@@ -82,7 +82,8 @@ def gemv_event_timing(model, T, reps=3):
     n_ext = lt.n_adapters * lt.r
     resid = torch.zeros((T, s.hidden_size), dtype=torch.float32, device=dev)
     qkv = torch.empty((T, s.q_size + 2 * s.kv_size), dtype=torch.float16, device=dev)
-    y2 = torch.empty((T, 3 * n_ext), dtype=torch.float32, device=dev)
+    kq = lib.mlora_gemv_split_kq(T, s.hidden_size, s.q_size + 2 * s.kv_size, 3 * n_ext)   # K-range blocks of the appended q/k/v rows
+    y2 = torch.empty((kq, T, 3 * n_ext), dtype=torch.float32, device=dev)
     logits = torch.empty((T, s.vocab_size), dtype=torch.float32, device=dev)
     F16, F32, STORE, ACC = lm.F16, lm.F32, lm.STORE, lm.ACCUMULATE
     H, I, Q, QKV = s.hidden_size, s.intermediate_size, s.q_size, s.q_size + 2 * s.kv_size
@@ -101,9 +102,9 @@ def gemv_event_timing(model, T, reps=3):
         wq, wo, wd, wg = ext[l]["qkv"], ext[l]["o"], ext[l]["down"], il[l]
         q_ext = wq.N - QKV
         o_ext = wo.N - H
-        add(lambda wq=wq, q_ext=q_ext: lib.mlora_gemv_frag_split(qkv.data_ptr(), F16, STORE, y2.data_ptr(), x_h.data.data_ptr(),
-                                                                 wq.data.data_ptr(), T, H, QKV, q_ext, st),
-            wq.N, H, T * QKV * 2 + T * q_ext * 4)
+        add(lambda wq=wq, q_ext=q_ext: lib.mlora_gemv_frag_split_kq(qkv.data_ptr(), y2.data_ptr(), kq, x_h.data.data_ptr(),
+                                                                    wq.data.data_ptr(), T, H, QKV, q_ext, st),
+            wq.N, H, T * QKV * 2 + kq * T * q_ext * 4)
         add(lambda wo=wo, o_ext=o_ext: lib.mlora_gemv_frag_acc_ksplit(resid.data_ptr(), y2.data_ptr(), part.data_ptr(), ks_o,
                                                                       x_q.data.data_ptr(), wo.data.data_ptr(), T, Q, H, o_ext,
                                                                       None, None, 0, None, 0, 0, st),
@@ -468,7 +469,7 @@ def main():
     }
     if not args.no_extras:
         g = gemv_event_timing(model, wl.batch)
-        out["roofline"] = {"kernel": "gemv_kernel / gemv_silu_cu_kernel (fragment-ordered weights and activations, T=32; the 129 GEMV launches of one decode step: adapter A rows appended to qkv / o, K split on o / down, SiLU epilogue on gate/up)", "bound": "hbm", "achieved": g["gbs"],
+        out["roofline"] = {"kernel": "gemv_kernel / gemv_split_cu_kernel / gemv_silu_cu_kernel (fragment-ordered weights and activations, T=32; the 129 GEMV launches of one decode step: adapter A rows appended to qkv / o, K split on o / down, SiLU epilogue on gate/up)", "bound": "hbm", "achieved": g["gbs"],
                            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g["gbs"] / HBM_PEAK_GBS, "traffic": profiled_gemv_traffic(),
                            "launches_timed": g["launches"], "avg_launch_us": g["avg_us"],
                            "algorithmic_bytes_per_launch": g["bytes_per_launch"]}

@@ -264,8 +264,9 @@ int mlora_paged_attn_prefill(void* out, const void* qkv, const void* k_cache, co
  *                               A bytes alone and with no dependence on the token->adapter table;
  *   mlora_rope_kv_append_lora - mlora_rope_kv_append, after adding scaling * B[p][id_t] . v to the q, k, v
  *                               rows of qkv (B[p] [n_ad, N_p, r] or NULL).  v_dense = 0: v_part holds the K-slice
- *                               partials written by mlora_gemv_frag_lora with this K; v_dense = 1: v_part is
- *                               y2 [T, 3 * n_ad * r] of mlora_gemv_frag_split (slot p = projection p);
+ *                               partials written by mlora_gemv_frag_lora with this K; v_dense = kq >= 1: v_part is
+ *                               y2 [kq][T, 3 * n_ad * r] of mlora_gemv_frag_split (kq = 1) or
+ *                               mlora_gemv_frag_split_kq (slot p = projection p; the kq blocks are added in order);
  *   mlora_lora_expand_rmsnorm - resid[t, :] += scaling * B[id_t] . v (B [n_ad, H, r]; v_part [kc][T][r] partials
  *                               of a shrink over K inputs, or y2 [T, n_ad * r] when v_dense = 1), then
  *                               y = RMSNorm(resid) as mlora_rmsnorm.
@@ -280,6 +281,14 @@ int mlora_gemv_frag_lora(void* y, int y_dtype, int mode, const void* xf, const v
  * halves of a channel.  Replaces: gate_proj, up_proj, op.silu and the multiply (llama_for_causal_lm.py:35-36) in
  * one launch; same result bits as mlora_gemv_frag followed by mlora_silu_mul. */
 int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p, int T, int K, int I, void* stream);
+/* The split GEMV with f16 y as one workgroup per compute unit: the appended rows are cut into kq ranges of K and come
+ * back as kq blocks of partial sums, y2 [kq][T][N_ext] fp32, which the reader adds in block order (pass kq as v_dense
+ * to mlora_rope_attn_decode / mlora_rope_kv_append_lora).  mlora_gemv_split_kq names kq for a shape (1: the form does
+ * not apply; mlora_gemv_frag_split_kq with kq == 1 is mlora_gemv_frag_split).  No counterpart in the reference beyond
+ * the linear itself (llama_for_causal_lm.py:44-47). */
+int mlora_gemv_split_kq(int T, int K, int N_main, int N_ext);
+int mlora_gemv_frag_split_kq(void* y, float* y2, int kq, const void* xf, const void* Wp, int T, int K, int N_main,
+                             int N_ext, void* stream);
 int mlora_gemv_frag_split(void* y, int y_dtype, int mode, float* y2, const void* xf, const void* Wp,
                           int T, int K, int N_main, int N_ext, void* stream);
 int mlora_rope_kv_append_lora(void* qkv, void* k_cache, void* v_cache,
@@ -359,7 +368,8 @@ int mlora_rmsnorm_ksplit(void* y, int y_layout, float* resid, const float* part,
  * Scratch buffers are caller-owned (sizes in elements):
  *   resid f32 [T*H]; xn, attn: mlora_frag_activation_elems(T, H | Hq*D) f16; qkv f16 [T*(Hq+2Hkv)*D];
  *   gate_up f16 [T*2I]; act: mlora_frag_activation_elems(T, I) f16; logits f32 [T*V];
- *   lora_ws: 5 * mlora_gather_mm_workspace_bytes(T, max(H, I, Hq*D), r) bytes.
+ *   lora_ws: 5 slots of max(mlora_gather_mm_workspace_bytes(T, max(H, I, Hq*D), r), 4 * T * n_ad * r) bytes;
+ *     with lora_dense, (3 * kq + 2) slots for kq = mlora_gemv_split_kq(T, H, (Hq+2Hkv)*D, 3 * n_ad * r) (at most 14).
  * ------------------------------------------------------------------------------------------- */
 typedef struct mlora_lora_proj {
   const void* A;   /* [n_ad, r, K] f16 or NULL */

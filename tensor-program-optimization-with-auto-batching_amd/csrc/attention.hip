@@ -393,6 +393,7 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
   constexpr int half = D / 2;
   __shared__ float sm[NW][16], sl[NW][16];
   __shared__ float lv[3][64];
+  __shared__ float lvq[LORA_MAX_KQ][3][64];     // K-range blocks of dense shrink results before they are added
   __shared__ __align__(16) f16 qs[16 * D];       // rotated q of the group's heads
   __shared__ __align__(16) f16 knew[D], vnew[D];   // the new token's rotated key and its value
   extern __shared__ float sacc[];                  // [NW][G][D]
@@ -510,9 +511,27 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
   const bool first = threadIdx.x < items;
   if (first) issue(threadIdx.x);
   if (adapted) {
-    for (int e = threadIdx.x; e < 3 * lx.r; e += NW * WAVE) {
-      const int pj = e / lx.r, j = e % lx.r;
-      lv[pj][j] = lx.B[pj] != nullptr ? lora_v_from(lx.src, pj, id, lx.r, b, j, lx.scaling) : 0.f;
+    if (lx.src.kc == 0 && lx.src.kq > 1) {
+      // dense shrink results in kq blocks of K-range partials: one thread per (block, entry) fetches, then the blocks
+      // are added in order - no thread waits for more than one load
+      for (int e = threadIdx.x; e < lx.src.kq * 3 * lx.r; e += NW * WAVE) {
+        const int q = e / (3 * lx.r), pj = (e / lx.r) % 3, j = e % lx.r;
+        lvq[q][pj][j] = lx.B[pj] != nullptr
+                            ? lx.src.v[((size_t)q * lx.src.T + b) * lx.src.ld + ((size_t)pj * lx.src.n_ad + id) * lx.r + j]
+                            : 0.f;
+      }
+      __syncthreads();
+      for (int e = threadIdx.x; e < 3 * lx.r; e += NW * WAVE) {
+        const int pj = e / lx.r, j = e % lx.r;
+        float a = lvq[0][pj][j];
+        for (int q = 1; q < lx.src.kq; ++q) a += lvq[q][pj][j];
+        lv[pj][j] = a * lx.scaling;
+      }
+    } else {
+      for (int e = threadIdx.x; e < 3 * lx.r; e += NW * WAVE) {
+        const int pj = e / lx.r, j = e % lx.r;
+        lv[pj][j] = lx.B[pj] != nullptr ? lora_v_from(lx.src, pj, id, lx.r, b, j, lx.scaling) : 0.f;
+      }
     }
     __syncthreads();
   }
@@ -811,6 +830,7 @@ extern "C" int mlora_rope_kv_append_lora(void* qkv, void* k_cache, void* v_cache
   LoraExpandQKV lx = {};
   lx.src.v = (const float*)v_part;
   lx.src.kc = v_dense ? 0 : lora_k_split(K).kc;
+  lx.src.kq = v_dense > 0 ? v_dense : 1;
   lx.src.T = T; lx.src.n_ad = n_ad; lx.src.ld = 3 * n_ad * r;
   for (int i = 0; i < 3; ++i) lx.B[i] = (const f16*)B[i];
   lx.ids = tok_adapter;
@@ -875,6 +895,7 @@ extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv
                 "rope_attn_decode: rank %d not in {8,16,32,64} or bad n_ad/K", r);
     lx.src.v = (const float*)v_part;
     lx.src.kc = v_dense ? 0 : lora_k_split(K).kc;
+    lx.src.kq = v_dense > 0 ? v_dense : 1;
     lx.src.T = B; lx.src.n_ad = n_ad; lx.src.ld = 3 * n_ad * r;
     for (int i = 0; i < 3; ++i) lx.B[i] = (const f16*)Bmat[i];
     lx.ids = tok_adapter;

@@ -37,12 +37,15 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
   const int Kmax = H > I ? (H > q_sz ? H : q_sz) : (I > q_sz ? I : q_sz);
   size_t slot = lora ? mlora_gather_mm_workspace_bytes(T, Kmax, r) : 0;
   if (dense && slot < (size_t)T * n_ad * r * sizeof(float)) slot = (size_t)T * n_ad * r * sizeof(float);
-  MLORA_CHECK(!lora || (p->lora_ws && p->lora_ws_bytes >= 5 * slot), MLORA_ERR_WORKSPACE,
-              "decode_step: lora_ws of %zu bytes given, %zu needed", p->lora_ws_bytes, 5 * slot);
+  // dense q/k/v shrink rows may come as kq blocks of K-range partials (one-workgroup-per-unit GEMV): 3 kq slots
+  const int kq = dense ? mlora_gemv_split_kq(T, H, qkv_sz, 3 * n_ad * r) : 1;
+  const size_t ws_need = (size_t)(3 * kq + 2) * slot;
+  MLORA_CHECK(!lora || (p->lora_ws && p->lora_ws_bytes >= ws_need), MLORA_ERR_WORKSPACE,
+              "decode_step: lora_ws of %zu bytes given, %zu needed", p->lora_ws_bytes, ws_need);
   char* ws = (char*)p->lora_ws;
   void* ws_qkv = ws;
-  void* ws_o = ws + 3 * slot;
-  void* ws_down = ws + 4 * slot;
+  void* ws_o = ws + (size_t)3 * kq * slot;
+  void* ws_down = ws + (size_t)(3 * kq + 1) * slot;
   auto delta = [&](void* y, int y_dtype, int ldy, const void* x, const mlora_lora_proj& lp, int K, int N) -> int {
     if (!lora || !lp.A) return MLORA_OK;
     return mlora_gather_mm(y, y_dtype, ldy, x, MLORA_FRAG, lp.A, lp.B, p->tok_adapter, sc, T, K, N, r, n_ad, ws_down, slot, stream);
@@ -85,10 +88,10 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
       const void* A3[3] = {L.lora[MLORA_Q].A, L.lora[MLORA_K].A, L.lora[MLORA_V].A};
       const void* B3[3] = {L.lora[MLORA_Q].A ? L.lora[MLORA_Q].B : nullptr, L.lora[MLORA_K].A ? L.lora[MLORA_K].B : nullptr,
                            L.lora[MLORA_V].A ? L.lora[MLORA_V].B : nullptr};
-      if (dense) STEP(mlora_gemv_frag_split(qkv, MLORA_F16, MLORA_STORE, (float*)ws_qkv, p->xn, L.qkv_p, T, H, qkv_sz, 3 * n_ad * r, stream));
+      if (dense) STEP(mlora_gemv_frag_split_kq(qkv, (float*)ws_qkv, kq, p->xn, L.qkv_p, T, H, qkv_sz, 3 * n_ad * r, stream));
       else STEP(mlora_gemv_frag_lora(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, ws_qkv, A3, 3, p->tok_adapter, r, n_ad, stream));
       STEP(mlora_rope_attn_decode(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos,
-                                  p->ctx, p->rope_cos, p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, ws_qkv, dense,
+                                  p->ctx, p->rope_cos, p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, ws_qkv, dense ? kq : 0,
                                   B3, p->tok_adapter, sc, H, r, n_ad, stream));
     } else {
       STEP(mlora_gemv_frag(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, stream));

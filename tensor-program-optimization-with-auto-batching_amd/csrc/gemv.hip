@@ -280,6 +280,100 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, 2) void gemv_silu_cu_kernel(f16* 
   }
 }
 
+// GEMV over a weight with appended shrink rows (q/k/v + the stacked A tables) as ONE workgroup per compute unit.
+// The main row tiles are dealt out evenly (NM or NM - 1 per unit); the few appended tiles are cut into kq ranges of K
+// and every (tile, range) piece goes to a unit of its own, starting with the units that got one main tile fewer, so
+// that no unit takes in more than NM tiles plus a 1/kq piece - with whole appended tiles in the deal, the units that
+// drew one would set the time of the launch.  A piece's fp32 partial goes to block `range` of y2 [kq][T][n_ext];
+// whoever reads the shrink results adds the blocks in range order.  Main rows: f16 store, the k order and the wave
+// reduction of gemv_kernel, hence its bits.
+template <int NM, int TT, int PIPE>
+__global__ __launch_bounds__(GEMV_WAVES* WAVE, 2) void gemv_split_cu_kernel(f16* __restrict__ y, float* __restrict__ y2,
+                                                                         const f16* __restrict__ x, const f16* __restrict__ W,
+                                                                         int T, int K, int n_main, int n_ext, int base, int rem,
+                                                                         int kq) {
+  constexpr int NT = NM + 1;                           // register tile NM is the piece of an appended tile
+  __shared__ f32x4 red[GEMV_WAVES][TT][WAVE];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int wg = blockIdx.x;
+  const int m0 = wg * base + (wg < rem ? wg : rem);    // first main tile of this workgroup
+  const int nm = base + (wg < rem ? 1 : 0);            // and how many it has
+  const int KB = K / KSTEP;
+  const int piece = (int)gridDim.x - 1 - wg;           // pieces are dealt from the last unit backwards
+  const bool has_ext = piece < (n_ext / 16) * kq;
+  const int et = has_ext ? piece / kq : 0, eq = has_ext ? piece % kq : 0;
+  const int ekb0 = has_ext ? (int)((long)eq * KB / kq) : 0, ekb1 = has_ext ? (int)((long)(eq + 1) * KB / kq) : 0;
+  const f16* wp = W + lane * 8;
+  size_t woff[NT];                                     // a missing main tile repeats the first one (cache hits) and is not stored
+#pragma unroll
+  for (int i = 0; i < NM; ++i) woff[i] = (size_t)(m0 + (i < nm ? i : 0)) * KB * 512;
+  woff[NM] = (size_t)(n_main / 16 + et) * KB * 512;
+  const f16* xp = x + lane * 8;
+  constexpr int XSTEP = TT * 512;
+
+  f32x4 acc[NT][TT];
+#pragma unroll
+  for (int i = 0; i < NT; ++i)
+#pragma unroll
+    for (int j = 0; j < TT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int S = (KB - wave + GEMV_WAVES - 1) / GEMV_WAVES;
+  f16x8 a[PIPE][NT], b[PIPE][TT];
+  auto load_stage = [&](int u, int s) {
+    const bool in = s < S;
+    const int ks = in ? wave + GEMV_WAVES * s : 0;
+#pragma unroll
+    for (int i = 0; i < NM; ++i) {
+      a[u][i] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(wp + (woff[i] + (size_t)ks * 512)));
+      if (!in) a[u][i] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+    a[u][NM] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    if (in && ks >= ekb0 && ks < ekb1)                 // wave-uniform: the piece covers only its range of K
+      a[u][NM] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(wp + (woff[NM] + (size_t)ks * 512)));
+#pragma unroll
+    for (int j = 0; j < TT; ++j) b[u][j] = ld8(xp + j * 512 + (size_t)ks * XSTEP);
+  };
+#pragma unroll
+  for (int u = 0; u < PIPE; ++u) load_stage(u, u);
+  for (int s0 = 0; s0 < S; s0 += PIPE) {
+#pragma unroll
+    for (int u = 0; u < PIPE; ++u) {
+#pragma unroll
+      for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int j = 0; j < TT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][i], b[u][j], acc[i][j], 0, 0, 0);
+      load_stage(u, s0 + u + PIPE);
+    }
+  }
+  // the waves' sums, one register tile at a time, added in wave order
+#pragma unroll
+  for (int i = 0; i < NT; ++i) {
+    const bool live = i < NM ? i < nm : has_ext;       // workgroup-uniform
+    if (live) {
+#pragma unroll
+      for (int j = 0; j < TT; ++j) red[wave][j][lane] = acc[i][j];
+      __syncthreads();
+      for (int e = threadIdx.x; e < TT * WAVE; e += GEMV_WAVES * WAVE) {
+        const int j = e >> 6, sl = e & 63;
+        f32x4 s = red[0][j][sl];
+#pragma unroll
+        for (int w = 1; w < GEMV_WAVES; ++w) s += red[w][j][sl];
+        const int t = j * 16 + (sl & 15);
+        if (t < T) {
+          if (i < NM) {
+            const int n = (m0 + i) * 16 + (sl >> 4) * 4;
+            *reinterpret_cast<f16x4*>(y + (size_t)t * n_main + n) = f16x4{(f16)s[0], (f16)s[1], (f16)s[2], (f16)s[3]};
+          } else {
+            const int n = et * 16 + (sl >> 4) * 4;
+            *reinterpret_cast<f32x4*>(y2 + ((size_t)eq * T + t) * n_ext + n) = s;
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
 // one thread per 16-byte chunk of the packed array
 __global__ __launch_bounds__(256) void pack_weight_kernel(f16* __restrict__ dst, const f16* __restrict__ src, int N, int K,
                                                           size_t chunks) {
@@ -482,6 +576,16 @@ extern "C" int mlora_gemv_frag_acc_ksplit(float* y, float* y2, float* part, int 
                                           ks, part);
 }
 
+// compute units of the current device (0 if it cannot be asked), read once
+static int gemv_n_cu() {
+  static const int n_cu = [] {
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cu = 0;
+    return cu;
+  }();
+  return n_cu;
+}
+
 extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p, int T, int K, int I, void* stream) {
   MLORA_CHECK(act && xf && Wil_p, MLORA_ERR_INVALID, "gemv_frag_silu: null pointer");
   MLORA_CHECK(T > 0 && T <= 64 && K > 0 && K % 32 == 0 && I > 0 && I % 32 == 0, MLORA_ERR_UNSUPPORTED,
@@ -492,11 +596,7 @@ extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p
   const LoraShrinkBatch sb = LoraShrinkBatch();
   const dim3 grid(I / 16), block(GEMV_WAVES * WAVE);
   // enough pairs for two or more per compute unit: one workgroup per unit with an equal share of the pairs
-  static const int n_cu = [] {
-    int dev = 0, cu = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cu = 0;
-    return cu;
-  }();
+  const int n_cu = gemv_n_cu();
   const int pairs = I / 16;
   const int per = n_cu > 0 ? ceil_div(pairs, n_cu) : 0;
   if ((T <= 32 || per <= 3) && n_cu > 0 && pairs >= 2 * n_cu && per <= 4) {
@@ -533,6 +633,48 @@ extern "C" int mlora_gemv_frag_split(void* y, int y_dtype, int mode, float* y2, 
               "gemv_frag_split: need y2, N_ext %% 4 == 0 and N_main %% 16 == 0 (N_main=%d N_ext=%d)", N_main, N_ext);
   if (T == 0) return MLORA_OK;
   return gemv_dispatch<true, true, false>(y, y_dtype, mode, xf, K, Wp, T, K, N_main + N_ext, stream, LoraShrinkBatch(), N_main, y2);
+}
+
+// K ranges of the appended rows in the one-workgroup-per-unit form of the split GEMV (1: that form does not apply)
+extern "C" int mlora_gemv_split_kq(int T, int K, int N_main, int N_ext) {
+  const int n_cu = gemv_n_cu();
+  if (T <= 0 || T > 32 || K <= 0 || K % 32 || N_main <= 0 || N_main % 16 || N_ext <= 0 || N_ext % 16 || n_cu <= 0) return 1;
+  const int main_tiles = N_main / 16, ext_tiles = N_ext / 16;
+  const int per = ceil_div(main_tiles, n_cu);
+  const int kq = LORA_MAX_KQ;
+  if (main_tiles < 2 * n_cu || per > 3 || (K / 32) / kq < 8 || ext_tiles * kq > n_cu) return 1;
+  return kq;
+}
+
+extern "C" int mlora_gemv_frag_split_kq(void* y, float* y2, int kq, const void* xf, const void* Wp, int T, int K, int N_main,
+                                        int N_ext, void* stream) {
+  if (int e = mlora_check_linear("gemv_frag_split_kq", y, MLORA_F16, MLORA_STORE, xf, K, Wp, T, K, N_main)) return e;
+  MLORA_CHECK(T <= 64, MLORA_ERR_UNSUPPORTED, "gemv_frag_split_kq: T=%d exceeds 64", T);
+  MLORA_CHECK(y2 && N_ext > 0 && N_ext % 4 == 0 && N_main % 16 == 0, MLORA_ERR_INVALID,
+              "gemv_frag_split_kq: need y2, N_ext %% 4 == 0 and N_main %% 16 == 0 (N_main=%d N_ext=%d)", N_main, N_ext);
+  MLORA_CHECK(kq == 1 || kq == mlora_gemv_split_kq(T, K, N_main, N_ext), MLORA_ERR_INVALID,
+              "gemv_frag_split_kq: kq=%d, mlora_gemv_split_kq gives %d", kq, mlora_gemv_split_kq(T, K, N_main, N_ext));
+  if (T == 0) return MLORA_OK;
+  if (kq == 1)
+    return gemv_dispatch<true, true, false>(y, MLORA_F16, MLORA_STORE, xf, K, Wp, T, K, N_main + N_ext, stream, LoraShrinkBatch(), N_main, y2);
+  const int n_cu = gemv_n_cu();
+  const int main_tiles = N_main / 16;
+  const int base = main_tiles / n_cu, rem = main_tiles % n_cu;
+  const int per = ceil_div(main_tiles, n_cu);
+  const dim3 g(n_cu), block(GEMV_WAVES * WAVE);
+  hipStream_t s = (hipStream_t)stream;
+#define MLORA_SPLIT_CU(NM, TT, PIPE)                                                                                       \
+  hipLaunchKernelGGL((gemv_split_cu_kernel<NM, TT, PIPE>), g, block, 0, s, (f16*)y, y2, (const f16*)xf, (const f16*)Wp, T, K, \
+                     N_main, N_ext, base, rem, kq)
+  if (T <= 16) {
+    if (per <= 2) MLORA_SPLIT_CU(2, 1, 4);
+    else MLORA_SPLIT_CU(3, 1, 4);
+  } else {
+    if (per <= 2) MLORA_SPLIT_CU(2, 2, 4);
+    else MLORA_SPLIT_CU(3, 2, 3);
+  }
+#undef MLORA_SPLIT_CU
+  return mlora_launch_status("gemv_frag_split_kq");
 }
 
 extern "C" size_t mlora_frag_activation_elems(int T, int K) {

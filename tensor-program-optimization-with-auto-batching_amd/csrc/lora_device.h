@@ -6,6 +6,7 @@
 constexpr int LORA_KCHUNK = 512;   // K elements one wave covers per pass: 64 lanes x 8 fp16
 constexpr int LORA_MAX_KC = 8;     // K-slices (fp32 partials) per token
 constexpr int LORA_MAX_PROJ = 3;   // projections that share x in one batched shrink (q, k, v)
+constexpr int LORA_MAX_KQ = 4;     // K-range blocks of dense shrink results
 
 struct LoraKSplit { int ci; int kc; };
 
@@ -152,16 +153,20 @@ __device__ __forceinline__ float lora_v(const float* __restrict__ vpart_proj, in
 
 // Where an expand finds v for (token t, projection slot p, adapter id):
 //   kc > 0  : K-slice partials v_part[p][c][t][:]                    (written by the shrink units)
-//   kc == 0 : dense shrink results v_all[t][(p * n_ad + id) * r + :]  (written by a GEMV over weight rows that have the
-//             A tables of all adapters appended; the adapter is picked here, by index)
+//   kc == 0 : dense shrink results v_all[q][t][(p * n_ad + id) * r + :]  (written by a GEMV over weight rows that have
+//             the A tables of all adapters appended; the adapter is picked here, by index).  kq >= 1 blocks q hold
+//             the partial sums of kq ranges of K, added here in range order.
 struct LoraVSource {
   const float* v;
-  int kc, T, n_ad, ld;
+  int kc, T, n_ad, ld, kq;
 };
 
 __device__ __forceinline__ float lora_v_from(const LoraVSource& s, int slot, int id, int r, int t, int j, float scaling) {
   if (s.kc > 0) return lora_v(s.v + (size_t)slot * s.kc * s.T * r, s.kc, s.T, r, t, j, scaling);
-  return s.v[(size_t)t * s.ld + ((size_t)slot * s.n_ad + id) * r + j] * scaling;
+  const float* __restrict__ p = s.v + (size_t)t * s.ld + ((size_t)slot * s.n_ad + id) * r + j;
+  float a = p[0];
+  for (int q = 1; q < s.kq; ++q) a += p[(size_t)q * s.T * s.ld];
+  return a * scaling;
 }
 
 // The same dot product in two halves, so that a caller can issue the row's loads before the v values are ready:

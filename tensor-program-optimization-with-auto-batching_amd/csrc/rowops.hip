@@ -333,6 +333,7 @@ extern "C" int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, co
   LoraExpandRow lx = {};
   lx.src.v = (const float*)v_part;
   lx.src.kc = v_dense ? 0 : lora_k_split(K).kc;
+  lx.src.kq = 1;
   lx.src.T = T; lx.src.n_ad = n_ad; lx.src.ld = n_ad * r;
   lx.B = (const f16*)B;
   lx.ids = tok_adapter;
@@ -355,6 +356,7 @@ extern "C" int mlora_rmsnorm_ksplit(void* y, int y_layout, float* resid, const f
                 "rmsnorm_ksplit: partials of a dense shrink need ld_part >= H + n_ad * r (ld_part=%d)", ld_part);
     lx.src.v = (const float*)v_part;
     lx.src.kc = v_dense ? 0 : lora_k_split(K).kc;
+    lx.src.kq = 1;
     lx.src.T = T; lx.src.n_ad = n_ad; lx.src.ld = n_ad * r;
     lx.B = (const f16*)B;
     lx.ids = tok_adapter;

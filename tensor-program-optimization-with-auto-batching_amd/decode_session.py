@@ -112,8 +112,9 @@ class NativeDecodeSession:
             "logits": torch.empty(T * V, dtype=f32, device=dev),
         }
         r = lt.r if lt is not None else 0
-        ws_bytes = 5 * max(_lib.lib().mlora_gather_mm_workspace_bytes(T, max(H, I, s.q_size), max(r, 8)),
-                           4 * T * (lt.n_adapters if lt is not None else 0) * max(r, 8))
+        # five slots (q, k, v, o, down); the dense q/k/v shrink may come as up to four K-range blocks of three slots
+        ws_bytes = 14 * max(_lib.lib().mlora_gather_mm_workspace_bytes(T, max(H, I, s.q_size), max(r, 8)),
+                            4 * T * (lt.n_adapters if lt is not None else 0) * max(r, 8))
         self.buf["lora_ws"] = torch.empty(ws_bytes // 4, dtype=f32, device=dev)
         # partials of the K-split o_proj / down_proj GEMVs (up to 3 slices of [T, H + appended adapter rows])
         ks_elems = 3 * T * (H + (lt.n_adapters * r if lt is not None else 0)) if ksplit else 0
