@@ -155,3 +155,22 @@ def test_native_step_between_33_and_64_requests():
     d, _, ld = _run(model, wl, prompts, ids, "dense", 5, synth, run_steps=1)
     err = float((ld - lg).abs().max() / lg.std())
     assert err <= 1e-2, err
+
+
+def test_native_step_at_most_16_requests():
+    """12 requests at the benchmark model's layer shapes (one token tile: the one-tile forms of the per-unit q/k/v and
+    SiLU GEMVs, K-range blocks of the appended adapter rows): the native step reproduces the per-operator path bit for
+    bit, and the dense-shrink variant agrees with it within rounding."""
+    synth, llama = load_pkg("synth"), load_pkg("llama")
+    wl = synth.config3(num_layers=2, batch=12, prompt_len=30)
+    ids = wl.adapter_ids.copy()
+    ids[5] = -1
+    model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, [wl.lora], DEV)
+    prompts = synth.prompts(wl)
+    a, ka, _ = _run(model, wl, prompts, ids, "py", 5, synth)
+    c, kc, lg = _run(model, wl, prompts, ids, "graph", 5, synth)
+    assert np.array_equal(a, c)
+    assert torch.equal(ka, kc)
+    d, _, ld = _run(model, wl, prompts, ids, "dense", 5, synth, run_steps=1)
+    err = float((ld - lg).abs().max() / lg.std())
+    assert err <= 1e-2, err
