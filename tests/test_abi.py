@@ -98,6 +98,12 @@ def test_argument_validation_of_fused_and_batched_entry_points():
     assert lib.mlora_gemv_ksplit(33, 11008, 4096) == 4 and lib.mlora_gemv_ksplit(32, 4096, 12288) == 1
     assert lib.mlora_gemv_ksplit(65, 11008, 4096) == 1 and lib.mlora_gemv_ksplit(64, 4096, 4352) == 3
     assert lib.mlora_gemv_ksplit_bytes(32, 4096, 4) == 3 * 32 * 4096 * 4 and lib.mlora_gemv_ksplit_bytes(32, 4096, 1) == 0
+    # K-range blocks of the appended rows in the per-unit split GEMV: 1 where the form does not apply (and without a device)
+    assert lib.mlora_gemv_split_kq(32, 4096, 12288, 768) in (1, 4)
+    assert lib.mlora_gemv_split_kq(33, 4096, 12288, 768) == 1 and lib.mlora_gemv_split_kq(32, 4096, 1024, 768) == 1
+    assert lib.mlora_gemv_split_kq(32, 4096, 12288, 772) == 1
+    assert lib.mlora_gemv_frag_split_kq(1, 1, 3, 1, 1, 32, 4096, 12288, 768, None) == -1 and b"kq" in lib.mlora_last_error()
+    assert lib.mlora_gemv_frag_split_kq(1, None, 1, 1, 1, 32, 4096, 12288, 768, None) == -1
     ksg = lambda ks, part, T=32, n_ext=0, y2=None, A=None: lib.mlora_gemv_frag_acc_ksplit(1, y2, part, ks, 1, 1, T, 4096, 4096, n_ext,
                                                                                          None, A, 1 if A else 0, None, 16, 4, None)
     assert ksg(2, None) == -1                        # split without a partials buffer
