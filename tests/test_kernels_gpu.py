@@ -738,6 +738,40 @@ def test_gemv_ksplit_with_appended_adapter_rows(ops, synth, T, K, r, n_ad):
     assert float((out[0][0] - out[1][0]).abs().max()) <= 1e-4
 
 
+@pytest.mark.parametrize("T,N_main,n_ad", [(32, 12288, 48), (12, 12288, 16), (32, 8192, 10), (20, 10240, 48)])
+def test_split_gemv_one_workgroup_per_unit(ops, synth, T, N_main, n_ad):
+    """The q/k/v GEMV with appended adapter rows as one workgroup per compute unit: the main rows carry the bits of the
+    ordinary split GEMV, and the K-range blocks of the appended rows add up to its second result within fp32 rounding."""
+    L = load_pkg("_lib")
+    lib = L.lib()
+    K, r = 4096, 16
+    n_ext = n_ad * r
+    kq = lib.mlora_gemv_split_kq(T, K, N_main, n_ext)
+    assert kq == 4
+    x = synth.normal(31, f"sc.x.{T}", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(31, f"sc.W.{N_main}.{n_ext}", (N_main + n_ext, K), 0.02, torch.float16, DEV)
+    xf, Wp = ops.FragActivation.pack(x), ops.PackedWeight(W)
+    st = torch.cuda.current_stream().cuda_stream
+    y_a = torch.full((T, N_main), float("nan"), dtype=torch.float16, device=DEV)
+    y_b = y_a.clone()
+    y2_a = torch.full((T, n_ext), float("nan"), dtype=torch.float32, device=DEV)
+    y2_b = torch.full((kq, T, n_ext), float("nan"), dtype=torch.float32, device=DEV)
+    L.check(lib.mlora_gemv_frag_split(y_a.data_ptr(), L.F16, L.STORE, y2_a.data_ptr(), xf.data.data_ptr(), Wp.data.data_ptr(), T, K,
+                                      N_main, n_ext, st))
+    L.check(lib.mlora_gemv_frag_split_kq(y_b.data_ptr(), y2_b.data_ptr(), kq, xf.data.data_ptr(), Wp.data.data_ptr(), T, K, N_main,
+                                         n_ext, st))
+    torch.cuda.synchronize()
+    assert torch.equal(y_a, y_b)
+    assert not torch.isnan(y2_b).any()
+    ref2 = _np(x).astype(np.float64) @ _np(W[N_main:]).astype(np.float64).T
+    assert max_rel_err(_np(y2_b.sum(0)), ref2, floor=1e-2) <= 5e-4
+    assert max_rel_err(_np(y2_a), ref2, floor=1e-2) <= 5e-4
+    # kq == 1 through the same entry point is the ordinary kernel
+    y_c, y2_c = torch.empty_like(y_a), torch.empty_like(y2_a)
+    L.check(lib.mlora_gemv_frag_split_kq(y_c.data_ptr(), y2_c.data_ptr(), 1, xf.data.data_ptr(), Wp.data.data_ptr(), T, K, N_main, n_ext, st))
+    assert torch.equal(y_c, y_a) and torch.equal(y2_c, y2_a)
+
+
 # ------------------------------------------------------------------ plain prefill GEMM through the vendor library
 @pytest.mark.parametrize("T,K,N", [(256, 4096, 4096), (300, 1024, 1000), (1024, 2752, 1024), (130, 64, 40), (70, 1024, 512)])
 def test_library_gemm_matches_oracle(ops, synth, T, K, N):
