@@ -248,12 +248,14 @@ __global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restric
 // ---------------------------------------------------------------------------------------------
 constexpr int ATT_WAVES = 4;
 
-// Waves per workgroup of the decode kernels: four when the launch has workgroups enough to fill the chip four deep
-// (every CU then holds 16 waves, one page each in flight), more when sequences x kv heads are few (small batches,
-// grouped-query models), so that a CU still has 16 pages in flight.  Limited by the LDS merge buffer [NW][G][D].
+// Waves per workgroup of the decode kernels.  A CU holds 16 waves either way (one page each in flight); few, large
+// workgroups spread the per-workgroup work (new token, merge of the waves' states) over more waves and keep a CU busy
+// when sequences x kv heads are few (small batches, grouped-query models); many small ones balance better when the
+// launch runs in several rounds (measured: eight waves up to 2048 workgroups' worth, four beyond).  Limited by the LDS
+// merge buffer [NW][G][D].
 int attn_waves(int B, int Hkv, int G, int D) {
   const long wgs = (long)B * Hkv;
-  int nw = wgs > 512 ? ATT_WAVES : wgs > 256 ? 8 : 16;
+  int nw = wgs > 2048 ? ATT_WAVES : wgs > 256 ? 8 : 16;
   while (nw > ATT_WAVES && (size_t)nw * G * D * sizeof(float) > 48 * 1024) nw >>= 1;
   return nw;
 }
