@@ -284,7 +284,7 @@ def _paged_setup(synth, n_seq, Hq, Hkv, D, lens_before, append, seed, n_pages=No
     return ref, perm, n_pages, cos, sin
 
 
-@pytest.mark.parametrize("Hq,Hkv,D,n_seq", [(32, 32, 128, 5), (16, 16, 64, 5), (8, 2, 128, 5), (32, 16, 128, 20), (8, 8, 64, 70)])
+@pytest.mark.parametrize("Hq,Hkv,D,n_seq", [(32, 32, 128, 5), (16, 16, 64, 5), (8, 2, 128, 5), (32, 16, 128, 20), (8, 8, 64, 70), (32, 32, 64, 70)])
 def test_paged_attention_prefill_then_decode(ops, synth, Hq, Hkv, D, n_seq):
     """Prefill ragged prompts, then two decode steps, against the oracle cache (page permutation shared).  The decode
     launches cover the three workgroup shapes: few (sequence, kv head) pairs, 257..512 of them, and more."""
@@ -576,13 +576,13 @@ def test_gather_mm_prefill_column_slice(ops, synth):
     assert np.array_equal(after[:, :N], before[:, :N]) and np.array_equal(after[:, 2 * N:], before[:, 2 * N:])
 
 
-@pytest.mark.parametrize("Hq,Hkv,D,rep", [(4, 4, 128, 1), (8, 2, 64, 1), (16, 1, 128, 1), (6, 3, 64, 1), (8, 8, 128, 6), (16, 16, 64, 9)])
+@pytest.mark.parametrize("Hq,Hkv,D,rep", [(4, 4, 128, 1), (8, 2, 64, 1), (16, 1, 128, 1), (6, 3, 64, 1), (8, 8, 128, 6), (16, 16, 64, 9), (32, 32, 64, 10)])
 def test_rope_attn_decode_one_launch_equals_two(ops, synth, Hq, Hkv, D, rep):
     """RoPE + append + decode attention in one launch: output and both caches equal, bit for bit, those of
     rope_kv_append followed by paged_attn_decode.  New tokens at the first and last slot of a page, in a fresh
     sequence (context 1) and deep into a sequence; MHA and grouped heads; an out-of-range sequence row."""
     kvm = load_pkg("kv_cache")
-    pos = [0, 15, 16, 31, 37, 100, 5] * rep          # rep > 1: enough (sequence, kv head) pairs for the 8- and 4-wave workgroups
+    pos = [0, 15, 16, 31, 37, 100, 5] * rep          # rep > 1: enough (sequence, kv head) pairs for the 8-wave (> 256) and 4-wave (> 2048) workgroups
     B = len(pos)
     n_pages, max_blocks = 40 * rep, 8
     perm = synth.permutation(13, "ra.pages", n_pages)
@@ -601,7 +601,7 @@ def test_rope_attn_decode_one_launch_equals_two(ops, synth, Hq, Hkv, D, rep):
     seqs = torch.tensor(list(range(B - 1)) + [B + 92], dtype=torch.int32, device=DEV)      # the last row names no sequence
     tpos = torch.tensor(pos, dtype=torch.int32, device=DEV)
     ctx = tpos + 1
-    for frag in (False, True):
+    for frag in ((False, True) if B <= 64 else (False,)):      # fragment order holds at most 64 rows
         k1, v1, q1 = k0.clone(), v0.clone(), qkv.clone()
         ops.rope_kv_append(q1, k1, v1, table, seqs, tpos, cos, sin, Hq, Hkv, D)
         want = ops.paged_attn_decode(q1, k1, v1, table, seqs, ctx, Hq, Hkv, D, frag=frag)
