@@ -31,16 +31,27 @@ class GatherMMLinear:
 
     weight [N, K] fp16 (bias-free).  Adapters are registered by name and kept stacked:
     lora_A [n_ad, r, K], lora_B [n_ad, N, r] (PEFT's `lora_A[name].weight`, `lora_B[name].weight`).
+    The branches of the reference forward (`lora_gatherbmm_linear_layer.py:6-54`) in its order: adapters disabled ->
+    base only (`:10-13`); `adapter_names` given -> base + the gathered per-request delta (`:14-20`); merged -> base
+    only, the active adapters live in the weight (`:21-22`); otherwise every active adapter is applied to every row
+    (`:23-52`; DoRA, which the reference inherits from PEFT there, is not offered).
     """
 
     def __init__(self, weight: torch.Tensor, pack: bool = True):
         self.out_features, self.in_features = weight.shape
+        self._pack = pack
         self.weight = ops.PackedWeight(weight) if pack else weight
         self.names = []
         self.scaling = {}
         self.lora_A = None
         self.lora_B = None
         self.disable_adapters = False
+        self.active_adapters = []
+        self.merged_adapters = []
+
+    @property
+    def merged(self) -> bool:
+        return bool(self.merged_adapters)
 
     def add_adapter(self, name: str, A: torch.Tensor, B: torch.Tensor, scaling: float):
         """A [r, K], B [N, r] - the PEFT parameter shapes."""
@@ -55,25 +66,70 @@ class GatherMMLinear:
         self.names.append(name)
         self.scaling[name] = float(scaling)
 
+    def set_adapter(self, names):
+        """The adapters applied to every row when a call names none (PEFT's active adapters)."""
+        names = [names] if isinstance(names, str) else list(names)
+        for n in names:
+            if n not in self.names:
+                raise ValueError(f"unknown adapter {n}")
+        self.active_adapters = names
+
+    def _rowmajor(self) -> torch.Tensor:
+        return self.weight.unpack() if isinstance(self.weight, ops.PackedWeight) else self.weight
+
+    def _add_to_weight(self, names, sign: float):
+        W = self._rowmajor().float()
+        for n in names:
+            i = self.names.index(n)
+            W += sign * self.scaling[n] * (self.lora_B[i].float() @ self.lora_A[i].float())
+        W = W.to(torch.float16)
+        self.weight = ops.PackedWeight(W) if self._pack else W
+
+    def merge(self, names=None):
+        """Fold adapters (default: the active ones) into the base weight: W += scaling * B . A, rounded to fp16."""
+        names = self.active_adapters if names is None else ([names] if isinstance(names, str) else list(names))
+        names = [n for n in names if n not in self.merged_adapters]
+        self._add_to_weight(names, 1.0)
+        self.merged_adapters += names
+
+    def unmerge(self):
+        """Subtract the merged adapters again (exact up to the fp16 rounding of the merged weight)."""
+        self._add_to_weight(self.merged_adapters, -1.0)
+        self.merged_adapters = []
+
+    def _delta(self, y, x2, ids_per_row, names):
+        """One gather-matmul call per distinct scaling among `names` (the reference folds scaling[name] into B per
+        request; the kernel takes one scaling per call, so rows of other scalings are masked)."""
+        by_scale = {}
+        for n in names:
+            by_scale.setdefault(self.scaling[n], set()).add(self.names.index(n))
+        for sc, rows in by_scale.items():
+            ids = ids_per_row if len(by_scale) == 1 else \
+                torch.where(torch.isin(ids_per_row, torch.tensor(sorted(rows), dtype=torch.int32, device=ids_per_row.device)),
+                            ids_per_row, torch.full_like(ids_per_row, -1))
+            ops.gather_mm(y, x2, self.lora_A, self.lora_B, ids, sc)
+
     def forward(self, x: torch.Tensor, adapter_names=None) -> torch.Tensor:
-        """x [B, S, K] or [B, K]; adapter_names: one name per request (len == x.shape[0]) or None.
-        Mirrors the branch structure of the reference forward: adapters disabled / no names -> base only;
-        names given -> base + gathered delta."""
+        """x [B, S, K] or [B, K]; adapter_names: one name per request (len == x.shape[0]; None or an unknown name =
+        no adapter for that request) or None."""
         shp = x.shape
         x2 = x.reshape(-1, shp[-1]).contiguous()
         y = ops.linear(x2, self.weight)
-        if self.disable_adapters or adapter_names is None or self.lora_A is None:
+        if self.disable_adapters or self.lora_A is None:
             return y.view(*shp[:-1], self.out_features)
-        if len(adapter_names) != shp[0]:
-            raise ValueError("Length of `adapter_names` should be the same as the number of inputs")
-        per_req = [self.names.index(n) if n is not None and n in self.names else -1 for n in adapter_names]
-        scal = {self.scaling[n] for n in adapter_names if n in self.scaling}
-        if len(scal) > 1:
-            raise ValueError("adapters of one call must share alpha / r")
-        rows_per_req = x2.shape[0] // shp[0]
-        ids = torch.tensor(per_req, dtype=torch.int32).repeat_interleave(rows_per_req).to(x.device)
-        if scal:
-            ops.gather_mm(y, x2, self.lora_A, self.lora_B, ids, scal.pop())
+        if adapter_names is not None:
+            if len(adapter_names) != shp[0]:
+                raise ValueError("Length of `adapter_names` should be the same as the number of inputs")
+            per_req = [self.names.index(n) if n is not None and n in self.names else -1 for n in adapter_names]
+            rows_per_req = x2.shape[0] // shp[0]
+            ids = torch.tensor(per_req, dtype=torch.int32).repeat_interleave(rows_per_req).to(x.device)
+            used = sorted({n for n in adapter_names if n in self.scaling})
+            if used:
+                self._delta(y, x2, ids, used)
+        elif not self.merged:
+            for n in self.active_adapters:             # every active adapter on every row, one after the other
+                ids = torch.full((x2.shape[0],), self.names.index(n), dtype=torch.int32, device=x.device)
+                ops.gather_mm(y, x2, self.lora_A, self.lora_B, ids, self.scaling[n])
         return y.view(*shp[:-1], self.out_features)
 
     __call__ = forward

@@ -98,6 +98,66 @@ def test_write_tensor_part(ops):
     assert np.array_equal(_np(Z), oracle.write_tensor_part_ref(_np(X), _np(Y), ids))
 
 
+# ------------------------------------------------------------------ the PEFT-seam module
+def test_gather_mm_linear_branches_of_the_reference_forward(ops, synth):
+    """`GatherMMLinear` against the restated hot branch of the reference forward (stack A and B * scaling per request,
+    two bmm, add) and its other branches: adapters disabled, active adapters on every row, merged, adapters of
+    different scaling in one call, a request without adapter."""
+    lora = load_pkg("lora")
+    Bq, S, K, N, r = 4, 6, 1024, 1024, 8
+    W = synth.normal(41, "gml.W", (N, K), 0.02, torch.float16, DEV)
+    x = synth.normal(41, "gml.x", (Bq, S, K), 1.0, torch.float16, DEV)
+    A = [synth.uniform(41, f"gml.A{i}", (r, K), 1.0 / np.sqrt(K), torch.float16, DEV) for i in range(4)]
+    Bm = [synth.normal(41, f"gml.B{i}", (N, r), 0.02, torch.float16, DEV) for i in range(4)]
+    layer = lora.GatherMMLinear(W)
+    for i in range(4):
+        layer.add_adapter(f"a{i}", A[i], Bm[i], 0.5)
+    base = _np(x).astype(np.float32) @ _np(W).astype(np.float32).T
+    base16 = _np(layer(x)).astype(np.float32)        # the fp16 base output the delta is added to (as in the fp16 reference model)
+    assert max_rel_err(base16, base) <= TOL
+    names = ["a2", "a0", "a3", "a1"]
+    got = layer(x, adapter_names=names)
+    ref = oracle.gather_bmm_hf_ref(base16, _np(x), [_np(a) for a in A], [_np(b) for b in Bm], [2, 0, 3, 1], 0.5)
+    assert got.shape == (Bq, S, N) and max_rel_err(_np(got), ref) <= TOL
+    # a request without adapter keeps the base rows
+    got = layer(x, adapter_names=["a2", None, "a3", "nope"])
+    assert torch.equal(got[1], layer(x[1:2], adapter_names=None)[0]) and not torch.equal(got[0], layer(x[0:1])[0])
+    # disabled: base only
+    layer.disable_adapters = True
+    assert max_rel_err(_np(layer(x, adapter_names=names)), base) <= TOL
+    layer.disable_adapters = False
+    # active adapters on every row, then the same adapters merged into the weight
+    layer.set_adapter(["a1", "a3"])
+    want, want16 = base16.copy(), base16.copy()
+    for i in (1, 3):                                  # the layer adds one adapter after the other into its fp16 output
+        d = 0.5 * (_np(x).astype(np.float32) @ _np(A[i]).astype(np.float32).T @ _np(Bm[i]).astype(np.float32).T)
+        want += d
+        want16 = (want16 + d).astype(np.float16).astype(np.float32)
+    assert max_rel_err(_np(layer(x)), want16) <= TOL
+    layer.merge()
+    Wm = W.float()
+    for i in (1, 3):
+        Wm = Wm + 0.5 * (Bm[i].float() @ A[i].float())
+    assert layer.merged and torch.equal(layer.weight.unpack(), Wm.half())     # the merged weight, rounded to fp16 once
+    assert max_rel_err(_np(layer(x)), _np(x).astype(np.float32) @ _np(Wm.half()).astype(np.float32).T) <= TOL
+    assert max_rel_err(_np(layer(x)), want, floor=5e-2) <= 5 * TOL             # close to the unmerged result
+    layer.unmerge()
+    # the weight went through two more fp16 roundings: back to the base output up to that noise
+    assert not layer.merged and max_rel_err(_np(layer(x, adapter_names=[None] * Bq)), base, floor=5e-2) <= 5 * TOL
+    # two scalings in one call
+    layer2 = lora.GatherMMLinear(W)
+    layer2.add_adapter("p", A[0], Bm[0], 0.5)
+    layer2.add_adapter("q", A[1], Bm[1], 2.0)
+    got = layer2(x, adapter_names=["p", "q", "q", "p"])
+    xs = _np(x).astype(np.float32)
+    want = base16.copy()
+    for b, (i, sc) in enumerate([(0, 0.5), (1, 2.0), (1, 2.0), (0, 0.5)]):
+        want[b] += sc * (xs[b] @ _np(A[i]).astype(np.float32).T @ _np(Bm[i]).astype(np.float32).T)
+    assert max_rel_err(_np(got), want) <= TOL
+    with pytest.raises(ValueError):
+        layer(x, adapter_names=["a0"])
+
+
 # ------------------------------------------------------------------ base linear
 @pytest.mark.parametrize("T,K,N", [(32, 4096, 4096), (32, 4096, 12288), (32, 11008, 4096), (32, 4096, 22016),
                                    (64, 4096, 4096), (4, 1024, 3072), (1, 1024, 1024), (17, 2752, 1024), (5, 64, 36)])
