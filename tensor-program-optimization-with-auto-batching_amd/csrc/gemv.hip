@@ -563,7 +563,7 @@ extern "C" int mlora_gemv_frag_acc_ksplit(float* y, float* y2, float* part, int 
   MLORA_CHECK(N_ext >= 0 && N_ext % 4 == 0 && (N_ext == 0 || (y2 && N_main % 16 == 0)), MLORA_ERR_INVALID,
               "gemv_frag_acc_ksplit: appended rows need y2, N_ext %% 4 == 0 and N_main %% 16 == 0 (N_main=%d N_ext=%d)", N_main, N_ext);
   MLORA_CHECK(!(A && N_ext), MLORA_ERR_INVALID, "gemv_frag_acc_ksplit: shrink units and appended rows are exclusive");
-  MLORA_CHECK(ks >= 1 && ks <= 4 && (ks == 1 || part) && (K / KSTEP) / ks >= 8, MLORA_ERR_INVALID,
+  MLORA_CHECK(ks >= 1 && ks <= 4 && (ks == 1 || (part && (K / KSTEP) / ks >= 8)), MLORA_ERR_INVALID,
               "gemv_frag_acc_ksplit: ks=%d outside 1..4, too many slices for K=%d, or no partials buffer", ks, K);
   if (A)
     if (int e = check_shrink_args("gemv_frag_acc_ksplit", v_part, A, n_proj, tok_adapter, r, n_ad)) return e;

@@ -714,7 +714,8 @@ def test_rope_append_page_row_writer_equals_per_token_kernel(ops, synth, Hq, Hkv
 
 # ------------------------------------------------------------------ K-split accumulating GEMV + RMSNorm that sums the partials
 @pytest.mark.parametrize("T,K,N,ks_expected", [(32, 11008, 4096, 4), (32, 4096, 4096, 4), (9, 4096, 4096, 4), (32, 4096, 4352, 3),
-                                               (32, 2048, 1024, 2), (40, 11008, 4096, 4), (64, 4096, 4096, 4), (40, 4096, 4352, 3), (32, 1024, 1024, 1)])
+                                               (32, 2048, 1024, 2), (40, 11008, 4096, 4), (64, 4096, 4096, 4), (40, 4096, 4352, 3), (32, 1024, 1024, 1),
+                                               (8, 128, 256, 1)])
 def test_gemv_ksplit_partials_summed_by_rmsnorm(ops, synth, T, K, N, ks_expected):
     """o_proj / down_proj shapes: slice 0 accumulates into the residual, the RMSNorm adds the other slices in order and
     stores the row back.  Checked against the fp64 product and against the unsplit kernels."""
