@@ -80,9 +80,11 @@ class DecodeSession:
 
 
 class NativeDecodeSession:
-    """The same fixed-batch greedy decode, one `mlora_decode_step` call per step (one adapter type), optionally
-    replayed from a captured graph.  The graph is re-used as long as the batch does not change; the host only
-    grows the block table when a sequence crosses a page boundary."""
+    """The same fixed-batch greedy decode, one `mlora_decode_step` call per step, optionally replayed from a
+    captured graph.  The graph is re-used as long as the batch does not change; the host only grows the block table
+    when a sequence crosses a page boundary.  `tid` names one adapter type (`adapter_ids` = weight ids, -1 = none) or,
+    as a tuple, several types of equal scaling served from their padded union (`adapter_ids` = rows of
+    `model.lora_union(tid)`, see `model.union_rows`)."""
 
     def __init__(self, model, kv, seq_ids, adapter_ids, first_tokens, tid=0, use_graph=True, dense_lora=None, fuse_silu=True, ksplit=True):
         import ctypes as C
@@ -94,13 +96,22 @@ class NativeDecodeSession:
         T = len(self.seq_ids)
         if T > 64:
             raise ValueError("NativeDecodeSession handles at most 64 sequences per step")
-        lt = model.lora_types[tid] if adapter_ids is not None and model.lora_types else None
+        lt = None
+        if adapter_ids is not None and model.lora_types:
+            lt = model.lora_union(tid)[0] if isinstance(tid, tuple) else model.lora_types[tid]
         i32 = lambda a: torch.as_tensor(np.asarray(a, dtype=np.int32)).to(dev)
         self.tokens = i32(first_tokens)
         self.rows = i32([kv.slot[q] for q in self.seq_ids])
         self.pos = i32([kv.lens[q] for q in self.seq_ids])
         self.ctx = self.pos + 1
-        self.tok_adapter = i32(lt.rows(np.asarray(adapter_ids, dtype=np.int32).reshape(-1))) if lt is not None else None
+        self.tok_adapter = None
+        if lt is not None:
+            ids = np.asarray(adapter_ids, dtype=np.int32).reshape(-1)
+            if not isinstance(tid, tuple):
+                ids = lt.rows(ids)                       # weight ids -> table rows
+            elif ids.size != T or (ids.size and (ids.min() < -1 or ids.max() >= lt.n_adapters)):
+                raise ValueError("NativeDecodeSession: bad union rows")
+            self.tok_adapter = i32(ids)
         H, I, V = s.hidden_size, s.intermediate_size, s.vocab_size
         f16, f32 = torch.float16, torch.float32
         fe = _lib.lib().mlora_frag_activation_elems

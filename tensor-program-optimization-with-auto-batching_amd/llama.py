@@ -124,16 +124,64 @@ class LlamaForCausalLM:
             self._il_cache = cache
         return cache
 
-    def dense_lora_weights(self, tid: int = 0):
-        """Per layer, the qkv / o / down weights with the stacked A tables of adapter type `tid` appended as extra
-        rows ([n_ad * r, K] per adapted projection; q, k, v slots always present for qkv, zero when not adapted),
-        in fragment order.  Cached; costs one more copy of those matrices."""
+    def lora_union(self, tids):
+        """-> (type, {tid: first table row}): one set of tables that serves the adapter types `tids` in one launch.
+        For a single type that is the type itself.  For several, the ranks are zero-padded to the largest (the
+        reference's padded strategy, `tvm/lora_only/case_study/multiple_ranks.py:66-95`) and the adapters of all
+        types are stacked, type after type; projections a type does not adapt are zero tables.  Zero rows of A give
+        v = 0 exactly and zero columns of B add 0 to every sum, so each token gets the delta of its own unpadded
+        adapter bit for bit.  The types must share one scaling (alpha / r).  Cached; costs a copy of the tables."""
+        tids = tuple(int(t) for t in tids)
+        if len(tids) == 1:
+            return self.lora_types[tids[0]], {tids[0]: 0}
+        cache = getattr(self, "_union_cache", None)
+        if cache is None:
+            cache = self._union_cache = {}
+        if tids in cache:
+            return cache[tids]
+        types = [self.lora_types[t] for t in tids]
+        if any(lt.scaling != types[0].scaling for lt in types):
+            raise ValueError("lora_union: the adapter types differ in scaling")
+        rmax = max(lt.r for lt in types)
+        base, n = {}, 0
+        for t, lt in zip(tids, types):
+            base[t] = n
+            n += lt.n_adapters
+        union = LoraType(rmax, types[0].scaling, n)
+        for key in sorted({k for lt in types for k in lt.tables}):
+            ref = next(lt.tables[key] for lt in types if key in lt.tables)
+            K, N = ref[0].shape[2], ref[1].shape[1]
+            A = torch.zeros((n, rmax, K), dtype=torch.float16, device=self.device)
+            B = torch.zeros((n, N, rmax), dtype=torch.float16, device=self.device)
+            for t, lt in zip(tids, types):
+                tab = lt.tables.get(key)
+                if tab is not None:
+                    A[base[t]:base[t] + lt.n_adapters, :lt.r] = tab[0]
+                    B[base[t]:base[t] + lt.n_adapters, :, :lt.r] = tab[1]
+            union.add(key[0], key[1], A, B)
+        cache[tids] = (union, base)
+        return cache[tids]
+
+    def union_rows(self, tids, T, pairs):
+        """Table rows [T] (int32, host) of a batch in the tables of `lora_union(tids)`; `pairs` as for `_ids`."""
+        _, base = self.lora_union(tids)
+        full = np.full(T, -1, dtype=np.int32)
+        for tid, ids in self._ids(T, pairs, host=True).items():
+            full = np.where(ids >= 0, ids + base[tid], full)
+        return full.astype(np.int32)
+
+    def dense_lora_weights(self, tid=0):
+        """Per layer, the qkv / o / down weights with the stacked A tables of adapter type `tid` (or of the union of
+        a tuple of types) appended as extra rows ([n_ad * r, K] per adapted projection; q, k, v slots always present
+        for qkv, zero when not adapted), in fragment order.  Cached; costs one more copy of those matrices."""
         cache = getattr(self, "_dense_cache", None)
         if cache is None:
             cache = self._dense_cache = {}
+        if isinstance(tid, tuple) and len(tid) == 1:
+            tid = tid[0]
         if tid in cache:
             return cache[tid]
-        lt = self.lora_types[tid]
+        lt = self.lora_union(tid)[0] if isinstance(tid, tuple) else self.lora_types[tid]
         out = []
         for l, L in enumerate(self.layers):
             ent = {}
@@ -316,8 +364,8 @@ class LlamaForCausalLM:
         return None
 
     # ------------------------------------------------------------------ reference entry points
-    def _ids(self, T, pairs):
-        """{tid: (positions | None, wids)} -> {tid: ids [T] int32 on device, -1 where the type is absent}."""
+    def _ids(self, T, pairs, host=False):
+        """{tid: (positions | None, wids)} -> {tid: ids [T] int32 on device (host: numpy), -1 where the type is absent}."""
         out = {}
         for tid, (sids, wids) in pairs.items():
             full = np.full(T, -1, dtype=np.int32)
@@ -329,7 +377,7 @@ class LlamaForCausalLM:
                 if p.size != w.size or (p.size and (p.min() < 0 or p.max() >= T)):
                     raise ValueError("sids / wids mismatch")
                 full[p] = w
-            out[tid] = torch.from_numpy(full).to(self.device)
+            out[tid] = full if host else torch.from_numpy(full).to(self.device)
         return out
 
     def _last_rows(self, kv):

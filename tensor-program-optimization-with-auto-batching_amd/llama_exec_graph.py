@@ -30,6 +30,11 @@ class LlamaExecConfig:
     # mix adapter types through the per-operator step recorded into a graph.  Same tokens: the native step with
     # ids-based LoRA shrink is bit-identical to the per-operator path.
     native_decode: bool = True
+    # Let the native step compute the LoRA shrink of all adapters as extra rows of the base GEMV (the fastest form
+    # while the adapters are few and low-rank: taken when every rank is at most 16).  It then also serves batches
+    # that mix adapter types of one scaling, and rows without adapter, from the types' zero-padded union.  The fp32
+    # summation order of x . A^T differs from the per-operator path, so a greedy token can differ at a near tie.
+    dense_lora: bool = False
 
 
 class LlamaExecGraph(ExecGraph):
@@ -129,9 +134,9 @@ class LlamaExecGraph(ExecGraph):
         seqs = self.check_seqs_finished(seqs, outputs)
         while seqs:
             method, params = self.seq_info.get_decode_method(seqs)
-            single = method == "decode_no_adapter" or method.startswith("decode_a")
             if getattr(self.exec_config, "native_decode", False) and len(seqs) <= 64:
-                seqs = self._decode_native(seqs, outputs, method, params) if single \
+                dense = self._dense_ok(method)
+                seqs = self._decode_native(seqs, outputs, method, params, dense) if dense or not method.startswith("mixed_decode") \
                     else self._decode_session(seqs, outputs, method, params)
                 continue
             tokens = torch.tensor([outputs[sid][-1] for sid in seqs], dtype=torch.int32)
@@ -148,16 +153,23 @@ class LlamaExecGraph(ExecGraph):
         for i, sid in enumerate(ordered):
             op.output_vars[original_positions[i]].var = np.asarray(outputs[sid], dtype=np.int64)
 
-    def _decode_native(self, seqs, outputs, method, params):
+    def _decode_native(self, seqs, outputs, method, params, dense=False):
         """Decode this batch with the native step until its composition changes (a sequence reaches its length
         limit or emits EOS); returns the sequences still running.  Without an EOS id the number of steps until
         the next length limit is known in advance and the tokens come back in one copy."""
         from .decode_session import NativeDecodeSession
-        tid = int(method[len("decode_a"):]) if method != "decode_no_adapter" else 0
-        wids = params[0] if params else None
+        if method.startswith("mixed_decode"):
+            # several types, or one type beside rows without adapter: rows of the types' padded union, -1 = no adapter
+            tids = self._method_tids(method)
+            pairs = {t: (params[2 * i], params[2 * i + 1]) for i, t in enumerate(tids)}
+            tid = tuple(tids)
+            wids = self.vm.union_rows(tids, len(seqs), pairs)
+        else:
+            tid = int(method[len("decode_a"):]) if method != "decode_no_adapter" else 0
+            wids = params[0] if params else None
         last = [outputs[sid][-1] for sid in seqs]
         ahead = min(self.seq_info.get_max_gen_len(sid) - len(outputs[sid]) for sid in seqs)
-        sess = NativeDecodeSession(self.vm, self.kv_cache, seqs, wids, last, tid=tid, use_graph=ahead >= 8, dense_lora=False)
+        sess = NativeDecodeSession(self.vm, self.kv_cache, seqs, wids, last, tid=tid, use_graph=ahead >= 8, dense_lora=None if dense else False)
         if self.eos_token_id is None and not self.measure:
             for _ in range(ahead):
                 sess.step(keep_history=True)
@@ -176,12 +188,23 @@ class LlamaExecGraph(ExecGraph):
             if len(left) != len(seqs):
                 return left
 
+    @staticmethod
+    def _method_tids(method):
+        return [int(t) for t in re.findall(r"_a(\d+)", method)]
+
+    def _dense_ok(self, method):
+        """Whether the native step with the dense shrink serves this entry point: asked for in the configuration,
+        ranks at most 16, and one scaling over its adapter types (they are served from their padded union)."""
+        types = [self.vm.lora_types[t] for t in self._method_tids(method)]
+        return bool(getattr(self.exec_config, "dense_lora", False) and types and max(lt.r for lt in types) <= 16
+                    and len({lt.scaling for lt in types}) == 1)
+
     def _decode_session(self, seqs, outputs, method, params):
         """A batch that mixes adapter types (`mixed_decode_a{i}_a{j}...`): the per-operator step with the tokens,
         positions and context lengths kept on the device, replayed from a graph when enough steps lie ahead.  Same
         kernels in the same order as the call-per-step path, so the same tokens."""
         from .decode_session import DecodeSession
-        tids = [int(t) for t in re.findall(r"_a(\d+)", method)]
+        tids = self._method_tids(method)
         pairs = {tid: (params[2 * i], params[2 * i + 1]) for i, tid in enumerate(tids)}
         last = [outputs[sid][-1] for sid in seqs]
         ahead = min(self.seq_info.get_max_gen_len(sid) - len(outputs[sid]) for sid in seqs)

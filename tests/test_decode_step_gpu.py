@@ -174,3 +174,52 @@ def test_native_step_at_most_16_requests():
     d, _, ld = _run(model, wl, prompts, ids, "dense", 5, synth, run_steps=1)
     err = float((ld - lg).abs().max() / lg.std())
     assert err <= 1e-2, err
+
+
+@pytest.mark.parametrize("ranks,dense", [((8, 16), False), ((8, 16), True), ((32, 8, 16), False)])
+def test_native_step_over_the_padded_union_of_adapter_types(ranks, dense):
+    """Several adapter types of one scaling in one batch, served by the native step from their zero-padded union
+    (the reference's padded strategy, `tvm/lora_only/case_study/multiple_ranks.py:66-95`), beside rows without
+    adapter.  The padding adds exact zeros: with the ids-based shrink the tokens and the whole K cache equal those of
+    the per-operator path on the unpadded tables bit for bit; with the dense shrink (x . A^T by the matrix cores,
+    another fp32 summation order) the first step's logits and keys agree with the ids-based ones to rounding noise."""
+    synth, llama, dsm = load_pkg("synth"), load_pkg("llama"), load_pkg("decode_session")
+    wl = synth.config3(num_layers=2, batch=20, prompt_len=24)
+    all7 = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")
+    targets = (("q_proj", "k_proj", "v_proj", "o_proj"), ("q_proj", "v_proj", "down_proj"), all7)
+    specs = [synth.LoraSpec(r=r, alpha=r / 2, n_adapters=3 + i, targets=targets[i]) for i, r in enumerate(ranks)]
+    model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, specs, DEV)
+    B = wl.batch
+    steps = 1 if dense else 10
+    tid = np.array([(b % (len(ranks) + 1)) - 1 for b in range(B)])              # -1 = no adapter
+    ids = {t: np.where(tid == t, np.arange(B) % specs[t].n_adapters, -1).astype(np.int32) for t in range(len(ranks))}
+    prompts = synth.randint(wl.seed, "union.prompts", (B, wl.prompt_len), wl.shape.vocab_size).numpy()
+    first = np.arange(B, dtype=np.int32) + 7
+    tids = tuple(range(len(ranks)))
+    out = {}
+    for kind in ("dense", "native") if dense else ("py", "native"):
+        blocks = -(-(wl.prompt_len + steps + 2) // 16)
+        kv = model.create_paged_kv_cache(B, B * blocks * 16, wl.prompt_len, 16, free_pages=synth.permutation(wl.seed, "union.pages", B * blocks),
+                                         max_seq_len=blocks * 16)
+        for b in range(B):
+            kv.add_sequence(b)
+        for b in range(B):           # prefill through the per-operator path, one request at a time
+            kv.begin_forward([b], [wl.prompt_len])
+            rows = {t: (None, np.full(wl.prompt_len, ids[t][b], dtype=np.int32)) for t in ids}
+            model.forward(model.embed(torch.from_numpy(np.ascontiguousarray(prompts[b]))), kv, model._ids(wl.prompt_len, rows),
+                          model._last_rows(kv))
+            kv.end_forward()
+        if kind == "py":
+            s = dsm.DecodeSession(model, kv, list(range(B)), ids, first)
+        else:
+            s = dsm.NativeDecodeSession(model, kv, list(range(B)), model.union_rows(tids, B, {t: (None, ids[t]) for t in ids}), first,
+                                        tid=tids, use_graph=not dense, dense_lora=(kind == "dense"))
+            assert s.dense_lora == (kind == "dense")
+        toks = [s.step().cpu().numpy().copy() for _ in range(steps)]
+        out[kind] = (np.stack(toks), kv.k.clone(), None if kind == "py" else s.buf["logits"].view(B, -1).clone())
+    if not dense:
+        assert np.array_equal(out["py"][0], out["native"][0])
+        assert torch.equal(out["py"][1], out["native"][1])
+    else:
+        for a, b in ((out["dense"][1].float(), out["native"][1].float()), (out["dense"][2], out["native"][2])):
+            assert (a - b).abs().max().item() <= 2e-3 * b.abs().max().item()

@@ -152,6 +152,36 @@ def test_mixed_adapter_types_graph_replayed_session_equals_call_per_step(c1):
     assert got == want
 
 
+def test_mixed_adapter_types_through_the_dense_native_step(c1):
+    """`LlamaExecConfig.dense_lora`: the mixed batch of two adapter types (ranks 8 and 16, one scaling) and requests
+    without adapter decodes through the native step over the types' padded union, the shrink done by the base GEMV's
+    matrix-core rows.  Checked against the oracle like the per-operator path: identical tokens up to the first step
+    the oracle itself decides by a near tie."""
+    wl, _, _ = c1
+    synth = load_pkg("synth")
+    spec1 = synth.LoraSpec(r=16, alpha=8.0, n_adapters=3, targets=("q_proj", "v_proj", "o_proj"))
+    specs = [wl.lora, spec1]
+    assert wl.lora.r == 8 and wl.lora.scaling == spec1.scaling
+    model = hip_model(wl, specs)
+    ref = oracle_model(wl, "mixed", specs)
+    B, P, max_gen_len = 6, 24, 12
+    prompts = synth.randint(13, "mixedd.prompts", (B, P), wl.shape.vocab_size).numpy()
+    tids = [0, 1, -1, 1, 0, -1]
+    wids = np.array([2, 0, -1, 2, 3, -1], dtype=np.int32)
+    tok_adapter = {"a0": np.where(np.array(tids) == 0, wids, -1).astype(np.int32),
+                   "a1": np.where(np.array(tids) == 1, wids, -1).astype(np.int32)}
+    n_pages = B * 4
+    perm = synth.permutation(13, "mixedd.pages", n_pages)
+    exp, margins, scales = oracle.greedy_generate_ref(ref, prompts, tok_adapter, max_gen_len, n_pages, wl.page_size,
+                                                      perm, return_logits=True)
+    wl2 = synth.Workload("mixedd", 13, wl.shape, wl.lora, batch=B, prompt_len=P, gen_len=max_gen_len)
+    got, batcher = run_hip_generate(model, wl2, prompts, wids, max_gen_len, perm, tids=[max(t, 0) for t in tids], dense_lora=True)
+    assert batcher.graph._dense_ok("mixed_decode_a0_a1") and (0, 1) in model._dense_cache
+    for b in range(B):
+        i = next((i for i in range(max_gen_len) if got[b][i] != exp[b][i]), None)
+        assert i is None or margins[b][i] < 2e-2 * scales[b][i], (b, i, got[b], exp[b], margins[b])
+
+
 def test_per_request_max_gen_len_and_eos(c1):
     """The batch shrinks as sequences hit their own max_gen_len or EOS; outputs keep request order."""
     wl, model, prompts = c1
