@@ -97,6 +97,8 @@ class LlamaAutoBatcherClass:
             if not ok:
                 raise RuntimeError(f"adapter type a{tid} ({cfg}) is not loaded in the model")
         if fuse_decode:
+            if getattr(self.exec_config, "batch_prefill", False) and "prefill" not in self.graph.batchable_op_types:
+                self.graph.batchable_op_types += ("prefill",)
             self.graph.fuse_batchable_ops()
         self.graph.set_exec_vars(self.model, self.model.device, None, self.tokenizer, self.seq_info,
                                  self.exec_config, eos_token_id=self.eos_token_id, free_pages=self.free_pages)

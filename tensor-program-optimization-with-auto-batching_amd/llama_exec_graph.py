@@ -35,6 +35,10 @@ class LlamaExecConfig:
     # that mix adapter types of one scaling, and rows without adapter, from the types' zero-padded union.  The fp32
     # summation order of x . A^T differs from the per-operator path, so a greedy token can differ at a near tie.
     dense_lora: bool = False
+    # Prefill the prompts of all requests in one forward pass instead of one pass per request (the reference's way).
+    # Same arithmetic per token, but larger token counts take other GEMM kernels and summation orders, so the first
+    # token of a request can differ from the per-request prefill at a near tie.
+    batch_prefill: bool = False
 
 
 class LlamaExecGraph(ExecGraph):
@@ -103,6 +107,8 @@ class LlamaExecGraph(ExecGraph):
         op.output_vars[0].var = ids
 
     def execute_prefill(self, op):
+        if len(op.seqids) > 1:
+            return self._prefill_batch(op)
         assert len(op.input_vars) == 1 and len(op.output_vars) == 1 and len(op.seqids) == 1, \
             "prefill node must have exactly 1 input var, 1 output var and 1 seqid"
         sid = op.seqids[0]
@@ -119,6 +125,35 @@ class LlamaExecGraph(ExecGraph):
         self.kv_cache.end_forward()
         self._toc(ev)
         op.output_vars[0].var = int(ops.argmax(logits).cpu()[0])
+
+    def _prefill_batch(self, op):
+        """The prompts of several requests in one forward pass (`LlamaExecConfig.batch_prefill`; the reference
+        prefills one sequence per call, `:58-92`): the prompts are concatenated in request order, every token carries
+        its request's adapter, attention stays inside each request's own pages, and the logits are taken at each
+        prompt's last token."""
+        n = len(op.seqids)
+        assert len(op.input_vars) == n and len(op.output_vars) == n, "prefill node needs one input and one output var per sequence"
+        prompts = [np.asarray(v.var, dtype=np.int32).reshape(-1) for v in op.input_vars]
+        lens = [int(p.size) for p in prompts]
+        T = sum(lens)
+        per_type = {}                                           # adapter type -> weight id per token, -1 elsewhere
+        start = 0
+        for sid, L in zip(op.seqids, lens):
+            self.kv_cache.add_sequence(sid)
+            adapter = self.seq_info.get_adapter_info(sid)
+            if adapter is not None:
+                per_type.setdefault(adapter["tid"], np.full(T, -1, dtype=np.int32))[start:start + L] = adapter["wid"]
+            start += L
+        hidden = self.vm["embed"](torch.from_numpy(np.ascontiguousarray(np.concatenate(prompts))))
+        ev = self._tic()
+        self.kv_cache.begin_forward(list(op.seqids), lens)
+        ids = self.vm._ids(T, {tid: (None, wids) for tid, wids in sorted(per_type.items())})
+        logits = self.vm.forward(hidden, self.kv_cache, ids, self.vm._last_rows(self.kv_cache))
+        self.kv_cache.end_forward()
+        self._toc(ev)
+        first = ops.argmax(logits).cpu().numpy()
+        for i in range(n):
+            op.output_vars[i].var = int(first[i])
 
     def check_seqs_finished(self, seqs_2_decode, outputs):
         return [sid for sid in seqs_2_decode

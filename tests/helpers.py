@@ -30,7 +30,7 @@ def n_pages_for(wl, max_gen_len):
 
 
 def run_hip_generate(model, wl, prompts, adapter_ids, max_gen_len, free_pages, tids=None, max_gen_lens=None,
-                     eos_token_id=None, native_decode=True, dense_lora=False):
+                     eos_token_id=None, native_decode=True, dense_lora=False, batch_prefill=False):
     """Drive the auto-batching front end the way `tvm/llama_auto_batcher/main.py:37-44` does."""
     ab = load_pkg("auto_batcher")
     lora = load_pkg("lora")
@@ -38,7 +38,8 @@ def run_hip_generate(model, wl, prompts, adapter_ids, max_gen_len, free_pages, t
     batcher = ab.LlamaAutoBatcherClass()
     batcher.set_model(model)
     batcher.set_exec_config(xg.LlamaExecConfig(max_prompt_len=wl.prompt_len, max_gen_len=max_gen_len, page_size=wl.page_size,
-                                               native_decode=native_decode, dense_lora=dense_lora))
+                                               native_decode=native_decode, dense_lora=dense_lora,
+                                               batch_prefill=batch_prefill))
     batcher.set_free_pages(free_pages)
     batcher.set_eos_token_id(eos_token_id)
     results = []

@@ -80,6 +80,25 @@ def test_exec_graph_fusion_levels():
     assert all(v.ops == [dec] for v in dec.input_vars)
 
 
+def test_exec_graph_fuses_prefill_too_when_it_is_batchable():
+    """With "prefill" among the batchable operation types (what `LlamaExecConfig.batch_prefill` asks compile() for),
+    the prefills of all requests fold into one operation whose variables and sequence ids stay aligned, and the
+    decode fusion after it is unchanged."""
+    ab = load_pkg("auto_batcher").LlamaAutoBatcherClass()
+    outs = [ab.generate(ab.create_var(np.arange(3 + i)), max_gen_len=4) for i in range(5)]
+    g = ab.graph
+    g.batchable_op_types += ("prefill",)
+    g.fuse_batchable_ops()
+    assert g.get_max_batch_sizes() == {"prefill": 5, "decode": 5}
+    ops_levels = [[n.op_type for n in lvl] for lvl in g.levels() if lvl and hasattr(lvl[0], "op_type")]
+    assert ops_levels == [["encode_prompt"] * 5, ["prefill"], ["decode"], ["decode_answer"] * 5]
+    pre = next(n for n in g.op_nodes if n.op_type == "prefill")
+    dec = next(n for n in g.op_nodes if n.op_type == "decode")
+    assert pre.seqids == dec.seqids == list(range(5))
+    assert [v.id for v in pre.output_vars] == [v.id for v in dec.input_vars]
+    assert [v.ops[0].output_vars[0] for v in dec.output_vars] == outs
+
+
 def test_exec_graph_unfused_keeps_separate_decodes():
     ab = load_pkg("auto_batcher").LlamaAutoBatcherClass()
     for _ in range(3):

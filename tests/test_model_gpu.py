@@ -182,6 +182,51 @@ def test_mixed_adapter_types_through_the_dense_native_step(c1):
         assert i is None or margins[b][i] < 2e-2 * scales[b][i], (b, i, got[b], exp[b], margins[b])
 
 
+def test_batched_prefill_of_all_requests_in_one_pass(c1):
+    """`LlamaExecConfig.batch_prefill`: the prefill operations of all requests fuse into one forward pass over the
+    concatenated prompts (two adapter types and requests without adapter).  Tokens against the oracle, which prefills
+    request by request: identical up to the first near tie.  Then ragged prompts (1 to 70 tokens): the K and V pages
+    written by the single pass equal those of the per-request prefill to rounding noise, same pages."""
+    wl, _, _ = c1
+    synth = load_pkg("synth")
+    spec1 = synth.LoraSpec(r=16, alpha=8.0, n_adapters=3, targets=("q_proj", "v_proj", "o_proj"))
+    specs = [wl.lora, spec1]
+    model = hip_model(wl, specs)
+    ref = oracle_model(wl, "mixed", specs)
+    B, P, max_gen_len = 6, 24, 8
+    prompts = synth.randint(14, "bp.prompts", (B, P), wl.shape.vocab_size).numpy()
+    tids = [0, 1, -1, 1, 0, -1]
+    wids = np.array([2, 0, -1, 2, 3, -1], dtype=np.int32)
+    tok_adapter = {"a0": np.where(np.array(tids) == 0, wids, -1).astype(np.int32),
+                   "a1": np.where(np.array(tids) == 1, wids, -1).astype(np.int32)}
+    n_pages = B * 4
+    perm = synth.permutation(14, "bp.pages", n_pages)
+    exp, margins, scales = oracle.greedy_generate_ref(ref, prompts, tok_adapter, max_gen_len, n_pages, wl.page_size,
+                                                      perm, return_logits=True)
+    wl2 = synth.Workload("bp", 14, wl.shape, wl.lora, batch=B, prompt_len=P, gen_len=max_gen_len)
+    got, batcher = run_hip_generate(model, wl2, prompts, wids, max_gen_len, perm, tids=[max(t, 0) for t in tids], batch_prefill=True)
+    assert batcher.graph.get_max_batch_sizes() == {"decode": B, "prefill": B}
+    for b in range(B):
+        i = next((i for i in range(max_gen_len) if got[b][i] != exp[b][i]), None)
+        assert i is None or margins[b][i] < 2e-2 * scales[b][i], (b, i, got[b], exp[b], margins[b])
+    # ragged prompts, prefill only (the first token already counts towards max_gen_len = 1)
+    lens = [1, 70, 17, 5, 64, 33]
+    ragged = [synth.randint(15, f"bp.ragged{i}", (L,), wl.shape.vocab_size).numpy() for i, L in enumerate(lens)]
+    wl3 = synth.Workload("bpr", 15, wl.shape, wl.lora, batch=B, prompt_len=max(lens), gen_len=1)
+    perm = synth.permutation(15, "bpr.pages", B * 6)
+    caches = []
+    for batch_prefill in (False, True):
+        tok, batcher = run_hip_generate(model, wl3, ragged, wids, 1, perm, tids=[max(t, 0) for t in tids], batch_prefill=batch_prefill)
+        kv = batcher.graph.kv_cache
+        caches.append((kv.k.float().clone(), kv.v.float().clone(), kv.block_table.clone(), tok))
+    assert torch.equal(caches[0][2], caches[1][2])
+    for a, b in zip(caches[0][:2], caches[1][:2]):
+        live = a != 0
+        assert torch.equal(live, b != 0)                  # the same slots were written
+        assert (a - b).abs().max().item() <= 2e-3 * a.abs().max().item()
+    assert sum(x == y for x, y in zip(caches[0][3], caches[1][3])) >= B - 1
+
+
 def test_per_request_max_gen_len_and_eos(c1):
     """The batch shrinks as sequences hit their own max_gen_len or EOS; outputs keep request order."""
     wl, model, prompts = c1
