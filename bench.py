@@ -368,6 +368,74 @@ def bench_c5_decode(args, synth, llama):
                      "frac": step_bytes / dt / 1e9 / HBM_PEAK_GBS, "traffic": None, "step_algorithmic_gb": step_bytes / 1e9}}))
 
 
+def bench_c1_generate(args, synth, llama):
+    """The reference's own CPU-runnable case, end to end through the auto-batching front end: 4 requests, each with
+    its own rank-8 adapter, 128-token prompts, 32 greedy tokens per request (per-request prefill, batched decode).
+    A step = one whole generate pass (requests registered, graph fused and executed).  The CPU baseline is the
+    numpy oracle's `greedy_generate_ref` on the same prompts, timed once; the token ids of both are compared."""
+    import torch
+    ab, xg, lora = _mod("auto_batcher"), _mod("llama_exec_graph"), _mod("lora")
+    dev = "cuda:0"
+    wl = synth.config1()
+    s = wl.shape
+    model = llama.LlamaForCausalLM.from_synthetic(wl.seed, s, [wl.lora], dev)
+    prompts = synth.prompts(wl)
+    prompts = prompts.numpy() if hasattr(prompts, "numpy") else np.asarray(prompts)
+    B, G = wl.batch, wl.gen_len
+    n_pages = B * (-(-(wl.prompt_len + G) // wl.page_size) + 1)
+    perm = synth.permutation(wl.seed, "c1.bench.pages", n_pages)
+
+    def one_pass():
+        b = ab.LlamaAutoBatcherClass()
+        b.set_model(model)
+        b.set_exec_config(xg.LlamaExecConfig(max_prompt_len=wl.prompt_len, max_gen_len=G, page_size=wl.page_size,
+                                             dense_lora=args.dense_lora, batch_prefill=args.batch_prefill))
+        b.set_free_pages(perm)
+        b.set_eos_token_id(None)
+        outs = []
+        for i in range(B):
+            v = b.create_var(np.asarray(prompts[i], dtype=np.int32))
+            b.set_adapter(lora.LoraConfig(r=wl.lora.r, alpha=wl.lora.scaling * wl.lora.r), wid=int(wl.adapter_ids[i]))
+            outs.append(b.generate(v, max_gen_len=G))
+        b.compile()
+        b.execute()
+        return [list(map(int, o.var)) for o in outs]
+
+    warm = min(args.warmup, 3)
+    steps = min(args.steps, 20)
+    for _ in range(warm):
+        got = one_pass()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        got = one_pass()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    out = {
+        "metric": "end-to-end generate tok/s, 2-layer plumbing model, 4 requests x 4 rank-8 adapters, 128-token prompts, 32 greedy tokens",
+        "value": B * G / dt, "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": dt * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": wl.name, "layers": s.num_hidden_layers, "hidden": s.hidden_size, "batch": B,
+                   "prompt_len": wl.prompt_len, "gen_len": G, "host_loop": "auto-batching front end, native decode step",
+                   "dense_lora": args.dense_lora, "batch_prefill": args.batch_prefill},
+        "roofline": {"kernel": "whole generate pass (4 prefills + 31 decode steps; launch- and host-bound at this size)", "bound": "hbm",
+                     "achieved": model.weight_bytes_per_step() * (B + G - 1) / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": model.weight_bytes_per_step() * (B + G - 1) / dt / 1e9 / HBM_PEAK_GBS, "traffic": None}}
+    if not args.no_cpu_baseline:
+        import oracle
+        w = {k: v.float().numpy() for k, v in synth.base_weights(wl.seed, s, torch.float16, "cpu").items()}
+        lw = {k: v.float().numpy() for k, v in synth.lora_weights(wl.seed, s, wl.lora, torch.float16, "cpu", tag="a0").items()}
+        ref = oracle.LlamaRef(s, w, lw, {"a0": wl.lora.scaling}, mode="mixed")
+        t0 = time.perf_counter()
+        exp = oracle.greedy_generate_ref(ref, prompts, {"a0": wl.adapter_ids}, G, n_pages, wl.page_size, perm)
+        t_cpu = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": B * G / t_cpu, "unit": "tok/s", "cores": os.cpu_count(), "kind": "port",
+                               "sample": "numpy oracle greedy_generate_ref, the whole workload once (fp32 arithmetic with fp16 "
+                                         f"rounding where the HIP path stores fp16); threads = BLAS default on {os.cpu_count()} cores"}
+        out["tokens_equal_oracle"] = bool(got == [list(map(int, e)) for e in exp])
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -376,13 +444,15 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="model depth (32 = the benchmark configuration)")
     ap.add_argument("--batch", type=int, default=32,
                     help="c3_decode: concurrent requests (32 = the benchmark configuration; up to 64 run the native step)")
-    ap.add_argument("--workload", default="c3_decode", choices=["c3_decode", "c4_prefill", "c5_decode"],
+    ap.add_argument("--workload", default="c3_decode", choices=["c3_decode", "c4_prefill", "c5_decode", "c1_generate"],
                     help="c3_decode is the benchmark the metric is quoted on; the other two time the prefill and the "
                          "256-request stress configurations with the same harness")
     ap.add_argument("--shape", default="llama2_7b", choices=["llama2_7b", "llama31_8b"],
                     help="c3_decode: model shape (llama2_7b = the benchmark configuration; llama31_8b = the reference's default "
                          "model: grouped-query attention, 8 kv heads, vocabulary 128256)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--dense-lora", action="store_true", help="c1_generate: LlamaExecConfig.dense_lora")
+    ap.add_argument("--batch-prefill", action="store_true", help="c1_generate: LlamaExecConfig.batch_prefill")
     ap.add_argument("--batch-order", action="store_true", help="c5_decode: keep the request order inside the batch (default: longest context first)")
     ap.add_argument("--own-gemm", action="store_true",
                     help="c4_prefill / c5_decode: base linears on this package's LDS GEMM instead of the vendor GEMM library")
@@ -406,6 +476,8 @@ def main():
         return bench_c4_prefill(args, synth, llama)
     if args.workload == "c5_decode":
         return bench_c5_decode(args, synth, llama)
+    if args.workload == "c1_generate":
+        return bench_c1_generate(args, synth, llama)
     if args.probe:
         wl = synth.config3(num_layers=2)
         model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, [wl.lora], dev)
