@@ -101,6 +101,26 @@ def test_c1_greedy_tokens_identical(c1):
         assert got[b][:stop] == exp[b][:stop], b
 
 
+def test_c1_greedy_tokens_with_the_dense_shrink(c1):
+    """The same four requests with `LlamaExecConfig.dense_lora`: the single-type decode batch runs the native step
+    with the adapters' A rows appended to the base GEMV.  Tokens against the oracle: identical up to the first step
+    the oracle itself decides by a near tie (margin below 2 % of the logit std)."""
+    wl, model, prompts = c1
+    synth = load_pkg("synth")
+    max_gen_len = wl.gen_len + 1
+    n_pages = n_pages_for(wl, max_gen_len)
+    perm = synth.permutation(wl.seed, "c1.pages.dense", n_pages)
+    ref = oracle_model(wl, "mixed")
+    exp, margins, scales = oracle.greedy_generate_ref(ref, prompts, {"a0": wl.adapter_ids}, max_gen_len, n_pages,
+                                                      wl.page_size, perm, return_logits=True)
+    got, batcher = run_hip_generate(model, wl, prompts, wl.adapter_ids, max_gen_len, perm, dense_lora=True)
+    assert batcher.graph._dense_ok("decode_a0") and 0 in model._dense_cache
+    for b in range(wl.batch):
+        assert len(got[b]) == max_gen_len
+        i = next((i for i in range(max_gen_len) if got[b][i] != exp[b][i]), None)
+        assert i is None or margins[b][i] < 2e-2 * scales[b][i], (b, i, margins[b][i], scales[b][i])
+
+
 def test_mixed_adapter_types_and_no_adapter(c1):
     """Requests without adapter, with type a0 and with a second adapter type in one decode batch:
     order_seqs / get_decode_method / mixed entry point against the oracle, tokens identical."""
