@@ -1,0 +1,128 @@
+"""Seeded random model shapes and request mixes: the native decode step and the auto-batching front end against the
+per-operator path, bit for bit.  The fixed-size tests cover the benchmark shapes; these cover the corners between them
+(one kv head, 64-wide heads with a 128-wide q block, 1 to 64 requests, ranks 8 to 64, any subset of the seven
+projections, one to seventy adapters, prompts that end on or next to a page boundary)."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import load_pkg
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+ALL = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")
+
+
+def _prefill(model, kv, prompts, ids, ops):
+    B, P = prompts.shape
+    for s in range(B):
+        kv.add_sequence(s)
+    kv.begin_forward(list(range(B)), [P] * B)
+    h = model.embed(torch.from_numpy(np.ascontiguousarray(prompts.reshape(-1))))
+    tok = model._ids(B * P, {0: (None, np.repeat(ids, P).astype(np.int32))}) if model.lora_types else None
+    logits = model.forward(h, kv, tok, model._last_rows(kv))
+    kv.end_forward()
+    return ops.argmax(logits).cpu().numpy()
+
+
+def test_native_step_on_random_model_shapes():
+    """Token ids and the whole K cache of `mlora_decode_step` (called per step and replayed from a graph, ids-based
+    LoRA shrink) equal those of the per-operator path on 120 random configurations."""
+    synth, llama, dsm, ops = load_pkg("synth"), load_pkg("llama"), load_pkg("decode_session"), load_pkg("ops")
+    rng = np.random.default_rng(20240611)
+    for case in range(120):
+        D = int(rng.choice([64, 128])); Hkv = int(rng.choice([1, 2, 4])); Hq = Hkv * int(rng.choice([1, 2, 4]))
+        hidden = int(rng.choice([256, 512, 1024])); inter = int(rng.choice([352, 704, 1408, 2816]))
+        layers = int(rng.choice([1, 2, 3]))
+        B = int(rng.choice([1, 2, 5, 16, 17, 32, 33, 48, 64])); P = int(rng.choice([3, 15, 16, 30])); steps = int(rng.choice([2, 5, 19]))
+        r = int(rng.choice([8, 16, 32, 64])); n_ad = int(rng.choice([1, 3, 8, 70])); k = int(rng.integers(0, 8))
+        targets = tuple(np.array(ALL)[sorted(rng.choice(7, size=k, replace=False))]) if k else ()
+        shape = synth.LlamaShape(hidden_size=hidden, intermediate_size=inter, num_attention_heads=Hq, num_key_value_heads=Hkv,
+                                 num_hidden_layers=layers, head_dim=D, vocab_size=int(rng.choice([512, 1000, 4096])))
+        seed = int(rng.integers(0, 1000))
+        specs = [synth.LoraSpec(r=r, alpha=r / 2, n_adapters=n_ad, targets=targets)] if targets else []
+        tag = (f"case {case}: B={B} P={P} steps={steps} hidden={hidden} inter={inter} Hq={Hq} Hkv={Hkv} D={D} L={layers} "
+               f"r={r} n_ad={n_ad} targets={targets}")
+        print(tag, flush=True)
+        model = llama.LlamaForCausalLM.from_synthetic(seed, shape, specs, DEV)
+        ids = rng.integers(-1, n_ad, size=B).astype(np.int32) if specs else np.full(B, -1, np.int32)
+        prompts = rng.integers(0, shape.vocab_size, size=(B, P)).astype(np.int32)
+        blocks = -(-(P + steps + 2) // 16)
+        outs = []
+        for kind in ("py", "graph", "nograph"):
+            perm = np.random.default_rng(seed).permutation(B * blocks)
+            kv = model.create_paged_kv_cache(B, B * blocks * 16, P, 16, free_pages=perm, max_seq_len=blocks * 16)
+            first = _prefill(model, kv, prompts, ids, ops)
+            if kind == "py":
+                s = dsm.DecodeSession(model, kv, list(range(B)), {0: ids} if specs else {}, first)
+            else:
+                s = dsm.NativeDecodeSession(model, kv, list(range(B)), ids if specs else None, first,
+                                            use_graph=(kind == "graph"), dense_lora=False)
+            toks = np.stack([s.step().cpu().numpy().copy() for _ in range(steps)])
+            outs.append((toks, kv.k.clone()))
+        for toks, kc in outs[1:]:
+            assert np.array_equal(toks, outs[0][0]), tag
+            assert torch.equal(kc, outs[0][1]), tag
+
+
+def test_front_end_on_random_request_mixes():
+    """Up to three adapter types (one scaling) and requests without adapter, per-request length limits and an
+    optional EOS id: the front end returns the same token ids whether decode batches take the native / recorded
+    step or one call per operator, on 80 random mixes."""
+    synth, llama, ab, xg, lora = (load_pkg(m) for m in ("synth", "llama", "auto_batcher", "llama_exec_graph", "lora"))
+    rng = np.random.default_rng(20240612)
+
+    def run(model, prompts, req, max_gen, lens, perm, eos, native):
+        b = ab.LlamaAutoBatcherClass()
+        b.set_model(model)
+        b.set_exec_config(xg.LlamaExecConfig(max_prompt_len=max(len(p) for p in prompts), max_gen_len=max_gen, page_size=16,
+                                             native_decode=native))
+        b.set_free_pages(perm)
+        b.set_eos_token_id(eos)
+        outs = []
+        for p, (tid, wid), mg in zip(prompts, req, lens):
+            v = b.create_var(np.asarray(p, dtype=np.int32))
+            if tid >= 0:
+                lt = model.lora_types[tid]
+                b.set_adapter(lora.LoraConfig(lt.r, lt.scaling * lt.r), wid=wid)
+            outs.append(b.generate(v, max_gen_len=mg))
+        b.compile()
+        b.execute()
+        return [list(np.asarray(o.var).reshape(-1)) for o in outs]
+
+    done = 0
+    while done < 80:
+        D = int(rng.choice([64, 128])); Hkv = int(rng.choice([1, 2, 4])); Hq = Hkv * int(rng.choice([1, 2]))
+        shape = synth.LlamaShape(hidden_size=int(rng.choice([256, 512])), intermediate_size=int(rng.choice([352, 704])),
+                                 num_attention_heads=Hq, num_key_value_heads=Hkv, num_hidden_layers=int(rng.choice([1, 2])),
+                                 head_dim=D, vocab_size=int(rng.choice([300, 1000])))
+        ntypes = int(rng.choice([0, 1, 2, 3]))
+        ranks = [int(x) for x in rng.choice([8, 16, 32, 64], size=ntypes, replace=False)] if ntypes else []
+        specs = [synth.LoraSpec(r=r, alpha=r / 2, n_adapters=int(rng.choice([1, 2, 5])),
+                                targets=tuple(np.array(ALL)[sorted(rng.choice(7, size=int(rng.integers(1, 8)), replace=False))]))
+                 for r in ranks]
+        seed = int(rng.integers(0, 1000))
+        nreq = int(rng.choice([1, 2, 3, 7, 12, 20])); max_gen = int(rng.choice([1, 3, 10, 20]))
+        req = []
+        for _ in range(nreq):
+            tid = int(rng.integers(-1, ntypes)) if ntypes else -1
+            req.append((tid, int(rng.integers(0, specs[tid].n_adapters)) if tid >= 0 else -1))
+        seen = []
+        for tid, _ in req:
+            if tid >= 0 and tid not in seen:
+                seen.append(tid)
+        if seen != list(range(len(seen))):       # the front end numbers adapter types by first use: keep the model's order
+            continue
+        model = llama.LlamaForCausalLM.from_synthetic(seed, shape, specs, DEV)
+        prompts = [rng.integers(0, shape.vocab_size, size=int(rng.integers(1, 40))).astype(np.int32) for _ in range(nreq)]
+        lens = [int(rng.integers(1, max_gen + 1)) for _ in range(nreq)]
+        eos = int(rng.integers(0, shape.vocab_size)) if rng.random() < 0.3 else None
+        pages = sum(-(-(len(p) + max_gen + 1) // 16) for p in prompts) + 2
+        perm = np.random.default_rng(seed).permutation(pages)
+        tag = f"mix {done}: nreq={nreq} ranks={ranks} max_gen={max_gen} eos={eos} Hq={Hq} Hkv={Hkv} D={D} req={req}"
+        print(tag, flush=True)
+        a = run(model, prompts, req, max_gen, lens, perm, eos, True)
+        b_ = run(model, prompts, req, max_gen, lens, perm, eos, False)
+        assert a == b_, tag
+        assert all(1 <= len(o) <= mg for o, mg in zip(a, lens)), tag
+        done += 1
