@@ -126,3 +126,134 @@ def test_front_end_on_random_request_mixes():
         assert a == b_, tag
         assert all(1 <= len(o) <= mg for o, mg in zip(a, lens)), tag
         done += 1
+
+
+def _rowmajor_caches(k, v, n_pages, Hkv, D):
+    """[page, head, slot, d] float64 views of the fragment-ordered K pages and the token-minor V pages."""
+    return (k.permute(0, 1, 4, 2, 3, 5).reshape(n_pages, Hkv, 16, D).double().cpu().numpy(),
+            v.permute(0, 1, 3, 2).double().cpu().numpy())
+
+
+def test_decode_attention_on_random_shapes():
+    """RoPE + append + decode attention in one launch equals the two separate launches bit for bit (output and both
+    caches), and the output equals a dense float64 softmax(q K^T / sqrt(D)) V over each sequence's pages to 3e-3, on
+    100 random (batch, heads, group size, head width, context) draws with shuffled pages."""
+    ops, kvm = load_pkg("ops"), load_pkg("kv_cache")
+    rng = np.random.default_rng(20240613)
+    for case in range(100):
+        D = int(rng.choice([64, 128])); Hkv = int(rng.choice([1, 2, 4, 8, 16, 32])); G = int(rng.choice([1, 2, 4, 8])); Hq = Hkv * G
+        B = int(rng.choice([1, 2, 7, 16, 33, 64, 90])); maxctx = int(rng.choice([1, 17, 100, 300]))
+        ctx = rng.integers(1, maxctx + 1, size=B)
+        max_blocks = -(-maxctx // 16) + 1
+        nb = [-(-int(c) // 16) for c in ctx]
+        n_pages = sum(nb) + 3
+        perm = rng.permutation(n_pages)
+        table = np.full((B, max_blocks), -1, dtype=np.int32)
+        o = 0
+        for b in range(B):
+            table[b, :nb[b]] = perm[o:o + nb[b]]
+            o += nb[b]
+        tag = f"case {case}: B={B} Hq={Hq} Hkv={Hkv} D={D} maxctx={maxctx}"
+        print(tag, flush=True)
+        cos, sin = kvm.rope_tables(D, 10000.0, max_blocks * 16)
+        cos, sin = torch.from_numpy(cos).to(DEV), torch.from_numpy(sin).to(DEV)
+        tab = torch.tensor(table, device=DEV)
+        g = torch.Generator(device="cpu").manual_seed(case)
+        k0 = torch.randn((n_pages, Hkv, D // 32, 4, 16, 8), generator=g).half().to(DEV)
+        v0 = torch.randn((n_pages, Hkv, D, 16), generator=g).half().to(DEV)
+        qkv = torch.randn((B, Hq + 2 * Hkv, D), generator=g).half().to(DEV)
+        seqs = torch.arange(B, dtype=torch.int32, device=DEV)
+        tpos = torch.tensor(ctx - 1, dtype=torch.int32, device=DEV)
+        ctxl = torch.tensor(ctx, dtype=torch.int32, device=DEV)
+        k1, v1, q1 = k0.clone(), v0.clone(), qkv.clone()
+        ops.rope_kv_append(q1, k1, v1, tab, seqs, tpos, cos, sin, Hq, Hkv, D)
+        want = ops.paged_attn_decode(q1, k1, v1, tab, seqs, ctxl, Hq, Hkv, D)
+        k2, v2 = k0.clone(), v0.clone()
+        got = ops.rope_attn_decode(qkv.clone(), k2, v2, tab, seqs, tpos, ctxl, cos, sin, Hq, Hkv, D)
+        assert torch.equal(k1, k2) and torch.equal(v1, v2) and torch.equal(got, want), tag
+        krm, vrm = _rowmajor_caches(k1, v1, n_pages, Hkv, D)
+        out = want.view(B, Hq, D).double().cpu().numpy()
+        qr = q1.double().cpu().numpy()
+        for b in range(min(B, 6)):
+            pages = table[b, :nb[b]]
+            K = krm[pages].transpose(1, 0, 2, 3).reshape(Hkv, -1, D)[:, :ctx[b]]
+            V = vrm[pages].transpose(1, 0, 2, 3).reshape(Hkv, -1, D)[:, :ctx[b]]
+            sc = np.einsum("hgd,hkd->hgk", qr[b, :Hq].reshape(Hkv, G, D), K) / np.sqrt(D)
+            sc -= sc.max(-1, keepdims=True)
+            p = np.exp(sc)
+            p /= p.sum(-1, keepdims=True)
+            ref = np.einsum("hgk,hkd->hgd", p, V).reshape(Hq, D)
+            assert np.abs(out[b] - ref).max() <= 3e-3 * np.abs(ref).max(), (tag, b)
+
+
+def test_prefill_append_and_attention_on_random_segments():
+    """Ragged prompt segments of several sequences in one call, some continuing a prefix that is already cached:
+    the append writes exactly the rotated keys and the values of the new tokens into their page slots (bit-exact,
+    nothing else touched, q rotated in place), and the causal attention output equals a dense float64 evaluation
+    over each token's own sequence to 2e-3, on 80 random draws."""
+    ops, kvm = load_pkg("ops"), load_pkg("kv_cache")
+    rng = np.random.default_rng(20240614)
+    for case in range(80):
+        D = int(rng.choice([64, 128])); Hkv = int(rng.choice([1, 2, 4, 8])); G = int(rng.choice([1, 2, 4, 8])); Hq = Hkv * G
+        S = int(rng.choice([1, 2, 3, 7, 20])); maxlen = int(rng.choice([1, 5, 16, 17, 40, 130]))
+        new = rng.integers(1, maxlen + 1, size=S)
+        pre = rng.integers(0, int(rng.choice([1, 20, 70])), size=S)
+        total = new + pre
+        max_blocks = -(-int(total.max()) // 16) + 1
+        nb = [-(-int(c) // 16) for c in total]
+        n_pages = sum(nb) + 2
+        perm = rng.permutation(n_pages)
+        n_seq = S + 2
+        rows = rng.permutation(n_seq)[:S]
+        table = np.full((n_seq, max_blocks), -1, dtype=np.int32)
+        o = 0
+        for s in range(S):
+            table[rows[s], :nb[s]] = perm[o:o + nb[s]]
+            o += nb[s]
+        T = int(new.sum())
+        tok_seq = np.concatenate([np.full(new[s], rows[s]) for s in range(S)]).astype(np.int32)
+        tok_pos = np.concatenate([np.arange(pre[s], total[s]) for s in range(S)]).astype(np.int32)
+        tag = f"case {case}: S={S} T={T} Hq={Hq} Hkv={Hkv} D={D} new={new.tolist()} pre={pre.tolist()}"
+        print(tag, flush=True)
+        cos, sin = kvm.rope_tables(D, 10000.0, max_blocks * 16)
+        cosd, sind = torch.from_numpy(cos).to(DEV), torch.from_numpy(sin).to(DEV)
+        tab = torch.tensor(table, device=DEV)
+        g = torch.Generator(device="cpu").manual_seed(1000 + case)
+        k = torch.randn((n_pages, Hkv, D // 32, 4, 16, 8), generator=g).half().to(DEV)
+        v = torch.randn((n_pages, Hkv, D, 16), generator=g).half().to(DEV)
+        qkv = torch.randn((T, Hq + 2 * Hkv, D), generator=g).half().to(DEV)
+        q_in = qkv.cpu().numpy()
+        k0rm, v0rm = (a.astype(np.float16) for a in _rowmajor_caches(k, v, n_pages, Hkv, D))
+        ts, tp = torch.tensor(tok_seq, device=DEV), torch.tensor(tok_pos, device=DEV)
+        ops.rope_kv_append(qkv, k, v, tab, ts, tp, cosd, sind, Hq, Hkv, D)
+        out = ops.paged_attn_prefill(qkv, k, v, tab, ts, tp, Hq, Hkv, D)
+        krm, vrm = _rowmajor_caches(k, v, n_pages, Hkv, D)
+        q_out = qkv.cpu().numpy()
+        half = D // 2
+
+        def rot(x, p):      # fp32 arithmetic on fp16 inputs, rounded once: element i pairs with element i + D/2
+            x = x.astype(np.float32)
+            c, s_ = cos[p].astype(np.float32), sin[p].astype(np.float32)
+            a, b = x[..., :half], x[..., half:]
+            return np.concatenate([a * c - b * s_, b * c + a * s_], axis=-1).astype(np.float16)
+
+        kexp, vexp = k0rm.copy(), v0rm.copy()
+        for t in range(T):
+            pg, sl = table[tok_seq[t], tok_pos[t] // 16], tok_pos[t] % 16
+            assert np.array_equal(q_out[t, :Hq], rot(q_in[t, :Hq], tok_pos[t])), (tag, "q", t)
+            kexp[pg, :, sl] = rot(q_in[t, Hq:Hq + Hkv], tok_pos[t])
+            vexp[pg, :, sl] = q_in[t, Hq + Hkv:]
+        assert np.array_equal(kexp, krm.astype(np.float16)) and np.array_equal(vexp, vrm.astype(np.float16)), tag
+        assert np.array_equal(q_out[:, Hq:], q_in[:, Hq:]), tag
+        got = out.double().cpu().numpy().reshape(T, Hq, D)
+        for t in range(T):
+            L = tok_pos[t] + 1
+            pages = table[tok_seq[t], :-(-L // 16)]
+            K = krm[pages].transpose(1, 0, 2, 3).reshape(Hkv, -1, D)[:, :L]
+            V = vrm[pages].transpose(1, 0, 2, 3).reshape(Hkv, -1, D)[:, :L]
+            sc = np.einsum("kgd,kld->kgl", q_out[t, :Hq].astype(np.float64).reshape(Hkv, G, D), K) / np.sqrt(D)
+            sc -= sc.max(-1, keepdims=True)
+            p = np.exp(sc)
+            p /= p.sum(-1, keepdims=True)
+            ref = np.einsum("kgl,kld->kgd", p, V).reshape(Hq, D)
+            assert np.abs(got[t] - ref).max() <= 2e-3 * max(np.abs(ref).max(), 1e-3), (tag, t)
