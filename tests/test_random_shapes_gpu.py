@@ -257,3 +257,90 @@ def test_prefill_append_and_attention_on_random_segments():
             p /= p.sum(-1, keepdims=True)
             ref = np.einsum("kgl,kld->kgd", p, V).reshape(Hq, D)
             assert np.abs(got[t] - ref).max() <= 2e-3 * max(np.abs(ref).max(), 1e-3), (tag, t)
+
+
+def _rel(got, ref, floor=1e-3):
+    scale = ref.abs().max().item()
+    return ((got.double() - ref).abs() / torch.clamp(ref.abs(), min=floor * scale)).max().item()
+
+
+def _gather_mm_float64(y0, x, A, B, ids, s):
+    ref = y0.double().clone()
+    for t in range(x.shape[0]):
+        a = int(ids[t])
+        if a >= 0:
+            ref[t] += s * (B[a].double() @ (A[a].double() @ x[t].double()))
+    return ref
+
+
+def test_lora_and_linear_kernels_on_random_shapes():
+    """160 random draws over three families: the gather-matmul (1 to 2100 tokens: one-launch, vector and matrix-core
+    paths; fp16 and fp32 y; row-major and fragment-ordered x; scattered ids and adapter segments) against a per-token
+    float64 product; the decode linear (1 to 64 tokens, widths up to 32000, store fp16 / fp32 and accumulate)
+    against the float64 product, fragment-ordered input equal to row-major input bit for bit; and the multi-rank /
+    multi-projection calls against one single-rank call per (projection, rank bucket), bit for bit."""
+    ops = load_pkg("ops")
+    rng = np.random.default_rng(20240615)
+    torch.manual_seed(20240615)
+    rel, gm_ref = _rel, _gather_mm_float64
+    n = 0
+    for case in range(160):
+        kind = rng.choice(["gm", "lin", "multi", "mproj"])
+        if kind == "gm":
+            T = int(rng.choice([1, 3, 16, 17, 33, 64, 65, 100, 256, 700, 1025, 1300, 2100]))
+            K = int(rng.choice([64, 256, 520, 1024, 2048, 4096])); N = int(rng.choice([16, 48, 264, 1024, 4096, 4112]))
+            r = int(rng.choice([8, 16, 32, 64])); n_ad = int(rng.choice([1, 2, 5, 17, 40]))
+            ydt = torch.float16 if rng.random() < 0.6 else torch.float32
+            x = torch.randn(T, K, device=DEV).half(); A = (torch.randn(n_ad, r, K, device=DEV) * 0.05).half(); B = (torch.randn(n_ad, N, r, device=DEV) * 0.05).half()
+            ids = torch.from_numpy(rng.integers(-1, n_ad, size=T).astype(np.int32)).to(DEV)
+            if T > 1024 and rng.random() < 0.7:     # adapter segments
+                seg = int(rng.choice([16, 48, 64, 100])); ids = torch.from_numpy((np.arange(T) // seg % (n_ad + 1) - 1).astype(np.int32)).to(DEV)
+            y0 = torch.randn(T, N, device=DEV).to(ydt); s = float(rng.choice([1.0, 0.5, 0.125]))
+            tag = f"gm T={T} K={K} N={N} r={r} n_ad={n_ad} {ydt}"
+            print(tag, flush=True)
+            xin = ops.FragActivation.pack(x) if (T <= 64 and K % 32 == 0 and rng.random() < 0.5) else x
+            got = ops.gather_mm(y0.clone(), xin, A, B, ids, s)
+            e = rel(got, gm_ref(y0, x, A, B, ids.cpu().numpy(), s), 1e-2)
+            tol = 2e-3 if ydt == torch.float16 else 5e-4
+            assert e <= tol * 2, (tag, e)
+        elif kind == "lin":
+            T = int(rng.choice([1, 5, 16, 31, 32, 33, 48, 64])); K = int(rng.choice([64, 512, 1024, 2752, 4096, 11008])); N = int(rng.choice([36, 1024, 4096, 4352, 12288, 13056, 22016, 32000]))
+            x = torch.randn(T, K, device=DEV).half(); W = (torch.randn(N, K, device=DEV) * 0.02).half()
+            ref = x.double() @ W.double().T
+            tag = f"lin T={T} K={K} N={N}"
+            print(tag, flush=True)
+            Wp = ops.PackedWeight(W); xf = ops.FragActivation.pack(x)
+            y16 = ops.linear(xf, Wp); y32 = ops.linear(xf, Wp, out_dtype=torch.float32)
+            r0 = torch.randn(T, N, device=DEV); racc = r0.clone(); ops.linear(xf, Wp, out=racc, accumulate=True)
+            assert rel(y16, ref) <= 4e-3, tag
+            assert rel(y32, ref, 1e-2) <= 1e-3, tag
+            assert rel(racc, r0.double() + ref, 1e-2) <= 1e-3, tag
+            assert torch.equal(y16, ops.linear(x, Wp)), tag
+            e = 0
+        else:
+            T = int(rng.choice([2, 20, 40, 64, 90, 300, 1100])); K = int(rng.choice([256, 1024, 2048]))
+            nb = int(rng.choice([1, 2, 3])); ranks = [int(rng.choice([8, 16, 32, 64])) for _ in range(nb)]; nads = [int(rng.choice([1, 3, 6])) for _ in range(nb)]
+            x = torch.randn(T, K, device=DEV).half()
+            tb = torch.from_numpy(rng.integers(-1, nb, size=T).astype(np.int32)).to(DEV)
+            ta = torch.from_numpy(np.array([rng.integers(0, nads[b]) if b >= 0 else -1 for b in tb.cpu().numpy()], dtype=np.int32)).to(DEV)
+            cols = [int(rng.choice([64, 128, 512])) for _ in range(3 if kind == "mproj" else 1)]
+            offs = [0] + list(np.cumsum(cols)[:-1])
+            ydt = torch.float16 if rng.random() < 0.6 else torch.float32
+            y0 = torch.randn(T, sum(cols), device=DEV).to(ydt)
+            projs = [[None if (rng.random() < 0.15 and nb > 1) else ((torch.randn(na, r, K, device=DEV) * 0.05).half(), (torch.randn(na, c, r, device=DEV) * 0.05).half(), float(rng.choice([1.0, 0.25])))
+                      for r, na in zip(ranks, nads)] for c in cols]
+            tag = f"{kind} T={T} K={K} cols={cols} ranks={ranks} nads={nads} {ydt}"
+            print(tag, flush=True)
+            xin = ops.FragActivation.pack(x) if (T <= 64 and rng.random() < 0.5) else x
+            if kind == "mproj":
+                got = ops.gather_mm_multi_proj(y0.clone(), xin, projs, offs, cols, tb, ta)
+            else:
+                got = ops.gather_mm_multi(y0.clone(), xin, projs[0], tb, ta)
+            want = y0.clone()
+            for p, (c0, c) in enumerate(zip(offs, cols)):
+                for b, bk in enumerate(projs[p]):
+                    if bk is not None:
+                        ops.gather_mm(want[:, c0:c0 + c], xin, bk[0], bk[1], torch.where(tb == b, ta, torch.full_like(ta, -1)), bk[2])
+            assert torch.equal(got, want), tag
+            e = 0
+        n += 1
