@@ -487,8 +487,26 @@ def main():
         dst.copy_(src)                       # plain copy kernel: reads 256 MiB, writes 256 MiB
         g = gemv_event_timing(model, wl.batch, reps=1)
         gm = gather_mm_timing(n_sets=8)
+        # two native decode steps of the 2-layer model at the benchmark's cache geometry (32 sequences at context 520
+        # in shuffled pages, cache pre-filled with N(0,1)): the fused RoPE + attention launch at its real shape
+        blocks = -(-(wl.prompt_len + 16) // wl.page_size)
+        kv = model.create_paged_kv_cache(wl.batch, wl.batch * blocks * wl.page_size, wl.prompt_len, wl.page_size,
+                                         free_pages=synth.permutation(wl.seed, "c3.pages", wl.batch * blocks),
+                                         max_seq_len=blocks * wl.page_size)
+        for l in range(wl.shape.num_hidden_layers):
+            kv.k[l].normal_()
+            kv.v[l].normal_()
+        for b in range(wl.batch):
+            kv.add_sequence(b)
+        kv.begin_forward(list(range(wl.batch)), [wl.prompt_len + 8] * wl.batch)
+        kv.end_forward()
+        sess = dsm.NativeDecodeSession(model, kv, list(range(wl.batch)), wl.adapter_ids, np.arange(wl.batch, dtype=np.int32),
+                                       use_graph=False)
+        sess.step()
+        sess.step()
         torch.cuda.synchronize()
-        print(json.dumps({"probe": True, "copy_bytes_each_way": 256 << 20, "gemv": g, "gather_matmul": gm}))
+        print(json.dumps({"probe": True, "copy_bytes_each_way": 256 << 20, "gemv": g, "gather_matmul": gm,
+                          "attention_kv_bytes_per_launch": int(wl.batch * (wl.prompt_len + 9.5) * 2 * wl.shape.kv_size * 2)}))
         return
     wl = synth.config3(num_layers=args.layers, batch=args.batch, shape=args.shape)
     t_setup = time.perf_counter()
