@@ -267,6 +267,7 @@ int mlora_paged_attn_prefill(void* out, const void* qkv, const void* k_cache, co
  *                               partials written by mlora_gemv_frag_lora with this K; v_dense = kq >= 1: v_part is
  *                               y2 [kq][T, 3 * n_ad * r] of mlora_gemv_frag_split (kq = 1) or
  *                               mlora_gemv_frag_split_kq (slot p = projection p; the kq blocks are added in order);
+ *                               v_dense must lie in 0..4 (the kernels keep at most four blocks), else MLORA_ERR_UNSUPPORTED;
  *   mlora_lora_expand_rmsnorm - resid[t, :] += scaling * B[id_t] . v (B [n_ad, H, r]; v_part [kc][T][r] partials
  *                               of a shrink over K inputs, or y2 [T, n_ad * r] when v_dense = 1), then
  *                               y = RMSNorm(resid) as mlora_rmsnorm.

@@ -22,7 +22,7 @@ softmax attention, rotate-half RoPE) and documents its own page allocator.
 """
 from .lora_ref import (  # noqa: F401
     gather_mm_ref, gather_bmm_hf_ref, lora_sequential_ref, take_matmul_ref,
-    write_tensor_part_ref, mixed_delta_ref, max_rel_err,
+    write_tensor_part_ref, mixed_delta_ref, max_rel_err, combined_tables_ref, lora_combined_ref,
 )
 from .llama_ref import (  # noqa: F401
     rmsnorm_ref, rope_tables, rope_ref, silu_mul_ref, PagedKVRef, attention_dense_ref,

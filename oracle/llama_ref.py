@@ -230,7 +230,8 @@ def greedy_generate_ref(model, prompts, tok_adapter, max_gen_len, n_pages, page_
     """Prefill each sequence, then batched greedy decode (`llama_exec_graph.py:58-141`).
 
     The first generated token is the prefill argmax (`:92`); decoding continues while the last token
-    is not EOS and fewer than `max_gen_len` tokens have been produced (`:94-100`); the batch shrinks
+    is not EOS and fewer than `max_gen_len` tokens have been produced (`:94-100`); that rule is first
+    applied after a decode step (`:110-138`), so every sequence decodes at least once; the batch shrinks
     as sequences finish.  `tok_adapter`: dict tag -> per-request adapter ids [B] (-1 = none).
     np.argmax breaks ties towards the lowest index (`:92,137`).
     Returns a list of B lists of token ids (each of length <= max_gen_len); with return_logits=True also
@@ -252,7 +253,7 @@ def greedy_generate_ref(model, prompts, tok_adapter, max_gen_len, n_pages, page_
         outputs[sid] = [int(np.argmax(logits[0]))]
         margins[sid].append(_margin(logits[0]))
         scales[sid].append(float(logits[0].std()))
-    live = [sid for sid in range(B) if _alive(outputs[sid], max_gen_len, eos_token_id)]
+    live = list(range(B))
     while live:
         toks = np.asarray([outputs[sid][-1] for sid in live])
         kv.begin_forward(live, [1] * len(live))

@@ -92,3 +92,40 @@ def mixed_delta_ref(h, types, dtype=np.float32):
         d = gather_mm_ref(np.zeros((len(sids), N), dtype), h_lcl, t["A"], t["B"], t["wids"], t["scaling"], dtype)
         delta = write_tensor_part_ref(delta, d, sids)
     return delta
+
+
+def combined_tables_ref(A_large, B_large, A_small, B_small):
+    """The 'combined' tables of `tvm/lora_only/case_study/two_ranks_with_combine.py:649-653`, in PEFT orientation:
+    r_mult = r_large / r_small small-rank adapters share one slot of rank r_large, adapter i * r_mult + j of the small
+    type taking rank entries j * r_small .. of slot i; the large-rank adapters come first.
+    A_* [n, r, K], B_* [n, N, r]  ->  A [n_large + n_small / r_mult, r_large, K], B [.., N, r_large]."""
+    A_large, B_large = np.asarray(A_large), np.asarray(B_large)
+    A_small, B_small = np.asarray(A_small), np.asarray(B_small)
+    r_mult = A_large.shape[1] // A_small.shape[1]
+    assert A_large.shape[1] == r_mult * A_small.shape[1] and A_small.shape[0] % r_mult == 0
+    groups = A_small.shape[0] // r_mult
+    A_sc = np.stack([np.concatenate([A_small[i * r_mult + j] for j in range(r_mult)], axis=0) for i in range(groups)])
+    B_sc = np.stack([np.concatenate([B_small[i * r_mult + j] for j in range(r_mult)], axis=1) for i in range(groups)])
+    return np.concatenate([A_large, A_sc], 0), np.concatenate([B_large, B_sc], 0)
+
+
+def lora_combined_ref(x, A, B, xids, wids, scaling, n_rows=None, dtype=np.float32):
+    """The 'combined' strategy's two kernels (`two_ranks_with_combine.py:343-398` take_matmul_combined and `:400-468`
+    fused_take_matmul_multiply_combined): combined row c uses slot wids[c]; rank entry j of that row belongs to token
+    xids[c * R + j]:
+        v[c, j]   = sum_k x[xids[c R + j], k] * A[wids[c], j, k]
+        out[t, n] = scaling * sum over (c, j) with xids[c R + j] == t of v[c, j] * B[wids[c], n, j]
+    The reference indexes the expand's operands `lv` and `lora_B` by wids[c] (`:437-446`), which is row c for the
+    only table it builds (wids = arange, `:1014`); this follows the row.  Returns out [n_rows, N] (no base added)."""
+    x = np.asarray(x, dtype=dtype)
+    A = np.asarray(A, dtype=dtype)
+    B = np.asarray(B, dtype=dtype)
+    xids = np.asarray(xids).reshape(len(wids), -1)
+    R = A.shape[1]
+    assert xids.shape[1] == R
+    out = np.zeros((x.shape[0] if n_rows is None else n_rows, B.shape[1]), dtype=dtype)
+    for c, w in enumerate(np.asarray(wids)):
+        v = np.einsum("jk,jk->j", x[xids[c]], A[w])          # [R]: entry j from its own token
+        for j in range(R):
+            out[xids[c, j]] += v[j] * B[w][:, j]
+    return out * dtype(scaling)

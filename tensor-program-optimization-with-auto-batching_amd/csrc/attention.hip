@@ -829,6 +829,8 @@ extern "C" int mlora_rope_kv_append_lora(void* qkv, void* k_cache, void* v_cache
   MLORA_CHECK(v_part && B && tok_adapter, MLORA_ERR_INVALID, "rope_kv_append_lora: null LoRA argument");
   MLORA_CHECK((r == 8 || r == 16 || r == 32 || r == 64) && n_ad > 0 && K > 0, MLORA_ERR_UNSUPPORTED,
               "rope_kv_append_lora: rank %d not in {8,16,32,64} or bad n_ad/K", r);
+  MLORA_CHECK(v_dense >= 0 && v_dense <= LORA_MAX_KQ, MLORA_ERR_UNSUPPORTED,
+              "rope_kv_append_lora: v_dense=%d outside 0..%d (K-range blocks of dense shrink results)", v_dense, LORA_MAX_KQ);
   LoraExpandQKV lx = {};
   lx.src.v = (const float*)v_part;
   lx.src.kc = v_dense ? 0 : lora_k_split(K).kc;
@@ -895,6 +897,8 @@ extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv
     MLORA_CHECK(Bmat && tok_adapter, MLORA_ERR_INVALID, "rope_attn_decode: null LoRA argument");
     MLORA_CHECK((r == 8 || r == 16 || r == 32 || r == 64) && n_ad > 0 && K > 0, MLORA_ERR_UNSUPPORTED,
                 "rope_attn_decode: rank %d not in {8,16,32,64} or bad n_ad/K", r);
+    MLORA_CHECK(v_dense >= 0 && v_dense <= LORA_MAX_KQ, MLORA_ERR_UNSUPPORTED,
+                "rope_attn_decode: v_dense=%d outside 0..%d (K-range blocks of dense shrink results)", v_dense, LORA_MAX_KQ);
     lx.src.v = (const float*)v_part;
     lx.src.kc = v_dense ? 0 : lora_k_split(K).kc;
     lx.src.kq = v_dense > 0 ? v_dense : 1;

@@ -93,6 +93,7 @@ class LlamaExecGraph(ExecGraph):
         self.step_ms.append(ms)
         if self.measure_file is not None:
             self.measure_file.write(f"{ms}\n")
+            self.measure_file.flush()                   # the file stays open across passes: keep it readable meanwhile
 
     # ------------------------------------------------------------------ operations
     def execute_encode_prompt(self, op):
@@ -165,8 +166,8 @@ class LlamaExecGraph(ExecGraph):
         seqs, original_positions = self.seq_info.order_seqs(op.seqids)
         outputs = {sid: [int(op.input_vars[original_positions[i]].var)] for i, sid in enumerate(seqs)}
         ordered = list(seqs)
-        # the first token (from prefill) already counts towards max_gen_len (`:94-100`)
-        seqs = self.check_seqs_finished(seqs, outputs)
+        # As in the reference (`:102-141`), the finish rule (`:94-100`) is applied only after a decode step: every
+        # sequence takes at least one step after its prefill, also when its first token is EOS or max_gen_len is 1.
         while seqs:
             method, params = self.seq_info.get_decode_method(seqs)
             if getattr(self.exec_config, "native_decode", False) and len(seqs) <= 64:
@@ -203,7 +204,7 @@ class LlamaExecGraph(ExecGraph):
             tid = int(method[len("decode_a"):]) if method != "decode_no_adapter" else 0
             wids = params[0] if params else None
         last = [outputs[sid][-1] for sid in seqs]
-        ahead = min(self.seq_info.get_max_gen_len(sid) - len(outputs[sid]) for sid in seqs)
+        ahead = max(1, min(self.seq_info.get_max_gen_len(sid) - len(outputs[sid]) for sid in seqs))
         sess = NativeDecodeSession(self.vm, self.kv_cache, seqs, wids, last, tid=tid, use_graph=ahead >= 8, dense_lora=None if dense else False)
         if self.eos_token_id is None and not self.measure:
             for _ in range(ahead):
@@ -242,7 +243,7 @@ class LlamaExecGraph(ExecGraph):
         tids = self._method_tids(method)
         pairs = {tid: (params[2 * i], params[2 * i + 1]) for i, tid in enumerate(tids)}
         last = [outputs[sid][-1] for sid in seqs]
-        ahead = min(self.seq_info.get_max_gen_len(sid) - len(outputs[sid]) for sid in seqs)
+        ahead = max(1, min(self.seq_info.get_max_gen_len(sid) - len(outputs[sid]) for sid in seqs))
         sess = DecodeSession(self.vm, self.kv_cache, seqs, self.vm._ids(len(seqs), pairs), last, use_graph=ahead >= 8)
         if self.eos_token_id is None and not self.measure:
             for _ in range(ahead):

@@ -114,6 +114,8 @@ class GatherMMLinear:
         no adapter for that request) or None."""
         shp = x.shape
         x2 = x.reshape(-1, shp[-1]).contiguous()
+        if self.disable_adapters and self.merged:
+            self.unmerge()                              # `lora_gatherbmm_linear_layer.py:10-13`: adapters off = base weight only
         y = ops.linear(x2, self.weight)
         if self.disable_adapters or self.lora_A is None:
             return y.view(*shp[:-1], self.out_features)

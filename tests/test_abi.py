@@ -89,6 +89,14 @@ def test_argument_validation_of_fused_and_batched_entry_points():
     assert ra(8, 8, 128, 0, 0) == 0
     assert lib.mlora_rope_attn_decode(1, 0, 1, 1, 1, 1, 4, 1, 1, 1, 1, 1, 64, 2, 8, 8, 128, 4, 2,
                                       1, 1, None, None, 0.5, 64, 16, 2, None) == -1     # LoRA without B / ids
+    # dense shrink results come in at most four K-range blocks: a larger count would overrun the kernel's LDS array
+    b3 = C.cast((C.c_void_p * 3)(1, 1, 1), C.c_void_p)       # host array of three (dummy) B table pointers
+    assert lib.mlora_rope_attn_decode(1, 0, 1, 1, 1, 1, 4, 1, 1, 1, 1, 1, 64, 2, 8, 8, 128, 4, 2,
+                                      1, 5, b3, 1, 0.5, 64, 16, 2, None) == -2 and b"v_dense" in lib.mlora_last_error()
+    assert lib.mlora_rope_attn_decode(1, 0, 1, 1, 1, 1, 4, 1, 1, 1, 1, 1, 64, 2, 8, 8, 128, 4, 2,
+                                      1, -1, b3, 1, 0.5, 64, 16, 2, None) == -2
+    assert lib.mlora_rope_kv_append_lora(1, 1, 1, 1, 4, 1, 1, 1, 1, 64, 2, 8, 8, 128, 4, 2,
+                                         1, 5, b3, 1, 0.5, 64, 16, 2, None) == -2 and b"v_dense" in lib.mlora_last_error()
     # SiLU epilogue GEMV and split GEMV
     assert lib.mlora_gemv_frag_silu(1, 1, 1, 65, 64, 64, None) == -2
     assert lib.mlora_gemv_frag_silu(1, 1, 1, 8, 64, 48, None) == -2

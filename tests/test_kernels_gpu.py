@@ -141,8 +141,14 @@ def test_gather_mm_linear_branches_of_the_reference_forward(ops, synth):
     assert layer.merged and torch.equal(layer.weight.unpack(), Wm.half())     # the merged weight, rounded to fp16 once
     assert max_rel_err(_np(layer(x)), _np(x).astype(np.float32) @ _np(Wm.half()).astype(np.float32).T) <= TOL
     assert max_rel_err(_np(layer(x)), want, floor=5e-2) <= 5 * TOL             # close to the unmerged result
+    # merged, then adapters disabled: the reference unmerges first (`lora_gatherbmm_linear_layer.py:10-13`), so the
+    # output is the base product again (the weight went through two more fp16 roundings) and the layer is unmerged
+    layer.disable_adapters = True
+    assert max_rel_err(_np(layer(x)), base, floor=5e-2) <= 5 * TOL and not layer.merged
+    layer.disable_adapters = False
+    layer.merge()
     layer.unmerge()
-    # the weight went through two more fp16 roundings: back to the base output up to that noise
+    # the weight went through more fp16 roundings: back to the base output up to that noise
     assert not layer.merged and max_rel_err(_np(layer(x, adapter_names=[None] * Bq)), base, floor=5e-2) <= 5 * TOL
     # two scalings in one call
     layer2 = lora.GatherMMLinear(W)

@@ -271,6 +271,31 @@ def test_per_request_max_gen_len_and_eos(c1):
             assert len(got[b]) <= lens[b]
 
 
+def test_one_decode_step_always_follows_prefill(c1):
+    """max_gen_len = 1, and EOS as the very first token: the reference's loop (`llama_exec_graph.py:102-141`) runs one
+    decode step for every sequence before its finish rule (`:94-100`) sees it, and that rule looks at the newest token
+    only: two tokens come back for max_gen_len = 1, and an EOS out of prefill does not end the sequence."""
+    wl, model, prompts = c1
+    synth = load_pkg("synth")
+    n_pages = n_pages_for(wl, 8)
+    perm = synth.permutation(5, "c1.pages.one", n_pages)
+    ref = oracle_model(wl, "mixed")
+    full, margins, scales = oracle.greedy_generate_ref(ref, prompts, {"a0": wl.adapter_ids}, 4, n_pages, wl.page_size, perm,
+                                                       return_logits=True)
+    decided = [all(m >= 2e-2 * s for m, s in zip(margins[b][:2], scales[b][:2])) for b in range(4)]
+    got, _ = run_hip_generate(model, wl, prompts, wl.adapter_ids, 4, perm, max_gen_lens=[1, 4, 1, 2])
+    assert [len(g) for g in got] == [2, 4, 2, 2]
+    for b in range(4):
+        if decided[b]:
+            assert got[b][:2] == full[b][:2]
+    eos = full[2][0]
+    got, _ = run_hip_generate(model, wl, prompts, wl.adapter_ids, 4, perm, eos_token_id=eos)
+    if all(m >= 2e-2 * s for m, s in zip(margins[2], scales[2])):
+        stop = next((i for i in range(1, 4) if full[2][i] == eos), 3)
+        assert got[2] == full[2][:stop + 1]
+    assert len(got[2]) >= 2
+
+
 def test_adapters_loaded_from_files_and_weight_id_translation(tmp_path):
     """Adapters stored as `lora_adapters/r{rank}_a{wid}.safetensors` are loaded for the types and weight ids the
     registered requests use (two ranks, weight ids out of order); tokens equal the oracle's, which indexes full

@@ -211,6 +211,23 @@ def test_greedy_stops_at_eos_and_respects_adapters():
     assert other != full                                  # the adapter index changes the output
 
 
+def test_greedy_always_takes_one_decode_step_after_prefill():
+    """The reference applies its finish rule only after a decode step (`llama_exec_graph.py:102-141`: the loop starts
+    with every sequence), so max_gen_len = 1 still yields two tokens and an EOS that comes out of prefill does not end its sequence."""
+    shape, ref, synth = _tiny()
+    prompts = synth.randint(2, "p", (2, 7), shape.vocab_size).numpy()
+    ids = {"a0": np.array([1, 1], np.int32)}
+    full = oracle.greedy_generate_ref(ref, prompts, ids, 8, 8)
+    one = oracle.greedy_generate_ref(ref, prompts, ids, 1, 8)
+    assert one == [full[0][:2], full[1][:2]]
+    # EOS as the prefill token is never looked at: only tokens produced by decode steps end a sequence
+    eos = full[0][0]
+    cut = oracle.greedy_generate_ref(ref, prompts, ids, 8, 8, eos_token_id=eos)
+    for b in range(2):
+        stop = next((i for i in range(1, len(full[b])) if full[b][i] == eos), len(full[b]) - 1)
+        assert cut[b] == full[b][:stop + 1] and len(cut[b]) >= 2
+
+
 def test_mixed_mode_rounds_storage_points_only():
     shape, ref32, synth = _tiny(mode="fp32")
     _, ref16, _ = _tiny(mode="mixed")

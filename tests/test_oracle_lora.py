@@ -127,6 +127,36 @@ def test_write_tensor_part_and_mixed_delta():
     assert np.all(delta[2] == 0)
 
 
+def test_combined_strategy_equals_sequential():
+    """The reference's own check (`two_ranks_with_combine.py:1090`: combined == sequential) on its table and index
+    construction (`:649-653`, `:1013-1014`): large-rank requests first, then small-rank requests, every request with
+    its own adapter ("distinct"), r_mult small adapters sharing one combined slot."""
+    rng = np.random.default_rng(11)
+    K, N, r_large, r_small = 48, 40, 8, 2
+    bl, bs = 3, 8                                             # requests of the large / small rank
+    A_l, B_l = rng.standard_normal((bl, r_large, K)), rng.standard_normal((bl, N, r_large))
+    A_s, B_s = rng.standard_normal((bs, r_small, K)), rng.standard_normal((bs, N, r_small))
+    x = rng.standard_normal((bl + bs, K))
+    A_c, B_c = oracle.combined_tables_ref(A_l, B_l, A_s, B_s)
+    r_mult = r_large // r_small
+    assert A_c.shape == (bl + bs // r_mult, r_large, K) and B_c.shape == (bl + bs // r_mult, N, r_large)
+    xids = [i for i in range(bl) for _ in range(r_large)] + [i for i in range(bl, bl + bs) for _ in range(r_small)]
+    wids = np.arange(bl + bs // r_mult)
+    got = oracle.lora_combined_ref(x, A_c, B_c, xids, wids, 2.0, dtype=np.float64)
+    # sequential: each request against its own adapter of its own rank
+    exp = np.zeros((bl + bs, N))
+    for t in range(bl):
+        exp[t] = 2.0 * (B_l[t] @ (A_l[t] @ x[t]))
+    for t in range(bs):
+        exp[bl + t] = 2.0 * (B_s[t] @ (A_s[t] @ x[bl + t]))
+    np.testing.assert_allclose(got, exp, rtol=1e-12, atol=1e-12)
+    # and the per-token oracle on the two types gives the same rows
+    ids_l = np.array(list(range(bl)) + [-1] * bs)
+    ids_s = np.array([-1] * bl + list(range(bs)))
+    two = gather_mm_ref(gather_mm_ref(np.zeros((bl + bs, N)), x, A_l, B_l, ids_l, 2.0, np.float64), x, A_s, B_s, ids_s, 2.0, np.float64)
+    np.testing.assert_allclose(two, exp, rtol=1e-12, atol=1e-12)
+
+
 def test_integer_payload_gather_is_exact():
     """With integer-valued operands the result is exact: the index gather itself is what is tested."""
     rng = np.random.default_rng(7)
