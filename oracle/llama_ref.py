@@ -68,16 +68,18 @@ def attention_dense_ref(q, K, V, q_pos):
     n, Hq, D = q.shape
     ctx, Hkv, _ = K.shape
     g = Hq // Hkv
-    out = np.empty((n, Hq, D), dtype=np.float64)
     mask = np.arange(ctx)[None, :] <= np.asarray(q_pos)[:, None]          # [n, ctx]
-    for h in range(Hq):
-        s = (q[:, h, :] @ K[:, h // g, :].T) / np.sqrt(D)                  # [n, ctx]
-        s = np.where(mask, s, -np.inf)
-        s = s - s.max(axis=-1, keepdims=True)
-        p = np.exp(s)
-        p /= p.sum(axis=-1, keepdims=True)
-        out[:, h, :] = p @ V[:, h // g, :]
-    return out.astype(np.float32)
+    # all heads at once as batched matrix products: [Hkv, g, n, D] x [Hkv, 1, D, ctx]
+    qh = q.reshape(n, Hkv, g, D).transpose(1, 2, 0, 3)
+    Kh = K.transpose(1, 2, 0)[:, None]                                     # [Hkv, 1, D, ctx]
+    Vh = V.transpose(1, 0, 2)[:, None]                                     # [Hkv, 1, ctx, D]
+    s = np.matmul(qh, Kh) / np.sqrt(D)                                     # [Hkv, g, n, ctx]
+    s = np.where(mask[None, None], s, -np.inf)
+    s = s - s.max(axis=-1, keepdims=True)
+    p = np.exp(s)
+    p /= p.sum(axis=-1, keepdims=True)
+    out = np.matmul(p, Vh)                                                 # [Hkv, g, n, D]
+    return out.transpose(2, 0, 1, 3).reshape(n, Hq, D).astype(np.float32)
 
 
 class PagedKVRef:

@@ -109,7 +109,7 @@ def test_native_step_against_oracle_c3_shape():
             got[b].append(int(nxt[b]))
     ties = check_tokens_against_oracle(got, exp, margins, scales)
     print("near-tie disagreements:", ties)
-    assert len(ties) <= 4
+    assert len(ties) <= 1          # measured: one of the 32 x 7 decisions, request 21 at step 5, a near tie of the oracle
 
 
 def test_full_depth_benchmark_model_native_equals_per_operator():

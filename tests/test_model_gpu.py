@@ -94,11 +94,20 @@ def test_c1_greedy_tokens_identical(c1):
     rel = np.array([m / s for mm, ss in zip(margins, scales) for m, s in zip(mm, ss)])
     print(f"oracle margins / logit std: min {rel.min():.3g}, below 2e-2: {(rel < 2e-2).sum()} of {rel.size}; "
           f"near-tie disagreements: {ties}")
+    assert ties == []                       # measured: no disagreement at all on this workload, near tie or not
     got, _ = run_hip_generate(model, wl, prompts, wl.adapter_ids, max_gen_len, perm)
-    assert all(len(g) == max_gen_len for g in got)
+    assert got == [list(map(int, e)) for e in exp]          # all 4 x 33 token ids identical, free-running
+    # against the all-fp32 oracle (no fp16 storage anywhere): its own trajectory, compared token by token up to the
+    # first difference of each request, which must sit at a step that oracle decides by a near tie
+    ref32 = oracle_model(wl, "fp32")
+    exp32, m32, s32 = oracle.greedy_generate_ref(ref32, prompts, {"a0": wl.adapter_ids}, max_gen_len, n_pages,
+                                                 wl.page_size, perm, return_logits=True)
+    same = 0
     for b in range(wl.batch):
-        stop = min([i for (bb, i) in ties if bb == b], default=max_gen_len)
-        assert got[b][:stop] == exp[b][:stop], b
+        i = next((i for i in range(max_gen_len) if got[b][i] != exp32[b][i]), None)
+        same += max_gen_len if i is None else i
+        assert i is None or m32[b][i] < 2e-2 * s32[b][i], (b, i, m32[b][i], s32[b][i])
+    print(f"tokens identical to the fp32 oracle's up to each request's first near tie: {same} of {wl.batch * max_gen_len}")
 
 
 def test_c1_greedy_tokens_with_the_dense_shrink(c1):

@@ -76,6 +76,13 @@ def test_attention_brute_force_tiny():
     q = rng.standard_normal((3, Hq, D)).astype(np.float32)
     pos = [0, 17, 39]
     np.testing.assert_allclose(attention_dense_ref(q, K, V, pos), _brute_attention(q, K, V, pos), rtol=1e-5, atol=1e-6)
+    # several kv heads with several query heads each: query head h must read kv head h // (Hq // Hkv)
+    ctx, Hq, Hkv, D = 21, 6, 3, 4
+    K = rng.standard_normal((ctx, Hkv, D)).astype(np.float32)
+    V = rng.standard_normal((ctx, Hkv, D)).astype(np.float32)
+    q = rng.standard_normal((4, Hq, D)).astype(np.float32)
+    pos = [3, 0, 20, 11]
+    np.testing.assert_allclose(attention_dense_ref(q, K, V, pos), _brute_attention(q, K, V, pos), rtol=1e-5, atol=1e-6)
 
 
 def _run_paged(perm, lens, chunks, seed=3, Hq=4, Hkv=2, D=8, round_fp16=False):
