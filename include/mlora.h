@@ -77,6 +77,19 @@ int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, int x_layout, 
                     const int32_t* tok_adapter, float scaling,
                     int T, int K, int N, int r, int n_ad,
                     void* workspace, size_t workspace_bytes, void* stream);
+/* mlora_gather_mm for callers that cannot allocate and have no workspace to hand over (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference: its tensors all come from
+ * the Python caller.  Same arguments, semantics and result bits as mlora_gather_mm, minus the workspace: the scratch
+ * the kernels need (shrink results of batches above 64 tokens) lives in a buffer built into the library,
+ * MLORA_GATHER_MM_STATIC_BYTES per GPU, held until the process ends.  The call allocates nothing.  Shapes with
+ * mlora_gather_mm_workspace_bytes(T, K, r) above that size are rejected with MLORA_ERR_WORKSPACE.  Every call on a
+ * GPU shares that GPU's buffer: calls that overlap in time on one GPU (two streams, two threads) race; the buffer's
+ * contents are never read before they are written within a call, so nothing needs clearing between calls. */
+#define MLORA_GATHER_MM_STATIC_BYTES (8u << 20)
+size_t mlora_gather_mm_static_max_bytes(void);
+int mlora_gather_mm_static(void* y, int y_dtype, int ldy, const void* x, int x_layout, const void* A, const void* B,
+                           const int32_t* tok_adapter, float scaling,
+                           int T, int K, int N, int r, int n_ad, void* stream);
 /* Several independent gather-matmul problems of one shape and one token->adapter table in ONE launch (decode
  * shapes: T <= 64 and (K-slices + 1) * T * r * 4 <= 48 KiB of LDS, else MLORA_ERR_UNSUPPORTED).
  * sets: DEVICE array of n_sets records of four pointers {y, x, A, B}, laid out as above.  This is how a decode step

@@ -23,6 +23,8 @@ SIGNATURES = {
     "mlora_last_error": (C.c_char_p, []),
     "mlora_gather_mm_workspace_bytes": (_z, [_i, _i, _i]),
     "mlora_gather_mm": (_i, [_p, _i, _i, _p, _i, _p, _p, _p, _f, _i, _i, _i, _i, _i, _p, _z, _p]),
+    "mlora_gather_mm_static_max_bytes": (_z, []),
+    "mlora_gather_mm_static": (_i, [_p, _i, _i, _p, _i, _p, _p, _p, _f, _i, _i, _i, _i, _i, _p]),
     "mlora_gather_mm_multi": (_i, [_p, _i, _i, _p, _i, _p, _i, _p, _p, _i, _i, _i, _p, _z, _p]),
     "mlora_gather_mm_multi_proj": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _p, _p, _p, _p, _i, _i, _p, _z, _p]),
     "mlora_gather_mm_batch": (_i, [_p, _i, _i, _i, _i, _p, _f, _i, _i, _i, _i, _i, _p]),

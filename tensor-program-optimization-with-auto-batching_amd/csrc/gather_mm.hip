@@ -11,6 +11,7 @@
 //             through a small LDS transpose so every lane touches contiguous y elements.
 // The adapter table is never materialised per token: the index lookup happens inside the kernels,
 // which is the optimisation of tvm/custom/fuse_take_matmul.py:85-105 kept in hand-written form.
+#include <mutex>
 #include <type_traits>
 
 #include "lora_device.h"
@@ -1268,6 +1269,57 @@ extern "C" int mlora_gather_mm(void* y, int y_dtype, int ldy, const void* x, int
                                void* workspace, size_t workspace_bytes, void* stream) {
   return gather_mm_impl(y, y_dtype, ldy, x, x_layout, A, B, tok_adapter, scaling, T, K, N, r, n_ad, workspace, workspace_bytes,
                         BucketFilter{nullptr, 0}, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// mlora_gather_mm without a caller workspace and without any allocation: the shrink results of the T > 64 kernels
+// (and the K-slice partials of the odd-shape pair) live in a file-scope device array.  Every device the library runs
+// on holds its own copy of the array at its own address until the process ends; the address is looked up once per
+// device, with that device current, and host code uses that address - never the array's name - from then on.
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[MLORA_GATHER_MM_STATIC_BYTES];
+
+namespace {
+constexpr int STATIC_MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[STATIC_MAX_DEVICES] = {};
+
+// Device address of `scratch` on the current device (nullptr after setting the error message).
+void* static_scratch_ptr() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) {
+    mlora_set_error(MLORA_ERR_LAUNCH, "gather_mm_static: cannot name the current device (%d)", dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      mlora_set_error(MLORA_ERR_LAUNCH, "gather_mm_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" size_t mlora_gather_mm_static_max_bytes(void) { return MLORA_GATHER_MM_STATIC_BYTES; }
+
+extern "C" int mlora_gather_mm_static(void* y, int y_dtype, int ldy, const void* x, int x_layout, const void* A, const void* B,
+                                      const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
+                                      void* stream) {
+  if (int e = check_lora_shape(T, K, N, r, n_ad)) return e;
+  const size_t need = mlora_gather_mm_workspace_bytes(T, K, r);
+  MLORA_CHECK(need <= (size_t)MLORA_GATHER_MM_STATIC_BYTES, MLORA_ERR_WORKSPACE,
+              "gather_mm_static: T=%d K=%d r=%d needs %zu bytes of scratch, the built-in buffer holds %zu (use mlora_gather_mm "
+              "with a workspace)", T, K, r, need, (size_t)MLORA_GATHER_MM_STATIC_BYTES);
+  if (T == 0) return MLORA_OK;
+  void* ws = static_scratch_ptr();
+  if (ws == nullptr) return MLORA_ERR_LAUNCH;
+  return gather_mm_impl(y, y_dtype, ldy, x, x_layout, A, B, tok_adapter, scaling, T, K, N, r, n_ad, ws,
+                        (size_t)MLORA_GATHER_MM_STATIC_BYTES, BucketFilter{nullptr, 0}, stream);
 }
 
 // One launch for n_proj projections that share x (columns col_offset[p] .. + n_cols[p] of y) and n_buckets rank buckets

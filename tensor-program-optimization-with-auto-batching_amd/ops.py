@@ -102,6 +102,25 @@ def gather_mm(y, x, A, B, tok_adapter, scaling: float, workspace=None):
     return y
 
 
+def gather_mm_static(y, x, A, B, tok_adapter, scaling: float):
+    """gather_mm through the entry point that allocates nothing: the kernels' scratch is a buffer built into the
+    library (raises for shapes whose scratch exceeds it).  Calls that overlap on one GPU share that buffer and race."""
+    xptr, xlay, T, K = _x_arg(x)
+    n_ad, r, K2 = A.shape
+    N = B.shape[1]
+    if K2 != K or B.shape != (n_ad, N, r) or y.shape != (T, N) or tok_adapter.shape != (T,):
+        raise ValueError("gather_mm_static: inconsistent shapes")
+    if T == 0:
+        return y
+    if not y.is_cuda or y.stride(1) != 1:
+        raise ValueError("gather_mm_static: y must be a GPU tensor with unit inner stride")
+    ldy = y.stride(0) if T > 1 else max(N, y.stride(0))
+    check(lib().mlora_gather_mm_static(y.data_ptr(), _dt(y), ldy, xptr, xlay, _dev(A, torch.float16, "A"),
+                                       _dev(B, torch.float16, "B"), _dev(tok_adapter, torch.int32, "tok_adapter"),
+                                       float(scaling), T, K, N, r, n_ad, _stream()))
+    return y
+
+
 def gather_mm_multi(y, x, buckets, tok_bucket, tok_adapter, workspace=None):
     """Adapters of several ranks in one batch: buckets = [(A [n_ad,r,K], B [n_ad,N,r], scaling) | None, ...]; token t uses
     adapter tok_adapter[t] of bucket tok_bucket[t] (-1 = none).  y is updated in place."""

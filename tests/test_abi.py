@@ -80,6 +80,11 @@ def test_argument_validation_of_fused_and_batched_entry_points():
     assert lib.mlora_gather_mm_batch(1, 4, 0, 64, 0, 1, 1.0, 65, 64, 64, 16, 2, None) == -2
     assert lib.mlora_gather_mm_batch(None, 4, 0, 64, 0, 1, 1.0, 8, 64, 64, 16, 2, None) == -1
     assert lib.mlora_gather_mm_batch(1, 0, 0, 64, 0, 1, 1.0, 8, 64, 64, 16, 2, None) == 0           # nothing to do
+    # the entry point without workspace: shapes beyond its built-in scratch are refused before anything else happens
+    assert lib.mlora_gather_mm_static_max_bytes() == 8 << 20
+    assert lib.mlora_gather_mm_static(1, 0, 64, 1, 0, 1, 1, 1, 1.0, 4097, 4096, 64, 64, 2, None) == -3 and b"scratch" in lib.mlora_last_error()
+    assert lib.mlora_gather_mm_static(1, 0, 64, 1, 0, 1, 1, 1, 1.0, 8, 64, 64, 12, 2, None) == -2
+    assert lib.mlora_gather_mm_static(1, 0, 64, 1, 0, 1, 1, 1, 1.0, 0, 64, 64, 16, 2, None) == 0
     # fused decode attention
     ra = lambda Hq, Hkv, D, B, lay: lib.mlora_rope_attn_decode(1, lay, 1, 1, 1, 1, 4, 1, 1, 1, 1, 1, 64, B, Hq, Hkv, D, 4, 2,
                                                                None, 0, None, None, 0.0, 0, 0, 0, None)
