@@ -60,7 +60,38 @@ def profiled_gemv_traffic():
     return int(m.group(1)) if m else None
 
 
-def gemv_event_timing(model, T, reps=3):
+def traffic_from_counters(fetch_csv, write_csv, layers_step=32):
+    """HBM bytes per GEMV launch, weighted over the launch mix of one decode step, from the two counter runs of
+    `bench.py --probe` (rocprofv3 --pmc FETCH_SIZE, then --pmc WRITE_SIZE, --output-format csv): each counter is scaled
+    by what it reads for the probe's plain 256 MiB device copy; the probe's GEMV launches come in the order qkv, o,
+    gate_up, down per layer and lm_head last, and a decode step issues each layer kind `layers_step` times and lm_head
+    once.  Needs no GPU."""
+    import csv
+    per_kind = {}
+    scale = {}
+    for name, path in (("fetch", fetch_csv), ("write", write_csv)):
+        rows = sorted(csv.DictReader(open(path)), key=lambda r: int(r["Dispatch_Id"]))
+        copy = max(float(r["Counter_Value"]) for r in rows if "copyBuffer" in r["Kernel_Name"])
+        scale[name] = 262144.0 / copy
+        gemv = [r for r in rows if "gemv" in r["Kernel_Name"] and "pack" not in r["Kernel_Name"]]
+        n_layers = (len(gemv) // 2 - 1) // 4            # the probe issues the mix twice (a warm-up pass, then the timed one)
+        block = gemv[len(gemv) // 2:]
+        assert len(block) == 4 * n_layers + 1, (len(gemv), n_layers)
+        kinds = ["qkv", "o", "gate_up", "down"] * n_layers + ["lm_head"]
+        for k, r in zip(kinds, block):
+            per_kind.setdefault(k, {}).setdefault(name, []).append(float(r["Counter_Value"]))
+    out, tot, n = {}, 0.0, 0
+    for k, d in per_kind.items():
+        kib = sum(d["fetch"]) / len(d["fetch"]) * scale["fetch"] + sum(d["write"]) / len(d["write"]) * scale["write"]
+        cnt = 1 if k == "lm_head" else layers_step
+        out[k] = {"hbm_bytes_per_launch": kib * 1024, "launches_per_step": cnt}
+        tot += cnt * kib * 1024
+        n += cnt
+    return {"scale_fetch": scale["fetch"], "scale_write": scale["write"], "per_kind": out, "gemv_mix_launches": n,
+            "gemv_mix_hbm_bytes_per_launch": tot / n}
+
+
+def gemv_event_timing(model, T, reps=3, per_kind=True):
     """Average duration of the weight-streaming GEMV over exactly the launches of one decode step (per layer: qkv with
     the adapters' A rows appended, o with A rows appended accumulating into the residual, gate/up with the SiLU
     epilogue, down accumulating - o and down with their K split; then lm_head: 129 launches on 129 distinct matrices),
@@ -93,43 +124,59 @@ def gemv_event_timing(model, T, reps=3):
     ks_o, ks_d = lib.mlora_gemv_ksplit(T, Q, H + n_ext), lib.mlora_gemv_ksplit(T, I, H)
     part = torch.empty(3 * T * (H + n_ext), dtype=torch.float32, device=dev)
 
-    def add(fn, rows, K, out_bytes):
+    kinds, nbytes = [], []
+
+    def add(kind, fn, rows, K, out_bytes):
         nonlocal total_bytes
         launches.append(fn)
-        total_bytes += rows * K * 2 + T * K * 2 + out_bytes
+        kinds.append(kind)
+        nbytes.append(rows * K * 2 + T * K * 2 + out_bytes)
+        total_bytes += nbytes[-1]
 
     for l in range(s.num_hidden_layers):
         wq, wo, wd, wg = ext[l]["qkv"], ext[l]["o"], ext[l]["down"], il[l]
         q_ext = wq.N - QKV
         o_ext = wo.N - H
-        add(lambda wq=wq, q_ext=q_ext: lib.mlora_gemv_frag_split_kq(qkv.data_ptr(), y2.data_ptr(), kq, x_h.data.data_ptr(),
+        add("qkv", lambda wq=wq, q_ext=q_ext: lib.mlora_gemv_frag_split_kq(qkv.data_ptr(), y2.data_ptr(), kq, x_h.data.data_ptr(),
                                                                     wq.data.data_ptr(), T, H, QKV, q_ext, st),
             wq.N, H, T * QKV * 2 + kq * T * q_ext * 4)
-        add(lambda wo=wo, o_ext=o_ext: lib.mlora_gemv_frag_acc_ksplit(resid.data_ptr(), y2.data_ptr(), part.data_ptr(), ks_o,
+        add("o", lambda wo=wo, o_ext=o_ext: lib.mlora_gemv_frag_acc_ksplit(resid.data_ptr(), y2.data_ptr(), part.data_ptr(), ks_o,
                                                                       x_q.data.data_ptr(), wo.data.data_ptr(), T, Q, H, o_ext,
                                                                       None, None, 0, None, 0, 0, st),
             wo.N, Q, T * H * 8 + T * o_ext * 4)
-        add(lambda wg=wg: lib.mlora_gemv_frag_silu(act.data.data_ptr(), x_h.data.data_ptr(), wg.data.data_ptr(), T, H, I, st),
+        add("gate_up", lambda wg=wg: lib.mlora_gemv_frag_silu(act.data.data_ptr(), x_h.data.data_ptr(), wg.data.data_ptr(), T, H, I, st),
             2 * I, H, T * I * 2)
-        add(lambda wd=wd: lib.mlora_gemv_frag_acc_ksplit(resid.data_ptr(), None, part.data_ptr(), ks_d, x_i.data.data_ptr(),
+        add("down", lambda wd=wd: lib.mlora_gemv_frag_acc_ksplit(resid.data_ptr(), None, part.data_ptr(), ks_d, x_i.data.data_ptr(),
                                                          wd.data.data_ptr(), T, I, H, 0, None, None, 0, None, 0, 0, st),
             H, I, T * H * 8)
-    add(lambda: lib.mlora_gemv_frag(logits.data_ptr(), F32, STORE, x_h.data.data_ptr(), model.lm_head.data.data_ptr(), T, H,
+    add("lm_head", lambda: lib.mlora_gemv_frag(logits.data_ptr(), F32, STORE, x_h.data.data_ptr(), model.lm_head.data.data_ptr(), T, H,
                                     s.vocab_size, st), s.vocab_size, H, T * s.vocab_size * 4)
-    best = None
-    for _ in range(reps + 1):          # first pass is a warm-up
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for fn in launches:
-            rc = fn()
-            if rc != 0:
-                raise RuntimeError(lib.mlora_last_error().decode())
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1)
-        best = ms if best is None else min(best, ms)
+    def timed(fns):
+        best = None
+        for _ in range(reps + 1):          # first pass is a warm-up
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for fn in fns:
+                rc = fn()
+                if rc != 0:
+                    raise RuntimeError(lib.mlora_last_error().decode())
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            best = ms if best is None else min(best, ms)
+        return best
+
+    best = timed(launches)
+    # the same launches one kind at a time (each kind's launches back to back on their distinct matrices)
+    per_kernel = {}
+    for kind in ("qkv", "o", "gate_up", "down", "lm_head") if per_kind else ():
+        idx = [i for i, k in enumerate(kinds) if k == kind]
+        ms = timed([launches[i] for i in idx])
+        by = sum(nbytes[i] for i in idx)
+        per_kernel[kind] = {"launches": len(idx), "avg_us": 1e3 * ms / len(idx), "bytes_per_launch": by / len(idx),
+                            "gbs": by / (ms * 1e-3) / 1e9, "frac": by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
     return {"launches": len(launches), "avg_us": 1e3 * best / len(launches), "bytes_per_launch": total_bytes / len(launches),
-            "gbs": total_bytes / (best * 1e-3) / 1e9}
+            "gbs": total_bytes / (best * 1e-3) / 1e9, "per_kernel": per_kernel, "kinds": kinds}
 
 
 def gather_mm_timing(n_sets=128):
@@ -173,22 +220,33 @@ def gather_mm_timing(n_sets=128):
     torch.cuda.synchronize()
     sec = e0.elapsed_time(e1) * 1e-3 / reps
     by = 2 * T * K + U * 2 * r * K + U * 2 * N * r + 4 * T * N + 4 * T
-    # the same sets as ONE launch (mlora_gather_mm_batch): what the op costs when it does not pay a launch per problem
-    batch = ops.GatherMMBatch([(y, x, A, B) for x, A, B, y in sets], ids, 1.0)
-    batch.run()
-    torch.cuda.synchronize()
-    reps = 3
-    e0.record()
-    for _ in range(reps):
+    # the same sets in ONE call (mlora_gather_mm_batch): what the op costs when it does not pay a launch per problem -
+    # as a shrink pass and an expand pass over all sets (two launches; what the call does when it is given a
+    # workspace), and as the single launch whose workgroups shrink into LDS and expand from there
+    def batch_time(stream_passes):
+        batch = ops.GatherMMBatch([(y, x, A, B) for x, A, B, y in sets], ids, 1.0, stream_passes=stream_passes)
         batch.run()
-    e1.record()
-    torch.cuda.synchronize()
-    bsec = e0.elapsed_time(e1) * 1e-3 / reps
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(5):
+            e0.record()
+            batch.run()
+            e1.record()
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) * 1e-3
+            best = t if best is None else min(best, t)
+        return {"us_per_set": best / n_sets * 1e6, "us_per_call": best * 1e6, "gbs": by * n_sets / best / 1e9,
+                "frac_of_hbm_peak": by * n_sets / best / 1e9 / HBM_PEAK_GBS}
+
+    two = batch_time(True)
+    two["launches"] = 2
+    one = batch_time(False)
+    one["launches"] = 1
     return {"workload": "T=64 K=N=4096 r=16 n_ad=32", "distinct_adapters": U, "sets": n_sets,
-            "bytes_per_call": by, "us_per_call": sec / n_sets * 1e6, "gbs": by * n_sets / sec / 1e9,
-            "frac_of_hbm_peak": by * n_sets / sec / 1e9 / HBM_PEAK_GBS,
-            "one_launch_for_all_sets": {"us_per_set": bsec / n_sets * 1e6, "gbs": by * n_sets / bsec / 1e9,
-                                        "frac_of_hbm_peak": by * n_sets / bsec / 1e9 / HBM_PEAK_GBS}}
+            "bytes_per_call": by, "single_call_latency_us": sec / n_sets * 1e6,
+            "one_call_per_set": {"us_per_call": sec / n_sets * 1e6, "gbs": by * n_sets / sec / 1e9,
+                                 "frac_of_hbm_peak": by * n_sets / sec / 1e9 / HBM_PEAK_GBS},
+            "one_call_for_all_sets": two, "one_launch_for_all_sets": one}
 
 
 def gather_mm_cpu_baseline(reps=20):
@@ -462,7 +520,13 @@ def main():
     ap.add_argument("--probe", action="store_true",
                     help="counter probe: a few GEMV / gather-matmul launches and a plain 256 MiB copy of known size "
                          "(the calibration for FETCH_SIZE / WRITE_SIZE), no decode loop")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: read the counter CSVs of two `rocprofv3 --pmc` runs of `bench.py --probe` (FETCH_SIZE, "
+                         "WRITE_SIZE) and print the HBM bytes per GEMV launch weighted over the launch mix of one decode step")
     args = ap.parse_args()
+    if args.traffic_from:
+        print(json.dumps(traffic_from_counters(*args.traffic_from)))
+        return
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (every box here has one GPU, and the "
               f"path has no collective: requests would simply be partitioned over GPUs).", file=sys.stderr)
@@ -485,7 +549,7 @@ def main():
         dst = torch.empty_like(src)
         torch.cuda.synchronize()
         dst.copy_(src)                       # plain copy kernel: reads 256 MiB, writes 256 MiB
-        g = gemv_event_timing(model, wl.batch, reps=1)
+        g = gemv_event_timing(model, wl.batch, reps=1, per_kind=False)    # exactly two passes over the mix: warm-up, timed
         gm = gather_mm_timing(n_sets=8)
         # two native decode steps of the 2-layer model at the benchmark's cache geometry (32 sequences at context 520
         # in shuffled pages, cache pre-filled with N(0,1)): the fused RoPE + attention launch at its real shape
@@ -513,7 +577,7 @@ def main():
     model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, [wl.lora], dev)
     prompts = synth.prompts(wl)
     total_new = args.warmup + args.steps + 1
-    max_len = wl.prompt_len + total_new
+    max_len = wl.prompt_len + total_new + 1
     blocks = -(-max_len // wl.page_size)
     perm = synth.permutation(wl.seed, "c3.pages", wl.batch * blocks)
     kv = model.create_paged_kv_cache(wl.batch, wl.batch * blocks * wl.page_size, wl.prompt_len, wl.page_size,
@@ -536,6 +600,24 @@ def main():
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
     tok_s = wl.batch * args.steps / dt
+    dense = bool(getattr(sess, "dense_lora", False))
+    # The timed session computes the LoRA shrink as extra rows of the base GEMV ("dense": taken while the adapters are
+    # few).  The front end's default is the ids-based shrink (bit-identical to the per-operator path): the same steps
+    # over the same pages once more with that form, for the record.
+    ids_ms = None
+    if not args.python_loop and dense and not args.no_extras:
+        for q in range(wl.batch):
+            kv.lens[q] = wl.prompt_len
+        s2 = dsm.NativeDecodeSession(model, kv, list(range(wl.batch)), wl.adapter_ids, first, use_graph=not args.no_graph, dense_lora=False)
+        for _ in range(args.warmup):
+            s2.step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            s2.step()
+        torch.cuda.synchronize()
+        ids_ms = (time.perf_counter() - t1) / args.steps * 1e3
+        del s2
 
     # algorithmic bytes of one step at the mean context of the timed region
     mean_ctx = ctx0 + (args.steps + 1) / 2.0
@@ -552,17 +634,20 @@ def main():
         "config": {"workload": wl.name, "layers": wl.shape.num_hidden_layers, "hidden": wl.shape.hidden_size,
                    "batch": wl.batch, "adapters": wl.lora.n_adapters, "rank": wl.lora.r, "lora_targets": list(wl.lora.targets),
                    "prompt_len": wl.prompt_len, "context_at_start": ctx0, "page_size": wl.page_size, "page_order": "random",
-                   "host_loop": "python" if args.python_loop else ("native" if args.no_graph else "native+graph")},
+                   "host_loop": "python" if args.python_loop else ("native" if args.no_graph else "native+graph"),
+                   "dense_lora": dense},
         "step_algorithmic_gb": step_bytes / 1e9,
         "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "setup_s": t_setup,
     }
+    if ids_ms is not None:
+        out["ids_shrink_variant"] = {"ms_per_step": ids_ms, "tok_s": wl.batch / (ids_ms * 1e-3), "dense_lora": False}
     if not args.no_extras:
         g = gemv_event_timing(model, wl.batch)
         out["roofline"] = {"kernel": "gemv_kernel / gemv_split_cu_kernel / gemv_silu_cu_kernel (fragment-ordered weights and activations, T=32; the 129 GEMV launches of one decode step: adapter A rows appended to qkv / o, K split on o / down, SiLU epilogue on gate/up)", "bound": "hbm", "achieved": g["gbs"],
                            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g["gbs"] / HBM_PEAK_GBS, "traffic": profiled_gemv_traffic(),
                            "launches_timed": g["launches"], "avg_launch_us": g["avg_us"],
-                           "algorithmic_bytes_per_launch": g["bytes_per_launch"]}
+                           "algorithmic_bytes_per_launch": g["bytes_per_launch"], "per_kernel": g["per_kernel"]}
         del sess, kv
         torch.cuda.empty_cache()
         out["gather_matmul"] = gather_mm_timing()

@@ -94,7 +94,12 @@ int mlora_gather_mm_static(void* y, int y_dtype, int ldy, const void* x, int x_l
  * shapes: T <= 64 and (K-slices + 1) * T * r * 4 <= 48 KiB of LDS, else MLORA_ERR_UNSUPPORTED).
  * sets: DEVICE array of n_sets records of four pointers {y, x, A, B}, laid out as above.  This is how a decode step
  * meets the op: every layer and projection has its own A / B / x / y, and the ~2 us of work per problem is far below
- * the cost of a launch.  Same result bits as n_sets calls of mlora_gather_mm.  Replaces the same reference code. */
+ * the cost of a launch.  Same result bits as n_sets calls of mlora_gather_mm.  Replaces the same reference code.
+ * workspace: NULL, or n_sets * mlora_gather_mm_workspace_bytes(T, K, r) bytes of device scratch.  With a workspace and
+ * eight or more sets the call runs as two streaming passes over all sets (a shrink launch that leaves its fp32
+ * partials in the workspace, then an expand launch): no request of either pass waits on more than the table row, which
+ * is what lets a many-problem call run at HBM bandwidth; without a workspace, or for fewer sets, one launch whose
+ * workgroups shrink into LDS and expand from there.  Same result bits either way. */
 /* Adapters of several ranks in one batch.  Bucket b holds the adapters of one rank and scaling,
  *   A [n_ad, r, K], B [n_ad, N, r]; token t uses adapter tok_adapter[t] of bucket tok_bucket[t]; a token whose
  *   bucket is outside [0, n_buckets) or whose adapter id is outside [0, n_ad) of its bucket is left untouched.
@@ -138,7 +143,8 @@ int mlora_gather_mm_multi_proj(void* y, int y_dtype, int ldy, const void* x, int
                                int T, int K, void* workspace, size_t workspace_bytes, void* stream);
 int mlora_gather_mm_batch(const void* const* sets, int n_sets, int y_dtype, int ldy, int x_layout,
                           const int32_t* tok_adapter, float scaling,
-                          int T, int K, int N, int r, int n_ad, void* stream);
+                          int T, int K, int N, int r, int n_ad,
+                          void* workspace, size_t workspace_bytes, void* stream);
 
 /* The two halves of the above, for callers that fuse differently:
  *   shrink: v_part[c, t, :] = A[id_t][:, chunk c] . x[t, chunk c]   (fp32 partials per K-chunk)

@@ -27,7 +27,7 @@ SIGNATURES = {
     "mlora_gather_mm_static": (_i, [_p, _i, _i, _p, _i, _p, _p, _p, _f, _i, _i, _i, _i, _i, _p]),
     "mlora_gather_mm_multi": (_i, [_p, _i, _i, _p, _i, _p, _i, _p, _p, _i, _i, _i, _p, _z, _p]),
     "mlora_gather_mm_multi_proj": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _p, _p, _p, _p, _i, _i, _p, _z, _p]),
-    "mlora_gather_mm_batch": (_i, [_p, _i, _i, _i, _i, _p, _f, _i, _i, _i, _i, _i, _p]),
+    "mlora_gather_mm_batch": (_i, [_p, _i, _i, _i, _i, _p, _f, _i, _i, _i, _i, _i, _p, _z, _p]),
     "mlora_lora_shrink": (_i, [_p, _p, _i, _p, _p, _i, _i, _i, _i, _p]),
     "mlora_lora_expand": (_i, [_p, _i, _i, _p, _p, _p, _f, _i, _i, _i, _i, _i, _p]),
     "mlora_write_tensor_part": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),

@@ -12,7 +12,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmlora_hip.so")
-SOURCES = ["api.hip", "gather_mm.hip", "gemv.hip", "gemm.hip", "rowops.hip", "attention.hip", "decode_step.hip", "library_gemm.hip"]
+SOURCES = ["api.hip", "gather_mm.hip", "gather_mm_batch.hip", "gemv.hip", "gemm.hip", "rowops.hip", "attention.hip", "decode_step.hip", "library_gemm.hip"]
 LINK_LIBS = ["-L/opt/rocm/lib", "-lhipblaslt"]   # the vendor GEMM library behind mlora_gemm_library
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", 
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -40,6 +40,7 @@ def build(force: bool = True, jobs: int = 6) -> str:
     objs = []
     todo = []
     hdr_m = max(os.path.getmtime(os.path.join(CSRC, "common.h")), os.path.getmtime(os.path.join(CSRC, "lora_device.h")),
+                os.path.getmtime(os.path.join(CSRC, "gather_mm_batch.h")),
                 os.path.getmtime(os.path.join(HERE, "..", "include", "mlora.h")))
     for src in SOURCES:
         s = os.path.join(CSRC, src)

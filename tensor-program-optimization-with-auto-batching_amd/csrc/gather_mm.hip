@@ -14,7 +14,7 @@
 #include <mutex>
 #include <type_traits>
 
-#include "lora_device.h"
+#include "gather_mm_batch.h"
 
 namespace {
 
@@ -135,13 +135,6 @@ __global__ __launch_bounds__(64) void lora_expand_kernel(YT* __restrict__ y, con
 // A launch can cover several independent problems (sets of y, x, A, B with a common shape and adapter table):
 // blockIdx.y selects the set.
 // ---------------------------------------------------------------------------------------------
-struct GmmSet {
-  void* y;
-  const f16* x;
-  const f16* A;
-  const f16* B;
-};
-
 constexpr int GMM_WAVES = 8;
 constexpr int GMM_THREADS = GMM_WAVES * WAVE;
 
@@ -1149,9 +1142,13 @@ static int gmm_one_launch(const GmmSet& one, const GmmSet* sets, int n_sets, int
   return mlora_launch_status("gather_mm");
 }
 
+// Problems in a launch from which the two streaming passes pay off (a launch boundary costs a few microseconds; below
+// this the single launch with its LDS hand-over is shorter).
+constexpr int GMM_STREAM_MIN_SETS = 8;
+
 extern "C" int mlora_gather_mm_batch(const void* const* sets, int n_sets, int y_dtype, int ldy, int x_layout,
                                      const int32_t* tok_adapter, float scaling, int T, int K, int N, int r, int n_ad,
-                                     void* stream) {
+                                     void* workspace, size_t workspace_bytes, void* stream) {
   if (int e = check_lora_shape(T, K, N, r, n_ad)) return e;
   MLORA_CHECK(sets && tok_adapter && n_sets >= 0 && n_sets <= 65535, MLORA_ERR_INVALID, "gather_mm_batch: null pointer or bad n_sets=%d", n_sets);
   MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "gather_mm_batch: bad y_dtype %d", y_dtype);
@@ -1161,6 +1158,13 @@ extern "C" int mlora_gather_mm_batch(const void* const* sets, int n_sets, int y_
   if (T == 0 || n_sets == 0) return MLORA_OK;
   MLORA_CHECK(gmm_one_launch_fits(T, K, r), MLORA_ERR_UNSUPPORTED,
               "gather_mm_batch: decode shapes only (T <= 64 and (kc + 1) * T * r * 4 <= 48 KiB; T=%d K=%d r=%d)", T, K, r);
+  if (workspace != nullptr && n_sets >= GMM_STREAM_MIN_SETS) {
+    const size_t need = (size_t)n_sets * mlora_gather_mm_workspace_bytes(T, K, r);
+    MLORA_CHECK(workspace_bytes >= need, MLORA_ERR_WORKSPACE, "gather_mm_batch: workspace of %zu bytes given, %zu needed for %d sets",
+                workspace_bytes, need, n_sets);
+    return gmm_batch_stream((const GmmSet*)sets, n_sets, y_dtype, ldy, x_layout, tok_adapter, scaling, T, K, N, r, n_ad,
+                            (float*)workspace, (hipStream_t)stream);
+  }
   return gmm_one_launch(GmmSet(), (const GmmSet*)sets, n_sets, y_dtype, ldy, x_layout, tok_adapter, scaling, T, K, N, r, n_ad,
                         (hipStream_t)stream);
 }

@@ -203,7 +203,9 @@ class GatherMMBatch:
     """Several gather-matmul problems of one shape and one token->adapter table, issued as one launch.
     sets: list of (y, x, A, B) as for gather_mm (x row-major); the tensors are kept alive by this object."""
 
-    def __init__(self, sets, tok_adapter, scaling: float):
+    def __init__(self, sets, tok_adapter, scaling: float, stream_passes: bool = True):
+        """stream_passes: give the call a workspace, which lets it run eight or more sets as a shrink pass and an
+        expand pass over all of them (same result bits as the single launch it uses otherwise)."""
         y0, x0, A0, B0 = sets[0]
         self.T, self.K = x0.shape
         self.n_ad, self.r, _ = A0.shape
@@ -222,11 +224,16 @@ class GatherMMBatch:
         _dev(tok_adapter, torch.int32, "tok_adapter")
         self.scaling = float(scaling)
         self.table = torch.tensor(ptrs, dtype=torch.int64, device=x0.device)
+        self.ws = None
+        if stream_passes:
+            n = len(sets) * lib().mlora_gather_mm_workspace_bytes(self.T, self.K, self.r)
+            self.ws = torch.empty(max(n, 16) // 4, dtype=torch.float32, device=x0.device)
 
     def run(self):
+        ws, nb = (self.ws.data_ptr(), self.ws.numel() * 4) if self.ws is not None else (None, 0)
         check(lib().mlora_gather_mm_batch(self.table.data_ptr(), len(self.sets), self.ydt, self.ldy, ROWMAJOR,
                                           self.ids.data_ptr(), self.scaling, self.T, self.K, self.N, self.r, self.n_ad,
-                                          _stream()))
+                                          ws, nb, _stream()))
 
 
 def lora_shrink(v_part, x, A, tok_adapter):

@@ -77,9 +77,10 @@ def test_argument_validation_of_fused_and_batched_entry_points():
     assert lib.mlora_gather_mm_multi_proj(1, 0, 128, 1, 0, C.cast(bk4, C.c_void_p), 2, 9, C.cast(co, C.c_void_p), C.cast(nc, C.c_void_p),
                                           1, 1, 8, 64, 1, 1 << 20, None) == -1         # more than 8 projections
     # batched gather-matmul: decode shapes only
-    assert lib.mlora_gather_mm_batch(1, 4, 0, 64, 0, 1, 1.0, 65, 64, 64, 16, 2, None) == -2
-    assert lib.mlora_gather_mm_batch(None, 4, 0, 64, 0, 1, 1.0, 8, 64, 64, 16, 2, None) == -1
-    assert lib.mlora_gather_mm_batch(1, 0, 0, 64, 0, 1, 1.0, 8, 64, 64, 16, 2, None) == 0           # nothing to do
+    assert lib.mlora_gather_mm_batch(1, 4, 0, 64, 0, 1, 1.0, 65, 64, 64, 16, 2, None, 0, None) == -2
+    assert lib.mlora_gather_mm_batch(None, 4, 0, 64, 0, 1, 1.0, 8, 64, 64, 16, 2, None, 0, None) == -1
+    assert lib.mlora_gather_mm_batch(1, 0, 0, 64, 0, 1, 1.0, 8, 64, 64, 16, 2, None, 0, None) == 0           # nothing to do
+    assert lib.mlora_gather_mm_batch(1, 16, 0, 64, 0, 1, 1.0, 8, 64, 64, 16, 2, 1, 64, None) == -3          # workspace too small for 16 sets
     # the entry point without workspace: shapes beyond its built-in scratch are refused before anything else happens
     assert lib.mlora_gather_mm_static_max_bytes() == 8 << 20
     assert lib.mlora_gather_mm_static(1, 0, 64, 1, 0, 1, 1, 1, 1.0, 4097, 4096, 64, 64, 2, None) == -3 and b"scratch" in lib.mlora_last_error()

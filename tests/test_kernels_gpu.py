@@ -473,20 +473,37 @@ def test_gather_mm_one_launch_equals_shrink_then_expand(ops, synth, T, K, N, r, 
     assert max_rel_err(_np(y1), ref) <= TOL
 
 
-def test_gather_mm_batch_equals_separate_calls(ops, synth):
-    """Five problems with their own x, A, B, y in one launch: same bits as five calls."""
-    T, K, N, r, n_ad = 48, 2048, 1024, 16, 12
-    ids = synth.randint(9, "gmb.ids", (T,), n_ad, DEV)
+@pytest.mark.parametrize("n_sets,T,K,N,r,n_ad,ydt,stream_passes", [
+    (5, 48, 2048, 1024, 16, 12, torch.float16, True),        # few sets: one launch, partials in LDS
+    (12, 48, 2048, 1024, 16, 12, torch.float16, False),      # many sets without a workspace: still one launch
+    (12, 48, 2048, 1024, 16, 12, torch.float16, True),       # many sets with a workspace: shrink pass + expand pass
+    (9, 64, 4096, 4096, 16, 32, torch.float16, True),        # the isolated-op benchmark shape (some adapters unused)
+    (8, 33, 1024, 2056, 8, 5, torch.float32, True),          # rank 8 (half-filled reduction), fp32 y, ragged row blocks
+    (8, 20, 11008, 512, 32, 3, torch.float16, True),         # rank 32 and three 512-wide chunks per K-slice: generic shrink unit
+    (10, 32, 1536, 264, 64, 40, torch.float32, True),        # rank 64, more adapters than tokens
+    (8, 7, 1000, 136, 16, 2, torch.float16, True),           # K with a partial last chunk; many tokens per adapter
+])
+def test_gather_mm_batch_equals_separate_calls(ops, synth, n_sets, T, K, N, r, n_ad, ydt, stream_passes):
+    """Several problems with their own x, A, B, y and one token->adapter table in one call: same bits as one
+    mlora_gather_mm call per problem, whether the call runs as one launch or as a shrink pass and an expand pass."""
+    print(f"case gather_mm_batch sets={n_sets} T={T} K={K} N={N} r={r} n_ad={n_ad} {ydt} stream={stream_passes}", flush=True)
+    ids = synth.randint(9, f"gmb.ids{T}.{n_ad}", (T,), n_ad + 1, DEV) - 1          # -1 = no adapter
+    ids = ids.to(torch.int32)
     sets, want = [], []
-    for j in range(5):
-        c = synth.gather_mm_case(seed=9, T=T, K=K, N=N, r=r, n_ad=n_ad, device=DEV, tag=f"gmb{j}")
-        y = c["y"].clone()
+    for j in range(n_sets):
+        c = synth.gather_mm_case(seed=9, T=T, K=K, N=N, r=r, n_ad=n_ad, device=DEV, tag=f"gmb{j}.{T}.{K}")
+        y = c["y"].to(ydt).clone()
         ops.gather_mm(y, c["x"], c["A"], c["B"], ids, 0.25)
         want.append(y)
-        sets.append((c["y"].clone(), c["x"], c["A"], c["B"]))
-    ops.GatherMMBatch(sets, ids, 0.25).run()
+        sets.append((c["y"].to(ydt).clone(), c["x"], c["A"], c["B"]))
+    batch = ops.GatherMMBatch(sets, ids, 0.25, stream_passes=stream_passes)
+    if batch.ws is not None:
+        batch.ws.fill_(float("nan"))                 # the workspace need not be initialised
+    batch.run()
+    torch.cuda.synchronize()
     for (y, _, _, _), w in zip(sets, want):
         assert torch.equal(y, w)
+    assert not torch.equal(sets[0][0], synth.gather_mm_case(seed=9, T=T, K=K, N=N, r=r, n_ad=n_ad, device=DEV, tag=f"gmb0.{T}.{K}")["y"].to(ydt))
 
 
 @pytest.mark.parametrize("ydt", [torch.float16, torch.float32])
