@@ -324,7 +324,7 @@ def bench_c4_prefill(args, synth, llama):
     dev = "cuda:0"
     wl = synth.config4(num_layers=args.layers)
     s = wl.shape
-    model = llama.LlamaForCausalLM.from_synthetic(wl.seed, s, [wl.lora], dev, library_gemm=not args.own_gemm)
+    model = llama.LlamaForCausalLM.from_synthetic(wl.seed, s, [wl.lora], dev)
     prompts = synth.prompts(wl)
     B, P = prompts.shape
     order = np.argsort(wl.adapter_ids, kind="stable")             # requests grouped into adapter segments
@@ -366,7 +366,7 @@ def bench_c4_prefill(args, synth, llama):
         "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": wl.name, "layers": L, "tokens": T, "segments": int(len(np.unique(wids))), "rank": wl.lora.r,
                    "lora_targets": list(wl.lora.targets),
-                   "base_gemm": "gemm_lds_kernel (this package)" if args.own_gemm else "vendor GEMM library (plain T=4096 GEMMs)"},
+                   "base_gemm": "gemm_lds_kernel (this package)"},
         "roofline": {"kernel": "whole prefill pass (base GEMMs 97 % of the flops)", "bound": "mfma", "achieved": flops / dt / 1e12,
                      "peak": 2500.0, "unit": "TFLOP/s", "frac": flops / dt / 1e12 / 2500.0, "traffic": None,
                      "flops_base": flops_base, "flops_lora": flops_lora, "flops_attention": flops_attn}}))
@@ -381,7 +381,7 @@ def bench_c5_decode(args, synth, llama):
     dev = "cuda:0"
     wl = synth.config5(num_layers=args.layers)
     s = wl.shape
-    model = llama.LlamaForCausalLM.from_synthetic(wl.seed, s, [wl.lora], dev, library_gemm=not args.own_gemm)
+    model = llama.LlamaForCausalLM.from_synthetic(wl.seed, s, [wl.lora], dev)
     B = wl.batch
     n_steps = args.warmup + args.steps
     # requests in adapter order, as the front end batches them (`llama_seq_info.py:61-75` sorts by adapter type and weight id)
@@ -420,7 +420,7 @@ def bench_c5_decode(args, synth, llama):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": wl.name, "layers": s.num_hidden_layers, "batch": B, "adapters_in_use": used,
                    "total_context": int(ctx.sum()), "host_loop": "python",
-                   "base_gemm": "gemm_lds_kernel (this package)" if args.own_gemm else "vendor GEMM library (plain T=256 GEMMs)"},
+                   "base_gemm": "this package's kernels"},
         "roofline": {"kernel": "whole decode step (paged attention 91 % of the bytes)", "bound": "hbm",
                      "achieved": step_bytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": step_bytes / dt / 1e9 / HBM_PEAK_GBS, "traffic": None, "step_algorithmic_gb": step_bytes / 1e9}}))
@@ -512,8 +512,6 @@ def main():
     ap.add_argument("--dense-lora", action="store_true", help="c1_generate: LlamaExecConfig.dense_lora")
     ap.add_argument("--batch-prefill", action="store_true", help="c1_generate: LlamaExecConfig.batch_prefill")
     ap.add_argument("--batch-order", action="store_true", help="c5_decode: keep the request order inside the batch (default: longest context first)")
-    ap.add_argument("--own-gemm", action="store_true",
-                    help="c4_prefill / c5_decode: base linears on this package's LDS GEMM instead of the vendor GEMM library")
     ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel event timing and the gather-matmul stream")
     ap.add_argument("--python-loop", action="store_true", help="issue every kernel from Python instead of mlora_decode_step")
     ap.add_argument("--no-graph", action="store_true", help="call mlora_decode_step every step instead of replaying a captured graph")

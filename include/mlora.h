@@ -179,16 +179,6 @@ int mlora_gemm(void* y, int y_dtype, int mode, const void* x, int ldx, const voi
 int mlora_linear(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W,
                  int T, int K, int N, void* stream);
 
-/* The same linear on a row-major W through the vendor GEMM library (hipBLASLt), for prefill-sized T where the
- * operation is a plain GEMM with nothing fused into it.  `workspace` is caller-owned device scratch of
- * mlora_gemm_library_workspace_bytes() bytes (may be NULL / 0: the library then picks an algorithm that needs
- * none).  The library handle and the per-shape algorithm choice are created on first use and kept for the life
- * of the process (the only state this entry point adds); the call itself allocates nothing.
- * Constraints: K % 8 == 0, N % 8 == 0, ldx % 8 == 0; MLORA_ACCUMULATE needs y_dtype = MLORA_F32. */
-size_t mlora_gemm_library_workspace_bytes(void);
-int mlora_gemm_library(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W,
-                       int T, int K, int N, void* workspace, size_t workspace_bytes, void* stream);
-
 /* Fragment-ordered weight layout for the same linears.  The reference re-lays out weights once at load
  * time as well (stack + transpose, tvm/llama_auto_batcher/compile_tvm.py:296-314); here the one-time step
  * stores W in the order the matrix cores consume it,

@@ -49,8 +49,6 @@ SIGNATURES = {
     "mlora_gemv_frag_split_kq": (_i, [_p, _p, _i, _p, _p, _i, _i, _i, _i, _p]),
     "mlora_rope_kv_append_lora": (_i, [_p, _p, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p]),
     "mlora_rope_attn_decode": (_i, [_p, _i, _p, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p]),
-    "mlora_gemm_library_workspace_bytes": (_z, []),
-    "mlora_gemm_library": (_i, [_p, _i, _i, _p, _i, _p, _i, _i, _i, _p, _z, _p]),
     "mlora_gemv_ksplit": (_i, [_i, _i, _i]),
     "mlora_gemv_ksplit_bytes": (_z, [_i, _i, _i]),
     "mlora_gemv_frag_acc_ksplit": (_i, [_p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _p, _p, _i, _p, _i, _i, _p]),

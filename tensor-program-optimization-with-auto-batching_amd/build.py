@@ -12,8 +12,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmlora_hip.so")
-SOURCES = ["api.hip", "gather_mm.hip", "gather_mm_batch.hip", "gemv.hip", "gemm.hip", "rowops.hip", "attention.hip", "decode_step.hip", "library_gemm.hip"]
-LINK_LIBS = ["-L/opt/rocm/lib", "-lhipblaslt"]   # the vendor GEMM library behind mlora_gemm_library
+SOURCES = ["api.hip", "gather_mm.hip", "gather_mm_batch.hip", "gemv.hip", "gemm.hip", "rowops.hip", "attention.hip", "decode_step.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", 
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
@@ -51,7 +50,7 @@ def build(force: bool = True, jobs: int = 6) -> str:
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(_run, todo))
     if todo or not os.path.exists(LIB):
-        _run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objs, *LINK_LIBS, "-o", LIB])
+        _run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB])
     return LIB
 
 

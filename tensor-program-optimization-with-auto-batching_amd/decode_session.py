@@ -46,7 +46,7 @@ class DecodeSession:
         self.rows = i32([kv.slot[s] for s in self.seq_ids])
         self.pos = i32([kv.lens[s] for s in self.seq_ids])
         self.ctx = self.pos + 1
-        self.use_graph = use_graph and B <= 64     # larger batches may call into the vendor GEMM library: not captured
+        self.use_graph = use_graph
         self.graph = None
         self._eager_steps = 0
         self.history = []

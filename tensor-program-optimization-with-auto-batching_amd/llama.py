@@ -54,12 +54,9 @@ class LoraType:
 
 
 class LlamaForCausalLM:
-    def __init__(self, shape: LlamaShape, device="cuda:0", library_gemm: bool = False):
-        """library_gemm: keep a row-major copy of the four layer matrices so that prefill-sized base linears (T > 64)
-        go to the vendor GEMM library; decode-sized ones always use this package's kernels."""
+    def __init__(self, shape: LlamaShape, device="cuda:0"):
         self.shape = shape
         self.device = torch.device(device)
-        self.library_gemm = library_gemm
         self.layers = []          # per layer dict: qkv, o, gate_up, down (PackedWeight), ln1, ln2 (fp16 [H])
         self.embed_tokens = None
         self.lm_head = None
@@ -76,10 +73,9 @@ class LlamaForCausalLM:
         dev = self.device
         qkv = torch.cat([w["q_proj"], w["k_proj"], w["v_proj"]], 0).to(dev, torch.float16)
         gu = torch.cat([w["gate_proj"], w["up_proj"]], 0).to(dev, torch.float16)
-        rm = self.library_gemm
         self.layers.append({
-            "qkv": ops.PackedWeight(qkv, rm), "o": ops.PackedWeight(w["o_proj"].to(dev, torch.float16), rm),
-            "gate_up": ops.PackedWeight(gu, rm), "down": ops.PackedWeight(w["down_proj"].to(dev, torch.float16), rm),
+            "qkv": ops.PackedWeight(qkv), "o": ops.PackedWeight(w["o_proj"].to(dev, torch.float16)),
+            "gate_up": ops.PackedWeight(gu), "down": ops.PackedWeight(w["down_proj"].to(dev, torch.float16)),
             "ln1": w["input_layernorm"].to(dev, torch.float16).contiguous(),
             "ln2": w["post_attention_layernorm"].to(dev, torch.float16).contiguous(),
         })
@@ -95,10 +91,10 @@ class LlamaForCausalLM:
         return len(self.lora_types) - 1
 
     @classmethod
-    def from_synthetic(cls, seed: int, shape: LlamaShape, lora_specs=(), device="cuda:0", synth=None, library_gemm=False):
+    def from_synthetic(cls, seed: int, shape: LlamaShape, lora_specs=(), device="cuda:0", synth=None):
         """Random-init model generated on the device (bit-identical to the CPU generation of the same seed)."""
         from . import synth as S
-        m = cls(shape, device, library_gemm)
+        m = cls(shape, device)
         for l in range(shape.num_hidden_layers):
             w = S.layer_weights(seed, shape, l, torch.float16, device)
             m.load_layer(l, {k.split(".", 2)[2]: v for k, v in w.items()})

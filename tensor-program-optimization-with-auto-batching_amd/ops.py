@@ -265,15 +265,12 @@ def write_tensor_part(X, Y, ids, out=None):
 class PackedWeight:
     """A [N, K] fp16 weight stored in matrix-core fragment order (see mlora_pack_weight)."""
 
-    def __init__(self, W: torch.Tensor, keep_rowmajor: bool = False):
-        """keep_rowmajor: also keep the row-major matrix, which lets `linear` hand prefill-sized products (T > 64) to
-        the vendor GEMM library (one more copy of the weight)."""
+    def __init__(self, W: torch.Tensor):
         N, K = W.shape
         self.N, self.K = N, K
         n = lib().mlora_packed_weight_elems(N, K)
         self.data = torch.empty(n, dtype=torch.float16, device=W.device)
         check(lib().mlora_pack_weight(_dev(self.data), _dev(W, torch.float16, "W"), N, K, _stream()))
-        self.rowmajor = W.contiguous() if keep_rowmajor else None
 
     @property
     def shape(self):
@@ -286,22 +283,9 @@ class PackedWeight:
         return v.permute(0, 3, 1, 2, 4).reshape(nt * 16, self.K)[: self.N].contiguous()
 
 
-LIBRARY_GEMM_MIN_T = 65       # up to 64 tokens the weight-streaming decode kernel of this package is used
-_lib_ws = {}
-
-
-def _library_workspace(device) -> torch.Tensor:
-    ws = _lib_ws.get(device)
-    if ws is None:
-        ws = _lib_ws[device] = torch.empty(lib().mlora_gemm_library_workspace_bytes(), dtype=torch.uint8, device=device)
-    return ws
-
-
 def linear(x, W, out=None, out_dtype=torch.float16, accumulate=False, kernel="auto"):
     """y (=|+=) x @ W.T.  x [T,K] f16 (row stride may exceed K) or a FragActivation, W [N,K] f16 or a
-    PackedWeight.  accumulate=True adds into the fp32 tensor `out`.  kernel: "auto" | "gemv" | "gemm" | "library"
-    (the vendor GEMM library on a row-major W; "auto" picks it for T >= 65 when W is row-major-capable, i.e. a
-    PackedWeight built with keep_rowmajor=True)."""
+    PackedWeight.  accumulate=True adds into the fp32 tensor `out`.  kernel: "auto" | "gemv" | "gemm"."""
     if isinstance(x, FragActivation):
         return _linear_frag(x, W, out, out_dtype, accumulate)
     T, K = x.shape
@@ -313,28 +297,6 @@ def linear(x, W, out=None, out_dtype=torch.float16, accumulate=False, kernel="au
         if out is None:
             out = torch.empty((0, N), dtype=torch.float32 if accumulate else out_dtype, device=x.device)
         return out
-    rm = W.rowmajor if packed else W
-    if kernel == "library" or (kernel == "auto" and packed and rm is not None and T >= LIBRARY_GEMM_MIN_T
-                               and K % 8 == 0 and N % 8 == 0):
-        if rm is None:
-            raise ValueError("linear: the library kernel needs a row-major weight (PackedWeight(..., keep_rowmajor=True))")
-        if not x.is_cuda or x.dtype != torch.float16 or x.stride(1) != 1:
-            raise ValueError("linear: x must be a GPU fp16 tensor with unit inner stride")
-        if out is None:
-            if accumulate:
-                raise ValueError("linear: accumulate needs out")
-            out = torch.empty((T, N), dtype=out_dtype, device=x.device)
-        if out.shape != (T, N):
-            raise ValueError(f"linear: out{tuple(out.shape)} expected {(T, N)}")
-        ws = _library_workspace(x.device)
-        ldx = x.stride(0) if T > 1 else max(K, x.stride(0))
-        rc = lib().mlora_gemm_library(_dev(out), _dt(out), ACCUMULATE if accumulate else STORE, x.data_ptr(), ldx,
-                                      _dev(rm, torch.float16, "W"), T, K, N, ws.data_ptr(), ws.numel(), _stream())
-        if rc == -2 and kernel == "auto" and packed:      # the vendor library has no algorithm for this shape: own GEMM
-            kernel = "gemm"
-        else:
-            check(rc)
-            return out
     if not x.is_cuda or x.dtype != torch.float16 or x.stride(1) != 1:
         raise ValueError("linear: x must be a GPU fp16 tensor with unit inner stride")
     ldx = x.stride(0) if T > 1 else max(K, x.stride(0))

@@ -19,10 +19,10 @@ def oracle_model(wl, mode="mixed", lora_specs=None):
     return oracle.LlamaRef(wl.shape, w, lora, scaling, mode=mode)
 
 
-def hip_model(wl, lora_specs=None, device="cuda:0", library_gemm=False):
+def hip_model(wl, lora_specs=None, device="cuda:0"):
     llama = load_pkg("llama")
     specs = [wl.lora] if lora_specs is None else lora_specs
-    return llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, specs, device, library_gemm=library_gemm)
+    return llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, specs, device)
 
 
 def n_pages_for(wl, max_gen_len):

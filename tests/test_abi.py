@@ -129,13 +129,6 @@ def test_argument_validation_of_fused_and_batched_entry_points():
     assert nk(2, None, 4096) == -1 and nk(2, 1, 1024) == -1 and nk(5, 1, 4096) == -1
     assert lib.mlora_rmsnorm_ksplit(1, 0, 1, 1, 2, 4096, 1, 1e-5, 4, 4096, 1, 1, 1, 1, 0.5, 4096, 16, 4, None) == -1   # dense partials need wider ld
     assert lib.mlora_rmsnorm_ksplit(1, 0, 1, 1, 2, 16384, 1, 1e-5, 4, 16384, None, 0, None, None, 0.0, 0, 0, 0, None) == -2   # H > 8192
-    # vendor-library GEMM: shape checks happen before any library call
-    assert lib.mlora_gemm_library_workspace_bytes() >= 1 << 20
-    assert lib.mlora_gemm_library(None, 0, 0, 1, 64, 1, 256, 64, 64, None, 0, None) == -1
-    assert lib.mlora_gemm_library(1, 0, 1, 1, 64, 1, 256, 64, 64, None, 0, None) == -2      # accumulate into fp16
-    assert lib.mlora_gemm_library(1, 0, 0, 1, 64, 1, 256, 60, 64, None, 0, None) == -2      # K % 8
-    assert lib.mlora_gemm_library(1, 0, 0, 1, 64, 1, 256, 64, 64, None, 4096, None) == -3   # bytes without a buffer
-    assert lib.mlora_gemm_library(1, 0, 0, 1, 64, 1, 0, 64, 64, None, 0, None) == 0
     # decode step: a plan without layers / with a token count beyond the decode tile
     plan = lm.DecodePlan()
     assert lib.mlora_decode_step(C.byref(plan), None) < 0

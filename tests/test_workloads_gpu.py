@@ -51,10 +51,8 @@ def _hip_prefill(model, prompts, wids, n_pages, page_size, perm, max_len):
     return kv, logits.cpu().numpy()
 
 
-@pytest.mark.parametrize("library_gemm", [False, True])
-def test_prefill_rank64_all_linears_adapter_segments(library_gemm):
-    """Five ragged prompts in three adapter segments, rank-64 LoRA on q, k, v, o, gate, up, down; base linears (248
-    tokens) on this package's GEMM and on the vendor GEMM library."""
+def test_prefill_rank64_all_linears_adapter_segments():
+    """Five ragged prompts in three adapter segments, rank-64 LoRA on q, k, v, o, gate, up, down (248 tokens)."""
     synth = load_pkg("synth")
     shape = _small_shape(synth)
     lora = synth.LoraSpec(r=64, alpha=32.0, n_adapters=6, targets=synth.LINEARS)
@@ -65,7 +63,7 @@ def test_prefill_rank64_all_linears_adapter_segments(library_gemm):
     n_pages = sum(-(-n // 16) for n in lens) + 4
     perm = synth.permutation(3, "c4s.pages", n_pages)
     tok_ids = {"a0": np.repeat(wl.adapter_ids, lens)}
-    model = hip_model(wl, library_gemm=library_gemm)
+    model = hip_model(wl)
     kvh, got = _hip_prefill(model, prompts, wl.adapter_ids, n_pages, 16, perm, 96)
     for mode, tol in (("mixed", 1e-2), ("fp32", 1.5e-2)):
         kvr, exp = _oracle_prefill(oracle_model(wl, mode), prompts, tok_ids, n_pages, 16, perm, 96)
