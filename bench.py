@@ -366,7 +366,7 @@ def bench_c4_prefill(args, synth, llama):
         "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": wl.name, "layers": L, "tokens": T, "segments": int(len(np.unique(wids))), "rank": wl.lora.r,
                    "lora_targets": list(wl.lora.targets),
-                   "base_gemm": "gemm_lds_kernel (this package)"},
+                   "base_gemm": "gemm_pp_kernel (this package), activations in fragment order"},
         "roofline": {"kernel": "whole prefill pass (base GEMMs 97 % of the flops)", "bound": "mfma", "achieved": flops / dt / 1e12,
                      "peak": 2500.0, "unit": "TFLOP/s", "frac": flops / dt / 1e12 / 2500.0, "traffic": None,
                      "flops_base": flops_base, "flops_lora": flops_lora, "flops_attention": flops_attn}}))

@@ -39,11 +39,13 @@ extern "C" {
 #define MLORA_ACCUMULATE  1
 
 /* Activation layouts.  MLORA_ROWMAJOR: x[T, K], innermost contiguous.  MLORA_FRAG: the order in which the
- * matrix cores consume the token block of a decode step (T <= 64),
- *     Xf[k/32][t/16][(k%32)/8][t%16][k%8]     with TT = 1, 2 or 4 sixteen-token tiles for T <= 16, 32, 64,
+ * matrix cores consume a token block,
+ *     Xf[k/32][t/16][(k%32)/8][t%16][k%8]     with TT sixteen-token tiles per 32-k step: TT = 1, 2 or 4 for
+ *                                             T <= 16, 32, 64 and ceil(T / 16) beyond,
  * so that the 16-token x 32-k operand fragment is one contiguous 1 KiB block; mlora_frag_activation_elems
- * gives the buffer size.  Producers (RMSNorm, SiLU*mul, decode attention) can write it directly, the decode
- * GEMV (mlora_gemv_frag) and the LoRA shrink read it; rows t >= T of the last tile are never read back. */
+ * gives the buffer size.  Producers (RMSNorm, SiLU*mul, attention) can write it directly; the decode GEMV, the
+ * persistent prefill GEMM (mlora_linear_frag) and the LoRA shrink read it.  Rows t >= T of the last tile hold
+ * whatever the buffer held: they reach only outputs that are never stored. */
 #define MLORA_ROWMAJOR 0
 #define MLORA_FRAG     1
 
@@ -196,13 +198,21 @@ int mlora_gemm_packed(void* y, int y_dtype, int mode, const void* x, int ldx, co
 int mlora_linear_packed(void* y, int y_dtype, int mode, const void* x, int ldx, const void* Wp,
                         int T, int K, int N, void* stream);
 
-/* Decode GEMV with both operands in fragment order: Wp as above, xf in MLORA_FRAG layout (T <= 64).  Every
- * operand load of the kernel is then a contiguous 1 KiB block.  mlora_pack_activation converts a row-major
- * x (row stride ldsrc) into fragment order for callers whose producer cannot write it directly. */
+/* Linear with both operands in fragment order: Wp as above, xf in MLORA_FRAG layout.  Every operand load of
+ * the kernel is then a contiguous 1 KiB block.  mlora_pack_activation converts a row-major x (row stride ldsrc)
+ * into fragment order for callers whose producer cannot write it directly.
+ * mlora_gemv_frag: the decode GEMV, T <= 64.  mlora_linear_frag: any T - the GEMV up to 64 tokens, beyond that
+ * the persistent matrix-core GEMM (needs K % 64 == 0), which copies both operands from global memory straight
+ * into LDS.  mlora_gemm_frag_preferred says whether that GEMM is the efficient choice for a shape (at least
+ * one 256 x 256 output block per compute unit); callers use it to decide which layout their producers write.
+ * Replaces, like the other linears: nn.Linear(bias=False) (llama_for_causal_lm.py:26-38,58-62). */
 size_t mlora_frag_activation_elems(int T, int K);
 int mlora_pack_activation(void* dst, const void* src, int ldsrc, int T, int K, void* stream);
 int mlora_gemv_frag(void* y, int y_dtype, int mode, const void* xf, const void* Wp,
                     int T, int K, int N, void* stream);
+int mlora_linear_frag(void* y, int y_dtype, int mode, const void* xf, const void* Wp,
+                      int T, int K, int N, void* stream);
+int mlora_gemm_frag_preferred(int T, int K, int N);
 
 /* y[t, :] = f16( x[t, :] * rsqrt(mean(x[t, :]^2) + eps) * w )   row-wise, statistics in fp32.
  * Replaces: nn.RMSNorm(hidden, -1, eps, bias=False) (llama_for_causal_lm.py:76-77,93).
@@ -243,7 +253,7 @@ int mlora_argmax(int32_t* ids, const float* logits, int B, int V, void* stream);
  *   first ctx_len[b] cached positions of sequence seq_ids[b] (the new token already appended).
  * mlora_paged_attn_prefill: query token t (sequence tok_seq[t], position tok_pos[t]) attends to cached
  *   positions 0..tok_pos[t]; tokens of a sequence must be consecutive in t with increasing positions.
- * q is read from qkv (already rotated).  out [T, Hq * D] f16 (decode: in out_layout).  D in {64, 128};
+ * q is read from qkv (already rotated).  out [T, Hq * D] f16 in out_layout.  D in {64, 128};
  * Hq % Hkv == 0, Hq / Hkv <= 16 and B <= 65535 for decode.
  * ------------------------------------------------------------------------------------------- */
 int mlora_rope_kv_append(void* qkv, void* k_cache, void* v_cache,
@@ -255,7 +265,7 @@ int mlora_paged_attn_decode(void* out, int out_layout, const void* qkv, const vo
                             const int32_t* block_table, int max_blocks,
                             const int32_t* seq_ids, const int32_t* ctx_len,
                             int B, int Hq, int Hkv, int D, int n_pages, int n_seq, void* stream);
-int mlora_paged_attn_prefill(void* out, const void* qkv, const void* k_cache, const void* v_cache,
+int mlora_paged_attn_prefill(void* out, int out_layout, const void* qkv, const void* k_cache, const void* v_cache,
                              const int32_t* block_table, int max_blocks,
                              const int32_t* tok_seq, const int32_t* tok_pos,
                              int T, int Hq, int Hkv, int D, int n_pages, int n_seq, void* stream);

@@ -42,6 +42,8 @@ SIGNATURES = {
     "mlora_frag_activation_elems": (_z, [_i, _i]),
     "mlora_pack_activation": (_i, [_p, _p, _i, _i, _i, _p]),
     "mlora_gemv_frag": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p]),
+    "mlora_linear_frag": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p]),
+    "mlora_gemm_frag_preferred": (_i, [_i, _i, _i]),
     "mlora_gemv_frag_lora": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _i, _p, _i, _i, _p]),
     "mlora_gemv_frag_silu": (_i, [_p, _p, _p, _i, _i, _i, _p]),
     "mlora_gemv_frag_split": (_i, [_p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _p]),
@@ -60,7 +62,7 @@ SIGNATURES = {
     "mlora_argmax": (_i, [_p, _p, _i, _i, _p]),
     "mlora_rope_kv_append": (_i, [_p, _p, _p, _p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
     "mlora_paged_attn_decode": (_i, [_p, _i, _p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
-    "mlora_paged_attn_prefill": (_i, [_p, _p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
+    "mlora_paged_attn_prefill": (_i, [_p, _i, _p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
 }
 
 

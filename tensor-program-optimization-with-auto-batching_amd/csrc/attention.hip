@@ -658,7 +658,7 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
 // pass per sequence with the other queries masked.
 // ---------------------------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256) void paged_attn_prefill_kernel(f16* __restrict__ out, const f16* __restrict__ qkv,
+__global__ __launch_bounds__(256) void paged_attn_prefill_kernel(f16* __restrict__ out, int frag_tt, const f16* __restrict__ qkv,
                                                                  const f16* __restrict__ k_cache,
                                                                  const f16* __restrict__ v_cache,
                                                                  const int32_t* __restrict__ block_table, int max_blocks,
@@ -771,7 +771,10 @@ __global__ __launch_bounds__(256) void paged_attn_prefill_kernel(f16* __restrict
     const int t = t0 + 4 * g + r;
     if (t < T) {
 #pragma unroll
-      for (int db = 0; db < NDB; ++db) out[((size_t)t * Hq + h) * D + db * 16 + qi] = (f16)(O[db][r] * ir);
+      for (int db = 0; db < NDB; ++db) {
+        const int c = h * D + db * 16 + qi;
+        out[frag_tt ? frag_offset(t, c, frag_tt) : (size_t)t * Hq * D + c] = (f16)(O[db][r] * ir);
+      }
     }
   }
 }
@@ -937,22 +940,24 @@ extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv
   return mlora_launch_status("rope_attn_decode");
 }
 
-extern "C" int mlora_paged_attn_prefill(void* out, const void* qkv, const void* k_cache, const void* v_cache,
+extern "C" int mlora_paged_attn_prefill(void* out, int out_layout, const void* qkv, const void* k_cache, const void* v_cache,
                                         const int32_t* block_table, int max_blocks, const int32_t* tok_seq,
                                         const int32_t* tok_pos, int T, int Hq, int Hkv, int D, int n_pages, int n_seq,
                                         void* stream) {
   if (int e = check_attn("paged_attn_prefill", Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
   MLORA_CHECK(out && qkv && k_cache && v_cache && block_table && tok_seq && tok_pos, MLORA_ERR_INVALID, "paged_attn_prefill: null pointer");
   MLORA_CHECK(T >= 0, MLORA_ERR_INVALID, "paged_attn_prefill: bad T=%d", T);
+  MLORA_CHECK(out_layout == MLORA_ROWMAJOR || out_layout == MLORA_FRAG, MLORA_ERR_INVALID, "paged_attn_prefill: bad out_layout %d", out_layout);
   if (T == 0) return MLORA_OK;
+  const int frag_tt = out_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   const float scale = 1.f / sqrtf((float)D);
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(ceil_div(T, 64), Hq);
   if (D == 128)
-    hipLaunchKernelGGL(paged_attn_prefill_kernel<128>, grid, dim3(256), 0, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
+    hipLaunchKernelGGL(paged_attn_prefill_kernel<128>, grid, dim3(256), 0, s, (f16*)out, frag_tt, (const f16*)qkv, (const f16*)k_cache,
                        (const f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, T, Hq, Hkv, n_pages, n_seq, scale);
   else
-    hipLaunchKernelGGL(paged_attn_prefill_kernel<64>, grid, dim3(256), 0, s, (f16*)out, (const f16*)qkv, (const f16*)k_cache,
+    hipLaunchKernelGGL(paged_attn_prefill_kernel<64>, grid, dim3(256), 0, s, (f16*)out, frag_tt, (const f16*)qkv, (const f16*)k_cache,
                        (const f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, T, Hq, Hkv, n_pages, n_seq, scale);
   return mlora_launch_status("paged_attn_prefill");
 }

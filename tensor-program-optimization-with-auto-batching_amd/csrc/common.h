@@ -38,7 +38,7 @@ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // 16-token tiles of the fragment-ordered activation layout: the tile count the decode GEMV is compiled
 // for (1, 2 or 4), so that producer and consumer agree on the stride between k-steps.
-static inline int mlora_frag_tiles(int T) { return T <= 16 ? 1 : (T <= 32 ? 2 : 4); }
+static inline int mlora_frag_tiles(int T) { return T <= 16 ? 1 : (T <= 32 ? 2 : (T <= 64 ? 4 : (T + 15) / 16)); }
 
 // ---------------------------------------------------------------------------------------------
 // device side

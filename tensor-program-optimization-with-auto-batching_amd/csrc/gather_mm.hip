@@ -461,8 +461,19 @@ __device__ __forceinline__ TileAdapters tile_adapters(int id) {
 // 16 tokens holds up to 16 adapters, costs one K loop instead of 16, with all the groups' loads in flight together.
 // Shrink of one 16-token tile by the four waves of a workgroup: K steps kb0 .. kb1-1 dealt to the waves in turn, the
 // waves' sums added in wave order through `red`, partial result rows written to v [T][R].
+// Where lane (token t, k-group g) finds its 8 k-entries of 32-k step 0, and the distance between consecutive steps:
+// row-major x [T, K] (frag_tt == 0) or fragment order with frag_tt sixteen-token tiles per 32-k step.
+__device__ __forceinline__ const f16* x_operand(const f16* __restrict__ x, int t, int g, int K, int frag_tt, int& step) {
+  if (frag_tt) {
+    step = frag_tt * 512;
+    return x + (size_t)(t >> 4) * 512 + g * 128 + (t & 15) * 8;
+  }
+  step = 32;
+  return x + (size_t)t * K + g * 8;
+}
+
 template <int R>
-__device__ __forceinline__ void shrink_tile_mfma(float* __restrict__ v, const f16* __restrict__ x, const f16* __restrict__ A,
+__device__ __forceinline__ void shrink_tile_mfma(float* __restrict__ v, const f16* __restrict__ x, int frag_tt, const f16* __restrict__ A,
                                                  const int32_t* __restrict__ ids, int T, int K, int n_ad,
                                                  const int32_t* __restrict__ bucket_of, int bucket, int t0, int kb0, int kb1,
                                                  f32x4 (*red)[8][WAVE]) {
@@ -474,7 +485,8 @@ __device__ __forceinline__ void shrink_tile_mfma(float* __restrict__ v, const f1
   const int raw = lora_token_id(ids, bucket_of, bucket, t0 + col, T);
   const int id = (raw >= 0 && raw < n_ad) ? raw : -1;
   const TileAdapters ta = tile_adapters(id);
-  const f16* __restrict__ xr = x + (size_t)tl * K + g * 8;
+  int xstep;
+  const f16* __restrict__ xr = x_operand(x, tl, g, K, frag_tt, xstep);
 #pragma unroll
   for (int g0 = 0; g0 < 16; g0 += GA) {
     if (g0 < ta.n) {                                             // uniform
@@ -484,7 +496,7 @@ __device__ __forceinline__ void shrink_tile_mfma(float* __restrict__ v, const f1
 #pragma unroll
         for (int i = 0; i < NT; ++i) acc[u][i] = f32x4{0.f, 0.f, 0.f, 0.f};
       for (int kb = kb0 + wave; kb < kb1; kb += SEG_WAVES) {
-        const f16x8 xf = ld8(xr + kb * 32);
+        const f16x8 xf = ld8(xr + (size_t)kb * xstep);
         f16x8 af[GA][NT];
 #pragma unroll
         for (int u = 0; u < GA; ++u) {
@@ -531,7 +543,7 @@ __device__ __forceinline__ void shrink_tile_mfma(float* __restrict__ v, const f1
 }
 
 template <int R>
-__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(float* __restrict__ v, const f16* __restrict__ x,
+__global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(float* __restrict__ v, const f16* __restrict__ x, int frag_tt,
                                                                             SegProjs pj,
                                                                             const int32_t* __restrict__ ids, int T, int K,
                                                                             int n_ad, const int32_t* __restrict__ bucket_of,
@@ -546,14 +558,14 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(floa
   const int per = (KB + gridDim.y - 1) / gridDim.y;
   const int kb0 = blockIdx.y * per, kb1 = min(KB, kb0 + per);
   v += ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * T * R;
-  shrink_tile_mfma<R>(v, x, A, ids, T, K, n_ad, bucket_of, bucket, blockIdx.x * 16, kb0, kb1, red);
+  shrink_tile_mfma<R>(v, x, frag_tt, A, ids, T, K, n_ad, bucket_of, bucket, blockIdx.x * 16, kb0, kb1, red);
 }
 
 // Prefill-sized shrink: FOUR token tiles per workgroup.  When all adapted tokens of the four tiles use one adapter (an
 // adapter segment of 64 tokens or more), an A fragment is loaded once per 64 tokens instead of once per 16; otherwise
 // the tiles are worked off one after the other as above.  Same sums, in the same order, either way.
 template <int R>
-__global__ __launch_bounds__(SEG_WAVES * WAVE, 2) void lora_shrink_quad_mfma_kernel(float* __restrict__ v, const f16* __restrict__ x,
+__global__ __launch_bounds__(SEG_WAVES * WAVE, 2) void lora_shrink_quad_mfma_kernel(float* __restrict__ v, const f16* __restrict__ x, int frag_tt,
                                                                                    SegProjs pj,
                                                                                    const int32_t* __restrict__ ids, int T, int K,
                                                                                    int n_ad, const int32_t* __restrict__ bucket_of,
@@ -581,13 +593,14 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE, 2) void lora_shrink_quad_mfma_ker
   const bool same = __ballot(idl == a) == have;
   if (!same) {
     for (int u = 0; u < QT; ++u)
-      if (tq + u * 16 < T) shrink_tile_mfma<R>(v, x, A, ids, T, K, n_ad, bucket_of, bucket, tq + u * 16, kb0, kb1, red);
+      if (tq + u * 16 < T) shrink_tile_mfma<R>(v, x, frag_tt, A, ids, T, K, n_ad, bucket_of, bucket, tq + u * 16, kb0, kb1, red);
     return;
   }
   const f16* __restrict__ Aa = A + (size_t)a * R * K + g * 8;
   const f16* xr[QT];
+  int xstep = 32;
 #pragma unroll
-  for (int u = 0; u < QT; ++u) xr[u] = x + (size_t)min(tq + u * 16 + col, T - 1) * K + g * 8;
+  for (int u = 0; u < QT; ++u) xr[u] = x_operand(x, min(tq + u * 16 + col, T - 1), g, K, frag_tt, xstep);
   f32x4 acc[QT][NT];
 #pragma unroll
   for (int u = 0; u < QT; ++u)
@@ -601,7 +614,7 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE, 2) void lora_shrink_quad_mfma_ker
       af[i] = row < R ? ld8(Aa + (size_t)row * K + kb * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
 #pragma unroll
-    for (int u = 0; u < QT; ++u) xf[u] = ld8(xr[u] + kb * 32);
+    for (int u = 0; u < QT; ++u) xf[u] = ld8(xr[u] + (size_t)kb * xstep);
 #pragma unroll
     for (int u = 0; u < QT; ++u)
 #pragma unroll
@@ -1032,8 +1045,8 @@ struct BucketFilter {
 static int shrink_impl(void* v_part, const void* x, int x_layout, const void* A, const int32_t* tok_adapter,
                        int T, int K, int r, int n_ad, BucketFilter bf, void* stream) {
   if (int e = check_lora_shape(T, K, 8, r, n_ad)) return e;
-  MLORA_CHECK(x_layout == MLORA_ROWMAJOR || (x_layout == MLORA_FRAG && T <= 64 && K % 32 == 0), MLORA_ERR_UNSUPPORTED,
-              "lora_shrink: fragment-ordered x needs T <= 64 and K %% 32 == 0 (layout=%d T=%d K=%d)", x_layout, T, K);
+  MLORA_CHECK(x_layout == MLORA_ROWMAJOR || (x_layout == MLORA_FRAG && K % 32 == 0), MLORA_ERR_UNSUPPORTED,
+              "lora_shrink: fragment-ordered x needs K %% 32 == 0 (layout=%d K=%d)", x_layout, K);
   MLORA_CHECK(v_part && x && A && tok_adapter, MLORA_ERR_INVALID, "lora_shrink: null pointer");
   if (T == 0) return MLORA_OK;
   const LoraKSplit ks = lora_k_split(K);
@@ -1170,7 +1183,7 @@ extern "C" int mlora_gather_mm_batch(const void* const* sets, int n_sets, int y_
 }
 
 template <int R>
-static void gmm_segments_r(const SegProjs& pj, int y_dtype, int ldy, const f16* x, const int32_t* ids, float scaling, int T, int K,
+static void gmm_segments_r(const SegProjs& pj, int y_dtype, int ldy, const f16* x, int frag_tt, const int32_t* ids, float scaling, int T, int K,
                            int n_ad, float* v, BucketFilter bf, hipStream_t s) {
   const int tiles = ceil_div(T, 16);
   int N = 0;
@@ -1188,16 +1201,16 @@ static void gmm_segments_r(const SegProjs& pj, int y_dtype, int ldy, const f16* 
   // workgroup, about two workgroups per compute unit.  Either set of kernels is correct for either input.
   const bool mixed = T <= 1024;
   if (mixed) {
-    hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles, splits, pj.n), dim3(SEG_WAVES * WAVE), 0, s, v, x, pj, ids, T, K, n_ad,
-                       bf.bucket_of, bf.bucket);
+    hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles, splits, pj.n), dim3(SEG_WAVES * WAVE), 0, s, v, x, frag_tt, pj, ids, T, K,
+                       n_ad, bf.bucket_of, bf.bucket);
   } else {
     const int quads = ceil_div(tiles, 4);
     splits = 256 / quads;                        // few K ranges: the expand adds the ranges' partial sums per token
     if (splits > kc) splits = kc;
     if (splits > K / 128) splits = K / 128;
     if (splits < 1) splits = 1;
-    hipLaunchKernelGGL((lora_shrink_quad_mfma_kernel<R>), dim3(quads, splits, pj.n), dim3(SEG_WAVES * WAVE), 0, s, v, x, pj, ids, T, K,
-                       n_ad, bf.bucket_of, bf.bucket);
+    hipLaunchKernelGGL((lora_shrink_quad_mfma_kernel<R>), dim3(quads, splits, pj.n), dim3(SEG_WAVES * WAVE), 0, s, v, x, frag_tt, pj, ids, T,
+                       K, n_ad, bf.bucket_of, bf.bucket);
   }
   // column blocks per workgroup: as many as leave about a thousand workgroups (per-workgroup set-up amortised)
   int nit = (int)(((long)tiles * pj.n * ceil_div(N, SEG_WAVES * 64)) / 1024);
@@ -1222,20 +1235,21 @@ static void gmm_segments_r(const SegProjs& pj, int y_dtype, int ldy, const f16* 
 }
 
 // shrink + expand on the matrix cores for pj.n projections; v = workspace viewed as [pj.n][splits][T, r] fp32
-static int gmm_segments(const SegProjs& pj, int y_dtype, int ldy, const f16* x, const int32_t* ids, float scaling, int T, int K,
+static int gmm_segments(const SegProjs& pj, int y_dtype, int ldy, const f16* x, int x_layout, const int32_t* ids, float scaling, int T, int K,
                         int r, int n_ad, float* v, BucketFilter bf, hipStream_t s) {
+  const int frag_tt = x_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   switch (r) {
-    case 8: gmm_segments_r<8>(pj, y_dtype, ldy, x, ids, scaling, T, K, n_ad, v, bf, s); break;
-    case 16: gmm_segments_r<16>(pj, y_dtype, ldy, x, ids, scaling, T, K, n_ad, v, bf, s); break;
-    case 32: gmm_segments_r<32>(pj, y_dtype, ldy, x, ids, scaling, T, K, n_ad, v, bf, s); break;
-    default: gmm_segments_r<64>(pj, y_dtype, ldy, x, ids, scaling, T, K, n_ad, v, bf, s); break;
+    case 8: gmm_segments_r<8>(pj, y_dtype, ldy, x, frag_tt, ids, scaling, T, K, n_ad, v, bf, s); break;
+    case 16: gmm_segments_r<16>(pj, y_dtype, ldy, x, frag_tt, ids, scaling, T, K, n_ad, v, bf, s); break;
+    case 32: gmm_segments_r<32>(pj, y_dtype, ldy, x, frag_tt, ids, scaling, T, K, n_ad, v, bf, s); break;
+    default: gmm_segments_r<64>(pj, y_dtype, ldy, x, frag_tt, ids, scaling, T, K, n_ad, v, bf, s); break;
   }
   return mlora_launch_status("gather_mm");
 }
 
-// the matrix-core kernels need row-major x, 16-byte aligned rows of y and whole 16-column tiles
+// the matrix-core kernels need 16-byte aligned rows of y and whole 16-column tiles
 static bool gmm_segments_fit(const void* y, int ldy, int x_layout, int T, int K, int N) {
-  return x_layout == MLORA_ROWMAJOR && T > 64 && K % 32 == 0 && N % 16 == 0 && ldy % 8 == 0 && (uintptr_t)y % 16 == 0;
+  return (x_layout == MLORA_ROWMAJOR || x_layout == MLORA_FRAG) && T > 64 && K % 32 == 0 && N % 16 == 0 && ldy % 8 == 0 && (uintptr_t)y % 16 == 0;
 }
 
 static int gather_mm_impl(void* y, int y_dtype, int ldy, const void* x, int x_layout, const void* A, const void* B,
@@ -1251,7 +1265,7 @@ static int gather_mm_impl(void* y, int y_dtype, int ldy, const void* x, int x_la
     MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "gather_mm: bad y_dtype %d", y_dtype);
     MLORA_CHECK(ldy >= N, MLORA_ERR_INVALID, "gather_mm: need ldy >= N (ldy=%d N=%d)", ldy, N);
     MLORA_CHECK(x_layout == MLORA_ROWMAJOR || (x_layout == MLORA_FRAG && K % 32 == 0), MLORA_ERR_UNSUPPORTED,
-                "gather_mm: fragment-ordered x needs T <= 64 and K %% 32 == 0 (layout=%d T=%d K=%d)", x_layout, T, K);
+                "gather_mm: fragment-ordered x needs K %% 32 == 0 (layout=%d K=%d)", x_layout, K);
     const GmmSet one = {y, (const f16*)x, (const f16*)A, (const f16*)B};
     return gmm_one_launch(one, nullptr, 1, y_dtype, ldy, x_layout, tok_adapter, scaling, T, K, N, r, n_ad, (hipStream_t)stream, bf);
   }
@@ -1261,7 +1275,7 @@ static int gather_mm_impl(void* y, int y_dtype, int ldy, const void* x, int x_la
     MLORA_CHECK(ldy >= N, MLORA_ERR_INVALID, "gather_mm: need ldy >= N (ldy=%d N=%d)", ldy, N);
     SegProjs pj = {};
     pj.A[0] = (const f16*)A; pj.B[0] = (const f16*)B; pj.y[0] = y; pj.N[0] = N; pj.n = 1;
-    return gmm_segments(pj, y_dtype, ldy, (const f16*)x, tok_adapter, scaling, T, K, r, n_ad, (float*)workspace, bf,
+    return gmm_segments(pj, y_dtype, ldy, (const f16*)x, x_layout, tok_adapter, scaling, T, K, r, n_ad, (float*)workspace, bf,
                         (hipStream_t)stream);
   }
   if (int e = shrink_impl(workspace, x, x_layout, A, tok_adapter, T, K, r, n_ad, bf, stream)) return e;
@@ -1447,7 +1461,7 @@ extern "C" int mlora_gather_mm_multi_proj(void* y, int y_dtype, int ldy, const v
       members[pj.n++] = p;
     }
     if (pj.n >= 2 && workspace_bytes >= (size_t)pj.n * mlora_gather_mm_workspace_bytes(T, K, lead->r)) {
-      if (int e = gmm_segments(pj, y_dtype, ldy, (const f16*)x, tok_adapter, lead->scaling, T, K, lead->r, lead->n_ad,
+      if (int e = gmm_segments(pj, y_dtype, ldy, (const f16*)x, x_layout, tok_adapter, lead->scaling, T, K, lead->r, lead->n_ad,
                                (float*)workspace, BucketFilter{tok_bucket, b}, (hipStream_t)stream))
         return e;
       for (int i = 0; i < pj.n; ++i) done[members[i] * n_buckets + b] = true;

@@ -1,10 +1,16 @@
 // Prefill-time base linear for gfx950:  y[T, N] (=|+=) x[T, K] . W[N, K]^T  for any T (MFMA-bound).
 //
-// Both operands are K-contiguous, which is the layout v_mfma_f32_16x16x32_f16 wants for its A and B
-// fragments (a lane holds 8 consecutive k of one row), so fragments are loaded straight from global
-// memory with 16-byte loads and reuse comes from the register tile: a wave owns a 64 x 64 output tile
-// (4 x 4 MFMA tiles, 16 MFMAs per 8 fragment loads), a workgroup of 4 waves owns 128 x 128, and the
-// next k-step's fragments are in flight while the current one is multiplied.
+// Three kernels, by operand layout and problem size:
+//   gemm_kernel      row-major or fragment-ordered W, fragments loaded straight from global memory into registers
+//                    (both operands are K-contiguous, which is what v_mfma_f32_16x16x32_f16 wants: a lane holds 8
+//                    consecutive k of one row); a wave owns 64 x 64 outputs.  Any shape; the small-T workhorse.
+//   gemm_lds_kernel  fragment-ordered W, register-staged LDS double buffer; 256 x 64 or 256 x 256 blocks.
+//   gemm_pp_kernel   fragment-ordered W and row-major or fragment-ordered x, both copied from global memory straight
+//                    into a four-stage LDS ring; persistent 256 x 256 blocks, eight waves.  The large-T kernel.
+// All three add the 32-k MFMA steps of an output in ascending k into one accumulator, so their results are the same
+// bits.
+#include <type_traits>
+
 #include "common.h"
 
 int mlora_check_linear(const char* who, const void* y, int y_dtype, int mode, const void* x, int ldx, const void* W,
@@ -13,6 +19,16 @@ int mlora_check_linear(const char* who, const void* y, int y_dtype, int mode, co
 namespace {
 
 enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2 };
+
+// compute units of the current device (0 if it cannot be asked), read once
+int gemm_n_cu() {
+  static const int n_cu = [] {
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cu = 0;
+    return cu;
+  }();
+  return n_cu;
+}
 
 constexpr int WT = 4;   // 16-wide MFMA tiles per wave along N and along T
 
@@ -238,6 +254,230 @@ __global__ __launch_bounds__(256) void gemm_lds_kernel(void* __restrict__ yv, co
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Eight-wave persistent variant for large token counts.  A workgroup owns 256 tokens x 256 weight rows at a time, a
+// wave 64 tokens x 128 rows of it (4 x 8 MFMA tiles, 128 accumulator registers), two waves per SIMD, one workgroup
+// per compute unit, which walks through its share of the output blocks.
+//   * Both operands go from global memory straight into LDS (global_load_lds_dwordx4: no register staging, no LDS
+//     store instructions) in fragment order, through a ring of four 32-k stages with three stages in flight ahead of
+//     the one being multiplied.  A weight fragment is copied as it lies in memory.  A token fragment likewise when the
+//     activations come in fragment order (x_tt > 0: Xf[k/32][t/16][4][16][8], one contiguous 1 KiB block per
+//     fragment); from row-major activations it is gathered 16 rows x 64 bytes by the load's per-lane addresses - half
+//     cache lines, which costs the load path a third of its speed.
+//   * The ring runs on across block boundaries: while the last stages of a block are multiplied and its results are
+//     stored, the first stages of the workgroup's next block are already in flight.
+//   * Fragment registers are double-buffered: the LDS reads of stage g + 1 are issued right before the MFMAs of stage
+//     g and complete under them.
+//   * fp16 results cross a small LDS buffer so that a store instruction writes whole 128-byte lines of a token row.
+// Blocks are numbered so that an XCD (workgroup id mod 8) works through a contiguous range of weight-row blocks, all
+// token blocks of one weight block next to each other: every XCD streams its own share of W through its L2 once.
+// ---------------------------------------------------------------------------------------------
+constexpr int PP_WAVES = 8;
+constexpr int PP_STAGES = 4;
+constexpr int PP_F = 16;                       // 16-row fragments per block side (256 tokens, 256 weight rows)
+constexpr int PP_STAGE_ELEMS = 2 * PP_F * 512; // fp16 elements of one 32-k stage: 16 weight fragments, then 16 token fragments
+constexpr int PP_OUT_LD = 64 + 4;              // fp16 elements per token row of a wave's output staging (padded: conflict-free writes)
+constexpr int PP_OUT_ELEMS = 16 * PP_OUT_LD;   // per wave: 16 tokens x 64 columns
+
+template <int OUT>
+__global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx, int x_tt,
+                                                                   const f16* __restrict__ Wp, int T, int K, int N, int gx, int gy) {
+  extern __shared__ __align__(16) f16 smem[];  // [PP_STAGES][PP_STAGE_ELEMS], then [PP_WAVES][PP_OUT_ELEMS]
+  constexpr int NW = PP_WAVES;
+  constexpr int LQ = 2 * PP_F / NW;            // fragments a wave fetches per stage (4)
+  constexpr int WTF = 4;                       // token fragments of a wave's tile (64 tokens)
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int nb = gx * gy;
+  const int KB = K / 32;
+  const int tiles = (N + 15) / 16;
+  const int G = gridDim.x;
+
+  // block number -> (weight-row block, token block)
+  auto block_of = [&](int L, int& n0, int& t0) {
+    int idx = L;
+    if ((nb & 7) == 0 && (G & 7) == 0) idx = (L & 7) * (nb >> 3) + (L >> 3);
+    n0 = (idx / gy) * (PP_F * 16);
+    t0 = (idx % gy) * (PP_F * 16);
+  };
+
+  // ---- loader role: wave w fetches fragments 4 w .. 4 w + 3 of every stage (waves 0-3: weights, waves 4-7: tokens)
+  const f16* src[LQ];
+  int step = 0;                                // elements between consecutive k-steps of this wave's sources
+  int load_L = blockIdx.x, load_kb = 0;        // the stage the loader issues next
+  auto load_block = [&](int L) {
+    int n0, t0;
+    block_of(L < nb ? L : blockIdx.x, n0, t0); // past the last block: valid addresses, the data is never multiplied
+    if (wave < NW / 2) {
+#pragma unroll
+      for (int q = 0; q < LQ; ++q) {
+        int nt = n0 / 16 + wave * LQ + q;
+        nt = nt < tiles ? nt : tiles - 1;      // rows past N: a valid fragment, results dropped
+        src[q] = Wp + (size_t)nt * KB * 512 + lane * 8;
+      }
+      step = 512;
+    } else if (x_tt > 0) {
+#pragma unroll
+      for (int q = 0; q < LQ; ++q) {
+        int tt = t0 / 16 + (wave - NW / 2) * LQ + q;
+        tt = tt < x_tt ? tt : x_tt - 1;
+        src[q] = x + (size_t)tt * 512 + lane * 8;
+      }
+      step = x_tt * 512;
+    } else {
+#pragma unroll
+      for (int q = 0; q < LQ; ++q) {
+        int t = t0 + ((wave - NW / 2) * LQ + q) * 16 + (lane & 15);
+        t = t < T ? t : T - 1;
+        src[q] = x + (size_t)t * ldx + (lane >> 4) * 8;
+      }
+      step = 32;
+    }
+  };
+  int ring = 0;                                // ring slot of the stage issued next
+  auto issue = [&]() {
+    f16* dst = smem + ring * PP_STAGE_ELEMS + wave * LQ * 512;
+#pragma unroll
+    for (int q = 0; q < LQ; ++q)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + (size_t)load_kb * step),
+                                       (__attribute__((address_space(3))) void*)(dst + q * 512), 16, 0, 0);
+    ring = (ring + 1) & (PP_STAGES - 1);
+    if (++load_kb == KB) {                     // uniform
+      load_kb = 0;
+      load_L += G;
+      load_block(load_L);
+    }
+  };
+
+  // ---- compute role: rows wn * 128 .., tokens wt * 64 ..
+  const int wn = wave & 1, wt = wave >> 1;
+  f32x4 acc[8][WTF];
+  f16x8 a[2][8], b[2][WTF];
+  int rd = 0;                                  // ring slot of the stage whose fragments are read next
+  auto read_frags = [&](auto U) {
+    constexpr int u = decltype(U)::value;
+    const f16* st = smem + rd * PP_STAGE_ELEMS + lane * 8;
+#pragma unroll
+    for (int j = 0; j < WTF; ++j) b[u][j] = ld8(st + (PP_F + wt * WTF + j) * 512);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[u][i] = ld8(st + (wn * 8 + i) * 512);
+    rd = (rd + 1) & (PP_STAGES - 1);
+  };
+  auto multiply = [&](auto U) {
+    constexpr int u = decltype(U)::value;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < WTF; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][i], b[u][j], acc[i][j], 0, 0, 0);
+  };
+  // One stage: its successor must be in LDS (this wave's share: at most the two stages issued after it still in flight;
+  // everybody's: the barrier).  The wait also covers this wave's fragment reads of the stage about to be multiplied,
+  // so after the barrier nobody reads that ring slot any more and it is refilled; then the reads of the successor go
+  // out, then the MFMAs.
+  auto stage = [&](auto U) {
+    constexpr int u = decltype(U)::value;
+    asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    issue();
+    read_frags(std::integral_constant<int, 1 - u>());
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(U);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  load_block(load_L);
+  issue();
+  issue();
+  issue();
+  asm volatile("s_waitcnt vmcnt(8)" ::: "memory");     // the first stage of this wave has landed
+  __syncthreads();
+  issue();
+  read_frags(std::integral_constant<int, 0>());
+  f16* ostage = smem + PP_STAGES * PP_STAGE_ELEMS + wave * PP_OUT_ELEMS;
+  const int r16 = lane & 15, g = lane >> 4;
+  for (int L = blockIdx.x; L < nb; L += G) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < WTF; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int kb = 0; kb < KB; kb += 2) {               // KB is even (checked by the launcher): the register sets alternate
+      stage(std::integral_constant<int, 0>());
+      stage(std::integral_constant<int, 1>());
+    }
+    int n0, t0;
+    block_of(L, n0, t0);
+    if constexpr (OUT == OUT_F16) {
+      // 16 tokens x 64 columns at a time through the wave's staging buffer: D[n][t] fragments in, token rows out
+#pragma unroll
+      for (int j = 0; j < WTF; ++j) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const f32x4 sacc = acc[h * 4 + i][j];
+            *reinterpret_cast<f16x4*>(ostage + r16 * PP_OUT_LD + i * 16 + g * 4) = f16x4{(f16)sacc[0], (f16)sacc[1], (f16)sacc[2], (f16)sacc[3]};
+          }
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            const int c = q * 64 + lane;           // 16-byte chunk: token row c / 8, columns (c % 8) * 8 ..
+            const int tr = c >> 3, cc = (c & 7) * 8;
+            const int t = t0 + (wt * WTF + j) * 16 + tr;
+            const int n = n0 + (wn * 8 + h * 4) * 16 + cc;
+            const f16x4 lo = *reinterpret_cast<const f16x4*>(ostage + tr * PP_OUT_LD + cc);
+            const f16x4 hi = *reinterpret_cast<const f16x4*>(ostage + tr * PP_OUT_LD + cc + 4);
+            if (t < T && n + 8 <= N) {
+              st8((f16*)yv + (size_t)t * N + n, f16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
+            } else if (t < T) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                if (n + e < N) ((f16*)yv)[(size_t)t * N + n + e] = lo[e];
+                if (n + 4 + e < N) ((f16*)yv)[(size_t)t * N + n + 4 + e] = hi[e];
+              }
+            }
+          }
+          __builtin_amdgcn_wave_barrier();
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < WTF; ++j) {
+        const int t = t0 + (wt * WTF + j) * 16 + r16;
+        if (t >= T) continue;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int n = n0 + (wn * 8 + i) * 16 + g * 4;
+          if (n >= N) continue;
+          const size_t o = (size_t)t * N + n;
+          if constexpr (OUT == OUT_F32) {
+            *reinterpret_cast<f32x4*>((float*)yv + o) = acc[i][j];
+          } else {
+            f32x4* p = reinterpret_cast<f32x4*>((float*)yv + o);
+            *p = *p + acc[i][j];
+          }
+        }
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the loads issued past the last block must not outlive the workgroup's LDS
+}
+
+template <int OUT>
+int launch_gemm_pp(void* y, const f16* x, int ldx, int x_tt, const f16* Wp, int T, int K, int N, hipStream_t s) {
+  constexpr size_t lds = ((size_t)PP_STAGES * PP_STAGE_ELEMS + (size_t)PP_WAVES * PP_OUT_ELEMS) * sizeof(f16);
+  static bool configured = false;                    // the attribute is per kernel, set once per process
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_pp_kernel<OUT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return mlora_set_error(MLORA_ERR_LAUNCH, "gemm_packed: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    configured = true;
+  }
+  const int gx = ceil_div(N, PP_F * 16), gy = ceil_div(T, PP_F * 16);
+  int n_cu = gemm_n_cu();
+  if (n_cu <= 0) n_cu = 256;
+  const int grid = gx * gy < n_cu ? gx * gy : n_cu;
+  hipLaunchKernelGGL((gemm_pp_kernel<OUT>), dim3(grid), dim3(PP_WAVES * WAVE), lds, s, y, x, ldx, x_tt, Wp, T, K, N, gx, gy);
+  return MLORA_OK;
+}
+
 template <int OUT, int FT, int FN, int WT_, int WN_>
 int launch_gemm_lds(void* y, const f16* x, int ldx, const f16* Wp, int T, int K, int N, hipStream_t s) {
   constexpr size_t lds = 2 * (LBK / 32) * (FT + FN) * 512 * sizeof(f16);
@@ -257,7 +497,11 @@ int launch_gemm_lds(void* y, const f16* x, int ldx, const f16* Wp, int T, int K,
 // over all CUs.
 template <int OUT>
 int launch_gemm_lds_auto(void* y, const f16* x, int ldx, const f16* Wp, int T, int K, int N, hipStream_t s) {
-  if ((long)ceil_div(T, 256) * ceil_div(N, 256) >= 256) return launch_gemm_lds<OUT, 16, 16, 8, 8>(y, x, ldx, Wp, T, K, N, s);
+  if ((long)ceil_div(T, 256) * ceil_div(N, 256) >= 256) {
+    // x rows must be 16-byte aligned for the direct-to-LDS loads (ldx % 8 == 0 is checked; the base may be a slice)
+    if (((uintptr_t)x & 15) == 0 && K % 64 == 0) return launch_gemm_pp<OUT>(y, x, ldx, 0, Wp, T, K, N, s);
+    return launch_gemm_lds<OUT, 16, 16, 8, 8>(y, x, ldx, Wp, T, K, N, s);
+  }
   return launch_gemm_lds<OUT, 16, 4, 4, 4>(y, x, ldx, Wp, T, K, N, s);
 }
 
@@ -308,4 +552,26 @@ extern "C" int mlora_linear_packed(void* y, int y_dtype, int mode, const void* x
                                    int N, void* stream) {
   if (T <= 64) return mlora_gemv_packed(y, y_dtype, mode, x, ldx, Wp, T, K, N, stream);
   return mlora_gemm_packed(y, y_dtype, mode, x, ldx, Wp, T, K, N, stream);
+}
+
+extern "C" int mlora_gemv_frag(void* y, int y_dtype, int mode, const void* xf, const void* Wp, int T, int K, int N, void* stream);
+
+// 256 x 256 output blocks: enough of them to give every compute unit one, and whole pairs of 32-k steps
+extern "C" int mlora_gemm_frag_preferred(int T, int K, int N) {
+  return T > 64 && K > 0 && K % 64 == 0 && N > 0 && (long)ceil_div(T, PP_F * 16) * ceil_div(N, PP_F * 16) >= 256;
+}
+
+extern "C" int mlora_linear_frag(void* y, int y_dtype, int mode, const void* xf, const void* Wp, int T, int K, int N,
+                                 void* stream) {
+  if (T <= 64) return mlora_gemv_frag(y, y_dtype, mode, xf, Wp, T, K, N, stream);
+  if (int e = mlora_check_linear("linear_frag", y, y_dtype, mode, xf, K, Wp, T, K, N)) return e;
+  MLORA_CHECK(K % 64 == 0, MLORA_ERR_UNSUPPORTED, "linear_frag: more than 64 fragment-ordered tokens need K %% 64 == 0 (K=%d)", K);
+  MLORA_CHECK(((uintptr_t)xf & 15) == 0, MLORA_ERR_INVALID, "linear_frag: xf must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  const int tt = mlora_frag_tiles(T);
+  int e;
+  if (mode == MLORA_ACCUMULATE) e = launch_gemm_pp<OUT_ACC_F32>(y, (const f16*)xf, 0, tt, (const f16*)Wp, T, K, N, s);
+  else if (y_dtype == MLORA_F32) e = launch_gemm_pp<OUT_F32>(y, (const f16*)xf, 0, tt, (const f16*)Wp, T, K, N, s);
+  else e = launch_gemm_pp<OUT_F16>(y, (const f16*)xf, 0, tt, (const f16*)Wp, T, K, N, s);
+  return e ? e : mlora_launch_status("linear_frag");
 }

@@ -684,8 +684,8 @@ extern "C" size_t mlora_frag_activation_elems(int T, int K) {
 
 extern "C" int mlora_pack_activation(void* dst, const void* src, int ldsrc, int T, int K, void* stream) {
   MLORA_CHECK(dst && src && dst != src, MLORA_ERR_INVALID, "pack_activation: null or aliasing pointers");
-  MLORA_CHECK(T > 0 && T <= 64 && K > 0 && K % 32 == 0 && ldsrc >= K && ldsrc % 8 == 0, MLORA_ERR_UNSUPPORTED,
-              "pack_activation: need 0 < T <= 64, K %% 32 == 0, ldsrc >= K (T=%d K=%d ldsrc=%d)", T, K, ldsrc);
+  MLORA_CHECK(T > 0 && K > 0 && K % 32 == 0 && ldsrc >= K && ldsrc % 8 == 0 && (size_t)mlora_frag_tiles(T) * 2 * K < 0x7fffffffULL,
+              MLORA_ERR_UNSUPPORTED, "pack_activation: need T > 0, K %% 32 == 0, ldsrc >= K (T=%d K=%d ldsrc=%d)", T, K, ldsrc);
   const int chunks = mlora_frag_tiles(T) * 16 * (K / 8);
   hipLaunchKernelGGL(pack_activation_kernel, dim3(ceil_div(chunks, 256)), dim3(256), 0, (hipStream_t)stream, (f16*)dst,
                      (const f16*)src, ldsrc, T, K, mlora_frag_tiles(T), chunks);

@@ -285,18 +285,121 @@ __global__ __launch_bounds__(ROW_THREADS) void argmax_kernel(int32_t* __restrict
   }
 }
 
+// RMSNorm of one 16-row token tile straight into fragment order, for token blocks of prefill size: wave r of the 16
+// norms row r of the tile (the same sums in the same order as the row kernel above: a lane plays the threads
+// lane, lane + 64, ... of that kernel's 512), the rows' 16-byte pieces meet in LDS, and every wave then writes whole
+// 1 KiB fragments.  (The row kernel would write each fragment 16 bytes at a time from 16 workgroups.)
+constexpr int TILE_PITCH = 128 + 8;    // fp16 elements per (k-step, k-group) slot of the staging buffer: 16 rows x 8, padded
+
+template <typename XT, int MC>
+__global__ __launch_bounds__(1024) void rmsnorm_tile_kernel(f16* __restrict__ y, const XT* __restrict__ x, const f16* __restrict__ w,
+                                                            float eps, int T, int H, int frag_tt) {
+  __shared__ __align__(16) f16 buf[2][64 * TILE_PITCH];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int tt = blockIdx.x, row = tt * 16 + wave;
+  const bool live = row < T;
+  const XT* xr = x + (size_t)(live ? row : 0) * H;
+  const int M = (H + 511) / 512;                      // 512-column blocks of a row (<= MC)
+  float v[MC][8];
+  float ssq[NORM_THREADS / WAVE];
+#pragma unroll
+  for (int q = 0; q < NORM_THREADS / WAVE; ++q) ssq[q] = 0.f;
+#pragma unroll
+  for (int m = 0; m < MC; ++m) {
+    const int c = m * 512 + lane * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[m][e] = 0.f;
+    if (live && c < H) {
+      if constexpr (sizeof(XT) == 2) {
+        const f16x8 t = ld8((const f16*)xr + c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[m][e] = (float)t[e];
+      } else {
+        const f32x4 lo = *reinterpret_cast<const f32x4*>((const float*)xr + c);
+        const f32x4 hi = *reinterpret_cast<const f32x4*>((const float*)xr + c + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[m][e] = lo[e];
+          v[m][4 + e] = hi[e];
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ssq[m % (NORM_THREADS / WAVE)] = fmaf(v[m][e], v[m][e], ssq[m % (NORM_THREADS / WAVE)]);
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int q = 0; q < NORM_THREADS / WAVE; ++q) ss += wave_sum(ssq[q]);
+  const float inv = rsqrtf(ss / (float)H + eps);
+#pragma unroll
+  for (int m = 0; m < MC; ++m) {
+    if (m < M) {                                       // uniform
+      const int c = m * 512 + lane * 8;
+      f16x8 o = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (c < H) {
+        const f16x8 wv = ld8(w + c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (f16)(v[m][e] * inv * (float)wv[e]);
+      }
+      f16* b = buf[m & 1];
+      st8(b + lane * TILE_PITCH + wave * 8, o);        // slot = (k-step within the block) * 4 + k-group = lane
+      __syncthreads();
+      const int ks = m * 16 + wave;                    // this wave's fragment of the block
+      if (ks * 32 < H) st8(y + ((size_t)ks * frag_tt + tt) * 512 + lane * 8, ld8(b + (wave * 4 + (lane >> 4)) * TILE_PITCH + (lane & 15) * 8));
+    }
+  }
+}
+
+// SiLU(gate) * up of a token block of prefill size into fragment order: a wave produces one whole fragment (16 tokens x
+// 32 columns, 1 KiB contiguous), the four waves of a workgroup four neighbouring k-steps, so that the rows are read in
+// runs of 256 bytes.
+__global__ __launch_bounds__(ROW_THREADS) void silu_mul_tile_kernel(f16* __restrict__ out, const f16* __restrict__ gate,
+                                                                    const f16* __restrict__ up, int ld, int T, int I, int frag_tt) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int tt = blockIdx.y, ks = blockIdx.x * (ROW_THREADS / WAVE) + wave;
+  const int c = ks * 32 + (lane >> 4) * 8;
+  if (c >= I) return;
+  const int t = tt * 16 + (lane & 15);
+  f16x8 o = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  if (t < T) {
+    const f16x8 g = ld8(gate + (size_t)t * ld + c);
+    const f16x8 u = ld8(up + (size_t)t * ld + c);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float gf = (float)g[e];
+      o[e] = (f16)(gf / (1.f + expf(-gf)) * (float)u[e]);
+    }
+  }
+  st8(out + ((size_t)ks * frag_tt + tt) * 512 + lane * 8, o);
+}
+
 }  // namespace
 
 static int rmsnorm_impl(const char* who, void* y, int y_layout, void* x, int x_dtype, const void* w, float eps, int T,
                         int H, const LoraExpandRow& lx, void* stream, const KSplitParts& kp = KSplitParts()) {
-  MLORA_CHECK(y_layout == MLORA_ROWMAJOR || (y_layout == MLORA_FRAG && T <= 64 && H % 32 == 0), MLORA_ERR_UNSUPPORTED,
-              "%s: fragment-ordered output needs T <= 64 and H %% 32 == 0 (layout=%d T=%d H=%d)", who, y_layout, T, H);
+  MLORA_CHECK(y_layout == MLORA_ROWMAJOR || (y_layout == MLORA_FRAG && H % 32 == 0), MLORA_ERR_UNSUPPORTED,
+              "%s: fragment-ordered output needs H %% 32 == 0 (layout=%d H=%d)", who, y_layout, H);
   const int frag_tt = y_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   MLORA_CHECK(y && x && w, MLORA_ERR_INVALID, "%s: null pointer", who);
   MLORA_CHECK(T >= 0 && H > 0 && H % 8 == 0 && H <= 16384, MLORA_ERR_UNSUPPORTED, "%s: need H %% 8 == 0, H <= 16384 (T=%d H=%d)", who, T, H);
   MLORA_CHECK(x_dtype == MLORA_F16 || x_dtype == MLORA_F32, MLORA_ERR_INVALID, "%s: bad x_dtype %d", who, x_dtype);
   if (T == 0) return MLORA_OK;
   hipStream_t s = (hipStream_t)stream;
+  if (frag_tt && T > 64 && H <= 4096 && lx.src.v == nullptr && kp.n == 0) {      // a prefill-sized block: whole fragments per store
+#define MLORA_RMS_TILE(XT, MC) \
+  hipLaunchKernelGGL((rmsnorm_tile_kernel<XT, MC>), dim3(frag_tt), dim3(1024), 0, s, (f16*)y, (const XT*)x, (const f16*)w, eps, T, H, frag_tt)
+    if (x_dtype == MLORA_F16) {
+      if (H <= 1024) MLORA_RMS_TILE(f16, 2);
+      else if (H <= 2048) MLORA_RMS_TILE(f16, 4);
+      else MLORA_RMS_TILE(f16, 8);
+    } else {
+      if (H <= 1024) MLORA_RMS_TILE(float, 2);
+      else if (H <= 2048) MLORA_RMS_TILE(float, 4);
+      else MLORA_RMS_TILE(float, 8);
+    }
+#undef MLORA_RMS_TILE
+    return mlora_launch_status(who);
+  }
   const int vpt = ceil_div(H, NORM_THREADS * 8);
   const size_t dyn = lx.src.v ? (size_t)H * sizeof(float) : 0;   // LDS staging of the expand deltas
 #define MLORA_RMS(XT, VPT) \
@@ -372,13 +475,18 @@ extern "C" int mlora_rmsnorm_ksplit(void* y, int y_layout, float* resid, const f
 
 extern "C" int mlora_silu_mul(void* out, int out_layout, const void* gate, const void* up, int ld, int T, int I,
                               void* stream) {
-  MLORA_CHECK(out_layout == MLORA_ROWMAJOR || (out_layout == MLORA_FRAG && T <= 64 && I % 32 == 0), MLORA_ERR_UNSUPPORTED,
-              "silu_mul: fragment-ordered output needs T <= 64 and I %% 32 == 0 (layout=%d T=%d I=%d)", out_layout, T, I);
+  MLORA_CHECK(out_layout == MLORA_ROWMAJOR || (out_layout == MLORA_FRAG && I % 32 == 0), MLORA_ERR_UNSUPPORTED,
+              "silu_mul: fragment-ordered output needs I %% 32 == 0 (layout=%d I=%d)", out_layout, I);
   const int frag_tt = out_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   MLORA_CHECK(out && gate && up, MLORA_ERR_INVALID, "silu_mul: null pointer");
   MLORA_CHECK(T >= 0 && I > 0 && I % 8 == 0 && ld >= I && ld % 8 == 0, MLORA_ERR_UNSUPPORTED, "silu_mul: need I %% 8 == 0, ld >= I, ld %% 8 == 0 (T=%d I=%d ld=%d)", T, I, ld);
   MLORA_CHECK(T <= 65535, MLORA_ERR_UNSUPPORTED, "silu_mul: T=%d exceeds 65535", T);
   if (T == 0) return MLORA_OK;
+  if (frag_tt && T > 64) {
+    hipLaunchKernelGGL(silu_mul_tile_kernel, dim3(ceil_div(I, 32 * (ROW_THREADS / WAVE)), frag_tt), dim3(ROW_THREADS), 0,
+                       (hipStream_t)stream, (f16*)out, (const f16*)gate, (const f16*)up, ld, T, I, frag_tt);
+    return mlora_launch_status("silu_mul");
+  }
   hipLaunchKernelGGL(silu_mul_kernel, dim3(ceil_div(I, ROW_THREADS * 8), T), dim3(ROW_THREADS), 0, (hipStream_t)stream,
                      (f16*)out, (const f16*)gate, (const f16*)up, ld, I, frag_tt);
   return mlora_launch_status("silu_mul");

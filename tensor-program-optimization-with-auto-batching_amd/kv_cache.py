@@ -110,7 +110,7 @@ class PagedKVCache:
     def attention_with_fused_qkv(self, layer, qkv, n_q_heads, out=None, frag=False):
         """qkv [T, Hq + 2 Hkv, D] (or [T, (Hq + 2 Hkv) * D]) fp16, token-major in begin_forward order.
         Rotates q in place, appends rotated k and v, attends causally; returns [T, Hq * D] fp16
-        (frag=True, decode only: as a FragActivation ready for the o_proj GEMV)."""
+        (frag=True: as a FragActivation ready for the o_proj product)."""
         if self._cur is None:
             raise RuntimeError("attention_with_fused_qkv outside begin_forward/end_forward")
         _, append_lens, decode, tok_seq, tok_pos, ctx = self._cur
@@ -122,7 +122,7 @@ class PagedKVCache:
             return ops.paged_attn_decode(qkv, self.k[layer], self.v[layer], self.block_table, tok_seq, ctx,
                                          n_q_heads, self.Hkv, self.D, out=out, frag=frag)
         return ops.paged_attn_prefill(qkv, self.k[layer], self.v[layer], self.block_table, tok_seq, tok_pos,
-                                      n_q_heads, self.Hkv, self.D, out=out)
+                                      n_q_heads, self.Hkv, self.D, out=out, frag=frag)
 
     def end_forward(self):
         seq_ids, append_lens = self._cur[0], self._cur[1]

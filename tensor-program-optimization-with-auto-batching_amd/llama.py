@@ -311,10 +311,14 @@ class LlamaForCausalLM:
         q_sz, kv_sz = s.q_size, s.kv_size
         resid = hidden
         # a decode step (one token per sequence, T <= 64) keeps its activations in fragment order
-        frag = T <= 64 and kv._cur is not None and kv._cur[2]
+        dec_frag = T <= 64 and kv._cur is not None and kv._cur[2]
+        # so does a pass large enough for the persistent GEMM on every linear of a layer, whose operand loads are then
+        # plain copies (norm, attention and SiLU write the order the matrix cores read)
+        frag = dec_frag or all(ops.gemm_frag_preferred(T, K, N) for K, N in
+                               ((H, q_sz + 2 * kv_sz), (q_sz, H), (H, 2 * I), (I, H)))
         # a decode step splits K of the two narrow accumulating GEMVs; the RMSNorm that reads the residual next adds
         # the partial results (the same kernels and slice counts as the native decode step)
-        ks_ws = self._ksplit_ws(T) if frag else None
+        ks_ws = self._ksplit_ws(T) if dec_frag else None
         parts = None
         for l, L in enumerate(self.layers):
             xn = ops.rmsnorm(resid, L["ln1"], s.rms_norm_eps, frag=frag, parts=parts)
@@ -327,7 +331,7 @@ class LlamaForCausalLM:
             if tok_adapter:
                 self._lora(resid, attn, l, "o_proj", tok_adapter)
             xn = ops.rmsnorm(resid, L["ln2"], s.rms_norm_eps, frag=frag, parts=parts)
-            if frag and I % 32 == 0 and not (tok_adapter and self._targets(l, "gate_proj", "up_proj")):
+            if dec_frag and I % 32 == 0 and not (tok_adapter and self._targets(l, "gate_proj", "up_proj")):
                 # decode step without an adapter on gate / up: the SiLU product is the epilogue of the GEMV (same bits)
                 act = ops.gate_up_silu(xn, self.interleaved_gate_up()[l])
             else:
@@ -354,7 +358,7 @@ class LlamaForCausalLM:
 
     @staticmethod
     def _linear_acc(x, W, resid, ks_ws):
-        if isinstance(x, ops.FragActivation) and isinstance(W, ops.PackedWeight):
+        if isinstance(x, ops.FragActivation) and isinstance(W, ops.PackedWeight) and x.T <= 64:
             return ops.linear_acc_ksplit(x, W, resid, ks_ws)
         ops.linear(x, W, out=resid, accumulate=True)
         return None

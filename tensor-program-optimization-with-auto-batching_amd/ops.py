@@ -33,7 +33,7 @@ def _dt(t: torch.Tensor) -> int:
 
 
 class FragActivation:
-    """A [T, K] fp16 activation block (T <= 64) stored in matrix-core fragment order (MLORA_FRAG)."""
+    """A [T, K] fp16 activation block stored in matrix-core fragment order (MLORA_FRAG)."""
 
     def __init__(self, T: int, K: int, device, data: torch.Tensor = None):
         self.T, self.K = T, K
@@ -61,7 +61,7 @@ class FragActivation:
 
     def unpack(self) -> torch.Tensor:
         """Back to row-major [T, K] (host-side index arithmetic on the device tensor; for tests)."""
-        TT = 1 if self.T <= 16 else (2 if self.T <= 32 else 4)
+        TT = 1 if self.T <= 16 else (2 if self.T <= 32 else (4 if self.T <= 64 else -(-self.T // 16)))
         v = self.data[: TT * 16 * self.K].view(self.K // 32, TT, 4, 16, 8)
         return v.permute(1, 3, 0, 2, 4).reshape(TT * 16, self.K)[: self.T].contiguous()
 
@@ -329,9 +329,14 @@ def _linear_frag(x, W, out, out_dtype, accumulate):
         out = torch.empty((T, N), dtype=out_dtype, device=x.device)
     if out.shape != (T, N):
         raise ValueError(f"linear: out{tuple(out.shape)} expected {(T, N)}")
-    check(lib().mlora_gemv_frag(_dev(out), _dt(out), ACCUMULATE if accumulate else STORE, x.data.data_ptr(),
-                                W.data.data_ptr(), T, K, N, _stream()))
+    check(lib().mlora_linear_frag(_dev(out), _dt(out), ACCUMULATE if accumulate else STORE, x.data.data_ptr(),
+                                  W.data.data_ptr(), T, K, N, _stream()))
     return out
+
+
+def gemm_frag_preferred(T: int, K: int, N: int) -> bool:
+    """Whether a [T, K] x [N, K]^T product of this size runs best with its activations in fragment order."""
+    return bool(lib().mlora_gemm_frag_preferred(T, K, N))
 
 
 def interleave_gate_up(gate_up: torch.Tensor) -> PackedWeight:
@@ -482,12 +487,11 @@ def rope_attn_decode(qkv, k_cache, v_cache, block_table, seq_ids, tok_pos, ctx_l
     return out
 
 
-def paged_attn_prefill(qkv, k_cache, v_cache, block_table, tok_seq, tok_pos, Hq, Hkv, D, out=None):
+def paged_attn_prefill(qkv, k_cache, v_cache, block_table, tok_seq, tok_pos, Hq, Hkv, D, out=None, frag=False):
     T = qkv.shape[0]
     n_seq, max_blocks = block_table.shape
-    if out is None:
-        out = torch.empty((T, Hq * D), dtype=torch.float16, device=qkv.device)
-    check(lib().mlora_paged_attn_prefill(_dev(out, torch.float16), _dev(qkv, torch.float16), _dev(k_cache, torch.float16),
+    out, optr, lay = _out_arg(out, T, Hq * D, frag, qkv.device)
+    check(lib().mlora_paged_attn_prefill(optr, lay, _dev(qkv, torch.float16), _dev(k_cache, torch.float16),
                                          _dev(v_cache, torch.float16), _dev(block_table, torch.int32), max_blocks,
                                          _dev(tok_seq, torch.int32), _dev(tok_pos, torch.int32), T, Hq, Hkv, D,
                                          k_cache.shape[0], n_seq, _stream()))

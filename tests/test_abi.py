@@ -39,8 +39,14 @@ def test_argument_validation_without_gpu():
     assert lib.mlora_gemv(1, 0, 1, 1, 64, 1, 4, 64, 64, None) == -2          # accumulate into fp16
     assert lib.mlora_gemv(1, 1, 0, 1, 60, 1, 4, 64, 64, None) == -1          # ldx < K
     assert lib.mlora_rmsnorm(1, 0, 1, 0, 1, 1e-5, 4, 12, None) == -2
-    assert lib.mlora_rmsnorm(1, 1, 1, 0, 1, 1e-5, 65, 64, None) == -2        # fragment order needs T <= 64
+    assert lib.mlora_rmsnorm(1, 1, 1, 0, 1, 1e-5, 65, 72, None) == -2        # fragment order needs H % 32 == 0
     assert lib.mlora_frag_activation_elems(17, 64) == 32 * 64 and lib.mlora_frag_activation_elems(33, 64) == 64 * 64
+    assert lib.mlora_frag_activation_elems(65, 64) == 80 * 64 and lib.mlora_frag_activation_elems(4096, 64) == 4096 * 64
+    assert lib.mlora_linear_frag(1, 0, 0, 16, 16, 100, 96, 64, None) == -2   # more than 64 fragment-ordered tokens: K % 64
+    assert b"K % 64" in lib.mlora_last_error()
+    assert lib.mlora_gemm_frag_preferred(4096, 4096, 4096) == 1 and lib.mlora_gemm_frag_preferred(4096, 4096, 4095 - 255) == 0
+    assert lib.mlora_gemm_frag_preferred(64, 4096, 1 << 20) == 0 and lib.mlora_gemm_frag_preferred(4096, 4128, 4096) == 0
+    assert lib.mlora_paged_attn_prefill(1, 7, 1, 1, 1, 1, 4, 1, 1, 5, 8, 8, 128, 4, 2, None) == -1    # unknown output layout
     assert lib.mlora_paged_attn_decode(1, 0, 1, 1, 1, 1, 4, 1, 1, 2, 8, 8, 96, 4, 2, None) == -2   # head_dim 96
     assert lib.mlora_paged_attn_decode(1, 0, 1, 1, 1, 1, 4, 1, 1, 2, 8, 3, 128, 4, 2, None) == -1  # Hq % Hkv
 

@@ -269,6 +269,69 @@ def test_gemm_lds_staged_block_kernel(ops, synth, T, K, N):
     assert torch.equal(ops.linear(wide[:, 32:32 + K], Wp, out_dtype=torch.float32), y32)
 
 
+@pytest.mark.parametrize("T,K,N", [(4096, 320, 4096), (4100, 128, 4104), (4000, 1024, 4200), (300, 512, 264), (65, 64, 16),
+                                   (4096, 4096, 4096)])
+def test_persistent_gemm_rowmajor_and_fragment_ordered_activations(ops, synth, T, K, N):
+    """The persistent 256 x 256 matrix-core GEMM (operands copied from global memory straight into LDS): row-major x
+    once there are 256 blocks and K % 64 == 0, fragment-ordered x of any T > 64.  Ragged token and column edges, all
+    three epilogues; rows past T of the last fragment hold NaN and must not reach a stored result; the same bits
+    whichever layout x comes in."""
+    print(f"case persistent gemm T={T} K={K} N={N}", flush=True)
+    x = synth.normal(13, f"pg.x.{T}.{K}", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(13, f"pg.W.{N}.{K}", (N, K), 0.02, torch.float16, DEV)
+    ref = _np(x).astype(np.float64) @ _np(W).astype(np.float64).T
+    Wp = ops.PackedWeight(W)
+    Tp = -(-T // 16) * 16
+    xpad = torch.full((Tp, K), float("nan"), dtype=torch.float16, device=DEV)
+    xpad[:T] = x
+    xf = ops.FragActivation(T, K, DEV, data=ops.FragActivation.pack(xpad).data)
+    assert torch.equal(xf.unpack(), x) and torch.equal(ops.FragActivation.pack(x).unpack(), x)
+    y16 = ops.linear(xf, Wp)
+    y32 = ops.linear(xf, Wp, out_dtype=torch.float32)
+    r0 = synth.normal(13, f"pg.r.{T}.{N}", (T, N), 1.0, torch.float32, DEV)
+    racc = r0.clone()
+    ops.linear(xf, Wp, out=racc, accumulate=True)
+    torch.cuda.synchronize()
+    assert max_rel_err(_np(y16), ref) <= TOL
+    assert max_rel_err(_np(y32), ref, floor=1e-2) <= 5e-4
+    assert max_rel_err(_np(racc), _np(r0) + ref, floor=1e-2) <= 5e-4
+    assert torch.equal(y16, ops.linear(x, Wp)) and torch.equal(y32, ops.linear(x, Wp, out_dtype=torch.float32))
+    racc2 = r0.clone()
+    ops.linear(x, Wp, out=racc2, accumulate=True)
+    assert torch.equal(racc, racc2)
+    assert ops.gemm_frag_preferred(T, K, N) == (T > 64 and K % 64 == 0 and -(-T // 256) * -(-N // 256) >= 256)
+
+
+def test_fragment_ordered_activations_need_whole_pairs_of_k_steps_beyond_64_tokens(ops, synth):
+    x = synth.normal(13, "pg.bad.x", (100, 96), 1.0, torch.float16, DEV)
+    Wp = ops.PackedWeight(synth.normal(13, "pg.bad.W", (64, 96), 0.02, torch.float16, DEV))
+    with pytest.raises(Exception, match="K % 64"):
+        ops.linear(ops.FragActivation.pack(x), Wp)
+    assert not ops.gemm_frag_preferred(100, 96, 64)
+
+
+def test_producers_write_fragment_order_for_prefill_sized_blocks(ops, synth):
+    """RMSNorm, SiLU*mul and the prefill attention writing fragment order for T > 64 == their row-major output; the
+    matrix-core LoRA kernels read it with the same bits."""
+    for T, H, dt in ((200, 1024, torch.float32), (4096, 4096, torch.float32), (130, 2048, torch.float16), (65, 4096, torch.float16),
+                     (1000, 1056, torch.float32), (77, 32, torch.float16), (300, 5120, torch.float32)):
+        x = synth.normal(14, f"fragp.x{T}.{H}", (T, H), 1.5, dt, DEV)
+        w = synth.normal(14, f"fragp.w{H}", (H,), 1.0, torch.float16, DEV)
+        assert torch.equal(ops.rmsnorm(x, w, 1e-5, frag=True).unpack(), ops.rmsnorm(x, w, 1e-5)), (T, H, dt)
+    for T, I in ((200, 1408), (4096, 11008), (65, 32), (333, 352)):
+        gu = synth.normal(14, f"fragp.gu{T}.{I}", (T, 2 * I), 2.0, torch.float16, DEV)
+        assert torch.equal(ops.silu_mul(gu, frag=True).unpack(), ops.silu_mul(gu)), (T, I)
+    for T2, pattern in ((300, "segments"), (1100, "segments"), (130, "random")):
+        c = synth.gather_mm_case(seed=5, T=T2, K=1024, N=512, r=16, n_ad=6, device=DEV, tag=f"fragp{T2}")
+        if pattern == "segments":
+            c["ids"] = torch.sort(c["ids"])[0].contiguous()
+        y1, y2 = c["y"].clone(), c["y"].clone()
+        ops.gather_mm(y1, c["x"], c["A"], c["B"], c["ids"], 0.5)
+        ops.gather_mm(y2, ops.FragActivation.pack(c["x"]), c["A"], c["B"], c["ids"], 0.5)
+        torch.cuda.synchronize()
+        assert torch.equal(y1, y2) and not torch.equal(y1, c["y"])
+
+
 def test_pack_weight_is_a_permutation(ops, synth):
     """Bit-exact: every element of W appears at its fragment-order position, padding rows are zero."""
     N, K = 40, 64
@@ -372,11 +435,17 @@ def test_paged_attention_prefill_then_decode(ops, synth, Hq, Hkv, D, n_seq):
         ref.end_forward()
         cache.begin_forward(sids, lens)
         frag = it == 1                      # one of the decode steps writes fragment order
-        got = cache.attention_with_fused_qkv(0, qkv.clone(), Hq, frag=frag)
+        qkv_rot = qkv.clone()               # rotated in place by the call
+        got = cache.attention_with_fused_qkv(0, qkv_rot, Hq, frag=frag)
+        cache_meta = (cache._cur[3], cache._cur[4])
         cache.end_forward()
         torch.cuda.synchronize()
         got = got.unpack() if frag else got
         assert max_rel_err(_np(got), exp) <= TOL, f"step {it}"
+        if it == 0:                         # the prefill attention writing fragment order: the same values
+            tok_seq, tok_pos = cache_meta
+            again = ops.paged_attn_prefill(qkv_rot, cache.k[0], cache.v[0], cache.block_table, tok_seq, tok_pos, Hq, Hkv, D, frag=True)
+            assert torch.equal(again.unpack(), got)
     # cache contents: rotated K and V, page by page, against the oracle's pages
     k_ref = oracle.f16(ref.k[0])                       # [n_pages, Hkv, 16, D]
     v_ref = oracle.f16(ref.v[0]).transpose(0, 1, 3, 2)  # -> [n_pages, Hkv, D, 16]
