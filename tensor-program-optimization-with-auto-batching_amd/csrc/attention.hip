@@ -854,8 +854,7 @@ extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qk
   if (int e = check_attn("paged_attn_decode", Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
   MLORA_CHECK(out && qkv && k_cache && v_cache && block_table && seq_ids && ctx_len, MLORA_ERR_INVALID, "paged_attn_decode: null pointer");
   MLORA_CHECK(B >= 0 && B <= 65535, MLORA_ERR_INVALID, "paged_attn_decode: bad B=%d (0..65535)", B);
-  MLORA_CHECK(out_layout == MLORA_ROWMAJOR || (out_layout == MLORA_FRAG && B <= 64), MLORA_ERR_UNSUPPORTED,
-              "paged_attn_decode: fragment-ordered output needs B <= 64 (layout=%d B=%d)", out_layout, B);
+  MLORA_CHECK(out_layout == MLORA_ROWMAJOR || out_layout == MLORA_FRAG, MLORA_ERR_INVALID, "paged_attn_decode: bad out_layout %d", out_layout);
   const int frag_tt = out_layout == MLORA_FRAG ? mlora_frag_tiles(B) : 0;
   if (B == 0) return MLORA_OK;
   const float scale = 1.f / sqrtf((float)D);
@@ -891,8 +890,7 @@ extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv
   MLORA_CHECK(out && qkv && k_cache && v_cache && block_table && seq_ids && tok_pos && ctx_len && rope_cos && rope_sin,
               MLORA_ERR_INVALID, "rope_attn_decode: null pointer");
   MLORA_CHECK(B >= 0 && B <= 65535 && max_pos > 0, MLORA_ERR_INVALID, "rope_attn_decode: bad B=%d (0..65535) max_pos=%d", B, max_pos);
-  MLORA_CHECK(out_layout == MLORA_ROWMAJOR || (out_layout == MLORA_FRAG && B <= 64), MLORA_ERR_UNSUPPORTED,
-              "rope_attn_decode: fragment-ordered output needs B <= 64 (layout=%d B=%d)", out_layout, B);
+  MLORA_CHECK(out_layout == MLORA_ROWMAJOR || out_layout == MLORA_FRAG, MLORA_ERR_INVALID, "rope_attn_decode: bad out_layout %d", out_layout);
   const int G = Hq / Hkv;
   MLORA_CHECK(G <= 16, MLORA_ERR_UNSUPPORTED, "rope_attn_decode: more than 16 query heads per kv head (%d)", G);
   LoraExpandQKV lx = {};

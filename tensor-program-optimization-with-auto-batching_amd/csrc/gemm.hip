@@ -478,6 +478,232 @@ int launch_gemm_pp(void* y, const f16* x, int ldx, int x_tt, const f16* Wp, int 
   return MLORA_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Token blocks between the decode GEMV and the persistent kernel above (65 to a few hundred tokens: a decode step of
+// many sequences, a short prefill).  The weights are read once and the matrix cores and the operand loads weigh about
+// the same, so the block is as tall as the token block allows and narrow enough to give every compute unit a
+// workgroup: FT x 8 fragments (128 or 256 tokens x 128 weight rows), eight waves, both operands in fragment order and
+// copied from global memory straight into a six-stage LDS ring of 32-k steps (the weight stream comes from HBM: five
+// stages, 40 KiB of it, are in flight per compute unit).  grid = (weight-row blocks, K slices, token blocks).
+// With K slices, slice 0 produces the result proper (store or accumulate) and slice s > 0 stores its fp32 partial
+// sums to part[s - 1][T][ld_part] - for the two narrow accumulating linears of a layer, whose partials the next
+// RMSNorm of the row adds in slice order.
+// ---------------------------------------------------------------------------------------------
+constexpr int MID_STAGES = 6;
+constexpr int MID_FN = 8;
+
+template <int OUT, int FT>
+__global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __restrict__ yv, float* __restrict__ part, int ld_part,
+                                                                    const f16* __restrict__ xf, int x_tt, const f16* __restrict__ Wp,
+                                                                    int T, int K, int N) {
+  constexpr int LF = MID_FN + FT;              // fragments per stage: weights, then tokens
+  constexpr int LQ = LF / PP_WAVES;            // ... of which a wave fetches LQ (fragment f = wave + 8 q)
+  constexpr int STAGE_ELEMS = LF * 512;
+  constexpr int WTF = FT / 4;                  // token fragments of a wave's tile
+  static_assert(LF % PP_WAVES == 0 && FT % 4 == 0, "fragments divide over the waves");
+  extern __shared__ __align__(16) f16 smem[];  // [MID_STAGES][STAGE_ELEMS]; the output staging reuses it after the K loop
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int KB = K / 32;
+  const int tiles = (N + 15) / 16;
+  const int n0 = blockIdx.x * MID_FN * 16, t0 = blockIdx.z * FT * 16;
+  const int per = (KB + gridDim.y - 1) / gridDim.y;
+  const int kb0 = blockIdx.y * per;
+  const int kb1 = kb0 + per < KB ? kb0 + per : KB;
+  const int nst = kb1 - kb0;                   // stages of this slice (>= 1: checked by the launcher)
+
+  const f16* src[LQ];
+  int step[LQ];
+#pragma unroll
+  for (int q = 0; q < LQ; ++q) {
+    const int f = wave + PP_WAVES * q;         // uniform
+    if (f < MID_FN) {
+      int nt = n0 / 16 + f;
+      nt = nt < tiles ? nt : tiles - 1;        // rows past N: a valid fragment, results dropped
+      src[q] = Wp + (size_t)nt * KB * 512 + lane * 8;
+      step[q] = 512;
+    } else {
+      int tt = t0 / 16 + f - MID_FN;
+      tt = tt < x_tt ? tt : x_tt - 1;          // tiles past T: a valid fragment, results dropped
+      src[q] = xf + (size_t)tt * 512 + lane * 8;
+      step[q] = x_tt * 512;
+    }
+  }
+  int ring = 0, load_kb = kb0;
+  auto issue = [&]() {
+    const int kb = load_kb < kb1 ? load_kb : kb1 - 1;   // past the slice: a valid address, into a slot nobody reads any more
+    f16* dst = smem + ring * STAGE_ELEMS + wave * 512;
+#pragma unroll
+    for (int q = 0; q < LQ; ++q)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + (size_t)kb * step[q]),
+                                       (__attribute__((address_space(3))) void*)(dst + q * PP_WAVES * 512), 16, 0, 0);
+    ring = ring + 1 == MID_STAGES ? 0 : ring + 1;
+    ++load_kb;
+  };
+
+  const int wn = wave & 1, wt = wave >> 1;     // weight rows wn * 64 .., tokens wt * WTF * 16 ..
+  f32x4 acc[4][WTF];
+  f16x8 a[2][4], b[2][WTF];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < WTF; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  int rd = 0;
+  auto read_frags = [&](auto U) {
+    constexpr int u = decltype(U)::value;
+    const f16* st = smem + rd * STAGE_ELEMS + lane * 8;
+#pragma unroll
+    for (int j = 0; j < WTF; ++j) b[u][j] = ld8(st + (MID_FN + wt * WTF + j) * 512);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a[u][i] = ld8(st + (wn * 4 + i) * 512);
+    rd = rd + 1 == MID_STAGES ? 0 : rd + 1;
+  };
+  auto multiply = [&](auto U) {
+    constexpr int u = decltype(U)::value;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < WTF; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][i], b[u][j], acc[i][j], 0, 0, 0);
+  };
+  // the wait: of this wave's loads at most those of the MID_STAGES - 2 youngest stages are still in flight, so the
+  // stage multiplied next has landed; with everybody's wait and fragment reads behind the barrier, the slot of the
+  // stage just read is refilled
+  auto wait_next = [&]() {
+    if constexpr (LQ == 2) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
+    static_assert(MID_STAGES == 6 && (LQ == 2 || LQ == 3), "the immediate above is (MID_STAGES - 2) * LQ");
+  };
+  auto stage = [&](auto U) {
+    constexpr int u = decltype(U)::value;
+    wait_next();
+    __syncthreads();
+    issue();
+    read_frags(std::integral_constant<int, 1 - u>());
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(U);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+#pragma unroll
+  for (int i = 0; i < MID_STAGES - 1; ++i) issue();
+  wait_next();
+  __syncthreads();
+  issue();
+  read_frags(std::integral_constant<int, 0>());
+  int g = 0;
+  for (; g + 1 < nst; g += 2) {
+    stage(std::integral_constant<int, 0>());
+    stage(std::integral_constant<int, 1>());
+  }
+  if (g < nst) stage(std::integral_constant<int, 0>());
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // nothing is in flight into the LDS that the epilogue reuses
+  __syncthreads();
+
+  const int r16 = lane & 15, gq = lane >> 4;
+  if (blockIdx.y > 0) {                        // a later K slice: fp32 partial sums
+    float* pp = part + (size_t)(blockIdx.y - 1) * T * ld_part;
+#pragma unroll
+    for (int j = 0; j < WTF; ++j) {
+      const int t = t0 + (wt * WTF + j) * 16 + r16;
+      if (t >= T) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + (wn * 4 + i) * 16 + gq * 4;
+        if (n < N) *reinterpret_cast<f32x4*>(pp + (size_t)t * ld_part + n) = acc[i][j];
+      }
+    }
+    return;
+  }
+  if constexpr (OUT == OUT_F16) {
+    // 16 tokens x 64 columns at a time through the wave's staging buffer: D[n][t] fragments in, token rows out
+    f16* ostage = smem + wave * PP_OUT_ELEMS;
+#pragma unroll
+    for (int j = 0; j < WTF; ++j) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const f32x4 sacc = acc[i][j];
+        *reinterpret_cast<f16x4*>(ostage + r16 * PP_OUT_LD + i * 16 + gq * 4) = f16x4{(f16)sacc[0], (f16)sacc[1], (f16)sacc[2], (f16)sacc[3]};
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const int c = q * 64 + lane;             // 16-byte chunk: token row c / 8, columns (c % 8) * 8 ..
+        const int tr = c >> 3, cc = (c & 7) * 8;
+        const int t = t0 + (wt * WTF + j) * 16 + tr;
+        const int n = n0 + wn * 64 + cc;
+        const f16x4 lo = *reinterpret_cast<const f16x4*>(ostage + tr * PP_OUT_LD + cc);
+        const f16x4 hi = *reinterpret_cast<const f16x4*>(ostage + tr * PP_OUT_LD + cc + 4);
+        if (t < T && n + 8 <= N) {
+          st8((f16*)yv + (size_t)t * N + n, f16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
+        } else if (t < T) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (n + e < N) ((f16*)yv)[(size_t)t * N + n + e] = lo[e];
+            if (n + 4 + e < N) ((f16*)yv)[(size_t)t * N + n + 4 + e] = hi[e];
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < WTF; ++j) {
+      const int t = t0 + (wt * WTF + j) * 16 + r16;
+      if (t >= T) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + (wn * 4 + i) * 16 + gq * 4;
+        if (n >= N) continue;
+        const size_t o = (size_t)t * N + n;
+        if constexpr (OUT == OUT_F32) {
+          *reinterpret_cast<f32x4*>((float*)yv + o) = acc[i][j];
+        } else {
+          f32x4* p = reinterpret_cast<f32x4*>((float*)yv + o);
+          *p = *p + acc[i][j];
+        }
+      }
+    }
+  }
+}
+
+// Block height and K slices of the mid-size kernel for a shape: 128-token blocks when 256-token ones would leave most
+// compute units without a workgroup.
+struct MidShape {
+  int ft, ksplit;
+};
+MidShape gemm_mid_shape(int T, int K, int N, int ksplit_max) {
+  const int cols = ceil_div(N, MID_FN * 16);
+  MidShape m;
+  m.ft = (T <= 128 || (long)cols * ceil_div(T, 256) * ksplit_max <= 128) ? 8 : 16;
+  int ks = 256 / (cols * ceil_div(T, m.ft * 16));
+  const int by_k = (K / 32) / 16;              // at least 16 k-steps per slice
+  if (ks > by_k) ks = by_k;
+  if (ks > ksplit_max) ks = ksplit_max;
+  m.ksplit = ks < 1 ? 1 : ks;
+  return m;
+}
+
+template <int OUT, int FT>
+int launch_gemm_mid_ft(void* y, float* part, int ld_part, int ksplit, const f16* xf, int x_tt, const f16* Wp, int T, int K, int N,
+                       hipStream_t s) {
+  constexpr size_t lds = (size_t)MID_STAGES * (MID_FN + FT) * 512 * sizeof(f16);
+  static_assert(lds >= (size_t)PP_WAVES * PP_OUT_ELEMS * sizeof(f16), "the output staging fits the ring");
+  static bool configured = false;                    // the attribute is per kernel, set once per process
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mid_kernel<OUT, FT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return mlora_set_error(MLORA_ERR_LAUNCH, "linear_frag: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    configured = true;
+  }
+  const dim3 grid(ceil_div(N, MID_FN * 16), ksplit, ceil_div(T, FT * 16));
+  hipLaunchKernelGGL((gemm_mid_kernel<OUT, FT>), grid, dim3(PP_WAVES * WAVE), lds, s, y, part, ld_part, xf, x_tt, Wp, T, K, N);
+  return MLORA_OK;
+}
+
+template <int OUT>
+int launch_gemm_mid(void* y, float* part, int ld_part, int ksplit, int ft, const f16* xf, int x_tt, const f16* Wp, int T, int K, int N,
+                    hipStream_t s) {
+  if (ft == 8) return launch_gemm_mid_ft<OUT, 8>(y, part, ld_part, ksplit, xf, x_tt, Wp, T, K, N, s);
+  return launch_gemm_mid_ft<OUT, 16>(y, part, ld_part, ksplit, xf, x_tt, Wp, T, K, N, s);
+}
+
 template <int OUT, int FT, int FN, int WT_, int WN_>
 int launch_gemm_lds(void* y, const f16* x, int ldx, const f16* Wp, int T, int K, int N, hipStream_t s) {
   constexpr size_t lds = 2 * (LBK / 32) * (FT + FN) * 512 * sizeof(f16);
@@ -565,13 +791,36 @@ extern "C" int mlora_linear_frag(void* y, int y_dtype, int mode, const void* xf,
                                  void* stream) {
   if (T <= 64) return mlora_gemv_frag(y, y_dtype, mode, xf, Wp, T, K, N, stream);
   if (int e = mlora_check_linear("linear_frag", y, y_dtype, mode, xf, K, Wp, T, K, N)) return e;
-  MLORA_CHECK(K % 64 == 0, MLORA_ERR_UNSUPPORTED, "linear_frag: more than 64 fragment-ordered tokens need K %% 64 == 0 (K=%d)", K);
+  MLORA_CHECK(K % 32 == 0, MLORA_ERR_UNSUPPORTED, "linear_frag: K %% 32 != 0 (K=%d)", K);
   MLORA_CHECK(((uintptr_t)xf & 15) == 0, MLORA_ERR_INVALID, "linear_frag: xf must be 16-byte aligned");
   hipStream_t s = (hipStream_t)stream;
+  const f16* x = (const f16*)xf;
+  const f16* W = (const f16*)Wp;
   const int tt = mlora_frag_tiles(T);
   int e;
-  if (mode == MLORA_ACCUMULATE) e = launch_gemm_pp<OUT_ACC_F32>(y, (const f16*)xf, 0, tt, (const f16*)Wp, T, K, N, s);
-  else if (y_dtype == MLORA_F32) e = launch_gemm_pp<OUT_F32>(y, (const f16*)xf, 0, tt, (const f16*)Wp, T, K, N, s);
-  else e = launch_gemm_pp<OUT_F16>(y, (const f16*)xf, 0, tt, (const f16*)Wp, T, K, N, s);
+  if (mlora_gemm_frag_preferred(T, K, N)) {
+    if (mode == MLORA_ACCUMULATE) e = launch_gemm_pp<OUT_ACC_F32>(y, x, 0, tt, W, T, K, N, s);
+    else if (y_dtype == MLORA_F32) e = launch_gemm_pp<OUT_F32>(y, x, 0, tt, W, T, K, N, s);
+    else e = launch_gemm_pp<OUT_F16>(y, x, 0, tt, W, T, K, N, s);
+  } else {
+    const int ft = gemm_mid_shape(T, K, N, 1).ft;
+    if (mode == MLORA_ACCUMULATE) e = launch_gemm_mid<OUT_ACC_F32>(y, nullptr, 0, 1, ft, x, tt, W, T, K, N, s);
+    else if (y_dtype == MLORA_F32) e = launch_gemm_mid<OUT_F32>(y, nullptr, 0, 1, ft, x, tt, W, T, K, N, s);
+    else e = launch_gemm_mid<OUT_F16>(y, nullptr, 0, 1, ft, x, tt, W, T, K, N, s);
+  }
   return e ? e : mlora_launch_status("linear_frag");
+}
+
+// K slices the mid-size kernel would use for resid [T, N] += xf . Wp^T with at most ks_max slices (T > 64)
+int mlora_gemm_mid_ksplit(int T, int K, int N, int ks_max) { return gemm_mid_shape(T, K, N, ks_max).ksplit; }
+
+// resid [T, N] fp32 += xf . Wp^T over ks K slices: slice 0 into resid, slices 1.. into part[ks - 1][T][ld_part] (T > 64)
+int mlora_gemm_mid_acc(float* resid, float* part, int ld_part, int ks, const void* xf, const void* Wp, int T, int K, int N,
+                       void* stream) {
+  MLORA_CHECK(K % 32 == 0 && ks >= 1 && (K / 32) / ks >= 1 && ((uintptr_t)xf & 15) == 0, MLORA_ERR_UNSUPPORTED,
+              "linear_frag (K slices): need K %% 32 == 0 and at least one 32-k step per slice (K=%d ks=%d)", K, ks);
+  const int ft = gemm_mid_shape(T, K, N, ks).ft;
+  const int e = launch_gemm_mid<OUT_ACC_F32>(resid, part, ld_part, ks, ft, (const f16*)xf, mlora_frag_tiles(T), (const f16*)Wp, T, K, N,
+                                             (hipStream_t)stream);
+  return e ? e : mlora_launch_status("linear_frag (K slices)");
 }

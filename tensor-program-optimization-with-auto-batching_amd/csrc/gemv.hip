@@ -538,8 +538,12 @@ extern "C" int mlora_gemv_frag_lora(void* y, int y_dtype, int mode, const void* 
 
 // A narrow weight (fewer than 512 row tiles) gives too few workgroups for four tiles each; splitting K over up to four
 // workgroups restores one equal workgroup per compute unit.  At least 24 k-steps per slice keep every wave's pipeline full.
+int mlora_gemm_mid_ksplit(int T, int K, int N, int ks_max);
+int mlora_gemm_mid_acc(float* resid, float* part, int ld_part, int ks, const void* xf, const void* Wp, int T, int K, int N, void* stream);
+
 extern "C" int mlora_gemv_ksplit(int T, int K, int N_total) {
-  if (T <= 0 || T > 64 || K <= 0 || K % 32 || N_total <= 0) return 1;
+  if (T <= 0 || K <= 0 || K % 32 || N_total <= 0) return 1;
+  if (T > 64) return mlora_gemm_mid_ksplit(T, K, N_total, 4);      // the matrix-core kernel for mid-size token blocks
   const int tiles = ceil_div(N_total, 16);
   if (tiles >= 512) return 1;
   const int groups = ceil_div(tiles, 4);      // row tiles per workgroup of the split kernel (see gemv_dispatch)
@@ -559,7 +563,11 @@ extern "C" int mlora_gemv_frag_acc_ksplit(float* y, float* y2, float* part, int 
                                           int N_main, int N_ext, void* v_part, const void* const* A, int n_proj,
                                           const int32_t* tok_adapter, int r, int n_ad, void* stream) {
   if (int e = mlora_check_linear("gemv_frag_acc_ksplit", y, MLORA_F32, MLORA_ACCUMULATE, xf, K, Wp, T, K, N_main)) return e;
-  MLORA_CHECK(T <= 64, MLORA_ERR_UNSUPPORTED, "gemv_frag_acc_ksplit: T=%d exceeds 64", T);
+  if (T > 64) {      // the matrix-core kernel for mid-size token blocks: K slices only, nothing rides along
+    MLORA_CHECK(N_ext == 0 && A == nullptr, MLORA_ERR_UNSUPPORTED, "gemv_frag_acc_ksplit: appended rows and shrink units need T <= 64 (T=%d)", T);
+    MLORA_CHECK(ks >= 1 && ks <= 4 && (ks == 1 || part), MLORA_ERR_INVALID, "gemv_frag_acc_ksplit: ks=%d outside 1..4, or no partials buffer", ks);
+    return mlora_gemm_mid_acc(y, part, N_main, ks, xf, Wp, T, K, N_main, stream);
+  }
   MLORA_CHECK(N_ext >= 0 && N_ext % 4 == 0 && (N_ext == 0 || (y2 && N_main % 16 == 0)), MLORA_ERR_INVALID,
               "gemv_frag_acc_ksplit: appended rows need y2, N_ext %% 4 == 0 and N_main %% 16 == 0 (N_main=%d N_ext=%d)", N_main, N_ext);
   MLORA_CHECK(!(A && N_ext), MLORA_ERR_INVALID, "gemv_frag_acc_ksplit: shrink units and appended rows are exclusive");

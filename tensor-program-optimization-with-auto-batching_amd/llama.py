@@ -312,13 +312,12 @@ class LlamaForCausalLM:
         resid = hidden
         # a decode step (one token per sequence, T <= 64) keeps its activations in fragment order
         dec_frag = T <= 64 and kv._cur is not None and kv._cur[2]
-        # so does a pass large enough for the persistent GEMM on every linear of a layer, whose operand loads are then
-        # plain copies (norm, attention and SiLU write the order the matrix cores read)
-        frag = dec_frag or all(ops.gemm_frag_preferred(T, K, N) for K, N in
-                               ((H, q_sz + 2 * kv_sz), (q_sz, H), (H, 2 * I), (I, H)))
+        # so does every larger pass: the operand loads of the matrix-core linears are then plain copies (norm, attention
+        # and SiLU write the order the matrix cores read)
+        frag = dec_frag or (T > 64 and H % 32 == 0 and q_sz % 32 == 0 and I % 32 == 0)
         # a decode step splits K of the two narrow accumulating GEMVs; the RMSNorm that reads the residual next adds
         # the partial results (the same kernels and slice counts as the native decode step)
-        ks_ws = self._ksplit_ws(T) if dec_frag else None
+        ks_ws = self._ksplit_ws(T) if dec_frag or (frag and T <= 256) else None
         parts = None
         for l, L in enumerate(self.layers):
             xn = ops.rmsnorm(resid, L["ln1"], s.rms_norm_eps, frag=frag, parts=parts)
@@ -343,7 +342,12 @@ class LlamaForCausalLM:
             if tok_adapter:
                 self._lora(resid, act, l, "down_proj", tok_adapter)
         if logits_rows is not None:
-            resid = resid[logits_rows].contiguous()       # prefill: never K-split (parts is None)
+            if parts is not None:                         # pending K-slice partials of the last down_proj, in slice order
+                pv = parts.part[: (parts.ks - 1) * T * parts.ld].view(parts.ks - 1, T, parts.ld)
+                for q in range(parts.ks - 1):
+                    resid += pv[q, :, :H]
+                parts = None
+            resid = resid[logits_rows].contiguous()
         xn = ops.rmsnorm(resid, self.norm, s.rms_norm_eps, frag=resid.shape[0] <= 64, parts=parts)
         return ops.linear(xn, self.lm_head, out_dtype=torch.float32)
 
@@ -358,7 +362,7 @@ class LlamaForCausalLM:
 
     @staticmethod
     def _linear_acc(x, W, resid, ks_ws):
-        if isinstance(x, ops.FragActivation) and isinstance(W, ops.PackedWeight) and x.T <= 64:
+        if isinstance(x, ops.FragActivation) and isinstance(W, ops.PackedWeight) and ks_ws is not None:
             return ops.linear_acc_ksplit(x, W, resid, ks_ws)
         ops.linear(x, W, out=resid, accumulate=True)
         return None

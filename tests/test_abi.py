@@ -42,8 +42,10 @@ def test_argument_validation_without_gpu():
     assert lib.mlora_rmsnorm(1, 1, 1, 0, 1, 1e-5, 65, 72, None) == -2        # fragment order needs H % 32 == 0
     assert lib.mlora_frag_activation_elems(17, 64) == 32 * 64 and lib.mlora_frag_activation_elems(33, 64) == 64 * 64
     assert lib.mlora_frag_activation_elems(65, 64) == 80 * 64 and lib.mlora_frag_activation_elems(4096, 64) == 4096 * 64
-    assert lib.mlora_linear_frag(1, 0, 0, 16, 16, 100, 96, 64, None) == -2   # more than 64 fragment-ordered tokens: K % 64
-    assert b"K % 64" in lib.mlora_last_error()
+    assert lib.mlora_linear_frag(1, 0, 0, 16, 16, 100, 48, 64, None) == -2   # fragment order: K % 32
+    assert lib.mlora_linear_frag(1, 0, 0, 24, 16, 100, 64, 64, None) == -1   # xf not 16-byte aligned
+    assert lib.mlora_gemv_ksplit(256, 4096, 4096) == 4 and lib.mlora_gemv_ksplit(256, 4096, 12288) == 2 and lib.mlora_gemv_ksplit(256, 4096, 32000) == 1
+    assert lib.mlora_gemv_frag_acc_ksplit(16, None, None, 2, 16, 16, 100, 64, 64, 0, None, None, 0, None, 0, 0, None) == -1   # slices without partials
     assert lib.mlora_gemm_frag_preferred(4096, 4096, 4096) == 1 and lib.mlora_gemm_frag_preferred(4096, 4096, 4095 - 255) == 0
     assert lib.mlora_gemm_frag_preferred(64, 4096, 1 << 20) == 0 and lib.mlora_gemm_frag_preferred(4096, 4128, 4096) == 0
     assert lib.mlora_paged_attn_prefill(1, 7, 1, 1, 1, 1, 4, 1, 1, 5, 8, 8, 128, 4, 2, None) == -1    # unknown output layout
@@ -97,7 +99,7 @@ def test_argument_validation_of_fused_and_batched_entry_points():
                                                                None, 0, None, None, 0.0, 0, 0, 0, None)
     assert ra(8, 8, 96, 2, 0) == -2                    # head_dim
     assert ra(34, 2, 128, 2, 0) == -2                  # 17 query heads per kv head
-    assert ra(8, 8, 128, 65, 1) == -2                  # fragment-ordered output needs B <= 64
+    assert ra(8, 8, 128, 65, 7) == -1                  # unknown output layout
     assert ra(8, 8, 128, 0, 0) == 0
     assert lib.mlora_rope_attn_decode(1, 0, 1, 1, 1, 1, 4, 1, 1, 1, 1, 1, 64, 2, 8, 8, 128, 4, 2,
                                       1, 1, None, None, 0.5, 64, 16, 2, None) == -1     # LoRA without B / ids

@@ -302,12 +302,35 @@ def test_persistent_gemm_rowmajor_and_fragment_ordered_activations(ops, synth, T
     assert ops.gemm_frag_preferred(T, K, N) == (T > 64 and K % 64 == 0 and -(-T // 256) * -(-N // 256) >= 256)
 
 
-def test_fragment_ordered_activations_need_whole_pairs_of_k_steps_beyond_64_tokens(ops, synth):
-    x = synth.normal(13, "pg.bad.x", (100, 96), 1.0, torch.float16, DEV)
-    Wp = ops.PackedWeight(synth.normal(13, "pg.bad.W", (64, 96), 0.02, torch.float16, DEV))
-    with pytest.raises(Exception, match="K % 64"):
-        ops.linear(ops.FragActivation.pack(x), Wp)
-    assert not ops.gemm_frag_preferred(100, 96, 64)
+@pytest.mark.parametrize("T,K,N", [(100, 96, 64), (256, 4096, 4096), (256, 11008, 4096), (200, 1024, 520), (129, 352, 1000), (70, 512, 4096)])
+def test_mid_size_token_blocks_with_k_slices(ops, synth, T, K, N):
+    """65 to a few hundred fragment-ordered tokens: the accumulating linear split over K slices (slice 0 into the
+    residual, the others into partials that the next RMSNorm of the row adds) equals the unsplit product up to the
+    summation order, and the norm output follows."""
+    print(f"case mid-size k-slices T={T} K={K} N={N}", flush=True)
+    x = synth.normal(15, f"mid.x.{T}.{K}", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(15, f"mid.W.{N}.{K}", (N, K), 0.02, torch.float16, DEV)
+    w = synth.normal(15, f"mid.w.{N}", (N,), 1.0, torch.float16, DEV)
+    r0 = synth.normal(15, f"mid.r.{T}.{N}", (T, N), 1.0, torch.float32, DEV)
+    Wp = ops.PackedWeight(W)
+    xf = ops.FragActivation.pack(x)
+    ref = _np(r0).astype(np.float64) + _np(x).astype(np.float64) @ _np(W).astype(np.float64).T
+    plain = r0.clone()
+    ops.linear(xf, Wp, out=plain, accumulate=True)
+    assert max_rel_err(_np(plain), ref, floor=1e-2) <= 5e-4
+    resid = r0.clone()
+    ws = torch.full((3 * T * N,), float("nan"), dtype=torch.float32, device=DEV)
+    parts = ops.linear_acc_ksplit(xf, Wp, resid, ws)
+    ks = 1 if parts is None else parts.ks
+    print(f"   K slices: {ks}", flush=True)
+    if N <= 4096 and K >= 2048:
+        assert ks == 4
+    xn = ops.rmsnorm(resid, w, 1e-5, frag=True, parts=parts) if N % 32 == 0 else ops.rmsnorm(resid, w, 1e-5, parts=parts)
+    torch.cuda.synchronize()
+    assert max_rel_err(_np(resid), ref, floor=1e-2) <= 5e-4          # the norm stored the summed row back
+    ref_n = ref / np.sqrt((ref ** 2).mean(-1, keepdims=True) + 1e-5) * _np(w).astype(np.float64)
+    got_n = xn.unpack() if isinstance(xn, ops.FragActivation) else xn
+    assert max_rel_err(_np(got_n), ref_n) <= TOL
 
 
 def test_producers_write_fragment_order_for_prefill_sized_blocks(ops, synth):
