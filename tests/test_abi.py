@@ -118,7 +118,7 @@ def test_argument_validation_of_fused_and_batched_entry_points():
     # K-split GEMV: slice counts, partials buffer, argument checks
     assert lib.mlora_gemv_ksplit(32, 11008, 4096) == 4 and lib.mlora_gemv_ksplit(32, 4096, 4352) == 3
     assert lib.mlora_gemv_ksplit(33, 11008, 4096) == 4 and lib.mlora_gemv_ksplit(32, 4096, 12288) == 1
-    assert lib.mlora_gemv_ksplit(65, 11008, 4096) == 1 and lib.mlora_gemv_ksplit(64, 4096, 4352) == 3
+    assert lib.mlora_gemv_ksplit(65, 11008, 4096) == 4 and lib.mlora_gemv_ksplit(64, 4096, 4352) == 3
     assert lib.mlora_gemv_ksplit_bytes(32, 4096, 4) == 3 * 32 * 4096 * 4 and lib.mlora_gemv_ksplit_bytes(32, 4096, 1) == 0
     # K-range blocks of the appended rows in the per-unit split GEMV: 1 where the form does not apply (and without a device)
     assert lib.mlora_gemv_split_kq(32, 4096, 12288, 768) in (1, 4)
@@ -130,7 +130,7 @@ def test_argument_validation_of_fused_and_batched_entry_points():
                                                                                          None, A, 1 if A else 0, None, 16, 4, None)
     assert ksg(2, None) == -1                        # split without a partials buffer
     assert ksg(5, 1) == -1                           # more than four slices
-    assert ksg(2, 1, T=70) == -2                     # the GEMV takes at most 64 tokens
+    assert ksg(2, 1, T=70) == -2                     # beyond 64 tokens: the matrix-core kernel, whose xf must be 16-byte aligned
     assert ksg(1, None, n_ext=64) == -1              # appended rows without y2
     assert ksg(2, 1, T=0) == 0
     nk = lambda ks, part, ld: lib.mlora_rmsnorm_ksplit(1, 0, 1, part, ks, ld, 1, 1e-5, 4, 4096, None, 0, None, None, 0.0, 0, 0, 0, None)
