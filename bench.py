@@ -375,7 +375,7 @@ def bench_c4_prefill(args, synth, llama):
 def bench_c5_decode(args, synth, llama):
     """The auto-batching stress configuration: 256 concurrent requests, Zipf(1.1) over 256 rank-16 adapters, context lengths uniform in
     128..2048 in a shuffled paged cache pre-filled with N(0,1) values; a step = one decode step of all 256 requests
-    (per-operator path: the token count exceeds the 64-token decode tile of the native step)."""
+    through the native step (one launch per operator beyond 64 sequences), replayed from a captured graph."""
     import torch
     dsm = _mod("decode_session")
     dev = "cuda:0"
@@ -400,7 +400,11 @@ def bench_c5_decode(args, synth, llama):
     kv.begin_forward(list(range(B)), [int(c) for c in ctx])          # claims the pages of the pre-filled contexts
     kv.end_forward()
     first = synth.randint(wl.seed, "c5.first", (B,), s.vocab_size).numpy()
-    sess = dsm.DecodeSession(model, kv, list(range(B)), {0: adapter_ids}, first, longest_first=not args.batch_order)
+    if args.python_loop:
+        sess = dsm.DecodeSession(model, kv, list(range(B)), {0: adapter_ids}, first, longest_first=not args.batch_order)
+    else:
+        sess = dsm.NativeDecodeSession(model, kv, list(range(B)), adapter_ids, first, use_graph=not args.no_graph,
+                                       longest_first=not args.batch_order)
     for _ in range(args.warmup):
         sess.step()
     torch.cuda.synchronize()
@@ -419,7 +423,8 @@ def bench_c5_decode(args, synth, llama):
         "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": wl.name, "layers": s.num_hidden_layers, "batch": B, "adapters_in_use": used,
-                   "total_context": int(ctx.sum()), "host_loop": "python",
+                   "total_context": int(ctx.sum()),
+                   "host_loop": "python" if args.python_loop else ("mlora_decode_step" if args.no_graph else "hipGraph replay of mlora_decode_step"),
                    "base_gemm": "this package's kernels"},
         "roofline": {"kernel": "whole decode step (paged attention 91 % of the bytes)", "bound": "hbm",
                      "achieved": step_bytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -17,15 +17,118 @@ __global__ void advance_kernel(int32_t* __restrict__ pos, int32_t* __restrict__ 
     if (int e_ = (call)) return e_;  \
   } while (0)
 
+// The step for more than 64 sequences: the same operator sequence with one launch per operator (the fused forms above
+// are built around a token block that fits one wave).  Activations stay in fragment order, the linears run on the
+// matrix-core kernel for mid-size token blocks, the two narrow accumulating ones split over K slices whose partials
+// the next RMSNorm adds, and the adapter deltas are matrix-core gather-matmuls (q, k, v and gate, up grouped).
+int decode_step_wide(const mlora_decode_plan* p, void* stream) {
+  const int T = p->T, H = p->hidden, I = p->inter, Hq = p->n_q_heads, Hkv = p->n_kv_heads, D = p->head_dim;
+  const int q_sz = Hq * D, kv_sz = Hkv * D, qkv_sz = q_sz + 2 * kv_sz;
+  MLORA_CHECK(H % 32 == 0 && I % 32 == 0 && q_sz % 32 == 0, MLORA_ERR_UNSUPPORTED,
+              "decode_step: more than 64 sequences need hidden, intermediate and q sizes that are multiples of 32");
+  const bool lora = p->tok_adapter != nullptr && p->lora_r > 0;
+  const int r = p->lora_r, n_ad = p->lora_n_ad;
+  const float sc = p->lora_scaling;
+  f16* qkv = (f16*)p->qkv;
+  f16* gu = (f16*)p->gate_up;
+  const int Kmax = H > I ? (H > q_sz ? H : q_sz) : (I > q_sz ? I : q_sz);
+  MLORA_CHECK(!lora || (p->lora_ws && p->lora_ws_bytes >= 3 * mlora_gather_mm_workspace_bytes(T, Kmax, r)), MLORA_ERR_WORKSPACE,
+              "decode_step: lora_ws of %zu bytes given, %zu needed", p->lora_ws_bytes, 3 * mlora_gather_mm_workspace_bytes(T, Kmax, r));
+  // adapter deltas of the projections lp[0..n) that read x and write column ranges of y: two or more go out as one group
+  auto deltas = [&](void* y, int y_dtype, int ldy, const void* x, int K, const mlora_lora_proj* const* lp, const int32_t* col,
+                    const int32_t* ncol, int n) -> int {
+    if (!lora) return MLORA_OK;
+    mlora_lora_bucket bk[3];
+    int32_t c[3], nc[3];
+    int live = 0;
+    for (int i = 0; i < n; ++i)
+      if (lp[i]->A) {
+        bk[live] = mlora_lora_bucket{lp[i]->A, lp[i]->B, r, n_ad, sc};
+        c[live] = col[i];
+        nc[live] = ncol[i];
+        ++live;
+      }
+    if (live >= 2)
+      return mlora_gather_mm_multi_proj(y, y_dtype, ldy, x, MLORA_FRAG, bk, 1, live, c, nc, nullptr, p->tok_adapter, T, K, p->lora_ws,
+                                        p->lora_ws_bytes, stream);
+    const size_t esz = y_dtype == MLORA_F16 ? 2 : 4;
+    for (int i = 0; i < live; ++i)
+      STEP(mlora_gather_mm((char*)y + (size_t)c[i] * esz, y_dtype, ldy, x, MLORA_FRAG, bk[i].A, bk[i].B, p->tok_adapter, sc, T, K, nc[i], r,
+                           n_ad, p->lora_ws, p->lora_ws_bytes, stream));
+    return MLORA_OK;
+  };
+  auto ksplit_of = [&](int K) -> int {
+    const int ks = p->ksplit_ws ? mlora_gemv_ksplit(T, K, H) : 1;
+    return ks > 1 && mlora_gemv_ksplit_bytes(T, H, ks) <= p->ksplit_ws_bytes ? ks : 1;
+  };
+  auto norm = [&](const void* w, int ks) -> int {
+    if (ks > 1)
+      return mlora_rmsnorm_ksplit(p->xn, MLORA_FRAG, p->resid, p->ksplit_ws, ks, H, w, p->eps, T, H, nullptr, 0, nullptr, nullptr, 0.f, 0,
+                                  0, 0, stream);
+    return mlora_rmsnorm(p->xn, MLORA_FRAG, p->resid, MLORA_F32, w, p->eps, T, H, stream);
+  };
+  int pending_ks = 1;
+  STEP(mlora_embed(p->resid, MLORA_F32, p->embed, p->tokens, T, H, p->vocab, stream));
+  for (int l = 0; l < p->n_layers; ++l) {
+    const mlora_layer& L = p->layers[l];
+    MLORA_CHECK(L.gate_up_p, MLORA_ERR_INVALID, "decode_step: layer %d needs gate_up_p", l);
+    STEP(norm(L.ln1, pending_ks));
+    STEP(mlora_linear_frag(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, stream));
+    {
+      const mlora_lora_proj* lp[3] = {&L.lora[MLORA_Q], &L.lora[MLORA_K], &L.lora[MLORA_V]};
+      const int32_t col[3] = {0, q_sz, q_sz + kv_sz}, ncol[3] = {q_sz, kv_sz, kv_sz};
+      STEP(deltas(qkv, MLORA_F16, qkv_sz, p->xn, H, lp, col, ncol, 3));
+    }
+    STEP(mlora_rope_kv_append(qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos, p->rope_cos, p->rope_sin,
+                              p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, stream));
+    STEP(mlora_paged_attn_decode(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->ctx, T, Hq,
+                                 Hkv, D, p->n_pages, p->n_seq, stream));
+    const int ks_o = ksplit_of(q_sz);
+    STEP(mlora_gemv_frag_acc_ksplit(p->resid, nullptr, p->ksplit_ws, ks_o, p->attn, L.o_p, T, q_sz, H, 0, nullptr, nullptr, 0, nullptr, 0, 0,
+                                    stream));
+    {
+      const mlora_lora_proj* lp[1] = {&L.lora[MLORA_O]};
+      const int32_t col[1] = {0}, ncol[1] = {H};
+      STEP(deltas(p->resid, MLORA_F32, H, p->attn, q_sz, lp, col, ncol, 1));
+    }
+    STEP(norm(L.ln2, ks_o));
+    STEP(mlora_linear_frag(gu, MLORA_F16, MLORA_STORE, p->xn, L.gate_up_p, T, H, 2 * I, stream));
+    {
+      const mlora_lora_proj* lp[2] = {&L.lora[MLORA_GATE], &L.lora[MLORA_UP]};
+      const int32_t col[2] = {0, I}, ncol[2] = {I, I};
+      STEP(deltas(gu, MLORA_F16, 2 * I, p->xn, H, lp, col, ncol, 2));
+    }
+    STEP(mlora_silu_mul(p->act, MLORA_FRAG, gu, gu + I, 2 * I, T, I, stream));
+    pending_ks = ksplit_of(I);
+    STEP(mlora_gemv_frag_acc_ksplit(p->resid, nullptr, p->ksplit_ws, pending_ks, p->act, L.down_p, T, I, H, 0, nullptr, nullptr, 0, nullptr, 0,
+                                    0, stream));
+    {
+      const mlora_lora_proj* lp[1] = {&L.lora[MLORA_DOWN]};
+      const int32_t col[1] = {0}, ncol[1] = {H};
+      STEP(deltas(p->resid, MLORA_F32, H, p->act, I, lp, col, ncol, 1));
+    }
+  }
+  STEP(norm(p->norm, pending_ks));
+  STEP(mlora_linear_frag(p->logits, MLORA_F32, MLORA_STORE, p->xn, p->lm_head_p, T, H, p->vocab, stream));
+  STEP(mlora_argmax(p->tokens, p->logits, T, p->vocab, stream));
+  hipLaunchKernelGGL(advance_kernel, dim3((T + 63) / 64), dim3(64), 0, (hipStream_t)stream, p->pos, p->ctx, T);
+  return mlora_launch_status("decode_step");
+}
+
 }  // namespace
 
 extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
   MLORA_CHECK(p && p->layers, MLORA_ERR_INVALID, "decode_step: null plan");
   const int T = p->T, H = p->hidden, I = p->inter, Hq = p->n_q_heads, Hkv = p->n_kv_heads, D = p->head_dim;
-  MLORA_CHECK(T > 0 && T <= 64, MLORA_ERR_UNSUPPORTED, "decode_step: T=%d outside 1..64", T);
+  MLORA_CHECK(T > 0 && T <= 65535, MLORA_ERR_UNSUPPORTED, "decode_step: T=%d outside 1..65535", T);
   MLORA_CHECK(p->tokens && p->rows && p->pos && p->ctx && p->resid && p->xn && p->qkv && p->attn && p->gate_up && p->act &&
                   p->logits && p->embed && p->norm && p->lm_head_p && p->block_table && p->rope_cos && p->rope_sin,
               MLORA_ERR_INVALID, "decode_step: null buffer");
+  if (T > 64) {
+    MLORA_CHECK(!(p->tok_adapter != nullptr && p->lora_r > 0 && p->lora_dense != 0), MLORA_ERR_UNSUPPORTED,
+                "decode_step: the dense shrink (adapter rows appended to the base weights) serves at most 64 sequences (T=%d)", T);
+    return decode_step_wide(p, stream);
+  }
   const int q_sz = Hq * D, kv_sz = Hkv * D, qkv_sz = q_sz + 2 * kv_sz;
   const bool lora = p->tok_adapter != nullptr && p->lora_r > 0;
   const bool dense = lora && p->lora_dense != 0;

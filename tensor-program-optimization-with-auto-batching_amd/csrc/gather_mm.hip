@@ -1391,7 +1391,7 @@ extern "C" int mlora_gather_mm_multi(void* y, int y_dtype, int ldy, const void* 
                                      const int32_t* tok_adapter, int T, int K, int N, void* workspace,
                                      size_t workspace_bytes, void* stream) {
   MLORA_CHECK(buckets && n_buckets > 0 && n_buckets <= 64, MLORA_ERR_INVALID, "gather_mm_multi: bad bucket list (n_buckets=%d)", n_buckets);
-  MLORA_CHECK(tok_bucket && tok_adapter, MLORA_ERR_INVALID, "gather_mm_multi: null id array");
+  MLORA_CHECK((tok_bucket || n_buckets == 1) && tok_adapter, MLORA_ERR_INVALID, "gather_mm_multi: null id array");
   // validate every bucket before the first launch, so that an error leaves y untouched
   for (int b = 0; b < n_buckets; ++b) {
     if (!buckets[b].A && !buckets[b].B) continue;       // this bucket's adapters do not target the projection
@@ -1422,7 +1422,8 @@ extern "C" int mlora_gather_mm_multi_proj(void* y, int y_dtype, int ldy, const v
                                           void* stream) {
   MLORA_CHECK(buckets && n_buckets > 0 && n_buckets <= 64 && n_proj > 0 && n_proj <= 8, MLORA_ERR_INVALID,
               "gather_mm_multi_proj: bad bucket list (n_buckets=%d n_proj=%d)", n_buckets, n_proj);
-  MLORA_CHECK(y && x && col_offset && n_cols && tok_bucket && tok_adapter, MLORA_ERR_INVALID, "gather_mm_multi_proj: null pointer");
+  MLORA_CHECK(y && x && col_offset && n_cols && (tok_bucket || n_buckets == 1) && tok_adapter, MLORA_ERR_INVALID,
+              "gather_mm_multi_proj: null pointer");
   MLORA_CHECK(y_dtype == MLORA_F16 || y_dtype == MLORA_F32, MLORA_ERR_INVALID, "gather_mm_multi_proj: bad y_dtype %d", y_dtype);
   // validate everything before the first launch, so that an error leaves y untouched
   for (int p = 0; p < n_proj; ++p) {

@@ -483,24 +483,28 @@ int launch_gemm_pp(void* y, const f16* x, int ldx, int x_tt, const f16* Wp, int 
 // many sequences, a short prefill).  The weights are read once and the matrix cores and the operand loads weigh about
 // the same, so the block is as tall as the token block allows and narrow enough to give every compute unit a
 // workgroup: FT x 8 fragments (128 or 256 tokens x 128 weight rows), eight waves, both operands in fragment order and
-// copied from global memory straight into a six-stage LDS ring of 32-k steps (the weight stream comes from HBM: five
-// stages, 40 KiB of it, are in flight per compute unit).  grid = (weight-row blocks, K slices, token blocks).
+// copied from global memory straight into an LDS ring.  A stage of the ring is TWO 32-k steps (32 or 48 KiB): with the
+// few MFMAs a wave has per 32-k step here (8 or 16), a barrier and a wait per step cost more than the step itself.
+// Four (three) stages, of which three (two) - 96 KiB - are in flight per compute unit.
+// grid = (weight-row blocks, K slices, token blocks).
 // With K slices, slice 0 produces the result proper (store or accumulate) and slice s > 0 stores its fp32 partial
 // sums to part[s - 1][T][ld_part] - for the two narrow accumulating linears of a layer, whose partials the next
 // RMSNorm of the row adds in slice order.
 // ---------------------------------------------------------------------------------------------
-constexpr int MID_STAGES = 6;
 constexpr int MID_FN = 8;
+constexpr int MID_KS = 2;                      // 32-k steps per stage
 
 template <int OUT, int FT>
 __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __restrict__ yv, float* __restrict__ part, int ld_part,
                                                                     const f16* __restrict__ xf, int x_tt, const f16* __restrict__ Wp,
                                                                     int T, int K, int N) {
-  constexpr int LF = MID_FN + FT;              // fragments per stage: weights, then tokens
-  constexpr int LQ = LF / PP_WAVES;            // ... of which a wave fetches LQ (fragment f = wave + 8 q)
+  constexpr int MID_STAGES = FT == 16 ? 3 : 4;
+  constexpr int SF = MID_FN + FT;              // fragments of one 32-k step: weights, then tokens
+  constexpr int LF = MID_KS * SF;              // fragments per stage
+  constexpr int LQ = LF / PP_WAVES;            // ... of which a wave fetches LQ (fragment f = wave + 8 q, k-step f / SF)
   constexpr int STAGE_ELEMS = LF * 512;
   constexpr int WTF = FT / 4;                  // token fragments of a wave's tile
-  static_assert(LF % PP_WAVES == 0 && FT % 4 == 0, "fragments divide over the waves");
+  static_assert(LF % PP_WAVES == 0 && FT % 4 == 0 && SF % PP_WAVES == 0, "fragments divide over the waves");
   extern __shared__ __align__(16) f16 smem[];  // [MID_STAGES][STAGE_ELEMS]; the output staging reuses it after the K loop
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int KB = K / 32;
@@ -509,13 +513,16 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
   const int per = (KB + gridDim.y - 1) / gridDim.y;
   const int kb0 = blockIdx.y * per;
   const int kb1 = kb0 + per < KB ? kb0 + per : KB;
-  const int nst = kb1 - kb0;                   // stages of this slice (>= 1: checked by the launcher)
+  const int nks = kb1 - kb0;                   // 32-k steps of this slice (>= 1: checked by the launcher)
+  const int nst = (nks + MID_KS - 1) / MID_KS; // stages
 
+  // fragment f = wave + 8 q of a stage: k-step f / SF of the stage, fragment f % SF of that step (SF % 8 == 0, so a
+  // wave fetches the same fragments of every step)
   const f16* src[LQ];
   int step[LQ];
 #pragma unroll
   for (int q = 0; q < LQ; ++q) {
-    const int f = wave + PP_WAVES * q;         // uniform
+    const int f = (wave + PP_WAVES * q) % SF;  // uniform
     if (f < MID_FN) {
       int nt = n0 / 16 + f;
       nt = nt < tiles ? nt : tiles - 1;        // rows past N: a valid fragment, results dropped
@@ -530,19 +537,21 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
   }
   int ring = 0, load_kb = kb0;
   auto issue = [&]() {
-    const int kb = load_kb < kb1 ? load_kb : kb1 - 1;   // past the slice: a valid address, into a slot nobody reads any more
     f16* dst = smem + ring * STAGE_ELEMS + wave * 512;
 #pragma unroll
-    for (int q = 0; q < LQ; ++q)
+    for (int q = 0; q < LQ; ++q) {
+      int kb = load_kb + (wave + PP_WAVES * q) / SF;
+      kb = kb < kb1 ? kb : kb1 - 1;            // past the slice: a valid address; the data is not multiplied
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + (size_t)kb * step[q]),
                                        (__attribute__((address_space(3))) void*)(dst + q * PP_WAVES * 512), 16, 0, 0);
+    }
     ring = ring + 1 == MID_STAGES ? 0 : ring + 1;
-    ++load_kb;
+    load_kb += MID_KS;
   };
 
   const int wn = wave & 1, wt = wave >> 1;     // weight rows wn * 64 .., tokens wt * WTF * 16 ..
   f32x4 acc[4][WTF];
-  f16x8 a[2][4], b[2][WTF];
+  f16x8 a[2][MID_KS][4], b[2][MID_KS][WTF];    // two register sets: the stage being multiplied and its successor
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -552,25 +561,35 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
     constexpr int u = decltype(U)::value;
     const f16* st = smem + rd * STAGE_ELEMS + lane * 8;
 #pragma unroll
-    for (int j = 0; j < WTF; ++j) b[u][j] = ld8(st + (MID_FN + wt * WTF + j) * 512);
+    for (int ks = 0; ks < MID_KS; ++ks) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a[u][i] = ld8(st + (wn * 4 + i) * 512);
+      for (int j = 0; j < WTF; ++j) b[u][ks][j] = ld8(st + (ks * SF + MID_FN + wt * WTF + j) * 512);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[u][ks][i] = ld8(st + (ks * SF + wn * 4 + i) * 512);
+    }
     rd = rd + 1 == MID_STAGES ? 0 : rd + 1;
   };
+  int done_ks = 0;                             // 32-k steps multiplied so far
   auto multiply = [&](auto U) {
     constexpr int u = decltype(U)::value;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int ks = 0; ks < MID_KS; ++ks) {
+      if (done_ks + ks < nks) {                // uniform: the last stage of an odd slice holds one step only
 #pragma unroll
-      for (int j = 0; j < WTF; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][i], b[u][j], acc[i][j], 0, 0, 0);
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < WTF; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][ks][i], b[u][ks][j], acc[i][j], 0, 0, 0);
+      }
+    }
+    done_ks += MID_KS;
   };
   // the wait: of this wave's loads at most those of the MID_STAGES - 2 youngest stages are still in flight, so the
   // stage multiplied next has landed; with everybody's wait and fragment reads behind the barrier, the slot of the
   // stage just read is refilled
   auto wait_next = [&]() {
-    if constexpr (LQ == 2) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
-    static_assert(MID_STAGES == 6 && (LQ == 2 || LQ == 3), "the immediate above is (MID_STAGES - 2) * LQ");
+    if constexpr (FT == 16) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+    static_assert((MID_STAGES - 2) * LQ == (FT == 16 ? 6 : 8), "the immediates above");
   };
   auto stage = [&](auto U) {
     constexpr int u = decltype(U)::value;
@@ -684,7 +703,7 @@ MidShape gemm_mid_shape(int T, int K, int N, int ksplit_max) {
 template <int OUT, int FT>
 int launch_gemm_mid_ft(void* y, float* part, int ld_part, int ksplit, const f16* xf, int x_tt, const f16* Wp, int T, int K, int N,
                        hipStream_t s) {
-  constexpr size_t lds = (size_t)MID_STAGES * (MID_FN + FT) * 512 * sizeof(f16);
+  constexpr size_t lds = (size_t)(FT == 16 ? 3 : 4) * MID_KS * (MID_FN + FT) * 512 * sizeof(f16);
   static_assert(lds >= (size_t)PP_WAVES * PP_OUT_ELEMS * sizeof(f16), "the output staging fits the ring");
   static bool configured = false;                    // the attribute is per kernel, set once per process
   if (!configured) {

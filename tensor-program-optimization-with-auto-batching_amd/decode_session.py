@@ -86,7 +86,10 @@ class NativeDecodeSession:
     as a tuple, several types of equal scaling served from their padded union (`adapter_ids` = rows of
     `model.lora_union(tid)`, see `model.union_rows`)."""
 
-    def __init__(self, model, kv, seq_ids, adapter_ids, first_tokens, tid=0, use_graph=True, dense_lora=None, fuse_silu=True, ksplit=True):
+    def __init__(self, model, kv, seq_ids, adapter_ids, first_tokens, tid=0, use_graph=True, dense_lora=None, fuse_silu=True, ksplit=True,
+                 longest_first=False):
+        """longest_first: as in DecodeSession - the batch runs internally in order of decreasing context length and
+        step() returns the tokens in the caller's order (`tokens` and `buf` stay in the internal order)."""
         import ctypes as C
         from . import _lib
         self.model, self.kv = model, kv
@@ -94,8 +97,14 @@ class NativeDecodeSession:
         s = model.shape
         dev = model.device
         T = len(self.seq_ids)
-        if T > 64:
-            raise ValueError("NativeDecodeSession handles at most 64 sequences per step")
+        self._inv = None
+        if longest_first and T > 1:
+            order = np.argsort(-np.asarray([kv.lens[q] for q in self.seq_ids], dtype=np.int64), kind="stable")
+            self.seq_ids = [self.seq_ids[i] for i in order]
+            if adapter_ids is not None:
+                adapter_ids = np.asarray(adapter_ids, dtype=np.int32).reshape(-1)[order]
+            first_tokens = torch.as_tensor(first_tokens).cpu().numpy().reshape(-1)[order]
+            self._inv = torch.from_numpy(np.argsort(order)).to(dev)
         lt = None
         if adapter_ids is not None and model.lora_types:
             lt = model.lora_union(tid)[0] if isinstance(tid, tuple) else model.lora_types[tid]
@@ -136,7 +145,9 @@ class NativeDecodeSession:
         # are small next to the base weight and most adapters are in use (the extra rows are read whether or not
         # an adapter has a token in the batch).
         if dense_lora is None:
-            dense_lora = lt is not None and lt.n_adapters <= 2 * T
+            dense_lora = lt is not None and lt.n_adapters <= 2 * T and T <= 64
+        if dense_lora and T > 64:
+            raise ValueError("NativeDecodeSession: the dense shrink serves at most 64 sequences per step")
         self.dense_lora = bool(dense_lora and lt is not None)
         ext = model.dense_lora_weights(tid) if self.dense_lora else None
         il = model.interleaved_gate_up() if (fuse_silu and s.intermediate_size % 32 == 0) else None
@@ -198,6 +209,7 @@ class NativeDecodeSession:
         else:
             self._enqueue()
         kv.end_forward()
+        out = self.tokens if self._inv is None else self.tokens.index_select(0, self._inv)
         if keep_history:
-            self.history.append(self.tokens.clone())
-        return self.tokens
+            self.history.append(out.clone() if self._inv is None else out)
+        return out

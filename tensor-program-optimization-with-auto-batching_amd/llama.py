@@ -348,7 +348,7 @@ class LlamaForCausalLM:
                     resid += pv[q, :, :H]
                 parts = None
             resid = resid[logits_rows].contiguous()
-        xn = ops.rmsnorm(resid, self.norm, s.rms_norm_eps, frag=resid.shape[0] <= 64, parts=parts)
+        xn = ops.rmsnorm(resid, self.norm, s.rms_norm_eps, frag=resid.shape[0] <= 64 or frag, parts=parts)
         return ops.linear(xn, self.lm_head, out_dtype=torch.float32)
 
     def _ksplit_ws(self, T):

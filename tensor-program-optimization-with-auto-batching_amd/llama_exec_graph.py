@@ -25,10 +25,10 @@ class LlamaExecConfig:
     max_prompt_len: int
     max_gen_len: int
     page_size: int
-    # Run decode batches of one adapter type (or none) and at most 64 sequences through the native decode step (one
-    # C call per step, graph replay when several steps lie ahead) instead of one call per operator, and batches that
-    # mix adapter types through the per-operator step recorded into a graph.  Same tokens: the native step with
-    # ids-based LoRA shrink is bit-identical to the per-operator path.
+    # Run decode batches of one adapter type (or none) through the native decode step (one C call per step, graph
+    # replay when several steps lie ahead) instead of one call per operator, and batches that mix adapter types
+    # through the per-operator step recorded into a graph.  Same tokens: the native step with ids-based LoRA shrink
+    # is bit-identical to the per-operator path.
     native_decode: bool = True
     # Let the native step compute the LoRA shrink of all adapters as extra rows of the base GEMV (the fastest form
     # while the adapters are few and low-rank: taken when every rank is at most 16).  It then also serves batches
@@ -170,8 +170,8 @@ class LlamaExecGraph(ExecGraph):
         # sequence takes at least one step after its prefill, also when its first token is EOS or max_gen_len is 1.
         while seqs:
             method, params = self.seq_info.get_decode_method(seqs)
-            if getattr(self.exec_config, "native_decode", False) and len(seqs) <= 64:
-                dense = self._dense_ok(method)
+            if getattr(self.exec_config, "native_decode", False):
+                dense = len(seqs) <= 64 and self._dense_ok(method)       # the dense shrink serves at most 64 sequences
                 seqs = self._decode_native(seqs, outputs, method, params, dense) if dense or not method.startswith("mixed_decode") \
                     else self._decode_session(seqs, outputs, method, params)
                 continue

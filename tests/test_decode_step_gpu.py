@@ -157,6 +157,49 @@ def test_native_step_between_33_and_64_requests():
     assert err <= 1e-2, err
 
 
+@pytest.mark.parametrize("batch,targets,r", [(65, ("q_proj", "k_proj", "v_proj", "o_proj"), 16), (128, ("q_proj", "v_proj"), 8),
+                                              (256, ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"), 16),
+                                              (100, (), 16)])
+def test_native_step_for_more_than_64_requests(batch, targets, r):
+    """Beyond the 64-token decode tile the native step issues one launch per operator (matrix-core linears on
+    fragment-ordered activations, K slices on o_proj and down_proj, grouped matrix-core LoRA): tokens and the whole K
+    cache are bit-identical to the per-operator path, eagerly and replayed from a graph, and the first step's logits
+    agree with the oracle."""
+    synth, llama = load_pkg("synth"), load_pkg("llama")
+    wl = synth.config3(num_layers=2, batch=batch, prompt_len=20)
+    lora = synth.LoraSpec(r=r, alpha=float(r), n_adapters=24, targets=targets or ("q_proj",))
+    ids = synth.randint(wl.seed, f"wide.ids{batch}", (batch,), 24).numpy().astype(np.int32)
+    ids[[3, batch - 1]] = -1
+    if not targets:
+        ids[:] = -1
+    wl = synth.Workload("wide", wl.seed, wl.shape, lora, batch=batch, prompt_len=20, gen_len=6, adapter_ids=ids)
+    model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, [wl.lora], DEV)
+    prompts = synth.prompts(wl)
+    steps = 5
+    a, ka, _ = _run(model, wl, prompts, ids, "py", steps, synth)
+    b, kb, lg = _run(model, wl, prompts, ids, "native", steps, synth)
+    c, kc, _ = _run(model, wl, prompts, ids, "graph", steps, synth)
+    assert np.array_equal(a, b) and np.array_equal(a, c)
+    assert torch.equal(ka, kb) and torch.equal(ka, kc)
+    with pytest.raises(ValueError, match="dense"):
+        _run(model, wl, prompts, ids, "dense", steps, synth, run_steps=1)
+    # the first decode step against the oracle, from the oracle's own prefill of the same prompts
+    ref = oracle_model(wl, "mixed")
+    blocks = -(-(wl.prompt_len + steps + 2) // 16)
+    kvr = ref.new_cache(batch * blocks, 16, blocks * 16, synth.permutation(wl.seed, "pages", batch * blocks))
+    for q in range(batch):
+        kvr.add_sequence(q)
+    kvr.begin_forward(list(range(batch)), [wl.prompt_len] * batch)
+    ref.forward(prompts.reshape(-1), kvr, {"a0": np.repeat(ids, wl.prompt_len)}, logits_rows=np.arange(batch))
+    kvr.end_forward()
+    kvr.begin_forward(list(range(batch)), [1] * batch)
+    exp = ref.forward(a[0], kvr, {"a0": ids})
+    kvr.end_forward()
+    err = float(np.abs(lg.float().cpu().numpy() - exp).max() / exp.std())
+    print(f"{batch} requests, first native step vs oracle: {err:.2e} of the logit std", flush=True)
+    assert err <= 1e-2
+
+
 def test_native_step_at_most_16_requests():
     """12 requests at the benchmark model's layer shapes (one token tile: the one-tile forms of the per-unit q/k/v and
     SiLU GEMVs, K-range blocks of the appended adapter rows): the native step reproduces the per-operator path bit for

@@ -126,8 +126,8 @@ def test_decode_more_than_64_requests_zipf_adapters_ragged_contexts():
         assert list(kvh.table_h[kvh.slot[s], :n_blk]) == list(kvr.tables[s])[:n_blk]
 
 
-@pytest.mark.parametrize("B,use_graph", [(70, False), (12, True)])
-def test_decode_session_longest_context_first_keeps_tokens_and_request_order(B, use_graph):
+@pytest.mark.parametrize("B,use_graph,native", [(70, False, False), (12, True, False), (70, True, True), (12, False, True)])
+def test_decode_session_longest_context_first_keeps_tokens_and_request_order(B, use_graph, native):
     """The session may run its batch internally in order of decreasing context length (the long sequences' attention
     workgroups start first); every operator treats rows independently, so each request's tokens and cache pages are
     those of the batch in request order, bit for bit, and come back in request order."""
@@ -148,7 +148,11 @@ def test_decode_session_longest_context_first_keeps_tokens_and_request_order(B, 
     for longest_first in (False, True):
         kv, logits = _hip_prefill(model, prompts, ids, n_pages, 16, perm, 112)
         first = logits.argmax(-1).astype(np.int32)
-        sess = dsm.DecodeSession(model, kv, list(range(B)), {0: ids}, first, use_graph=use_graph, longest_first=longest_first)
+        if native:
+            sess = dsm.NativeDecodeSession(model, kv, list(range(B)), ids, first, use_graph=use_graph, longest_first=longest_first,
+                                           dense_lora=False)
+        else:
+            sess = dsm.DecodeSession(model, kv, list(range(B)), {0: ids}, first, use_graph=use_graph, longest_first=longest_first)
         toks = np.stack([sess.step().cpu().numpy().copy() for _ in range(steps)])
         rows = [[kv.k[0][p].clone() for p in kv.pages_of(s)] for s in range(B)]
         runs.append((toks, rows, [kv.lens[s] for s in range(B)]))
