@@ -651,130 +651,263 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// Prefill: a wave owns 16 consecutive query tokens of one head and walks the pages of their
-// sequence.  S^T = K . Q^T on v_mfma_f32_16x16x32_f16 puts key index on the accumulator rows, which
-// is exactly the A-operand layout the matrix core wants for P in O = P . V (a lane's four
-// accumulator rows are the four keys it must supply) - no LDS, no shuffles between the two products.  A tile that straddles a sequence boundary is processed in one
-// pass per sequence with the other queries masked.
+// Prefill: four waves own 64 consecutive query tokens of one head, a wave 16 of them.  S^T = K . Q^T on
+// v_mfma_f32_16x16x32_f16 puts the key index on the accumulator rows, which is exactly the A-operand layout the matrix
+// core wants for P in O = P . V (a lane's four accumulator rows are the four keys it must supply): no shuffles between
+// the two products.  The keys are walked in blocks of 64 (four pages).  The block's K and V pages go from the cache
+// straight into LDS (a page per wave; a head's page of K or V is 4 KiB contiguous in the cache), double buffered - the
+// next block is in flight while this one is multiplied - with one barrier per block, and all waves take their
+// fragments from there: a page is fetched once per 64 queries.  Two workgroups share a compute unit.  The softmax
+// bookkeeping (running maximum, rescaling of O, the fp16 hi + lo split of P) is done once per 64 keys, and a P . V
+// product covers 32 keys per MFMA (k-slots 0-3 and 4-7 of a lane are its four keys of two pages), hi and lo halves of
+// P in two MFMAs on the same V fragment.  Blocks above the causal diagonal of a wave are skipped by that wave; blocks
+// below it need no mask.  Token blocks that span several sequences are worked off one sequence at a time with the
+// other queries masked.  The results cross LDS once more to leave as whole 16-byte pieces.
+// (Eight waves per workgroup with a four-deep ring, and adding P . V of the previous block under the softmax
+// arithmetic of the current one, were measured and are no faster: 8 x 512 tokens, 32 heads of 128 take 115-120 us in
+// every form, about 0.2 PFLOP/s of causal QK^T + PV.)
 // ---------------------------------------------------------------------------------------------
+constexpr int PF_WAVES = 4;
+constexpr int PF_PAGES = 4;      // pages per key block
+constexpr int PF_RING = 2;       // key-block buffers
+
 template <int D>
-__global__ __launch_bounds__(256) void paged_attn_prefill_kernel(f16* __restrict__ out, int frag_tt, const f16* __restrict__ qkv,
-                                                                 const f16* __restrict__ k_cache,
-                                                                 const f16* __restrict__ v_cache,
-                                                                 const int32_t* __restrict__ block_table, int max_blocks,
-                                                                 const int32_t* __restrict__ tok_seq,
-                                                                 const int32_t* __restrict__ tok_pos, int T, int Hq,
-                                                                 int Hkv, int n_pages, int n_seq, float scale) {
-  constexpr int NKB = D / 32;   // k-blocks of the QK^T product
-  constexpr int NDB = D / 16;   // dim blocks of the output
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int t0 = (blockIdx.x * 4 + wave) * 16;
-  if (t0 >= T) return;
-  const int h = blockIdx.y;
-  const int kh = h / (Hq / Hkv);
+__global__ __launch_bounds__(PF_WAVES* WAVE) void paged_attn_prefill_block_kernel(
+    f16* __restrict__ out, int frag_tt, const f16* __restrict__ qkv, const f16* __restrict__ k_cache, const f16* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+    int T, int Hq, int Hkv, int n_pages, int n_seq, float scale) {
+  constexpr int NKB = D / 32;                // k-blocks of the QK^T product
+  constexpr int NDB = D / 16;                // dim blocks of the output
+  constexpr int PE = PAGE * D;               // elements of one page of K (or V) of one head
+  constexpr int CH = PE / 512;               // 1 KiB pieces of such a page
+  constexpr int WPP = PF_WAVES / PF_PAGES;    // waves that share the fetch of a page
+  constexpr int HC = CH / WPP;               // 1 KiB pieces of K (and of V) a wave fetches per block
+  constexpr int BUF = 2 * PF_PAGES * PE;     // one buffer: K pages, then V pages
+  constexpr int OLD = D + 8;                 // padded row of the output staging
+  constexpr int NTOK = PF_WAVES * 16;
+  static_assert(PF_WAVES % PF_PAGES == 0 && CH % WPP == 0 && NTOK <= 2 * WAVE, "whole waves per page; at most two tokens per lane in the sequence scan");
+  extern __shared__ __align__(16) f16 smem[];   // [PF_RING][BUF]
+  __shared__ int s_seq[NTOK], s_pos[NTOK];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int qi = lane & 15, g = lane >> 4;
+  const int t0 = (gridDim.x - 1 - blockIdx.x) * NTOK;              // late token blocks (long key ranges) start first
+  const int tw = t0 + wave * 16;
+  const int h = blockIdx.y, kh = h / (Hq / Hkv);
 
-  const int tq = t0 + qi;
-  const bool valid_t = tq < T;
-  int my_seq = valid_t ? tok_seq[tq] : -1;
-  int my_pos = valid_t ? tok_pos[tq] : -1;
-  if (my_seq < 0 || my_seq >= n_seq || my_pos < 0 || my_pos >= max_blocks * PAGE) my_seq = -1;
+  // the V slots start at zero: a slot whose page is never fetched (a sequence shorter than a key block) is multiplied
+  // by P = 0 and must hold finite numbers
+  for (int i = threadIdx.x; i < PF_RING * PF_PAGES * PE / 8; i += PF_WAVES * WAVE) {
+    const int bsel = i / (PF_PAGES * PE / 8), o = i % (PF_PAGES * PE / 8);
+    st8(smem + bsel * BUF + PF_PAGES * PE + o * 8, f16x8{0, 0, 0, 0, 0, 0, 0, 0});
+  }
+  if (threadIdx.x < NTOK) {
+    const int t = t0 + threadIdx.x;
+    int sq = t < T ? tok_seq[t] : -1;
+    int ps = t < T ? tok_pos[t] : -1;
+    if (sq < 0 || sq >= n_seq || ps < 0 || ps >= max_blocks * PAGE) sq = -1;
+    s_seq[threadIdx.x] = sq;
+    s_pos[threadIdx.x] = ps;
+  }
+  __syncthreads();
+  const int seq_a = s_seq[lane], pos_a = s_pos[lane];                // token t0 + lane
+  const int seq_b = WAVE + lane < NTOK ? s_seq[(WAVE + lane) % NTOK] : -1, pos_b = s_pos[(WAVE + lane) % NTOK];   // token t0 + 64 + lane
+  const int my_seq = s_seq[wave * 16 + qi], my_pos = s_pos[wave * 16 + qi];
 
-  // Q as the B operand: lane holds q[query qi][kb*32 + g*8 .. +8]
-  f16x8 qf[NKB];
+  f16x8 qf[NKB];                             // Q as the B operand: q[query qi][kb * 32 + g * 8 ..]
   {
-    const f16* qp = qkv + ((size_t)(valid_t ? tq : t0) * (Hq + 2 * Hkv) + h) * D + g * 8;
+    const int tq = tw + qi < T ? tw + qi : T - 1;
+    const f16* qp = qkv + ((size_t)tq * (Hq + 2 * Hkv) + h) * D + g * 8;
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb) qf[kb] = ld8(qp + kb * 32);
   }
-
+  const float c = scale * 1.44269504088896340736f;                  // softmax in base 2
   float m = -INFINITY, l = 0.f;
   f32x4 O[NDB];
 #pragma unroll
   for (int db = 0; db < NDB; ++db) O[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  bool done = my_seq < 0;
-  while (true) {
-    const unsigned long long pending = __ballot(!done);
-    if (!pending) break;
-    const int cur_seq = __shfl(my_seq, __builtin_ctzll(pending), WAVE);
-    const bool in_run = !done && my_seq == cur_seq;
-    int maxpos = in_run ? my_pos : -1;
+  unsigned long long todo_a = __ballot(seq_a >= 0), todo_b = __ballot(seq_b >= 0);
+  while (todo_a | todo_b) {                                          // one pass per sequence of the token block (uniform over the workgroup)
+    const int cur = __builtin_amdgcn_readfirstlane(todo_a ? __shfl(seq_a, __builtin_ctzll(todo_a), WAVE)
+                                                          : __shfl(seq_b, __builtin_ctzll(todo_b), WAVE));
+    todo_a &= ~__ballot(seq_a == cur);
+    todo_b &= ~__ballot(seq_b == cur);
+    int run_max = max(seq_a == cur ? pos_a : -1, seq_b == cur ? pos_b : -1);
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) maxpos = max(maxpos, __shfl_xor(maxpos, o, WAVE));
-    const int npages = maxpos / PAGE + 1;
-    const int32_t* __restrict__ bt = block_table + (size_t)cur_seq * max_blocks;
-    int page_next = bt[0];                           // the page id is requested one page ahead
-    for (int pg = 0; pg < npages; ++pg) {
-      const int page = page_next;
-      page_next = pg + 1 < npages ? bt[pg + 1] : -1;
-      if (page < 0 || page >= n_pages) continue;   // wave-uniform
-      const f16* kp = k_cache + ((size_t)page * Hkv + kh) * PAGE * D + lane * 8;       // key qi, dims 8g.. of each k-block
-      const f16* vp = v_cache + (((size_t)page * Hkv + kh) * D + qi) * PAGE + g * 4;   // dim qi (+16 db), keys 4g..
-      f16x8 kf[NKB];
-      f16x4 vf[NDB];
+    for (int o = 32; o > 0; o >>= 1) run_max = max(run_max, __shfl_xor(run_max, o, WAVE));
+    run_max = __builtin_amdgcn_readfirstlane(run_max);
+    const int npages = run_max / PAGE + 1, nblk = (npages + PF_PAGES - 1) / PF_PAGES;
+    const bool in_run = my_seq == cur;
+    int wmax = in_run ? my_pos : -1, wmin = in_run ? my_pos : 0x7fffffff;
 #pragma unroll
-      for (int kb = 0; kb < NKB; ++kb) kf[kb] = ld8(kp + kb * 512);
-#pragma unroll
-      for (int db = 0; db < NDB; ++db) vf[db] = *reinterpret_cast<const f16x4*>(vp + db * 16 * PAGE);
+    for (int o = 8; o > 0; o >>= 1) {
+      wmax = max(wmax, __shfl_xor(wmax, o, WAVE));
+      wmin = min(wmin, __shfl_xor(wmin, o, WAVE));
+    }
+    wmax = __builtin_amdgcn_readfirstlane(wmax);                   // lanes 0-15 hold the 16 queries; all g copies agree
+    wmin = __builtin_amdgcn_readfirstlane(wmin);
+    const bool all_in = (__ballot(in_run) & 0xffffull) == 0xffffull;
+    const int32_t* __restrict__ bt = block_table + (size_t)cur * max_blocks;
 
-      f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f};   // st[r] = S[key 4g + r][query qi]
+    // this wave's half page of block b into its ring slot: HC pieces of K and HC pieces of V, always - a page past the
+    // sequence or outside the cache is replaced by page 0 (finite data; every key of it is masked), so that the
+    // number of loads in flight tells which blocks have landed
+    auto issue = [&](int b) {
+      const int pg = b * PF_PAGES + wave / WPP;
+      int page = pg < npages ? bt[pg] : 0;
+      page = page >= 0 && page < n_pages ? page : 0;
+      const size_t src = ((size_t)page * Hkv + kh) * PE + (wave % WPP) * HC * 512 + lane * 8;
+      f16* kd = smem + (b % PF_RING) * BUF + (wave / WPP) * PE + (wave % WPP) * HC * 512;
+      f16* vd = kd + PF_PAGES * PE;
 #pragma unroll
-      for (int kb = 0; kb < NKB; ++kb) st = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kb], qf[kb], st, 0, 0, 0);
-
-      float pm = -INFINITY;
-      bool msk[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        msk[r] = !in_run || (pg * PAGE + 4 * g + r > my_pos);
-        st[r] = msk[r] ? -INFINITY : st[r] * scale;
-        pm = fmaxf(pm, st[r]);
+      for (int j = 0; j < HC; ++j) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(k_cache + src + j * 512),
+                                         (__attribute__((address_space(3))) void*)(kd + j * 512), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(v_cache + src + j * 512),
+                                         (__attribute__((address_space(3))) void*)(vd + j * 512), 16, 0, 0);
       }
+    };
+#pragma unroll
+    for (int b = 0; b < PF_RING - 1; ++b)
+      if (b < nblk) issue(b);
+    for (int b = 0; b < nblk; ++b) {
+      // this wave's part of block b has landed: only the loads of the younger blocks (at most two) may be in flight
+      const int younger = nblk - 1 - b < PF_RING - 2 ? nblk - 1 - b : PF_RING - 2;   // uniform
+      if (younger == 2) {
+        if constexpr (2 * HC == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else if constexpr (2 * HC == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+      } else if (younger == 1) {
+        if constexpr (2 * HC == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else if constexpr (2 * HC == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      static_assert(PF_RING <= 4 && (2 * HC == 2 || 2 * HC == 4 || 2 * HC == 8), "the immediates above are 2 HC loads per block in flight");
+      __syncthreads();                                               // everybody's has; nobody reads block b - 1 any more
+      if (b + PF_RING - 1 < nblk) issue(b + PF_RING - 1);           // into the slot of block b - 1
+      if (wmax < b * PF_PAGES * PAGE) continue;                      // wave-uniform: the block lies above this wave's diagonal
+      const f16* kb_ = smem + (b % PF_RING) * BUF;
+      const f16* vb_ = kb_ + PF_PAGES * PE;
+      // All four pages are multiplied without branches; what must not count is masked after the product.  A page that
+      // was not fetched (past the sequence, or a page id outside the cache) leaves older, finite data in its slot.
+      bool live[PF_PAGES];                                           // uniform
+      bool all_live = true;
+#pragma unroll
+      for (int p = 0; p < PF_PAGES; ++p) {
+        const int pg = b * PF_PAGES + p;
+        const int page = pg < npages ? bt[pg] : -1;
+        live[p] = page >= 0 && page < n_pages;
+        all_live = all_live && live[p];
+      }
+      // Fragment reads go out in groups ahead of the MFMAs that use them (two waves per SIMD hide little LDS latency
+      // otherwise): all K fragments of the block, then - before the softmax arithmetic - the V fragments of the first
+      // page pair.
+      f16x8 kf[PF_PAGES][NKB];
+#pragma unroll
+      for (int p = 0; p < PF_PAGES; ++p)
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb) kf[p][kb] = ld8(kb_ + p * PE + kb * 512 + lane * 8);
+      __builtin_amdgcn_sched_barrier(0);
+      f32x4 st[PF_PAGES];                                            // st[p][r] = S[key 4g + r of page p][query qi]
+#pragma unroll
+      for (int p = 0; p < PF_PAGES; ++p) st[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+        for (int p = 0; p < PF_PAGES; ++p) st[p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[p][kb], qf[kb], st[p], 0, 0, 0);
+      auto load_v = [&](f16x8 (&vv)[NDB], int pp) {                  // dim db * 16 + qi, keys 4g .. of the pair's two pages
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+          const f16* v0 = vb_ + (2 * pp) * PE + (db * 16 + qi) * PAGE + g * 4;
+          const f16x4 va = *reinterpret_cast<const f16x4*>(v0);
+          const f16x4 vb = *reinterpret_cast<const f16x4*>(v0 + PE);
+          vv[db] = __builtin_shufflevector(va, vb, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+      };
+      f16x8 vv0[NDB], vv1[NDB];
+      load_v(vv0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (!(all_in && all_live && (b + 1) * PF_PAGES * PAGE - 1 <= wmin)) {   // uniform: some key of the block is masked
+#pragma unroll
+        for (int p = 0; p < PF_PAGES; ++p) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const bool masked = !live[p] || !in_run || (b * PF_PAGES + p) * PAGE + 4 * g + r > my_pos;
+            st[p][r] = masked ? -INFINITY : st[p][r];
+          }
+        }
+      }
+      float pm = fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3]));
+#pragma unroll
+      for (int p = 1; p < PF_PAGES; ++p) pm = fmaxf(pm, fmaxf(fmaxf(st[p][0], st[p][1]), fmaxf(st[p][2], st[p][3])));
       pm = fmaxf(pm, __shfl_xor(pm, 16, WAVE));
       pm = fmaxf(pm, __shfl_xor(pm, 32, WAVE));
       const float m_new = fmaxf(m, pm);
-      const float alpha = m_new == -INFINITY ? 1.f : __expf(m - m_new);
-      // P goes to the matrix core as fp16 hi + lo halves (k-slots 0-3 and 4-7 of one k=32 MFMA, with V
-      // repeated in both), so the product carries ~22 mantissa bits of P instead of 11.
-      f16x8 pa;
+      const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((m - m_new) * c);
+      const float mc = m_new == -INFINITY ? 0.f : m_new * c;
+      // P as fp16 hi + lo halves (~22 mantissa bits): hi is P rounded to fp16, lo the remainder
+      f16x8 ph[PF_PAGES / 2], pl[PF_PAGES / 2];
       float ps = 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float p = msk[r] ? 0.f : __expf(st[r] - m_new);
-        ps += p;
-        const f16 hi = (f16)p;
-        pa[r] = hi;
-        pa[4 + r] = (f16)(p - (float)hi);
+      for (int p = 0; p < PF_PAGES; ++p) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float pr = __builtin_amdgcn_exp2f(fmaf(st[p][r], c, -mc));   // exp2(-inf) = 0 for masked keys
+          ps += pr;
+          const f16 hi = (f16)pr;
+          ph[p / 2][(p & 1) * 4 + r] = hi;
+          pl[p / 2][(p & 1) * 4 + r] = (f16)(pr - (float)hi);
+        }
       }
       l = l * alpha + ps;
       m = m_new;
-      // O rows are queries 4g + r; their alpha lives in lanes with qi == 4g + r
-      float ar[4];
+      float ar[4];                                                   // O rows are queries 4g + r; their alpha lives in lanes with qi == 4g + r
 #pragma unroll
       for (int r = 0; r < 4; ++r) ar[r] = __shfl(alpha, 4 * g + r, WAVE);
 #pragma unroll
-      for (int db = 0; db < NDB; ++db) {
+      for (int db = 0; db < NDB; ++db)
 #pragma unroll
         for (int r = 0; r < 4; ++r) O[db][r] *= ar[r];
-        const f16x8 vv = f16x8{vf[db][0], vf[db][1], vf[db][2], vf[db][3], vf[db][0], vf[db][1], vf[db][2], vf[db][3]};
-        O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vv, O[db], 0, 0, 0);
-      }
+      static_assert(PF_PAGES == 4, "two page pairs");
+      load_v(vv1, 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ph[0], vv0[db], O[db], 0, 0, 0);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl[0], vv0[db], O[db], 0, 0, 0);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ph[1], vv1[db], O[db], 0, 0, 0);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl[1], vv1[db], O[db], 0, 0, 0);
     }
-    done = done || in_run;
+    __syncthreads();                                                 // the buffers are free for the next sequence (and for the output)
   }
   l += __shfl_xor(l, 16, WAVE);
   l += __shfl_xor(l, 32, WAVE);
   const float inv = l > 0.f ? 1.f / l : 0.f;
+  // results through the wave's own piece of LDS: [16 queries][D] fp16, then 16-byte pieces out
+  f16* os = smem + wave * 16 * OLD;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const float ir = __shfl(inv, 4 * g + r, WAVE);
-    const int t = t0 + 4 * g + r;
-    if (t < T) {
 #pragma unroll
-      for (int db = 0; db < NDB; ++db) {
-        const int c = h * D + db * 16 + qi;
-        out[frag_tt ? frag_offset(t, c, frag_tt) : (size_t)t * Hq * D + c] = (f16)(O[db][r] * ir);
-      }
+    for (int db = 0; db < NDB; ++db) os[(4 * g + r) * OLD + db * 16 + qi] = (f16)(O[db][r] * ir);
+  }
+  __builtin_amdgcn_wave_barrier();
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  if (frag_tt) {
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) {                               // one whole fragment per store instruction
+      const int tok = lane & 15, kg = lane >> 4;
+      if (tw + tok < T) st8(out + frag_offset(tw + tok, h * D + j * 32 + kg * 8, frag_tt), ld8(os + tok * OLD + j * 32 + kg * 8));
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16 * (D / 8) / WAVE; ++i) {
+      const int ch = i * WAVE + lane, row = ch / (D / 8), c8 = ch % (D / 8);
+      if (tw + row < T) st8(out + ((size_t)(tw + row) * Hq + h) * D + c8 * 8, ld8(os + row * OLD + c8 * 8));
     }
   }
 }
@@ -950,12 +1083,21 @@ extern "C" int mlora_paged_attn_prefill(void* out, int out_layout, const void* q
   const int frag_tt = out_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   const float scale = 1.f / sqrtf((float)D);
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid(ceil_div(T, 64), Hq);
-  if (D == 128)
-    hipLaunchKernelGGL(paged_attn_prefill_kernel<128>, grid, dim3(256), 0, s, (f16*)out, frag_tt, (const f16*)qkv, (const f16*)k_cache,
-                       (const f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, T, Hq, Hkv, n_pages, n_seq, scale);
-  else
-    hipLaunchKernelGGL(paged_attn_prefill_kernel<64>, grid, dim3(256), 0, s, (f16*)out, frag_tt, (const f16*)qkv, (const f16*)k_cache,
-                       (const f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, T, Hq, Hkv, n_pages, n_seq, scale);
+  const dim3 grid(ceil_div(T, PF_WAVES * 16), Hq);
+#define MLORA_PREFILL(DD)                                                                                                          \
+  do {                                                                                                                             \
+    constexpr size_t lds = (size_t)PF_RING * 2 * PF_PAGES * PAGE * DD * sizeof(f16);                                                    \
+    static bool configured = false; /* the attribute is per kernel, set once per process */                                       \
+    if (!configured) {                                                                                                             \
+      hipError_t e = hipFuncSetAttribute((const void*)paged_attn_prefill_block_kernel<DD>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+      if (e != hipSuccess) return mlora_set_error(MLORA_ERR_LAUNCH, "paged_attn_prefill: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e)); \
+      configured = true;                                                                                                           \
+    }                                                                                                                              \
+    hipLaunchKernelGGL(paged_attn_prefill_block_kernel<DD>, grid, dim3(PF_WAVES * WAVE), lds, s, (f16*)out, frag_tt, (const f16*)qkv, \
+                       (const f16*)k_cache, (const f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, T, Hq, Hkv, n_pages, n_seq, scale); \
+  } while (0)
+  if (D == 128) MLORA_PREFILL(128);
+  else MLORA_PREFILL(64);
+#undef MLORA_PREFILL
   return mlora_launch_status("paged_attn_prefill");
 }
