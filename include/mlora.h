@@ -253,6 +253,9 @@ int mlora_argmax(int32_t* ids, const float* logits, int B, int V, void* stream);
  *   first ctx_len[b] cached positions of sequence seq_ids[b] (the new token already appended).
  * mlora_paged_attn_prefill: query token t (sequence tok_seq[t], position tok_pos[t]) attends to cached
  *   positions 0..tok_pos[t]; tokens of a sequence must be consecutive in t with increasing positions.
+ * The attention kernels multiply whole pages and mask afterwards: every slot of a page that a block table names
+ * must hold finite numbers before its first use (allocate the cache zero-filled), or P = 0 times a non-finite V
+ * turns the output into NaN.
  * q is read from qkv (already rotated).  out [T, Hq * D] f16 in out_layout.  D in {64, 128};
  * Hq % Hkv == 0, Hq / Hkv <= 16 and B <= 65535 for decode.
  * ------------------------------------------------------------------------------------------- */
