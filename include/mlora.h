@@ -14,6 +14,19 @@
  *   - return value 0 = success, negative = MLORA_ERR_*; mlora_last_error() gives the message of the
  *     last failure on the calling thread;
  *   - shapes are validated on the host before any launch; a rejected call launches nothing.
+ *
+ * Two tiers of entry points
+ *   PUBLIC, one per reference operator - what a binding of the reference needs and what stays stable:
+ *     mlora_gather_mm (+ _workspace_bytes, _static, _multi, _multi_proj, _batch), mlora_lora_shrink / _expand,
+ *     mlora_write_tensor_part, mlora_linear / mlora_linear_packed / mlora_linear_frag (and the gemv / gemm kernels
+ *     they dispatch to), mlora_pack_weight, mlora_pack_activation, mlora_rmsnorm, mlora_silu_mul, mlora_embed,
+ *     mlora_argmax, mlora_rope_kv_append, mlora_paged_attn_decode, mlora_paged_attn_prefill, and
+ *     mlora_decode_step (one whole decode step from a plan).
+ *   INTERNAL, the fused forms from "Decode-step variants" down to mlora_rmsnorm_ksplit - the building blocks of
+ *     mlora_decode_step, exported so that the Python host can run the same step operator by operator (the parity
+ *     tests compare the two bit for bit).  Their argument lists follow the tiling of the kernels (K-range block
+ *     counts, appended weight rows, partial buffers) and may change with it; a binding should call
+ *     mlora_decode_step instead.
  */
 #ifndef MLORA_H
 #define MLORA_H
@@ -289,7 +302,9 @@ int mlora_paged_attn_prefill(void* out, int out_layout, const void* qkv, const v
  *                               partials written by mlora_gemv_frag_lora with this K; v_dense = kq >= 1: v_part is
  *                               y2 [kq][T, 3 * n_ad * r] of mlora_gemv_frag_split (kq = 1) or
  *                               mlora_gemv_frag_split_kq (slot p = projection p; the kq blocks are added in order);
- *                               v_dense must lie in 0..4 (the kernels keep at most four blocks), else MLORA_ERR_UNSUPPORTED;
+ *                               v_dense must lie in 0..4 (the kernels keep at most four blocks), else MLORA_ERR_UNSUPPORTED.
+ *                               (One argument for two facts - which form the shrink results have, and how many
+ *                               blocks - because the ids-based form has no block count: 0 is not a count.)
  *   mlora_lora_expand_rmsnorm - resid[t, :] += scaling * B[id_t] . v (B [n_ad, H, r]; v_part [kc][T][r] partials
  *                               of a shrink over K inputs, or y2 [T, n_ad * r] when v_dense = 1), then
  *                               y = RMSNorm(resid) as mlora_rmsnorm.

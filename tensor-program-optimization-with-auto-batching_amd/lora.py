@@ -1,7 +1,7 @@
 """LoRA adapter description and the adapter-indexed linear layer.
 
 `LoraConfig` is the reference's dataclass (`tvm/llama_auto_batcher/lora.py:5-8`); `scaling = alpha / r`
-(`lora.py:13`).  `GatherMMLinear` is the drop-in for the PEFT custom module
+(`lora.py:13`); `Lora` its adapter definition with the four protocol methods (`lora.py:10-24`).  `GatherMMLinear` is the drop-in for the PEFT custom module
 `GatherBMMLinear` (`huggingface/custom_peft/lora_gatherbmm_linear_layer.py:5-54`): same forward contract
 (`forward(x, adapter_names=[...])`, one adapter per request), but the per-request stack of A / B and the
 two bmm launches are replaced by one gather-matmul call that indexes the stacked adapter table inside
@@ -24,6 +24,45 @@ class LoraConfig:
     @property
     def scaling(self) -> float:
         return self.alpha / self.r
+
+
+class Lora:
+    """The reference's adapter definition (`tvm/llama_auto_batcher/lora.py:10-24`) on this package's operators: the
+    four protocol methods its compiler checks for (`compile_tvm.py:29-93`) with the same names, argument order and
+    meaning.  Parameters come in the reference's orientation, `lora_A [in_features, r]` and `lora_B [r, out_features]`
+    (the transposes of PEFT's `lora_A.weight` / `lora_B.weight`).  For ONE adapter
+    `post_computation(weight_application(x, lora_A, lora_B))` is the delta that the model adds to the base linear's
+    output; the serving path computes the same per token from the stacked tables of all adapters
+    (`ops.gather_mm`, see `stack`)."""
+
+    def __init__(self, in_features: int, out_features: int, config: LoraConfig):
+        self.in_features, self.out_features, self.config = in_features, out_features, config
+        self.scaling = config.alpha / config.r
+
+    def define_parameters(self, in_features: int, out_features: int, config: LoraConfig) -> tuple:
+        """Shapes and dtype of the adapter's parameters, in the order `weight_application` takes them."""
+        return ((in_features, config.r), "float16"), ((config.r, out_features), "float16")
+
+    def weight_application(self, x: torch.Tensor, lora_A: torch.Tensor, lora_B: torch.Tensor) -> torch.Tensor:
+        """(x . lora_A) . lora_B on the base-linear kernels: x [T, in] fp16 -> [T, out] fp16 (fp32 accumulation)."""
+        r = lora_A.shape[1]
+        rp = -(-r // 32) * 32                 # the base-linear kernels take K in multiples of 32: exact zeros up to there
+        At = torch.zeros((rp, lora_A.shape[0]), dtype=torch.float16, device=x.device)
+        At[:r] = lora_A.t()
+        Bt = torch.zeros((lora_B.shape[1], rp), dtype=torch.float16, device=x.device)
+        Bt[:, :r] = lora_B.t()
+        return ops.linear(ops.linear(x, At), Bt)
+
+    def post_computation(self, y: torch.Tensor) -> torch.Tensor:
+        return y * self.scaling
+
+    @staticmethod
+    def stack(params):
+        """[(lora_A [in, r], lora_B [r, out]), ...] of equal rank -> the stacked tables of the gather-matmul,
+        A [n_ad, r, in] and B [n_ad, out, r]."""
+        A = torch.stack([a.t() for a, _ in params]).contiguous()
+        B = torch.stack([b.t() for _, b in params]).contiguous()
+        return A, B
 
 
 class GatherMMLinear:

@@ -66,6 +66,36 @@ def test_gather_mm_no_adapter_rows_untouched_and_index_exact(ops, synth):
     assert np.array_equal(_np(y)[ids < 0], ys[ids < 0])
 
 
+def test_lora_adapter_definition_equals_the_gathered_delta(ops, synth):
+    """The reference's adapter class (`define_parameters`, `weight_application`, `post_computation`,
+    `tvm/llama_auto_batcher/lora.py:10-24`) applied adapter by adapter equals the delta that the gather-matmul adds
+    for the rows of that adapter."""
+    lora = load_pkg("lora")
+    T, K, N, r, n_ad = 48, 1024, 768, 16, 5
+    cfg = lora.LoraConfig(r, 8.0)
+    ad = lora.Lora(K, N, cfg)
+    (sa, da), (sb, db) = ad.define_parameters(K, N, cfg)
+    assert sa == (K, r) and sb == (r, N) and da == db == "float16" and ad.scaling == 0.5
+    params = [(synth.normal(17, f"lad.A{i}", sa, 0.05, torch.float16, DEV), synth.normal(17, f"lad.B{i}", sb, 0.05, torch.float16, DEV))
+              for i in range(n_ad)]
+    x = synth.normal(17, "lad.x", (T, K), 1.0, torch.float16, DEV)
+    ids = synth.randint(17, "lad.ids", (T,), n_ad + 1, DEV).to(torch.int32) - 1          # -1: no adapter
+    A, B = lora.Lora.stack(params)
+    y = torch.zeros((T, N), dtype=torch.float32, device=DEV)
+    ops.gather_mm(y, x, A, B, ids, ad.scaling)
+    torch.cuda.synchronize()
+    for i in range(n_ad):
+        rows = (ids == i).nonzero().flatten()
+        if len(rows) == 0:
+            continue
+        want = ad.post_computation(ad.weight_application(x[rows].contiguous(), *params[i]).float())
+        ref = (_np(x[rows]).astype(np.float64) @ _np(params[i][0]).astype(np.float64) @ _np(params[i][1]).astype(np.float64)) * ad.scaling
+        assert max_rel_err(_np(y[rows]), ref) <= TOL
+        # the two-linear form stores x . A and the result in fp16: held to the fp16 step of the largest entries
+        assert float(np.abs(_np(want) - ref).max() / np.abs(ref).max()) <= TOL
+    assert not y[ids < 0].any()
+
+
 def test_gather_mm_into_column_slice(ops, synth):
     """y may be a column slice of a fused projection output (row stride > N); other columns stay untouched."""
     T, K, N, r, n_ad = 32, 1024, 256, 16, 4
