@@ -227,6 +227,38 @@ int mlora_linear_frag(void* y, int y_dtype, int mode, const void* xf, const void
                       int T, int K, int N, void* stream);
 int mlora_gemm_frag_preferred(int T, int K, int N);
 
+/* The prefill linear that carries its LoRA deltas as extra k-steps of the base GEMM, for token blocks that agree on
+ * one adapter: y (=|+=) [xf | v_hi | v_lo] . [Wp | B[a] | B[a]]^T per 256-token block whose tokens all name adapter a,
+ * with v = scaling * x . A[a]^T split into fp16 hi + lo halves - no second pass over y.
+ *   mlora_lora_block_adapters - blk_adapter[b] = the adapter all valid tokens of block b (256 tokens) name, or -1
+ *                               (no adapter, or several); tok_rest[t] = -1 where the block's delta rides in the GEMM,
+ *                               else tok_adapter[t]: the ids a separate mlora_gather_mm still has to serve;
+ *   mlora_lora_shrink_split   - the matrix-core shrink of n_proj <= 3 projections that read the same x, then
+ *                               v_hi[p], v_lo[p] [T][r] fp16 (r in {32, 64}); workspace: n_proj *
+ *                               mlora_gather_mm_workspace_bytes(T, K, r) bytes; rows of tokens without adapter hold
+ *                               nothing meaningful and are not read by mlora_linear_frag_lora;
+ *   mlora_linear_frag_lora    - mlora_linear_frag on a shape that mlora_gemm_frag_preferred accepts, with up to three
+ *                               projections = row ranges [n_begin, n_begin + n_rows) of the fused weight (on 256-row
+ *                               boundaries), each with its B table [n_ad][n_rows][r] and its v halves.
+ * Against mlora_linear_frag followed by mlora_gather_mm the result differs in where it is rounded (once, after the
+ * sum, instead of after the base product and again after the delta) and in the fp32 summation order.
+ * Replaces: the base linear plus q_ft_proj / v_ft_proj style deltas of the prefill entry points
+ * (tvm/llama_auto_batcher/compile_tvm.py:116-160). */
+typedef struct mlora_fused_lora {
+  const void* B;      /* [n_ad][n_rows][r] fp16, row-major */
+  const void* v_hi;   /* [T][r] fp16 */
+  const void* v_lo;
+  int n_begin;
+  int n_rows;
+} mlora_fused_lora;
+int mlora_lora_block_adapters(int32_t* blk_adapter, int32_t* tok_rest, const int32_t* tok_adapter, int T, int n_ad,
+                              void* stream);
+int mlora_lora_shrink_split(void* const* v_hi, void* const* v_lo, const void* x, int x_layout, const void* const* A, int n_proj,
+                            const int32_t* tok_adapter, float scaling, int T, int K, int r, int n_ad,
+                            void* workspace, size_t workspace_bytes, void* stream);
+int mlora_linear_frag_lora(void* y, int y_dtype, int mode, const void* xf, const void* Wp, int T, int K, int N,
+                           const mlora_fused_lora* projs, int n_proj, const int32_t* blk_adapter, int r, void* stream);
+
 /* y[t, :] = f16( x[t, :] * rsqrt(mean(x[t, :]^2) + eps) * w )   row-wise, statistics in fp32.
  * Replaces: nn.RMSNorm(hidden, -1, eps, bias=False) (llama_for_causal_lm.py:76-77,93).
  * x [T, H] f16 or f32 (x_dtype), w [H] f16, y [T, H] f16 in y_layout.  H % 8 == 0, H <= 16384. */

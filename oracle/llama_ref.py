@@ -192,10 +192,32 @@ class LlamaRef:
         return y
 
     def _proj(self, x, l, proj, tok_adapter):
-        """Projection whose output is stored (fp16 in mixed mode): base rounded, then delta added and rounded."""
-        y = self.rnd(x @ self.w[f"layers.{l}.{proj}"].T)
+        """Projection whose output is stored (fp16 in mixed mode): base rounded, then delta added and rounded.
+        With `fuse_blocks` = n set (the HIP prefill carries the delta inside the base GEMM for every n-token block whose
+        tokens all name one adapter of the pass's single adapter type): base + delta rounded ONCE for those tokens."""
+        base = x @ self.w[f"layers.{l}.{proj}"].T
+        y = self.rnd(base)
         y2 = self._delta_into(y, x, l, proj, tok_adapter)
-        return y if y2 is y else self.rnd(y2)
+        if y2 is y:
+            return y
+        out = self.rnd(y2)
+        once = self._rounded_once(tok_adapter, x.shape[0])
+        if once is not None and once.any():
+            delta = self._delta_into(np.zeros_like(base), x, l, proj, tok_adapter)
+            out = np.array(out)
+            out[once] = self.rnd(base[once] + delta[once])
+        return out
+
+    def _rounded_once(self, tok_adapter, T):
+        n = getattr(self, "fuse_blocks", None)
+        if not n or self.mode != "mixed" or not tok_adapter or len(tok_adapter) != 1:
+            return None
+        ids = np.asarray(next(iter(tok_adapter.values())))
+        once = np.zeros(T, dtype=bool)
+        for t0 in range(0, T, n):
+            blk = ids[t0:t0 + n]
+            once[t0:t0 + n] = blk[0] >= 0 and bool((blk == blk[0]).all())
+        return once
 
     def _proj_residual(self, resid, x, l, proj, tok_adapter):
         """Projection accumulated into the fp32 residual stream: resid + base, then + delta."""

@@ -44,6 +44,9 @@ SIGNATURES = {
     "mlora_gemv_frag": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p]),
     "mlora_linear_frag": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p]),
     "mlora_gemm_frag_preferred": (_i, [_i, _i, _i]),
+    "mlora_lora_block_adapters": (_i, [_p, _p, _p, _i, _i, _p]),
+    "mlora_lora_shrink_split": (_i, [_p, _p, _p, _i, _p, _i, _p, _f, _i, _i, _i, _i, _p, _z, _p]),
+    "mlora_linear_frag_lora": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p, _i, _p, _i, _p]),
     "mlora_gemv_frag_lora": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _i, _p, _i, _i, _p]),
     "mlora_gemv_frag_silu": (_i, [_p, _p, _p, _i, _i, _i, _p]),
     "mlora_gemv_frag_split": (_i, [_p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _p]),
@@ -69,6 +72,10 @@ SIGNATURES = {
 
 class LoraBucket(C.Structure):
     _fields_ = [("A", _p), ("B", _p), ("r", _i), ("n_ad", _i), ("scaling", _f)]
+
+
+class FusedLora(C.Structure):
+    _fields_ = [("B", _p), ("v_hi", _p), ("v_lo", _p), ("n_begin", _i), ("n_rows", _i)]
 
 
 class LoraProj(C.Structure):

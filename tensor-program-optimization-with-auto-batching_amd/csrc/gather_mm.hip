@@ -1182,12 +1182,12 @@ extern "C" int mlora_gather_mm_batch(const void* const* sets, int n_sets, int y_
                         (hipStream_t)stream);
 }
 
+// Shrink of pj.n projections on the matrix cores into v [pj.n][splits][T][R] fp32; returns the number of K ranges
+// (`splits`) whose partial sums a reader adds in range order.
 template <int R>
-static void gmm_segments_r(const SegProjs& pj, int y_dtype, int ldy, const f16* x, int frag_tt, const int32_t* ids, float scaling, int T, int K,
-                           int n_ad, float* v, BucketFilter bf, hipStream_t s) {
+static int gmm_segments_shrink_r(const SegProjs& pj, const f16* x, int frag_tt, const int32_t* ids, int T, int K, int n_ad, float* v,
+                                 BucketFilter bf, hipStream_t s) {
   const int tiles = ceil_div(T, 16);
-  int N = 0;
-  for (int i = 0; i < pj.n; ++i) N = pj.N[i] > N ? pj.N[i] : N;
   // few token tiles: split K over workgroups so that the shrink still covers the chip (partials fit the workspace,
   // which holds lora_k_split(K).kc slices of [T, r] per projection); the same split whatever the number of
   // projections, so that a projection's sums do not depend on what shares its launch
@@ -1199,8 +1199,7 @@ static void gmm_segments_r(const SegProjs& pj, int y_dtype, int ldy, const f16* 
   // Up to 1024 tokens the call is taken to be a decode batch (one token per sequence, tiles that mix many adapters);
   // beyond that a prefill whose tokens come in adapter segments: four token tiles per shrink workgroup, two per expand
   // workgroup, about two workgroups per compute unit.  Either set of kernels is correct for either input.
-  const bool mixed = T <= 1024;
-  if (mixed) {
+  if (T <= 1024) {
     hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles, splits, pj.n), dim3(SEG_WAVES * WAVE), 0, s, v, x, frag_tt, pj, ids, T, K,
                        n_ad, bf.bucket_of, bf.bucket);
   } else {
@@ -1212,6 +1211,17 @@ static void gmm_segments_r(const SegProjs& pj, int y_dtype, int ldy, const f16* 
     hipLaunchKernelGGL((lora_shrink_quad_mfma_kernel<R>), dim3(quads, splits, pj.n), dim3(SEG_WAVES * WAVE), 0, s, v, x, frag_tt, pj, ids, T,
                        K, n_ad, bf.bucket_of, bf.bucket);
   }
+  return splits;
+}
+
+template <int R>
+static void gmm_segments_r(const SegProjs& pj, int y_dtype, int ldy, const f16* x, int frag_tt, const int32_t* ids, float scaling, int T, int K,
+                           int n_ad, float* v, BucketFilter bf, hipStream_t s) {
+  const int tiles = ceil_div(T, 16);
+  int N = 0;
+  for (int i = 0; i < pj.n; ++i) N = pj.N[i] > N ? pj.N[i] : N;
+  const bool mixed = T <= 1024;
+  const int splits = gmm_segments_shrink_r<R>(pj, x, frag_tt, ids, T, K, n_ad, v, bf, s);
   // column blocks per workgroup: as many as leave about a thousand workgroups (per-workgroup set-up amortised)
   int nit = (int)(((long)tiles * pj.n * ceil_div(N, SEG_WAVES * 64)) / 1024);
   nit = nit < 1 ? 1 : (nit > 8 ? 8 : nit);
@@ -1232,6 +1242,54 @@ static void gmm_segments_r(const SegProjs& pj, int y_dtype, int ldy, const f16* 
     else MLORA_EXPAND_MFMA(lora_expand_pair_mfma_kernel, float);
   }
 #undef MLORA_EXPAND_MFMA
+}
+
+// ---------------------------------------------------------------------------------------------
+// Pieces of the prefill linear that carries its LoRA delta as extra k-steps of the base GEMM (gemm.hip): the adapter a
+// 256-token block agrees on, and the shrink results as fp16 hi + lo halves.
+// ---------------------------------------------------------------------------------------------
+constexpr int FUSE_BLOCK = 256;            // token block of the persistent GEMM
+
+// blk[b] = the adapter every valid token of block b names (-1: tokens without adapter or of several adapters);
+// rest[t] = -1 where the block's delta rides in the GEMM, else ids[t] (what a separate gather-matmul still has to do)
+__global__ __launch_bounds__(FUSE_BLOCK) void lora_block_adapters_kernel(int32_t* __restrict__ blk, int32_t* __restrict__ rest,
+                                                                       const int32_t* __restrict__ ids, int T, int n_ad) {
+  __shared__ int s_first, s_bad;
+  const int t = blockIdx.x * FUSE_BLOCK + threadIdx.x;
+  if (threadIdx.x == 0) {
+    const int raw = ids[blockIdx.x * FUSE_BLOCK];        // the block's first token exists
+    s_first = (raw >= 0 && raw < n_ad) ? raw : -1;
+    s_bad = 0;
+  }
+  __syncthreads();
+  const int raw = t < T ? ids[t] : s_first;
+  const int id = (raw >= 0 && raw < n_ad) ? raw : -1;
+  if (id != s_first) s_bad = 1;                            // benign race: every writer stores 1
+  __syncthreads();
+  const int a = (s_bad || s_first < 0) ? -1 : s_first;
+  if (threadIdx.x == 0) blk[blockIdx.x] = a;
+  if (t < T) rest[t] = a >= 0 ? -1 : id;
+}
+
+// vh, vl [T][R] fp16: hi and lo halves of scaling * (sum of the K-range partials of the shrink, in range order) - the
+// values and the split the expand kernels use
+template <int R>
+__global__ __launch_bounds__(256) void lora_v_split_kernel(f16* __restrict__ vh, f16* __restrict__ vl, const float* __restrict__ v,
+                                                           int splits, float scaling, int T) {
+  const int e = blockIdx.x * 256 + threadIdx.x;              // four rank entries of one token
+  const int t = e / (R / 4), j = (e % (R / 4)) * 4;
+  if (t >= T) return;
+  f32x4 sum = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int sp = 0; sp < splits; ++sp) sum += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + t) * R + j);
+  f16x4 h, l;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float f = sum[q] * scaling;
+    h[q] = (f16)f;
+    l[q] = (f16)(f - (float)h[q]);
+  }
+  *reinterpret_cast<f16x4*>(vh + (size_t)t * R + j) = h;
+  *reinterpret_cast<f16x4*>(vl + (size_t)t * R + j) = l;
 }
 
 // shrink + expand on the matrix cores for pj.n projections; v = workspace viewed as [pj.n][splits][T, r] fp32
@@ -1477,6 +1535,48 @@ extern "C" int mlora_gather_mm_multi_proj(void* y, int y_dtype, int ldy, const v
         return e;
     }
   return MLORA_OK;
+}
+
+extern "C" int mlora_lora_block_adapters(int32_t* blk_adapter, int32_t* tok_rest, const int32_t* tok_adapter, int T, int n_ad,
+                                         void* stream) {
+  MLORA_CHECK(blk_adapter && tok_rest && tok_adapter, MLORA_ERR_INVALID, "lora_block_adapters: null pointer");
+  MLORA_CHECK(T >= 0 && n_ad > 0, MLORA_ERR_INVALID, "lora_block_adapters: bad T=%d n_ad=%d", T, n_ad);
+  if (T == 0) return MLORA_OK;
+  hipLaunchKernelGGL(lora_block_adapters_kernel, dim3(ceil_div(T, FUSE_BLOCK)), dim3(FUSE_BLOCK), 0, (hipStream_t)stream, blk_adapter, tok_rest,
+                     tok_adapter, T, n_ad);
+  return mlora_launch_status("lora_block_adapters");
+}
+
+extern "C" int mlora_lora_shrink_split(void* const* v_hi, void* const* v_lo, const void* x, int x_layout, const void* const* A, int n_proj,
+                                       const int32_t* tok_adapter, float scaling, int T, int K, int r, int n_ad, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
+  MLORA_CHECK(v_hi && v_lo && x && A && tok_adapter && n_proj >= 1 && n_proj <= SEG_MAX_PROJ, MLORA_ERR_INVALID,
+              "lora_shrink_split: null pointer or n_proj outside 1..%d", SEG_MAX_PROJ);
+  MLORA_CHECK((r == 32 || r == 64) && n_ad > 0 && n_ad <= 65535, MLORA_ERR_UNSUPPORTED, "lora_shrink_split: rank %d not in {32, 64} or bad n_ad %d", r, n_ad);
+  MLORA_CHECK(T > 64 && K > 0 && K % 32 == 0 && (x_layout == MLORA_ROWMAJOR || x_layout == MLORA_FRAG), MLORA_ERR_UNSUPPORTED,
+              "lora_shrink_split: needs T > 64, K %% 32 == 0 (T=%d K=%d layout=%d)", T, K, x_layout);
+  MLORA_CHECK(workspace && workspace_bytes >= (size_t)n_proj * mlora_gather_mm_workspace_bytes(T, K, r), MLORA_ERR_WORKSPACE,
+              "lora_shrink_split: workspace of %zu bytes given, %zu needed", workspace_bytes, (size_t)n_proj * mlora_gather_mm_workspace_bytes(T, K, r));
+  SegProjs pj = {};
+  for (int i = 0; i < n_proj; ++i) {
+    MLORA_CHECK(A[i] && v_hi[i] && v_lo[i], MLORA_ERR_INVALID, "lora_shrink_split: null table or output of projection %d", i);
+    pj.A[i] = (const f16*)A[i];
+  }
+  pj.n = n_proj;
+  hipStream_t s = (hipStream_t)stream;
+  const int frag_tt = x_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
+  float* v = (float*)workspace;
+  const BucketFilter bf{nullptr, 0};
+  int splits;
+  if (r == 32) splits = gmm_segments_shrink_r<32>(pj, (const f16*)x, frag_tt, tok_adapter, T, K, n_ad, v, bf, s);
+  else splits = gmm_segments_shrink_r<64>(pj, (const f16*)x, frag_tt, tok_adapter, T, K, n_ad, v, bf, s);
+  for (int i = 0; i < n_proj; ++i) {
+    const float* vi = v + (size_t)i * splits * T * r;
+    const dim3 grid(ceil_div(T * (r / 4), 256));
+    if (r == 32) hipLaunchKernelGGL((lora_v_split_kernel<32>), grid, dim3(256), 0, s, (f16*)v_hi[i], (f16*)v_lo[i], vi, splits, scaling, T);
+    else hipLaunchKernelGGL((lora_v_split_kernel<64>), grid, dim3(256), 0, s, (f16*)v_hi[i], (f16*)v_lo[i], vi, splits, scaling, T);
+  }
+  return mlora_launch_status("lora_shrink_split");
 }
 
 extern "C" int mlora_write_tensor_part(void* Z, const void* X, const void* Y, const int32_t* ids, int B, int A, int PH,

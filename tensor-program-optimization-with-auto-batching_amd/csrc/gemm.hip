@@ -279,9 +279,29 @@ constexpr int PP_STAGE_ELEMS = 2 * PP_F * 512; // fp16 elements of one 32-k stag
 constexpr int PP_OUT_LD = 64 + 4;              // fp16 elements per token row of a wave's output staging (padded: conflict-free writes)
 constexpr int PP_OUT_ELEMS = 16 * PP_OUT_LD;   // per wave: 16 tokens x 64 columns
 
-template <int OUT>
+// LoRA deltas that ride in the GEMM as extra k-steps: y = [x | v_hi | v_lo] . [W | B[a] | B[a]]^T for a 256-token block
+// whose tokens all name adapter a (blk_adapter[block] >= 0), v = scaling * x . A[a]^T as fp16 hi + lo halves [T][r].
+// Projections are row ranges of the fused weight, each with its own B table [n_ad][rows][r] (row-major, r in {32, 64})
+// and its own v; a 256-row block lies inside one range (checked by the launcher).  n_proj == 0: a plain GEMM.
+struct PPLora {
+  const f16* B[3];
+  const f16* vh[3];
+  const f16* vl[3];
+  int n_begin[3], n_rows[3];
+  int n_proj, r;
+  const int32_t* blk_adapter;
+};
+
+__device__ __forceinline__ unsigned long long uniform64(unsigned long long v) {
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+  return ((unsigned long long)hi << 32) | lo;
+}
+
+// LORA = false is the plain GEMM (lo is ignored)
+template <int OUT, bool LORA>
 __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx, int x_tt,
-                                                                   const f16* __restrict__ Wp, int T, int K, int N, int gx, int gy) {
+                                                                   const f16* __restrict__ Wp, int T, int K, int N, int gx, int gy,
+                                                                   PPLora lo) {
   extern __shared__ __align__(16) f16 smem[];  // [PP_STAGES][PP_STAGE_ELEMS], then [PP_WAVES][PP_OUT_ELEMS]
   constexpr int NW = PP_WAVES;
   constexpr int LQ = 2 * PP_F / NW;            // fragments a wave fetches per stage (4)
@@ -299,14 +319,58 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
     n0 = (idx / gy) * (PP_F * 16);
     t0 = (idx % gy) * (PP_F * 16);
   };
+  // the LoRA part of a block: projection slot and adapter (-1: none), everything uniform
+  auto lora_of = [&](int n0, int t0, int& slot) -> int {
+    slot = -1;
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+      if (i < lo.n_proj && n0 >= lo.n_begin[i] && n0 < lo.n_begin[i] + lo.n_rows[i]) slot = i;
+    if (slot < 0) return -1;
+    return lo.blk_adapter[t0 / (PP_F * 16)];
+  };
+  const int E = LORA ? 2 * (lo.r / 32) : 0;     // extra k-steps of a block with a delta: hi halves, then lo halves
 
   // ---- loader role: wave w fetches fragments 4 w .. 4 w + 3 of every stage (waves 0-3: weights, waves 4-7: tokens)
   const f16* src[LQ];
   int step = 0;                                // elements between consecutive k-steps of this wave's sources
   int load_L = blockIdx.x, load_kb = 0;        // the stage the loader issues next
+  int load_nst = KB;                           // stages of the block being loaded (KB, or KB + E with a delta)
+  const f16* l_src = nullptr;                  // LoRA stages of that block (all uniform): row 0 of the block in B[a] (weight waves) or in v_hi (token waves) ...
+  long l_lo = 0;                               // ... the distance from v_hi to v_lo (token waves; 0 for weight waves) ...
+  int l_rows = 1;                              // ... and the rows that exist from there on (rows past them repeat the last one; their results are dropped)
   auto load_block = [&](int L) {
     int n0, t0;
     block_of(L < nb ? L : blockIdx.x, n0, t0); // past the last block: valid addresses, the data is never multiplied
+    load_nst = KB;
+    if constexpr (LORA) {
+      int slot;
+      const int a = L < nb ? lora_of(n0, t0, slot) : -1;
+      if (a >= 0) {
+        load_nst = __builtin_amdgcn_readfirstlane(KB + E);
+        const f16* Bt = lo.B[0];
+        const f16* vh = lo.vh[0];
+        const f16* vl = lo.vl[0];
+        int nbeg = lo.n_begin[0], nrows = lo.n_rows[0];
+#pragma unroll
+        for (int i = 1; i < 3; ++i)
+          if (i == slot) {                     // uniform select: the struct is never indexed dynamically
+            Bt = lo.B[i]; vh = lo.vh[i]; vl = lo.vl[i]; nbeg = lo.n_begin[i]; nrows = lo.n_rows[i];
+          }
+        if (wave < NW / 2) {
+          l_src = Bt + ((size_t)a * nrows + (n0 - nbeg)) * lo.r;
+          l_lo = 0;
+          l_rows = nrows - (n0 - nbeg);
+        } else {
+          l_src = vh + (size_t)t0 * lo.r;
+          l_lo = vl - vh;
+          l_rows = T - t0;
+        }
+        // all of this is the same in every lane: say so, it lives in scalar registers across the K loop
+        l_src = (const f16*)uniform64((unsigned long long)l_src);
+        l_lo = (long)uniform64((unsigned long long)l_lo);
+        l_rows = __builtin_amdgcn_readfirstlane(l_rows);
+      }
+    }
     if (wave < NW / 2) {
 #pragma unroll
       for (int q = 0; q < LQ; ++q) {
@@ -334,17 +398,35 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
     }
   };
   int ring = 0;                                // ring slot of the stage issued next
-  auto issue = [&]() {
+  // PLAIN: the caller knows that this stage is an ordinary k-step and not the last of its block (no tests at all)
+  auto issue = [&](auto PLAIN) {
+    constexpr bool plain = decltype(PLAIN)::value;
     f16* dst = smem + ring * PP_STAGE_ELEMS + wave * LQ * 512;
+    if (plain || !LORA || load_kb < KB) {
 #pragma unroll
-    for (int q = 0; q < LQ; ++q)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + (size_t)load_kb * step),
-                                       (__attribute__((address_space(3))) void*)(dst + q * 512), 16, 0, 0);
+      for (int q = 0; q < LQ; ++q)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + (size_t)load_kb * step),
+                                         (__attribute__((address_space(3))) void*)(dst + q * 512), 16, 0, 0);
+    } else {                                   // a LoRA stage: 16 rows x 64 bytes per fragment, gathered by the lanes' addresses
+      const int j = load_kb - KB, RB = lo.r / 32;
+      const int ks = (j < RB ? j : j - RB) * 32;
+#pragma unroll
+      for (int q = 0; q < LQ; ++q) {
+        int row = ((wave & 3) * LQ + q) * 16 + (lane & 15);
+        row = row < l_rows ? row : l_rows - 1;
+        const f16* p = l_src + (j < RB ? 0 : l_lo) + ((size_t)row * lo.r + ks + (lane >> 4) * 8);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p,
+                                         (__attribute__((address_space(3))) void*)(dst + q * 512), 16, 0, 0);
+      }
+    }
     ring = (ring + 1) & (PP_STAGES - 1);
-    if (++load_kb == KB) {                     // uniform
-      load_kb = 0;
-      load_L += G;
-      load_block(load_L);
+    ++load_kb;
+    if constexpr (!plain) {
+      if (load_kb == load_nst) {               // uniform
+        load_kb = 0;
+        load_L += G;
+        load_block(load_L);
+      }
     }
   };
 
@@ -373,11 +455,11 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
   // everybody's: the barrier).  The wait also covers this wave's fragment reads of the stage about to be multiplied,
   // so after the barrier nobody reads that ring slot any more and it is refilled; then the reads of the successor go
   // out, then the MFMAs.
-  auto stage = [&](auto U) {
+  auto stage = [&](auto U, auto PLAIN) {
     constexpr int u = decltype(U)::value;
     asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
     __syncthreads();
-    issue();
+    issue(PLAIN);
     read_frags(std::integral_constant<int, 1 - u>());
     __builtin_amdgcn_sched_barrier(0);
     multiply(U);
@@ -385,12 +467,12 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
   };
 
   load_block(load_L);
-  issue();
-  issue();
-  issue();
+  issue(std::false_type());
+  issue(std::false_type());
+  issue(std::false_type());
   asm volatile("s_waitcnt vmcnt(8)" ::: "memory");     // the first stage of this wave has landed
   __syncthreads();
-  issue();
+  issue(std::false_type());
   read_frags(std::integral_constant<int, 0>());
   f16* ostage = smem + PP_STAGES * PP_STAGE_ELEMS + wave * PP_OUT_ELEMS;
   const int r16 = lane & 15, g = lane >> 4;
@@ -399,12 +481,24 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
     for (int i = 0; i < 8; ++i)
 #pragma unroll
       for (int j = 0; j < WTF; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int kb = 0; kb < KB; kb += 2) {               // KB is even (checked by the launcher): the register sets alternate
-      stage(std::integral_constant<int, 0>());
-      stage(std::integral_constant<int, 1>());
-    }
     int n0, t0;
     block_of(L, n0, t0);
+    int nst = KB;                                      // KB and E are even (checked by the launcher): the register sets alternate
+    if constexpr (LORA) {
+      int slot;
+      if (lora_of(n0, t0, slot) >= 0) nst += E;
+      nst = __builtin_amdgcn_readfirstlane(nst);
+    }
+    for (int kb = 0; kb < nst; kb += 2) {
+      // (the plain GEMM keeps one copy of the pair: with two, the compiler's register allocation of this loop falls apart)
+      if (LORA && load_kb + 2 < KB) {                    // uniform: the two stages fetched next are ordinary k-steps inside their block
+        stage(std::integral_constant<int, 0>(), std::true_type());
+        stage(std::integral_constant<int, 1>(), std::true_type());
+      } else {
+        stage(std::integral_constant<int, 0>(), std::false_type());
+        stage(std::integral_constant<int, 1>(), std::false_type());
+      }
+    }
     if constexpr (OUT == OUT_F16) {
       // 16 tokens x 64 columns at a time through the wave's staging buffer: D[n][t] fragments in, token rows out
 #pragma unroll
@@ -462,11 +556,13 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
 }
 
 template <int OUT>
-int launch_gemm_pp(void* y, const f16* x, int ldx, int x_tt, const f16* Wp, int T, int K, int N, hipStream_t s) {
+int launch_gemm_pp(void* y, const f16* x, int ldx, int x_tt, const f16* Wp, int T, int K, int N, hipStream_t s,
+                   const PPLora& lo = PPLora()) {
   constexpr size_t lds = ((size_t)PP_STAGES * PP_STAGE_ELEMS + (size_t)PP_WAVES * PP_OUT_ELEMS) * sizeof(f16);
   static bool configured = false;                    // the attribute is per kernel, set once per process
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_pp_kernel<OUT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_pp_kernel<OUT, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)gemm_pp_kernel<OUT, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return mlora_set_error(MLORA_ERR_LAUNCH, "gemm_packed: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     configured = true;
   }
@@ -474,7 +570,8 @@ int launch_gemm_pp(void* y, const f16* x, int ldx, int x_tt, const f16* Wp, int 
   int n_cu = gemm_n_cu();
   if (n_cu <= 0) n_cu = 256;
   const int grid = gx * gy < n_cu ? gx * gy : n_cu;
-  hipLaunchKernelGGL((gemm_pp_kernel<OUT>), dim3(grid), dim3(PP_WAVES * WAVE), lds, s, y, x, ldx, x_tt, Wp, T, K, N, gx, gy);
+  if (lo.n_proj > 0) hipLaunchKernelGGL((gemm_pp_kernel<OUT, true>), dim3(grid), dim3(PP_WAVES * WAVE), lds, s, y, x, ldx, x_tt, Wp, T, K, N, gx, gy, lo);
+  else hipLaunchKernelGGL((gemm_pp_kernel<OUT, false>), dim3(grid), dim3(PP_WAVES * WAVE), lds, s, y, x, ldx, x_tt, Wp, T, K, N, gx, gy, lo);
   return MLORA_OK;
 }
 
@@ -828,6 +925,36 @@ extern "C" int mlora_linear_frag(void* y, int y_dtype, int mode, const void* xf,
     else e = launch_gemm_mid<OUT_F16>(y, nullptr, 0, 1, ft, x, tt, W, T, K, N, s);
   }
   return e ? e : mlora_launch_status("linear_frag");
+}
+
+extern "C" int mlora_linear_frag_lora(void* y, int y_dtype, int mode, const void* xf, const void* Wp, int T, int K, int N,
+                                      const mlora_fused_lora* projs, int n_proj, const int32_t* blk_adapter, int r, void* stream) {
+  if (int e = mlora_check_linear("linear_frag_lora", y, y_dtype, mode, xf, K, Wp, T, K, N)) return e;
+  MLORA_CHECK(mlora_gemm_frag_preferred(T, K, N) && ((uintptr_t)xf & 15) == 0, MLORA_ERR_UNSUPPORTED,
+              "linear_frag_lora: only shapes of the persistent GEMM (mlora_gemm_frag_preferred; T=%d K=%d N=%d)", T, K, N);
+  MLORA_CHECK(projs && blk_adapter && n_proj >= 1 && n_proj <= 3 && (r == 32 || r == 64), MLORA_ERR_UNSUPPORTED,
+              "linear_frag_lora: 1..3 projections of rank 32 or 64 (n_proj=%d r=%d)", n_proj, r);
+  PPLora lo = {};
+  for (int i = 0; i < n_proj; ++i) {
+    const mlora_fused_lora& p = projs[i];
+    MLORA_CHECK(p.B && p.v_hi && p.v_lo && (((uintptr_t)p.B | (uintptr_t)p.v_hi | (uintptr_t)p.v_lo) & 15) == 0, MLORA_ERR_INVALID,
+                "linear_frag_lora: null or unaligned table of projection %d", i);
+    // a 256-row block of the GEMM must lie inside one projection
+    MLORA_CHECK(p.n_begin >= 0 && p.n_rows > 0 && p.n_begin % (PP_F * 16) == 0 && p.n_begin + p.n_rows <= N &&
+                    (p.n_rows % (PP_F * 16) == 0 || p.n_begin + p.n_rows == N),
+                MLORA_ERR_UNSUPPORTED, "linear_frag_lora: rows %d..%d of projection %d do not fall on 256-row blocks", p.n_begin,
+                p.n_begin + p.n_rows, i);
+    lo.B[i] = (const f16*)p.B; lo.vh[i] = (const f16*)p.v_hi; lo.vl[i] = (const f16*)p.v_lo;
+    lo.n_begin[i] = p.n_begin; lo.n_rows[i] = p.n_rows;
+  }
+  lo.n_proj = n_proj; lo.r = r; lo.blk_adapter = blk_adapter;
+  hipStream_t s = (hipStream_t)stream;
+  const int tt = mlora_frag_tiles(T);
+  int e;
+  if (mode == MLORA_ACCUMULATE) e = launch_gemm_pp<OUT_ACC_F32>(y, (const f16*)xf, 0, tt, (const f16*)Wp, T, K, N, s, lo);
+  else if (y_dtype == MLORA_F32) e = launch_gemm_pp<OUT_F32>(y, (const f16*)xf, 0, tt, (const f16*)Wp, T, K, N, s, lo);
+  else e = launch_gemm_pp<OUT_F16>(y, (const f16*)xf, 0, tt, (const f16*)Wp, T, K, N, s, lo);
+  return e ? e : mlora_launch_status("linear_frag_lora");
 }
 
 // K slices the mid-size kernel would use for resid [T, N] += xf . Wp^T with at most ks_max slices (T > 64)

@@ -318,29 +318,49 @@ class LlamaForCausalLM:
         # a decode step splits K of the two narrow accumulating GEMVs; the RMSNorm that reads the residual next adds
         # the partial results (the same kernels and slice counts as the native decode step)
         ks_ws = self._ksplit_ws(T) if dec_frag or (frag and T <= 256) else None
+        # a prefill-sized pass of one adapter type of rank 32 or 64: where a 256-token block agrees on one adapter its
+        # deltas ride in the base GEMM as extra k-steps; `rest` names the tokens that still need the separate call
+        fuse = None
+        if tok_adapter and "multi" not in tok_adapter and frag and T > 64 and ops.gemm_frag_preferred(T, H, H):
+            (tid, ids), = tok_adapter.items()
+            lt = self.lora_types[tid]
+            if lt.r in (32, 64):
+                blk, rest = ops.lora_block_adapters(ids, lt.n_adapters)
+                fuse = (lt, ids, blk, {tid: rest} if bool((rest >= 0).any()) else None)     # one read-back per pass
         parts = None
         for l, L in enumerate(self.layers):
             xn = ops.rmsnorm(resid, L["ln1"], s.rms_norm_eps, frag=frag, parts=parts)
-            qkv = ops.linear(xn, L["qkv"])
-            if tok_adapter:
-                self._lora_group(qkv, xn, l, (("q_proj", 0, q_sz), ("k_proj", q_sz, kv_sz), ("v_proj", q_sz + kv_sz, kv_sz)),
-                                 tok_adapter)
+            qkv_projs = (("q_proj", 0, q_sz), ("k_proj", q_sz, kv_sz), ("v_proj", q_sz + kv_sz, kv_sz))
+            qkv = self._fused_linear(fuse, xn, L["qkv"], l, qkv_projs) if fuse else None
+            if qkv is None:
+                qkv = ops.linear(xn, L["qkv"])
+                if tok_adapter:
+                    self._lora_group(qkv, xn, l, qkv_projs, tok_adapter)
             attn = kv.attention_with_fused_qkv(l, qkv, s.num_attention_heads, frag=frag)
-            parts = self._linear_acc(attn, L["o"], resid, ks_ws)
-            if tok_adapter:
-                self._lora(resid, attn, l, "o_proj", tok_adapter)
+            if fuse and self._fused_linear(fuse, attn, L["o"], l, (("o_proj", 0, H),), resid=resid) is not None:
+                parts = None
+            else:
+                parts = self._linear_acc(attn, L["o"], resid, ks_ws)
+                if tok_adapter:
+                    self._lora(resid, attn, l, "o_proj", tok_adapter)
             xn = ops.rmsnorm(resid, L["ln2"], s.rms_norm_eps, frag=frag, parts=parts)
             if dec_frag and I % 32 == 0 and not (tok_adapter and self._targets(l, "gate_proj", "up_proj")):
                 # decode step without an adapter on gate / up: the SiLU product is the epilogue of the GEMV (same bits)
                 act = ops.gate_up_silu(xn, self.interleaved_gate_up()[l])
             else:
-                gu = ops.linear(xn, L["gate_up"])
-                if tok_adapter:
-                    self._lora_group(gu, xn, l, (("gate_proj", 0, I), ("up_proj", I, I)), tok_adapter)
+                gu_projs = (("gate_proj", 0, I), ("up_proj", I, I))
+                gu = self._fused_linear(fuse, xn, L["gate_up"], l, gu_projs) if fuse else None
+                if gu is None:
+                    gu = ops.linear(xn, L["gate_up"])
+                    if tok_adapter:
+                        self._lora_group(gu, xn, l, gu_projs, tok_adapter)
                 act = ops.silu_mul(gu, frag=frag)
-            parts = self._linear_acc(act, L["down"], resid, ks_ws)
-            if tok_adapter:
-                self._lora(resid, act, l, "down_proj", tok_adapter)
+            if fuse and self._fused_linear(fuse, act, L["down"], l, (("down_proj", 0, H),), resid=resid) is not None:
+                parts = None
+            else:
+                parts = self._linear_acc(act, L["down"], resid, ks_ws)
+                if tok_adapter:
+                    self._lora(resid, act, l, "down_proj", tok_adapter)
         if logits_rows is not None:
             if parts is not None:                         # pending K-slice partials of the last down_proj, in slice order
                 pv = parts.part[: (parts.ks - 1) * T * parts.ld].view(parts.ks - 1, T, parts.ld)
@@ -350,6 +370,34 @@ class LlamaForCausalLM:
             resid = resid[logits_rows].contiguous()
         xn = ops.rmsnorm(resid, self.norm, s.rms_norm_eps, frag=resid.shape[0] <= 64 or frag, parts=parts)
         return ops.linear(xn, self.lm_head, out_dtype=torch.float32)
+
+    def _fused_linear(self, fuse, x, W, l, projs, resid=None):
+        """The base linear of `projs` = ((name, first row, rows), ...) with the adapter deltas as extra k-steps of the
+        GEMM, then the separate gather-matmul for the tokens whose 256-token block mixes adapters.  resid: accumulate
+        into it (o_proj, down_proj).  Returns None when the shape or the row ranges do not allow it."""
+        lt, ids, blk, rest = fuse
+        T, K = x.shape
+        N = W.shape[0]
+        live = [(proj, c0, n, lt.tables.get((l, proj))) for proj, c0, n in projs]
+        live = [e for e in live if e[3] is not None]
+        if not live or not ops.gemm_frag_preferred(T, K, N) or any(c0 % 256 or (n % 256 and c0 + n != N) for _, c0, n, _ in live):
+            return None
+        key = (T, lt.r)
+        if getattr(self, "_v_split_key", None) != key:
+            self._v_split = [tuple(torch.empty((T, lt.r), dtype=torch.float16, device=self.device) for _ in range(2)) for _ in range(3)]
+            self._v_split_key = key
+        vs = ops.lora_shrink_split(x, [tab[0] for *_, tab in live], ids, lt.scaling, self._workspace(T, K, lt.r), out=self._v_split[:len(live)])
+        fused = [(tab[1], vh, vl, c0, n) for (_, c0, n, tab), (vh, vl) in zip(live, vs)]
+        if resid is not None:
+            y = ops.linear_frag_lora(x, W, fused, blk, lt.r, out=resid, accumulate=True)
+        else:
+            y = ops.linear_frag_lora(x, W, fused, blk, lt.r)
+        if rest is not None:
+            if resid is not None:
+                self._lora(y, x, l, projs[0][0], rest)
+            else:
+                self._lora_group(y, x, l, projs, rest)
+        return y
 
     def _ksplit_ws(self, T):
         """fp32 scratch for the K-split partials of o_proj / down_proj at T tokens (grown on demand, reused)."""

@@ -339,6 +339,60 @@ def gemm_frag_preferred(T: int, K: int, N: int) -> bool:
     return bool(lib().mlora_gemm_frag_preferred(T, K, N))
 
 
+def lora_block_adapters(tok_adapter: torch.Tensor, n_ad: int):
+    """ids [T] int32 -> (blk_adapter [ceil(T / 256)]: the adapter a 256-token block agrees on or -1,
+    tok_rest [T]: -1 where the block's delta can ride in the GEMM, else the token's id)."""
+    T = tok_adapter.shape[0]
+    blk = torch.empty((max(-(-T // 256), 1),), dtype=torch.int32, device=tok_adapter.device)
+    rest = torch.empty((max(T, 1),), dtype=torch.int32, device=tok_adapter.device)[:T]
+    check(lib().mlora_lora_block_adapters(blk.data_ptr(), rest.data_ptr(), _dev(tok_adapter, torch.int32), T, n_ad, _stream()))
+    return blk, rest
+
+
+def lora_shrink_split(x, A_list, tok_adapter, scaling: float, workspace, out=None):
+    """The matrix-core shrink of up to three projections that read x (A [n_ad, r, K] each), as fp16 hi + lo halves:
+    -> [(v_hi [T, r], v_lo [T, r]), ...]."""
+    import ctypes as C
+    xp, lay, T, K = _x_arg(x)
+    n_ad, r, _ = A_list[0].shape
+    dev = tok_adapter.device
+    if out is None:
+        out = [(torch.empty((T, r), dtype=torch.float16, device=dev), torch.empty((T, r), dtype=torch.float16, device=dev)) for _ in A_list]
+    n = len(A_list)
+    hi = (C.c_void_p * n)(*[o[0].data_ptr() for o in out])
+    lo = (C.c_void_p * n)(*[o[1].data_ptr() for o in out])
+    Ap = (C.c_void_p * n)(*[_dev(a, torch.float16, "A") for a in A_list])
+    check(lib().mlora_lora_shrink_split(C.cast(hi, C.c_void_p), C.cast(lo, C.c_void_p), xp, lay, C.cast(Ap, C.c_void_p), n,
+                                        _dev(tok_adapter, torch.int32), float(scaling), T, K, r, n_ad, _dev(workspace, torch.float32),
+                                        workspace.numel() * 4, _stream()))
+    return out
+
+
+def linear_frag_lora(x: FragActivation, W: PackedWeight, projs, blk_adapter, r: int, out=None, out_dtype=torch.float16, accumulate=False):
+    """`linear(x, W)` with the LoRA deltas of `projs` = [(B [n_ad, rows, r], v_hi, v_lo, first row, rows), ...] carried as
+    extra k-steps of the GEMM for the token blocks that `blk_adapter` gives an adapter (shapes of the persistent GEMM)."""
+    import ctypes as C
+    from ._lib import FusedLora
+    T, K = x.shape
+    N, K2 = W.shape
+    if K2 != K:
+        raise ValueError(f"linear_frag_lora: x{x.shape} vs W{W.shape}")
+    if out is None:
+        if accumulate:
+            raise ValueError("linear_frag_lora: accumulate needs out")
+        out = torch.empty((T, N), dtype=out_dtype, device=x.device)
+    if out.shape != (T, N):
+        raise ValueError(f"linear_frag_lora: out{tuple(out.shape)} expected {(T, N)}")
+    arr = (FusedLora * len(projs))()
+    for e, (B, vh, vl, n0, rows) in zip(arr, projs):
+        if B.shape[1] != rows or B.shape[2] != r or vh.shape != (T, r) or vl.shape != (T, r):
+            raise ValueError("linear_frag_lora: table or v shape")
+        e.B, e.v_hi, e.v_lo, e.n_begin, e.n_rows = _dev(B, torch.float16, "B"), _dev(vh, torch.float16, "v_hi"), _dev(vl, torch.float16, "v_lo"), n0, rows
+    check(lib().mlora_linear_frag_lora(_dev(out), _dt(out), ACCUMULATE if accumulate else STORE, x.data.data_ptr(), W.data.data_ptr(),
+                                       T, K, N, C.cast(arr, C.c_void_p), len(projs), _dev(blk_adapter, torch.int32), r, _stream()))
+    return out
+
+
 def interleave_gate_up(gate_up: torch.Tensor) -> PackedWeight:
     """[2I, K] (gate rows, then up rows) -> PackedWeight whose 16-row tiles alternate gate and up."""
     I2, K = gate_up.shape

@@ -385,6 +385,69 @@ def test_producers_write_fragment_order_for_prefill_sized_blocks(ops, synth):
         assert torch.equal(y1, y2) and not torch.equal(y1, c["y"])
 
 
+@pytest.mark.parametrize("r,acc", [(64, False), (32, False), (64, True)])
+def test_prefill_linear_with_lora_as_extra_k_steps(ops, synth, r, acc):
+    """The persistent GEMM carrying the adapter deltas of the 256-token blocks that agree on one adapter (two
+    projections = two row ranges with their own tables), the separate gather-matmul serving the rest: against the
+    float64 evaluation, for fp16 output and for accumulation into fp32."""
+    T, K, N, n_ad = 4000, 320, 4096, 5
+    half = N // 2
+    x = synth.normal(19, "fl.x", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(19, "fl.W", (N, K), 0.05, torch.float16, DEV)
+    A = [synth.normal(19, f"fl.A{p}", (n_ad, r, K), 0.05, torch.float16, DEV) for p in range(2)]
+    B = [synth.normal(19, f"fl.B{p}", (n_ad, half, r), 0.05, torch.float16, DEV) for p in range(2)]
+    ids = np.full(T, 1, np.int32)
+    ids[:1024] = 2                       # four whole blocks of adapter 2
+    ids[1024:1100] = 4                   # a block that mixes adapters 4 and 0
+    ids[1100:1280] = 0
+    ids[1280:1536] = -1                  # a block without adapter
+    ids[1536:1800] = 3                   # adapter 3 ends inside a block, adapter 1 takes over
+    ids_d = torch.from_numpy(ids).to(DEV)
+    blk, rest = ops.lora_block_adapters(ids_d, n_ad)
+    want_blk = np.array([2, 2, 2, 2, -1, -1, 3, -1] + [1] * 8, np.int32)
+    assert np.array_equal(blk.cpu().numpy(), want_blk)
+    rest_h = rest.cpu().numpy()
+    assert np.array_equal(rest_h, np.where(np.repeat(want_blk, 256)[:T] >= 0, -1, ids))
+    scaling = 0.5
+    ws = torch.empty(2 * ops.lib().mlora_gather_mm_workspace_bytes(T, K, r) // 4 + 4, dtype=torch.float32, device=DEV)
+    xf = ops.FragActivation.pack(x)
+    vs = ops.lora_shrink_split(xf, A, ids_d, scaling, ws)
+    projs = [(B[p], vs[p][0], vs[p][1], p * half, half) for p in range(2)]
+    Wp = ops.PackedWeight(W)
+    xd, Wd = _np(x).astype(np.float64), _np(W).astype(np.float64)
+    base = xd @ Wd.T
+    delta = np.zeros_like(base)
+    for p in range(2):
+        Ad, Bd = _np(A[p]).astype(np.float64), _np(B[p]).astype(np.float64)
+        for a in range(n_ad):
+            rows = np.nonzero(ids == a)[0]
+            delta[rows, p * half:(p + 1) * half] = scaling * (xd[rows] @ Ad[a].T) @ Bd[a].T
+    if acc:
+        r0 = synth.normal(19, "fl.r0", (T, N), 1.0, torch.float32, DEV)
+        y = r0.clone()
+        ops.linear_frag_lora(xf, Wp, projs, blk, r, out=y, accumulate=True)
+        base = base + _np(r0).astype(np.float64)
+    else:
+        y = ops.linear_frag_lora(xf, Wp, projs, blk, r)
+    torch.cuda.synchronize()
+    in_gemm = np.repeat(want_blk, 256)[:T] >= 0
+    y0 = _np(y).astype(np.float64)
+    tol, floor = (5e-4, 1e-2) if acc else (TOL, 1e-3)
+    # blocks with an adapter: base and delta summed before the one rounding; the other rows: the base product alone
+    assert max_rel_err(y0[in_gemm], (base + delta)[in_gemm], floor=floor) <= tol
+    assert max_rel_err(y0[~in_gemm], base[~in_gemm], floor=floor) <= tol
+    assert np.abs(delta[in_gemm]).max() > 0.5 and np.abs(delta[~in_gemm]).max() > 0.5        # the deltas matter
+    for p in range(2):                   # the tokens of mixed blocks: the separate call on the rest ids, added to the stored y
+        ops.gather_mm(y[:, p * half:(p + 1) * half], xf, A[p], B[p], rest, scaling)
+    torch.cuda.synchronize()
+    y1 = _np(y).astype(np.float64)
+    assert np.array_equal(y1[in_gemm], y0[in_gemm])
+    assert max_rel_err(y1[~in_gemm], (y0 + delta)[~in_gemm], floor=floor) <= tol
+    # without any delta in the blocks the entry equals the plain GEMM bit for bit
+    none = torch.full_like(blk, -1)
+    assert torch.equal(ops.linear_frag_lora(xf, Wp, projs, none, r), ops.linear(xf, Wp))
+
+
 def test_pack_weight_is_a_permutation(ops, synth):
     """Bit-exact: every element of W appears at its fragment-order position, padding rows are zero."""
     N, K = 40, 64

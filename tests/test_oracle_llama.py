@@ -257,3 +257,31 @@ def test_mixed_mode_rounds_storage_points_only():
 
 def test_argmax_tie_rule():
     assert int(np.argmax(np.array([1.0, 3.0, 3.0, 2.0]))) == 1
+
+
+def test_mixed_mode_rounds_fused_blocks_once():
+    """`fuse_blocks` moves one rounding point of the mixed mode (base + delta rounded once for the tokens of an
+    adapter-uniform block) and nothing else: the fp32 mode ignores it, tokens of mixed blocks keep two roundings,
+    and the change stays within an fp16 step."""
+    import oracle
+    synth = load_pkg("synth")
+    shape = synth.LlamaShape(hidden_size=64, intermediate_size=128, num_attention_heads=4, num_key_value_heads=4,
+                             num_hidden_layers=1, head_dim=16, vocab_size=50)
+    spec = synth.LoraSpec(r=8, alpha=16.0, n_adapters=3, targets=("q_proj", "gate_proj"))
+    import torch
+    w = {k: v.float().numpy() for k, v in synth.base_weights(5, shape, torch.float16, "cpu").items()}
+    lw = {k: v.float().numpy() for k, v in synth.lora_weights(5, shape, spec, torch.float16, "cpu", tag="a0").items()}
+    x = oracle.f16(np.random.default_rng(0).normal(size=(8, 64)).astype(np.float32))
+    ids = np.array([1, 1, 1, 1, 2, 0, 2, 2], np.int32)            # block 0 (4 tokens) uniform, block 1 mixed
+    outs = {}
+    for mode in ("mixed", "fp32"):
+        for fb in (None, 4):
+            m = oracle.LlamaRef(shape, w, lw, {"a0": spec.scaling}, mode=mode)
+            m.fuse_blocks = fb
+            outs[(mode, fb)] = m._proj(x, 0, "q_proj", {"a0": ids})
+    assert np.array_equal(outs[("fp32", None)], outs[("fp32", 4)])
+    a, b = outs[("mixed", None)], outs[("mixed", 4)]
+    assert np.array_equal(a[4:], b[4:]) and not np.array_equal(a[:4], b[:4])
+    exact = outs[("fp32", None)]
+    assert np.abs(b[:4] - exact[:4]).max() <= np.abs(a[:4] - exact[:4]).max() + 1e-7     # one rounding is no worse than two
+    assert np.array_equal(b[:4], oracle.f16(exact[:4]))
