@@ -106,7 +106,9 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(f16* __restrict__
         const f16* __restrict__ B = lx.B + (size_t)id * H * lx.r;
         const int lpr = lx.r >> 3;                  // lanes (16-byte chunks) per output column
         const int chunks = H * lpr;
-        constexpr int NB = 8;
+        // one batch is 16 chunks per thread: all of B[id] for rank 16 and H = 4096, so that the table is requested once,
+        // as a whole, right behind the adapter id
+        constexpr int NB = VPT == 1 ? 16 : 8;
         f16x8 bv[NB];
         auto load_batch = [&](int q0) {
 #pragma unroll
@@ -116,37 +118,44 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(f16* __restrict__
             if (q < chunks) bv[u] = ld8(B + (size_t)q * 8);
           }
         };
-        // the shrink results and the first batch of B go out together, before the barrier that publishes lv
+        // the first batch of B and the shrink results go out together, before the barrier that publishes lv
+        load_batch(0);
         float lvv = 0.f;
         if (threadIdx.x < lx.r) {
           if (PARTS && lx.src.kc == 0) {            // dense shrink rows were K-split with the matrix: add their partials
             const size_t col = (size_t)id * lx.r + threadIdx.x;
             float a = lx.src.v[(size_t)row * lx.src.ld + col];
-            for (int q = 0; q < kp.n; ++q) a += kp.p[q * kp.stride + (size_t)row * kp.ld + H + col];
+            float pq[MAX_PARTS];                    // all requested before the first is added
+#pragma unroll
+            for (int q = 0; q < MAX_PARTS; ++q) pq[q] = q < kp.n ? kp.p[q * kp.stride + (size_t)row * kp.ld + H + col] : 0.f;
+#pragma unroll
+            for (int q = 0; q < MAX_PARTS; ++q)
+              if (q < kp.n) a += pq[q];
             lvv = a * lx.scaling;
           } else {
             lvv = lora_v_from(lx.src, 0, id, lx.r, row, threadIdx.x, lx.scaling);
           }
         }
-        load_batch(0);
         if (threadIdx.x < lx.r) lv[threadIdx.x] = lvv;
         __syncthreads();
+        // a thread's chunks all cover the same 8 ranks (the thread count is a multiple of the chunks per column)
+        const int sub = threadIdx.x % lpr;
+        float lvr[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) lvr[e] = lv[sub * 8 + e];
         for (int q0 = 0; q0 < chunks; q0 += NORM_THREADS * NB) {
           float part[NB];
 #pragma unroll
           for (int u = 0; u < NB; ++u) {
-            const int q = q0 + u * NORM_THREADS + threadIdx.x;
-            const int sub = q % lpr;
             float s = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) s = fmaf((float)bv[u][e], lv[sub * 8 + e], s);
+            for (int e = 0; e < 8; ++e) s = fmaf((float)bv[u][e], lvr[e], s);
             part[u] = s;
           }
           if (q0 + NORM_THREADS * NB < chunks) load_batch(q0 + NORM_THREADS * NB);   // next batch flies during the reduce
 #pragma unroll
           for (int u = 0; u < NB; ++u) {
             const int q = q0 + u * NORM_THREADS + threadIdx.x;
-            const int sub = q % lpr;
             float s = part[u];
             for (int o = 1; o < lpr; o <<= 1) s += __shfl_xor(s, o, WAVE);   // neighbouring groups of 8 first
             if (sub == 0 && q < chunks) delta[q / lpr] = s;
