@@ -579,54 +579,58 @@ int launch_gemm_pp(void* y, const f16* x, int ldx, int x_tt, const f16* Wp, int 
 // Token blocks between the decode GEMV and the persistent kernel above (65 to a few hundred tokens: a decode step of
 // many sequences, a short prefill).  The weights are read once and the matrix cores and the operand loads weigh about
 // the same, so the block is as tall as the token block allows and narrow enough to give every compute unit a
-// workgroup: FT x 8 fragments (128 or 256 tokens x 128 weight rows), eight waves, both operands in fragment order and
-// copied from global memory straight into an LDS ring.  A stage of the ring is TWO 32-k steps (32 or 48 KiB): with the
-// few MFMAs a wave has per 32-k step here (8 or 16), a barrier and a wait per step cost more than the step itself.
-// Four (three) stages, of which three (two) - 96 KiB - are in flight per compute unit.
+// workgroup: FT x FN fragments (128 or 256 tokens x 128 or 64 weight rows), eight waves, both operands in fragment
+// order and copied from global memory straight into an LDS ring.  A stage of the ring is TWO 32-k steps: with the
+// few MFMAs a wave has per 32-k step here (4 to 16), a barrier and a wait per step cost more than the step itself.
+// Four (three) stages, of which three (two) are in flight per compute unit.
+// (Measured on this kernel: a deeper ring for the weights alone, with waves that fetch only weights, changes
+// nothing - a workgroup's weight stream runs at 12 to 19 GB/s whatever it keeps in flight, and the launch as a whole
+// at 2 to 3.4 TB/s; with the weights coming from L2 instead the same loop is 1.5 times faster.)
 // grid = (weight-row blocks, K slices, token blocks).
 // With K slices, slice 0 produces the result proper (store or accumulate) and slice s > 0 stores its fp32 partial
 // sums to part[s - 1][T][ld_part] - for the two narrow accumulating linears of a layer, whose partials the next
 // RMSNorm of the row adds in slice order.
 // ---------------------------------------------------------------------------------------------
-constexpr int MID_FN = 8;
 constexpr int MID_KS = 2;                      // 32-k steps per stage
 
-template <int OUT, int FT>
+template <int OUT, int FT, int FN>
 __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __restrict__ yv, float* __restrict__ part, int ld_part,
                                                                     const f16* __restrict__ xf, int x_tt, const f16* __restrict__ Wp,
                                                                     int T, int K, int N) {
   constexpr int MID_STAGES = FT == 16 ? 3 : 4;
-  constexpr int SF = MID_FN + FT;              // fragments of one 32-k step: weights, then tokens
+  constexpr int SF = FN + FT;                  // fragments of one 32-k step: weights, then tokens
   constexpr int LF = MID_KS * SF;              // fragments per stage
-  constexpr int LQ = LF / PP_WAVES;            // ... of which a wave fetches LQ (fragment f = wave + 8 q, k-step f / SF)
+  constexpr int LQ = LF / PP_WAVES;            // ... of which a wave fetches LQ (fragment f = wave + 8 q: fragment f % SF of k-step f / SF)
   constexpr int STAGE_ELEMS = LF * 512;
   constexpr int WTF = FT / 4;                  // token fragments of a wave's tile
-  static_assert(LF % PP_WAVES == 0 && FT % 4 == 0 && SF % PP_WAVES == 0, "fragments divide over the waves");
+  constexpr int WNF = FN / 2;                  // weight fragments of a wave's tile
+  constexpr int VM = (MID_STAGES - 2) * LQ;    // a wave's loads that may still be in flight when the next stage is read
+  static_assert(LF % PP_WAVES == 0 && FT % 4 == 0 && FN % 2 == 0 && WNF <= 4, "fragments divide over the waves");
+  static_assert(VM == 5 || VM == 6 || VM == 8, "wait_next has an instruction for each of these");
   extern __shared__ __align__(16) f16 smem[];  // [MID_STAGES][STAGE_ELEMS]; the output staging reuses it after the K loop
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int KB = K / 32;
   const int tiles = (N + 15) / 16;
-  const int n0 = blockIdx.x * MID_FN * 16, t0 = blockIdx.z * FT * 16;
+  const int n0 = blockIdx.x * FN * 16, t0 = blockIdx.z * FT * 16;
   const int per = (KB + gridDim.y - 1) / gridDim.y;
   const int kb0 = blockIdx.y * per;
   const int kb1 = kb0 + per < KB ? kb0 + per : KB;
   const int nks = kb1 - kb0;                   // 32-k steps of this slice (>= 1: checked by the launcher)
   const int nst = (nks + MID_KS - 1) / MID_KS; // stages
 
-  // fragment f = wave + 8 q of a stage: k-step f / SF of the stage, fragment f % SF of that step (SF % 8 == 0, so a
-  // wave fetches the same fragments of every step)
   const f16* src[LQ];
-  int step[LQ];
+  int step[LQ], kso[LQ];
 #pragma unroll
   for (int q = 0; q < LQ; ++q) {
     const int f = (wave + PP_WAVES * q) % SF;  // uniform
-    if (f < MID_FN) {
+    kso[q] = (wave + PP_WAVES * q) / SF;
+    if (f < FN) {
       int nt = n0 / 16 + f;
       nt = nt < tiles ? nt : tiles - 1;        // rows past N: a valid fragment, results dropped
       src[q] = Wp + (size_t)nt * KB * 512 + lane * 8;
       step[q] = 512;
     } else {
-      int tt = t0 / 16 + f - MID_FN;
+      int tt = t0 / 16 + f - FN;
       tt = tt < x_tt ? tt : x_tt - 1;          // tiles past T: a valid fragment, results dropped
       src[q] = xf + (size_t)tt * 512 + lane * 8;
       step[q] = x_tt * 512;
@@ -637,7 +641,7 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
     f16* dst = smem + ring * STAGE_ELEMS + wave * 512;
 #pragma unroll
     for (int q = 0; q < LQ; ++q) {
-      int kb = load_kb + (wave + PP_WAVES * q) / SF;
+      int kb = load_kb + kso[q];
       kb = kb < kb1 ? kb : kb1 - 1;            // past the slice: a valid address; the data is not multiplied
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + (size_t)kb * step[q]),
                                        (__attribute__((address_space(3))) void*)(dst + q * PP_WAVES * 512), 16, 0, 0);
@@ -646,11 +650,11 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
     load_kb += MID_KS;
   };
 
-  const int wn = wave & 1, wt = wave >> 1;     // weight rows wn * 64 .., tokens wt * WTF * 16 ..
-  f32x4 acc[4][WTF];
-  f16x8 a[2][MID_KS][4], b[2][MID_KS][WTF];    // two register sets: the stage being multiplied and its successor
+  const int wn = wave & 1, wt = wave >> 1;     // weight rows wn * WNF * 16 .., tokens wt * WTF * 16 ..
+  f32x4 acc[WNF][WTF];
+  f16x8 a[2][MID_KS][WNF], b[2][MID_KS][WTF];  // two register sets: the stage being multiplied and its successor
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < WNF; ++i)
 #pragma unroll
     for (int j = 0; j < WTF; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   int rd = 0;
@@ -660,9 +664,9 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
 #pragma unroll
     for (int ks = 0; ks < MID_KS; ++ks) {
 #pragma unroll
-      for (int j = 0; j < WTF; ++j) b[u][ks][j] = ld8(st + (ks * SF + MID_FN + wt * WTF + j) * 512);
+      for (int j = 0; j < WTF; ++j) b[u][ks][j] = ld8(st + (ks * SF + FN + wt * WTF + j) * 512);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) a[u][ks][i] = ld8(st + (ks * SF + wn * 4 + i) * 512);
+      for (int i = 0; i < WNF; ++i) a[u][ks][i] = ld8(st + (ks * SF + wn * WNF + i) * 512);
     }
     rd = rd + 1 == MID_STAGES ? 0 : rd + 1;
   };
@@ -673,7 +677,7 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
     for (int ks = 0; ks < MID_KS; ++ks) {
       if (done_ks + ks < nks) {                // uniform: the last stage of an odd slice holds one step only
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < WNF; ++i)
 #pragma unroll
           for (int j = 0; j < WTF; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][ks][i], b[u][ks][j], acc[i][j], 0, 0, 0);
       }
@@ -684,9 +688,9 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
   // stage multiplied next has landed; with everybody's wait and fragment reads behind the barrier, the slot of the
   // stage just read is refilled
   auto wait_next = [&]() {
-    if constexpr (FT == 16) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
+    if constexpr (VM == 5) asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory");
+    else if constexpr (VM == 6) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
-    static_assert((MID_STAGES - 2) * LQ == (FT == 16 ? 6 : 8), "the immediates above");
   };
   auto stage = [&](auto U) {
     constexpr int u = decltype(U)::value;
@@ -721,30 +725,31 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
       const int t = t0 + (wt * WTF + j) * 16 + r16;
       if (t >= T) continue;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int n = n0 + (wn * 4 + i) * 16 + gq * 4;
+      for (int i = 0; i < WNF; ++i) {
+        const int n = n0 + (wn * WNF + i) * 16 + gq * 4;
         if (n < N) *reinterpret_cast<f32x4*>(pp + (size_t)t * ld_part + n) = acc[i][j];
       }
     }
     return;
   }
   if constexpr (OUT == OUT_F16) {
-    // 16 tokens x 64 columns at a time through the wave's staging buffer: D[n][t] fragments in, token rows out
+    // 16 tokens x (16 WNF) columns at a time through the wave's staging buffer: D[n][t] fragments in, token rows out
     f16* ostage = smem + wave * PP_OUT_ELEMS;
+    constexpr int CPR = WNF * 2;               // 16-byte chunks per token row
 #pragma unroll
     for (int j = 0; j < WTF; ++j) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < WNF; ++i) {
         const f32x4 sacc = acc[i][j];
         *reinterpret_cast<f16x4*>(ostage + r16 * PP_OUT_LD + i * 16 + gq * 4) = f16x4{(f16)sacc[0], (f16)sacc[1], (f16)sacc[2], (f16)sacc[3]};
       }
       __builtin_amdgcn_wave_barrier();
 #pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        const int c = q * 64 + lane;             // 16-byte chunk: token row c / 8, columns (c % 8) * 8 ..
-        const int tr = c >> 3, cc = (c & 7) * 8;
+      for (int q = 0; q < 16 * CPR / WAVE; ++q) {
+        const int c = q * 64 + lane;             // 16-byte chunk: token row c / CPR, columns (c % CPR) * 8 ..
+        const int tr = c / CPR, cc = (c % CPR) * 8;
         const int t = t0 + (wt * WTF + j) * 16 + tr;
-        const int n = n0 + wn * 64 + cc;
+        const int n = n0 + wn * WNF * 16 + cc;
         const f16x4 lo = *reinterpret_cast<const f16x4*>(ostage + tr * PP_OUT_LD + cc);
         const f16x4 hi = *reinterpret_cast<const f16x4*>(ostage + tr * PP_OUT_LD + cc + 4);
         if (t < T && n + 8 <= N) {
@@ -765,8 +770,8 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
       const int t = t0 + (wt * WTF + j) * 16 + r16;
       if (t >= T) continue;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int n = n0 + (wn * 4 + i) * 16 + gq * 4;
+      for (int i = 0; i < WNF; ++i) {
+        const int n = n0 + (wn * WNF + i) * 16 + gq * 4;
         if (n >= N) continue;
         const size_t o = (size_t)t * N + n;
         if constexpr (OUT == OUT_F32) {
@@ -780,44 +785,53 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
   }
 }
 
-// Block height and K slices of the mid-size kernel for a shape: 128-token blocks when 256-token ones would leave most
-// compute units without a workgroup.
+// Block shape and K slices of the mid-size kernel for a shape: 128-token blocks when 256-token ones would leave most
+// compute units without a workgroup, and 64 weight rows per block instead of 128 when that still leaves half of them
+// idle (up to 128 tokens: 170 instead of 192 us for the four linears of a 4096 / 11008 layer; with two token blocks
+// the narrow form loses, so it is not taken there).
 struct MidShape {
-  int ft, ksplit;
+  int ft, fn, ksplit;
 };
 MidShape gemm_mid_shape(int T, int K, int N, int ksplit_max) {
-  const int cols = ceil_div(N, MID_FN * 16);
+  const int by_k = (K / 32) / 16 < 1 ? 1 : (K / 32) / 16;   // at least 16 k-steps per slice
+  const int ks_cap = ksplit_max < by_k ? ksplit_max : by_k;
   MidShape m;
-  m.ft = (T <= 128 || (long)cols * ceil_div(T, 256) * ksplit_max <= 128) ? 8 : 16;
-  int ks = 256 / (cols * ceil_div(T, m.ft * 16));
-  const int by_k = (K / 32) / 16;              // at least 16 k-steps per slice
-  if (ks > by_k) ks = by_k;
-  if (ks > ksplit_max) ks = ksplit_max;
+  const int cols8 = ceil_div(N, 128);
+  m.ft = (T <= 128 || (long)cols8 * ceil_div(T, 256) * ksplit_max <= 128) ? 8 : 16;
+  const int tb = ceil_div(T, m.ft * 16);
+  m.fn = (long)cols8 * tb * ks_cap <= 128 ? 4 : 8;
+  const int cols = ceil_div(N, m.fn * 16);
+  int ks = 256 / (cols * tb);
+  if (ks > ks_cap) ks = ks_cap;
   m.ksplit = ks < 1 ? 1 : ks;
   return m;
 }
 
-template <int OUT, int FT>
-int launch_gemm_mid_ft(void* y, float* part, int ld_part, int ksplit, const f16* xf, int x_tt, const f16* Wp, int T, int K, int N,
-                       hipStream_t s) {
-  constexpr size_t lds = (size_t)(FT == 16 ? 3 : 4) * MID_KS * (MID_FN + FT) * 512 * sizeof(f16);
+template <int OUT, int FT, int FN>
+int launch_gemm_mid_shape(void* y, float* part, int ld_part, int ksplit, const f16* xf, int x_tt, const f16* Wp, int T, int K, int N,
+                          hipStream_t s) {
+  constexpr size_t lds = (size_t)(FT == 16 ? 3 : 4) * MID_KS * (FN + FT) * 512 * sizeof(f16);
   static_assert(lds >= (size_t)PP_WAVES * PP_OUT_ELEMS * sizeof(f16), "the output staging fits the ring");
   static bool configured = false;                    // the attribute is per kernel, set once per process
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_mid_kernel<OUT, FT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mid_kernel<OUT, FT, FN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return mlora_set_error(MLORA_ERR_LAUNCH, "linear_frag: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     configured = true;
   }
-  const dim3 grid(ceil_div(N, MID_FN * 16), ksplit, ceil_div(T, FT * 16));
-  hipLaunchKernelGGL((gemm_mid_kernel<OUT, FT>), grid, dim3(PP_WAVES * WAVE), lds, s, y, part, ld_part, xf, x_tt, Wp, T, K, N);
+  const dim3 grid(ceil_div(N, FN * 16), ksplit, ceil_div(T, FT * 16));
+  hipLaunchKernelGGL((gemm_mid_kernel<OUT, FT, FN>), grid, dim3(PP_WAVES * WAVE), lds, s, y, part, ld_part, xf, x_tt, Wp, T, K, N);
   return MLORA_OK;
 }
 
 template <int OUT>
-int launch_gemm_mid(void* y, float* part, int ld_part, int ksplit, int ft, const f16* xf, int x_tt, const f16* Wp, int T, int K, int N,
+int launch_gemm_mid(void* y, float* part, int ld_part, const MidShape& m, const f16* xf, int x_tt, const f16* Wp, int T, int K, int N,
                     hipStream_t s) {
-  if (ft == 8) return launch_gemm_mid_ft<OUT, 8>(y, part, ld_part, ksplit, xf, x_tt, Wp, T, K, N, s);
-  return launch_gemm_mid_ft<OUT, 16>(y, part, ld_part, ksplit, xf, x_tt, Wp, T, K, N, s);
+  if (m.ft == 8) {
+    if (m.fn == 4) return launch_gemm_mid_shape<OUT, 8, 4>(y, part, ld_part, m.ksplit, xf, x_tt, Wp, T, K, N, s);
+    return launch_gemm_mid_shape<OUT, 8, 8>(y, part, ld_part, m.ksplit, xf, x_tt, Wp, T, K, N, s);
+  }
+  if (m.fn == 4) return launch_gemm_mid_shape<OUT, 16, 4>(y, part, ld_part, m.ksplit, xf, x_tt, Wp, T, K, N, s);
+  return launch_gemm_mid_shape<OUT, 16, 8>(y, part, ld_part, m.ksplit, xf, x_tt, Wp, T, K, N, s);
 }
 
 template <int OUT, int FT, int FN, int WT_, int WN_>
@@ -919,10 +933,10 @@ extern "C" int mlora_linear_frag(void* y, int y_dtype, int mode, const void* xf,
     else if (y_dtype == MLORA_F32) e = launch_gemm_pp<OUT_F32>(y, x, 0, tt, W, T, K, N, s);
     else e = launch_gemm_pp<OUT_F16>(y, x, 0, tt, W, T, K, N, s);
   } else {
-    const int ft = gemm_mid_shape(T, K, N, 1).ft;
-    if (mode == MLORA_ACCUMULATE) e = launch_gemm_mid<OUT_ACC_F32>(y, nullptr, 0, 1, ft, x, tt, W, T, K, N, s);
-    else if (y_dtype == MLORA_F32) e = launch_gemm_mid<OUT_F32>(y, nullptr, 0, 1, ft, x, tt, W, T, K, N, s);
-    else e = launch_gemm_mid<OUT_F16>(y, nullptr, 0, 1, ft, x, tt, W, T, K, N, s);
+    const MidShape m = gemm_mid_shape(T, K, N, 1);
+    if (mode == MLORA_ACCUMULATE) e = launch_gemm_mid<OUT_ACC_F32>(y, nullptr, 0, m, x, tt, W, T, K, N, s);
+    else if (y_dtype == MLORA_F32) e = launch_gemm_mid<OUT_F32>(y, nullptr, 0, m, x, tt, W, T, K, N, s);
+    else e = launch_gemm_mid<OUT_F16>(y, nullptr, 0, m, x, tt, W, T, K, N, s);
   }
   return e ? e : mlora_launch_status("linear_frag");
 }
@@ -965,8 +979,9 @@ int mlora_gemm_mid_acc(float* resid, float* part, int ld_part, int ks, const voi
                        void* stream) {
   MLORA_CHECK(K % 32 == 0 && ks >= 1 && (K / 32) / ks >= 1 && ((uintptr_t)xf & 15) == 0, MLORA_ERR_UNSUPPORTED,
               "linear_frag (K slices): need K %% 32 == 0 and at least one 32-k step per slice (K=%d ks=%d)", K, ks);
-  const int ft = gemm_mid_shape(T, K, N, ks).ft;
-  const int e = launch_gemm_mid<OUT_ACC_F32>(resid, part, ld_part, ks, ft, (const f16*)xf, mlora_frag_tiles(T), (const f16*)Wp, T, K, N,
+  MidShape m = gemm_mid_shape(T, K, N, ks);
+  m.ksplit = ks;                               // the caller's partial buffers were sized for ks slices
+  const int e = launch_gemm_mid<OUT_ACC_F32>(resid, part, ld_part, m, (const f16*)xf, mlora_frag_tiles(T), (const f16*)Wp, T, K, N,
                                              (hipStream_t)stream);
   return e ? e : mlora_launch_status("linear_frag (K slices)");
 }
