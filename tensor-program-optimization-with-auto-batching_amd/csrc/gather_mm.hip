@@ -1272,13 +1272,18 @@ __global__ __launch_bounds__(FUSE_BLOCK) void lora_block_adapters_kernel(int32_t
 }
 
 // vh, vl [T][R] fp16: hi and lo halves of scaling * (sum of the K-range partials of the shrink, in range order) - the
-// values and the split the expand kernels use
+// values and the split the expand kernels use.  blockIdx.y = projection; v = [n_proj][splits][T, R] fp32.
+struct VSplitOut {
+  f16* vh[SEG_MAX_PROJ];
+  f16* vl[SEG_MAX_PROJ];
+};
 template <int R>
-__global__ __launch_bounds__(256) void lora_v_split_kernel(f16* __restrict__ vh, f16* __restrict__ vl, const float* __restrict__ v,
-                                                           int splits, float scaling, int T) {
+__global__ __launch_bounds__(256) void lora_v_split_kernel(VSplitOut o, const float* __restrict__ v, int splits, float scaling, int T) {
   const int e = blockIdx.x * 256 + threadIdx.x;              // four rank entries of one token
   const int t = e / (R / 4), j = (e % (R / 4)) * 4;
   if (t >= T) return;
+  const int pj = blockIdx.y;
+  v += (size_t)pj * splits * T * R;
   f32x4 sum = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int sp = 0; sp < splits; ++sp) sum += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + t) * R + j);
   f16x4 h, l;
@@ -1288,8 +1293,8 @@ __global__ __launch_bounds__(256) void lora_v_split_kernel(f16* __restrict__ vh,
     h[q] = (f16)f;
     l[q] = (f16)(f - (float)h[q]);
   }
-  *reinterpret_cast<f16x4*>(vh + (size_t)t * R + j) = h;
-  *reinterpret_cast<f16x4*>(vl + (size_t)t * R + j) = l;
+  *reinterpret_cast<f16x4*>(o.vh[pj] + (size_t)t * R + j) = h;
+  *reinterpret_cast<f16x4*>(o.vl[pj] + (size_t)t * R + j) = l;
 }
 
 // shrink + expand on the matrix cores for pj.n projections; v = workspace viewed as [pj.n][splits][T, r] fp32
@@ -1570,12 +1575,14 @@ extern "C" int mlora_lora_shrink_split(void* const* v_hi, void* const* v_lo, con
   int splits;
   if (r == 32) splits = gmm_segments_shrink_r<32>(pj, (const f16*)x, frag_tt, tok_adapter, T, K, n_ad, v, bf, s);
   else splits = gmm_segments_shrink_r<64>(pj, (const f16*)x, frag_tt, tok_adapter, T, K, n_ad, v, bf, s);
+  VSplitOut vo = {};
   for (int i = 0; i < n_proj; ++i) {
-    const float* vi = v + (size_t)i * splits * T * r;
-    const dim3 grid(ceil_div(T * (r / 4), 256));
-    if (r == 32) hipLaunchKernelGGL((lora_v_split_kernel<32>), grid, dim3(256), 0, s, (f16*)v_hi[i], (f16*)v_lo[i], vi, splits, scaling, T);
-    else hipLaunchKernelGGL((lora_v_split_kernel<64>), grid, dim3(256), 0, s, (f16*)v_hi[i], (f16*)v_lo[i], vi, splits, scaling, T);
+    vo.vh[i] = (f16*)v_hi[i];
+    vo.vl[i] = (f16*)v_lo[i];
   }
+  const dim3 grid(ceil_div(T * (r / 4), 256), n_proj);
+  if (r == 32) hipLaunchKernelGGL((lora_v_split_kernel<32>), grid, dim3(256), 0, s, vo, v, splits, scaling, T);
+  else hipLaunchKernelGGL((lora_v_split_kernel<64>), grid, dim3(256), 0, s, vo, v, splits, scaling, T);
   return mlora_launch_status("lora_shrink_split");
 }
 
