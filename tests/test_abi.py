@@ -137,6 +137,27 @@ def test_argument_validation_of_fused_and_batched_entry_points():
     assert nk(2, None, 4096) == -1 and nk(2, 1, 1024) == -1 and nk(5, 1, 4096) == -1
     assert lib.mlora_rmsnorm_ksplit(1, 0, 1, 1, 2, 4096, 1, 1e-5, 4, 4096, 1, 1, 1, 1, 0.5, 4096, 16, 4, None) == -1   # dense partials need wider ld
     assert lib.mlora_rmsnorm_ksplit(1, 0, 1, 1, 2, 16384, 1, 1e-5, 4, 16384, None, 0, None, None, 0.0, 0, 0, 0, None) == -2   # H > 8192
+    # prefill linear that carries the LoRA deltas of adapter-uniform 256-token blocks as extra k-steps
+    assert lib.mlora_lora_block_adapters(None, 1, 1, 512, 4, None) == -1
+    assert lib.mlora_lora_block_adapters(1, 1, 1, 0, 4, None) == 0 and lib.mlora_lora_block_adapters(1, 1, 1, 512, 0, None) == -1
+    p3 = C.cast((C.c_void_p * 3)(16, 16, 16), C.c_void_p)
+    ss = lambda r=64, T=4096, K=4096, wsb=1 << 30, n_proj=3: lib.mlora_lora_shrink_split(p3, p3, 16, 1, p3, n_proj, 1, 0.5, T, K, r, 64, 16, wsb, None)
+    assert ss(r=16) == -2 and b"rank" in lib.mlora_last_error()      # ranks 32 and 64 only
+    assert ss(T=64) == -2 and ss(K=4100) == -2 and ss(n_proj=4) == -1
+    assert ss(wsb=1024) == -3 and b"workspace" in lib.mlora_last_error()
+    fl = (lm.FusedLora * 2)()
+    for i, e in enumerate(fl):
+        e.B, e.v_hi, e.v_lo, e.n_begin, e.n_rows = 16, 16, 16, 4096 * i, 4096
+    lf = lambda r=64, T=4096, N=8192, n_proj=2, blk=16: lib.mlora_linear_frag_lora(16, 0, 0, 16, 16, T, 4096, N, C.cast(fl, C.c_void_p), n_proj,
+                                                                                    blk, r, None)
+    assert lf(r=16) == -2 and lf(n_proj=4) == -2 and lf(blk=None) == -2
+    assert lf(T=256, N=4096) == -2 and b"persistent" in lib.mlora_last_error()      # too few 256 x 256 blocks for that kernel
+    fl[1].n_begin = 4096 + 128
+    assert lf() == -2 and b"256-row" in lib.mlora_last_error()
+    fl[1].n_begin, fl[1].n_rows = 4096, 8192
+    assert lf() == -2                                                              # rows past N
+    fl[1].n_rows, fl[1].v_lo = 4096, None
+    assert lf() == -1
     # decode step: a plan without layers / with a token count beyond the decode tile
     plan = lm.DecodePlan()
     assert lib.mlora_decode_step(C.byref(plan), None) < 0
