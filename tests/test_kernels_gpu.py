@@ -448,6 +448,38 @@ def test_prefill_linear_with_lora_as_extra_k_steps(ops, synth, r, acc):
     assert torch.equal(ops.linear_frag_lora(xf, Wp, projs, none, r), ops.linear(xf, Wp))
 
 
+def test_prefill_linear_with_lora_three_projections_and_a_ragged_last_one(ops, synth):
+    """Three projections of unequal width, the last ending 64 rows into a 256-row block of the GEMM, rank 32, every
+    block with an adapter: against the float64 evaluation."""
+    T, K, r, n_ad = 4096, 256, 32, 3
+    widths = [1024, 2048, 1088]
+    N = sum(widths)
+    begins = [0, 1024, 3072]
+    x = synth.normal(23, "fl3.x", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(23, "fl3.W", (N, K), 0.05, torch.float16, DEV)
+    A = [synth.normal(23, f"fl3.A{p}", (n_ad, r, K), 0.05, torch.float16, DEV) for p in range(3)]
+    B = [synth.normal(23, f"fl3.B{p}", (n_ad, widths[p], r), 0.05, torch.float16, DEV) for p in range(3)]
+    ids = np.repeat(np.array([0, 1, 2, 1], np.int32), T // 4)
+    ids_d = torch.from_numpy(ids).to(DEV)
+    blk, rest = ops.lora_block_adapters(ids_d, n_ad)
+    assert np.array_equal(blk.cpu().numpy(), np.repeat(np.array([0, 1, 2, 1], np.int32), 4)) and (rest.cpu().numpy() == -1).all()
+    scaling = 0.25
+    ws = torch.empty(3 * ops.lib().mlora_gather_mm_workspace_bytes(T, K, r) // 4 + 4, dtype=torch.float32, device=DEV)
+    xf = ops.FragActivation.pack(x)
+    vs = ops.lora_shrink_split(xf, A, ids_d, scaling, ws)
+    projs = [(B[p], vs[p][0], vs[p][1], begins[p], widths[p]) for p in range(3)]
+    y = ops.linear_frag_lora(xf, ops.PackedWeight(W), projs, blk, r)
+    torch.cuda.synchronize()
+    xd = _np(x).astype(np.float64)
+    ref = xd @ _np(W).astype(np.float64).T
+    for p in range(3):
+        Ad, Bd = _np(A[p]).astype(np.float64), _np(B[p]).astype(np.float64)
+        for a in range(n_ad):
+            rows = np.nonzero(ids == a)[0]
+            ref[rows, begins[p]:begins[p] + widths[p]] += scaling * (xd[rows] @ Ad[a].T) @ Bd[a].T
+    assert max_rel_err(_np(y).astype(np.float64), ref, floor=1e-3) <= TOL
+
+
 def test_pack_weight_is_a_permutation(ops, synth):
     """Bit-exact: every element of W appears at its fragment-order position, padding rows are zero."""
     N, K = 40, 64
