@@ -495,9 +495,11 @@ __device__ __forceinline__ void shrink_tile_mfma(float* __restrict__ v, const f1
       for (int u = 0; u < GA; ++u)
 #pragma unroll
         for (int i = 0; i < NT; ++i) acc[u][i] = f32x4{0.f, 0.f, 0.f, 0.f};
-      for (int kb = kb0 + wave; kb < kb1; kb += SEG_WAVES) {
-        const f16x8 xf = ld8(xr + (size_t)kb * xstep);
-        f16x8 af[GA][NT];
+      // two register sets: the k-step after this one is requested before this one is multiplied
+      f16x8 xf[2], af[2][GA][NT];
+      auto load = [&](int s, int kb) {
+        const int kk = kb < kb1 ? kb : kb1 - 1;                  // past the range: a valid address, the data is not multiplied
+        xf[s] = ld8(xr + (size_t)kk * xstep);
 #pragma unroll
         for (int u = 0; u < GA; ++u) {
           if (g0 + u < ta.n) {
@@ -505,17 +507,29 @@ __device__ __forceinline__ void shrink_tile_mfma(float* __restrict__ v, const f1
 #pragma unroll
             for (int i = 0; i < NT; ++i) {
               const int row = i * 16 + col;
-              af[u][i] = row < R ? ld8(Aa + (size_t)row * K + kb * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+              af[s][u][i] = row < R ? ld8(Aa + (size_t)row * K + kk * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
             }
           }
         }
+      };
+      auto multiply = [&](int s) {
 #pragma unroll
         for (int u = 0; u < GA; ++u) {
           if (g0 + u < ta.n) {
 #pragma unroll
             for (int i = 0; i < NT; ++i)
-              acc[u][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[u][i], xf, acc[u][i], 0, 0, 0);   // rows: rank index, cols: tokens
+              acc[u][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[s][u][i], xf[s], acc[u][i], 0, 0, 0);   // rows: rank index, cols: tokens
           }
+        }
+      };
+      int kb = kb0 + wave;
+      if (kb < kb1) load(0, kb);
+      for (; kb < kb1; kb += 2 * SEG_WAVES) {
+        load(1, kb + SEG_WAVES);
+        multiply(0);
+        if (kb + SEG_WAVES < kb1) {
+          load(0, kb + 2 * SEG_WAVES);
+          multiply(1);
         }
       }
 #pragma unroll
@@ -606,19 +620,33 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE, 2) void lora_shrink_quad_mfma_ker
   for (int u = 0; u < QT; ++u)
 #pragma unroll
     for (int i = 0; i < NT; ++i) acc[u][i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int kb = kb0 + wave; kb < kb1; kb += SEG_WAVES) {
-    f16x8 af[NT], xf[QT];
+  // two register sets: the k-step after this one is requested before this one is multiplied
+  f16x8 af[2][NT], xf[2][QT];
+  auto load = [&](int s, int kb) {
+    const int kk = kb < kb1 ? kb : kb1 - 1;      // past the range: a valid address, the data is not multiplied
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
       const int row = i * 16 + col;
-      af[i] = row < R ? ld8(Aa + (size_t)row * K + kb * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      af[s][i] = row < R ? ld8(Aa + (size_t)row * K + kk * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
 #pragma unroll
-    for (int u = 0; u < QT; ++u) xf[u] = ld8(xr[u] + (size_t)kb * xstep);
+    for (int u = 0; u < QT; ++u) xf[s][u] = ld8(xr[u] + (size_t)kk * xstep);
+  };
+  auto multiply = [&](int s) {
 #pragma unroll
     for (int u = 0; u < QT; ++u)
 #pragma unroll
-      for (int i = 0; i < NT; ++i) acc[u][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], xf[u], acc[u][i], 0, 0, 0);
+      for (int i = 0; i < NT; ++i) acc[u][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[s][i], xf[s][u], acc[u][i], 0, 0, 0);
+  };
+  int kb = kb0 + wave;
+  if (kb < kb1) load(0, kb);
+  for (; kb < kb1; kb += 2 * SEG_WAVES) {
+    load(1, kb + SEG_WAVES);
+    multiply(0);
+    if (kb + SEG_WAVES < kb1) {
+      load(0, kb + 2 * SEG_WAVES);
+      multiply(1);
+    }
   }
   // the four waves' sums, tile by tile, added in wave order; wave w stores A-tile i = w, w + 4, ... of the token tile
 #pragma unroll
