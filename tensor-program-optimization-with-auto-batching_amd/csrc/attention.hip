@@ -651,28 +651,33 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// Prefill: four waves own 64 consecutive query tokens of one head, a wave 16 of them.  S^T = K . Q^T on
-// v_mfma_f32_16x16x32_f16 puts the key index on the accumulator rows, which is exactly the A-operand layout the matrix
+// Prefill: four waves own 128 consecutive query tokens of one head, a wave 32 of them as two 16-query tiles.  S^T = K . Q^T
+// on v_mfma_f32_16x16x32_f16 puts the key index on the accumulator rows, which is exactly the A-operand layout the matrix
 // core wants for P in O = P . V (a lane's four accumulator rows are the four keys it must supply): no shuffles between
 // the two products.  The keys are walked in blocks of 64 (four pages).  The block's K and V pages go from the cache
 // straight into LDS (a page per wave; a head's page of K or V is 4 KiB contiguous in the cache), double buffered - the
 // next block is in flight while this one is multiplied - with one barrier per block, and all waves take their
-// fragments from there: a page is fetched once per 64 queries.  Two workgroups share a compute unit.  The softmax
-// bookkeeping (running maximum, rescaling of O, the fp16 hi + lo split of P) is done once per 64 keys, and a P . V
+// fragments from there: a page is fetched once per 128 queries, and a K or V fragment read from LDS is multiplied with
+// both of the wave's query tiles - with one tile per wave the LDS reads (32 KiB per wave and block for 48 MFMAs) were
+// what the kernel waited for, and more waves per SIMD only made that worse.  Two workgroups share a compute unit.  The
+// softmax bookkeeping (running maximum, rescaling of O, the fp16 hi + lo split of P) is done once per 64 keys and tile
+// - the two tiles' chains are independent, which gives the scheduler something to fill the waits with - and a P . V
 // product covers 32 keys per MFMA (k-slots 0-3 and 4-7 of a lane are its four keys of two pages), hi and lo halves of
-// P in two MFMAs on the same V fragment.  Blocks above the causal diagonal of a wave are skipped by that wave; blocks
+// P in two MFMAs on the same V fragment.  Blocks above the causal diagonal of a tile are skipped by that tile; blocks
 // below it need no mask.  Token blocks that span several sequences are worked off one sequence at a time with the
 // other queries masked.  The results cross LDS once more to leave as whole 16-byte pieces.
-// (Eight waves per workgroup with a four-deep ring, and adding P . V of the previous block under the softmax
-// arithmetic of the current one, were measured and are no faster: 8 x 512 tokens, 32 heads of 128 take 115-120 us in
-// every form, about 0.2 PFLOP/s of causal QK^T + PV.)
+// (8 x 512 tokens, 32 heads of 128: 90 us, 0.19 PFLOP/s of causal QK^T + PV; one sequence of 4096: 550 us, 0.25.  With one
+// query tile per wave: 121 and 599 us; that form with eight waves per workgroup and four waves per SIMD: 102 and 655;
+// with 32-key blocks and a four-deep ring: 134 and 732; adding P . V of the previous block under the softmax arithmetic
+// of the current one: no faster.)
 // ---------------------------------------------------------------------------------------------
 constexpr int PF_WAVES = 4;
+constexpr int PF_QT = 2;         // 16-query tiles per wave: a K or V fragment read from LDS serves that many MFMAs
 constexpr int PF_PAGES = 4;      // pages per key block
 constexpr int PF_RING = 2;       // key-block buffers
 
 template <int D>
-__global__ __launch_bounds__(PF_WAVES* WAVE) void paged_attn_prefill_block_kernel(
+__global__ __launch_bounds__(PF_WAVES* WAVE, 2) void paged_attn_prefill_block_kernel(
     f16* __restrict__ out, int frag_tt, const f16* __restrict__ qkv, const f16* __restrict__ k_cache, const f16* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
     int T, int Hq, int Hkv, int n_pages, int n_seq, float scale) {
@@ -684,14 +689,17 @@ __global__ __launch_bounds__(PF_WAVES* WAVE) void paged_attn_prefill_block_kerne
   constexpr int HC = CH / WPP;               // 1 KiB pieces of K (and of V) a wave fetches per block
   constexpr int BUF = 2 * PF_PAGES * PE;     // one buffer: K pages, then V pages
   constexpr int OLD = D + 8;                 // padded row of the output staging
-  constexpr int NTOK = PF_WAVES * 16;
+  constexpr int QT = PF_QT;                  // 16-query tiles of a wave
+  constexpr int WTOK = 16 * QT;              // queries of a wave
+  constexpr int NTOK = PF_WAVES * WTOK;
   static_assert(PF_WAVES % PF_PAGES == 0 && CH % WPP == 0 && NTOK <= 2 * WAVE, "whole waves per page; at most two tokens per lane in the sequence scan");
+  static_assert((size_t)NTOK * OLD <= (size_t)PF_RING * BUF, "the output staging fits the ring");
   extern __shared__ __align__(16) f16 smem[];   // [PF_RING][BUF]
   __shared__ int s_seq[NTOK], s_pos[NTOK];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int qi = lane & 15, g = lane >> 4;
   const int t0 = (gridDim.x - 1 - blockIdx.x) * NTOK;              // late token blocks (long key ranges) start first
-  const int tw = t0 + wave * 16;
+  const int tw = t0 + wave * WTOK;
   const int h = blockIdx.y, kh = h / (Hq / Hkv);
 
   // the V slots start at zero: a slot whose page is never fetched (a sequence shorter than a key block) is multiplied
@@ -700,31 +708,42 @@ __global__ __launch_bounds__(PF_WAVES* WAVE) void paged_attn_prefill_block_kerne
     const int bsel = i / (PF_PAGES * PE / 8), o = i % (PF_PAGES * PE / 8);
     st8(smem + bsel * BUF + PF_PAGES * PE + o * 8, f16x8{0, 0, 0, 0, 0, 0, 0, 0});
   }
-  if (threadIdx.x < NTOK) {
-    const int t = t0 + threadIdx.x;
+  for (int i = threadIdx.x; i < NTOK; i += PF_WAVES * WAVE) {
+    const int t = t0 + i;
     int sq = t < T ? tok_seq[t] : -1;
     int ps = t < T ? tok_pos[t] : -1;
     if (sq < 0 || sq >= n_seq || ps < 0 || ps >= max_blocks * PAGE) sq = -1;
-    s_seq[threadIdx.x] = sq;
-    s_pos[threadIdx.x] = ps;
+    s_seq[i] = sq;
+    s_pos[i] = ps;
   }
   __syncthreads();
   const int seq_a = s_seq[lane], pos_a = s_pos[lane];                // token t0 + lane
   const int seq_b = WAVE + lane < NTOK ? s_seq[(WAVE + lane) % NTOK] : -1, pos_b = s_pos[(WAVE + lane) % NTOK];   // token t0 + 64 + lane
-  const int my_seq = s_seq[wave * 16 + qi], my_pos = s_pos[wave * 16 + qi];
+  int my_seq[QT], my_pos[QT];
+#pragma unroll
+  for (int u = 0; u < QT; ++u) {
+    my_seq[u] = s_seq[wave * WTOK + u * 16 + qi];
+    my_pos[u] = s_pos[wave * WTOK + u * 16 + qi];
+  }
 
-  f16x8 qf[NKB];                             // Q as the B operand: q[query qi][kb * 32 + g * 8 ..]
-  {
-    const int tq = tw + qi < T ? tw + qi : T - 1;
+  f16x8 qf[QT][NKB];                         // Q as the B operand: q[query qi of tile u][kb * 32 + g * 8 ..]
+#pragma unroll
+  for (int u = 0; u < QT; ++u) {
+    const int tq = tw + u * 16 + qi < T ? tw + u * 16 + qi : T - 1;
     const f16* qp = qkv + ((size_t)tq * (Hq + 2 * Hkv) + h) * D + g * 8;
 #pragma unroll
-    for (int kb = 0; kb < NKB; ++kb) qf[kb] = ld8(qp + kb * 32);
+    for (int kb = 0; kb < NKB; ++kb) qf[u][kb] = ld8(qp + kb * 32);
   }
   const float c = scale * 1.44269504088896340736f;                  // softmax in base 2
-  float m = -INFINITY, l = 0.f;
-  f32x4 O[NDB];
+  float m[QT], l[QT];
+  f32x4 O[QT][NDB];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) O[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int u = 0; u < QT; ++u) {
+    m[u] = -INFINITY;
+    l[u] = 0.f;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) O[u][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
   unsigned long long todo_a = __ballot(seq_a >= 0), todo_b = __ballot(seq_b >= 0);
   while (todo_a | todo_b) {                                          // one pass per sequence of the token block (uniform over the workgroup)
@@ -737,19 +756,27 @@ __global__ __launch_bounds__(PF_WAVES* WAVE) void paged_attn_prefill_block_kerne
     for (int o = 32; o > 0; o >>= 1) run_max = max(run_max, __shfl_xor(run_max, o, WAVE));
     run_max = __builtin_amdgcn_readfirstlane(run_max);
     const int npages = run_max / PAGE + 1, nblk = (npages + PF_PAGES - 1) / PF_PAGES;
-    const bool in_run = my_seq == cur;
-    int wmax = in_run ? my_pos : -1, wmin = in_run ? my_pos : 0x7fffffff;
+    // per query tile: is it part of this sequence, and between which positions do its queries lie
+    bool in_run[QT], all_in[QT];
+    int tmax[QT], tmin[QT];
+    int wmax = -1;
 #pragma unroll
-    for (int o = 8; o > 0; o >>= 1) {
-      wmax = max(wmax, __shfl_xor(wmax, o, WAVE));
-      wmin = min(wmin, __shfl_xor(wmin, o, WAVE));
+    for (int u = 0; u < QT; ++u) {
+      in_run[u] = my_seq[u] == cur;
+      int hi = in_run[u] ? my_pos[u] : -1, lo = in_run[u] ? my_pos[u] : 0x7fffffff;
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) {
+        hi = max(hi, __shfl_xor(hi, o, WAVE));
+        lo = min(lo, __shfl_xor(lo, o, WAVE));
+      }
+      tmax[u] = __builtin_amdgcn_readfirstlane(hi);                  // lanes 0-15 hold the 16 queries; all g copies agree
+      tmin[u] = __builtin_amdgcn_readfirstlane(lo);
+      all_in[u] = (__ballot(in_run[u]) & 0xffffull) == 0xffffull;
+      wmax = max(wmax, tmax[u]);
     }
-    wmax = __builtin_amdgcn_readfirstlane(wmax);                   // lanes 0-15 hold the 16 queries; all g copies agree
-    wmin = __builtin_amdgcn_readfirstlane(wmin);
-    const bool all_in = (__ballot(in_run) & 0xffffull) == 0xffffull;
     const int32_t* __restrict__ bt = block_table + (size_t)cur * max_blocks;
 
-    // this wave's half page of block b into its ring slot: HC pieces of K and HC pieces of V, always - a page past the
+    // this wave's part of block b into its ring slot: HC pieces of K and HC pieces of V, always - a page past the
     // sequence or outside the cache is replaced by page 0 (finite data; every key of it is masked), so that the
     // number of loads in flight tells which blocks have landed
     auto issue = [&](int b) {
@@ -790,7 +817,7 @@ __global__ __launch_bounds__(PF_WAVES* WAVE) void paged_attn_prefill_block_kerne
       if (wmax < b * PF_PAGES * PAGE) continue;                      // wave-uniform: the block lies above this wave's diagonal
       const f16* kb_ = smem + (b % PF_RING) * BUF;
       const f16* vb_ = kb_ + PF_PAGES * PE;
-      // All four pages are multiplied without branches; what must not count is masked after the product.  A page that
+      // All pages are multiplied without branches; what must not count is masked after the product.  A page that
       // was not fetched (past the sequence, or a page id outside the cache) leaves older, finite data in its slot.
       bool live[PF_PAGES];                                           // uniform
       bool all_live = true;
@@ -801,23 +828,79 @@ __global__ __launch_bounds__(PF_WAVES* WAVE) void paged_attn_prefill_block_kerne
         live[p] = page >= 0 && page < n_pages;
         all_live = all_live && live[p];
       }
-      // Fragment reads go out in groups ahead of the MFMAs that use them (two waves per SIMD hide little LDS latency
-      // otherwise): all K fragments of the block, then - before the softmax arithmetic - the V fragments of the first
-      // page pair.
-      f16x8 kf[PF_PAGES][NKB];
+      bool act[QT];                                                  // uniform: the tile has queries at or below the block
 #pragma unroll
-      for (int p = 0; p < PF_PAGES; ++p)
+      for (int u = 0; u < QT; ++u) act[u] = tmax[u] >= b * PF_PAGES * PAGE;
+      // S^T of the block for the wave's query tiles: a K fragment is read from LDS once and multiplied with every tile
+      f32x4 st[QT][PF_PAGES];                                        // st[u][p][r] = S[key 4g + r of page p][query qi of tile u]
 #pragma unroll
-        for (int kb = 0; kb < NKB; ++kb) kf[p][kb] = ld8(kb_ + p * PE + kb * 512 + lane * 8);
-      __builtin_amdgcn_sched_barrier(0);
-      f32x4 st[PF_PAGES];                                            // st[p][r] = S[key 4g + r of page p][query qi]
+      for (int u = 0; u < QT; ++u)
 #pragma unroll
-      for (int p = 0; p < PF_PAGES; ++p) st[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int p = 0; p < PF_PAGES; ++p) st[u][p] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kb = 0; kb < NKB; ++kb)
+      for (int p = 0; p < PF_PAGES; ++p) {
+        f16x8 kf[NKB];
 #pragma unroll
-        for (int p = 0; p < PF_PAGES; ++p) st[p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[p][kb], qf[kb], st[p], 0, 0, 0);
-      auto load_v = [&](f16x8 (&vv)[NDB], int pp) {                  // dim db * 16 + qi, keys 4g .. of the pair's two pages
+        for (int kb = 0; kb < NKB; ++kb) kf[kb] = ld8(kb_ + p * PE + kb * 512 + lane * 8);
+#pragma unroll
+        for (int u = 0; u < QT; ++u) {
+          if (act[u]) {
+#pragma unroll
+            for (int kb = 0; kb < NKB; ++kb) st[u][p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kb], qf[u][kb], st[u][p], 0, 0, 0);
+          }
+        }
+      }
+      // online softmax per tile; P as fp16 hi + lo halves (~22 mantissa bits): hi is P rounded to fp16, lo the remainder
+      f16x8 ph[QT][PF_PAGES / 2], pl[QT][PF_PAGES / 2];
+#pragma unroll
+      for (int u = 0; u < QT; ++u) {
+        if (!act[u]) continue;
+        if (!(all_in[u] && all_live && (b + 1) * PF_PAGES * PAGE - 1 <= tmin[u])) {   // uniform: some key of the block is masked
+#pragma unroll
+          for (int p = 0; p < PF_PAGES; ++p) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const bool masked = !live[p] || !in_run[u] || (b * PF_PAGES + p) * PAGE + 4 * g + r > my_pos[u];
+              st[u][p][r] = masked ? -INFINITY : st[u][p][r];
+            }
+          }
+        }
+        float pm = fmaxf(fmaxf(st[u][0][0], st[u][0][1]), fmaxf(st[u][0][2], st[u][0][3]));
+#pragma unroll
+        for (int p = 1; p < PF_PAGES; ++p) pm = fmaxf(pm, fmaxf(fmaxf(st[u][p][0], st[u][p][1]), fmaxf(st[u][p][2], st[u][p][3])));
+        pm = fmaxf(pm, __shfl_xor(pm, 16, WAVE));
+        pm = fmaxf(pm, __shfl_xor(pm, 32, WAVE));
+        const float m_new = fmaxf(m[u], pm);
+        const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((m[u] - m_new) * c);
+        const float mc = m_new == -INFINITY ? 0.f : m_new * c;
+        float ps = 0.f;
+#pragma unroll
+        for (int p = 0; p < PF_PAGES; ++p) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float pr = __builtin_amdgcn_exp2f(fmaf(st[u][p][r], c, -mc));   // exp2(-inf) = 0 for masked keys
+            ps += pr;
+            const f16 hi = (f16)pr;
+            ph[u][p / 2][(p & 1) * 4 + r] = hi;
+            pl[u][p / 2][(p & 1) * 4 + r] = (f16)(pr - (float)hi);
+          }
+        }
+        l[u] = l[u] * alpha + ps;
+        m[u] = m_new;
+        float ar[4];                                                 // O rows are queries 4g + r; their alpha lives in lanes with qi == 4g + r
+#pragma unroll
+        for (int r = 0; r < 4; ++r) ar[r] = __shfl(alpha, 4 * g + r, WAVE);
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) O[u][db][r] *= ar[r];
+      }
+      // O += P . V: a V fragment (dim db * 16 + qi, keys 4g .. of the pair's two pages) is read once for all tiles
+      static_assert(PF_PAGES % 2 == 0, "page pairs");
+#pragma unroll
+      for (int pp = 0; pp < PF_PAGES / 2; ++pp) {
+        __builtin_amdgcn_sched_barrier(0);                           // the V fragments are not requested before they fit the register file
+        f16x8 vv[NDB];
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
           const f16* v0 = vb_ + (2 * pp) * PE + (db * 16 + qi) * PAGE + g * 4;
@@ -825,87 +908,48 @@ __global__ __launch_bounds__(PF_WAVES* WAVE) void paged_attn_prefill_block_kerne
           const f16x4 vb = *reinterpret_cast<const f16x4*>(v0 + PE);
           vv[db] = __builtin_shufflevector(va, vb, 0, 1, 2, 3, 4, 5, 6, 7);
         }
-      };
-      f16x8 vv0[NDB], vv1[NDB];
-      load_v(vv0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      if (!(all_in && all_live && (b + 1) * PF_PAGES * PAGE - 1 <= wmin)) {   // uniform: some key of the block is masked
 #pragma unroll
-        for (int p = 0; p < PF_PAGES; ++p) {
+        for (int u = 0; u < QT; ++u) {
+          if (!act[u]) continue;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const bool masked = !live[p] || !in_run || (b * PF_PAGES + p) * PAGE + 4 * g + r > my_pos;
-            st[p][r] = masked ? -INFINITY : st[p][r];
-          }
+          for (int db = 0; db < NDB; ++db) O[u][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ph[u][pp], vv[db], O[u][db], 0, 0, 0);
+#pragma unroll
+          for (int db = 0; db < NDB; ++db) O[u][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl[u][pp], vv[db], O[u][db], 0, 0, 0);
         }
       }
-      float pm = fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3]));
-#pragma unroll
-      for (int p = 1; p < PF_PAGES; ++p) pm = fmaxf(pm, fmaxf(fmaxf(st[p][0], st[p][1]), fmaxf(st[p][2], st[p][3])));
-      pm = fmaxf(pm, __shfl_xor(pm, 16, WAVE));
-      pm = fmaxf(pm, __shfl_xor(pm, 32, WAVE));
-      const float m_new = fmaxf(m, pm);
-      const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((m - m_new) * c);
-      const float mc = m_new == -INFINITY ? 0.f : m_new * c;
-      // P as fp16 hi + lo halves (~22 mantissa bits): hi is P rounded to fp16, lo the remainder
-      f16x8 ph[PF_PAGES / 2], pl[PF_PAGES / 2];
-      float ps = 0.f;
-#pragma unroll
-      for (int p = 0; p < PF_PAGES; ++p) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float pr = __builtin_amdgcn_exp2f(fmaf(st[p][r], c, -mc));   // exp2(-inf) = 0 for masked keys
-          ps += pr;
-          const f16 hi = (f16)pr;
-          ph[p / 2][(p & 1) * 4 + r] = hi;
-          pl[p / 2][(p & 1) * 4 + r] = (f16)(pr - (float)hi);
-        }
-      }
-      l = l * alpha + ps;
-      m = m_new;
-      float ar[4];                                                   // O rows are queries 4g + r; their alpha lives in lanes with qi == 4g + r
-#pragma unroll
-      for (int r = 0; r < 4; ++r) ar[r] = __shfl(alpha, 4 * g + r, WAVE);
-#pragma unroll
-      for (int db = 0; db < NDB; ++db)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) O[db][r] *= ar[r];
-      static_assert(PF_PAGES == 4, "two page pairs");
-      load_v(vv1, 1);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int db = 0; db < NDB; ++db) O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ph[0], vv0[db], O[db], 0, 0, 0);
-#pragma unroll
-      for (int db = 0; db < NDB; ++db) O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl[0], vv0[db], O[db], 0, 0, 0);
-#pragma unroll
-      for (int db = 0; db < NDB; ++db) O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ph[1], vv1[db], O[db], 0, 0, 0);
-#pragma unroll
-      for (int db = 0; db < NDB; ++db) O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl[1], vv1[db], O[db], 0, 0, 0);
     }
     __syncthreads();                                                 // the buffers are free for the next sequence (and for the output)
   }
-  l += __shfl_xor(l, 16, WAVE);
-  l += __shfl_xor(l, 32, WAVE);
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  // results through the wave's own piece of LDS: [16 queries][D] fp16, then 16-byte pieces out
-  f16* os = smem + wave * 16 * OLD;
+  // results through the wave's own piece of LDS: [16 QT queries][D] fp16, then 16-byte pieces out
+  f16* os = smem + wave * WTOK * OLD;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const float ir = __shfl(inv, 4 * g + r, WAVE);
+  for (int u = 0; u < QT; ++u) {
+    float lu = l[u];
+    lu += __shfl_xor(lu, 16, WAVE);
+    lu += __shfl_xor(lu, 32, WAVE);
+    const float inv = lu > 0.f ? 1.f / lu : 0.f;
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) os[(4 * g + r) * OLD + db * 16 + qi] = (f16)(O[db][r] * ir);
+    for (int r = 0; r < 4; ++r) {
+      const float ir = __shfl(inv, 4 * g + r, WAVE);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) os[(u * 16 + 4 * g + r) * OLD + db * 16 + qi] = (f16)(O[u][db][r] * ir);
+    }
   }
   __builtin_amdgcn_wave_barrier();
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   if (frag_tt) {
 #pragma unroll
-    for (int j = 0; j < D / 32; ++j) {                               // one whole fragment per store instruction
-      const int tok = lane & 15, kg = lane >> 4;
-      if (tw + tok < T) st8(out + frag_offset(tw + tok, h * D + j * 32 + kg * 8, frag_tt), ld8(os + tok * OLD + j * 32 + kg * 8));
+    for (int u = 0; u < QT; ++u) {
+#pragma unroll
+      for (int j = 0; j < D / 32; ++j) {                             // one whole fragment per store instruction
+        const int tok = lane & 15, kg = lane >> 4;
+        const int t = tw + u * 16 + tok;
+        if (t < T) st8(out + frag_offset(t, h * D + j * 32 + kg * 8, frag_tt), ld8(os + (u * 16 + tok) * OLD + j * 32 + kg * 8));
+      }
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < 16 * (D / 8) / WAVE; ++i) {
+    for (int i = 0; i < WTOK * (D / 8) / WAVE; ++i) {
       const int ch = i * WAVE + lane, row = ch / (D / 8), c8 = ch % (D / 8);
       if (tw + row < T) st8(out + ((size_t)(tw + row) * Hq + h) * D + c8 * 8, ld8(os + row * OLD + c8 * 8));
     }
@@ -1083,7 +1127,7 @@ extern "C" int mlora_paged_attn_prefill(void* out, int out_layout, const void* q
   const int frag_tt = out_layout == MLORA_FRAG ? mlora_frag_tiles(T) : 0;
   const float scale = 1.f / sqrtf((float)D);
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid(ceil_div(T, PF_WAVES * 16), Hq);
+  const dim3 grid(ceil_div(T, PF_WAVES * 16 * PF_QT), Hq);
 #define MLORA_PREFILL(DD)                                                                                                          \
   do {                                                                                                                             \
     constexpr size_t lds = (size_t)PF_RING * 2 * PF_PAGES * PAGE * DD * sizeof(f16);                                                    \
