@@ -669,8 +669,8 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
 // Workgroups are dispatched longest key range first over all heads (grid = (heads, token blocks), late token blocks
 // first): with the token block as the fast grid dimension the long workgroups of the last heads started late and ran
 // alone at the end - 0.9 resident waves per SIMD on average, 551 instead of 336 us for one sequence of 4096 tokens.
-// (8 x 512 tokens, 32 heads of 128: 77 us, 0.22 PFLOP/s of causal QK^T + PV; one sequence of 4096: 336 us, 0.41.  Before the
-// dispatch order was changed: 90 and 551 us; with one query tile per wave on top of that: 121 and 599 us; that form with eight waves per workgroup and four waves per SIMD: 102 and 655;
+// (8 x 512 tokens, 32 heads of 128: 73 us, 0.24 PFLOP/s of causal QK^T + PV; one sequence of 4096: 315 us, 0.44.  With O and l
+// rescaled in every block: 77 and 336 us; before the dispatch order was changed: 90 and 551 us; with one query tile per wave on top of that: 121 and 599 us; that form with eight waves per workgroup and four waves per SIMD: 102 and 655;
 // with 32-key blocks and a four-deep ring: 134 and 732; adding P . V of the previous block under the softmax arithmetic
 // of the current one: no faster.)
 // ---------------------------------------------------------------------------------------------
@@ -875,9 +875,25 @@ __global__ __launch_bounds__(PF_WAVES* WAVE, 2) void paged_attn_prefill_block_ke
         for (int p = 1; p < PF_PAGES; ++p) pm = fmaxf(pm, fmaxf(fmaxf(st[u][p][0], st[u][p][1]), fmaxf(st[u][p][2], st[u][p][3])));
         pm = fmaxf(pm, __shfl_xor(pm, 16, WAVE));
         pm = fmaxf(pm, __shfl_xor(pm, 32, WAVE));
-        const float m_new = fmaxf(m[u], pm);
-        const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((m[u] - m_new) * c);
-        const float mc = m_new == -INFINITY ? 0.f : m_new * c;
+        // The reference maximum m moves - and O and l are rescaled - only when some query of the tile meets a score more
+        // than 2^8 above it (always in the tile's first block); otherwise the block's P are taken relative to the old
+        // reference and may reach 256, which fp16 holds exactly as well.  After the first blocks of a sequence that
+        // saves the rescaling arithmetic (32 multiplies, four cross-lane moves, an exponential) of almost every block.
+        const bool need = (pm - m[u]) * c > 8.f;                     // m = -inf: true for a finite pm, false (NaN) for pm = -inf
+        if (__ballot(need)) {                                        // wave-uniform
+          const float m_new = fmaxf(m[u], pm);
+          const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((m[u] - m_new) * c);
+          l[u] *= alpha;
+          m[u] = m_new;
+          float ar[4];                                               // O rows are queries 4g + r; their alpha lives in lanes with qi == 4g + r
+#pragma unroll
+          for (int r = 0; r < 4; ++r) ar[r] = __shfl(alpha, 4 * g + r, WAVE);
+#pragma unroll
+          for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) O[u][db][r] *= ar[r];
+        }
+        const float mc = m[u] == -INFINITY ? 0.f : m[u] * c;
         float ps = 0.f;
 #pragma unroll
         for (int p = 0; p < PF_PAGES; ++p) {
@@ -890,15 +906,7 @@ __global__ __launch_bounds__(PF_WAVES* WAVE, 2) void paged_attn_prefill_block_ke
             pl[u][p / 2][(p & 1) * 4 + r] = (f16)(pr - (float)hi);
           }
         }
-        l[u] = l[u] * alpha + ps;
-        m[u] = m_new;
-        float ar[4];                                                 // O rows are queries 4g + r; their alpha lives in lanes with qi == 4g + r
-#pragma unroll
-        for (int r = 0; r < 4; ++r) ar[r] = __shfl(alpha, 4 * g + r, WAVE);
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) O[u][db][r] *= ar[r];
+        l[u] += ps;
       }
       // O += P . V: a V fragment (dim db * 16 + qi, keys 4g .. of the pair's two pages) is read once for all tiles
       static_assert(PF_PAGES % 2 == 0, "page pairs");
