@@ -113,13 +113,14 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qk
   }
 }
 
-// Prefill-sized variant that moves 16 bytes at a time: one WAVE per (16 consecutive tokens, head of q / k / v), four heads per
-// workgroup, no barriers.  Lane l owns the sequence and position of token l % 16 of the tile and hands them to the lanes
-// that work on that token; the lanes of a load cover whole half rows of a head (128 contiguous bytes at D = 128), so every
-// cache line is consumed by the instruction that fetches it.  q heads are rotated in place in chunks of 8 pairs.  When
-// the 16 tokens are slots 0..15 of one page (prompts that start on a page boundary), K leaves as 16-byte pieces of its
-// fragment chunk rows and V is transposed through LDS into the page's contiguous [D][16] block; other tiles fall back to
-// element-wise writes.  Measured at 4096 tokens, D = 128: 32 + 2 x 32 heads 37 us (5.4 TB/s), 32 + 2 x 8 heads 22 us; the
+// Variant for more than 64 tokens that moves 16 bytes at a time: one WAVE per (16 consecutive tokens, head of q / k / v),
+// four heads per workgroup, no barriers.  Lane l owns the sequence, position and cache page of token l % 16 of the tile and
+// hands them to the lanes that work on that token; the lanes of a load cover whole half rows of a head (128 contiguous
+// bytes at D = 128), so every cache line is consumed by the instruction that fetches it.  q heads are rotated in place in
+// chunks of 8 pairs.  A rotated K chunk is one 16-byte piece of its token's page (fragment order), wherever the token
+// lies.  V of a tile that is slots 0..15 of one page (prompts that start on a page boundary) is transposed through LDS
+// into the page's contiguous [D][16] block; V of other tiles (a decode step: every token its own sequence) goes out
+// element by element.  Measured at 4096 prompt tokens, D = 128: 32 + 2 x 32 heads 37 us (5.4 TB/s), 32 + 2 x 8 heads 22 us; the
 // earlier mapping (a lane kept one token, 64-byte pieces per token and load, V gathered 2 bytes at a time) took 53 / 31 us.
 // Same arithmetic per element as rope_kv_append_kernel.  rope_cos / rope_sin must be 16-byte aligned.
 template <int D>
@@ -197,29 +198,38 @@ __global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restric
   }
   const bool is_v = hh >= Hq + Hkv;                           // wave-uniform
   const int kh = is_v ? hh - Hq - Hkv : hh - Hq;
-  const int seq0 = __shfl(seq, 0, WAVE), pos0 = __shfl(pos, 0, WAVE);
-  bool al = __ballot(seq >= 0 && seq == seq0 && pos == pos0 + tk) == ~0ull && (pos0 % PAGE) == 0;   // wave-uniform
-  int page = -1;
-  if (al) {
-    page = block_table[(size_t)seq0 * max_blocks + pos0 / PAGE];
-    if (page < 0 || page >= n_pages) al = false;
+  // the cache page of the lane's own token (-1: nothing to store), then of the tokens the lane works on
+  int page_own = -1;
+  if (seq >= 0) {
+    page_own = block_table[(size_t)seq * max_blocks + pos / PAGE];
+    if (page_own >= n_pages) page_own = -1;
   }
-  if (al && !is_v) {
-    // K: a fragment chunk row holds the 16 tokens' 16-byte pieces side by side
-    f16* kd = k_cache + ((size_t)page * Hkv + kh) * PAGE * D;
+  int pagej[NPASS];
+#pragma unroll
+  for (int j = 0; j < NPASS; ++j) pagej[j] = __shfl(page_own, tkj[j], WAVE);
+  if (!is_v) {
+    // K: a token's chunk of 8 elements is one 16-byte piece of its page's fragment rows (the pieces of a page's 16
+    // tokens lie side by side: a tile that is one whole page writes whole lines)
 #pragma unroll
     for (int j = 0; j < NPASS; ++j) {
+      if (pagej[j] < 0) continue;
       const f16* ksrc = qkv + ((size_t)(t0 + tkj[j]) * HH + Hq + kh) * D;
+      f16* kd = k_cache + ((size_t)pagej[j] * Hkv + kh) * PAGE * D;
+      const int slot = posj[j] % PAGE;
       f16x8 o_lo, o_hi;
       rot_chunk(ksrc, posj[j], ch, o_lo, o_hi);
-      st8(kd + ((size_t)ch * 16 + tkj[j]) * 8, o_lo);
-      st8(kd + ((size_t)(ch + NCH) * 16 + tkj[j]) * 8, o_hi);
+      st8(kd + ((size_t)ch * 16 + slot) * 8, o_lo);
+      st8(kd + ((size_t)(ch + NCH) * 16 + slot) * 8, o_hi);
     }
     return;
   }
+  const int seq0 = __shfl(seq, 0, WAVE), pos0 = __shfl(pos, 0, WAVE);
+  const bool al = __ballot(page_own >= 0 && seq == seq0 && pos == pos0 + tk) == ~0ull && (pos0 % PAGE) == 0;   // wave-uniform
   if (al) {
-    // V: the 16 x D tile is transposed through the wave's own LDS rows (row stride 20 elements: the 2-byte writes
-    // of a pass spread over the banks, the 8-byte reads stay aligned), then leaves as one contiguous 32 D bytes.
+    // V of a tile that is one whole page: the 16 x D tile is transposed through the wave's own LDS rows (row stride 20
+    // elements: the 2-byte writes of a pass spread over the banks, the 8-byte reads stay aligned), then leaves as the
+    // page's contiguous 32 D bytes.
+    const int page = __shfl(page_own, 0, WAVE);
     f16(*vt)[VT_LD] = vts[wave];
 #pragma unroll
     for (int j = 0; j < NPASS; ++j) {
@@ -246,26 +256,24 @@ __global__ __launch_bounds__(256) void rope_kv_append_tile_kernel(f16* __restric
     }
     return;
   }
-  for (int it = lane; it < 16 * half; it += WAVE) {           // element-wise: tokens of several pages or sequences
-    const int tke = it / half, i = it % half;
-    const int seq_e = __shfl(seq, tke, WAVE), pos_e = __shfl(pos, tke, WAVE);
-    if (seq_e < 0) continue;
-    const int pg = block_table[(size_t)seq_e * max_blocks + pos_e / PAGE];
-    if (pg < 0 || pg >= n_pages) continue;
-    const int slot = pos_e % PAGE;
-    if (is_v) {
-      const f16* vsrc = qkv + ((size_t)(t0 + tke) * HH + Hq + Hkv + kh) * D;
-      f16* vd = v_cache + ((size_t)pg * Hkv + kh) * D * PAGE + slot;
-      vd[(size_t)i * PAGE] = vsrc[i];
-      vd[(size_t)(i + half) * PAGE] = vsrc[i + half];
-    } else {
-      const f16* ksrc = qkv + ((size_t)(t0 + tke) * HH + Hq + kh) * D;
-      const float c = rope_cos[(size_t)pos_e * half + i], s = rope_sin[(size_t)pos_e * half + i];
-      const float x1 = (float)ksrc[i], x2 = (float)ksrc[i + half];
-      f16* kd = k_cache + ((size_t)pg * Hkv + kh) * PAGE * D;
-      kd[k_page_offset(slot, i)] = rot(x1, x2, c, s, false);
-      kd[k_page_offset(slot, i + half)] = rot(x1, x2, c, s, true);
-    }
+  // V of tokens of several pages or sequences (a decode step: every token its own sequence): element-wise into each
+  // token's slot of its page, all loads of the wave issued before the first store
+  f16x8 xv[NPASS][2];
+#pragma unroll
+  for (int j = 0; j < NPASS; ++j) {
+    const int tl = t0 + tkj[j] < T ? t0 + tkj[j] : T - 1;
+    const f16* vsrc = qkv + ((size_t)tl * HH + Hq + Hkv + kh) * D;
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) xv[j][hf] = ld8(vsrc + hf * half + ch * 8);
+  }
+#pragma unroll
+  for (int j = 0; j < NPASS; ++j) {
+    if (pagej[j] < 0) continue;
+    f16* vd = v_cache + ((size_t)pagej[j] * Hkv + kh) * D * PAGE + posj[j] % PAGE;
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vd[(size_t)(hf * half + ch * 8 + e) * PAGE] = xv[j][hf][e];
   }
 }
 
@@ -704,8 +712,9 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
 // Workgroups are dispatched longest key range first over all heads (grid = (heads, token blocks), late token blocks
 // first): with the token block as the fast grid dimension the long workgroups of the last heads started late and ran
 // alone at the end - 0.9 resident waves per SIMD on average, 551 instead of 336 us for one sequence of 4096 tokens.
-// (8 x 512 tokens, 32 heads of 128: 73 us, 0.24 PFLOP/s of causal QK^T + PV; one sequence of 4096: 315 us, 0.44.  With O and l
-// rescaled in every block: 77 and 336 us; before the dispatch order was changed: 90 and 551 us; with one query tile per wave on top of that: 121 and 599 us; that form with eight waves per workgroup and four waves per SIMD: 102 and 655;
+// (8 x 512 tokens, 32 heads of 128: 71 us, 0.24 PFLOP/s of causal QK^T + PV; one sequence of 4096: 304 us, 0.45.  With the hi half
+// of P rounded to nearest, converted back and subtracted - ten instructions per pair of probabilities instead of six: 73 and 315 us; with O and l
+// rescaled in every block on top of that: 77 and 336 us; before the dispatch order was changed: 90 and 551 us; with one query tile per wave on top of that: 121 and 599 us; that form with eight waves per workgroup and four waves per SIMD: 102 and 655;
 // with 32-key blocks and a four-deep ring: 134 and 732; adding P . V of the previous block under the softmax arithmetic
 // of the current one: no faster.)
 // ---------------------------------------------------------------------------------------------
@@ -933,12 +942,20 @@ __global__ __launch_bounds__(PF_WAVES* WAVE, 2) void paged_attn_prefill_block_ke
 #pragma unroll
         for (int p = 0; p < PF_PAGES; ++p) {
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float pr = __builtin_amdgcn_exp2f(fmaf(st[u][p][r], c, -mc));   // exp2(-inf) = 0 for masked keys
-            ps += pr;
-            const f16 hi = (f16)pr;
-            ph[u][p / 2][(p & 1) * 4 + r] = hi;
-            pl[u][p / 2][(p & 1) * 4 + r] = (f16)(pr - (float)hi);
+          for (int r = 0; r < 4; r += 2) {
+            // hi = P cut to fp16's eleven significant bits (a mask: exact in fp16 down to its normal range), lo = the
+            // exact remainder cut to eleven bits of its own; both pairs leave through one two-element conversion each
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(st[u][p][r], c, -mc));       // exp2(-inf) = 0 for masked keys
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(st[u][p][r + 1], c, -mc));
+            ps += p0;
+            ps += p1;
+            const float h0 = __builtin_bit_cast(float, __builtin_bit_cast(unsigned, p0) & 0xffffe000u);
+            const float h1 = __builtin_bit_cast(float, __builtin_bit_cast(unsigned, p1) & 0xffffe000u);
+            const auto hh = __builtin_amdgcn_cvt_pkrtz(h0, h1), ll = __builtin_amdgcn_cvt_pkrtz(p0 - h0, p1 - h1);
+            ph[u][p / 2][(p & 1) * 4 + r] = hh[0];
+            ph[u][p / 2][(p & 1) * 4 + r + 1] = hh[1];
+            pl[u][p / 2][(p & 1) * 4 + r] = ll[0];
+            pl[u][p / 2][(p & 1) * 4 + r + 1] = ll[1];
           }
         }
         l[u] += ps;
