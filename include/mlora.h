@@ -21,7 +21,9 @@
  *     mlora_write_tensor_part, mlora_linear / mlora_linear_packed / mlora_linear_frag (and the gemv / gemm kernels
  *     they dispatch to), mlora_pack_weight, mlora_pack_activation, mlora_rmsnorm, mlora_silu_mul, mlora_embed,
  *     mlora_argmax, mlora_rope_kv_append, mlora_paged_attn_decode, mlora_paged_attn_prefill, and
- *     mlora_decode_step (one whole decode step from a plan).
+ *     mlora_decode_step (one whole decode step from a plan); for prefill passes whose tokens come in adapter
+ *     segments, mlora_linear_frag_lora and mlora_linear_frag_silu (linear, LoRA delta and - for gate / up - the
+ *     SiLU product in one GEMM).
  *   INTERNAL, the fused forms from "Decode-step variants" down to mlora_rmsnorm_ksplit - the building blocks of
  *     mlora_decode_step, exported so that the Python host can run the same step operator by operator (the parity
  *     tests compare the two bit for bit).  Their argument lists follow the tiling of the kernels (K-range block
@@ -257,6 +259,20 @@ int mlora_lora_shrink_split(void* const* v_hi, void* const* v_lo, const void* x,
                             const int32_t* tok_adapter, float scaling, int T, int K, int r, int n_ad,
                             void* workspace, size_t workspace_bytes, void* stream);
 int mlora_linear_frag_lora(void* y, int y_dtype, int mode, const void* xf, const void* Wp, int T, int K, int N,
+                           const mlora_fused_lora* projs, int n_proj, const int32_t* blk_adapter, int r, void* stream);
+
+/* Gate/up projection of a prefill-sized token block with the SiLU product in the epilogue of the persistent GEMM:
+ *   act = f16( silu(f16(gate)) * f16(up) ),  [gate | up] = xf . Wp^T (+ the LoRA deltas as in mlora_linear_frag_lora),
+ * written in MLORA_FRAG order for the down projection; the [T, 2I] projection output never reaches memory.
+ * Wp is the fragment-ordered fused [2I, K] matrix (gate rows, then up rows) that mlora_linear_frag takes - no second
+ * copy; I % 32 == 0 and mlora_gemm_frag_preferred(T, K, 2I).  n_proj = 0: no adapters (projs, blk_adapter may be NULL).
+ * Otherwise projs names the gate projection (n_begin = 0), the up projection (n_begin = I) or both (n_rows = I each),
+ * and every token of a 256-token block must name the block's adapter blk_adapter[b] or none: a block that mixes
+ * adapters needs its deltas before the SiLU and has to take mlora_linear_frag_lora, mlora_gather_mm and
+ * mlora_silu_mul instead.  Same result bits as those calls in sequence.
+ * Replaces: gate_proj, up_proj, op.silu and the multiply (llama_for_causal_lm.py:35-36) with the LoRA of
+ * lora.py:26-30 on either projection, in one launch. */
+int mlora_linear_frag_silu(void* act, const void* xf, const void* Wp, int T, int K, int I,
                            const mlora_fused_lora* projs, int n_proj, const int32_t* blk_adapter, int r, void* stream);
 
 /* y[t, :] = f16( x[t, :] * rsqrt(mean(x[t, :]^2) + eps) * w )   row-wise, statistics in fp32.

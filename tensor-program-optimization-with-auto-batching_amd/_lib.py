@@ -47,6 +47,7 @@ SIGNATURES = {
     "mlora_lora_block_adapters": (_i, [_p, _p, _p, _i, _i, _p]),
     "mlora_lora_shrink_split": (_i, [_p, _p, _p, _i, _p, _i, _p, _f, _i, _i, _i, _i, _p, _z, _p]),
     "mlora_linear_frag_lora": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p, _i, _p, _i, _p]),
+    "mlora_linear_frag_silu": (_i, [_p, _p, _p, _i, _i, _i, _p, _i, _p, _i, _p]),
     "mlora_gemv_frag_lora": (_i, [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _i, _p, _i, _i, _p]),
     "mlora_gemv_frag_silu": (_i, [_p, _p, _p, _i, _i, _i, _p]),
     "mlora_gemv_frag_split": (_i, [_p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _p]),

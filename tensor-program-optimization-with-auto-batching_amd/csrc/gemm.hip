@@ -18,7 +18,7 @@ int mlora_check_linear(const char* who, const void* y, int y_dtype, int mode, co
 
 namespace {
 
-enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2 };
+enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2, OUT_SILU = 3 };
 
 // compute units of the current device (0 if it cannot be asked), read once
 int gemm_n_cu() {
@@ -297,6 +297,12 @@ __device__ __forceinline__ unsigned long long uniform64(unsigned long long v) {
   return ((unsigned long long)hi << 32) | lo;
 }
 
+// OUT_SILU: Wp is the fused [2 I, K] gate / up matrix (N = 2 I, gate rows first) and the output is
+// act = silu(f16(gate)) * f16(up) [T, I] in fragment order (tiles per 32-k step: x_tt).  A block is 256 tokens x 128
+// channels: the ring slots of a stage hold, for each of the two row groups of waves, four gate tiles and then the four
+// up tiles of the same channels, so that a lane ends up with both halves of its channels and the product never leaves
+// the registers.  LoRA deltas: slot 0 of `lo` is the gate projection, slot 1 the up projection (B == nullptr: not
+// adapted); each rides as its own extra k-steps, in which only that half of a wave's tiles is multiplied.
 // LORA = false is the plain GEMM (lo is ignored)
 template <int OUT, bool LORA>
 __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx, int x_tt,
@@ -306,21 +312,28 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
   constexpr int NW = PP_WAVES;
   constexpr int LQ = 2 * PP_F / NW;            // fragments a wave fetches per stage (4)
   constexpr int WTF = 4;                       // token fragments of a wave's tile (64 tokens)
+  constexpr bool SILU = OUT == OUT_SILU;
+  constexpr int BN = SILU ? PP_F * 8 : PP_F * 16;   // output columns of a block (SILU: channels, each a gate and an up row)
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int nb = gx * gy;
   const int KB = K / 32;
   const int tiles = (N + 15) / 16;
+  const int I = N / 2, itiles = I / 16;        // SILU: channels and their 16-row tiles
   const int G = gridDim.x;
 
   // block number -> (weight-row block, token block)
   auto block_of = [&](int L, int& n0, int& t0) {
     int idx = L;
     if ((nb & 7) == 0 && (G & 7) == 0) idx = (L & 7) * (nb >> 3) + (L >> 3);
-    n0 = (idx / gy) * (PP_F * 16);
+    n0 = (idx / gy) * BN;
     t0 = (idx % gy) * (PP_F * 16);
   };
   // the LoRA part of a block: projection slot and adapter (-1: none), everything uniform
   auto lora_of = [&](int n0, int t0, int& slot) -> int {
+    if constexpr (SILU) {
+      slot = 0;
+      return lo.blk_adapter[t0 / (PP_F * 16)];
+    }
     slot = -1;
 #pragma unroll
     for (int i = 0; i < 3; ++i)
@@ -328,7 +341,9 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
     if (slot < 0) return -1;
     return lo.blk_adapter[t0 / (PP_F * 16)];
   };
-  const int E = LORA ? 2 * (lo.r / 32) : 0;     // extra k-steps of a block with a delta: hi halves, then lo halves
+  const int EP = LORA ? 2 * (lo.r / 32) : 0;    // extra k-steps per projection of a block with a delta: hi halves, then lo halves
+  const bool has_gate = SILU && LORA && lo.B[0] != nullptr;
+  const int E = SILU ? EP * ((lo.B[0] != nullptr) + (lo.B[1] != nullptr)) : EP;
 
   // ---- loader role: wave w fetches fragments 4 w .. 4 w + 3 of every stage (waves 0-3: weights, waves 4-7: tokens)
   const f16* src[LQ];
@@ -338,6 +353,7 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
   const f16* l_src = nullptr;                  // LoRA stages of that block (all uniform): row 0 of the block in B[a] (weight waves) or in v_hi (token waves) ...
   long l_lo = 0;                               // ... the distance from v_hi to v_lo (token waves; 0 for weight waves) ...
   int l_rows = 1;                              // ... and the rows that exist from there on (rows past them repeat the last one; their results are dropped)
+  int l_a = -1, l_n0 = 0, l_t0 = 0;            // SILU: adapter, first channel and first token of that block (the stages' addresses are formed per stage)
   auto load_block = [&](int L) {
     int n0, t0;
     block_of(L < nb ? L : blockIdx.x, n0, t0); // past the last block: valid addresses, the data is never multiplied
@@ -345,8 +361,12 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
     if constexpr (LORA) {
       int slot;
       const int a = L < nb ? lora_of(n0, t0, slot) : -1;
-      if (a >= 0) {
-        load_nst = __builtin_amdgcn_readfirstlane(KB + E);
+      if (a >= 0) load_nst = __builtin_amdgcn_readfirstlane(KB + E);
+      if (SILU) {
+        l_a = a;
+        l_n0 = n0;
+        l_t0 = t0;
+      } else if (a >= 0) {
         const f16* Bt = lo.B[0];
         const f16* vh = lo.vh[0];
         const f16* vl = lo.vl[0];
@@ -374,8 +394,15 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
     if (wave < NW / 2) {
 #pragma unroll
       for (int q = 0; q < LQ; ++q) {
-        int nt = n0 / 16 + wave * LQ + q;
-        nt = nt < tiles ? nt : tiles - 1;      // rows past N: a valid fragment, results dropped
+        int nt;
+        if constexpr (SILU) {                  // slots 8 wn + 0..3: gate tiles of channels n0 + 64 wn .., slots 8 wn + 4..7: their up tiles
+          int it = n0 / 16 + (wave >> 1) * LQ + q;
+          it = it < itiles ? it : itiles - 1;
+          nt = it + (wave & 1) * itiles;
+        } else {
+          nt = n0 / 16 + wave * LQ + q;
+          nt = nt < tiles ? nt : tiles - 1;    // rows past N: a valid fragment, results dropped
+        }
         src[q] = Wp + (size_t)nt * KB * 512 + lane * 8;
       }
       step = 512;
@@ -407,6 +434,31 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
       for (int q = 0; q < LQ; ++q)
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + (size_t)load_kb * step),
                                          (__attribute__((address_space(3))) void*)(dst + q * 512), 16, 0, 0);
+    } else if constexpr (SILU) {               // a LoRA stage of the gate or of the up projection
+      const int j = load_kb - KB, RB = lo.r / 32;
+      const bool up = !(has_gate && j < EP);   // uniform
+      const int jj = has_gate && up ? j - EP : j;
+      const bool lo_half = jj >= RB;
+      const int ks = (lo_half ? jj - RB : jj) * 32;
+      const f16* base;
+      int row0, rows;
+      if (wave < NW / 2) {                     // rows of the projection's table for this wave's channels (used by the waves of that half only)
+        base = (up ? lo.B[1] : lo.B[0]) + (size_t)l_a * I * lo.r;
+        row0 = l_n0 + (wave >> 1) * (LQ * 16);
+        rows = I;
+      } else {
+        base = up ? (lo_half ? lo.vl[1] : lo.vh[1]) : (lo_half ? lo.vl[0] : lo.vh[0]);
+        row0 = l_t0 + (wave & 3) * (LQ * 16);
+        rows = T;
+      }
+#pragma unroll
+      for (int q = 0; q < LQ; ++q) {
+        int row = row0 + q * 16 + (lane & 15);
+        row = row < rows ? row : rows - 1;
+        const f16* p = base + ((size_t)row * lo.r + ks + (lane >> 4) * 8);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p,
+                                         (__attribute__((address_space(3))) void*)(dst + q * 512), 16, 0, 0);
+      }
     } else {                                   // a LoRA stage: 16 rows x 64 bytes per fragment, gathered by the lanes' addresses
       const int j = load_kb - KB, RB = lo.r / 32;
       const int ks = (j < RB ? j : j - RB) * 32;
@@ -444,25 +496,34 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
     for (int i = 0; i < 8; ++i) a[u][i] = ld8(st + (wn * 8 + i) * 512);
     rd = (rd + 1) & (PP_STAGES - 1);
   };
-  auto multiply = [&](auto U) {
+  // half (uniform): -1 all eight row tiles, 0 / 1 the first / last four (a LoRA stage of the gate / up projection)
+  auto multiply = [&](auto U, int half) {
     constexpr int u = decltype(U)::value;
+    if (half != 1) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+      for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < WTF; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][i], b[u][j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < WTF; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][i], b[u][j], acc[i][j], 0, 0, 0);
+    }
+    if (half != 0) {
+#pragma unroll
+      for (int i = 4; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < WTF; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][i], b[u][j], acc[i][j], 0, 0, 0);
+    }
   };
   // One stage: its successor must be in LDS (this wave's share: at most the two stages issued after it still in flight;
   // everybody's: the barrier).  The wait also covers this wave's fragment reads of the stage about to be multiplied,
   // so after the barrier nobody reads that ring slot any more and it is refilled; then the reads of the successor go
   // out, then the MFMAs.
-  auto stage = [&](auto U, auto PLAIN) {
+  auto stage = [&](auto U, auto PLAIN, int half) {
     constexpr int u = decltype(U)::value;
     asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
     __syncthreads();
     issue(PLAIN);
     read_frags(std::integral_constant<int, 1 - u>());
     __builtin_amdgcn_sched_barrier(0);
-    multiply(U);
+    multiply(U, half);
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -491,15 +552,43 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_pp_kernel(void* __rest
     }
     for (int kb = 0; kb < nst; kb += 2) {
       // (the plain GEMM keeps one copy of the pair: with two, the compiler's register allocation of this loop falls apart)
-      if (LORA && load_kb + 2 < KB) {                    // uniform: the two stages fetched next are ordinary k-steps inside their block
-        stage(std::integral_constant<int, 0>(), std::true_type());
-        stage(std::integral_constant<int, 1>(), std::true_type());
+      if constexpr (SILU && LORA) {
+        // one copy of the pair; a pair of LoRA stages belongs to one projection and multiplies that half of the tiles only
+        const int half = kb < KB ? -1 : (has_gate && kb - KB < EP ? 0 : 1);   // uniform
+        stage(std::integral_constant<int, 0>(), std::false_type(), half);
+        stage(std::integral_constant<int, 1>(), std::false_type(), half);
+      } else if (LORA && load_kb + 2 < KB) {             // uniform: the two stages fetched next are ordinary k-steps inside their block
+        stage(std::integral_constant<int, 0>(), std::true_type(), -1);
+        stage(std::integral_constant<int, 1>(), std::true_type(), -1);
       } else {
-        stage(std::integral_constant<int, 0>(), std::false_type());
-        stage(std::integral_constant<int, 1>(), std::false_type());
+        stage(std::integral_constant<int, 0>(), std::false_type(), -1);
+        stage(std::integral_constant<int, 1>(), std::false_type(), -1);
       }
     }
-    if constexpr (OUT == OUT_F16) {
+    if constexpr (SILU) {
+      // acc[i] and acc[4 + i] are the gate and the up half of channels n0 + wn * 64 + i * 16 + 4 g .. + 3 for token r16 of
+      // token fragment j: four products = one 8-byte piece of the output fragment; the pieces of a store instruction
+      // are 512 contiguous bytes
+#pragma unroll
+      for (int j = 0; j < WTF; ++j) {
+        const int t = t0 + (wt * WTF + j) * 16 + r16;
+        if ((t >> 4) >= x_tt) continue;                  // the token tile does not exist
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int c = n0 + (wn * 4 + i) * 16 + g * 4;
+          if (c >= I) continue;
+          f16x4 o = f16x4{0, 0, 0, 0};                   // rows past T inside the last tile: zeros, as the separate kernel writes them
+          if (t < T) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float gf = (float)(f16)acc[i][j][r];
+              o[r] = (f16)(gf / (1.f + expf(-gf)) * (float)(f16)acc[4 + i][j][r]);
+            }
+          }
+          *reinterpret_cast<f16x4*>((f16*)yv + ((size_t)(c >> 5) * x_tt + (t >> 4)) * 512 + ((c & 31) >> 3) * 128 + (t & 15) * 8 + (c & 7)) = o;
+        }
+      }
+    } else if constexpr (OUT == OUT_F16) {
       // 16 tokens x 64 columns at a time through the wave's staging buffer: D[n][t] fragments in, token rows out
 #pragma unroll
       for (int j = 0; j < WTF; ++j) {
@@ -566,7 +655,7 @@ int launch_gemm_pp(void* y, const f16* x, int ldx, int x_tt, const f16* Wp, int 
     if (e != hipSuccess) return mlora_set_error(MLORA_ERR_LAUNCH, "gemm_packed: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     configured = true;
   }
-  const int gx = ceil_div(N, PP_F * 16), gy = ceil_div(T, PP_F * 16);
+  const int gx = OUT == OUT_SILU ? ceil_div(N / 2, PP_F * 8) : ceil_div(N, PP_F * 16), gy = ceil_div(T, PP_F * 16);
   int n_cu = gemm_n_cu();
   if (n_cu <= 0) n_cu = 256;
   const int grid = gx * gy < n_cu ? gx * gy : n_cu;
@@ -969,6 +1058,36 @@ extern "C" int mlora_linear_frag_lora(void* y, int y_dtype, int mode, const void
   else if (y_dtype == MLORA_F32) e = launch_gemm_pp<OUT_F32>(y, (const f16*)xf, 0, tt, (const f16*)Wp, T, K, N, s, lo);
   else e = launch_gemm_pp<OUT_F16>(y, (const f16*)xf, 0, tt, (const f16*)Wp, T, K, N, s, lo);
   return e ? e : mlora_launch_status("linear_frag_lora");
+}
+
+extern "C" int mlora_linear_frag_silu(void* act, const void* xf, const void* Wp, int T, int K, int I, const mlora_fused_lora* projs,
+                                      int n_proj, const int32_t* blk_adapter, int r, void* stream) {
+  MLORA_CHECK(act && xf && Wp, MLORA_ERR_INVALID, "linear_frag_silu: null pointer");
+  MLORA_CHECK(T > 0 && K > 0 && I > 0 && I % 32 == 0 && I <= (1 << 29), MLORA_ERR_UNSUPPORTED,
+              "linear_frag_silu: need I %% 32 == 0 (T=%d K=%d I=%d)", T, K, I);
+  MLORA_CHECK(mlora_gemm_frag_preferred(T, K, 2 * I) && (((uintptr_t)xf | (uintptr_t)act) & 15) == 0, MLORA_ERR_UNSUPPORTED,
+              "linear_frag_silu: only shapes of the persistent GEMM (mlora_gemm_frag_preferred; T=%d K=%d N=%d)", T, K, 2 * I);
+  MLORA_CHECK(n_proj >= 0 && n_proj <= 2, MLORA_ERR_UNSUPPORTED, "linear_frag_silu: at most the gate and the up projection (n_proj=%d)", n_proj);
+  PPLora lo = {};
+  if (n_proj > 0) {
+    MLORA_CHECK(projs && blk_adapter && (r == 32 || r == 64), MLORA_ERR_UNSUPPORTED,
+                "linear_frag_silu: projections of rank 32 or 64 with the blocks' adapters (r=%d)", r);
+    for (int i = 0; i < n_proj; ++i) {
+      const mlora_fused_lora& p = projs[i];
+      MLORA_CHECK(p.B && p.v_hi && p.v_lo && (((uintptr_t)p.B | (uintptr_t)p.v_hi | (uintptr_t)p.v_lo) & 15) == 0, MLORA_ERR_INVALID,
+                  "linear_frag_silu: null or unaligned table of projection %d", i);
+      MLORA_CHECK((p.n_begin == 0 || p.n_begin == I) && p.n_rows == I, MLORA_ERR_UNSUPPORTED,
+                  "linear_frag_silu: projection %d must be the gate rows 0..I or the up rows I..2I (n_begin=%d n_rows=%d I=%d)", i,
+                  p.n_begin, p.n_rows, I);
+      const int slot = p.n_begin == 0 ? 0 : 1;
+      MLORA_CHECK(lo.B[slot] == nullptr, MLORA_ERR_INVALID, "linear_frag_silu: two projections over the same rows");
+      lo.B[slot] = (const f16*)p.B; lo.vh[slot] = (const f16*)p.v_hi; lo.vl[slot] = (const f16*)p.v_lo;
+      lo.n_begin[slot] = p.n_begin; lo.n_rows[slot] = p.n_rows;
+    }
+    lo.n_proj = n_proj; lo.r = r; lo.blk_adapter = blk_adapter;
+  }
+  const int e = launch_gemm_pp<OUT_SILU>(act, (const f16*)xf, 0, mlora_frag_tiles(T), (const f16*)Wp, T, K, 2 * I, (hipStream_t)stream, lo);
+  return e ? e : mlora_launch_status("linear_frag_silu");
 }
 
 // K slices the mid-size kernel would use for resid [T, N] += xf . Wp^T with at most ks_max slices (T > 64)

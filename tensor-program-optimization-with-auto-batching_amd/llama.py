@@ -349,12 +349,15 @@ class LlamaForCausalLM:
                 act = ops.gate_up_silu(xn, self.interleaved_gate_up()[l])
             else:
                 gu_projs = (("gate_proj", 0, I), ("up_proj", I, I))
-                gu = self._fused_linear(fuse, xn, L["gate_up"], l, gu_projs) if fuse else None
-                if gu is None:
-                    gu = ops.linear(xn, L["gate_up"])
-                    if tok_adapter:
-                        self._lora_group(gu, xn, l, gu_projs, tok_adapter)
-                act = ops.silu_mul(gu, frag=frag)
+                # a prefill-sized pass: the SiLU product leaves the GEMM itself wherever no token needs a separate delta
+                act = self._gate_up_silu(fuse, xn, L["gate_up"], l, gu_projs, bool(tok_adapter)) if frag and T > 64 else None
+                if act is None:
+                    gu = self._fused_linear(fuse, xn, L["gate_up"], l, gu_projs) if fuse else None
+                    if gu is None:
+                        gu = ops.linear(xn, L["gate_up"])
+                        if tok_adapter:
+                            self._lora_group(gu, xn, l, gu_projs, tok_adapter)
+                    act = ops.silu_mul(gu, frag=frag)
             if fuse and self._fused_linear(fuse, act, L["down"], l, (("down_proj", 0, H),), resid=resid) is not None:
                 parts = None
             else:
@@ -382,11 +385,7 @@ class LlamaForCausalLM:
         live = [e for e in live if e[3] is not None]
         if not live or not ops.gemm_frag_preferred(T, K, N) or any(c0 % 256 or (n % 256 and c0 + n != N) for _, c0, n, _ in live):
             return None
-        key = (T, lt.r)
-        if getattr(self, "_v_split_key", None) != key:
-            self._v_split = [tuple(torch.empty((T, lt.r), dtype=torch.float16, device=self.device) for _ in range(2)) for _ in range(3)]
-            self._v_split_key = key
-        vs = ops.lora_shrink_split(x, [tab[0] for *_, tab in live], ids, lt.scaling, self._workspace(T, K, lt.r), out=self._v_split[:len(live)])
+        vs = ops.lora_shrink_split(x, [tab[0] for *_, tab in live], ids, lt.scaling, self._workspace(T, K, lt.r), out=self._v_split_bufs(T, lt.r)[:len(live)])
         fused = [(tab[1], vh, vl, c0, n) for (_, c0, n, tab), (vh, vl) in zip(live, vs)]
         if resid is not None:
             y = ops.linear_frag_lora(x, W, fused, blk, lt.r, out=resid, accumulate=True)
@@ -398,6 +397,35 @@ class LlamaForCausalLM:
             else:
                 self._lora_group(y, x, l, projs, rest)
         return y
+
+    def _gate_up_silu(self, fuse, x, W, l, projs, adapters):
+        """silu(gate) * up in fragment order out of the persistent GEMM of the fused gate/up projection: without
+        adapters on these projections, or with their deltas as extra k-steps when every 256-token block of the pass
+        agrees on one adapter.  Returns None where that does not apply (shape, a block that mixes adapters, a rank
+        or a mix of adapter types that the extra k-steps do not take)."""
+        T, K = x.shape
+        N = W.shape[0]
+        if not isinstance(x, ops.FragActivation) or not isinstance(W, ops.PackedWeight) or (N // 2) % 32 or not ops.gemm_frag_preferred(T, K, N):
+            return None
+        if not adapters or not self._targets(l, *(p for p, _, _ in projs)):
+            return ops.linear_frag_silu(x, W)
+        if fuse is None or fuse[3] is not None:
+            return None
+        lt, ids, blk, _ = fuse
+        live = [(c0, n, lt.tables.get((l, proj))) for proj, c0, n in projs]
+        live = [e for e in live if e[2] is not None]
+        if not live:                                     # the tables belong to an adapter type that is not in this pass
+            return ops.linear_frag_silu(x, W)
+        vs = ops.lora_shrink_split(x, [tab[0] for *_, tab in live], ids, lt.scaling, self._workspace(T, K, lt.r), out=self._v_split_bufs(T, lt.r)[:len(live)])
+        return ops.linear_frag_silu(x, W, [(tab[1], vh, vl, c0, n) for (c0, n, tab), (vh, vl) in zip(live, vs)], blk, lt.r)
+
+    def _v_split_bufs(self, T, r):
+        """fp16 hi / lo halves of the shrink results of up to three projections (reused from call to call)."""
+        key = (T, r)
+        if getattr(self, "_v_split_key", None) != key:
+            self._v_split = [tuple(torch.empty((T, r), dtype=torch.float16, device=self.device) for _ in range(2)) for _ in range(3)]
+            self._v_split_key = key
+        return self._v_split
 
     def _ksplit_ws(self, T):
         """fp32 scratch for the K-split partials of o_proj / down_proj at T tokens (grown on demand, reused)."""

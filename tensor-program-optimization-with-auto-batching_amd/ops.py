@@ -393,6 +393,32 @@ def linear_frag_lora(x: FragActivation, W: PackedWeight, projs, blk_adapter, r: 
     return out
 
 
+def linear_frag_silu(x: FragActivation, W: PackedWeight, projs=(), blk_adapter=None, r: int = 0, out: FragActivation = None) -> FragActivation:
+    """silu(gate) * up of the fused gate/up projection `W` [2I, K] in the epilogue of the persistent GEMM, in fragment
+    order.  `projs` as for linear_frag_lora, over the gate rows (first row 0) and / or the up rows (first row I); every
+    256-token block must agree on one adapter (lora_block_adapters leaves no rest)."""
+    import ctypes as C
+    from ._lib import FusedLora
+    T, K = x.shape
+    N, K2 = W.shape
+    I = N // 2
+    if K2 != K or N % 2:
+        raise ValueError(f"linear_frag_silu: x{x.shape} vs W{W.shape}")
+    if out is None:
+        out = FragActivation(T, I, x.device)
+    if out.shape != (T, I):
+        raise ValueError(f"linear_frag_silu: out{tuple(out.shape)} expected {(T, I)}")
+    arr = (FusedLora * max(len(projs), 1))()
+    for e, (B, vh, vl, n0, rows) in zip(arr, projs):
+        if B.shape[1] != rows or B.shape[2] != r or vh.shape != (T, r) or vl.shape != (T, r):
+            raise ValueError("linear_frag_silu: table or v shape")
+        e.B, e.v_hi, e.v_lo, e.n_begin, e.n_rows = _dev(B, torch.float16, "B"), _dev(vh, torch.float16, "v_hi"), _dev(vl, torch.float16, "v_lo"), n0, rows
+    check(lib().mlora_linear_frag_silu(out.data.data_ptr(), x.data.data_ptr(), W.data.data_ptr(), T, K, I,
+                                       C.cast(arr, C.c_void_p) if projs else None, len(projs),
+                                       _dev(blk_adapter, torch.int32) if projs else None, r, _stream()))
+    return out
+
+
 def interleave_gate_up(gate_up: torch.Tensor) -> PackedWeight:
     """[2I, K] (gate rows, then up rows) -> PackedWeight whose 16-row tiles alternate gate and up."""
     I2, K = gate_up.shape

@@ -158,6 +158,20 @@ def test_argument_validation_of_fused_and_batched_entry_points():
     assert lf() == -2                                                              # rows past N
     fl[1].n_rows, fl[1].v_lo = 4096, None
     assert lf() == -1
+    # gate/up projection with the SiLU product in the epilogue of the persistent GEMM
+    fs = (lm.FusedLora * 2)()
+    for i, e in enumerate(fs):
+        e.B, e.v_hi, e.v_lo, e.n_begin, e.n_rows = 16, 16, 16, 4096 * i, 4096
+    sl = lambda act=16, T=4096, I=4096, n_proj=2, blk=16, r=64: lib.mlora_linear_frag_silu(act, 16, 16, T, 4096, I, C.cast(fs, C.c_void_p), n_proj,
+                                                                                            blk, r, None)
+    assert sl(act=None) == -1 and sl(I=4100) == -2 and sl(n_proj=3) == -2 and sl(r=16) == -2 and sl(blk=None) == -2
+    assert sl(T=256, I=2048) == -2 and b"persistent" in lib.mlora_last_error()
+    fs[1].n_begin = 2048
+    assert sl() == -2 and b"gate rows" in lib.mlora_last_error()                   # neither rows 0..I nor rows I..2I
+    fs[1].n_begin = 0
+    assert sl() == -1 and b"same rows" in lib.mlora_last_error()
+    fs[1].n_begin, fs[1].B = 4096, None
+    assert sl() == -1
     # decode step: a plan without layers / with a token count beyond the decode tile
     plan = lm.DecodePlan()
     assert lib.mlora_decode_step(C.byref(plan), None) < 0

@@ -448,6 +448,51 @@ def test_prefill_linear_with_lora_as_extra_k_steps(ops, synth, r, acc):
     assert torch.equal(ops.linear_frag_lora(xf, Wp, projs, none, r), ops.linear(xf, Wp))
 
 
+@pytest.mark.parametrize("T,K,I,r,which", [(4096, 256, 4096, 0, ""), (1000, 128, 8224, 0, ""), (4096, 256, 4096, 64, "gu"),
+                                            (3000, 128, 5664, 32, "gu"), (4096, 256, 4096, 32, "g"), (4096, 256, 4096, 64, "u")])
+def test_prefill_gate_up_with_silu_in_the_gemm_epilogue(ops, synth, T, K, I, r, which):
+    """silu(gate) * up out of the persistent GEMM (channel counts that are and are not multiples of the 128-channel
+    block, a ragged last token tile, adapters on both projections, on one, on none, blocks without adapter): the same
+    bits as the fused projection (with its deltas as extra k-steps), stored as fp16, followed by the separate SiLU
+    kernel - and that pair against the float64 evaluation."""
+    n_ad = 3
+    x = synth.normal(29, "fs.x", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(29, "fs.W", (2 * I, K), 0.08, torch.float16, DEV)
+    xf, Wp = ops.FragActivation.pack(x), ops.PackedWeight(W)
+    ref = _np(x).astype(np.float64) @ _np(W).astype(np.float64).T
+    if not which:
+        gu = ops.linear(xf, Wp)
+        act = ops.linear_frag_silu(xf, Wp)
+    else:
+        ids = np.repeat(np.array([1, 0, -1, 2, 1, 2, 0, 0, 2, 1, -1, 1, 0, 2, 1, 1], np.int32), 256)[:T]
+        ids_d = torch.from_numpy(ids).to(DEV)
+        blk, rest = ops.lora_block_adapters(ids_d, n_ad)
+        assert (rest.cpu().numpy() == -1).all()
+        sel = [p for p, c in enumerate("gu") if c in which]
+        A = [synth.normal(29, f"fs.A{p}", (n_ad, r, K), 0.05, torch.float16, DEV) for p in sel]
+        B = [synth.normal(29, f"fs.B{p}", (n_ad, I, r), 0.05, torch.float16, DEV) for p in sel]
+        ws = torch.empty(len(sel) * ops.lib().mlora_gather_mm_workspace_bytes(T, K, r) // 4 + 4, dtype=torch.float32, device=DEV)
+        vs = ops.lora_shrink_split(xf, A, ids_d, 0.5, ws)
+        projs = [(B[i], vs[i][0], vs[i][1], p * I, I) for i, p in enumerate(sel)]
+        # (the separate projection wants its row ranges on 256-row blocks; the other channel counts meet float64 only)
+        gu = ops.linear_frag_lora(xf, Wp, projs, blk, r) if I % 256 == 0 else None
+        act = ops.linear_frag_silu(xf, Wp, projs, blk, r)
+        xd = _np(x).astype(np.float64)
+        for i, p in enumerate(sel):
+            Ad, Bd = _np(A[i]).astype(np.float64), _np(B[i]).astype(np.float64)
+            for a in range(n_ad):
+                rows = np.nonzero(ids == a)[0]
+                ref[rows, p * I:(p + 1) * I] += 0.5 * (xd[rows] @ Ad[a].T) @ Bd[a].T
+    if gu is not None:
+        want = ops.silu_mul(gu, frag=True)
+        torch.cuda.synchronize()
+        assert torch.equal(act.data, want.data)
+    g, u = ref[:, :I], ref[:, I:]
+    got = _np(act.unpack()).astype(np.float64)
+    assert np.abs(got).max() > 1.0
+    assert max_rel_err(got, g / (1.0 + np.exp(-g)) * u, floor=2e-2) <= 2 * TOL     # two fp16 roundings on the way (gate / up, then the product)
+
+
 def test_prefill_linear_with_lora_three_projections_and_a_ragged_last_one(ops, synth):
     """Three projections of unequal width, the last ending 64 rows into a 256-row block of the GEMM, rank 32, every
     block with an adapter: against the float64 evaluation."""
