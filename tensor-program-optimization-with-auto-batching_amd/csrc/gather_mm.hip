@@ -476,7 +476,7 @@ template <int R>
 __device__ __forceinline__ void shrink_tile_mfma(float* __restrict__ v, const f16* __restrict__ x, int frag_tt, const f16* __restrict__ A,
                                                  const int32_t* __restrict__ ids, int T, int K, int n_ad,
                                                  const int32_t* __restrict__ bucket_of, int bucket, int t0, int kb0, int kb1,
-                                                 f32x4 (*red)[8][WAVE]) {
+                                                 f32x4 (*red)[8][WAVE], int only_group = -1) {
   constexpr int NT = (R + 15) / 16;     // 16-row tiles of A[a]; rank 8 uses half a tile
   constexpr int GA = 8 / NT;            // adapters per pass: 32 accumulator registers
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -489,7 +489,7 @@ __device__ __forceinline__ void shrink_tile_mfma(float* __restrict__ v, const f1
   const f16* __restrict__ xr = x_operand(x, tl, g, K, frag_tt, xstep);
 #pragma unroll
   for (int g0 = 0; g0 < 16; g0 += GA) {
-    if (g0 < ta.n) {                                             // uniform
+    if (g0 < ta.n && (only_group < 0 || g0 == only_group * GA)) {   // uniform
       f32x4 acc[GA][NT];
 #pragma unroll
       for (int u = 0; u < GA; ++u)
@@ -562,17 +562,22 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_shrink_mfma_kernel(floa
                                                                             const int32_t* __restrict__ ids, int T, int K,
                                                                             int n_ad, const int32_t* __restrict__ bucket_of,
                                                                             int bucket) {
-  // blockIdx.y selects one of gridDim.y contiguous ranges of 32-k steps; its partial sums go to v[blockIdx.y][T][R]
+  // blockIdx.y selects one of gridDim.y contiguous ranges of 32-k steps; its partial sums go to v[blockIdx.y][T][R].
+  // blockIdx.z = projection * NG + group: the tile's adapters are taken in the order of their first token, GA to a group,
+  // and every group has a workgroup of its own (a tile of a decode batch holds up to 16 adapters: their passes over K
+  // run side by side instead of one after the other; a workgroup whose group is empty leaves at once).
+  constexpr int NG = 16 / (8 / ((R + 15) / 16));
   __shared__ f32x4 red[SEG_WAVES][8][WAVE];
+  const int proj = blockIdx.z / NG, group = blockIdx.z % NG;
   const f16* __restrict__ A = pj.A[0];
 #pragma unroll
   for (int i = 1; i < SEG_MAX_PROJ; ++i)
-    if (i == blockIdx.z) A = pj.A[i];                    // uniform select: the struct is never indexed dynamically
+    if (i == proj) A = pj.A[i];                          // uniform select: the struct is never indexed dynamically
   const int KB = K / 32;
   const int per = (KB + gridDim.y - 1) / gridDim.y;
   const int kb0 = blockIdx.y * per, kb1 = min(KB, kb0 + per);
-  v += ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * T * R;
-  shrink_tile_mfma<R>(v, x, frag_tt, A, ids, T, K, n_ad, bucket_of, bucket, blockIdx.x * 16, kb0, kb1, red);
+  v += ((size_t)proj * gridDim.y + blockIdx.y) * T * R;
+  shrink_tile_mfma<R>(v, x, frag_tt, A, ids, T, K, n_ad, bucket_of, bucket, blockIdx.x * 16, kb0, kb1, red, group);
 }
 
 // Prefill-sized shrink: FOUR token tiles per workgroup.  When all adapted tokens of the four tiles use one adapter (an
@@ -894,7 +899,7 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mixed_mfma_kerne
     }
   v += (size_t)blockIdx.z * splits * T * R;
   constexpr int KS = (R + 31) / 32;     // k-steps of 32 rank entries (ranks 8 and 16: one partly filled step)
-  constexpr int GB = 8 / KS;            // adapters whose fragments are in flight together: 32 registers
+  constexpr int GB = 16 / KS;           // adapters whose fragments are in flight together: 64 registers
   constexpr int CT = 4;                 // 16-column tiles per wave
   constexpr int LD = 16 * CT + 4;       // padded row of the transposition buffer (floats): conflict-free both ways
   __shared__ float stage[SEG_WAVES][16][LD];
@@ -910,6 +915,7 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mixed_mfma_kerne
   if (!all) return;                     // the same for every wave of the workgroup
   const int a_first = __builtin_amdgcn_readfirstlane(__shfl(id, __builtin_ctz(all), WAVE));
   const bool one_adapter = ((unsigned)__ballot(id == a_first) & 0xffffu) == all;
+  const TileAdapters ta = tile_adapters(id);                     // the tile's distinct adapters and their rows, found once
   // the token tile of v as the B operand, hi and lo halves: lane holds v[token col][ks*32 + 8g .. +7]
   f16x8 vh[KS], vl[KS];
 #pragma unroll
@@ -962,40 +968,32 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mixed_mfma_kerne
               acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf, vl[ks], acc, 0, 0, 0);
             }
           } else {
-            unsigned todo = all;
-            while (todo) {                                             // uniform: GB adapters of the tile per round
-              int ga[GB];
-              unsigned grows[GB];
+            // the tile's adapters GB at a time (ranks up to 32: all sixteen at once): their B fragments are requested
+            // together, then every adapter's product goes to the tokens bound to it
 #pragma unroll
-              for (int u = 0; u < GB; ++u) {
-                ga[u] = -1;
-                grows[u] = 0u;
-                if (todo) {
-                  ga[u] = __builtin_amdgcn_readfirstlane(__shfl(id, __builtin_ctz(todo), WAVE));
-                  grows[u] = (unsigned)__ballot(id == ga[u]) & 0xffffu & todo;
-                  todo &= ~grows[u];
-                }
-              }
-              f16x8 bf[GB][KS];
+            for (int g0 = 0; g0 < 16; g0 += GB) {
+              if (g0 < ta.n) {                                         // uniform
+                f16x8 bf[GB][KS];
 #pragma unroll
-              for (int u = 0; u < GB; ++u) {
-                if (ga[u] >= 0) {
-                  const f16* __restrict__ Ba = B + (size_t)ga[u] * N * R + g * 8;
+                for (int u = 0; u < GB; ++u) {
+                  if (g0 + u < ta.n) {
+                    const f16* __restrict__ Ba = B + (size_t)ta.a[g0 + u] * N * R + g * 8;
 #pragma unroll
-                  for (int ks = 0; ks < KS; ++ks)
-                    bf[u][ks] = (ks * 32 + g * 8) < R ? ld8(Ba + (size_t)(nb + col) * R + ks * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-                }
-              }
-#pragma unroll
-              for (int u = 0; u < GB; ++u) {
-                if (ga[u] >= 0) {
-                  f32x4 d = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                  for (int ks = 0; ks < KS; ++ks) {
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf[u][ks], vh[ks], d, 0, 0, 0);
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf[u][ks], vl[ks], d, 0, 0, 0);
+                    for (int ks = 0; ks < KS; ++ks)
+                      bf[u][ks] = (ks * 32 + g * 8) < R ? ld8(Ba + (size_t)(nb + col) * R + ks * 32) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
                   }
-                  if ((grows[u] >> col) & 1u) acc = d;
+                }
+#pragma unroll
+                for (int u = 0; u < GB; ++u) {
+                  if (g0 + u < ta.n) {
+                    f32x4 d = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                      d = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf[u][ks], vh[ks], d, 0, 0, 0);
+                      d = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf[u][ks], vl[ks], d, 0, 0, 0);
+                    }
+                    if ((ta.rows[g0 + u] >> col) & 1u) acc = d;
+                  }
                 }
               }
             }
@@ -1228,7 +1226,8 @@ static int gmm_segments_shrink_r(const SegProjs& pj, const f16* x, int frag_tt, 
   // beyond that a prefill whose tokens come in adapter segments: four token tiles per shrink workgroup, two per expand
   // workgroup, about two workgroups per compute unit.  Either set of kernels is correct for either input.
   if (T <= 1024) {
-    hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles, splits, pj.n), dim3(SEG_WAVES * WAVE), 0, s, v, x, frag_tt, pj, ids, T, K,
+    constexpr int NG = 16 / (8 / ((R + 15) / 16));   // adapter groups of a tile, each with its own workgroup
+    hipLaunchKernelGGL((lora_shrink_mfma_kernel<R>), dim3(tiles, splits, pj.n * NG), dim3(SEG_WAVES * WAVE), 0, s, v, x, frag_tt, pj, ids, T, K,
                        n_ad, bf.bucket_of, bf.bucket);
   } else {
     const int quads = ceil_div(tiles, 4);
