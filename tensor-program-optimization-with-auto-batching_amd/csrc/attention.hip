@@ -712,7 +712,10 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
 // Workgroups are dispatched longest key range first over all heads (grid = (heads, token blocks), late token blocks
 // first): with the token block as the fast grid dimension the long workgroups of the last heads started late and ran
 // alone at the end - 0.9 resident waves per SIMD on average, 551 instead of 336 us for one sequence of 4096 tokens.
-// (8 x 512 tokens, 32 heads of 128: 71 us, 0.24 PFLOP/s of causal QK^T + PV; one sequence of 4096: 304 us, 0.45.  With the hi half
+// (8 x 512 tokens, 32 heads of 128: 60 us, 0.29 PFLOP/s of causal QK^T + PV; one sequence of 4096: 269 us, 0.51.  With the V pieces
+// in LDS in cache order - the 8-byte V reads of 16 neighbouring dims then fall on every other 16-byte bank group, twice: by
+// counters 60 % of the LDS cycles were bank conflicts - and the compiler's own pairing of these reads (two dims of one page,
+// then 28 register moves per 16 MFMAs to put an operand's halves side by side): 71 and 304 us.  With the hi half
 // of P rounded to nearest, converted back and subtracted - ten instructions per pair of probabilities instead of six: 73 and 315 us; with O and l
 // rescaled in every block on top of that: 77 and 336 us; before the dispatch order was changed: 90 and 551 us; with one query tile per wave on top of that: 121 and 599 us; that form with eight waves per workgroup and four waves per SIMD: 102 and 655;
 // with 32-key blocks and a four-deep ring: 134 and 732; adding P . V of the previous block under the softmax arithmetic
@@ -722,6 +725,12 @@ constexpr int PF_WAVES = 4;
 constexpr int PF_QT = 2;         // 16-query tiles per wave: a K or V fragment read from LDS serves that many MFMAs
 constexpr int PF_PAGES = 4;      // pages per key block
 constexpr int PF_RING = 2;       // key-block buffers
+
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
 
 template <int D>
 __global__ __launch_bounds__(PF_WAVES* WAVE, 2) void paged_attn_prefill_block_kernel(
@@ -832,15 +841,22 @@ __global__ __launch_bounds__(PF_WAVES* WAVE, 2) void paged_attn_prefill_block_ke
       const int pg = b * PF_PAGES + wave / WPP;
       int page = pg < npages ? bt[pg] : 0;
       page = page >= 0 && page < n_pages ? page : 0;
-      const size_t src = ((size_t)page * Hkv + kh) * PE + (wave % WPP) * HC * 512 + lane * 8;
+      const size_t src = ((size_t)page * Hkv + kh) * PE + (wave % WPP) * HC * 512;
       f16* kd = smem + (b % PF_RING) * BUF + (wave / WPP) * PE + (wave % WPP) * HC * 512;
-      f16* vd = kd + PF_PAGES * PE;
+      // the V pieces of a page pair alternate (piece j of the even page, piece j of the odd page, piece j + 1 ...): a
+      // lane's four keys of both pages are then 1 KiB apart and one two-address LDS read delivers the whole operand
+      f16* vd = smem + (b % PF_RING) * BUF + PF_PAGES * PE + ((((wave / WPP) >> 1) * CH + (wave % WPP) * HC) * 2 + ((wave / WPP) & 1)) * 512;
+      // K pieces keep their order.  A 1 KiB piece of V is 32 dims x (two 16-byte halves of the 16 keys): lane l fetches
+      // half l / 32 of dim l % 32, so that the LDS copy holds the 32 first halves side by side, then the 32 second
+      // halves - the 16 lanes that read the same half of 16 neighbouring dims then hit 16 different 16-byte bank groups
+      // (in cache order they hit every other one, twice)
+      const int vsrc = (lane & 31) * PAGE + (lane >> 5) * 8;
 #pragma unroll
       for (int j = 0; j < HC; ++j) {
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(k_cache + src + j * 512),
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(k_cache + src + j * 512 + lane * 8),
                                          (__attribute__((address_space(3))) void*)(kd + j * 512), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(v_cache + src + j * 512),
-                                         (__attribute__((address_space(3))) void*)(vd + j * 512), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(v_cache + src + j * 512 + vsrc),
+                                         (__attribute__((address_space(3))) void*)(vd + j * 1024), 16, 0, 0);
       }
     };
 #pragma unroll
@@ -881,11 +897,7 @@ __global__ __launch_bounds__(PF_WAVES* WAVE, 2) void paged_attn_prefill_block_ke
 #pragma unroll
       for (int u = 0; u < QT; ++u) act[u] = tmax[u] >= b * PF_PAGES * PAGE;
       // S^T of the block for the wave's query tiles: a K fragment is read from LDS once and multiplied with every tile
-      f32x4 st[QT][PF_PAGES];                                        // st[u][p][r] = S[key 4g + r of page p][query qi of tile u]
-#pragma unroll
-      for (int u = 0; u < QT; ++u)
-#pragma unroll
-        for (int p = 0; p < PF_PAGES; ++p) st[u][p] = f32x4{0.f, 0.f, 0.f, 0.f};
+      f32x4 st[QT][PF_PAGES];                                        // st[u][p][r] = S[key 4g + r of page p][query qi of tile u] (tiles at work only)
 #pragma unroll
       for (int p = 0; p < PF_PAGES; ++p) {
         f16x8 kf[NKB];
@@ -893,9 +905,11 @@ __global__ __launch_bounds__(PF_WAVES* WAVE, 2) void paged_attn_prefill_block_ke
         for (int kb = 0; kb < NKB; ++kb) kf[kb] = ld8(kb_ + p * PE + kb * 512 + lane * 8);
 #pragma unroll
         for (int u = 0; u < QT; ++u) {
-          if (act[u]) {
+          if (act[u]) {                                              // the first product starts from a zero operand, not from zeroed registers
+            f32x4 sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[0], qf[u][0], f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
-            for (int kb = 0; kb < NKB; ++kb) st[u][p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kb], qf[u][kb], st[u][p], 0, 0, 0);
+            for (int kb = 1; kb < NKB; ++kb) sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kb], qf[u][kb], sacc, 0, 0, 0);
+            st[u][p] = sacc;
           }
         }
       }
@@ -905,20 +919,27 @@ __global__ __launch_bounds__(PF_WAVES* WAVE, 2) void paged_attn_prefill_block_ke
       for (int u = 0; u < QT; ++u) {
         if (!act[u]) continue;
         if (!(all_in[u] && all_live && (b + 1) * PF_PAGES * PAGE - 1 <= tmin[u])) {   // uniform: some key of the block is masked
+          // key (p, r) of this lane lies `p * PAGE + r` behind the block's first key of the lane's group: one
+          // subtraction per tile, then a compare with a constant per score
+          const int lim = in_run[u] ? my_pos[u] - (b * PF_PAGES * PAGE + 4 * g) : -1;
 #pragma unroll
           for (int p = 0; p < PF_PAGES; ++p) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const bool masked = !live[p] || !in_run[u] || (b * PF_PAGES + p) * PAGE + 4 * g + r > my_pos[u];
+              const bool masked = !live[p] || p * PAGE + r > lim;
               st[u][p][r] = masked ? -INFINITY : st[u][p][r];
             }
           }
         }
-        float pm = fmaxf(fmaxf(st[u][0][0], st[u][0][1]), fmaxf(st[u][0][2], st[u][0][3]));
-#pragma unroll
-        for (int p = 1; p < PF_PAGES; ++p) pm = fmaxf(pm, fmaxf(fmaxf(st[u][p][0], st[u][p][1]), fmaxf(st[u][p][2], st[u][p][3])));
-        pm = fmaxf(pm, __shfl_xor(pm, 16, WAVE));
-        pm = fmaxf(pm, __shfl_xor(pm, 32, WAVE));
+        // the block's maximum per query: the scores are finite or -inf, never NaN, so the three-input maximum is taken as
+        // the instruction gives it (through fmaxf the compiler first passes every score through a quieting v_max)
+        static_assert(PF_PAGES == 4, "the tree below names the sixteen scores of four pages");
+        const float t0 = max3_raw(st[u][0][0], st[u][0][1], st[u][0][2]), t1 = max3_raw(st[u][0][3], st[u][1][0], st[u][1][1]);
+        const float t2 = max3_raw(st[u][1][2], st[u][1][3], st[u][2][0]), t3 = max3_raw(st[u][2][1], st[u][2][2], st[u][2][3]);
+        const float t4 = max3_raw(st[u][3][0], st[u][3][1], st[u][3][2]);
+        float pm = max3_raw(max3_raw(t0, t1, t2), max3_raw(t3, t4, st[u][3][3]), t0);
+        pm = max3_raw(pm, __shfl_xor(pm, 16, WAVE), pm);
+        pm = max3_raw(pm, __shfl_xor(pm, 32, WAVE), pm);
         // The reference maximum m moves - and O and l are rescaled - only when some query of the tile meets a score more
         // than 2^8 above it (always in the tile's first block); otherwise the block's P are taken relative to the old
         // reference and may reach 256, which fp16 holds exactly as well.  After the first blocks of a sequence that
@@ -966,13 +987,18 @@ __global__ __launch_bounds__(PF_WAVES* WAVE, 2) void paged_attn_prefill_block_ke
       for (int pp = 0; pp < PF_PAGES / 2; ++pp) {
         __builtin_amdgcn_sched_barrier(0);                           // the V fragments are not requested before they fit the register file
         f16x8 vv[NDB];
+        // dim db * 16 + qi, keys 4 g .. of the pair's two pages: piece db / 2 of the pair, half g / 2, then dim (db % 2) * 16 + qi
+        // of that piece; the odd page's copy lies 1 KiB behind.  One two-address read per operand, written out: left to
+        // itself the compiler pairs the reads of two neighbouring dims of one page and then moves the halves together,
+        // 28 register moves per 16 MFMAs.  Reads issued this way are not in the compiler's count of outstanding LDS
+        // operations, hence the explicit wait.
+        const unsigned vaddr = (unsigned)(size_t)(const __attribute__((address_space(3))) f16*)(vb_ + pp * CH * 1024 + ((g >> 1) * 32 + qi) * 8 + (g & 1) * 4);
 #pragma unroll
-        for (int db = 0; db < NDB; ++db) {
-          const f16* v0 = vb_ + (2 * pp) * PE + (db * 16 + qi) * PAGE + g * 4;
-          const f16x4 va = *reinterpret_cast<const f16x4*>(v0);
-          const f16x4 vb = *reinterpret_cast<const f16x4*>(v0 + PE);
-          vv[db] = __builtin_shufflevector(va, vb, 0, 1, 2, 3, 4, 5, 6, 7);
+        for (int db = 0; db < NDB; db += 2) {
+          asm volatile("ds_read2_b64 %0, %2 offset1:128\n\tds_read2_b64 %1, %2 offset0:32 offset1:160"
+                       : "=&v"(vv[db]), "=&v"(vv[db + 1]) : "v"(vaddr + (db >> 1) * 2048));
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
         for (int u = 0; u < QT; ++u) {
           if (!act[u]) continue;
