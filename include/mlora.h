@@ -410,6 +410,9 @@ int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v
  * that reader is always an RMSNorm, so the sum is formed there and no extra pass or atomics are needed
  * (results do not depend on scheduling).
  *   mlora_gemv_ksplit          - the number of slices (1..4) this library uses for (T, K, N_total); 1 = no split;
+ *   mlora_gemv_shrink_rows     - what shrink units that ride in the launch (mlora_gemv_frag_acc_ksplit with A) add to
+ *                                N_total in that rule: they occupy workgroups like rows do; a constant allowance
+ *                                (0 without units), so that the slice count does not depend on the adapters of a batch;
  *   mlora_gemv_ksplit_bytes    - size of the partials buffer, part [ks-1][T][N_total] fp32;
  *   mlora_gemv_frag_acc_ksplit - y[T, N_main] (fp32) += xf . Wp^T over slice 0, partials of the other slices to
  *                                `part`.  N_ext > 0: appended rows as in mlora_gemv_frag_split (their slice-0 result
@@ -424,6 +427,7 @@ int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v
  * down_proj linears with the residual add of :79-84) and mlora_rmsnorm (:76-77).
  * ------------------------------------------------------------------------------------------- */
 int mlora_gemv_ksplit(int T, int K, int N_total);
+int mlora_gemv_shrink_rows(int K, int n_proj, int n_ad);
 size_t mlora_gemv_ksplit_bytes(int T, int N_total, int ks);
 int mlora_gemv_frag_acc_ksplit(float* y, float* y2, float* part, int ks, const void* xf, const void* Wp,
                                int T, int K, int N_main, int N_ext,

@@ -57,6 +57,7 @@ SIGNATURES = {
     "mlora_rope_attn_decode": (_i, [_p, _i, _p, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p]),
     "mlora_gemv_ksplit": (_i, [_i, _i, _i]),
     "mlora_gemv_ksplit_bytes": (_z, [_i, _i, _i]),
+    "mlora_gemv_shrink_rows": (_i, [_i, _i, _i]),
     "mlora_gemv_frag_acc_ksplit": (_i, [_p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _p, _p, _i, _p, _i, _i, _p]),
     "mlora_rmsnorm_ksplit": (_i, [_p, _i, _p, _p, _i, _i, _p, _f, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p]),
     "mlora_lora_expand_rmsnorm": (_i, [_p, _i, _p, _p, _i, _p, _p, _f, _p, _f, _i, _i, _i, _i, _i, _p]),

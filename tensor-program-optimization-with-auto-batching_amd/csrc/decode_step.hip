@@ -155,10 +155,13 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
   };
   // K split of the two narrow accumulating GEMVs: the slices' partials are summed by the RMSNorm that reads the
   // residual next.  N_total counts the appended adapter rows of the dense shrink.
+  // Shrink units that ride in the launch count as the workgroups they are (a launch of more workgroups than compute
+  // units ends with a second round on a few of them).
   auto ksplit_of = [&](int K, bool has_lora) -> int {
-    const int n_total = H + (dense && has_lora ? n_ad * r : 0);
+    const int ld_part = H + (dense && has_lora ? n_ad * r : 0);
+    const int n_total = ld_part + (!dense && has_lora ? mlora_gemv_shrink_rows(K, 1, n_ad) : 0);
     const int ks = p->ksplit_ws ? mlora_gemv_ksplit(T, K, n_total) : 1;
-    return ks > 1 && mlora_gemv_ksplit_bytes(T, n_total, ks) <= p->ksplit_ws_bytes ? ks : 1;
+    return ks > 1 && mlora_gemv_ksplit_bytes(T, ld_part, ks) <= p->ksplit_ws_bytes ? ks : 1;
   };
   // o_proj / down_proj: resid += x . W^T with the adapter's shrink riding along (dense: appended rows; else shrink units)
   auto acc_gemv = [&](const void* x, const void* Wp, int K, const mlora_lora_proj& lp, void* v_ws, int ks) -> int {

@@ -554,6 +554,15 @@ extern "C" int mlora_gemv_ksplit(int T, int K, int N_total) {
   return ks < 1 ? 1 : ks;
 }
 
+// What the shrink units that ride in a launch weigh in the K-split rule: sixteen workgroups' worth of rows, whatever
+// the number of adapters - the slice count (and with it the order in which a row's partial sums are added) must not
+// depend on which adapters a batch happens to hold.  Sixteen adapters of rank 16 over K = 4096 are exactly that many
+// workgroups of units; with more, the launch exceeds the compute units by the difference.
+extern "C" int mlora_gemv_shrink_rows(int K, int n_proj, int n_ad) {
+  if (K <= 0 || n_proj <= 0 || n_ad <= 0) return 0;
+  return 256;
+}
+
 extern "C" size_t mlora_gemv_ksplit_bytes(int T, int N_total, int ks) {
   if (T <= 0 || N_total <= 0 || ks <= 1) return 0;
   return (size_t)(ks - 1) * T * N_total * sizeof(float);

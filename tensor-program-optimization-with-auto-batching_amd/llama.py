@@ -304,6 +304,8 @@ class LlamaForCausalLM:
         """hidden [T, H] fp32 (updated in place), tokens in kv.begin_forward order -> logits fp32."""
         s = self.shape
         tok_adapter = tok_adapter or {}
+        # the adapter types of this pass (a batch merged beforehand may name any loaded type)
+        lora_tids = tuple(range(len(self.lora_types))) if "multi" in tok_adapter else tuple(tok_adapter)
         if len(tok_adapter) > 1:            # several adapter types (ranks) in the batch: one multi-rank call per projection
             tok_adapter = self._merge_types(tok_adapter)
         T = hidden.shape[0]
@@ -340,7 +342,7 @@ class LlamaForCausalLM:
             if fuse and self._fused_linear(fuse, attn, L["o"], l, (("o_proj", 0, H),), resid=resid) is not None:
                 parts = None
             else:
-                parts = self._linear_acc(attn, L["o"], resid, ks_ws)
+                parts = self._linear_acc(attn, L["o"], resid, ks_ws, self._riding_rows(l, "o_proj", lora_tids, T, q_sz))
                 if tok_adapter:
                     self._lora(resid, attn, l, "o_proj", tok_adapter)
             xn = ops.rmsnorm(resid, L["ln2"], s.rms_norm_eps, frag=frag, parts=parts)
@@ -361,7 +363,7 @@ class LlamaForCausalLM:
             if fuse and self._fused_linear(fuse, act, L["down"], l, (("down_proj", 0, H),), resid=resid) is not None:
                 parts = None
             else:
-                parts = self._linear_acc(act, L["down"], resid, ks_ws)
+                parts = self._linear_acc(act, L["down"], resid, ks_ws, self._riding_rows(l, "down_proj", lora_tids, T, I))
                 if tok_adapter:
                     self._lora(resid, act, l, "down_proj", tok_adapter)
         if logits_rows is not None:
@@ -436,10 +438,18 @@ class LlamaForCausalLM:
             ws = self._ksplit_buf = torch.empty(need, dtype=torch.float32, device=self.device)
         return ws
 
+    def _riding_rows(self, l, proj, tids, T, K):
+        """What the shrink units of an adapted o_proj / down_proj weigh in the K-split rule of a decode step (the native
+        step launches them with the GEMV; this path keeps the same slice count, hence the same sums).  tids: the
+        adapter types of the pass."""
+        if T > 64 or not any(self.lora_types[t].tables.get((l, proj)) is not None for t in tids):
+            return 0
+        return ops.lib().mlora_gemv_shrink_rows(K, 1, 1)
+
     @staticmethod
-    def _linear_acc(x, W, resid, ks_ws):
+    def _linear_acc(x, W, resid, ks_ws, riding_rows=0):
         if isinstance(x, ops.FragActivation) and isinstance(W, ops.PackedWeight) and ks_ws is not None:
-            return ops.linear_acc_ksplit(x, W, resid, ks_ws)
+            return ops.linear_acc_ksplit(x, W, resid, ks_ws, riding_rows)
         ops.linear(x, W, out=resid, accumulate=True)
         return None
 

@@ -456,16 +456,18 @@ class KSplitParts:
         self.part, self.ks, self.ld = part, ks, ld
 
 
-def linear_acc_ksplit(x: FragActivation, W: PackedWeight, resid: torch.Tensor, ws: torch.Tensor = None):
+def linear_acc_ksplit(x: FragActivation, W: PackedWeight, resid: torch.Tensor, ws: torch.Tensor = None, riding_rows: int = 0):
     """resid [T, N] fp32 += x @ W.T as `linear(..., accumulate=True)`, with K split over several workgroups when the
     library recommends it for this shape and `ws` (fp32 scratch) is large enough: slice 0 lands in resid, the other
     slices in the returned KSplitParts, which the caller hands to the next `rmsnorm(resid, ..., parts=...)`.
-    Returns None when the GEMV ran unsplit."""
+    Returns None when the GEMV ran unsplit.  riding_rows: what the native decode step's launch of this linear carries
+    besides the weight rows (`mlora_gemv_shrink_rows` for the shrink units of an adapted projection) - the slice count
+    follows the same rule here, so that both paths add the same partial sums."""
     T, K = x.shape
     N, K2 = W.shape
     if K2 != K or resid.shape != (T, N) or resid.dtype != torch.float32:
         raise ValueError(f"linear_acc_ksplit: x{x.shape} W{W.shape} resid{tuple(resid.shape)}")
-    ks = lib().mlora_gemv_ksplit(T, K, N) if ws is not None else 1
+    ks = lib().mlora_gemv_ksplit(T, K, N + riding_rows) if ws is not None else 1
     if ks > 1 and ws.numel() * 4 < lib().mlora_gemv_ksplit_bytes(T, N, ks):
         ks = 1
     check(lib().mlora_gemv_frag_acc_ksplit(_dev(resid, torch.float32), None, _dev(ws, torch.float32) if ks > 1 else None, ks,

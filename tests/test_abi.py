@@ -120,6 +120,9 @@ def test_argument_validation_of_fused_and_batched_entry_points():
     assert lib.mlora_gemv_ksplit(33, 11008, 4096) == 4 and lib.mlora_gemv_ksplit(32, 4096, 12288) == 1
     assert lib.mlora_gemv_ksplit(65, 11008, 4096) == 4 and lib.mlora_gemv_ksplit(64, 4096, 4352) == 3
     assert lib.mlora_gemv_ksplit_bytes(32, 4096, 4) == 3 * 32 * 4096 * 4 and lib.mlora_gemv_ksplit_bytes(32, 4096, 1) == 0
+    # shrink units riding in the launch weigh a constant number of rows in that rule (the slice count must not follow the batch)
+    assert lib.mlora_gemv_shrink_rows(4096, 1, 16) == lib.mlora_gemv_shrink_rows(11008, 1, 200) == 256 and lib.mlora_gemv_shrink_rows(4096, 0, 16) == 0
+    assert lib.mlora_gemv_ksplit(32, 4096, 4096 + lib.mlora_gemv_shrink_rows(4096, 1, 16)) == 3
     # K-range blocks of the appended rows in the per-unit split GEMV: 1 where the form does not apply (and without a device)
     assert lib.mlora_gemv_split_kq(32, 4096, 12288, 768) in (1, 4)
     assert lib.mlora_gemv_split_kq(33, 4096, 12288, 768) == 1 and lib.mlora_gemv_split_kq(32, 4096, 1024, 768) == 1
