@@ -22,6 +22,13 @@ constexpr int KSTEP = 32;   // k per MFMA
 
 enum { OUT_F16 = 0, OUT_F32 = 1, OUT_ACC_F32 = 2, OUT_SILU_FRAG = 3 };
 
+// v / d for a uniform divisor 1..4 (the slice counts of a launch): shifts and one multiply instead of the division
+// sequences - a hundred scalar instructions each, three times over - that stood before a workgroup's first load
+__device__ __forceinline__ int udiv_le4(int v, int d) {
+  const unsigned u = (unsigned)v;
+  return (int)(d == 4 ? u >> 2 : d == 3 ? u / 3u : d == 2 ? u >> 1 : u);
+}
+
 // With SHRINK the first `shrink_blocks` workgroups of the launch do LoRA shrink units (one per wave) on the same
 // x instead of a GEMV tile: the adapter work rides in the GEMV launch and finishes long before it does.
 template <int NT, int TT, int OUT, bool PACKED, bool XFRAG, bool SHRINK, int PIPE = 4>   // PIPE: k-steps in flight per wave
@@ -47,8 +54,9 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, (NT * TT > 8 ? 2 : 4)) void gemv_
   // partial tile to part[s - 1][t][n]; whoever reads y next adds the partials in slice order.
   int slice = 0;
   if (ksplit > 1) {
-    slice = bid % ksplit;
-    bid /= ksplit;
+    const int q = udiv_le4(bid, ksplit);
+    slice = bid - q * ksplit;
+    bid = q;
   }
   const int r16 = lane & 15;
   const int kg = lane >> 4;
@@ -92,8 +100,8 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, (NT * TT > 8 ? 2 : 4)) void gemv_
 
   // wave w takes k-steps w, w + 8, w + 16, ...; stage s of this wave is k-step w + 8 s.
   // PIPE stages are always in flight: each buffer is refilled right after it is consumed.
-  const int kb0 = ksplit > 1 ? (int)((long)slice * KB / ksplit) : 0;
-  const int kb1 = ksplit > 1 ? (int)((long)(slice + 1) * KB / ksplit) : KB;
+  const int kb0 = ksplit > 1 ? udiv_le4(slice * KB, ksplit) : 0;
+  const int kb1 = ksplit > 1 ? udiv_le4((slice + 1) * KB, ksplit) : KB;
   const int S = (kb1 - kb0 - wave + GEMV_WAVES - 1) / GEMV_WAVES;
   f16x8 a[PIPE][NT], b[PIPE][TT];
   auto load_stage = [&](int u, int s) {
@@ -302,8 +310,8 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, 2) void gemv_split_cu_kernel(f16*
   const int KB = K / KSTEP;
   const int piece = (int)gridDim.x - 1 - wg;           // pieces are dealt from the last unit backwards
   const bool has_ext = piece < (n_ext / 16) * kq;
-  const int et = has_ext ? piece / kq : 0, eq = has_ext ? piece % kq : 0;
-  const int ekb0 = has_ext ? (int)((long)eq * KB / kq) : 0, ekb1 = has_ext ? (int)((long)(eq + 1) * KB / kq) : 0;
+  const int et = has_ext ? udiv_le4(piece, kq) : 0, eq = has_ext ? piece - et * kq : 0;
+  const int ekb0 = has_ext ? udiv_le4(eq * KB, kq) : 0, ekb1 = has_ext ? udiv_le4((eq + 1) * KB, kq) : 0;
   const f16* wp = W + lane * 8;
   size_t woff[NT];                                     // a missing main tile repeats the first one (cache hits) and is not stored
 #pragma unroll
