@@ -443,13 +443,26 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
   __shared__ __align__(16) f16 knew[D], vnew[D];   // the new token's rotated key and its value
   extern __shared__ float sacc[];                  // [NW][G][D]
 
+  // Three dependent rounds of scalar loads stand before the first page request - the arguments, then what they point at
+  // for this sequence, then its page ids - and every workgroup of the launch waits them out at the same time.  All
+  // arguments are therefore fetched at once (the empty asm statements make the compiler materialise them here instead
+  // of at their first use, each group behind a wait of its own), and the loads of a round are unconditional, with
+  // clamped indices, so that they go out together.
+  asm volatile("" ::"s"(out), "s"(qkv), "s"(k_cache), "s"(v_cache), "s"(block_table), "s"(max_blocks), "s"(seq_ids), "s"(tok_pos));
+  asm volatile("" ::"s"(ctx_len), "s"(rope_cos), "s"(rope_sin), "s"(max_pos), "s"(Hq), "s"(Hkv), "s"(n_pages), "s"(n_seq));
+  asm volatile("" ::"s"(scale), "s"(frag_tt), "s"(lx.src.v), "s"(lx.src.kc), "s"(lx.src.kq), "s"(lx.src.T), "s"(lx.ids), "s"(lx.scaling));
+  asm volatile("" ::"s"(lx.B[0]), "s"(lx.B[1]), "s"(lx.B[2]), "s"(lx.r), "s"(lx.n_ad), "s"(lx.src.n_ad), "s"(lx.src.ld));
   const int b = blockIdx.y, kh = blockIdx.x;
   const int G = Hq / Hkv;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
+  const bool lora = lx.src.v != nullptr;
   const int seq = seq_ids[b];
   const int pos = tok_pos[b];
   int ctx = ctx_len[b];
+  const int id_raw = (lora ? lx.ids : seq_ids)[b];
+  asm volatile("" ::"s"(seq), "s"(pos), "s"(ctx), "s"(id_raw));
+  const int id = lora ? id_raw : -1;
   const bool seq_ok = seq >= 0 && seq < n_seq;
   if (!seq_ok) ctx = 0;
   if (ctx > max_blocks * PAGE) ctx = max_blocks * PAGE;
@@ -457,17 +470,19 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
   const int32_t* __restrict__ bt = block_table + (size_t)(seq_ok ? seq : 0) * max_blocks;
   const bool pos_ok = seq_ok && pos >= 0 && pos < max_pos && pos / PAGE < max_blocks;   // the append condition of rope_kv_append
   const int new_pg = pos_ok ? pos / PAGE : -1, new_slot = pos & (PAGE - 1);
-  const int new_page = pos_ok ? bt[new_pg] : -1;
-  const bool lora = lx.src.v != nullptr;
-  const int id = lora ? lx.ids[b] : -1;
   const bool adapted = lora && id >= 0 && id < lx.n_ad;
 
   // The wave's first TWO pages are requested before anything else: together with the other waves' that is enough traffic
   // to keep the memory system busy for the whole time the new token takes (the second buffer lives in registers the
   // accumulators only need later, and is gone after the second page).
   constexpr bool PF2 = RG <= 2;      // the wide-rank variant has no registers to spare for the second buffer
-  int page = wave < npages ? bt[wave] : -1;
-  const int page2 = PF2 && wave + NW < npages ? bt[wave + NW] : -1;
+  const int e_new = bt[pos_ok ? new_pg : 0];
+  const int e_first = bt[wave < max_blocks ? wave : 0];
+  const int e_second = bt[wave + NW < max_blocks ? wave + NW : 0];
+  asm volatile("" ::"s"(e_new), "s"(e_first), "s"(e_second));
+  const int new_page = pos_ok ? e_new : -1;
+  int page = wave < npages ? e_first : -1;
+  const int page2 = PF2 && wave + NW < npages ? e_second : -1;
   f16x8 kf[NKB], kf2[PF2 ? NKB : 1];
   f16x4 vf[NDB], vf2[PF2 ? NDB : 1];
   auto load_into = [&](f16x8 (&k)[NKB], f16x4 (&v)[NDB], int pgid) {

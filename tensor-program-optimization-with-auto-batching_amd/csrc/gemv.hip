@@ -39,6 +39,9 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, (NT * TT > 8 ? 2 : 4)) void gemv_
   constexpr int TILES = NT * TT;
   constexpr int HT = TILES > 8 ? TILES / 2 : TILES;   // accumulator tiles summed per pass through LDS (64 KiB holds 8)
   __shared__ f32x4 red[GEMV_WAVES][HT][WAVE];
+  // all arguments in one round of scalar loads, ahead of the first weight request (the compiler would fetch each
+  // group at its first use, a dependent round each time)
+  asm volatile("" ::"s"(yv), "s"(x), "s"(ldx), "s"(W), "s"(T), "s"(K), "s"(N), "s"(shrink_blocks), "s"(n_main), "s"(y2), "s"(ksplit), "s"(part));
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps the k-loop control scalar
   const int lane = threadIdx.x & 63;
   int bid = blockIdx.x;
@@ -299,16 +302,17 @@ template <int NM, int TT, int PIPE>
 __global__ __launch_bounds__(GEMV_WAVES* WAVE, 2) void gemv_split_cu_kernel(f16* __restrict__ y, float* __restrict__ y2,
                                                                          const f16* __restrict__ x, const f16* __restrict__ W,
                                                                          int T, int K, int n_main, int n_ext, int base, int rem,
-                                                                         int kq) {
+                                                                         int kq, int n_wg) {   // n_wg: the grid size, as an argument (gridDim comes from a later scalar load)
   constexpr int NT = NM + 1;                           // register tile NM is the piece of an appended tile
   __shared__ f32x4 red[GEMV_WAVES][TT][WAVE];
+  asm volatile("" ::"s"(y), "s"(y2), "s"(x), "s"(W), "s"(T), "s"(K), "s"(n_main), "s"(n_ext), "s"(base), "s"(rem), "s"(kq), "s"(n_wg));   // all arguments (and the grid size) in one round of scalar loads
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int wg = blockIdx.x;
   const int m0 = wg * base + (wg < rem ? wg : rem);    // first main tile of this workgroup
   const int nm = base + (wg < rem ? 1 : 0);            // and how many it has
   const int KB = K / KSTEP;
-  const int piece = (int)gridDim.x - 1 - wg;           // pieces are dealt from the last unit backwards
+  const int piece = n_wg - 1 - wg;                     // pieces are dealt from the last unit backwards
   const bool has_ext = piece < (n_ext / 16) * kq;
   const int et = has_ext ? udiv_le4(piece, kq) : 0, eq = has_ext ? piece - et * kq : 0;
   const int ekb0 = has_ext ? udiv_le4(eq * KB, kq) : 0, ekb1 = has_ext ? udiv_le4((eq + 1) * KB, kq) : 0;
@@ -690,7 +694,7 @@ extern "C" int mlora_gemv_frag_split_kq(void* y, float* y2, int kq, const void* 
   hipStream_t s = (hipStream_t)stream;
 #define MLORA_SPLIT_CU(NM, TT, PIPE)                                                                                       \
   hipLaunchKernelGGL((gemv_split_cu_kernel<NM, TT, PIPE>), g, block, 0, s, (f16*)y, y2, (const f16*)xf, (const f16*)Wp, T, K, \
-                     N_main, N_ext, base, rem, kq)
+                     N_main, N_ext, base, rem, kq, n_cu)
   if (T <= 16) {
     if (per <= 2) MLORA_SPLIT_CU(2, 1, 4);
     else MLORA_SPLIT_CU(3, 1, 4);

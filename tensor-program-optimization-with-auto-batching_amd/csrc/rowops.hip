@@ -51,6 +51,10 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(f16* __restrict__
   __shared__ float lds[NORM_THREADS / WAVE];
   __shared__ float lv[64];
   extern __shared__ float delta[];    // H floats when a LoRA expand is attached, otherwise empty
+  // every argument is fetched now, in one round of scalar loads (left alone, the compiler fetches each group at its
+  // first use, a dependent round each time)
+  asm volatile("" ::"s"(y), "s"(x), "s"(w), "s"(eps), "s"(H), "s"(frag_tt), "s"(lx.src.v), "s"(lx.src.kc), "s"(lx.src.kq), "s"(lx.src.T));
+  asm volatile("" ::"s"(lx.src.n_ad), "s"(lx.src.ld), "s"(lx.B), "s"(lx.ids), "s"(lx.scaling), "s"(lx.r), "s"(lx.n_ad), "s"(kp.p), "s"(kp.n), "s"(kp.ld), "s"(kp.stride));
   const int row = blockIdx.x;
   XT* xr = x + (size_t)row * H;
   // The row and the norm weight are requested first: neither depends on the adapter id, so their latency
