@@ -313,12 +313,17 @@ __global__ __launch_bounds__(NW * WAVE, 4) void paged_attn_decode_kernel(
   __shared__ float sm[NW][16], sl[NW][16];
   extern __shared__ float sacc[];   // [NW][G][D]
 
+  // arguments, then the sequence's scalars, then its first page ids: three grouped rounds of scalar loads (see
+  // rope_attn_decode_kernel)
+  asm volatile("" ::"s"(out), "s"(qkv), "s"(k_cache), "s"(v_cache), "s"(block_table), "s"(max_blocks), "s"(seq_ids), "s"(ctx_len));
+  asm volatile("" ::"s"(Hq), "s"(Hkv), "s"(n_pages), "s"(n_seq), "s"(scale), "s"(frag_tt));
   const int b = blockIdx.y, kh = blockIdx.x;
   const int G = Hq / Hkv;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
   const int seq = seq_ids[b];
   int ctx = ctx_len[b];
+  asm volatile("" ::"s"(seq), "s"(ctx));
   if (seq < 0 || seq >= n_seq) ctx = 0;
   if (ctx > max_blocks * PAGE) ctx = max_blocks * PAGE;
   const int npages = (ctx + PAGE - 1) / PAGE;
@@ -339,7 +344,8 @@ __global__ __launch_bounds__(NW * WAVE, 4) void paged_attn_decode_kernel(
 #pragma unroll
   for (int db = 0; db < NDB; ++db) O[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  int page = wave < npages ? bt[wave] : -1;
+  const int e_first = bt[wave < max_blocks ? wave : 0];
+  int page = wave < npages ? e_first : -1;
   for (int pg = wave; pg < npages; pg += NW) {
     const int next = pg + NW < npages ? bt[pg + NW] : -1;   // the next page id is requested one page ahead
     if (page >= 0 && page < n_pages) {                      // wave-uniform
