@@ -145,9 +145,16 @@ __device__ __forceinline__ void lora_shrink_unit(const LoraShrinkBatch& b, int u
 
 // v[j] = scaling * sum_c v_part[c][t][j] for one token, summed in slice order (the order every consumer uses,
 // so fused and stand-alone expands agree bit for bit).
+// The slices are requested together and then added one by one: as a loop over kc, every addition waited for its own
+// load - up to eight dependent round trips in front of an expand.
 __device__ __forceinline__ float lora_v(const float* __restrict__ vpart_proj, int kc, int T, int r, int t, int j, float scaling) {
+  float part[LORA_MAX_KC];
+#pragma unroll
+  for (int c = 0; c < LORA_MAX_KC; ++c) part[c] = c < kc ? vpart_proj[((size_t)c * T + t) * r + j] : 0.f;
   float v = 0.f;
-  for (int c = 0; c < kc; ++c) v += vpart_proj[((size_t)c * T + t) * r + j];
+#pragma unroll
+  for (int c = 0; c < LORA_MAX_KC; ++c)
+    if (c < kc) v += part[c];
   return v * scaling;
 }
 
@@ -164,8 +171,13 @@ struct LoraVSource {
 __device__ __forceinline__ float lora_v_from(const LoraVSource& s, int slot, int id, int r, int t, int j, float scaling) {
   if (s.kc > 0) return lora_v(s.v + (size_t)slot * s.kc * s.T * r, s.kc, s.T, r, t, j, scaling);
   const float* __restrict__ p = s.v + (size_t)t * s.ld + ((size_t)slot * s.n_ad + id) * r + j;
-  float a = p[0];
-  for (int q = 1; q < s.kq; ++q) a += p[(size_t)q * s.T * s.ld];
+  float part[LORA_MAX_KQ];
+#pragma unroll
+  for (int q = 0; q < LORA_MAX_KQ; ++q) part[q] = q == 0 || q < s.kq ? p[(size_t)q * s.T * s.ld] : 0.f;   // all blocks requested together
+  float a = part[0];
+#pragma unroll
+  for (int q = 1; q < LORA_MAX_KQ; ++q)
+    if (q < s.kq) a += part[q];
   return a * scaling;
 }
 
