@@ -472,6 +472,19 @@ __device__ __forceinline__ const f16* x_operand(const f16* __restrict__ x, int t
   return x + (size_t)t * K + g * 8;
 }
 
+// sum over the K ranges of a shrink's partial results, four rank entries at a time, in range order; the ranges are
+// requested together (a loop with a load and an addition per turn waits out a round trip per range)
+__device__ __forceinline__ f32x4 sum_ranges(const float* __restrict__ p, int splits, size_t stride) {
+  f32x4 part[LORA_MAX_KC];
+#pragma unroll
+  for (int sp = 0; sp < LORA_MAX_KC; ++sp) part[sp] = sp < splits ? *reinterpret_cast<const f32x4*>(p + sp * stride) : f32x4{0.f, 0.f, 0.f, 0.f};
+  f32x4 sum = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int sp = 0; sp < LORA_MAX_KC; ++sp)
+    if (sp < splits) sum += part[sp];
+  return sum;
+}
+
 template <int R>
 __device__ __forceinline__ void shrink_tile_mfma(float* __restrict__ v, const f16* __restrict__ x, int frag_tt, const f16* __restrict__ A,
                                                  const int32_t* __restrict__ ids, int T, int K, int n_ad,
@@ -738,7 +751,7 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE, 2) void lora_expand_pair_mfma_ker
     f32x4 sum = f32x4{0.f, 0.f, 0.f, 0.f};
     if ((todo[u] >> tok) & 1u) {
       const int t = t0[u] + tok;
-      for (int sp = 0; sp < splits; ++sp) sum += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + t) * R + j);
+      sum = sum_ranges(v + (size_t)t * R + j, splits, (size_t)T * R);
 #pragma unroll
       for (int q = 0; q < 4; ++q) sum[q] *= scaling;
     }
@@ -926,11 +939,9 @@ __global__ __launch_bounds__(SEG_WAVES * WAVE) void lora_expand_mixed_mfma_kerne
     for (int e = 0; e < 8; ++e) f[e] = 0.f;
     // rows of unadapted tokens are never read (their v holds nothing) and enter the product as zeros
     if (j < R && id >= 0) {
-      f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
-      for (int sp = 0; sp < splits; ++sp) {           // the K-range partials of the shrink, summed in range order
-        lo += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + tl) * R + j);
-        hi += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + tl) * R + j + 4);
-      }
+      // the K-range partials of the shrink, summed in range order
+      const f32x4 lo = sum_ranges(v + (size_t)tl * R + j, splits, (size_t)T * R);
+      const f32x4 hi = sum_ranges(v + (size_t)tl * R + j + 4, splits, (size_t)T * R);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         f[e] = lo[e] * scaling;
@@ -1311,8 +1322,7 @@ __global__ __launch_bounds__(256) void lora_v_split_kernel(VSplitOut o, const fl
   if (t >= T) return;
   const int pj = blockIdx.y;
   v += (size_t)pj * splits * T * R;
-  f32x4 sum = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int sp = 0; sp < splits; ++sp) sum += *reinterpret_cast<const f32x4*>(v + ((size_t)sp * T + t) * R + j);
+  const f32x4 sum = sum_ranges(v + (size_t)t * R + j, splits, (size_t)T * R);
   f16x4 h, l;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
