@@ -430,6 +430,16 @@ void launch_gemv(void* y, int out, const f16* x, int ldx, const f16* W, int T, i
 // traffic and the time of a launch follows the most loaded compute unit: wide matrices (>= 768 tiles) take four tiles
 // per wave, which keeps one or two equal workgroups on every unit; narrow ones one tile (or, with a partials buffer,
 // four tiles and a K split - see mlora_gemv_ksplit).
+// compute units of the current device (0 if it cannot be asked), read once
+int gemv_n_cu() {
+  static const int n_cu = [] {
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cu = 0;
+    return cu;
+  }();
+  return n_cu;
+}
+
 template <bool PACKED, bool XFRAG, bool SHRINK = false>
 int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K, int N, void* stream,
                   const LoraShrinkBatch& sb = LoraShrinkBatch(), int n_main = -1, float* y2 = nullptr, int ksplit = 1,
@@ -442,6 +452,14 @@ int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const 
   const int tiles = ceil_div(N, 16);
   if constexpr (PACKED && XFRAG) {
     if (T <= 32 && (ksplit > 1 || tiles >= 768)) {
+      // three tiles per workgroup where that gives every compute unit exactly one workgroup's worth or less (768 tiles on
+      // 256 units: with four tiles a quarter of the units would stay idle and the others set the time); same bits
+      const int n_cu = gemv_n_cu();
+      if (ksplit == 1 && n_cu > 0 && tiles % 3 == 0 && tiles / 3 <= n_cu && ceil_div(tiles, 4) < tiles / 3) {
+        if (T <= 16) launch_gemv<3, 1, PACKED, XFRAG, SHRINK, 4>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part);
+        else launch_gemv<3, 2, PACKED, XFRAG, SHRINK, 4>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part);
+        return mlora_launch_status("gemv");
+      }
       if (T <= 16) launch_gemv<4, 1, PACKED, XFRAG, SHRINK, 4>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part);
       else launch_gemv<4, 2, PACKED, XFRAG, SHRINK, 3>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part);
       return mlora_launch_status("gemv");
@@ -603,16 +621,6 @@ extern "C" int mlora_gemv_frag_acc_ksplit(float* y, float* y2, float* part, int 
                                            shrink_batch(xf, v_part, A, n_proj, tok_adapter, T, K, r, n_ad), N_main, y2, ks, part);
   return gemv_dispatch<true, true, false>(y, MLORA_F32, MLORA_ACCUMULATE, xf, K, Wp, T, K, N, stream, LoraShrinkBatch(), N_main, y2,
                                           ks, part);
-}
-
-// compute units of the current device (0 if it cannot be asked), read once
-static int gemv_n_cu() {
-  static const int n_cu = [] {
-    int dev = 0, cu = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cu = 0;
-    return cu;
-  }();
-  return n_cu;
 }
 
 extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p, int T, int K, int I, void* stream) {
