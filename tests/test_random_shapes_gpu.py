@@ -274,6 +274,48 @@ def _gather_mm_float64(y0, x, A, B, ids, s):
     return ref
 
 
+def test_append_of_many_single_tokens_equals_the_small_batch_kernel():
+    """A decode step of 65 to 300 sequences appends one token each through the 16-token tile kernel (tokens of a tile in
+    different sequences and pages, slots anywhere in a page, a ragged last tile, rows without a valid sequence): the
+    rotated q, and every byte of the K and V caches, equal those written by the per-token kernel that serves up to 64
+    tokens, called on the same tokens in pieces."""
+    ops, kvm = load_pkg("ops"), load_pkg("kv_cache")
+    rng = np.random.default_rng(20241125)
+    for case in range(12):
+        D = int(rng.choice([64, 128])); Hkv = int(rng.choice([1, 2, 8])); Hq = Hkv * int(rng.choice([1, 4]))
+        T = int(rng.choice([65, 96, 129, 200, 256, 300]))
+        max_blocks = 6
+        pos = rng.integers(0, max_blocks * 16, size=T)
+        pos[: min(T, 8)] = [0, 15, 16, 31, 32, 47, 95, 80][: min(T, 8)]
+        n_seq = T + 3
+        rows = rng.permutation(n_seq)[:T].astype(np.int32)
+        bad = rng.choice(T, size=3, replace=False)
+        rows[bad[0]] = -1                       # no sequence
+        pos[bad[1]] = max_blocks * 16 + 5       # position outside the table
+        n_pages = n_seq * max_blocks + 1
+        table = rng.permutation(n_pages - 1)[: n_seq * max_blocks].reshape(n_seq, max_blocks).astype(np.int32)
+        table[rows[bad[2]], min(pos[bad[2]] // 16, max_blocks - 1)] = -1    # page never assigned
+        tag = f"case {case}: T={T} Hq={Hq} Hkv={Hkv} D={D}"
+        print(tag, flush=True)
+        cos, sin = kvm.rope_tables(D, 10000.0, max_blocks * 16)
+        cosd, sind = torch.from_numpy(cos).to(DEV), torch.from_numpy(sin).to(DEV)
+        tab = torch.tensor(table, device=DEV)
+        g = torch.Generator(device="cpu").manual_seed(77 + case)
+        k0 = torch.randn((n_pages, Hkv, D // 32, 4, 16, 8), generator=g).half().to(DEV)
+        v0 = torch.randn((n_pages, Hkv, D, 16), generator=g).half().to(DEV)
+        qkv0 = torch.randn((T, Hq + 2 * Hkv, D), generator=g).half().to(DEV)
+        ts, tp = torch.tensor(rows, device=DEV), torch.tensor(pos.astype(np.int32), device=DEV)
+        k1, v1, q1 = k0.clone(), v0.clone(), qkv0.clone()
+        ops.rope_kv_append(q1, k1, v1, tab, ts, tp, cosd, sind, Hq, Hkv, D)
+        k2, v2, q2 = k0.clone(), v0.clone(), qkv0.clone()
+        for a in range(0, T, 50):
+            b = min(T, a + 50)
+            ops.rope_kv_append(q2[a:b], k2, v2, tab, ts[a:b].contiguous(), tp[a:b].contiguous(), cosd, sind, Hq, Hkv, D)
+        torch.cuda.synchronize()
+        assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(v1, v2), tag
+        assert not torch.equal(k1, k0) and not torch.equal(v1, v0), tag
+
+
 def test_lora_and_linear_kernels_on_random_shapes():
     """160 random draws over three families: the gather-matmul (1 to 2100 tokens: one-launch, vector and matrix-core
     paths; fp16 and fp32 y; row-major and fragment-ordered x; scattered ids and adapter segments) against a per-token
