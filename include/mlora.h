@@ -237,8 +237,8 @@ int mlora_gemm_frag_preferred(int T, int K, int N);
  *                               else tok_adapter[t]: the ids a separate mlora_gather_mm still has to serve;
  *   mlora_lora_shrink_split   - the matrix-core shrink of n_proj <= 3 projections that read the same x, then
  *                               v_hi[p], v_lo[p] [T][r] fp16 (r in {32, 64}); workspace: n_proj *
- *                               mlora_gather_mm_workspace_bytes(T, K, r) bytes; rows of tokens without adapter hold
- *                               nothing meaningful and are not read by mlora_linear_frag_lora;
+ *                               mlora_gather_mm_workspace_bytes(T, K, r) bytes; rows of tokens without adapter
+ *                               (id outside [0, n_ad)) are zero, so such a token gets a zero delta;
  *   mlora_linear_frag_lora    - mlora_linear_frag on a shape that mlora_gemm_frag_preferred accepts, with up to three
  *                               projections = row ranges [n_begin, n_begin + n_rows) of the fused weight (on 256-row
  *                               boundaries), each with its B table [n_ad][n_rows][r] and its v halves.
@@ -315,8 +315,10 @@ int mlora_argmax(int32_t* ids, const float* logits, int B, int V, void* stream);
  * mlora_paged_attn_prefill: query token t (sequence tok_seq[t], position tok_pos[t]) attends to cached
  *   positions 0..tok_pos[t]; tokens of a sequence must be consecutive in t with increasing positions.
  * The attention kernels multiply whole pages and mask afterwards: every slot of a page that a block table names
- * must hold finite numbers before its first use (allocate the cache zero-filled), or P = 0 times a non-finite V
- * turns the output into NaN.
+ * must hold finite numbers before its first use, or P = 0 times a non-finite V turns the output into NaN.  The
+ * prefill kernel also reads PAGE 0 in place of every page slot past a sequence's end (and of a page id outside
+ * [0, n_pages)), again with P = 0: page 0 must hold finite numbers whether or not a block table names it.
+ * Allocating the whole cache zero-filled satisfies both.
  * q is read from qkv (already rotated).  out [T, Hq * D] f16 in out_layout.  D in {64, 128};
  * Hq % Hkv == 0, Hq / Hkv <= 16 and B <= 65535 for decode.
  * ------------------------------------------------------------------------------------------- */

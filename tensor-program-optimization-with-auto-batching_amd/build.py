@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmlora_hip.so")
 SOURCES = ["api.hip", "gather_mm.hip", "gather_mm_batch.hip", "gemv.hip", "gemm.hip", "rowops.hip", "attention.hip", "decode_step.hip"]
-FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", 
+FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-mllvm", "-amdgpu-kernarg-preload-count=16",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 

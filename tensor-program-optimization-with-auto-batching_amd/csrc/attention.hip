@@ -1243,12 +1243,11 @@ extern "C" int mlora_paged_attn_prefill(void* out, int out_layout, const void* q
 #define MLORA_PREFILL(DD)                                                                                                          \
   do {                                                                                                                             \
     constexpr size_t lds = (size_t)PF_RING * 2 * PF_PAGES * PAGE * DD * sizeof(f16);                                                    \
-    static bool configured = false; /* the attribute is per kernel, set once per process */                                       \
-    if (!configured) {                                                                                                             \
-      hipError_t e = hipFuncSetAttribute((const void*)paged_attn_prefill_block_kernel<DD>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
-      if (e != hipSuccess) return mlora_set_error(MLORA_ERR_LAUNCH, "paged_attn_prefill: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e)); \
-      configured = true;                                                                                                           \
-    }                                                                                                                              \
+    /* the attribute is per kernel, set once per process; a local static is initialised by one thread */                           \
+    static const hipError_t configured =                                                                                           \
+        hipFuncSetAttribute((const void*)paged_attn_prefill_block_kernel<DD>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+    if (configured != hipSuccess)                                                                                                  \
+      return mlora_set_error(MLORA_ERR_LAUNCH, "paged_attn_prefill: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(configured)); \
     hipLaunchKernelGGL(paged_attn_prefill_block_kernel<DD>, grid, dim3(PF_WAVES * WAVE), lds, s, (f16*)out, frag_tt, (const f16*)qkv, \
                        (const f16*)k_cache, (const f16*)v_cache, block_table, max_blocks, tok_seq, tok_pos, T, Hq, Hkv, n_pages, n_seq, scale); \
   } while (0)

@@ -71,7 +71,6 @@ int decode_step_wide(const mlora_decode_plan* p, void* stream) {
   STEP(mlora_embed(p->resid, MLORA_F32, p->embed, p->tokens, T, H, p->vocab, stream));
   for (int l = 0; l < p->n_layers; ++l) {
     const mlora_layer& L = p->layers[l];
-    MLORA_CHECK(L.gate_up_p, MLORA_ERR_INVALID, "decode_step: layer %d needs gate_up_p", l);
     STEP(norm(L.ln1, pending_ks));
     STEP(mlora_linear_frag(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, stream));
     {
@@ -124,6 +123,20 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
   MLORA_CHECK(p->tokens && p->rows && p->pos && p->ctx && p->resid && p->xn && p->qkv && p->attn && p->gate_up && p->act &&
                   p->logits && p->embed && p->norm && p->lm_head_p && p->block_table && p->rope_cos && p->rope_sin,
               MLORA_ERR_INVALID, "decode_step: null buffer");
+  // every layer of the plan is looked at before the first launch: a rejected call enqueues nothing
+  {
+    const bool any_lora = p->tok_adapter != nullptr && p->lora_r > 0;
+    for (int l = 0; l < p->n_layers; ++l) {
+      const mlora_layer& L = p->layers[l];
+      MLORA_CHECK(L.ln1 && L.ln2 && L.qkv_p && L.o_p && L.down_p && L.k_cache && L.v_cache, MLORA_ERR_INVALID,
+                  "decode_step: layer %d has a null weight, norm or cache pointer", l);
+      const bool gu_lora = any_lora && (L.lora[MLORA_GATE].A || L.lora[MLORA_UP].A);
+      MLORA_CHECK(L.gate_up_p || (T <= 64 && L.gate_up_il_p && !gu_lora), MLORA_ERR_INVALID, "decode_step: layer %d needs gate_up_p", l);
+      if (any_lora)
+        for (int j = 0; j < 7; ++j)
+          MLORA_CHECK(!L.lora[j].A || L.lora[j].B, MLORA_ERR_INVALID, "decode_step: layer %d projection %d has A but no B table", l, j);
+    }
+  }
   if (T > 64) {
     MLORA_CHECK(!(p->tok_adapter != nullptr && p->lora_r > 0 && p->lora_dense != 0), MLORA_ERR_UNSUPPORTED,
                 "decode_step: the dense shrink (adapter rows appended to the base weights) serves at most 64 sequences (T=%d)", T);
@@ -213,7 +226,6 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
     if (L.gate_up_il_p && !gu_lora) {
       STEP(mlora_gemv_frag_silu(p->act, p->xn, L.gate_up_il_p, T, H, I, stream));
     } else {
-      MLORA_CHECK(L.gate_up_p, MLORA_ERR_INVALID, "decode_step: layer %d needs gate_up_p", l);
       STEP(mlora_gemv_frag(gu, MLORA_F16, MLORA_STORE, p->xn, L.gate_up_p, T, H, 2 * I, stream));
       STEP(delta(gu, MLORA_F16, 2 * I, p->xn, L.lora[MLORA_GATE], H, I));
       STEP(delta(gu + I, MLORA_F16, 2 * I, p->xn, L.lora[MLORA_UP], H, I));

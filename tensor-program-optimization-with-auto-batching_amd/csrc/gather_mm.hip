@@ -1316,19 +1316,26 @@ struct VSplitOut {
   f16* vl[SEG_MAX_PROJ];
 };
 template <int R>
-__global__ __launch_bounds__(256) void lora_v_split_kernel(VSplitOut o, const float* __restrict__ v, int splits, float scaling, int T) {
+__global__ __launch_bounds__(256) void lora_v_split_kernel(VSplitOut o, const float* __restrict__ v, int splits, float scaling, int T,
+                                                           const int32_t* __restrict__ ids, int n_ad) {
   const int e = blockIdx.x * 256 + threadIdx.x;              // four rank entries of one token
   const int t = e / (R / 4), j = (e % (R / 4)) * 4;
   if (t >= T) return;
   const int pj = blockIdx.y;
   v += (size_t)pj * splits * T * R;
-  const f32x4 sum = sum_ranges(v + (size_t)t * R + j, splits, (size_t)T * R);
-  f16x4 h, l;
+  // the shrink writes rows of adapted tokens only: a token without adapter gets zeros here (what the workspace holds
+  // in its row is left over from earlier calls), so that its delta in a block of the extra-k-step linear is zero
+  const int id = ids[t];
+  const bool adapted = id >= 0 && id < n_ad;
+  f16x4 h = f16x4{0, 0, 0, 0}, l = h;
+  if (adapted) {
+    const f32x4 sum = sum_ranges(v + (size_t)t * R + j, splits, (size_t)T * R);
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const float f = sum[q] * scaling;
-    h[q] = (f16)f;
-    l[q] = (f16)(f - (float)h[q]);
+    for (int q = 0; q < 4; ++q) {
+      const float f = sum[q] * scaling;
+      h[q] = (f16)f;
+      l[q] = (f16)(f - (float)h[q]);
+    }
   }
   *reinterpret_cast<f16x4*>(o.vh[pj] + (size_t)t * R + j) = h;
   *reinterpret_cast<f16x4*>(o.vl[pj] + (size_t)t * R + j) = l;
@@ -1618,8 +1625,8 @@ extern "C" int mlora_lora_shrink_split(void* const* v_hi, void* const* v_lo, con
     vo.vl[i] = (f16*)v_lo[i];
   }
   const dim3 grid(ceil_div(T * (r / 4), 256), n_proj);
-  if (r == 32) hipLaunchKernelGGL((lora_v_split_kernel<32>), grid, dim3(256), 0, s, vo, v, splits, scaling, T);
-  else hipLaunchKernelGGL((lora_v_split_kernel<64>), grid, dim3(256), 0, s, vo, v, splits, scaling, T);
+  if (r == 32) hipLaunchKernelGGL((lora_v_split_kernel<32>), grid, dim3(256), 0, s, vo, v, splits, scaling, T, tok_adapter, n_ad);
+  else hipLaunchKernelGGL((lora_v_split_kernel<64>), grid, dim3(256), 0, s, vo, v, splits, scaling, T, tok_adapter, n_ad);
   return mlora_launch_status("lora_shrink_split");
 }
 

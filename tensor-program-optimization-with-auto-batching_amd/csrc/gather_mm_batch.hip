@@ -119,6 +119,148 @@ __global__ __launch_bounds__(LORA_MAX_KC* WAVE, (RESIDENT ? 4 : 2)) void gmm_bat
   }
 }
 
+// Pass 1 as a persistent launch: one workgroup per compute unit walks (set, adapter in use) pairs, and the whole of pair
+// i + 1 - the wave's slice of A[a], 16 rows, and the x rows of a's first two tokens - is requested before pair i is
+// reduced.  As one short-lived workgroup per pair, every pair paid its own memory round trips with an empty pipeline
+// (table row, set pointers, then A and x); here a workgroup pays them once per launch: the token->adapter table is
+// the same for all sets, so the adapters in use and their token masks are found once, the set pointers of a
+// workgroup's pairs are fetched 64 pairs at a time, one pair per lane, and handed out by lane reads, and adapters
+// without a token cost nothing.  The arithmetic of a pair is that of gmm_batch_shrink_kernel<true>: the same bits.
+struct ShrinkPair {
+  f16x8 a[16];           // the wave's K-slice of the adapter's 16 rows of A (rows past the rank are zero)
+  f16x8 x0, x1;          // the slice of the x rows of the adapter's first two tokens
+  const f16* x;          // x of the pair's set
+  unsigned long long mask;
+  int set;
+};
+
+__global__ __launch_bounds__(LORA_MAX_KC* WAVE, 1) void gmm_batch_shrink_pers_kernel(BatchArgs a, int n_sets) {
+  extern __shared__ float part_all[];           // [2][kc][T][r]: the partials of a pair, double buffered
+  __shared__ unsigned long long s_mask[WAVE];
+  __shared__ int s_used[WAVE];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int r = a.r, K = a.K, T = a.T, kc = a.kc;
+  constexpr int G = 16;
+  const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  const int raw = lane < T ? a.ids[lane] : -1;
+  const int id = (raw >= 0 && raw < a.n_ad) ? raw : -1;
+  // the adapters in use, in the order of their first token, with the tokens of each (every wave finds the same list)
+  int n_used = 0;
+  for (unsigned long long todo = __ballot(id >= 0); todo;) {
+    const int ad = __builtin_amdgcn_readlane(id, __builtin_ctzll(todo));
+    const unsigned long long m = __ballot(id == ad);
+    if (threadIdx.x == 0) {
+      s_used[n_used] = ad;
+      s_mask[n_used] = m;
+    }
+    ++n_used;
+    todo &= ~m;
+  }
+  __syncthreads();
+  const int total = n_sets * n_used;
+  const int n_wg = gridDim.x, wg = blockIdx.x;
+  const int my_pairs = wg < total ? (total - wg + n_wg - 1) / n_wg : 0;
+  const int kbase = wave * LORA_KCHUNK + lane * 8;
+  const bool in = kbase < K;
+  const size_t part_sz = (size_t)kc * T * r;
+
+  for (int c0 = 0; c0 < my_pairs; c0 += WAVE) {
+    // lane l holds where pair c0 + l of this workgroup lives
+    const int qi = c0 + lane;
+    unsigned long long pA = 0, px = 0;
+    int pu = 0, pset = 0;
+    if (qi < my_pairs) {
+      const int q = wg + qi * n_wg;
+      pset = q / n_used;
+      pu = q - pset * n_used;
+      const GmmSet* sp = a.sets + pset;
+      pA = (unsigned long long)sp->A;
+      px = (unsigned long long)sp->x;
+    }
+    const int nchunk = my_pairs - c0 < WAVE ? my_pairs - c0 : WAVE;
+    auto lane_u64 = [](unsigned long long v, int l) -> unsigned long long {
+      const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)v, l);
+      const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(v >> 32), l);
+      return ((unsigned long long)hi << 32) | lo;
+    };
+    auto fetch = [&](int i, ShrinkPair& P) {
+      const int u = __builtin_amdgcn_readlane(pu, i);
+      P.set = __builtin_amdgcn_readlane(pset, i);
+      P.x = (const f16*)lane_u64(px, i);
+      P.mask = s_mask[u];
+      const f16* __restrict__ A = (const f16*)lane_u64(pA, i) + (size_t)s_used[u] * r * K;
+      unsigned long long m = P.mask;
+      const int t0 = __builtin_ctzll(m);
+      m &= m - 1;
+      const int t1 = m ? __builtin_ctzll(m) : t0;
+      // x ahead of A: loads come back in request order, so the products of row j can start as soon as row j is in
+      P.x0 = in ? x_slice(P.x, t0, kbase, K, a.frag_tt) : zero8;
+      P.x1 = in ? x_slice(P.x, t1, kbase, K, a.frag_tt) : zero8;
+#pragma unroll
+      for (int j = 0; j < G; ++j) P.a[j] = (j < r && in) ? ld8(A + (size_t)j * K + kbase) : zero8;
+    };
+    auto reduce = [&](ShrinkPair& P, int buf) {
+      float* __restrict__ pb = part_all + (size_t)buf * part_sz;
+      float* __restrict__ vp = pb + (size_t)wave * T * r;
+      unsigned long long m = P.mask;
+      int t0 = __builtin_ctzll(m);
+      m &= m - 1;
+      int t1 = -1;
+      if (m) {
+        t1 = __builtin_ctzll(m);
+        m &= m - 1;
+      }
+      f16x8 x0 = P.x0, x1 = P.x1;
+      while (true) {
+        int n0 = -1, n1 = -1;                    // the adapter's next token pair: requested now, used in the next round
+        f16x8 y0 = zero8, y1 = zero8;
+        if (m) {
+          n0 = __builtin_ctzll(m);
+          m &= m - 1;
+          if (m) {
+            n1 = __builtin_ctzll(m);
+            m &= m - 1;
+          }
+          if (in) {
+            y0 = x_slice(P.x, n0, kbase, K, a.frag_tt);
+            y1 = x_slice(P.x, n1 >= 0 ? n1 : n0, kbase, K, a.frag_tt);
+          }
+        }
+        float p0[G], p1[G];
+#pragma unroll
+        for (int j = 0; j < G; ++j) {
+          p0[j] = dot8(P.a[j], x0, 0.f);
+          p1[j] = dot8(P.a[j], x1, 0.f);
+        }
+        const int j0 = reduce_transpose<G>(p0, lane);
+        if (j0 < r && (lane & (WAVE / G - 1)) == 0) vp[(size_t)t0 * r + j0] = p0[0];
+        const int j1 = reduce_transpose<G>(p1, lane);
+        if (t1 >= 0 && j1 < r && (lane & (WAVE / G - 1)) == 0) vp[(size_t)t1 * r + j1] = p1[0];
+        if (n0 < 0) break;
+        t0 = n0; t1 = n1; x0 = y0; x1 = y1;
+      }
+      __syncthreads();
+      // the slices' partials, added in slice order and scaled; the other buffer is free for the next pair meanwhile
+      float* __restrict__ vout = a.ws + (size_t)P.set * a.ws_stride;
+      for (int e = threadIdx.x; e < T * r; e += blockDim.x) {
+        const int t = e / r, j = e % r;
+        if ((P.mask >> t) & 1) vout[e] = lora_v(pb, kc, T, r, t, j, a.scaling);
+      }
+    };
+    if (c0 > 0) __syncthreads();                 // the previous chunk's last pair may still be read from buffer 0
+    ShrinkPair P0, P1;
+    fetch(0, P0);
+    for (int i = 0; i < nchunk; i += 2) {
+      if (i + 1 < nchunk) fetch(i + 1, P1);
+      reduce(P0, 0);
+      if (i + 1 < nchunk) {
+        if (i + 2 < nchunk) fetch(i + 2, P0);
+        reduce(P1, 1);
+      }
+    }
+  }
+}
+
 template <typename YT, int N>
 struct YRow;
 template <> struct YRow<f16, 8> { typedef f16x8 type; };
@@ -310,7 +452,18 @@ int gmm_batch_stream(const GmmSet* sets, int n_sets, int y_dtype, int ldy, int x
   // otherwise only the adapters in use are read.
   int speculate = n_ad <= T / 2;
   const size_t lds = (size_t)ks.kc * T * r * sizeof(float);
-  if (r <= 16 && ks.ci == 1) hipLaunchKernelGGL(gmm_batch_shrink_kernel<true>, dim3(n_ad, n_sets), dim3(ks.kc * WAVE), lds, s, a, speculate);
+  // enough pairs for two or more per compute unit: the persistent form (two partial buffers; its LDS is reserved once)
+  static const int n_cu = [] {
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cu = 0;
+    return cu;
+  }();
+  static const hipError_t pers_lds =
+      hipFuncSetAttribute((const void*)gmm_batch_shrink_pers_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * LORA_MAX_KC * WAVE * 16 * (int)sizeof(float));
+  const int pairs_est = n_sets * (n_ad < T ? n_ad : T);
+  if (r <= 16 && ks.ci == 1 && n_cu > 0 && pers_lds == hipSuccess && pairs_est >= 2 * n_cu)
+    hipLaunchKernelGGL(gmm_batch_shrink_pers_kernel, dim3(n_cu), dim3(ks.kc * WAVE), 2 * lds, s, a, n_sets);
+  else if (r <= 16 && ks.ci == 1) hipLaunchKernelGGL(gmm_batch_shrink_kernel<true>, dim3(n_ad, n_sets), dim3(ks.kc * WAVE), lds, s, a, speculate);
   else hipLaunchKernelGGL(gmm_batch_shrink_kernel<false>, dim3(n_ad, n_sets), dim3(ks.kc * WAVE), lds, s, a, 0);
   switch (r) {
     case 8: launch_expand<8>(a, n_sets, y_dtype, speculate, s); break;

@@ -648,13 +648,15 @@ template <int OUT>
 int launch_gemm_pp(void* y, const f16* x, int ldx, int x_tt, const f16* Wp, int T, int K, int N, hipStream_t s,
                    const PPLora& lo = PPLora()) {
   constexpr size_t lds = ((size_t)PP_STAGES * PP_STAGE_ELEMS + (size_t)PP_WAVES * PP_OUT_ELEMS) * sizeof(f16);
-  static bool configured = false;                    // the attribute is per kernel, set once per process
-  if (!configured) {
+  // the attribute is per kernel, set once per process (the initialiser of a local static runs once, also when several
+  // host threads make their first call together)
+  static const hipError_t configured = [] {
     hipError_t e = hipFuncSetAttribute((const void*)gemm_pp_kernel<OUT, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e == hipSuccess) e = hipFuncSetAttribute((const void*)gemm_pp_kernel<OUT, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return mlora_set_error(MLORA_ERR_LAUNCH, "gemm_packed: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-    configured = true;
-  }
+    return e;
+  }();
+  if (configured != hipSuccess)
+    return mlora_set_error(MLORA_ERR_LAUNCH, "gemm_packed: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(configured));
   const int gx = OUT == OUT_SILU ? ceil_div(N / 2, PP_F * 8) : ceil_div(N, PP_F * 16), gy = ceil_div(T, PP_F * 16);
   int n_cu = gemm_n_cu();
   if (n_cu <= 0) n_cu = 256;
@@ -901,12 +903,10 @@ int launch_gemm_mid_shape(void* y, float* part, int ld_part, int ksplit, const f
                           hipStream_t s) {
   constexpr size_t lds = (size_t)(FT == 16 ? 3 : 4) * MID_KS * (FN + FT) * 512 * sizeof(f16);
   static_assert(lds >= (size_t)PP_WAVES * PP_OUT_ELEMS * sizeof(f16), "the output staging fits the ring");
-  static bool configured = false;                    // the attribute is per kernel, set once per process
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_mid_kernel<OUT, FT, FN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return mlora_set_error(MLORA_ERR_LAUNCH, "linear_frag: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-    configured = true;
-  }
+  static const hipError_t configured =               // the attribute is per kernel, set once per process, by one thread
+      hipFuncSetAttribute((const void*)gemm_mid_kernel<OUT, FT, FN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (configured != hipSuccess)
+    return mlora_set_error(MLORA_ERR_LAUNCH, "linear_frag: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(configured));
   const dim3 grid(ceil_div(N, FN * 16), ksplit, ceil_div(T, FT * 16));
   hipLaunchKernelGGL((gemm_mid_kernel<OUT, FT, FN>), grid, dim3(PP_WAVES * WAVE), lds, s, y, part, ld_part, xf, x_tt, Wp, T, K, N);
   return MLORA_OK;
@@ -926,12 +926,11 @@ int launch_gemm_mid(void* y, float* part, int ld_part, const MidShape& m, const 
 template <int OUT, int FT, int FN, int WT_, int WN_>
 int launch_gemm_lds(void* y, const f16* x, int ldx, const f16* Wp, int T, int K, int N, hipStream_t s) {
   constexpr size_t lds = 2 * (LBK / 32) * (FT + FN) * 512 * sizeof(f16);
-  static bool configured = false;                    // the attribute is per kernel, set once per process
-  if (!configured && lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_lds_kernel<OUT, FT, FN, WT_, WN_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return mlora_set_error(MLORA_ERR_LAUNCH, "gemm_packed: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-    configured = true;
-  }
+  static const hipError_t configured =               // the attribute is per kernel, set once per process, by one thread
+      lds > 64 * 1024 ? hipFuncSetAttribute((const void*)gemm_lds_kernel<OUT, FT, FN, WT_, WN_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
+                      : hipSuccess;
+  if (configured != hipSuccess)
+    return mlora_set_error(MLORA_ERR_LAUNCH, "gemm_packed: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(configured));
   hipLaunchKernelGGL((gemm_lds_kernel<OUT, FT, FN, WT_, WN_>), dim3(ceil_div(N, FN * 16), ceil_div(T, FT * 16)), dim3(256), lds, s,
                      y, x, ldx, Wp, T, K, N);
   return MLORA_OK;

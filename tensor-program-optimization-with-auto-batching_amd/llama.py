@@ -322,8 +322,11 @@ class LlamaForCausalLM:
         ks_ws = self._ksplit_ws(T) if dec_frag or (frag and T <= 256) else None
         # a prefill-sized pass of one adapter type of rank 32 or 64: where a 256-token block agrees on one adapter its
         # deltas ride in the base GEMM as extra k-steps; `rest` names the tokens that still need the separate call
+        # (a prefill pass only: the choice needs one read-back, which a decode step recorded into a graph cannot make)
         fuse = None
-        if tok_adapter and "multi" not in tok_adapter and frag and T > 64 and ops.gemm_frag_preferred(T, H, H):
+        is_decode = kv._cur is not None and bool(kv._cur[2])
+        if (tok_adapter and "multi" not in tok_adapter and frag and T > 64 and not is_decode
+                and not torch.cuda.is_current_stream_capturing() and ops.gemm_frag_preferred(T, H, H)):
             (tid, ids), = tok_adapter.items()
             lt = self.lora_types[tid]
             if lt.r in (32, 64):

@@ -165,3 +165,58 @@ def test_adapter_files_round_trip_and_wid_translation(tmp_path):
         af.load_lora_type(d, 16, 8.0, [7], shape, device="cpu")
     with pytest.raises(ValueError):
         af.load_lora_type(d, 16, 8.0, [1, 1], shape, device="cpu")
+
+
+class _StubTokenizer:
+    """The three things the front end asks of a tokenizer (`tvm/llama_auto_batcher/llama_exec_graph.py:52-56,143-147`,
+    `llama_auto_batcher.py:21`): call -> {'input_ids': ...}, decode, eos_token_id.  One token per character."""
+    eos_token_id = 3
+
+    def __call__(self, text, **kwargs):
+        ids = [ord(c) - 28 for c in text]
+        return {"input_ids": [ids] if kwargs.get("return_tensors") else ids}
+
+    def decode(self, ids):
+        return "".join(chr(int(i) + 28) for i in np.asarray(ids).reshape(-1))
+
+
+def test_text_prompt_path_with_a_stub_tokenizer():
+    """encode_prompt turns a text prompt into a [1, n] int32 id array through the tokenizer (id arrays pass through
+    unchanged), decode_answer turns generated ids back into text, the EOS id defaults to the tokenizer's; both node
+    kinds insist on exactly one input, one output and one sequence, as the reference's asserts do."""
+    eg, xg = load_pkg("llama_exec_graph"), load_pkg("exec_graph")
+    g = eg.LlamaExecGraph()
+    g.tokenizer = _StubTokenizer()
+    text = "hello auto-batching"
+    v_in, v_ids, v_out, v_txt = (xg.VarNode(i, None) for i in range(4))
+    v_in.var = text
+    enc = xg.OpNode("encode_prompt", [v_in], [v_ids], [0])
+    g.execute_op(enc)
+    assert v_ids.var.dtype == np.int32 and v_ids.var.shape == (1, len(text))
+    assert v_ids.var.reshape(-1).tolist() == [ord(c) - 28 for c in text]
+    v_in.var = np.array([5, 6, 7])                                    # token ids instead of text: no tokenizer call
+    g.execute_op(enc)
+    assert v_ids.var.tolist() == [[5, 6, 7]] and v_ids.var.dtype == np.int32
+    v_out.var = np.array([76, 77, 78], np.int32)
+    dec = xg.OpNode("decode_answer", [v_out], [v_txt], [0])
+    g.execute_op(dec)
+    assert v_txt.var == "hij"
+    g.tokenizer = None                                                # without a tokenizer the ids are the answer ...
+    g.execute_op(dec)
+    assert v_txt.var is v_out.var
+    v_in.var = "text"                                                 # ... and a text prompt is refused
+    with pytest.raises(AssertionError):
+        g.execute_op(enc)
+    with pytest.raises(AssertionError):
+        g.execute_op(xg.OpNode("encode_prompt", [v_in, v_in], [v_ids], [0]))
+    with pytest.raises(AssertionError):
+        g.execute_op(xg.OpNode("decode_answer", [v_out], [v_txt], [0, 1]))
+    # the EOS id is the tokenizer's unless one is given (set_exec_vars reads it before it builds the cache)
+    class _NoCacheGraph(eg.LlamaExecGraph):
+        def set_kv_cache(self, delete_prev=True):
+            pass
+    g2 = _NoCacheGraph()
+    g2.set_exec_vars(None, "cpu", None, _StubTokenizer(), None, None)
+    assert g2.eos_token_id == 3
+    g2.set_exec_vars(None, "cpu", None, _StubTokenizer(), None, None, eos_token_id=11)
+    assert g2.eos_token_id == 11

@@ -448,6 +448,45 @@ def test_prefill_linear_with_lora_as_extra_k_steps(ops, synth, r, acc):
     assert torch.equal(ops.linear_frag_lora(xf, Wp, projs, none, r), ops.linear(xf, Wp))
 
 
+@pytest.mark.parametrize("r", [32, 64])
+def test_extra_k_step_linear_block_with_unadapted_tokens(ops, synth, r):
+    """A caller-built block table in which adapter blocks also hold tokens that name no adapter (id -1, or an id past the
+    table): those tokens get the base product alone - their rows of the split shrink result are zero, whatever the
+    workspace held - and the adapted tokens of the same block get base + delta."""
+    T, K, N, n_ad = 4096, 256, 4096, 3
+    x = synth.normal(23, "flu.x", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(23, "flu.W", (N, K), 0.05, torch.float16, DEV)
+    A = synth.normal(23, "flu.A", (n_ad, r, K), 0.05, torch.float16, DEV)
+    B = synth.normal(23, "flu.B", (n_ad, N, r), 0.05, torch.float16, DEV)
+    ids = np.repeat(np.arange(16, dtype=np.int32) % n_ad, 256)
+    holes = synth.randint(23, "flu.holes", (T,), 4).numpy() == 0          # a quarter of the tokens without adapter
+    ids[holes] = -1
+    ids[5::97] = n_ad + 2                                                  # and a few with an id past the table
+    ids[256 * 3:256 * 4] = -1                                              # one block without any adapter
+    blk = np.arange(16, dtype=np.int32) % n_ad
+    blk[3] = -1
+    ids_d, blk_d = torch.from_numpy(ids).to(DEV), torch.from_numpy(blk).to(DEV)
+    ws = torch.full((ops.lib().mlora_gather_mm_workspace_bytes(T, K, r) // 4 + 4,), float("nan"), dtype=torch.float32, device=DEV)
+    xf = ops.FragActivation.pack(x)
+    (vh, vl), = ops.lora_shrink_split(xf, [A], ids_d, 0.5, ws)
+    torch.cuda.synchronize()
+    adapted = (ids >= 0) & (ids < n_ad)
+    assert not _np(vh)[~adapted].any() and not _np(vl)[~adapted].any()
+    assert np.isfinite(_np(vh)).all() and np.isfinite(_np(vl)).all() and np.abs(_np(vh)[adapted]).max() > 0.1
+    y = ops.linear_frag_lora(xf, ops.PackedWeight(W), [(B, vh, vl, 0, N)], blk_d, r)
+    torch.cuda.synchronize()
+    xd, Wd, Ad, Bd = (_np(t).astype(np.float64) for t in (x, W, A, B))
+    want = xd @ Wd.T
+    for a in range(n_ad):
+        rows = np.nonzero(ids == a)[0]
+        want[rows] += 0.5 * (xd[rows] @ Ad[a].T) @ Bd[a].T
+    y0 = _np(y).astype(np.float64)
+    assert np.isfinite(y0).all()
+    assert max_rel_err(y0, want, floor=1e-3) <= TOL
+    plain = _np(ops.linear(xf, ops.PackedWeight(W)))
+    assert np.array_equal(_np(y)[~adapted], plain[~adapted])              # a zero delta leaves the base product's bits
+
+
 @pytest.mark.parametrize("T,K,I,r,which", [(4096, 256, 4096, 0, ""), (1000, 128, 8224, 0, ""), (4096, 256, 4096, 64, "gu"),
                                             (3000, 128, 5664, 32, "gu"), (4096, 256, 4096, 32, "g"), (4096, 256, 4096, 64, "u")])
 def test_prefill_gate_up_with_silu_in_the_gemm_epilogue(ops, synth, T, K, I, r, which):
@@ -744,6 +783,9 @@ def test_gather_mm_one_launch_equals_shrink_then_expand(ops, synth, T, K, N, r, 
     (8, 20, 11008, 512, 32, 3, torch.float16, True),         # rank 32 and three 512-wide chunks per K-slice: generic shrink unit
     (10, 32, 1536, 264, 64, 40, torch.float32, True),        # rank 64, more adapters than tokens
     (8, 7, 1000, 136, 16, 2, torch.float16, True),           # K with a partial last chunk; many tokens per adapter
+    (24, 64, 4096, 1024, 16, 32, torch.float16, True),       # enough (set, adapter) pairs for the persistent shrink pass
+    (40, 40, 1100, 264, 8, 16, torch.float32, True),         # the persistent pass at rank 8 with a partial last K chunk
+    (600, 64, 512, 64, 16, 32, torch.float16, True),         # more than 64 pairs per workgroup: several pointer chunks
 ])
 def test_gather_mm_batch_equals_separate_calls(ops, synth, n_sets, T, K, N, r, n_ad, ydt, stream_passes):
     """Several problems with their own x, A, B, y and one token->adapter table in one call: same bits as one

@@ -384,3 +384,68 @@ def test_front_end_native_decode_equals_per_operator_decode(c1):
     a, _ = run_hip_generate(model, wl, prompts, none, 8, perm, native_decode=False)
     b, _ = run_hip_generate(model, wl, prompts, none, 8, perm, native_decode=True)
     assert a == b
+
+
+def test_prefill_pass_with_fused_and_separate_lora_blocks(monkeypatch):
+    """A prefill pass in which some 256-token blocks agree on one adapter (their deltas ride in the base GEMMs as extra
+    k-steps) and others straddle two sequences with different adapters or hold tokens without adapter (the separate
+    gather-matmul serves those tokens): the same pass with every delta through the separate call gives the same logits
+    up to where the sum is rounded, and the same greedy tokens wherever the margin decides."""
+    synth, llama, ops = load_pkg("synth"), load_pkg("llama"), load_pkg("ops")
+    shape = synth.LlamaShape(hidden_size=1024, intermediate_size=1024, num_attention_heads=8, num_key_value_heads=8,
+                             num_hidden_layers=1, head_dim=128, vocab_size=512)
+    spec = synth.LoraSpec(r=32, alpha=16.0, n_adapters=3,
+                          targets=("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"))
+    model = llama.LlamaForCausalLM.from_synthetic(31, shape, [spec], DEV)
+    lens = [448, 576] * 16                                   # 16384 tokens: sequence boundaries fall inside 256-token blocks
+    B, T = len(lens), sum(lens)
+    assert ops.gemm_frag_preferred(T, shape.hidden_size, shape.hidden_size)
+    seq_ad = (np.arange(B, dtype=np.int32) // 2) % 3         # pairs of sequences share an adapter ...
+    seq_ad[5] = -1                                           # ... one sequence has none
+    tok_ad = np.repeat(seq_ad, lens).astype(np.int32)
+    blk, rest = ops.lora_block_adapters(torch.from_numpy(tok_ad).to(DEV), spec.n_adapters)
+    assert bool((blk >= 0).any()) and bool((rest >= 0).any())          # both kinds of block are in the pass
+    tokens = synth.randint(31, "fuse.prompts", (T,), shape.vocab_size)
+    last = torch.from_numpy(np.cumsum(lens) - 1).to(DEV)
+
+    def run():
+        kv = model.create_paged_kv_cache(B, T + 16 * B, T, 16)
+        for s_ in range(B):
+            kv.add_sequence(s_)
+        kv.begin_forward(list(range(B)), lens)
+        logits = model.forward(model.embed(tokens), kv, {0: torch.from_numpy(tok_ad).to(DEV)}, logits_rows=last)
+        kv.end_forward()
+        torch.cuda.synchronize()
+        return logits.float().cpu().numpy(), kv
+
+    calls = {"fused": 0}
+    real_fused = ops.linear_frag_lora
+
+    def spy(*a, **k):
+        calls["fused"] += 1
+        return real_fused(*a, **k)
+
+    monkeypatch.setattr(ops, "linear_frag_lora", spy)
+    got, kv_f = run()
+    assert calls["fused"] >= 3                               # qkv, o and down at least took the fused entry
+    # the same pass with no block taking the extra k-steps: every delta through the separate gather-matmul
+    monkeypatch.setattr(ops, "lora_block_adapters",
+                        lambda ids, n_ad: (torch.full((-(-ids.numel() // 256),), -1, dtype=torch.int32, device=ids.device), ids.clone()))
+    want, kv_s = run()
+    std = want.std()
+    assert np.isfinite(got).all() and np.abs(got - want).max() / std <= 1e-2
+    assert np.sqrt(np.mean((got - want) ** 2)) / std <= 2e-3
+    top2 = np.sort(want, axis=-1)[:, -2:]
+    decided = (top2[:, 1] - top2[:, 0]) / std >= 2e-2
+    assert decided.sum() >= B // 2
+    assert np.array_equal(got.argmax(-1)[decided], want.argmax(-1)[decided])
+    # and the deltas matter: without adapters the logits differ visibly
+    kv0 = model.create_paged_kv_cache(B, T + 16 * B, T, 16)
+    for s_ in range(B):
+        kv0.add_sequence(s_)
+    kv0.begin_forward(list(range(B)), lens)
+    none = model.forward(model.embed(tokens), kv0, None, logits_rows=last).float().cpu().numpy()
+    kv0.end_forward()
+    adapted_rows = seq_ad >= 0
+    assert np.abs(none - want)[adapted_rows].max() / std > 5e-2
+    assert np.abs(none - want)[~adapted_rows].max() / std <= 1e-2

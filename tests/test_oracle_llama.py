@@ -285,3 +285,44 @@ def test_mixed_mode_rounds_fused_blocks_once():
     exact = outs[("fp32", None)]
     assert np.abs(b[:4] - exact[:4]).max() <= np.abs(a[:4] - exact[:4]).max() + 1e-7     # one rounding is no worse than two
     assert np.array_equal(b[:4], oracle.f16(exact[:4]))
+
+
+def test_lora_wiring_equals_merged_weights():
+    """Where the oracle places the LoRA delta (computed from the projection's own input - the normed residual, the
+    attention output, the SiLU product - and added to that projection's output, on all 7 linears): one adapter bound to
+    every token gives the logits of a model WITHOUT LoRA whose weights are W + scaling * B[a] . A[a]
+    (`huggingface/custom_peft/lora_gatherbmm_linear_layer.py:21-22`, the merged branch; `tvm/llama_auto_batcher/lora.py:16-24`).
+    A delta wired to the wrong input, the wrong projection or with a dropped scaling fails this; the model without
+    the adapter differs visibly."""
+    synth = load_pkg("synth")
+    shape = synth.LlamaShape(hidden_size=64, intermediate_size=128, num_attention_heads=4, num_key_value_heads=2,
+                             num_hidden_layers=2, head_dim=16, vocab_size=128)
+    w = {k: v.numpy() for k, v in synth.base_weights(7, shape, torch.float32, "cpu", std=0.2).items()}
+    targets = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")
+    spec = synth.LoraSpec(r=8, alpha=4.0, n_adapters=3, targets=targets)
+    lw = {k: v.numpy() * 5 for k, v in synth.lora_weights(7, shape, spec, torch.float32, "cpu").items()}
+    a = 1
+    ref = LlamaRef(shape, w, lw, {"a0": spec.scaling}, mode="fp32")
+    merged = dict(w)
+    for l in range(shape.num_hidden_layers):
+        for p in targets:
+            A, B = lw[f"layers.{l}.{p}.lora_A.a0"][a], lw[f"layers.{l}.{p}.lora_B.a0"][a]
+            merged[f"layers.{l}.{p}"] = (w[f"layers.{l}.{p}"].astype(np.float64) + spec.scaling * B.astype(np.float64) @ A.astype(np.float64)).astype(np.float32)
+    plain = LlamaRef(shape, merged, mode="fp32")
+    bare = LlamaRef(shape, w, mode="fp32")
+    ids = synth.randint(7, "p", (2, 11), shape.vocab_size).numpy()
+    outs = []
+    for r, tok in ((ref, {"a0": np.full(22, a, np.int32)}), (plain, None), (bare, None)):
+        kv = r.new_cache(4, 16, 32)
+        for s in range(2):
+            kv.add_sequence(s)
+        kv.begin_forward([0, 1], [11, 11])
+        l0 = r.forward(ids.reshape(-1), kv, tok)
+        kv.end_forward()
+        kv.begin_forward([0, 1], [1, 1])                    # and one cached decode step
+        l1 = r.forward(np.array([3, 5]), kv, None if tok is None else {"a0": np.full(2, a, np.int32)})
+        kv.end_forward()
+        outs.append(np.concatenate([l0, l1]))
+    with_lora, with_merged, without = outs
+    assert np.abs(with_lora - with_merged).max() <= 1e-4 * np.abs(with_merged).max()
+    assert np.abs(with_lora - without).max() >= 0.1 * with_merged.std()
