@@ -452,7 +452,7 @@ def bench_c1_generate(args, synth, llama):
         b = ab.LlamaAutoBatcherClass()
         b.set_model(model)
         b.set_exec_config(xg.LlamaExecConfig(max_prompt_len=wl.prompt_len, max_gen_len=G, page_size=wl.page_size,
-                                             dense_lora=args.dense_lora, batch_prefill=args.batch_prefill))
+                                             dense_lora=not args.ids_lora, batch_prefill=args.batch_prefill))
         b.set_free_pages(perm)
         b.set_eos_token_id(None)
         outs = []
@@ -480,7 +480,7 @@ def bench_c1_generate(args, synth, llama):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": wl.name, "layers": s.num_hidden_layers, "hidden": s.hidden_size, "batch": B,
                    "prompt_len": wl.prompt_len, "gen_len": G, "host_loop": "auto-batching front end, native decode step",
-                   "dense_lora": args.dense_lora, "batch_prefill": args.batch_prefill},
+                   "dense_lora": not args.ids_lora, "batch_prefill": args.batch_prefill},
         "roofline": {"kernel": "whole generate pass (4 prefills + 31 decode steps; launch- and host-bound at this size)", "bound": "hbm",
                      "achieved": model.weight_bytes_per_step() * (B + G - 1) / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": model.weight_bytes_per_step() * (B + G - 1) / dt / 1e9 / HBM_PEAK_GBS, "traffic": None}}
@@ -514,7 +514,8 @@ def main():
                     help="c3_decode: model shape (llama2_7b = the benchmark configuration; llama31_8b = the reference's default "
                          "model: grouped-query attention, 8 kv heads, vocabulary 128256)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--dense-lora", action="store_true", help="c1_generate: LlamaExecConfig.dense_lora")
+    ap.add_argument("--ids-lora", action="store_true",
+                    help="c1_generate: LlamaExecConfig.dense_lora = False (the ids-based shrink instead of the default dense one)")
     ap.add_argument("--batch-prefill", action="store_true", help="c1_generate: LlamaExecConfig.batch_prefill")
     ap.add_argument("--batch-order", action="store_true", help="c5_decode: keep the request order inside the batch (default: longest context first)")
     ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel event timing and the gather-matmul stream")
@@ -605,8 +606,8 @@ def main():
     tok_s = wl.batch * args.steps / dt
     dense = bool(getattr(sess, "dense_lora", False))
     # The timed session computes the LoRA shrink as extra rows of the base GEMV ("dense": taken while the adapters are
-    # few).  The front end's default is the ids-based shrink (bit-identical to the per-operator path): the same steps
-    # over the same pages once more with that form, for the record.
+    # few; the session's and the front end's default, LlamaExecConfig.dense_lora).  The ids-based shrink (bit-identical to
+    # the per-operator path, LlamaExecConfig.dense_lora = False) runs the same steps over the same pages once more, for the record.
     ids_ms = None
     if not args.python_loop and dense and not args.no_extras:
         for q in range(wl.batch):

@@ -120,16 +120,27 @@ __global__ __launch_bounds__(LORA_MAX_KC* WAVE, (RESIDENT ? 4 : 2)) void gmm_bat
 }
 
 // Pass 1 as a persistent launch: one workgroup per compute unit walks (set, adapter in use) pairs, and the whole of pair
-// i + 1 - the wave's slice of A[a], 16 rows, and the x rows of a's first two tokens - is requested before pair i is
+// i + 1 - the wave's slice of A[a], 16 rows, and the x rows of a's first four tokens - is requested before pair i is
 // reduced.  As one short-lived workgroup per pair, every pair paid its own memory round trips with an empty pipeline
 // (table row, set pointers, then A and x); here a workgroup pays them once per launch: the token->adapter table is
 // the same for all sets, so the adapters in use and their token masks are found once, the set pointers of a
 // workgroup's pairs are fetched 64 pairs at a time, one pair per lane, and handed out by lane reads, and adapters
-// without a token cost nothing.  The arithmetic of a pair is that of gmm_batch_shrink_kernel<true>: the same bits.
+// without a token cost nothing.  Every load of the pipeline is unconditional (addresses are clamped into the tables
+// and what a lane must not use is zeroed where it is used): only then can the waits be counted per register, and a
+// wait for pair i leaves the requests of pair i + 1 in flight.  The arithmetic of a pair is that of
+// gmm_batch_shrink_kernel<true>: the same bits.
+// (pointers that were put together from lane reads are plain integers to the compiler: they are declared as pointers
+// into global memory, or every load through them would be a flat load, whose completion cannot be counted per register)
+typedef const __attribute__((address_space(1))) f16* gf16p;
+__device__ __forceinline__ f16x8 gld8(gf16p p) { return *reinterpret_cast<const __attribute__((address_space(1))) f16x8*>(p); }
+__device__ __forceinline__ f16x8 gx_slice(gf16p x, int t, int k, int K, int frag_tt) {
+  return gld8(x + (frag_tt ? frag_offset(t, k, frag_tt) : (size_t)t * K + k));
+}
+
 struct ShrinkPair {
-  f16x8 a[16];           // the wave's K-slice of the adapter's 16 rows of A (rows past the rank are zero)
-  f16x8 x0, x1;          // the slice of the x rows of the adapter's first two tokens
-  const f16* x;          // x of the pair's set
+  f16x8 a[16];           // the wave's K-slice of the adapter's 16 rows of A (rows past the rank repeat the last row)
+  f16x8 x[4];            // the slice of the x rows of the adapter's first four tokens (fewer: the last one repeated)
+  gf16p xs;              // x of the pair's set
   unsigned long long mask;
   int set;
 };
@@ -159,9 +170,13 @@ __global__ __launch_bounds__(LORA_MAX_KC* WAVE, 1) void gmm_batch_shrink_pers_ke
   __syncthreads();
   const int total = n_sets * n_used;
   const int n_wg = gridDim.x, wg = blockIdx.x;
+  // pairs wg, wg + n_wg, ...: the adapters of one set are worked on by neighbouring workgroups at the same time (a
+  // contiguous range of pairs per workgroup measured 6 % slower)
   const int my_pairs = wg < total ? (total - wg + n_wg - 1) / n_wg : 0;
   const int kbase = wave * LORA_KCHUNK + lane * 8;
   const bool in = kbase < K;
+  const int kld = in ? kbase : 0;               // where this lane reads; what it reads past K is multiplied by zeros
+  const int rlast = r - 1;
   const size_t part_sz = (size_t)kc * T * r;
 
   for (int c0 = 0; c0 < my_pairs; c0 += WAVE) {
@@ -186,45 +201,30 @@ __global__ __launch_bounds__(LORA_MAX_KC* WAVE, 1) void gmm_batch_shrink_pers_ke
     auto fetch = [&](int i, ShrinkPair& P) {
       const int u = __builtin_amdgcn_readlane(pu, i);
       P.set = __builtin_amdgcn_readlane(pset, i);
-      P.x = (const f16*)lane_u64(px, i);
+      P.xs = (gf16p)lane_u64(px, i);
       P.mask = s_mask[u];
-      const f16* __restrict__ A = (const f16*)lane_u64(pA, i) + (size_t)s_used[u] * r * K;
+      const gf16p A = (gf16p)lane_u64(pA, i) + (size_t)s_used[u] * r * K;
       unsigned long long m = P.mask;
-      const int t0 = __builtin_ctzll(m);
-      m &= m - 1;
-      const int t1 = m ? __builtin_ctzll(m) : t0;
+      int t = __builtin_ctzll(m);
       // x ahead of A: loads come back in request order, so the products of row j can start as soon as row j is in
-      P.x0 = in ? x_slice(P.x, t0, kbase, K, a.frag_tt) : zero8;
-      P.x1 = in ? x_slice(P.x, t1, kbase, K, a.frag_tt) : zero8;
 #pragma unroll
-      for (int j = 0; j < G; ++j) P.a[j] = (j < r && in) ? ld8(A + (size_t)j * K + kbase) : zero8;
+      for (int q = 0; q < 4; ++q) {
+        P.x[q] = gx_slice(P.xs, t, kld, K, a.frag_tt);
+        m &= m - 1;
+        if (m) t = __builtin_ctzll(m);
+      }
+#pragma unroll
+      for (int j = 0; j < G; ++j) P.a[j] = gld8(A + (size_t)(j < r ? j : rlast) * K + kld);
     };
     auto reduce = [&](ShrinkPair& P, int buf) {
       float* __restrict__ pb = part_all + (size_t)buf * part_sz;
       float* __restrict__ vp = pb + (size_t)wave * T * r;
       unsigned long long m = P.mask;
-      int t0 = __builtin_ctzll(m);
-      m &= m - 1;
-      int t1 = -1;
-      if (m) {
-        t1 = __builtin_ctzll(m);
-        m &= m - 1;
-      }
-      f16x8 x0 = P.x0, x1 = P.x1;
-      while (true) {
-        int n0 = -1, n1 = -1;                    // the adapter's next token pair: requested now, used in the next round
-        f16x8 y0 = zero8, y1 = zero8;
-        if (m) {
-          n0 = __builtin_ctzll(m);
-          m &= m - 1;
-          if (m) {
-            n1 = __builtin_ctzll(m);
-            m &= m - 1;
-          }
-          if (in) {
-            y0 = x_slice(P.x, n0, kbase, K, a.frag_tt);
-            y1 = x_slice(P.x, n1 >= 0 ? n1 : n0, kbase, K, a.frag_tt);
-          }
+      // one token pair: the products of the 16 rows with both tokens, reduced over the lanes, into the wave's partials
+      auto token_pair = [&](f16x8 x0, f16x8 x1, int t0, int t1) {
+        if (!in) {
+          x0 = zero8;
+          x1 = zero8;
         }
         float p0[G], p1[G];
 #pragma unroll
@@ -236,8 +236,27 @@ __global__ __launch_bounds__(LORA_MAX_KC* WAVE, 1) void gmm_batch_shrink_pers_ke
         if (j0 < r && (lane & (WAVE / G - 1)) == 0) vp[(size_t)t0 * r + j0] = p0[0];
         const int j1 = reduce_transpose<G>(p1, lane);
         if (t1 >= 0 && j1 < r && (lane & (WAVE / G - 1)) == 0) vp[(size_t)t1 * r + j1] = p1[0];
-        if (n0 < 0) break;
-        t0 = n0; t1 = n1; x0 = y0; x1 = y1;
+      };
+      auto next_token = [&]() -> int {
+        if (!m) return -1;
+        const int t = __builtin_ctzll(m);
+        m &= m - 1;
+        return t;
+      };
+      int t0 = next_token(), t1 = next_token();
+      token_pair(P.x[0], P.x[1], t0, t1);
+      t0 = next_token();
+      if (t0 >= 0) {                             // a third and fourth token: their rows came with the pair
+        t1 = next_token();
+        token_pair(P.x[2], P.x[3], t0, t1);
+        t0 = next_token();
+        while (t0 >= 0) {                        // more than four tokens of one adapter: fetched now (this drains the pipeline)
+          t1 = next_token();
+          const f16x8 x0 = gx_slice(P.xs, t0, kld, K, a.frag_tt);
+          const f16x8 x1 = gx_slice(P.xs, t1 >= 0 ? t1 : t0, kld, K, a.frag_tt);
+          token_pair(x0, x1, t0, t1);
+          t0 = next_token();
+        }
       }
       __syncthreads();
       // the slices' partials, added in slice order and scaled; the other buffer is free for the next pair meanwhile
@@ -247,16 +266,24 @@ __global__ __launch_bounds__(LORA_MAX_KC* WAVE, 1) void gmm_batch_shrink_pers_ke
         if ((P.mask >> t) & 1) vout[e] = lora_v(pb, kc, T, r, t, j, a.scaling);
       }
     };
-    if (c0 > 0) __syncthreads();                 // the previous chunk's last pair may still be read from buffer 0
+    if (c0 > 0) __syncthreads();                 // the previous chunk's last pair may still be read from its buffer
+    // Two pairs in turn, each in registers of its own; no request sits behind a condition inside the loop, and the last
+    // one or two pairs of the chunk are worked off after it.
     ShrinkPair P0, P1;
     fetch(0, P0);
-    for (int i = 0; i < nchunk; i += 2) {
-      if (i + 1 < nchunk) fetch(i + 1, P1);
+    int i = 0;
+    for (; i + 2 < nchunk; i += 2) {
+      fetch(i + 1, P1);
       reduce(P0, 0);
-      if (i + 1 < nchunk) {
-        if (i + 2 < nchunk) fetch(i + 2, P0);
-        reduce(P1, 1);
-      }
+      fetch(i + 2, P0);
+      reduce(P1, 1);
+    }
+    if (i + 1 < nchunk) {
+      fetch(i + 1, P1);
+      reduce(P0, 0);
+      reduce(P1, 1);
+    } else {
+      reduce(P0, 0);
     }
   }
 }

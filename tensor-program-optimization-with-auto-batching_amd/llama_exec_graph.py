@@ -30,11 +30,14 @@ class LlamaExecConfig:
     # through the per-operator step recorded into a graph.  Same tokens: the native step with ids-based LoRA shrink
     # is bit-identical to the per-operator path.
     native_decode: bool = True
-    # Let the native step compute the LoRA shrink of all adapters as extra rows of the base GEMV (the fastest form
-    # while the adapters are few and low-rank: taken when every rank is at most 16).  It then also serves batches
-    # that mix adapter types of one scaling, and rows without adapter, from the types' zero-padded union.  The fp32
-    # summation order of x . A^T differs from the per-operator path, so a greedy token can differ at a near tie.
-    dense_lora: bool = False
+    # Let the native step compute the LoRA shrink of all adapters as extra rows of the base GEMV: the fastest form
+    # while the adapters are few and low-rank, taken where it applies (every rank at most 16, one scaling, at most 64
+    # sequences and no more adapters than twice the batch) and what the headline benchmark times.  It then also serves
+    # batches that mix adapter types of one scaling, and rows without adapter, from the types' zero-padded union.
+    # The fp32 summation order of x . A^T differs from the per-operator path, so a greedy token can differ from that
+    # path at a near tie (against the oracle the two forms are equally close); False keeps the ids-based shrink, whose
+    # tokens are bit-identical to the per-operator path.
+    dense_lora: bool = True
     # Prefill the prompts of all requests in one forward pass instead of one pass per request (the reference's way).
     # Same arithmetic per token, but larger token counts take other GEMM kernels and summation orders, so the first
     # token of a request can differ from the per-request prefill at a near tie.

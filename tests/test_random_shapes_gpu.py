@@ -76,7 +76,7 @@ def test_front_end_on_random_request_mixes():
         b = ab.LlamaAutoBatcherClass()
         b.set_model(model)
         b.set_exec_config(xg.LlamaExecConfig(max_prompt_len=max(len(p) for p in prompts), max_gen_len=max_gen, page_size=16,
-                                             native_decode=native))
+                                             native_decode=native, dense_lora=False))    # the bit-identical routing
         b.set_free_pages(perm)
         b.set_eos_token_id(eos)
         outs = []
