@@ -898,7 +898,10 @@ __global__ __launch_bounds__(PF_WAVES* WAVE, 2) void paged_attn_prefill_block_ke
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       }
       static_assert(PF_RING <= 4 && (2 * HC == 2 || 2 * HC == 4 || 2 * HC == 8), "the immediates above are 2 HC loads per block in flight");
-      __syncthreads();                                               // everybody's has; nobody reads block b - 1 any more
+      // everybody's has; nobody reads block b - 1 any more.  The bare barrier: __syncthreads() would first wait for the
+      // loads of the younger blocks as well (see bare_barrier)
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      bare_barrier();
       if (b + PF_RING - 1 < nblk) issue(b + PF_RING - 1);           // into the slot of block b - 1
       if (wmax < b * PF_PAGES * PAGE) continue;                      // wave-uniform: the block lies above this wave's diagonal
       const f16* kb_ = smem + (b % PF_RING) * BUF;

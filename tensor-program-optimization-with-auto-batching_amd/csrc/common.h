@@ -77,3 +77,14 @@ __device__ __forceinline__ float dot8(f16x8 a, f16x8 b, float c) {
   c = dot2(f16x2{a[6], a[7]}, f16x2{b[6], b[7]}, c);
   return c;
 }
+
+// A workgroup barrier and nothing else.  __syncthreads() is a fence and then the barrier, and for the fence the compiler
+// waits for EVERY memory request of the wave (s_waitcnt vmcnt(0)) - also for the direct-to-LDS loads of later stages,
+// which a software pipeline means to keep in flight across the barrier: with __syncthreads() a ring of several stages
+// runs as if it had one.  The caller first waits for exactly what the barrier must publish (its own s_waitcnt: the
+// loads of the stage that is read next, and its LDS accesses).
+__device__ __forceinline__ void bare_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}

@@ -673,10 +673,13 @@ int launch_gemm_pp(void* y, const f16* x, int ldx, int x_tt, const f16* Wp, int 
 // workgroup: FT x FN fragments (128 or 256 tokens x 128 or 64 weight rows), eight waves, both operands in fragment
 // order and copied from global memory straight into an LDS ring.  A stage of the ring is TWO 32-k steps: with the
 // few MFMAs a wave has per 32-k step here (4 to 16), a barrier and a wait per step cost more than the step itself.
-// Four (three) stages, of which three (two) are in flight per compute unit.
-// (Measured on this kernel: a deeper ring for the weights alone, with waves that fetch only weights, changes
-// nothing - a workgroup's weight stream runs at 12 to 19 GB/s whatever it keeps in flight, and the launch as a whole
-// at 2 to 3.4 TB/s; with the weights coming from L2 instead the same loop is 1.5 times faster.)
+// Four (three) stages, of which three (two) are in flight per compute unit - across the barrier of a stage, which is
+// the bare instruction (bare_barrier): behind __syncthreads() the compiler first waits for every request in flight,
+// the ring ran as if it had one stage and the launch pulled 2 to 3.4 TB/s of weights whatever its depth.
+// What bounds the kernel now is what the second-level caches hand to the compute units: at 256 tokens the counters
+// show 417 MB of requests per 100 MB matrix (each weight fragment for two token blocks, the token block once per
+// row block), 70 % of them hits, delivered at 8 to 10 TB/s over the chip - every tiling that gives all compute units
+// a workgroup has to take in about that much.
 // grid = (weight-row blocks, K slices, token blocks).
 // With K slices, slice 0 produces the result proper (store or accumulate) and slice s > 0 stores its fp32 partial
 // sums to part[s - 1][T][ld_part] - for the two narrow accumulating linears of a layer, whose partials the next
@@ -786,7 +789,7 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
   auto stage = [&](auto U) {
     constexpr int u = decltype(U)::value;
     wait_next();
-    __syncthreads();
+    bare_barrier();
     issue();
     read_frags(std::integral_constant<int, 1 - u>());
     __builtin_amdgcn_sched_barrier(0);
@@ -796,7 +799,7 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
 #pragma unroll
   for (int i = 0; i < MID_STAGES - 1; ++i) issue();
   wait_next();
-  __syncthreads();
+  bare_barrier();
   issue();
   read_frags(std::integral_constant<int, 0>());
   int g = 0;
