@@ -109,7 +109,7 @@ def gemv_event_timing(model, T, reps=3, per_kind=True):
     x_i = ops.FragActivation(T, s.intermediate_size, dev)
     act = ops.FragActivation(T, s.intermediate_size, dev)
     for x in (x_h, x_q, x_i):
-        x.data.zero_()
+        x.data.normal_()                  # (the matrix cores' clock depends on the operand bits: no constant activations)
     n_ext = lt.n_adapters * lt.r
     resid = torch.zeros((T, s.hidden_size), dtype=torch.float32, device=dev)
     qkv = torch.empty((T, s.q_size + 2 * s.kv_size), dtype=torch.float16, device=dev)
@@ -152,8 +152,9 @@ def gemv_event_timing(model, T, reps=3, per_kind=True):
     add("lm_head", lambda: lib.mlora_gemv_frag(logits.data_ptr(), F32, STORE, x_h.data.data_ptr(), model.lm_head.data.data_ptr(), T, H,
                                     s.vocab_size, st), s.vocab_size, H, T * s.vocab_size * 4)
     def timed(fns):
-        best = None
-        for _ in range(reps + 1):          # first pass is a warm-up
+        """Median over the timed passes (the first pass is a warm-up and is left out)."""
+        times = []
+        for i in range(reps + 1):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             for fn in fns:
@@ -162,9 +163,9 @@ def gemv_event_timing(model, T, reps=3, per_kind=True):
                     raise RuntimeError(lib.mlora_last_error().decode())
             e1.record()
             torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1)
-            best = ms if best is None else min(best, ms)
-        return best
+            if i > 0 or reps == 0:
+                times.append(e0.elapsed_time(e1))
+        return float(np.median(times))
 
     best = timed(launches)
     # the same launches one kind at a time (each kind's launches back to back on their distinct matrices)
@@ -547,6 +548,7 @@ def main():
     if args.workload == "c1_generate":
         return bench_c1_generate(args, synth, llama)
     if args.probe:
+        ops = _mod("ops")
         wl = synth.config3(num_layers=2)
         model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, [wl.lora], dev)
         src = torch.zeros(256 << 20, dtype=torch.uint8, device=dev)
@@ -555,6 +557,13 @@ def main():
         dst.copy_(src)                       # plain copy kernel: reads 256 MiB, writes 256 MiB
         g = gemv_event_timing(model, wl.batch, reps=1, per_kind=False)    # exactly two passes over the mix: warm-up, timed
         gm = gather_mm_timing(n_sets=8)
+        # the mid-size linear (gemm_mid_kernel) on a 256-token block: q/k/v and the accumulating o projection with its K slices
+        x256 = ops.FragActivation.pack(torch.randn(256, wl.shape.hidden_size, device=dev, dtype=torch.float16))
+        r256 = torch.zeros((256, wl.shape.hidden_size), dtype=torch.float32, device=dev)
+        for _ in range(2):
+            ops.linear(x256, model.layers[0]["qkv"])
+            ops.linear(x256, model.layers[1]["gate_up"])
+            ops.linear(x256, model.layers[0]["o"], out=r256, accumulate=True)
         # two native decode steps of the 2-layer model at the benchmark's cache geometry (32 sequences at context 520
         # in shuffled pages, cache pre-filled with N(0,1)): the fused RoPE + attention launch at its real shape
         blocks = -(-(wl.prompt_len + 16) // wl.page_size)

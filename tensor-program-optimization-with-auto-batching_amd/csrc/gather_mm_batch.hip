@@ -258,7 +258,9 @@ __global__ __launch_bounds__(LORA_MAX_KC* WAVE, 1) void gmm_batch_shrink_pers_ke
           t0 = next_token();
         }
       }
-      __syncthreads();
+      // the partials are in LDS; the bare barrier: __syncthreads() would first wait for the next pair's requests as well
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      bare_barrier();
       // the slices' partials, added in slice order and scaled; the other buffer is free for the next pair meanwhile
       float* __restrict__ vout = a.ws + (size_t)P.set * a.ws_stride;
       for (int e = threadIdx.x; e < T * r; e += blockDim.x) {
@@ -266,7 +268,10 @@ __global__ __launch_bounds__(LORA_MAX_KC* WAVE, 1) void gmm_batch_shrink_pers_ke
         if ((P.mask >> t) & 1) vout[e] = lora_v(pb, kc, T, r, t, j, a.scaling);
       }
     };
-    if (c0 > 0) __syncthreads();                 // the previous chunk's last pair may still be read from its buffer
+    if (c0 > 0) {                                // the previous chunk's last pair may still be read from its buffer
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      bare_barrier();
+    }
     // Two pairs in turn, each in registers of its own; no request sits behind a condition inside the loop, and the last
     // one or two pairs of the chunk are worked off after it.
     ShrinkPair P0, P1;
