@@ -60,12 +60,13 @@ def profiled_gemv_traffic():
     return int(m.group(1)) if m else None
 
 
-def traffic_from_counters(fetch_csv, write_csv, layers_step=32):
+def traffic_from_counters(fetch_csv, write_csv, layers_step=32, layers_probe=2):
     """HBM bytes per GEMV launch, weighted over the launch mix of one decode step, from the two counter runs of
     `bench.py --probe` (rocprofv3 --pmc FETCH_SIZE, then --pmc WRITE_SIZE, --output-format csv): each counter is scaled
     by what it reads for the probe's plain 256 MiB device copy; the probe's GEMV launches come in the order qkv, o,
-    gate_up, down per layer and lm_head last, and a decode step issues each layer kind `layers_step` times and lm_head
-    once.  Needs no GPU."""
+    gate_up, down per layer and lm_head last (a warm-up pass, then the timed one, over the probe's `layers_probe`
+    layers; the GEMV launches of the decode steps at the end of the probe come after them and are not used), and a
+    decode step issues each layer kind `layers_step` times and lm_head once.  Needs no GPU."""
     import csv
     per_kind = {}
     scale = {}
@@ -74,9 +75,10 @@ def traffic_from_counters(fetch_csv, write_csv, layers_step=32):
         copy = max(float(r["Counter_Value"]) for r in rows if "copyBuffer" in r["Kernel_Name"])
         scale[name] = 262144.0 / copy
         gemv = [r for r in rows if "gemv" in r["Kernel_Name"] and "pack" not in r["Kernel_Name"]]
-        n_layers = (len(gemv) // 2 - 1) // 4            # the probe issues the mix twice (a warm-up pass, then the timed one)
-        block = gemv[len(gemv) // 2:]
-        assert len(block) == 4 * n_layers + 1, (len(gemv), n_layers)
+        n_layers = layers_probe
+        per_pass = 4 * n_layers + 1
+        assert len(gemv) >= 2 * per_pass, (len(gemv), n_layers)
+        block = gemv[per_pass:2 * per_pass]             # the second of the two passes over the mix
         kinds = ["qkv", "o", "gate_up", "down"] * n_layers + ["lm_head"]
         for k, r in zip(kinds, block):
             per_kind.setdefault(k, {}).setdefault(name, []).append(float(r["Counter_Value"]))
@@ -180,9 +182,11 @@ def gemv_event_timing(model, T, reps=3, per_kind=True):
             "gbs": total_bytes / (best * 1e-3) / 1e9, "per_kernel": per_kernel, "kinds": kinds}
 
 
-def gather_mm_timing(n_sets=128):
+def gather_mm_timing(n_sets=128, torch_init=False):
     """Isolated gather-matmul at the decode shape (T=64, K=N=4096, r=16, 32 adapters): n_sets distinct
-    operand sets (> 1 GiB, larger than the 256 MB last-level cache) issued back to back."""
+    operand sets (> 1 GiB, larger than the 256 MB last-level cache) issued back to back.  torch_init fills the
+    operands with torch's own generator (two launches per tensor instead of the counter-based generator's two
+    dozen: for runs under a counter profiler, which records every launch)."""
     import torch
     ops, synth = _mod("ops"), _mod("synth")
     dev = "cuda:0"
@@ -191,6 +195,12 @@ def gather_mm_timing(n_sets=128):
     U = len(np.unique(ids.cpu().numpy()))
     sets = []
     for j in range(n_sets):
+        if torch_init:
+            sets.append((torch.randn((T, K), dtype=torch.float16, device=dev),
+                         torch.randn((n_ad, r, K), dtype=torch.float16, device=dev) * 0.02,
+                         torch.randn((n_ad, N, r), dtype=torch.float16, device=dev) * 0.02,
+                         torch.randn((T, N), dtype=torch.float16, device=dev)))
+            continue
         sets.append((synth.normal(1, f"b.x{j}", (T, K), 1.0, torch.float16, dev),
                      synth.normal(1, f"b.A{j}", (n_ad, r, K), 0.02, torch.float16, dev),
                      synth.normal(1, f"b.B{j}", (n_ad, N, r), 0.02, torch.float16, dev),
@@ -549,15 +559,24 @@ def main():
         return bench_c1_generate(args, synth, llama)
     if args.probe:
         ops = _mod("ops")
+
+        def stage(name):                     # progress on stderr: names the stage a profiler run stopped in
+            print(f"[probe] {name}", file=sys.stderr, flush=True)
+
+        stage("model")
         wl = synth.config3(num_layers=2)
         model = llama.LlamaForCausalLM.from_synthetic(wl.seed, wl.shape, [wl.lora], dev)
         src = torch.zeros(256 << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
         torch.cuda.synchronize()
+        stage("copy")
         dst.copy_(src)                       # plain copy kernel: reads 256 MiB, writes 256 MiB
+        stage("gemv")
         g = gemv_event_timing(model, wl.batch, reps=1, per_kind=False)    # exactly two passes over the mix: warm-up, timed
-        gm = gather_mm_timing(n_sets=8)
+        stage("gather_mm")
+        gm = gather_mm_timing(n_sets=24, torch_init=True)     # enough (set, adapter) pairs for the persistent shrink pass
         # the mid-size linear (gemm_mid_kernel) on a 256-token block: q/k/v and the accumulating o projection with its K slices
+        stage("mid-size linears")
         x256 = ops.FragActivation.pack(torch.randn(256, wl.shape.hidden_size, device=dev, dtype=torch.float16))
         r256 = torch.zeros((256, wl.shape.hidden_size), dtype=torch.float32, device=dev)
         for _ in range(2):
@@ -566,6 +585,7 @@ def main():
             ops.linear(x256, model.layers[0]["o"], out=r256, accumulate=True)
         # two native decode steps of the 2-layer model at the benchmark's cache geometry (32 sequences at context 520
         # in shuffled pages, cache pre-filled with N(0,1)): the fused RoPE + attention launch at its real shape
+        stage("decode steps")
         blocks = -(-(wl.prompt_len + 16) // wl.page_size)
         kv = model.create_paged_kv_cache(wl.batch, wl.batch * blocks * wl.page_size, wl.prompt_len, wl.page_size,
                                          free_pages=synth.permutation(wl.seed, "c3.pages", wl.batch * blocks),
