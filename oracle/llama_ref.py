@@ -224,10 +224,14 @@ class LlamaRef:
         resid = resid + x @ self.w[f"layers.{l}.{proj}"].T
         return self._delta_into(resid, x, l, proj, tok_adapter)
 
-    def forward(self, tokens, kv, tok_adapter=None, logits_rows=None):
-        """tokens [T] (sequence-major, as announced to kv.begin_forward) -> logits [T or len(rows), V] float32."""
+    def forward(self, tokens, kv, tok_adapter=None, logits_rows=None, tap_depths=()):
+        """tokens [T] (sequence-major, as announced to kv.begin_forward) -> logits [T or len(rows), V] float32.
+        tap_depths: layer counts d at which the logits of the model cut off after d layers (final norm and head on
+        the residual stream as it stands there) are kept in self.taps[d] - what a pass of a d-layer model over the
+        same weights returns, without a second pass."""
         s = self.shape
         eps = s.rms_norm_eps
+        self.taps = {}
         resid = np.asarray(self.w["embed_tokens"], dtype=np.float32)[np.asarray(tokens)]
         T = resid.shape[0]
         for l in range(s.num_hidden_layers):
@@ -243,9 +247,14 @@ class LlamaRef:
             u = self._proj(xn, l, "up_proj", tok_adapter)
             act = self.rnd(silu_mul_ref(g, u))
             resid = self._proj_residual(resid, act, l, "down_proj", tok_adapter)
+            if l + 1 in tap_depths and l + 1 < s.num_hidden_layers:
+                self.taps[l + 1] = self._head(resid, logits_rows)
+        return self._head(resid, logits_rows)
+
+    def _head(self, resid, logits_rows):
         if logits_rows is not None:
             resid = resid[np.asarray(logits_rows)]
-        xn = self.rnd(rmsnorm_ref(resid, self.w["norm"], eps))
+        xn = self.rnd(rmsnorm_ref(resid, self.w["norm"], self.shape.rms_norm_eps))
         return (xn @ self.w["lm_head"].T).astype(np.float32)
 
 

@@ -326,3 +326,34 @@ def test_lora_wiring_equals_merged_weights():
     with_lora, with_merged, without = outs
     assert np.abs(with_lora - with_merged).max() <= 1e-4 * np.abs(with_merged).max()
     assert np.abs(with_lora - without).max() >= 0.1 * with_merged.std()
+
+
+def test_depth_taps_equal_shallower_models():
+    """`forward(..., tap_depths=)` keeps the logits of the model cut off after d layers: bit for bit what a d-layer model
+    over the same weights returns for the same tokens (the GPU tests read the error at several depths off one pass)."""
+    import dataclasses
+    synth = load_pkg("synth")
+    shape = synth.LlamaShape(hidden_size=64, intermediate_size=128, num_attention_heads=4, num_key_value_heads=2,
+                             num_hidden_layers=5, head_dim=16, vocab_size=96)
+    w = {k: v.numpy() for k, v in synth.base_weights(3, shape, torch.float32, "cpu", std=0.2).items()}
+    spec = synth.LoraSpec(r=4, alpha=8.0, n_adapters=2, targets=("q_proj", "v_proj", "down_proj"))
+    lw = {k: v.numpy() * 3 for k, v in synth.lora_weights(3, shape, spec, torch.float32, "cpu").items()}
+    ids = synth.randint(3, "p", (13,), shape.vocab_size).numpy()
+    tok = {"a0": np.array([0] * 6 + [1] * 4 + [-1] * 3, np.int32)}
+    for mode in ("fp32", "mixed"):
+        full = LlamaRef(shape, w, lw, {"a0": spec.scaling}, mode=mode)
+        kv = full.new_cache(2, 16, 16)
+        kv.add_sequence(0)
+        kv.begin_forward([0], [13])
+        top = full.forward(ids, kv, tok, logits_rows=[3, 12], tap_depths=(1, 3, 5))
+        kv.end_forward()
+        assert sorted(full.taps) == [1, 3]                  # the full depth is the return value itself
+        for d in (1, 3, 5):
+            cut = LlamaRef(dataclasses.replace(shape, num_hidden_layers=d), w, lw, {"a0": spec.scaling}, mode=mode)
+            kvd = cut.new_cache(2, 16, 16)
+            kvd.add_sequence(0)
+            kvd.begin_forward([0], [13])
+            exp = cut.forward(ids, kvd, tok, logits_rows=[3, 12])
+            kvd.end_forward()
+            assert np.array_equal(exp, top if d == 5 else full.taps[d]), (mode, d)
+        assert np.abs(full.taps[1] - top).max() > 1e-3      # the depths do differ
