@@ -95,16 +95,19 @@ def traffic_from_counters(fetch_csv, write_csv, layers_step=32, layers_probe=2):
 
 def gemv_event_timing(model, T, reps=3, per_kind=True):
     """Average duration of the weight-streaming GEMV over exactly the launches of one decode step (per layer: qkv with
-    the adapters' A rows appended, o with A rows appended accumulating into the residual, gate/up with the SiLU
-    epilogue, down accumulating - o and down with their K split; then lm_head: 129 launches on 129 distinct matrices),
-    issued back to back as in a decode step and bracketed by one event pair on the launch stream."""
+    the adapters' A rows appended, o accumulating into the residual with the riders that expand its adapter delta (or,
+    where the library does not serve the shape that way, with A rows appended), gate/up with the SiLU epilogue, down
+    accumulating - o and down with their K split; then lm_head: 129 launches on 129 distinct matrices), issued back to
+    back as in a decode step and bracketed by one event pair on the launch stream."""
     import torch
     ops, lm = _mod("ops"), _mod("_lib")
     lib = lm.lib()
     s = model.shape
     dev = model.device
     lt = model.lora_types[0]
-    ext = model.dense_lora_weights(0)
+    ks_ride = lib.mlora_gemv_delta_ride_ksplit(T, s.q_size, s.hidden_size, lt.r)
+    ride = ks_ride > 0 and bool(lib.mlora_rope_attn_oshrink_ok(T, s.num_attention_heads, s.num_key_value_heads, s.head_dim, lt.r))
+    ext = model.dense_lora_weights(0, with_o=not ride)
     il = model.interleaved_gate_up()
     x_h = ops.FragActivation(T, s.hidden_size, dev)
     x_q = ops.FragActivation(T, s.q_size, dev)
@@ -125,6 +128,10 @@ def gemv_event_timing(model, T, reps=3, per_kind=True):
     # o and down split K over several workgroups as in the decode step; the partial results go to `part`
     ks_o, ks_d = lib.mlora_gemv_ksplit(T, Q, H + n_ext), lib.mlora_gemv_ksplit(T, I, H)
     part = torch.empty(3 * T * (H + n_ext), dtype=torch.float32, device=dev)
+    # the riders' inputs: the o shrink as one share per attention head, every token on an adapter (T tokens over n_ad adapters)
+    ids = (torch.arange(T, device=dev) % lt.n_adapters).to(torch.int32)
+    vpart = torch.randn((s.num_attention_heads, T, lt.r), dtype=torch.float32, device=dev)
+    used = min(T, lt.n_adapters)
 
     kinds, nbytes = [], []
 
@@ -142,10 +149,19 @@ def gemv_event_timing(model, T, reps=3, per_kind=True):
         add("qkv", lambda wq=wq, q_ext=q_ext: lib.mlora_gemv_frag_split_kq(qkv.data_ptr(), y2.data_ptr(), kq, x_h.data.data_ptr(),
                                                                     wq.data.data_ptr(), T, H, QKV, q_ext, st),
             wq.N, H, T * QKV * 2 + kq * T * q_ext * 4)
-        add("o", lambda wo=wo, o_ext=o_ext: lib.mlora_gemv_frag_acc_ksplit(resid.data_ptr(), y2.data_ptr(), part.data_ptr(), ks_o,
-                                                                      x_q.data.data_ptr(), wo.data.data_ptr(), T, Q, H, o_ext,
-                                                                      None, None, 0, None, 0, 0, st),
-            wo.N, Q, T * H * 8 + T * o_ext * 4)
+        tab_o = lt.tables.get((l, "o_proj"))
+        if ride and tab_o is not None:
+            # base weight + riders: the weight, the token block, the residual read and written, the B rows of the adapters
+            # in use and the head shares of the shrink (the slice partials and the delta rows are not counted, as before)
+            add("o", lambda wo=wo, Bo=tab_o[1]: lib.mlora_gemv_frag_acc_ksplit_delta(resid.data_ptr(), part.data_ptr(), ks_ride, x_q.data.data_ptr(),
+                                                                                 wo.data.data_ptr(), T, Q, H, vpart.data_ptr(), vpart.shape[0],
+                                                                                 Bo.data_ptr(), ids.data_ptr(), lt.scaling, lt.r, lt.n_adapters, st),
+                wo.N, Q, T * H * 8 + used * H * lt.r * 2 + vpart.numel() * 4)
+        else:
+            add("o", lambda wo=wo, o_ext=o_ext: lib.mlora_gemv_frag_acc_ksplit(resid.data_ptr(), y2.data_ptr(), part.data_ptr(), ks_o,
+                                                                          x_q.data.data_ptr(), wo.data.data_ptr(), T, Q, H, o_ext,
+                                                                          None, None, 0, None, 0, 0, st),
+                wo.N, Q, T * H * 8 + T * o_ext * 4)
         add("gate_up", lambda wg=wg: lib.mlora_gemv_frag_silu(act.data.data_ptr(), x_h.data.data_ptr(), wg.data.data_ptr(), T, H, I, st),
             2 * I, H, T * I * 2)
         add("down", lambda wd=wd: lib.mlora_gemv_frag_acc_ksplit(resid.data_ptr(), None, part.data_ptr(), ks_d, x_i.data.data_ptr(),
@@ -677,7 +693,7 @@ def main():
         out["ids_shrink_variant"] = {"ms_per_step": ids_ms, "tok_s": wl.batch / (ids_ms * 1e-3), "dense_lora": False}
     if not args.no_extras:
         g = gemv_event_timing(model, wl.batch)
-        out["roofline"] = {"kernel": "gemv_kernel / gemv_split_cu_kernel / gemv_silu_cu_kernel (fragment-ordered weights and activations, T=32; the 129 GEMV launches of one decode step: adapter A rows appended to qkv / o, K split on o / down, SiLU epilogue on gate/up)", "bound": "hbm", "achieved": g["gbs"],
+        out["roofline"] = {"kernel": "gemv_kernel / gemv_split_cu_kernel / gemv_silu_cu_kernel (fragment-ordered weights and activations, T=32; the 129 GEMV launches of one decode step: adapter A rows appended to qkv, expand riders in o, K split on o / down, SiLU epilogue on gate/up)", "bound": "hbm", "achieved": g["gbs"],
                            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g["gbs"] / HBM_PEAK_GBS, "traffic": profiled_gemv_traffic(),
                            "launches_timed": g["launches"], "avg_launch_us": g["avg_us"],
                            "algorithmic_bytes_per_launch": g["bytes_per_launch"], "per_kernel": g["per_kernel"]}

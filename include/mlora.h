@@ -400,6 +400,22 @@ int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv, void* k_c
                            int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
                            const void* v_part, int v_dense, const void* const* Bmat, const int32_t* tok_adapter,
                            float scaling, int K, int r, int n_ad, void* stream);
+/* The same launch, which in addition takes the o projection's LoRA shrink off the attention output where it is
+ * produced: o_vpart[h][b][j] = sum over the D dims of head h of f16(out[b, h, d]) * o_A[id_b][j][h D + d]  (fp32,
+ * [Hq][B][r]; o_A [n_ad, r, Hq * D]; rows of tokens without adapter are left untouched), one share per query head,
+ * for a consumer that adds the Hq shares in head order (mlora_gemv_frag_acc_ksplit_delta).  out and the caches are
+ * those of mlora_rope_attn_decode bit for bit.  tok_adapter, r and n_ad serve both the q/k/v expand (if v_part is
+ * given) and the o shrink.  mlora_rope_attn_oshrink_ok says whether the launch for (B, Hq, Hkv, D) has room for
+ * rank r (its Hq / Hkv * r * D / 8 items must fit one workgroup).  Replaces: the lora_A half of the o projection's
+ * injected forward (tvm/llama_auto_batcher/lora.py:16-24, compile_tvm.py:126-134). */
+int mlora_rope_attn_oshrink_ok(int B, int Hq, int Hkv, int D, int r);
+int mlora_rope_attn_decode_oshrink(void* out, int out_layout, const void* qkv, void* k_cache, void* v_cache,
+                                   const int32_t* block_table, int max_blocks,
+                                   const int32_t* seq_ids, const int32_t* tok_pos, const int32_t* ctx_len,
+                                   const float* rope_cos, const float* rope_sin, int max_pos,
+                                   int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                                   const void* v_part, int v_dense, const void* const* Bmat, const int32_t* tok_adapter,
+                                   float scaling, int K, int r, int n_ad, const void* o_A, void* o_vpart, void* stream);
 int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v_part, int v_dense, const void* B,
                               const int32_t* tok_adapter, float scaling, const void* w, float eps,
                               int T, int H, int K, int r, int n_ad, void* stream);
@@ -425,10 +441,25 @@ int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v
  *                                += part[0][t, :H] + ... + part[ks-2][t, :H], stored back, then y = RMSNorm(resid).
  *                                ld_part = N_total of the GEMV that wrote `part`; with v_dense = 1 the shrink results
  *                                are y2 plus columns H.. of the partials.
+ *   mlora_gemv_frag_acc_ksplit_delta - the same accumulating K-split GEMV over the base weight alone, with the
+ *                                projection's LoRA expand done by workgroups that ride at the front of the launch.  The
+ *                                shrink results come as n_vpart shares, vpart [n_vpart][T][r] fp32 (added in share
+ *                                order; mlora_rope_attn_decode_oshrink writes one share per attention head):
+ *                                delta[t, :] = scaling * B[id_t] . sum_h vpart[h][t] (zeros for a token without adapter)
+ *                                goes to slot ks-1 of `part` ([ks][T][N] fp32: ks-1 slice partials, then the delta
+ *                                rows), so a reader that adds ks slots (mlora_rmsnorm_ksplit with ks + 1, no B) obtains
+ *                                y + x . W^T + delta.  ks must be mlora_gemv_delta_ride_ksplit(T, K, N, r) (0: the shape
+ *                                is not served; T <= 64, rank 8, 16, 32 or 64; at most 3, so that the reader adds at
+ *                                most 3 slots).
  * These replace the same reference operators as mlora_gemv_frag (llama_for_causal_lm.py:31-33,44-47, the o_proj and
- * down_proj linears with the residual add of :79-84) and mlora_rmsnorm (:76-77).
+ * down_proj linears with the residual add of :79-84), mlora_rmsnorm (:76-77) and, for the delta form, the LoRA branch
+ * of the injected linear forward (tvm/llama_auto_batcher/lora.py:16-24).
  * ------------------------------------------------------------------------------------------- */
 int mlora_gemv_ksplit(int T, int K, int N_total);
+int mlora_gemv_delta_ride_ksplit(int T, int K, int N, int r);
+int mlora_gemv_frag_acc_ksplit_delta(float* y, float* part, int ks, const void* xf, const void* Wp, int T, int K, int N,
+                                     const float* vpart, int n_vpart, const void* B, const int32_t* tok_adapter, float scaling,
+                                     int r, int n_ad, void* stream);
 int mlora_gemv_shrink_rows(int K, int n_proj, int n_ad);
 size_t mlora_gemv_ksplit_bytes(int T, int N_total, int ks);
 int mlora_gemv_frag_acc_ksplit(float* y, float* y2, float* part, int ks, const void* xf, const void* Wp,
@@ -454,6 +485,11 @@ int mlora_rmsnorm_ksplit(void* y, int y_layout, float* resid, const float* part,
  * lora_dense != 0: qkv_p, o_p and down_p have the stacked A tables of their adapted projections appended as extra
  * rows (q, k, v slots in that order, n_ad * r rows each, zero rows for a slot that is not adapted), and the shrink
  * is part of the base GEMV; otherwise shrink units ride in the GEMV launch and read the A pointers.
+ * lora_dense == 2: as 1, except that o_p is the base weight alone: the attention launch writes the o projection's
+ * shrink as one share per head (mlora_rope_attn_decode_oshrink) and riders of the o GEMV launch expand it
+ * (mlora_gemv_frag_acc_ksplit_delta).  Needs mlora_rope_attn_oshrink_ok(T, Hq, Hkv, D, r), ks =
+ * mlora_gemv_delta_ride_ksplit(T, Hq*D, H, r) > 0, a ksplit_ws of ks slots of [T, H], and Hq * T * r floats in a
+ * lora_ws slot.
  * Per step: tokens[t] (in) is embedded, attends at position pos[t] of sequence row rows[t] (ctx[t] = pos[t] + 1
  * positions visible), and tokens[t] (out) receives the greedy next token; pos and ctx are then incremented on the
  * device, so the call can be replayed from a captured graph without host work while no new page is needed.

@@ -29,6 +29,17 @@ struct LoraExpandQKV {
   int r, n_ad;
 };
 
+// The o projection's LoRA shrink taken off the attention output where it is produced: the workgroup of (sequence t,
+// kv head) adds nothing to the output itself but writes, for each of its query heads h, the head's share of
+// v = A[id_t] . attn[t, :]  -  vpart[h][t][j] = sum over the head's D dims of f16(attn[t, h, d]) * A[id_t][j][h D + d]
+// (fp32) - so that the consumer adds Hq head shares per (token, rank entry) in head order and needs no pass over K.
+struct OShrinkHeads {
+  const f16* A;           // [n_ad, r, Hq * D]; nullptr: no shrink in this launch
+  float* vpart;           // [Hq, T, r]
+  const int32_t* ids;     // [T]
+  int r, n_ad, T;
+};
+
 // grid (T, Hq + 2 Hkv), 64 threads: thread i rotates the pair (i, i + D/2) of one head of one token
 __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qkv, f16* __restrict__ k_cache,
                                                             f16* __restrict__ v_cache,
@@ -438,12 +449,13 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ seq_ids,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ ctx_len, const float* __restrict__ rope_cos,
     const float* __restrict__ rope_sin, int max_pos, int Hq, int Hkv, int n_pages, int n_seq, float scale, int frag_tt,
-    LoraExpandQKV lx) {
+    LoraExpandQKV lx, OShrinkHeads os) {
   constexpr int NKB = D / 32;
   constexpr int NDB = D / 16;
   constexpr int half = D / 2;
   __shared__ float sm[NW][16], sl[NW][16];
   __shared__ float lv[3][64];
+  __shared__ f16x8 oslice[NW * WAVE];            // a thread's piece of A_o[id] waits here from the prologue to the epilogue
   __shared__ float lvq[LORA_MAX_KQ][3][64];     // K-range blocks of dense shrink results before they are added
   __shared__ __align__(16) f16 qs[16 * D];       // rotated q of the group's heads
   __shared__ __align__(16) f16 knew[D], vnew[D];   // the new token's rotated key and its value
@@ -458,6 +470,7 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
   asm volatile("" ::"s"(ctx_len), "s"(rope_cos), "s"(rope_sin), "s"(max_pos), "s"(Hq), "s"(Hkv), "s"(n_pages), "s"(n_seq));
   asm volatile("" ::"s"(scale), "s"(frag_tt), "s"(lx.src.v), "s"(lx.src.kc), "s"(lx.src.kq), "s"(lx.src.T), "s"(lx.ids), "s"(lx.scaling));
   asm volatile("" ::"s"(lx.B[0]), "s"(lx.B[1]), "s"(lx.B[2]), "s"(lx.r), "s"(lx.n_ad), "s"(lx.src.n_ad), "s"(lx.src.ld));
+  asm volatile("" ::"s"(os.A), "s"(os.vpart), "s"(os.ids), "s"(os.r), "s"(os.n_ad), "s"(os.T));
   const int b = blockIdx.y, kh = blockIdx.x;
   const int G = Hq / Hkv;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -467,8 +480,10 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
   const int pos = tok_pos[b];
   int ctx = ctx_len[b];
   const int id_raw = (lora ? lx.ids : seq_ids)[b];
-  asm volatile("" ::"s"(seq), "s"(pos), "s"(ctx), "s"(id_raw));
+  const int oid_raw = (os.A != nullptr ? os.ids : seq_ids)[b];
+  asm volatile("" ::"s"(seq), "s"(pos), "s"(ctx), "s"(id_raw), "s"(oid_raw));
   const int id = lora ? id_raw : -1;
+  const bool o_on = os.A != nullptr && oid_raw >= 0 && oid_raw < os.n_ad;        // uniform
   const bool seq_ok = seq >= 0 && seq < n_seq;
   if (!seq_ok) ctx = 0;
   if (ctx > max_blocks * PAGE) ctx = max_blocks * PAGE;
@@ -576,6 +591,15 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
   };
   const bool first = threadIdx.x < items;
   if (first) issue(threadIdx.x);
+  // the o shrink's operand: thread (query head qh, rank entry j, 8-dim piece c) takes its 16 bytes of A_o[id] now and
+  // parks them in LDS once they are there (the launcher has checked that the G * r * D / 8 items fit the workgroup)
+  constexpr int OPC = D / 8;
+  const bool o_mine = o_on && (int)threadIdx.x < G * os.r * OPC;
+  f16x8 oa = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  if (o_mine) {
+    const int oc = threadIdx.x % OPC, oj = (threadIdx.x / OPC) % os.r, oq = threadIdx.x / (OPC * os.r);
+    oa = ld8(os.A + ((size_t)oid_raw * os.r + oj) * ((size_t)Hq * D) + (size_t)(kh * G + oq) * D + oc * 8);
+  }
   if (adapted) {
     if (lx.src.kc == 0 && lx.src.kq > 1) {
       // dense shrink results in kq blocks of K-range partials: one thread per (block, entry) fetches, then the blocks
@@ -602,6 +626,7 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
     __syncthreads();
   }
   if (first) finish();
+  if (o_mine) oslice[threadIdx.x] = oa;
   for (int it = threadIdx.x + NW * WAVE; it < items; it += NW * WAVE) {
     issue(it);
     finish();
@@ -710,7 +735,19 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
     }
     const int h = kh * G + qh;
     const size_t oo = frag_tt ? frag_offset(b, h * D + d, frag_tt) : ((size_t)b * Hq + h) * D + d;
-    out[oo] = (f16)(L > 0.f ? o / L : 0.f);
+    const f16 of = (f16)(L > 0.f ? o / L : 0.f);
+    out[oo] = of;
+    if (o_on) qs[qh * D + d] = of;                           // the rotated queries are no longer needed: the outputs as stored
+  }
+  if (o_on) {                                                // uniform
+    __syncthreads();
+    if (o_mine) {
+      const int oc = threadIdx.x % OPC, oj = (threadIdx.x / OPC) % os.r, oq = threadIdx.x / (OPC * os.r);
+      float sum = dot8(oslice[threadIdx.x], *reinterpret_cast<const f16x8*>(&qs[oq * D + oc * 8]), 0.f);
+#pragma unroll
+      for (int o = 1; o < OPC; o <<= 1) sum += __shfl_xor(sum, o, WAVE);      // the D / 8 pieces of a row sit in neighbouring lanes
+      if (oc == 0) os.vpart[((size_t)(kh * G + oq) * os.T + b) * os.r + oj] = sum;
+    }
   }
 }
 
@@ -1172,12 +1209,21 @@ extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qk
   return mlora_launch_status("paged_attn_decode");
 }
 
-extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv, void* k_cache, void* v_cache,
-                                      const int32_t* block_table, int max_blocks, const int32_t* seq_ids,
-                                      const int32_t* tok_pos, const int32_t* ctx_len, const float* rope_cos,
-                                      const float* rope_sin, int max_pos, int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
-                                      const void* v_part, int v_dense, const void* const* Bmat, const int32_t* tok_adapter,
-                                      float scaling, int K, int r, int n_ad, void* stream) {
+// the o shrink's items (query heads of a kv head x rank entries x 8-dim pieces) must fit the workgroup the launch uses
+extern "C" int mlora_rope_attn_oshrink_ok(int B, int Hq, int Hkv, int D, int r) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || (D != 64 && D != 128)) return 0;
+  if (r != 8 && r != 16 && r != 32 && r != 64) return 0;
+  const int G = Hq / Hkv;
+  if (G > 16) return 0;
+  return G * r * (D / 8) <= attn_waves(B, Hkv, G, D) * WAVE ? 1 : 0;
+}
+
+static int rope_attn_decode_impl(void* out, int out_layout, const void* qkv, void* k_cache, void* v_cache,
+                                 const int32_t* block_table, int max_blocks, const int32_t* seq_ids,
+                                 const int32_t* tok_pos, const int32_t* ctx_len, const float* rope_cos,
+                                 const float* rope_sin, int max_pos, int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                                 const void* v_part, int v_dense, const void* const* Bmat, const int32_t* tok_adapter,
+                                 float scaling, int K, int r, int n_ad, const void* o_A, void* o_vpart, void* stream) {
   if (int e = check_attn("rope_attn_decode", Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
   MLORA_CHECK(out && qkv && k_cache && v_cache && block_table && seq_ids && tok_pos && ctx_len && rope_cos && rope_sin,
               MLORA_ERR_INVALID, "rope_attn_decode: null pointer");
@@ -1201,6 +1247,16 @@ extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv
     lx.scaling = scaling;
     lx.r = r; lx.n_ad = n_ad;
   }
+  OShrinkHeads os = {};
+  if (o_A != nullptr) {
+    MLORA_CHECK(o_vpart && tok_adapter && n_ad > 0, MLORA_ERR_INVALID, "rope_attn_decode: null o-shrink argument");
+    MLORA_CHECK(mlora_rope_attn_oshrink_ok(B > 0 ? B : 1, Hq, Hkv, D, r), MLORA_ERR_UNSUPPORTED,
+                "rope_attn_decode: the o shrink of rank %d does not fit the workgroup of this launch (B=%d Hq=%d Hkv=%d D=%d)", r, B, Hq, Hkv, D);
+    os.A = (const f16*)o_A;
+    os.vpart = (float*)o_vpart;
+    os.ids = tok_adapter;
+    os.r = r; os.n_ad = n_ad; os.T = B;
+  }
   if (B == 0) return MLORA_OK;
   const int frag_tt = out_layout == MLORA_FRAG ? mlora_frag_tiles(B) : 0;
   const float scale = 1.f / sqrtf((float)D);
@@ -1210,7 +1266,7 @@ extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv
 #define MLORA_ROPE_ATTN(DD, RG, NWV)                                                                                             \
   hipLaunchKernelGGL((rope_attn_decode_kernel<DD, RG, NWV>), dim3(Hkv, B), dim3(NWV * WAVE), lds, s, (f16*)out, (const f16*)qkv, \
                      (f16*)k_cache, (f16*)v_cache, block_table, max_blocks, seq_ids, tok_pos, ctx_len, rope_cos, rope_sin,       \
-                     max_pos, Hq, Hkv, n_pages, n_seq, scale, frag_tt, lx)
+                     max_pos, Hq, Hkv, n_pages, n_seq, scale, frag_tt, lx, os)
 #define MLORA_ROPE_ATTN_NW(DD, RG)             \
   do {                                         \
     if (nw == 16) MLORA_ROPE_ATTN(DD, RG, 16); \
@@ -1228,6 +1284,30 @@ extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv
 #undef MLORA_ROPE_ATTN_NW
 #undef MLORA_ROPE_ATTN
   return mlora_launch_status("rope_attn_decode");
+}
+
+extern "C" int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv, void* k_cache, void* v_cache,
+                                      const int32_t* block_table, int max_blocks, const int32_t* seq_ids,
+                                      const int32_t* tok_pos, const int32_t* ctx_len, const float* rope_cos,
+                                      const float* rope_sin, int max_pos, int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                                      const void* v_part, int v_dense, const void* const* Bmat, const int32_t* tok_adapter,
+                                      float scaling, int K, int r, int n_ad, void* stream) {
+  return rope_attn_decode_impl(out, out_layout, qkv, k_cache, v_cache, block_table, max_blocks, seq_ids, tok_pos, ctx_len, rope_cos,
+                               rope_sin, max_pos, B, Hq, Hkv, D, n_pages, n_seq, v_part, v_dense, Bmat, tok_adapter, scaling, K, r, n_ad,
+                               nullptr, nullptr, stream);
+}
+
+extern "C" int mlora_rope_attn_decode_oshrink(void* out, int out_layout, const void* qkv, void* k_cache, void* v_cache,
+                                              const int32_t* block_table, int max_blocks, const int32_t* seq_ids,
+                                              const int32_t* tok_pos, const int32_t* ctx_len, const float* rope_cos,
+                                              const float* rope_sin, int max_pos, int B, int Hq, int Hkv, int D, int n_pages,
+                                              int n_seq, const void* v_part, int v_dense, const void* const* Bmat,
+                                              const int32_t* tok_adapter, float scaling, int K, int r, int n_ad, const void* o_A,
+                                              void* o_vpart, void* stream) {
+  MLORA_CHECK(o_A && o_vpart, MLORA_ERR_INVALID, "rope_attn_decode_oshrink: null o-shrink argument");
+  return rope_attn_decode_impl(out, out_layout, qkv, k_cache, v_cache, block_table, max_blocks, seq_ids, tok_pos, ctx_len, rope_cos,
+                               rope_sin, max_pos, B, Hq, Hkv, D, n_pages, n_seq, v_part, v_dense, Bmat, tok_adapter, scaling, K, r, n_ad,
+                               o_A, o_vpart, stream);
 }
 
 extern "C" int mlora_paged_attn_prefill(void* out, int out_layout, const void* qkv, const void* k_cache, const void* v_cache,

@@ -147,12 +147,19 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
   const bool dense = lora && p->lora_dense != 0;
   const int r = p->lora_r, n_ad = p->lora_n_ad;
   const float sc = p->lora_scaling;
+  // the o projection's delta from riders of its GEMV launch (o_p is then the base weight alone)
+  const bool o_ride = dense && p->lora_dense == 2;
+  const int ks_ride = o_ride ? mlora_gemv_delta_ride_ksplit(T, q_sz, H, r) : 0;
+  MLORA_CHECK(!o_ride || (ks_ride > 0 && mlora_rope_attn_oshrink_ok(T, Hq, Hkv, D, r) && p->ksplit_ws &&
+                          mlora_gemv_ksplit_bytes(T, H, ks_ride + 1) <= p->ksplit_ws_bytes),
+              MLORA_ERR_UNSUPPORTED, "decode_step: lora_dense = 2 is not served for T=%d, rank %d, or ksplit_ws is too small", T, r);
   f16* qkv = (f16*)p->qkv;
   f16* gu = (f16*)p->gate_up;
   // LoRA scratch: slots 0-2 q/k/v partials, slot 3 o_proj, slot 4 down_proj / stand-alone calls
   const int Kmax = H > I ? (H > q_sz ? H : q_sz) : (I > q_sz ? I : q_sz);
   size_t slot = lora ? mlora_gather_mm_workspace_bytes(T, Kmax, r) : 0;
   if (dense && slot < (size_t)T * n_ad * r * sizeof(float)) slot = (size_t)T * n_ad * r * sizeof(float);
+  if (o_ride && slot < (size_t)Hq * T * r * sizeof(float)) slot = (size_t)Hq * T * r * sizeof(float);   // the o shrink's head shares
   // dense q/k/v shrink rows may come as kq blocks of K-range partials (one-workgroup-per-unit GEMV): 3 kq slots
   const int kq = dense ? mlora_gemv_split_kq(T, H, qkv_sz, 3 * n_ad * r) : 1;
   const size_t ws_need = (size_t)(3 * kq + 2) * slot;
@@ -203,25 +210,44 @@ extern "C" int mlora_decode_step(const mlora_decode_plan* p, void* stream) {
     const mlora_layer& L = p->layers[l];
     STEP(norm(L.ln1, pending_B, ws_down, I, pending_ks));
     const bool qkv_lora = lora && (L.lora[MLORA_Q].A || L.lora[MLORA_K].A || L.lora[MLORA_V].A);
+    const bool o_lora = lora && L.lora[MLORA_O].A;
+    const bool o_via_ride = o_lora && o_ride;   // the attention launch writes the o shrink's head shares, riders of the o GEMV expand them
     if (qkv_lora) {
       const void* A3[3] = {L.lora[MLORA_Q].A, L.lora[MLORA_K].A, L.lora[MLORA_V].A};
       const void* B3[3] = {L.lora[MLORA_Q].A ? L.lora[MLORA_Q].B : nullptr, L.lora[MLORA_K].A ? L.lora[MLORA_K].B : nullptr,
                            L.lora[MLORA_V].A ? L.lora[MLORA_V].B : nullptr};
       if (dense) STEP(mlora_gemv_frag_split_kq(qkv, (float*)ws_qkv, kq, p->xn, L.qkv_p, T, H, qkv_sz, 3 * n_ad * r, stream));
       else STEP(mlora_gemv_frag_lora(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, ws_qkv, A3, 3, p->tok_adapter, r, n_ad, stream));
-      STEP(mlora_rope_attn_decode(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos,
-                                  p->ctx, p->rope_cos, p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, ws_qkv, dense ? kq : 0,
-                                  B3, p->tok_adapter, sc, H, r, n_ad, stream));
+      if (o_via_ride)
+        STEP(mlora_rope_attn_decode_oshrink(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows,
+                                            p->pos, p->ctx, p->rope_cos, p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq,
+                                            ws_qkv, dense ? kq : 0, B3, p->tok_adapter, sc, H, r, n_ad, L.lora[MLORA_O].A, ws_o, stream));
+      else
+        STEP(mlora_rope_attn_decode(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos,
+                                    p->ctx, p->rope_cos, p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, ws_qkv,
+                                    dense ? kq : 0, B3, p->tok_adapter, sc, H, r, n_ad, stream));
     } else {
       STEP(mlora_gemv_frag(qkv, MLORA_F16, MLORA_STORE, p->xn, L.qkv_p, T, H, qkv_sz, stream));
-      STEP(mlora_rope_attn_decode(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos,
-                                  p->ctx, p->rope_cos, p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, nullptr, 0,
-                                  nullptr, nullptr, 0.f, 0, 0, 0, stream));
+      if (o_via_ride)
+        STEP(mlora_rope_attn_decode_oshrink(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows,
+                                            p->pos, p->ctx, p->rope_cos, p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq,
+                                            nullptr, 0, nullptr, p->tok_adapter, sc, H, r, n_ad, L.lora[MLORA_O].A, ws_o, stream));
+      else
+        STEP(mlora_rope_attn_decode(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos,
+                                    p->ctx, p->rope_cos, p->rope_sin, p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, nullptr, 0,
+                                    nullptr, nullptr, 0.f, 0, 0, 0, stream));
     }
-    const bool o_lora = lora && L.lora[MLORA_O].A;
-    const int ks_o = ksplit_of(q_sz, o_lora);
-    STEP(acc_gemv(p->attn, L.o_p, q_sz, L.lora[MLORA_O], ws_o, ks_o));
-    STEP(norm(L.ln2, o_lora ? L.lora[MLORA_O].B : nullptr, ws_o, q_sz, ks_o));
+    if (o_via_ride) {
+      // base GEMV + riders; the delta rows are one more slot of partials for the norm, which has no table to stream
+      STEP(mlora_gemv_frag_acc_ksplit_delta(p->resid, p->ksplit_ws, ks_ride, p->attn, L.o_p, T, q_sz, H, (const float*)ws_o, Hq,
+                                            L.lora[MLORA_O].B, p->tok_adapter, sc, r, n_ad, stream));
+      STEP(mlora_rmsnorm_ksplit(p->xn, MLORA_FRAG, p->resid, p->ksplit_ws, ks_ride + 1, H, L.ln2, p->eps, T, H, nullptr, 0, nullptr, nullptr,
+                                0.f, 0, 0, 0, stream));
+    } else {
+      const int ks_o = ksplit_of(q_sz, o_lora);
+      STEP(acc_gemv(p->attn, L.o_p, q_sz, L.lora[MLORA_O], ws_o, ks_o));
+      STEP(norm(L.ln2, o_lora ? L.lora[MLORA_O].B : nullptr, ws_o, q_sz, ks_o));
+    }
     const bool gu_lora = lora && (L.lora[MLORA_GATE].A || L.lora[MLORA_UP].A);
     if (L.gate_up_il_p && !gu_lora) {
       STEP(mlora_gemv_frag_silu(p->act, p->xn, L.gate_up_il_p, T, H, I, stream));

@@ -29,15 +29,86 @@ __device__ __forceinline__ int udiv_le4(int v, int d) {
   return (int)(d == 4 ? u >> 2 : d == 3 ? u / 3u : d == 2 ? u >> 1 : u);
 }
 
+// The expand of a LoRA delta by workgroups that ride at the front of an accumulating GEMV launch.  The shrink results
+// come as `n_vpart` shares per (token, rank entry) - vpart [n_vpart, T, r] fp32, e.g. one share per attention head from
+// the kernel that produced the launch's token block - which rider (t, part) adds in share order before it writes
+// delta[t][c] = scaling * B[id_t][c] . v for its share of the N columns into `out` [T, N] fp32 (zeros for a token
+// without adapter): a row block that the reader of y adds like a K-slice partial.  The GEMV's own rows stay the base
+// weight (no appended adapter rows), and the norm that follows has no table to stream - its B rows arrive here, a few
+// KiB per rider, under the shadow of the weight stream.
+struct LoraDeltaRide {
+  const float* vpart;   // [n_vpart, T, r]
+  const f16* B;         // [n_ad, N, r]
+  const int32_t* ids;   // [T]
+  float* out;           // [T, N]
+  float scaling;
+  int n_vpart, T, N, r, n_ad, per_token;
+};
+
+constexpr int RIDE_BQ = 2;     // 16-byte chunks of B per rider thread: a rider is short, and there are many of them
+
+__device__ __forceinline__ void lora_delta_ride(const LoraDeltaRide& d, int unit, float* __restrict__ lds) {
+  constexpr int NTH = GEMV_WAVES * WAVE;
+  const int tid = threadIdx.x;
+  const int t = unit / d.per_token, part = unit - t * d.per_token;
+  const int ncol = d.N / d.per_token, c0 = part * ncol;
+  float* __restrict__ out = d.out + (size_t)t * d.N + c0;
+  const int id = d.ids[t];                                   // uniform
+  if (id < 0 || id >= d.n_ad) {
+    for (int c = tid * 4; c < ncol; c += NTH * 4) *reinterpret_cast<f32x4*>(out + c) = f32x4{0.f, 0.f, 0.f, 0.f};
+    return;
+  }
+  const int r = d.r, lpr = r >> 3;                           // 16-byte chunks per row of B
+  const int nq = ncol * lpr;                                 // chunks of this rider's rows of B: at most RIDE_BQ per thread
+  // one round of requests: the rider's rows of B (uniform base + 32-bit lane offset) and the shares of v
+  f16x8 bv[RIDE_BQ];
+  const f16* __restrict__ Bp = d.B + ((size_t)id * d.N + c0) * r;
+#pragma unroll
+  for (int u = 0; u < RIDE_BQ; ++u) {
+    const int q = u * NTH + tid;
+    bv[u] = ld8(Bp + (unsigned)((q < nq ? q : 0) * 8));
+  }
+  float* __restrict__ sh = lds;                              // [n_vpart][r] shares, then [r] their sum
+  float* __restrict__ lv = lds + d.n_vpart * r;
+  for (int e = tid; e < d.n_vpart * r; e += NTH) {
+    const int h = e / r, jj = e - h * r;
+    sh[e] = d.vpart[((size_t)h * d.T + t) * r + jj];
+  }
+  __syncthreads();
+  if (tid < r) {
+    float a = 0.f;
+    for (int h = 0; h < d.n_vpart; ++h) a += sh[h * r + tid];      // share order
+    lv[tid] = a * d.scaling;
+  }
+  __syncthreads();
+  // a thread's chunks all cover the same 8 ranks (the thread count is a multiple of the chunks per row)
+  const int csub = tid % lpr;
+  float lvr[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) lvr[e] = lv[csub * 8 + e];
+#pragma unroll
+  for (int u = 0; u < RIDE_BQ; ++u) {
+    const int q = u * NTH + tid;
+    float sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum = fmaf((float)bv[u][e], lvr[e], sum);
+    for (int o = 1; o < lpr; o <<= 1) sum += __shfl_xor(sum, o, WAVE);
+    if (csub == 0 && q < nq) out[q / lpr] = sum;
+  }
+}
+
 // With SHRINK the first `shrink_blocks` workgroups of the launch do LoRA shrink units (one per wave) on the same
 // x instead of a GEMV tile: the adapter work rides in the GEMV launch and finishes long before it does.
+// An accumulating launch without shrink units may instead carry `ride_blocks` delta riders (lora_delta_ride).
 template <int NT, int TT, int OUT, bool PACKED, bool XFRAG, bool SHRINK, int PIPE = 4>   // PIPE: k-steps in flight per wave
 __global__ __launch_bounds__(GEMV_WAVES* WAVE, (NT * TT > 8 ? 2 : 4)) void gemv_kernel(void* __restrict__ yv, const f16* __restrict__ x, int ldx,
                                                                 const f16* __restrict__ W, int T, int K, int N,
                                                                 LoraShrinkBatch sb, int shrink_blocks, int n_main,
-                                                                float* __restrict__ y2, int ksplit, float* __restrict__ part) {
+                                                                float* __restrict__ y2, int ksplit, float* __restrict__ part,
+                                                                LoraDeltaRide dr, int ride_blocks) {
   constexpr int TILES = NT * TT;
   constexpr int HT = TILES > 8 ? TILES / 2 : TILES;   // accumulator tiles summed per pass through LDS (64 KiB holds 8)
+  constexpr bool RIDE = OUT == OUT_ACC_F32 && PACKED && XFRAG && !SHRINK;   // the launches that may carry delta riders
   __shared__ f32x4 red[GEMV_WAVES][HT][WAVE];
   // all arguments in one round of scalar loads, ahead of the first weight request (the compiler would fetch each
   // group at its first use, a dependent round each time)
@@ -45,6 +116,13 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, (NT * TT > 8 ? 2 : 4)) void gemv_
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps the k-loop control scalar
   const int lane = threadIdx.x & 63;
   int bid = blockIdx.x;
+  if constexpr (RIDE) {
+    if (bid < ride_blocks) {                       // uniform
+      lora_delta_ride(dr, bid, reinterpret_cast<float*>(&red[0][0][0]));
+      return;
+    }
+    bid -= ride_blocks;
+  }
   if constexpr (SHRINK) {
     if (bid < shrink_blocks) {
       const int unit = bid * GEMV_WAVES + wave;
@@ -418,12 +496,13 @@ __global__ __launch_bounds__(256) void pack_activation_kernel(f16* __restrict__ 
 
 template <int NT, int TT, bool PACKED, bool XFRAG, bool SHRINK, int PIPE = 4>
 void launch_gemv(void* y, int out, const f16* x, int ldx, const f16* W, int T, int K, int N, hipStream_t s,
-                 const LoraShrinkBatch& sb, int n_main, float* y2, int ksplit = 1, float* part = nullptr) {
+                 const LoraShrinkBatch& sb, int n_main, float* y2, int ksplit = 1, float* part = nullptr,
+                 const LoraDeltaRide& dr = LoraDeltaRide(), int rblocks = 0) {
   const int sblocks = SHRINK ? ceil_div(lora_shrink_units(sb), GEMV_WAVES) : 0;
-  const dim3 grid(ceil_div(N, 16 * NT) * ksplit + sblocks), block(GEMV_WAVES * WAVE);
-  if (out == OUT_F16) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F16, PACKED, XFRAG, SHRINK, PIPE>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2, ksplit, part);
-  else if (out == OUT_F32) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F32, PACKED, XFRAG, SHRINK, PIPE>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2, ksplit, part);
-  else hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_ACC_F32, PACKED, XFRAG, SHRINK, PIPE>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2, ksplit, part);
+  const dim3 grid(ceil_div(N, 16 * NT) * ksplit + sblocks + rblocks), block(GEMV_WAVES * WAVE);
+  if (out == OUT_F16) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F16, PACKED, XFRAG, SHRINK, PIPE>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2, ksplit, part, dr, 0);
+  else if (out == OUT_F32) hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_F32, PACKED, XFRAG, SHRINK, PIPE>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2, ksplit, part, dr, 0);
+  else hipLaunchKernelGGL((gemv_kernel<NT, TT, OUT_ACC_F32, PACKED, XFRAG, SHRINK, PIPE>), grid, block, 0, s, y, x, ldx, W, T, K, N, sb, sblocks, n_main, y2, ksplit, part, dr, rblocks);
 }
 
 // Rows per workgroup.  Every workgroup reads the whole token block, so its L2 traffic is T / (16 NT) of the weight
@@ -443,7 +522,7 @@ int gemv_n_cu() {
 template <bool PACKED, bool XFRAG, bool SHRINK = false>
 int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const void* W, int T, int K, int N, void* stream,
                   const LoraShrinkBatch& sb = LoraShrinkBatch(), int n_main = -1, float* y2 = nullptr, int ksplit = 1,
-                  float* part = nullptr) {
+                  float* part = nullptr, const LoraDeltaRide& dr = LoraDeltaRide(), int rblocks = 0) {
   if (n_main < 0) n_main = N;
   const int out = mode == MLORA_ACCUMULATE ? OUT_ACC_F32 : (y_dtype == MLORA_F32 ? OUT_F32 : OUT_F16);
   hipStream_t s = (hipStream_t)stream;
@@ -460,8 +539,8 @@ int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const 
         else launch_gemv<3, 2, PACKED, XFRAG, SHRINK, 4>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part);
         return mlora_launch_status("gemv");
       }
-      if (T <= 16) launch_gemv<4, 1, PACKED, XFRAG, SHRINK, 4>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part);
-      else launch_gemv<4, 2, PACKED, XFRAG, SHRINK, 3>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part);
+      if (T <= 16) launch_gemv<4, 1, PACKED, XFRAG, SHRINK, 4>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part, dr, rblocks);
+      else launch_gemv<4, 2, PACKED, XFRAG, SHRINK, 3>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part, dr, rblocks);
       return mlora_launch_status("gemv");
     }
   }
@@ -480,7 +559,7 @@ int gemv_dispatch(void* y, int y_dtype, int mode, const void* x, int ldx, const 
     // traffic instead of four times): 5.3 -> 4.4 ms of GEMV per decode step at T = 64
     if constexpr (PACKED && XFRAG) {
       if (ksplit > 1 || tiles >= 768) {           // one workgroup per unit with four row tiles: the token block is read once per unit
-        launch_gemv<4, 4, PACKED, XFRAG, SHRINK, 2>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part);
+        launch_gemv<4, 4, PACKED, XFRAG, SHRINK, 2>(y, out, xp, ldx, Wp, T, K, N, s, sb, n_main, y2, ksplit, part, dr, rblocks);
         return mlora_launch_status("gemv");
       }
       if (tiles > 256) {                          // 257..511 tiles as one-tile workgroups would need a second, thin round
@@ -623,6 +702,50 @@ extern "C" int mlora_gemv_frag_acc_ksplit(float* y, float* y2, float* part, int 
                                           ks, part);
 }
 
+// Riders per token of the delta-carrying launch below (0: the shape is not served): a rider thread keeps at most
+// RIDE_BQ 16-byte chunks of B, the launch must be K-split (it is the split form of the kernel that carries riders),
+// and with riders the slices are chosen as if the matrix had 256 more rows (sixteen workgroups' worth, as for the
+// riding shrink units: a constant, so that the slice count does not depend on the batch).
+static int delta_ride_per_token(int T, int K, int N, int r) {
+  if (T <= 0 || T > 64 || K <= 0 || K % 32 || N <= 0 || N % 16) return 0;
+  if (r != 8 && r != 16 && r != 32 && r != 64) return 0;
+  const int per_thread = ceil_div(N * (r / 8), GEMV_WAVES * WAVE);
+  const int per_token = ceil_div(per_thread, RIDE_BQ);
+  if (N % per_token || (N / per_token) % 4) return 0;
+  if (mlora_gemv_ksplit(T, K, N + 256) < 2) return 0;
+  return per_token;
+}
+
+// at most three slices: with the delta rows the reader then adds three slots, the most the RMSNorm takes
+extern "C" int mlora_gemv_delta_ride_ksplit(int T, int K, int N, int r) {
+  if (delta_ride_per_token(T, K, N, r) <= 0) return 0;
+  const int ks = mlora_gemv_ksplit(T, K, N + 256);
+  return ks > 3 ? 3 : ks;
+}
+
+extern "C" int mlora_gemv_frag_acc_ksplit_delta(float* y, float* part, int ks, const void* xf, const void* Wp, int T, int K, int N,
+                                                const float* vpart, int n_vpart, const void* B, const int32_t* tok_adapter,
+                                                float scaling, int r, int n_ad, void* stream) {
+  if (int e = mlora_check_linear("gemv_frag_acc_ksplit_delta", y, MLORA_F32, MLORA_ACCUMULATE, xf, K, Wp, T, K, N)) return e;
+  MLORA_CHECK(part && vpart && B && tok_adapter && n_ad > 0, MLORA_ERR_INVALID, "gemv_frag_acc_ksplit_delta: null pointer or no adapters");
+  const int per_token = delta_ride_per_token(T, K, N, r);
+  MLORA_CHECK(per_token > 0 && ks == mlora_gemv_delta_ride_ksplit(T, K, N, r) && (K / KSTEP) / ks >= 8, MLORA_ERR_UNSUPPORTED,
+              "gemv_frag_acc_ksplit_delta: T=%d K=%d N=%d r=%d ks=%d not served (mlora_gemv_delta_ride_ksplit gives %d)", T, K, N, r, ks,
+              mlora_gemv_delta_ride_ksplit(T, K, N, r));
+  MLORA_CHECK(n_vpart >= 1 && (size_t)(n_vpart + 1) * r * sizeof(float) <= 32 * 1024, MLORA_ERR_UNSUPPORTED,
+              "gemv_frag_acc_ksplit_delta: %d shares of rank %d do not fit the rider's LDS", n_vpart, r);
+  LoraDeltaRide dr;
+  dr.vpart = vpart;
+  dr.B = (const f16*)B;
+  dr.ids = tok_adapter;
+  dr.out = part + (size_t)(ks - 1) * T * N;       // the slot behind the K-slice partials
+  dr.scaling = scaling;
+  dr.n_vpart = n_vpart; dr.T = T; dr.N = N; dr.r = r; dr.n_ad = n_ad;
+  dr.per_token = per_token;
+  return gemv_dispatch<true, true, false>(y, MLORA_F32, MLORA_ACCUMULATE, xf, K, Wp, T, K, N, stream, LoraShrinkBatch(), N, nullptr, ks,
+                                          part, dr, T * per_token);
+}
+
 extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p, int T, int K, int I, void* stream) {
   MLORA_CHECK(act && xf && Wil_p, MLORA_ERR_INVALID, "gemv_frag_silu: null pointer");
   MLORA_CHECK(T > 0 && T <= 64 && K > 0 && K % 32 == 0 && I > 0 && I % 32 == 0, MLORA_ERR_UNSUPPORTED,
@@ -656,9 +779,9 @@ extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p
 #undef MLORA_SILU_CU
     return mlora_launch_status("gemv_frag_silu");
   }
-  if (T <= 16) hipLaunchKernelGGL((gemv_kernel<2, 1, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);
-  else if (T <= 32) hipLaunchKernelGGL((gemv_kernel<2, 2, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);
-  else hipLaunchKernelGGL((gemv_kernel<2, 4, OUT_SILU_FRAG, true, true, false, 2>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr);
+  if (T <= 16) hipLaunchKernelGGL((gemv_kernel<2, 1, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr, LoraDeltaRide(), 0);
+  else if (T <= 32) hipLaunchKernelGGL((gemv_kernel<2, 2, OUT_SILU_FRAG, true, true, false>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr, LoraDeltaRide(), 0);
+  else hipLaunchKernelGGL((gemv_kernel<2, 4, OUT_SILU_FRAG, true, true, false, 2>), grid, block, 0, s, act, xp, K, Wp, T, K, 2 * I, sb, 0, 2 * I, nullptr, 1, nullptr, LoraDeltaRide(), 0);
   return mlora_launch_status("gemv_frag_silu");
 }
 

@@ -133,8 +133,9 @@ class NativeDecodeSession:
         }
         r = lt.r if lt is not None else 0
         # five slots (q, k, v, o, down); the dense q/k/v shrink may come as up to four K-range blocks of three slots
+        # (a slot also holds the o shrink's head shares, [heads, T, r] fp32)
         ws_bytes = 14 * max(_lib.lib().mlora_gather_mm_workspace_bytes(T, max(H, I, s.q_size), max(r, 8)),
-                            4 * T * (lt.n_adapters if lt is not None else 0) * max(r, 8))
+                            4 * T * (lt.n_adapters if lt is not None else 0) * max(r, 8), 4 * s.num_attention_heads * T * max(r, 8))
         self.buf["lora_ws"] = torch.empty(ws_bytes // 4, dtype=f32, device=dev)
         # partials of the K-split o_proj / down_proj GEMVs (up to 3 slices of [T, H + appended adapter rows])
         ks_elems = 3 * T * (H + (lt.n_adapters * r if lt is not None else 0)) if ksplit else 0
@@ -149,7 +150,13 @@ class NativeDecodeSession:
         if dense_lora and T > 64:
             raise ValueError("NativeDecodeSession: the dense shrink serves at most 64 sequences per step")
         self.dense_lora = bool(dense_lora and lt is not None)
-        ext = model.dense_lora_weights(tid) if self.dense_lora else None
+        # the o projection without appended rows: the attention launch writes its shrink as one share per head and riders
+        # of the o GEMV launch expand it (base weight alone, no table for the norm to stream) - where the library serves
+        # the shape that way and there is room for the delta rows behind the slice partials
+        ks_ride = _lib.lib().mlora_gemv_delta_ride_ksplit(T, s.q_size, H, r) if (self.dense_lora and ksplit) else 0
+        self.o_delta_ride = bool(ks_ride > 0 and 4 * ks_elems >= _lib.lib().mlora_gemv_ksplit_bytes(T, H, ks_ride + 1) and
+                                 _lib.lib().mlora_rope_attn_oshrink_ok(T, s.num_attention_heads, s.num_key_value_heads, s.head_dim, r))
+        ext = model.dense_lora_weights(tid, with_o=not self.o_delta_ride) if self.dense_lora else None
         il = model.interleaved_gate_up() if (fuse_silu and s.intermediate_size % 32 == 0) else None
         for l, L in enumerate(model.layers):
             if il is not None:
@@ -168,7 +175,7 @@ class NativeDecodeSession:
         p.n_q_heads, p.n_kv_heads, p.head_dim, p.vocab, p.eps = s.num_attention_heads, s.num_key_value_heads, s.head_dim, V, s.rms_norm_eps
         if lt is not None:
             p.lora_r, p.lora_n_ad, p.lora_scaling = lt.r, lt.n_adapters, lt.scaling
-            p.lora_dense = 1 if self.dense_lora else 0
+            p.lora_dense = (2 if self.o_delta_ride else 1) if self.dense_lora else 0
         p.layers = C.cast(layers, C.POINTER(_lib.Layer))
         p.embed, p.norm, p.lm_head_p = model.embed_tokens.data_ptr(), model.norm.data_ptr(), model.lm_head.data.data_ptr()
         p.rope_cos, p.rope_sin, p.max_pos = kv.rope_cos.data_ptr(), kv.rope_sin.data_ptr(), kv.max_pos

@@ -166,17 +166,19 @@ class LlamaForCausalLM:
             full = np.where(ids >= 0, ids + base[tid], full)
         return full.astype(np.int32)
 
-    def dense_lora_weights(self, tid=0):
+    def dense_lora_weights(self, tid=0, with_o=True):
         """Per layer, the qkv / o / down weights with the stacked A tables of adapter type `tid` (or of the union of
         a tuple of types) appended as extra rows ([n_ad * r, K] per adapted projection; q, k, v slots always present
-        for qkv, zero when not adapted), in fragment order.  Cached; costs one more copy of those matrices."""
+        for qkv, zero when not adapted), in fragment order.  with_o=False leaves o as the base weight (its delta then
+        comes from riders of the GEMV launch).  Cached; costs one more copy of those matrices."""
         cache = getattr(self, "_dense_cache", None)
         if cache is None:
             cache = self._dense_cache = {}
         if isinstance(tid, tuple) and len(tid) == 1:
             tid = tid[0]
-        if tid in cache:
-            return cache[tid]
+        ck = (tid, bool(with_o))
+        if ck in cache:
+            return cache[ck]
         lt = self.lora_union(tid)[0] if isinstance(tid, tuple) else self.lora_types[tid]
         out = []
         for l, L in enumerate(self.layers):
@@ -192,12 +194,12 @@ class LlamaForCausalLM:
             else:
                 ent["qkv"] = L["qkv"]
             for key, proj, K in (("o", "o_proj", self.shape.q_size), ("down", "down_proj", I)):
-                if (l, proj) in lt.tables:
+                if (l, proj) in lt.tables and (with_o or key != "o"):
                     ent[key] = ops.PackedWeight(torch.cat([L[key].unpack(), slot(proj, K)]))
                 else:
                     ent[key] = L[key]
             out.append(ent)
-        cache[tid] = out
+        cache[ck] = out
         return out
 
     def create_paged_kv_cache(self, max_batch_size, max_total_seq_len, prefill_chunk_size, page_size,

@@ -475,6 +475,28 @@ def linear_acc_ksplit(x: FragActivation, W: PackedWeight, resid: torch.Tensor, w
     return KSplitParts(ws, ks, N) if ks > 1 else None
 
 
+def linear_acc_ksplit_delta(x: FragActivation, W: PackedWeight, resid: torch.Tensor, ws: torch.Tensor, vpart, B, tok_adapter, scaling: float):
+    """resid [T, N] fp32 += x @ W.T over K slices, with the LoRA expand scaling * B[id] @ sum_h vpart[h, t] of every token
+    done by workgroups riding in the same launch (vpart [n_shares, T, r] fp32: the shrink results as shares that are
+    added in order): returns the KSplitParts (slice partials, then the delta rows) that the next
+    `rmsnorm(resid, ..., parts=...)` adds - or None when the library does not serve the shape this way (nothing is
+    launched then)."""
+    T, K = x.shape
+    N, K2 = W.shape
+    n_ad, N2, r = B.shape
+    if K2 != K or N2 != N or vpart.dim() != 3 or tuple(vpart.shape[1:]) != (T, r) or resid.shape != (T, N) or resid.dtype != torch.float32:
+        raise ValueError(f"linear_acc_ksplit_delta: x{x.shape} W{W.shape} vpart{tuple(vpart.shape)} B{tuple(B.shape)} resid{tuple(resid.shape)}")
+    ks = lib().mlora_gemv_delta_ride_ksplit(T, K, N, r)
+    if ks <= 0:
+        return None
+    if ws.numel() * 4 < lib().mlora_gemv_ksplit_bytes(T, N, ks + 1):
+        raise ValueError("linear_acc_ksplit_delta: workspace too small")
+    check(lib().mlora_gemv_frag_acc_ksplit_delta(_dev(resid, torch.float32), _dev(ws, torch.float32), ks, x.data.data_ptr(), W.data.data_ptr(),
+                                                 T, K, N, _dev(vpart, torch.float32), vpart.shape[0], _dev(B, torch.float16, "B"),
+                                                 _dev(tok_adapter, torch.int32), float(scaling), r, n_ad, _stream()))
+    return KSplitParts(ws, ks + 1, N)
+
+
 def rmsnorm(x, w, eps: float, out=None, frag=False, parts: KSplitParts = None):
     """Row-wise RMSNorm of x [T, H] (f16 | f32); frag=True writes a FragActivation.  With `parts` (x fp32) the K-split
     partials are first added to x in place."""
@@ -556,11 +578,26 @@ def paged_attn_decode(qkv, k_cache, v_cache, block_table, seq_ids, ctx_len, Hq, 
 
 
 def rope_attn_decode(qkv, k_cache, v_cache, block_table, seq_ids, tok_pos, ctx_len, rope_cos, rope_sin, Hq, Hkv, D,
-                     out=None, frag=False):
-    """rope_kv_append + paged_attn_decode of one decode step in one launch (no LoRA); qkv is left unrotated."""
+                     out=None, frag=False, o_shrink=None):
+    """rope_kv_append + paged_attn_decode of one decode step in one launch (no LoRA on q, k, v); qkv is left unrotated.
+    o_shrink = (A [n_ad, r, Hq * D] f16, tok_adapter [B] int32): the launch also writes the o projection's shrink as
+    one share per query head and the call returns (out, vpart [Hq, B, r] fp32; rows of tokens without adapter are NaN)."""
     B = qkv.shape[0]
     n_seq, max_blocks = block_table.shape
     out, optr, lay = _out_arg(out, B, Hq * D, frag, qkv.device)
+    if o_shrink is not None:
+        A, ids = o_shrink
+        n_ad, r, Kq = A.shape
+        if Kq != Hq * D or not lib().mlora_rope_attn_oshrink_ok(B, Hq, Hkv, D, r):
+            raise ValueError(f"rope_attn_decode: o shrink A{tuple(A.shape)} not served for B={B} Hq={Hq} Hkv={Hkv} D={D}")
+        vpart = torch.full((Hq, B, r), float("nan"), dtype=torch.float32, device=qkv.device)
+        check(lib().mlora_rope_attn_decode_oshrink(optr, lay, _dev(qkv, torch.float16), _dev(k_cache, torch.float16),
+                                                   _dev(v_cache, torch.float16), _dev(block_table, torch.int32), max_blocks,
+                                                   _dev(seq_ids, torch.int32), _dev(tok_pos, torch.int32), _dev(ctx_len, torch.int32),
+                                                   _dev(rope_cos, torch.float32), _dev(rope_sin, torch.float32), rope_cos.shape[0],
+                                                   B, Hq, Hkv, D, k_cache.shape[0], n_seq, None, 0, None, _dev(ids, torch.int32), 0.0,
+                                                   0, r, n_ad, _dev(A, torch.float16, "A"), vpart.data_ptr(), _stream()))
+        return out, vpart
     check(lib().mlora_rope_attn_decode(optr, lay, _dev(qkv, torch.float16), _dev(k_cache, torch.float16),
                                        _dev(v_cache, torch.float16), _dev(block_table, torch.int32), max_blocks,
                                        _dev(seq_ids, torch.int32), _dev(tok_pos, torch.int32), _dev(ctx_len, torch.int32),

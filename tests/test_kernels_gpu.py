@@ -969,6 +969,7 @@ def test_rope_attn_decode_one_launch_equals_two(ops, synth, Hq, Hkv, D, rep):
     rope_kv_append followed by paged_attn_decode.  New tokens at the first and last slot of a page, in a fresh
     sequence (context 1) and deep into a sequence; MHA and grouped heads; an out-of-range sequence row."""
     kvm = load_pkg("kv_cache")
+    lib_ok = load_pkg("_lib").lib().mlora_rope_attn_oshrink_ok
     pos = [0, 15, 16, 31, 37, 100, 5] * rep          # rep > 1: enough (sequence, kv head) pairs for the 8-wave (> 256) and 4-wave (> 2048) workgroups
     B = len(pos)
     n_pages, max_blocks = 40 * rep, 8
@@ -999,6 +1000,29 @@ def test_rope_attn_decode_one_launch_equals_two(ops, synth, Hq, Hkv, D, rep):
         a, b_ = (got.unpack(), want.unpack()) if frag else (got, want)
         assert torch.equal(a, b_)
         assert float(a[:B - 1].abs().max()) > 0 and float(a[B - 1].abs().max()) == 0
+        # the same launch with the o projection's shrink taken off its output: same bits out, and per query head
+        # vpart[h, b, :] = A[id_b][:, h D : (h + 1) D] . out[b, h, :] for the rows that name an adapter
+        for r in (8, 16):
+            if not lib_ok(B, Hq, Hkv, D, r):
+                continue
+            n_ad = 5
+            A = synth.normal(13, f"ra.A{r}.{Hq * D}", (n_ad, r, Hq * D), 0.05, torch.float16, DEV)
+            ids = (np.arange(B) % (n_ad + 1) - 1).astype(np.int32)          # -1, 0, 1, ...
+            k3, v3, q3 = k0.clone(), v0.clone(), qkv.clone()
+            got3, vpart = ops.rope_attn_decode(q3, k3, v3, table, seqs, tpos, ctx, cos, sin, Hq, Hkv, D, frag=frag,
+                                               o_shrink=(A, torch.from_numpy(ids).to(DEV)))
+            assert torch.equal(k3, k2) and torch.equal(v3, v2)
+            a3 = got3.unpack() if frag else got3
+            assert torch.equal(a3, a)
+            o64 = _np(a3).astype(np.float64).reshape(B, Hq, D)
+            vp = _np(vpart)
+            for b in range(B):
+                if ids[b] < 0:
+                    assert np.isnan(vp[:, b]).all()                         # untouched
+                    continue
+                A64 = _np(A[ids[b]]).astype(np.float64).reshape(r, Hq, D)
+                ref = np.einsum("rhd,hd->hr", A64, o64[b])
+                assert np.abs(vp[:, b] - ref).max() <= 1e-5 + 1e-4 * np.abs(ref).max(), (b, r)
 
 
 @pytest.mark.parametrize("Hq,Hkv,D", [(4, 4, 128), (8, 2, 64)])
@@ -1124,6 +1148,67 @@ def test_gemv_ksplit_with_appended_adapter_rows(ops, synth, T, K, r, n_ad):
         assert max_rel_err(_np(resid), ref, floor=1e-2) <= 5e-4
         assert max_rel_err(_np(y), oracle.rmsnorm_ref(ref, _np(w), 1e-5)) <= TOL
     assert float((out[0][0] - out[1][0]).abs().max()) <= 1e-4
+
+
+@pytest.mark.parametrize("T,K,N,r,n_ad,shares", [(32, 4096, 4096, 16, 16, 32), (7, 4096, 4096, 8, 3, 32), (64, 11008, 4096, 16, 5, 1),
+                                                (20, 4096, 4096, 32, 4, 8), (33, 2048, 2048, 64, 2, 16), (32, 4096, 1024, 16, 16, 32),
+                                                (32, 512, 4096, 16, 16, 4)])
+def test_gemv_ksplit_with_delta_riders(ops, synth, T, K, N, r, n_ad, shares):
+    """The accumulating K-split GEMV over the base weight with the projection's LoRA expand done by riders of the launch
+    from shrink results that come as shares (K ranges of A . x here, one per attention head in the decode step):
+    residual + x . W^T + scaling * B[id] . (A[id] . x) once the RMSNorm has added the slots, against the fp64 evaluation;
+    tokens without adapter get exactly the plain K-split result."""
+    print(f"case delta_riders T={T} K={K} N={N} r={r} n_ad={n_ad} shares={shares}", flush=True)
+    lib = load_pkg("_lib").lib()
+    ks = lib.mlora_gemv_delta_ride_ksplit(T, K, N, r)
+    x = synth.normal(29, f"dr.x.{T}.{K}", (T, K), 1.0, torch.float16, DEV)
+    W = synth.normal(29, f"dr.W.{N}.{K}", (N, K), 0.02, torch.float16, DEV)
+    A = synth.normal(29, f"dr.A.{r}.{K}", (n_ad, r, K), 0.02, torch.float16, DEV)
+    B = synth.normal(29, f"dr.B.{N}.{r}", (n_ad, N, r), 0.5, torch.float16, DEV)
+    w = synth.normal(29, f"dr.w.{N}", (N,), 1.0, torch.float16, DEV)
+    r0 = synth.normal(29, f"dr.r.{T}.{N}", (T, N), 1.0, torch.float32, DEV)
+    ids = synth.randint(29, f"dr.ids.{T}", (T,), n_ad + 1).numpy().astype(np.int32) - 1       # -1 = no adapter
+    ids[0] = -1
+    ids[-1] = n_ad - 1
+    ids_d = torch.from_numpy(ids).to(DEV)
+    # the shrink as `shares` K ranges per token, NaN where a token has no adapter (never read)
+    x64 = _np(x).astype(np.float64)
+    vp = np.full((shares, T, r), np.nan, np.float32)
+    step = K // shares
+    for t in range(T):
+        if ids[t] >= 0:
+            At = _np(A[ids[t]]).astype(np.float64)
+            for h in range(shares):
+                vp[h, t] = At[:, h * step:(h + 1) * step] @ x64[t, h * step:(h + 1) * step]
+    vpart = torch.from_numpy(vp).to(DEV)
+    xf, Wp = ops.FragActivation.pack(x), ops.PackedWeight(W)
+    ws = torch.full((4 * T * N,), float("nan"), dtype=torch.float32, device=DEV)
+    racc = r0.clone()
+    parts = ops.linear_acc_ksplit_delta(xf, Wp, racc, ws, vpart, B, ids_d, 0.75)
+    if K == 512:                                     # too short for a K split: the library says so and launches nothing
+        assert ks == 0 and parts is None and torch.equal(racc, r0)
+        return
+    assert ks >= 2 and parts is not None and parts.ks == ks + 1
+    y = ops.rmsnorm(racc, w, 1e-5, parts=parts)
+    torch.cuda.synchronize()
+    ref = _np(r0).astype(np.float64) + x64 @ _np(W).astype(np.float64).T
+    delta = np.zeros((T, N))
+    for t in range(T):
+        if ids[t] >= 0:
+            delta[t] = 0.75 * (_np(B[ids[t]]).astype(np.float64) @ (_np(A[ids[t]]).astype(np.float64) @ x64[t]))
+    assert np.abs(delta).max() > 0.5                 # the deltas are visible at this scale
+    assert max_rel_err(_np(racc), ref + delta, floor=1e-2) <= 5e-4
+    assert max_rel_err(_np(y), oracle.rmsnorm_ref(ref + delta, _np(w), 1e-5)) <= TOL
+    # rows without adapter: the delta slot holds zeros, the row equals the plain K-split call with the same slice count
+    r1 = r0.clone()
+    ws1 = torch.empty_like(ws)
+    assert min(lib.mlora_gemv_ksplit(T, K, N + 256), 3) == ks
+    load_pkg("_lib").check(lib.mlora_gemv_frag_acc_ksplit(r1.data_ptr(), None, ws1.data_ptr(), ks, xf.data.data_ptr(), Wp.data.data_ptr(), T, K, N, 0,
+                                                          None, None, 0, None, 0, 0, torch.cuda.current_stream().cuda_stream))
+    ops.rmsnorm(r1, w, 1e-5, parts=ops.KSplitParts(ws1, ks, N))
+    none = np.nonzero(ids < 0)[0]
+    assert torch.equal(racc[none], r1[none])
+    assert not torch.equal(racc[-1], r1[-1])
 
 
 @pytest.mark.parametrize("T,N_main,n_ad", [(32, 12288, 48), (12, 12288, 16), (32, 8192, 10), (20, 10240, 48)])

@@ -123,7 +123,7 @@ def test_c1_greedy_tokens_with_the_dense_shrink(c1):
     exp, margins, scales = oracle.greedy_generate_ref(ref, prompts, {"a0": wl.adapter_ids}, max_gen_len, n_pages,
                                                       wl.page_size, perm, return_logits=True)
     got, batcher = run_hip_generate(model, wl, prompts, wl.adapter_ids, max_gen_len, perm, dense_lora=True)
-    assert batcher.graph._dense_ok("decode_a0") and 0 in model._dense_cache
+    assert batcher.graph._dense_ok("decode_a0") and any(k[0] == 0 for k in model._dense_cache)
     for b in range(wl.batch):
         assert len(got[b]) == max_gen_len
         i = next((i for i in range(max_gen_len) if got[b][i] != exp[b][i]), None)
@@ -205,7 +205,7 @@ def test_mixed_adapter_types_through_the_dense_native_step(c1):
                                                       perm, return_logits=True)
     wl2 = synth.Workload("mixedd", 13, wl.shape, wl.lora, batch=B, prompt_len=P, gen_len=max_gen_len)
     got, batcher = run_hip_generate(model, wl2, prompts, wids, max_gen_len, perm, tids=[max(t, 0) for t in tids], dense_lora=True)
-    assert batcher.graph._dense_ok("mixed_decode_a0_a1") and (0, 1) in model._dense_cache
+    assert batcher.graph._dense_ok("mixed_decode_a0_a1") and any(k[0] == (0, 1) for k in model._dense_cache)
     for b in range(B):
         i = next((i for i in range(max_gen_len) if got[b][i] != exp[b][i]), None)
         assert i is None or margins[b][i] < 2e-2 * scales[b][i], (b, i, got[b], exp[b], margins[b])
