@@ -65,6 +65,59 @@ def test_native_step_on_random_model_shapes():
             assert torch.equal(kc, outs[0][1]), tag
 
 
+def test_dense_native_step_on_random_model_shapes():
+    """The dense-shrink native step - adapter A rows inside the q/k/v (and down) GEMV, the o projection's shrink taken off
+    the attention launch in head shares and expanded by riders of the o GEMV launch where the library serves the shape
+    that way, appended A rows and the expand inside the RMSNorm where it does not - against the ids-based native step
+    (which is bit-identical to the per-operator path, see above) on 60 random configurations: first-step logits agree to
+    rounding-flip noise, tokens on every row whose top-2 margin is decided, cached keys to a few fp16 ulps.  Both forms of
+    the o projection must have been drawn."""
+    synth, llama, dsm, ops = load_pkg("synth"), load_pkg("llama"), load_pkg("decode_session"), load_pkg("ops")
+    rng = np.random.default_rng(20240613)
+    ride_seen = {True: 0, False: 0}
+    for case in range(60):
+        D = int(rng.choice([64, 128])); Hkv = int(rng.choice([1, 2, 4, 8])); Hq = Hkv * int(rng.choice([1, 2, 4]))
+        if case % 2 == 0:                                        # wide attention outputs: the o GEMV is K-split there, which is what carries riders
+            Hq, Hkv, D = [(16, 4, 128), (16, 8, 128), (32, 8, 128), (16, 16, 128), (32, 8, 64), (32, 32, 64)][int(rng.integers(0, 6))]
+        hidden = int(rng.choice([512, 1024, 2048, 4096])); inter = int(rng.choice([704, 1408, 2816]))
+        layers = int(rng.choice([1, 2]))
+        B = int(rng.choice([1, 3, 16, 17, 32, 33, 64])); P = int(rng.choice([3, 16, 30]))
+        r = int(rng.choice([8, 16, 32, 64])); n_ad = int(rng.choice([1, 3, 8, 24]))
+        extra = tuple(np.array(ALL)[sorted(rng.choice(7, size=int(rng.integers(0, 5)), replace=False))])
+        targets = tuple(t for t in ALL if t == "o_proj" or t in extra)
+        shape = synth.LlamaShape(hidden_size=hidden, intermediate_size=inter, num_attention_heads=Hq, num_key_value_heads=Hkv,
+                                 num_hidden_layers=layers, head_dim=D, vocab_size=int(rng.choice([512, 1000])))
+        seed = int(rng.integers(0, 1000))
+        tag = (f"case {case}: B={B} P={P} hidden={hidden} inter={inter} Hq={Hq} Hkv={Hkv} D={D} L={layers} r={r} n_ad={n_ad} "
+               f"targets={targets}")
+        print(tag, flush=True)
+        model = llama.LlamaForCausalLM.from_synthetic(seed, shape, [synth.LoraSpec(r=r, alpha=r / 2, n_adapters=n_ad, targets=targets)], DEV)
+        ids = rng.integers(-1, n_ad, size=B).astype(np.int32)
+        ids[rng.integers(0, B)] = n_ad - 1                       # at least one adapted row
+        prompts = rng.integers(0, shape.vocab_size, size=(B, P)).astype(np.int32)
+        blocks = -(-(P + 3) // 16)
+        res = {}
+        for kind in ("ids", "dense"):
+            perm = np.random.default_rng(seed).permutation(B * blocks)
+            kv = model.create_paged_kv_cache(B, B * blocks * 16, P, 16, free_pages=perm, max_seq_len=blocks * 16)
+            first = _prefill(model, kv, prompts, ids, ops)
+            sess = dsm.NativeDecodeSession(model, kv, list(range(B)), ids, first, use_graph=False, dense_lora=(kind == "dense"))
+            tok = sess.step().cpu().numpy().copy()
+            res[kind] = (tok, sess.buf["logits"].view(B, -1).clone(), kv.k.clone())
+            if kind == "dense":
+                assert sess.dense_lora, tag
+                ride_seen[bool(sess.o_delta_ride)] += 1
+        (ti, li, ki), (td, ld, kd) = res["ids"], res["dense"]
+        err = float((ld - li).abs().max() / li.std())
+        assert err <= 1e-2, (tag, err)
+        assert float((ki.float() - kd.float()).abs().max()) <= 2.0 ** -5 * max(1.0, float(ki.float().abs().max())), tag
+        top = torch.topk(li, 2, dim=-1).values
+        decided = ((top[:, 0] - top[:, 1]) >= 2e-2 * li.std(dim=-1)).cpu().numpy()
+        assert np.array_equal(td[decided], ti[decided]), tag
+    print("o projection by riders / by appended rows:", ride_seen, flush=True)
+    assert ride_seen[True] >= 10 and ride_seen[False] >= 10, ride_seen
+
+
 def test_front_end_on_random_request_mixes():
     """Up to three adapter types (one scaling) and requests without adapter, per-request length limits and an
     optional EOS id: the front end returns the same token ids whether decode batches take the native / recorded
