@@ -253,33 +253,35 @@ __device__ __forceinline__ void amax_merge(float& v, int& i, float ov, int oi) {
   }
 }
 
-__global__ __launch_bounds__(ROW_THREADS) void argmax_kernel(int32_t* __restrict__ ids, const float* __restrict__ logits, int V) {
-  __shared__ float lv[ROW_THREADS / WAVE];
-  __shared__ int li[ROW_THREADS / WAVE];
+constexpr int AMAX_THREADS = 1024;   // one row per workgroup: many threads, few requests each
+__global__ __launch_bounds__(AMAX_THREADS) void argmax_kernel(int32_t* __restrict__ ids, const float* __restrict__ logits, int V) {
+  __shared__ float lv[AMAX_THREADS / WAVE];
+  __shared__ int li[AMAX_THREADS / WAVE];
   const int row = blockIdx.x;
   const float* p = logits + (size_t)row * V;
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  // 16-byte loads, four in flight per thread; elements are merged in increasing index order within a thread and the
-  // merge keeps the lower index on ties, so the result is the first maximum whatever the traversal order
+  // 16-byte loads, eight in flight per thread (a vocabulary of 32000 is one round of requests); elements are merged in
+  // increasing index order within a thread and the merge keeps the lower index on ties, so the result is the first
+  // maximum whatever the traversal order
   const int V4 = ((size_t)p % 16 == 0) ? V / 4 : 0;
-  for (int c0 = threadIdx.x; c0 < V4; c0 += ROW_THREADS * 4) {
-    f32x4 q[4];
+  for (int c0 = threadIdx.x; c0 < V4; c0 += AMAX_THREADS * 8) {
+    f32x4 q[8];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int c = c0 + u * ROW_THREADS;
+    for (int u = 0; u < 8; ++u) {
+      const int c = c0 + u * AMAX_THREADS;
       q[u] = c < V4 ? *reinterpret_cast<const f32x4*>(p + 4 * (size_t)c) : f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int c = c0 + u * ROW_THREADS;
+    for (int u = 0; u < 8; ++u) {
+      const int c = c0 + u * AMAX_THREADS;
       if (c < V4) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) amax_merge(bv, bi, q[u][e], 4 * c + e);
       }
     }
   }
-  for (int c = 4 * V4 + threadIdx.x; c < V; c += ROW_THREADS) amax_merge(bv, bi, p[c], c);
+  for (int c = 4 * V4 + threadIdx.x; c < V; c += AMAX_THREADS) amax_merge(bv, bi, p[c], c);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     const float ov = __shfl_xor(bv, o, WAVE);
@@ -293,7 +295,7 @@ __global__ __launch_bounds__(ROW_THREADS) void argmax_kernel(int32_t* __restrict
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int w = 1; w < ROW_THREADS / WAVE; ++w) amax_merge(bv, bi, lv[w], li[w]);
+    for (int w = 1; w < AMAX_THREADS / WAVE; ++w) amax_merge(bv, bi, lv[w], li[w]);
     ids[row] = bi == 0x7fffffff ? 0 : bi;
   }
 }
@@ -520,6 +522,6 @@ extern "C" int mlora_argmax(int32_t* ids, const float* logits, int B, int V, voi
   MLORA_CHECK(ids && logits, MLORA_ERR_INVALID, "argmax: null pointer");
   MLORA_CHECK(B >= 0 && V > 0, MLORA_ERR_INVALID, "argmax: bad shape B=%d V=%d", B, V);
   if (B == 0) return MLORA_OK;
-  hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(ROW_THREADS), 0, (hipStream_t)stream, ids, logits, V);
+  hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(AMAX_THREADS), 0, (hipStream_t)stream, ids, logits, V);
   return mlora_launch_status("argmax");
 }
