@@ -403,7 +403,7 @@ int mlora_rope_attn_decode(void* out, int out_layout, const void* qkv, void* k_c
 /* The same launch, which in addition takes the o projection's LoRA shrink off the attention output where it is
  * produced: o_vpart[h][b][j] = sum over the D dims of head h of f16(out[b, h, d]) * o_A[id_b][j][h D + d]  (fp32,
  * [Hq][B][r]; o_A [n_ad, r, Hq * D]; rows of tokens without adapter are left untouched), one share per query head,
- * for a consumer that adds the Hq shares in head order (mlora_gemv_frag_acc_ksplit_delta).  out and the caches are
+ * for a consumer that adds the Hq shares in a fixed order (mlora_gemv_frag_acc_ksplit_delta).  out and the caches are
  * those of mlora_rope_attn_decode bit for bit.  tok_adapter, r and n_ad serve both the q/k/v expand (if v_part is
  * given) and the o shrink.  mlora_rope_attn_oshrink_ok says whether the launch for (B, Hq, Hkv, D) has room for
  * rank r (its Hq / Hkv * r * D / 8 items must fit one workgroup).  Replaces: the lora_A half of the o projection's
@@ -416,6 +416,20 @@ int mlora_rope_attn_decode_oshrink(void* out, int out_layout, const void* qkv, v
                                    int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
                                    const void* v_part, int v_dense, const void* const* Bmat, const int32_t* tok_adapter,
                                    float scaling, int K, int r, int n_ad, const void* o_A, void* o_vpart, void* stream);
+/* The decode attention without the RoPE / append part (mlora_paged_attn_decode: out bit for bit) that also writes the
+ * o projection's shrink in head shares, as mlora_rope_attn_decode_oshrink does (same o_A, o_vpart, tok_adapter, r, n_ad;
+ * mlora_rope_attn_oshrink_ok applies), and the expand of such shares as a launch of its own:
+ *   y[t, :] += scaling * B[id_t] . sum_h vpart[h][t]   for the tokens that name an adapter (y fp32 [T, N], B [n_ad, N, r];
+ *   mlora_lora_expand_shares_ok(N, r): N % 16 == 0, rank 8, 16, 32 or 64, N dividing over a token's workgroups).
+ * Together they are the o projection's adapter delta of a decode step of more than 64 sequences (mlora_decode_step takes
+ * them where both apply).  Replace: tvm/llama_auto_batcher/lora.py:16-24 for the o projection (compile_tvm.py:126-134). */
+int mlora_paged_attn_decode_oshrink(void* out, int out_layout, const void* qkv, const void* k_cache, const void* v_cache,
+                                    const int32_t* block_table, int max_blocks, const int32_t* seq_ids, const int32_t* ctx_len,
+                                    int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                                    const int32_t* tok_adapter, int r, int n_ad, const void* o_A, void* o_vpart, void* stream);
+int mlora_lora_expand_shares_ok(int N, int r);
+int mlora_lora_expand_shares(float* y, const float* vpart, int n_vpart, const void* B, const int32_t* tok_adapter, float scaling,
+                             int T, int N, int r, int n_ad, void* stream);
 int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v_part, int v_dense, const void* B,
                               const int32_t* tok_adapter, float scaling, const void* w, float eps,
                               int T, int H, int K, int r, int n_ad, void* stream);
@@ -443,7 +457,7 @@ int mlora_lora_expand_rmsnorm(void* y, int y_layout, float* resid, const void* v
  *                                are y2 plus columns H.. of the partials.
  *   mlora_gemv_frag_acc_ksplit_delta - the same accumulating K-split GEMV over the base weight alone, with the
  *                                projection's LoRA expand done by workgroups that ride at the front of the launch.  The
- *                                shrink results come as n_vpart shares, vpart [n_vpart][T][r] fp32 (added in share
+ *                                shrink results come as n_vpart shares, vpart [n_vpart][T][r] fp32 (added in a fixed
  *                                order; mlora_rope_attn_decode_oshrink writes one share per attention head):
  *                                delta[t, :] = scaling * B[id_t] . sum_h vpart[h][t] (zeros for a token without adapter)
  *                                goes to slot ks-1 of `part` ([ks][T][N] fp32: ks-1 slice partials, then the delta

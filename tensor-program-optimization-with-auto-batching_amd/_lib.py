@@ -62,6 +62,9 @@ SIGNATURES = {
     "mlora_gemv_delta_ride_ksplit": (_i, [_i, _i, _i, _i]),
     "mlora_gemv_frag_acc_ksplit_delta": (_i, [_p, _p, _i, _p, _p, _i, _i, _i, _p, _i, _p, _p, _f, _i, _i, _p]),
     "mlora_rope_attn_oshrink_ok": (_i, [_i, _i, _i, _i, _i]),
+    "mlora_paged_attn_decode_oshrink": (_i, [_p, _i, _p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i, _i, _p, _p, _p]),
+    "mlora_lora_expand_shares_ok": (_i, [_i, _i]),
+    "mlora_lora_expand_shares": (_i, [_p, _p, _i, _p, _p, _f, _i, _i, _i, _i, _p]),
     "mlora_rope_attn_decode_oshrink": (_i, [_p, _i, _p, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p, _p, _p]),
     "mlora_rmsnorm_ksplit": (_i, [_p, _i, _p, _p, _i, _i, _p, _f, _i, _i, _p, _i, _p, _p, _f, _i, _i, _i, _p]),
     "mlora_lora_expand_rmsnorm": (_i, [_p, _i, _p, _p, _i, _p, _p, _f, _p, _f, _i, _i, _i, _i, _i, _p]),

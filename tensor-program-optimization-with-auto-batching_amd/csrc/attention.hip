@@ -40,6 +40,26 @@ struct OShrinkHeads {
   int r, n_ad, T;
 };
 
+// thread (query head qh, rank entry j, 8-dim piece c) of the workgroup of kv head kh: its 16 bytes of A[id] ...
+template <int D>
+__device__ __forceinline__ f16x8 oshrink_piece(const OShrinkHeads& os, int id, int G, int kh, int Hq) {
+  constexpr int OPC = D / 8;
+  const int oc = threadIdx.x % OPC, oj = (threadIdx.x / OPC) % os.r, oq = threadIdx.x / (OPC * os.r);
+  return ld8(os.A + ((size_t)id * os.r + oj) * ((size_t)Hq * D) + (size_t)(kh * G + oq) * D + oc * 8);
+}
+
+// ... and its product with the head's output as stored (outs: the workgroup's G x D fp16 outputs in LDS, published by a
+// barrier), summed over the D / 8 pieces of the row, which sit in neighbouring lanes
+template <int D>
+__device__ __forceinline__ void oshrink_head_shares(const OShrinkHeads& os, f16x8 a8, const f16* __restrict__ outs, int G, int kh, int b) {
+  constexpr int OPC = D / 8;
+  const int oc = threadIdx.x % OPC, oj = (threadIdx.x / OPC) % os.r, oq = threadIdx.x / (OPC * os.r);
+  float sum = dot8(a8, *reinterpret_cast<const f16x8*>(&outs[oq * D + oc * 8]), 0.f);
+#pragma unroll
+  for (int o = 1; o < OPC; o <<= 1) sum += __shfl_xor(sum, o, WAVE);
+  if (oc == 0) os.vpart[((size_t)(kh * G + oq) * os.T + b) * os.r + oj] = sum;
+}
+
 // grid (T, Hq + 2 Hkv), 64 threads: thread i rotates the pair (i, i + D/2) of one head of one token
 __global__ __launch_bounds__(64) void rope_kv_append_kernel(f16* __restrict__ qkv, f16* __restrict__ k_cache,
                                                             f16* __restrict__ v_cache,
@@ -318,23 +338,31 @@ template <int D, int NW>   // NW waves per workgroup share the pages of one (seq
 __global__ __launch_bounds__(NW * WAVE, 4) void paged_attn_decode_kernel(
     f16* __restrict__ out, const f16* __restrict__ qkv, const f16* __restrict__ k_cache, const f16* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ seq_ids,
-    const int32_t* __restrict__ ctx_len, int Hq, int Hkv, int n_pages, int n_seq, float scale, int frag_tt) {
+    const int32_t* __restrict__ ctx_len, int Hq, int Hkv, int n_pages, int n_seq, float scale, int frag_tt, OShrinkHeads os) {
   constexpr int NKB = D / 32;   // k-blocks of the QK^T product
   constexpr int NDB = D / 16;   // dim blocks of the output
   __shared__ float sm[NW][16], sl[NW][16];
+  __shared__ __align__(16) f16 outs[16 * D];   // the workgroup's outputs as stored, for the o shrink
   extern __shared__ float sacc[];   // [NW][G][D]
 
   // arguments, then the sequence's scalars, then its first page ids: three grouped rounds of scalar loads (see
   // rope_attn_decode_kernel)
   asm volatile("" ::"s"(out), "s"(qkv), "s"(k_cache), "s"(v_cache), "s"(block_table), "s"(max_blocks), "s"(seq_ids), "s"(ctx_len));
   asm volatile("" ::"s"(Hq), "s"(Hkv), "s"(n_pages), "s"(n_seq), "s"(scale), "s"(frag_tt));
+  asm volatile("" ::"s"(os.A), "s"(os.vpart), "s"(os.ids), "s"(os.r), "s"(os.n_ad), "s"(os.T));
   const int b = blockIdx.y, kh = blockIdx.x;
   const int G = Hq / Hkv;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
   const int seq = seq_ids[b];
   int ctx = ctx_len[b];
-  asm volatile("" ::"s"(seq), "s"(ctx));
+  const int oid_raw = (os.A != nullptr ? os.ids : seq_ids)[b];
+  asm volatile("" ::"s"(seq), "s"(ctx), "s"(oid_raw));
+  // the o shrink (see OShrinkHeads): the thread's 16 bytes of A[id] are requested now and wait in registers for the epilogue
+  const bool o_on = os.A != nullptr && oid_raw >= 0 && oid_raw < os.n_ad;        // uniform
+  const bool o_mine = o_on && (int)threadIdx.x < G * os.r * (D / 8);
+  f16x8 oa = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  if (o_mine) oa = oshrink_piece<D>(os, oid_raw, G, kh, Hq);
   if (seq < 0 || seq >= n_seq) ctx = 0;
   if (ctx > max_blocks * PAGE) ctx = max_blocks * PAGE;
   const int npages = (ctx + PAGE - 1) / PAGE;
@@ -430,7 +458,13 @@ __global__ __launch_bounds__(NW * WAVE, 4) void paged_attn_decode_kernel(
     }
     const int h = kh * G + qh;
     const size_t oo = frag_tt ? frag_offset(b, h * D + d, frag_tt) : ((size_t)b * Hq + h) * D + d;
-    out[oo] = (f16)(L > 0.f ? o / L : 0.f);
+    const f16 of = (f16)(L > 0.f ? o / L : 0.f);
+    out[oo] = of;
+    if (o_on) outs[qh * D + d] = of;
+  }
+  if (o_on) {                                                // uniform
+    __syncthreads();
+    if (o_mine) oshrink_head_shares<D>(os, oa, outs, G, kh, b);
   }
 }
 
@@ -596,10 +630,7 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
   constexpr int OPC = D / 8;
   const bool o_mine = o_on && (int)threadIdx.x < G * os.r * OPC;
   f16x8 oa = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-  if (o_mine) {
-    const int oc = threadIdx.x % OPC, oj = (threadIdx.x / OPC) % os.r, oq = threadIdx.x / (OPC * os.r);
-    oa = ld8(os.A + ((size_t)oid_raw * os.r + oj) * ((size_t)Hq * D) + (size_t)(kh * G + oq) * D + oc * 8);
-  }
+  if (o_mine) oa = oshrink_piece<D>(os, oid_raw, G, kh, Hq);
   if (adapted) {
     if (lx.src.kc == 0 && lx.src.kq > 1) {
       // dense shrink results in kq blocks of K-range partials: one thread per (block, entry) fetches, then the blocks
@@ -741,13 +772,7 @@ __global__ __launch_bounds__(NW * WAVE, 4) void rope_attn_decode_kernel(
   }
   if (o_on) {                                                // uniform
     __syncthreads();
-    if (o_mine) {
-      const int oc = threadIdx.x % OPC, oj = (threadIdx.x / OPC) % os.r, oq = threadIdx.x / (OPC * os.r);
-      float sum = dot8(oslice[threadIdx.x], *reinterpret_cast<const f16x8*>(&qs[oq * D + oc * 8]), 0.f);
-#pragma unroll
-      for (int o = 1; o < OPC; o <<= 1) sum += __shfl_xor(sum, o, WAVE);      // the D / 8 pieces of a row sit in neighbouring lanes
-      if (oc == 0) os.vpart[((size_t)(kh * G + oq) * os.T + b) * os.r + oj] = sum;
-    }
+    if (o_mine) oshrink_head_shares<D>(os, oslice[threadIdx.x], qs, G, kh, b);
   }
 }
 
@@ -1176,10 +1201,10 @@ extern "C" int mlora_rope_kv_append_lora(void* qkv, void* k_cache, void* v_cache
                              rope_cos, rope_sin, max_pos, T, Hq, Hkv, D, n_pages, n_seq, lx, stream);
 }
 
-extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qkv, const void* k_cache, const void* v_cache,
-                                       const int32_t* block_table, int max_blocks, const int32_t* seq_ids,
-                                       const int32_t* ctx_len, int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
-                                       void* stream) {
+static int paged_attn_decode_impl(void* out, int out_layout, const void* qkv, const void* k_cache, const void* v_cache,
+                                  const int32_t* block_table, int max_blocks, const int32_t* seq_ids,
+                                  const int32_t* ctx_len, int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                                  const int32_t* tok_adapter, int r, int n_ad, const void* o_A, void* o_vpart, void* stream) {
   if (int e = check_attn("paged_attn_decode", Hq, Hkv, D, n_pages, n_seq, max_blocks)) return e;
   MLORA_CHECK(out && qkv && k_cache && v_cache && block_table && seq_ids && ctx_len, MLORA_ERR_INVALID, "paged_attn_decode: null pointer");
   MLORA_CHECK(B >= 0 && B <= 65535, MLORA_ERR_INVALID, "paged_attn_decode: bad B=%d (0..65535)", B);
@@ -1190,12 +1215,22 @@ extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qk
   hipStream_t s = (hipStream_t)stream;
   const int G = Hq / Hkv;
   MLORA_CHECK(G <= 16, MLORA_ERR_UNSUPPORTED, "paged_attn_decode: more than 16 query heads per kv head (%d)", G);
+  OShrinkHeads os = {};
+  if (o_A != nullptr) {
+    MLORA_CHECK(o_vpart && tok_adapter && n_ad > 0, MLORA_ERR_INVALID, "paged_attn_decode: null o-shrink argument");
+    MLORA_CHECK(mlora_rope_attn_oshrink_ok(B, Hq, Hkv, D, r), MLORA_ERR_UNSUPPORTED,
+                "paged_attn_decode: the o shrink of rank %d does not fit the workgroup of this launch (B=%d Hq=%d Hkv=%d D=%d)", r, B, Hq, Hkv, D);
+    os.A = (const f16*)o_A;
+    os.vpart = (float*)o_vpart;
+    os.ids = tok_adapter;
+    os.r = r; os.n_ad = n_ad; os.T = B;
+  }
   const int nw = attn_waves(B, Hkv, G, D);
   const size_t lds = (size_t)nw * G * D * sizeof(float);
 #define MLORA_ATTN(DD, NWV)                                                                                                   \
   hipLaunchKernelGGL((paged_attn_decode_kernel<DD, NWV>), dim3(Hkv, B), dim3(NWV * WAVE), lds, s, (f16*)out, (const f16*)qkv, \
                      (const f16*)k_cache, (const f16*)v_cache, block_table, max_blocks, seq_ids, ctx_len, Hq, Hkv, n_pages,   \
-                     n_seq, scale, frag_tt)
+                     n_seq, scale, frag_tt, os)
   if (D == 128) {
     if (nw == 16) MLORA_ATTN(128, 16);
     else if (nw == 8) MLORA_ATTN(128, 8);
@@ -1207,6 +1242,24 @@ extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qk
   }
 #undef MLORA_ATTN
   return mlora_launch_status("paged_attn_decode");
+}
+
+extern "C" int mlora_paged_attn_decode(void* out, int out_layout, const void* qkv, const void* k_cache, const void* v_cache,
+                                       const int32_t* block_table, int max_blocks, const int32_t* seq_ids,
+                                       const int32_t* ctx_len, int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                                       void* stream) {
+  return paged_attn_decode_impl(out, out_layout, qkv, k_cache, v_cache, block_table, max_blocks, seq_ids, ctx_len, B, Hq, Hkv, D, n_pages,
+                                n_seq, nullptr, 0, 0, nullptr, nullptr, stream);
+}
+
+extern "C" int mlora_paged_attn_decode_oshrink(void* out, int out_layout, const void* qkv, const void* k_cache, const void* v_cache,
+                                               const int32_t* block_table, int max_blocks, const int32_t* seq_ids,
+                                               const int32_t* ctx_len, int B, int Hq, int Hkv, int D, int n_pages, int n_seq,
+                                               const int32_t* tok_adapter, int r, int n_ad, const void* o_A, void* o_vpart,
+                                               void* stream) {
+  MLORA_CHECK(o_A && o_vpart, MLORA_ERR_INVALID, "paged_attn_decode_oshrink: null o-shrink argument");
+  return paged_attn_decode_impl(out, out_layout, qkv, k_cache, v_cache, block_table, max_blocks, seq_ids, ctx_len, B, Hq, Hkv, D, n_pages,
+                                n_seq, tok_adapter, r, n_ad, o_A, o_vpart, stream);
 }
 
 // the o shrink's items (query heads of a kv head x rank entries x 8-dim pieces) must fit the workgroup the launch uses

@@ -67,6 +67,11 @@ int decode_step_wide(const mlora_decode_plan* p, void* stream) {
                                   0, 0, stream);
     return mlora_rmsnorm(p->xn, MLORA_FRAG, p->resid, MLORA_F32, w, p->eps, T, H, stream);
   };
+  // An adapted o projection: the attention launch leaves the shrink as one share per head, and a launch of expand
+  // workgroups adds the deltas to the residual behind the base linear - instead of a shrink pass over the attention
+  // output and an expand pass (where the shapes allow it; the per-operator Python path takes the same decision).
+  const bool o_shares = lora && mlora_rope_attn_oshrink_ok(T, Hq, Hkv, D, r) && mlora_lora_expand_shares_ok(H, r) &&
+                        p->lora_ws_bytes >= (size_t)Hq * T * r * sizeof(float);
   int pending_ks = 1;
   STEP(mlora_embed(p->resid, MLORA_F32, p->embed, p->tokens, T, H, p->vocab, stream));
   for (int l = 0; l < p->n_layers; ++l) {
@@ -80,12 +85,20 @@ int decode_step_wide(const mlora_decode_plan* p, void* stream) {
     }
     STEP(mlora_rope_kv_append(qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->pos, p->rope_cos, p->rope_sin,
                               p->max_pos, T, Hq, Hkv, D, p->n_pages, p->n_seq, stream));
-    STEP(mlora_paged_attn_decode(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->ctx, T, Hq,
-                                 Hkv, D, p->n_pages, p->n_seq, stream));
+    const bool o_by_shares = o_shares && L.lora[MLORA_O].A;
+    if (o_by_shares)
+      STEP(mlora_paged_attn_decode_oshrink(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->ctx,
+                                           T, Hq, Hkv, D, p->n_pages, p->n_seq, p->tok_adapter, r, n_ad, L.lora[MLORA_O].A, p->lora_ws,
+                                           stream));
+    else
+      STEP(mlora_paged_attn_decode(p->attn, MLORA_FRAG, qkv, L.k_cache, L.v_cache, p->block_table, p->max_blocks, p->rows, p->ctx, T, Hq,
+                                   Hkv, D, p->n_pages, p->n_seq, stream));
     const int ks_o = ksplit_of(q_sz);
     STEP(mlora_gemv_frag_acc_ksplit(p->resid, nullptr, p->ksplit_ws, ks_o, p->attn, L.o_p, T, q_sz, H, 0, nullptr, nullptr, 0, nullptr, 0, 0,
                                     stream));
-    {
+    if (o_by_shares) {
+      STEP(mlora_lora_expand_shares(p->resid, (const float*)p->lora_ws, Hq, L.lora[MLORA_O].B, p->tok_adapter, sc, T, H, r, n_ad, stream));
+    } else {
       const mlora_lora_proj* lp[1] = {&L.lora[MLORA_O]};
       const int32_t col[1] = {0}, ncol[1] = {H};
       STEP(deltas(p->resid, MLORA_F32, H, p->attn, q_sz, lp, col, ncol, 1));

@@ -31,7 +31,7 @@ __device__ __forceinline__ int udiv_le4(int v, int d) {
 
 // The expand of a LoRA delta by workgroups that ride at the front of an accumulating GEMV launch.  The shrink results
 // come as `n_vpart` shares per (token, rank entry) - vpart [n_vpart, T, r] fp32, e.g. one share per attention head from
-// the kernel that produced the launch's token block - which rider (t, part) adds in share order before it writes
+// the kernel that produced the launch's token block - which rider (t, part) adds in a fixed order before it writes
 // delta[t][c] = scaling * B[id_t][c] . v for its share of the N columns into `out` [T, N] fp32 (zeros for a token
 // without adapter): a row block that the reader of y adds like a K-slice partial.  The GEMV's own rows stay the base
 // weight (no appended adapter rows), and the norm that follows has no table to stream - its B rows arrive here, a few
@@ -43,10 +43,13 @@ struct LoraDeltaRide {
   float* out;           // [T, N]
   float scaling;
   int n_vpart, T, N, r, n_ad, per_token;
+  int accumulate;       // out[t, :] += delta for the tokens that have an adapter, others untouched (the stand-alone launch)
 };
 
 constexpr int RIDE_BQ = 2;     // 16-byte chunks of B per rider thread: a rider is short, and there are many of them
+constexpr int SOLO_BQ = 8;     // ... and per thread of the stand-alone launch: one round of fewer, larger workgroups
 
+template <int BQ>
 __device__ __forceinline__ void lora_delta_ride(const LoraDeltaRide& d, int unit, float* __restrict__ lds) {
   constexpr int NTH = GEMV_WAVES * WAVE;
   const int tid = threadIdx.x;
@@ -55,46 +58,65 @@ __device__ __forceinline__ void lora_delta_ride(const LoraDeltaRide& d, int unit
   float* __restrict__ out = d.out + (size_t)t * d.N + c0;
   const int id = d.ids[t];                                   // uniform
   if (id < 0 || id >= d.n_ad) {
-    for (int c = tid * 4; c < ncol; c += NTH * 4) *reinterpret_cast<f32x4*>(out + c) = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (!d.accumulate)
+      for (int c = tid * 4; c < ncol; c += NTH * 4) *reinterpret_cast<f32x4*>(out + c) = f32x4{0.f, 0.f, 0.f, 0.f};
     return;
   }
   const int r = d.r, lpr = r >> 3;                           // 16-byte chunks per row of B
-  const int nq = ncol * lpr;                                 // chunks of this rider's rows of B: at most RIDE_BQ per thread
+  const int nq = ncol * lpr;                                 // chunks of this rider's rows of B: at most BQ per thread
   // one round of requests: the rider's rows of B (uniform base + 32-bit lane offset) and the shares of v
-  f16x8 bv[RIDE_BQ];
+  f16x8 bv[BQ];
   const f16* __restrict__ Bp = d.B + ((size_t)id * d.N + c0) * r;
 #pragma unroll
-  for (int u = 0; u < RIDE_BQ; ++u) {
+  for (int u = 0; u < BQ; ++u) {
     const int q = u * NTH + tid;
     bv[u] = ld8(Bp + (unsigned)((q < nq ? q : 0) * 8));
   }
-  float* __restrict__ sh = lds;                              // [n_vpart][r] shares, then [r] their sum
-  float* __restrict__ lv = lds + d.n_vpart * r;
+  // the row's old values, where the deltas are added in place: requested with everything else
+  const int csub = tid % lpr;                                // a thread's chunks all cover ranks 8 csub .. (512 % lpr == 0)
+  float yold[BQ];
+#pragma unroll
+  for (int u = 0; u < BQ; ++u) {
+    const int q = u * NTH + tid;
+    yold[u] = d.accumulate && csub == 0 && q < nq ? out[q / lpr] : 0.f;
+  }
+  // v[j] = scaling * sum of the shares: thread e = h r + j takes the shares h, h + 512 / r, ... of entry j (512 % r == 0),
+  // the lanes of a wave that hold the same j add up by shuffles, the eight waves' sums meet in LDS - a fixed order
+  float* __restrict__ wsum = lds;                            // [8][r], then v [r]
+  float* __restrict__ lv = lds + GEMV_WAVES * r;
+  float a = 0.f;
   for (int e = tid; e < d.n_vpart * r; e += NTH) {
     const int h = e / r, jj = e - h * r;
-    sh[e] = d.vpart[((size_t)h * d.T + t) * r + jj];
+    a += d.vpart[((size_t)h * d.T + t) * r + jj];
   }
+  for (int o = r; o < WAVE; o <<= 1) a += __shfl_xor(a, o, WAVE);
+  if ((tid & (WAVE - 1)) < r) wsum[(tid >> 6) * r + (tid & (WAVE - 1))] = a;
   __syncthreads();
   if (tid < r) {
-    float a = 0.f;
-    for (int h = 0; h < d.n_vpart; ++h) a += sh[h * r + tid];      // share order
-    lv[tid] = a * d.scaling;
+    float sum = wsum[tid];
+#pragma unroll
+    for (int w = 1; w < GEMV_WAVES; ++w) sum += wsum[w * r + tid];
+    lv[tid] = sum * d.scaling;
   }
   __syncthreads();
-  // a thread's chunks all cover the same 8 ranks (the thread count is a multiple of the chunks per row)
-  const int csub = tid % lpr;
   float lvr[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) lvr[e] = lv[csub * 8 + e];
 #pragma unroll
-  for (int u = 0; u < RIDE_BQ; ++u) {
+  for (int u = 0; u < BQ; ++u) {
     const int q = u * NTH + tid;
     float sum = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) sum = fmaf((float)bv[u][e], lvr[e], sum);
     for (int o = 1; o < lpr; o <<= 1) sum += __shfl_xor(sum, o, WAVE);
-    if (csub == 0 && q < nq) out[q / lpr] = sum;
+    if (csub == 0 && q < nq) out[q / lpr] = yold[u] + sum;
   }
+}
+
+// the riders as a launch of their own (token blocks beyond what the decode GEMV serves): y[t, :] += delta
+__global__ __launch_bounds__(GEMV_WAVES* WAVE) void lora_expand_shares_kernel(LoraDeltaRide d) {
+  __shared__ float lds[(GEMV_WAVES + 1) * 64];
+  lora_delta_ride<SOLO_BQ>(d, blockIdx.x, lds);
 }
 
 // With SHRINK the first `shrink_blocks` workgroups of the launch do LoRA shrink units (one per wave) on the same
@@ -118,7 +140,7 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE, (NT * TT > 8 ? 2 : 4)) void gemv_
   int bid = blockIdx.x;
   if constexpr (RIDE) {
     if (bid < ride_blocks) {                       // uniform
-      lora_delta_ride(dr, bid, reinterpret_cast<float*>(&red[0][0][0]));
+      lora_delta_ride<RIDE_BQ>(dr, bid, reinterpret_cast<float*>(&red[0][0][0]));
       return;
     }
     bid -= ride_blocks;
@@ -732,8 +754,7 @@ extern "C" int mlora_gemv_frag_acc_ksplit_delta(float* y, float* part, int ks, c
   MLORA_CHECK(per_token > 0 && ks == mlora_gemv_delta_ride_ksplit(T, K, N, r) && (K / KSTEP) / ks >= 8, MLORA_ERR_UNSUPPORTED,
               "gemv_frag_acc_ksplit_delta: T=%d K=%d N=%d r=%d ks=%d not served (mlora_gemv_delta_ride_ksplit gives %d)", T, K, N, r, ks,
               mlora_gemv_delta_ride_ksplit(T, K, N, r));
-  MLORA_CHECK(n_vpart >= 1 && (size_t)(n_vpart + 1) * r * sizeof(float) <= 32 * 1024, MLORA_ERR_UNSUPPORTED,
-              "gemv_frag_acc_ksplit_delta: %d shares of rank %d do not fit the rider's LDS", n_vpart, r);
+  MLORA_CHECK(n_vpart >= 1, MLORA_ERR_INVALID, "gemv_frag_acc_ksplit_delta: no shares");
   LoraDeltaRide dr;
   dr.vpart = vpart;
   dr.B = (const f16*)B;
@@ -742,8 +763,37 @@ extern "C" int mlora_gemv_frag_acc_ksplit_delta(float* y, float* part, int ks, c
   dr.scaling = scaling;
   dr.n_vpart = n_vpart; dr.T = T; dr.N = N; dr.r = r; dr.n_ad = n_ad;
   dr.per_token = per_token;
+  dr.accumulate = 0;
   return gemv_dispatch<true, true, false>(y, MLORA_F32, MLORA_ACCUMULATE, xf, K, Wp, T, K, N, stream, LoraShrinkBatch(), N, nullptr, ks,
                                           part, dr, T * per_token);
+}
+
+extern "C" int mlora_lora_expand_shares_ok(int N, int r) {
+  if (N <= 0 || N % 16 || (r != 8 && r != 16 && r != 32 && r != 64)) return 0;
+  const int per_token = ceil_div(ceil_div(N * (r / 8), GEMV_WAVES * WAVE), SOLO_BQ);
+  return N % per_token == 0 && (N / per_token) % 4 == 0 ? 1 : 0;
+}
+
+extern "C" int mlora_lora_expand_shares(float* y, const float* vpart, int n_vpart, const void* B, const int32_t* tok_adapter, float scaling,
+                                        int T, int N, int r, int n_ad, void* stream) {
+  MLORA_CHECK(y && vpart && B && tok_adapter && n_ad > 0, MLORA_ERR_INVALID, "lora_expand_shares: null pointer or no adapters");
+  MLORA_CHECK(T >= 0 && mlora_lora_expand_shares_ok(N, r), MLORA_ERR_UNSUPPORTED,
+              "lora_expand_shares: need N %% 16 == 0, rank 8, 16, 32 or 64 and N dividing over the workgroups of a token (N=%d r=%d)", N, r);
+  MLORA_CHECK(n_vpart >= 1, MLORA_ERR_INVALID, "lora_expand_shares: no shares");
+  const int per_token = ceil_div(ceil_div(N * (r / 8), GEMV_WAVES * WAVE), SOLO_BQ);
+  MLORA_CHECK((long)T * per_token <= 0x7fffffffL, MLORA_ERR_UNSUPPORTED, "lora_expand_shares: T=%d is too many tokens", T);
+  if (T == 0) return MLORA_OK;
+  LoraDeltaRide dr;
+  dr.vpart = vpart;
+  dr.B = (const f16*)B;
+  dr.ids = tok_adapter;
+  dr.out = y;
+  dr.scaling = scaling;
+  dr.n_vpart = n_vpart; dr.T = T; dr.N = N; dr.r = r; dr.n_ad = n_ad;
+  dr.per_token = per_token;
+  dr.accumulate = 1;
+  hipLaunchKernelGGL(lora_expand_shares_kernel, dim3(T * per_token), dim3(GEMV_WAVES * WAVE), 0, (hipStream_t)stream, dr);
+  return mlora_launch_status("lora_expand_shares");
 }
 
 extern "C" int mlora_gemv_frag_silu(void* act, const void* xf, const void* Wil_p, int T, int K, int I, void* stream) {

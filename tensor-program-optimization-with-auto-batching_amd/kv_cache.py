@@ -107,10 +107,11 @@ class PagedKVCache:
             ctx = None
         self._cur = (list(seq_ids), list(append_lens), decode, tok_seq, tok_pos, ctx)
 
-    def attention_with_fused_qkv(self, layer, qkv, n_q_heads, out=None, frag=False):
+    def attention_with_fused_qkv(self, layer, qkv, n_q_heads, out=None, frag=False, o_shrink=None):
         """qkv [T, Hq + 2 Hkv, D] (or [T, (Hq + 2 Hkv) * D]) fp16, token-major in begin_forward order.
         Rotates q in place, appends rotated k and v, attends causally; returns [T, Hq * D] fp16
-        (frag=True: as a FragActivation ready for the o_proj product)."""
+        (frag=True: as a FragActivation ready for the o_proj product).  o_shrink (a decode step only): see
+        ops.paged_attn_decode - the call then returns (attention output, head shares of the o projection's shrink)."""
         if self._cur is None:
             raise RuntimeError("attention_with_fused_qkv outside begin_forward/end_forward")
         _, append_lens, decode, tok_seq, tok_pos, ctx = self._cur
@@ -120,7 +121,9 @@ class PagedKVCache:
                            self.rope_cos, self.rope_sin, n_q_heads, self.Hkv, self.D)
         if decode:
             return ops.paged_attn_decode(qkv, self.k[layer], self.v[layer], self.block_table, tok_seq, ctx,
-                                         n_q_heads, self.Hkv, self.D, out=out, frag=frag)
+                                         n_q_heads, self.Hkv, self.D, out=out, frag=frag, o_shrink=o_shrink)
+        if o_shrink is not None:
+            raise ValueError("attention_with_fused_qkv: o_shrink is for decode steps")
         return ops.paged_attn_prefill(qkv, self.k[layer], self.v[layer], self.block_table, tok_seq, tok_pos,
                                       n_q_heads, self.Hkv, self.D, out=out, frag=frag)
 

@@ -334,6 +334,12 @@ class LlamaForCausalLM:
             if lt.r in (32, 64):
                 blk, rest = ops.lora_block_adapters(ids, lt.n_adapters)
                 fuse = (lt, ids, blk, {tid: rest} if bool((rest >= 0).any()) else None)     # one read-back per pass
+        o_shares = None
+        if tok_adapter and "multi" not in tok_adapter and len(tok_adapter) == 1 and is_decode and T > 64 and frag:
+            (tid, ids), = tok_adapter.items()
+            lt = self.lora_types[tid]
+            if ops.o_shrink_served(T, s.num_attention_heads, s.num_key_value_heads, s.head_dim, H, lt.r):
+                o_shares = (lt, ids)
         parts = None
         for l, L in enumerate(self.layers):
             xn = ops.rmsnorm(resid, L["ln1"], s.rms_norm_eps, frag=frag, parts=parts)
@@ -343,13 +349,24 @@ class LlamaForCausalLM:
                 qkv = ops.linear(xn, L["qkv"])
                 if tok_adapter:
                     self._lora_group(qkv, xn, l, qkv_projs, tok_adapter)
-            attn = kv.attention_with_fused_qkv(l, qkv, s.num_attention_heads, frag=frag)
-            if fuse and self._fused_linear(fuse, attn, L["o"], l, (("o_proj", 0, H),), resid=resid) is not None:
-                parts = None
-            else:
+            # a decode step of more than 64 sequences of one adapter type: the o projection's shrink comes off the
+            # attention launch in head shares and a launch of expand workgroups adds the deltas behind the base linear
+            # (what the native step does for such a batch; same kernels, same order)
+            o_sh = None
+            if o_shares is not None and (l, "o_proj") in o_shares[0].tables:
+                o_sh = o_shares[0].tables[(l, "o_proj")]
+            if o_sh is not None:
+                attn, vpart = kv.attention_with_fused_qkv(l, qkv, s.num_attention_heads, frag=frag, o_shrink=(o_sh[0], o_shares[1]))
                 parts = self._linear_acc(attn, L["o"], resid, ks_ws, self._riding_rows(l, "o_proj", lora_tids, T, q_sz))
-                if tok_adapter:
-                    self._lora(resid, attn, l, "o_proj", tok_adapter)
+                ops.lora_expand_shares(resid, vpart, o_sh[1], o_shares[1], o_shares[0].scaling)
+            else:
+                attn = kv.attention_with_fused_qkv(l, qkv, s.num_attention_heads, frag=frag)
+                if fuse and self._fused_linear(fuse, attn, L["o"], l, (("o_proj", 0, H),), resid=resid) is not None:
+                    parts = None
+                else:
+                    parts = self._linear_acc(attn, L["o"], resid, ks_ws, self._riding_rows(l, "o_proj", lora_tids, T, q_sz))
+                    if tok_adapter:
+                        self._lora(resid, attn, l, "o_proj", tok_adapter)
             xn = ops.rmsnorm(resid, L["ln2"], s.rms_norm_eps, frag=frag, parts=parts)
             if dec_frag and I % 32 == 0 and not (tok_adapter and self._targets(l, "gate_proj", "up_proj")):
                 # decode step without an adapter on gate / up: the SiLU product is the epilogue of the GEMV (same bits)

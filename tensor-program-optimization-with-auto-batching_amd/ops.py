@@ -566,10 +566,41 @@ def rope_kv_append(qkv, k_cache, v_cache, block_table, tok_seq, tok_pos, rope_co
                                      max_pos, T, Hq, Hkv, D, n_pages, n_seq, _stream()))
 
 
-def paged_attn_decode(qkv, k_cache, v_cache, block_table, seq_ids, ctx_len, Hq, Hkv, D, out=None, frag=False):
+def o_shrink_served(B: int, Hq: int, Hkv: int, D: int, N: int, r: int) -> bool:
+    """Whether a decode step of B sequences can take the o projection's adapter delta as head shares off the attention
+    launch plus a launch of expand workgroups (the rule the native step applies for more than 64 sequences)."""
+    return bool(lib().mlora_rope_attn_oshrink_ok(B, Hq, Hkv, D, r)) and bool(lib().mlora_lora_expand_shares_ok(N, r))
+
+
+def lora_expand_shares(y, vpart, B, tok_adapter, scaling: float):
+    """y [T, N] fp32 += scaling * B[id] @ sum_h vpart[h, t] for the tokens that name an adapter (vpart [shares, T, r] fp32)."""
+    T, N = y.shape
+    n_ad, N2, r = B.shape
+    if N2 != N or y.dtype != torch.float32 or vpart.dim() != 3 or tuple(vpart.shape[1:]) != (T, r):
+        raise ValueError(f"lora_expand_shares: y{tuple(y.shape)} vpart{tuple(vpart.shape)} B{tuple(B.shape)}")
+    check(lib().mlora_lora_expand_shares(_dev(y, torch.float32), _dev(vpart, torch.float32), vpart.shape[0], _dev(B, torch.float16, "B"),
+                                         _dev(tok_adapter, torch.int32), float(scaling), T, N, r, n_ad, _stream()))
+    return y
+
+
+def paged_attn_decode(qkv, k_cache, v_cache, block_table, seq_ids, ctx_len, Hq, Hkv, D, out=None, frag=False, o_shrink=None):
+    """o_shrink = (A [n_ad, r, Hq * D] f16, tok_adapter [B] int32): the launch also writes the o projection's shrink as one
+    share per query head and the call returns (out, vpart [Hq, B, r] fp32; rows of tokens without adapter are not written)."""
     B = qkv.shape[0]
     n_seq, max_blocks = block_table.shape
     out, optr, lay = _out_arg(out, B, Hq * D, frag, qkv.device)
+    if o_shrink is not None:
+        A, ids = o_shrink
+        n_ad, r, Kq = A.shape
+        if Kq != Hq * D or not lib().mlora_rope_attn_oshrink_ok(B, Hq, Hkv, D, r):
+            raise ValueError(f"paged_attn_decode: o shrink A{tuple(A.shape)} not served for B={B} Hq={Hq} Hkv={Hkv} D={D}")
+        vpart = torch.empty((Hq, B, r), dtype=torch.float32, device=qkv.device)
+        check(lib().mlora_paged_attn_decode_oshrink(optr, lay, _dev(qkv, torch.float16), _dev(k_cache, torch.float16),
+                                                    _dev(v_cache, torch.float16), _dev(block_table, torch.int32), max_blocks,
+                                                    _dev(seq_ids, torch.int32), _dev(ctx_len, torch.int32), B, Hq, Hkv, D,
+                                                    k_cache.shape[0], n_seq, _dev(ids, torch.int32), r, n_ad,
+                                                    _dev(A, torch.float16, "A"), vpart.data_ptr(), _stream()))
+        return out, vpart
     check(lib().mlora_paged_attn_decode(optr, lay, _dev(qkv, torch.float16), _dev(k_cache, torch.float16),
                                         _dev(v_cache, torch.float16), _dev(block_table, torch.int32), max_blocks,
                                         _dev(seq_ids, torch.int32), _dev(ctx_len, torch.int32), B, Hq, Hkv, D,

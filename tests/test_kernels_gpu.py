@@ -1211,6 +1211,62 @@ def test_gemv_ksplit_with_delta_riders(ops, synth, T, K, N, r, n_ad, shares):
     assert not torch.equal(racc[-1], r1[-1])
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,D,r,N", [(100, 8, 8, 128, 16, 1024), (20, 8, 2, 64, 8, 512), (300, 4, 4, 128, 32, 2048), (70, 16, 16, 64, 16, 4096)])
+def test_o_projection_delta_by_head_shares(ops, synth, B, Hq, Hkv, D, r, N):
+    """The o projection's adapter delta of a decode step of any size: the decode attention launch also writes the shrink
+    as one share per query head (same output bits as the plain launch; shares against the fp64 products of the stored
+    output with the head's columns of A), and the expand launch adds scaling * B[id] . (sum of shares) to an fp32 matrix
+    for the adapted tokens and leaves the others alone - together y + scaling * B[id] . (A[id] . attn)."""
+    kvm = load_pkg("kv_cache")
+    assert ops.o_shrink_served(B, Hq, Hkv, D, N, r)
+    n_ad = 6
+    rng = np.random.default_rng(B)
+    ctx = rng.integers(1, 90, size=B).astype(np.int32)
+    max_blocks = 6
+    n_pages = int(sum(-(-c // 16) for c in ctx)) + 3
+    perm = synth.permutation(17, f"os.pages.{B}", n_pages)
+    table = np.full((B, max_blocks), -1, dtype=np.int32)
+    o = 0
+    for b, c in enumerate(ctx):
+        nb = -(-int(c) // 16)
+        table[b, :nb] = perm[o:o + nb]
+        o += nb
+    table = torch.tensor(table, device=DEV)
+    kc = synth.normal(17, f"os.k{D}.{B}", (n_pages, Hkv, D // 32, 4, 16, 8), 1.0, torch.float16, DEV)
+    vc = synth.normal(17, f"os.v{D}.{B}", (n_pages, Hkv, D, 16), 1.0, torch.float16, DEV)
+    qkv = synth.normal(17, f"os.q{D}.{B}", (B, Hq + 2 * Hkv, D), 1.0, torch.float16, DEV)
+    seqs = torch.arange(B, dtype=torch.int32, device=DEV)
+    ctx_d = torch.from_numpy(ctx).to(DEV)
+    A = synth.normal(17, f"os.A{r}.{Hq * D}", (n_ad, r, Hq * D), 0.05, torch.float16, DEV)
+    Bm = synth.normal(17, f"os.B{r}.{N}", (n_ad, N, r), 0.3, torch.float16, DEV)
+    ids = (np.arange(B) % (n_ad + 1) - 1).astype(np.int32)                # -1, 0, 1, ...
+    ids_d = torch.from_numpy(ids).to(DEV)
+    want = ops.paged_attn_decode(qkv, kc, vc, table, seqs, ctx_d, Hq, Hkv, D)
+    got, vpart = ops.paged_attn_decode(qkv, kc, vc, table, seqs, ctx_d, Hq, Hkv, D, o_shrink=(A, ids_d))
+    assert torch.equal(got, want)
+    o64 = _np(got).astype(np.float64).reshape(B, Hq, D)
+    vp = _np(vpart)
+    v_full = np.zeros((B, r))
+    for b in range(B):
+        if ids[b] < 0:
+            continue
+        A64 = _np(A[ids[b]]).astype(np.float64).reshape(r, Hq, D)
+        ref = np.einsum("rhd,hd->hr", A64, o64[b])
+        assert np.abs(vp[:, b] - ref).max() <= 1e-5 + 1e-4 * np.abs(ref).max(), b
+        v_full[b] = ref.sum(0)
+    y0 = synth.normal(17, f"os.y.{B}.{N}", (B, N), 1.0, torch.float32, DEV)
+    y = y0.clone()
+    ops.lora_expand_shares(y, vpart, Bm, ids_d, 0.5)
+    torch.cuda.synchronize()
+    exp = _np(y0).astype(np.float64)
+    for b in range(B):
+        if ids[b] >= 0:
+            exp[b] += 0.5 * (_np(Bm[ids[b]]).astype(np.float64) @ v_full[b])
+    assert max_rel_err(_np(y), exp, floor=1e-2) <= 5e-4
+    none = np.nonzero(ids < 0)[0]
+    assert torch.equal(y[none], y0[none]) and not torch.equal(y[1], y0[1])
+
+
 @pytest.mark.parametrize("T,N_main,n_ad", [(32, 12288, 48), (12, 12288, 16), (32, 8192, 10), (20, 10240, 48)])
 def test_split_gemv_one_workgroup_per_unit(ops, synth, T, N_main, n_ad):
     """The q/k/v GEMV with appended adapter rows as one workgroup per compute unit: the main rows carry the bits of the
