@@ -319,14 +319,15 @@ class LlamaForCausalLM:
         # so does every larger pass: the operand loads of the matrix-core linears are then plain copies (norm, attention
         # and SiLU write the order the matrix cores read)
         frag = dec_frag or (T > 64 and H % 32 == 0 and q_sz % 32 == 0 and I % 32 == 0)
-        # a decode step splits K of the two narrow accumulating GEMVs; the RMSNorm that reads the residual next adds
-        # the partial results (the same kernels and slice counts as the native decode step)
-        ks_ws = self._ksplit_ws(T) if dec_frag or (frag and T <= 256) else None
+        is_decode = kv._cur is not None and bool(kv._cur[2])
+        # a decode step (of any number of sequences) and a short prefill split K of the two narrow accumulating linears;
+        # the RMSNorm that reads the residual next adds the partial results (the same kernels and slice counts as the
+        # native decode step)
+        ks_ws = self._ksplit_ws(T) if dec_frag or (frag and (T <= 256 or is_decode)) else None
         # a prefill-sized pass of one adapter type of rank 32 or 64: where a 256-token block agrees on one adapter its
         # deltas ride in the base GEMM as extra k-steps; `rest` names the tokens that still need the separate call
         # (a prefill pass only: the choice needs one read-back, which a decode step recorded into a graph cannot make)
         fuse = None
-        is_decode = kv._cur is not None and bool(kv._cur[2])
         if (tok_adapter and "multi" not in tok_adapter and frag and T > 64 and not is_decode
                 and not torch.cuda.is_current_stream_capturing() and ops.gemm_frag_preferred(T, H, H)):
             (tid, ids), = tok_adapter.items()

@@ -28,13 +28,24 @@ def _prefill(model, kv, prompts, ids, ops):
 def test_native_step_on_random_model_shapes():
     """Token ids and the whole K cache of `mlora_decode_step` (called per step and replayed from a graph, ids-based
     LoRA shrink) equal those of the per-operator path on 120 random configurations."""
+    _native_step_equals_per_operator_path(20240611, 120, [1, 2, 5, 16, 17, 32, 33, 48, 64], [2, 5, 19])
+
+
+def test_native_step_on_random_model_shapes_above_64_requests():
+    """The same on 60 random configurations of 65 to 520 requests: one launch per operator on fragment-ordered
+    activations (one, two or three 256-token blocks), K slices on o_proj and down_proj, grouped-query shapes, ranks 8 to
+    64, the o projection's delta from head shares of the attention launch where the shape is served that way."""
+    _native_step_equals_per_operator_path(20241126, 60, [65, 66, 80, 128, 129, 200, 256, 257, 300, 520], [2, 4])
+
+
+def _native_step_equals_per_operator_path(rng_seed, cases, batches, step_counts):
     synth, llama, dsm, ops = load_pkg("synth"), load_pkg("llama"), load_pkg("decode_session"), load_pkg("ops")
-    rng = np.random.default_rng(20240611)
-    for case in range(120):
+    rng = np.random.default_rng(rng_seed)
+    for case in range(cases):
         D = int(rng.choice([64, 128])); Hkv = int(rng.choice([1, 2, 4])); Hq = Hkv * int(rng.choice([1, 2, 4]))
         hidden = int(rng.choice([256, 512, 1024])); inter = int(rng.choice([352, 704, 1408, 2816]))
         layers = int(rng.choice([1, 2, 3]))
-        B = int(rng.choice([1, 2, 5, 16, 17, 32, 33, 48, 64])); P = int(rng.choice([3, 15, 16, 30])); steps = int(rng.choice([2, 5, 19]))
+        B = int(rng.choice(batches)); P = int(rng.choice([3, 15, 16, 30])); steps = int(rng.choice(step_counts))
         r = int(rng.choice([8, 16, 32, 64])); n_ad = int(rng.choice([1, 3, 8, 70])); k = int(rng.integers(0, 8))
         targets = tuple(np.array(ALL)[sorted(rng.choice(7, size=k, replace=False))]) if k else ()
         shape = synth.LlamaShape(hidden_size=hidden, intermediate_size=inter, num_attention_heads=Hq, num_key_value_heads=Hkv,
