@@ -670,7 +670,7 @@ int launch_gemm_pp(void* y, const f16* x, int ldx, int x_tt, const f16* Wp, int 
 // Token blocks between the decode GEMV and the persistent kernel above (65 to a few hundred tokens: a decode step of
 // many sequences, a short prefill).  The weights are read once and the matrix cores and the operand loads weigh about
 // the same, so the block is as tall as the token block allows and narrow enough to give every compute unit a
-// workgroup: FT x FN fragments (128 or 256 tokens x 128 or 64 weight rows), eight waves, both operands in fragment
+// workgroup: FT x FN fragments (128 or 256 tokens x 128, 96 or 64 weight rows), eight waves, both operands in fragment
 // order and copied from global memory straight into an LDS ring.  A stage of the ring is TWO 32-k steps: with the
 // few MFMAs a wave has per 32-k step here (4 to 16), a barrier and a wait per step cost more than the step itself.
 // Four (three) stages, of which three (two) are in flight per compute unit - across the barrier of a stage, which is
@@ -694,13 +694,16 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
   constexpr int MID_STAGES = FT == 16 ? 3 : 4;
   constexpr int SF = FN + FT;                  // fragments of one 32-k step: weights, then tokens
   constexpr int LF = MID_KS * SF;              // fragments per stage
-  constexpr int LQ = LF / PP_WAVES;            // ... of which a wave fetches LQ (fragment f = wave + 8 q: fragment f % SF of k-step f / SF)
+  constexpr int LQ = (LF + PP_WAVES - 1) / PP_WAVES;   // ... of which a wave fetches LQ (fragment f = wave + 8 q: fragment f % SF of k-step f / SF)
+  constexpr int LREM = LF % PP_WAVES;          // ... or, when they do not divide, the waves from LREM on one fewer
   constexpr int STAGE_ELEMS = LF * 512;
   constexpr int WTF = FT / 4;                  // token fragments of a wave's tile
   constexpr int WNF = FN / 2;                  // weight fragments of a wave's tile
   constexpr int VM = (MID_STAGES - 2) * LQ;    // a wave's loads that may still be in flight when the next stage is read
-  static_assert(LF % PP_WAVES == 0 && FT % 4 == 0 && FN % 2 == 0 && WNF <= 4, "fragments divide over the waves");
+  constexpr int VM1 = (MID_STAGES - 2) * (LQ - 1);   // ... for the waves with one fragment fewer
+  static_assert(FT % 4 == 0 && FN % 2 == 0 && WNF <= 4, "the tile divides over the waves");
   static_assert(VM == 5 || VM == 6 || VM == 8, "wait_next has an instruction for each of these");
+  static_assert(LREM == 0 || VM1 == 5 || VM1 == 6, "wait_next has an instruction for each of these");
   extern __shared__ __align__(16) f16 smem[];  // [MID_STAGES][STAGE_ELEMS]; the output staging reuses it after the K loop
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int KB = K / 32;
@@ -716,7 +719,7 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
   int step[LQ], kso[LQ];
 #pragma unroll
   for (int q = 0; q < LQ; ++q) {
-    const int f = (wave + PP_WAVES * q) % SF;  // uniform
+    const int f = (wave + PP_WAVES * q) % SF;  // uniform (past LF for the last q of a wave with one fewer: set up, never issued)
     kso[q] = (wave + PP_WAVES * q) / SF;
     if (f < FN) {
       int nt = n0 / 16 + f;
@@ -735,6 +738,7 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
     f16* dst = smem + ring * STAGE_ELEMS + wave * 512;
 #pragma unroll
     for (int q = 0; q < LQ; ++q) {
+      if (LREM != 0 && q == LQ - 1 && wave >= LREM) break;      // uniform
       int kb = load_kb + kso[q];
       kb = kb < kb1 ? kb : kb1 - 1;            // past the slice: a valid address; the data is not multiplied
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + (size_t)kb * step[q]),
@@ -782,6 +786,11 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
   // stage multiplied next has landed; with everybody's wait and fragment reads behind the barrier, the slot of the
   // stage just read is refilled
   auto wait_next = [&]() {
+    if (LREM != 0 && wave >= LREM) {             // uniform
+      if constexpr (VM1 == 5) asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
+      return;
+    }
     if constexpr (VM == 5) asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory");
     else if constexpr (VM == 6) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
@@ -839,8 +848,9 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
       }
       __builtin_amdgcn_wave_barrier();
 #pragma unroll
-      for (int q = 0; q < 16 * CPR / WAVE; ++q) {
+      for (int q = 0; q < (16 * CPR + WAVE - 1) / WAVE; ++q) {
         const int c = q * 64 + lane;             // 16-byte chunk: token row c / CPR, columns (c % CPR) * 8 ..
+        if ((16 * CPR) % WAVE != 0 && c >= 16 * CPR) break;
         const int tr = c / CPR, cc = (c % CPR) * 8;
         const int t = t0 + (wt * WTF + j) * 16 + tr;
         const int n = n0 + wn * WNF * 16 + cc;
@@ -882,7 +892,8 @@ __global__ __launch_bounds__(PP_WAVES* WAVE, 2) void gemm_mid_kernel(void* __res
 // Block shape and K slices of the mid-size kernel for a shape: 128-token blocks when 256-token ones would leave most
 // compute units without a workgroup, and 64 weight rows per block instead of 128 when that still leaves half of them
 // idle (up to 128 tokens: 170 instead of 192 us for the four linears of a 4096 / 11008 layer; with two token blocks
-// the narrow form loses, so it is not taken there).
+// the narrow form loses, so it is not taken there); 96 rows for the launches without K slices where that fills more
+// units in the same number of rounds.
 struct MidShape {
   int ft, fn, ksplit;
 };
@@ -894,6 +905,15 @@ MidShape gemm_mid_shape(int T, int K, int N, int ksplit_max) {
   m.ft = (T <= 128 || (long)cols8 * ceil_div(T, 256) * ksplit_max <= 128) ? 8 : 16;
   const int tb = ceil_div(T, m.ft * 16);
   m.fn = (long)cols8 * tb * ks_cap <= 128 ? 4 : 8;
+  if (ks_cap == 1 && m.fn == 8) {
+    // 96 rows per block where that takes no more rounds of the compute units than 128: more units busy, fewer bytes
+    // per workgroup (q/k/v at 256 tokens: 256 workgroups instead of 192, 43.9 -> 41.2 us; gate/up 230 instead of 172,
+    // 69.0 -> 63.3 us)
+    int n_cu = gemm_n_cu();
+    if (n_cu <= 0) n_cu = 256;
+    const int w8 = cols8 * tb, w6 = ceil_div(N, 96) * tb;
+    if (ceil_div(w6, n_cu) * (m.ft + 6) < ceil_div(w8, n_cu) * (m.ft + 8)) m.fn = 6;
+  }
   const int cols = ceil_div(N, m.fn * 16);
   int ks = 256 / (cols * tb);
   if (ks > ks_cap) ks = ks_cap;
@@ -920,9 +940,11 @@ int launch_gemm_mid(void* y, float* part, int ld_part, const MidShape& m, const 
                     hipStream_t s) {
   if (m.ft == 8) {
     if (m.fn == 4) return launch_gemm_mid_shape<OUT, 8, 4>(y, part, ld_part, m.ksplit, xf, x_tt, Wp, T, K, N, s);
+    if (m.fn == 6) return launch_gemm_mid_shape<OUT, 8, 6>(y, part, ld_part, m.ksplit, xf, x_tt, Wp, T, K, N, s);
     return launch_gemm_mid_shape<OUT, 8, 8>(y, part, ld_part, m.ksplit, xf, x_tt, Wp, T, K, N, s);
   }
   if (m.fn == 4) return launch_gemm_mid_shape<OUT, 16, 4>(y, part, ld_part, m.ksplit, xf, x_tt, Wp, T, K, N, s);
+  if (m.fn == 6) return launch_gemm_mid_shape<OUT, 16, 6>(y, part, ld_part, m.ksplit, xf, x_tt, Wp, T, K, N, s);
   return launch_gemm_mid_shape<OUT, 16, 8>(y, part, ld_part, m.ksplit, xf, x_tt, Wp, T, K, N, s);
 }
 

@@ -300,12 +300,13 @@ def test_gemm_lds_staged_block_kernel(ops, synth, T, K, N):
 
 
 @pytest.mark.parametrize("T,K,N", [(4096, 320, 4096), (4100, 128, 4104), (4000, 1024, 4200), (300, 512, 264), (65, 64, 16),
-                                   (4096, 4096, 4096)])
+                                   (4096, 4096, 4096), (256, 512, 12288), (256, 128, 12200), (200, 256, 22016)])
 def test_persistent_gemm_rowmajor_and_fragment_ordered_activations(ops, synth, T, K, N):
     """The persistent 256 x 256 matrix-core GEMM (operands copied from global memory straight into LDS): row-major x
-    once there are 256 blocks and K % 64 == 0, fragment-ordered x of any T > 64.  Ragged token and column edges, all
-    three epilogues; rows past T of the last fragment hold NaN and must not reach a stored result; the same bits
-    whichever layout x comes in."""
+    once there are 256 blocks and K % 64 == 0, fragment-ordered x of any T > 64 (below 256 blocks the mid-size kernel;
+    the last three shapes take its 96-row blocks, with 128 and with 256 tokens per block).  Ragged token and column
+    edges, all three epilogues; rows past T of the last fragment hold NaN and must not reach a stored result; the same
+    bits whichever layout x comes in."""
     print(f"case persistent gemm T={T} K={K} N={N}", flush=True)
     x = synth.normal(13, f"pg.x.{T}.{K}", (T, K), 1.0, torch.float16, DEV)
     W = synth.normal(13, f"pg.W.{N}.{K}", (N, K), 0.02, torch.float16, DEV)
